@@ -1,0 +1,157 @@
+/*
+ * twinkle_amd — C ABI of the MI355X (gfx950) multi-LoRA hot path.
+ *
+ * Plain pointers and sizes only; every pointer named "device" is HIP device
+ * memory owned by the caller.  All work is ordered on the stream that is
+ * passed in (a hipStream_t cast to void*; NULL = the null stream).  No call
+ * allocates, frees, synchronises the device or keeps state between calls,
+ * except where stated.  Return value: TK_OK or a negative TK_ERR_* code.
+ *
+ * The reference (modelscope/twinkle) is pure Python and has no FFI for this
+ * path; each entry point below names the reference code whose work it takes
+ * over (paths relative to the reference checkout).
+ */
+#ifndef TWINKLE_AMD_H
+#define TWINKLE_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* tk_stream_t; /* hipStream_t */
+
+enum {
+  TK_OK = 0,
+  TK_ERR_INVALID = -1,     /* bad argument (null pointer, negative size, misaligned stride) */
+  TK_ERR_WORKSPACE = -2,   /* workspace smaller than the matching *_bytes() query */
+  TK_ERR_UNSUPPORTED = -3, /* shape outside what the kernels handle (see each call) */
+  TK_ERR_LAUNCH = -4       /* HIP reported an error at launch */
+};
+
+enum { TK_DTYPE_F32 = 0, TK_DTYPE_BF16 = 1 };
+enum { TK_KEY_I32 = 0, TK_KEY_I64 = 1 };
+
+/* Rows per forward tile and per weight-gradient chunk (fixed at build time). */
+#define TK_TILE_ROWS 32
+#define TK_CHUNK_ROWS 512
+#define TK_MAX_GROUPS 16384
+#define TK_MAX_RANK 128
+
+const char* tk_version(void);
+const char* tk_error_string(int code);
+
+/* ---------------------------------------------------------------------------
+ * Segment builder: rows -> groups, stable.
+ *
+ * Replaces the reference's mask-based ordering
+ *   src/twinkle/model/transformers/moe/expert_parallel.py:254-255 (one_hot mask),
+ *   src/twinkle/model/transformers/moe/ep_utils.py:99-118 (masked_select order),
+ *   src/twinkle/model/transformers/moe/ep_utils.py:191 (per-group counts),
+ *   src/twinkle/model/transformers/moe/expert_parallel.py:347-349 (host cumsum
+ *   with .item() syncs),
+ * and widens MultiLora.adapter()'s one-adapter-per-call selection
+ *   (src/twinkle/model/multi_lora.py:126-163) to one adapter id per row.
+ *
+ * keys[f] in [0, num_groups) is the group of flat row f (top-k routing: f = k*T + t).
+ * perm_out[j]  = flat row placed at sorted position j (stable: ties keep ascending f),
+ * offsets_out[g] = first sorted position of group g, offsets_out[num_groups] = rows.
+ * Both are int64 like the reference's tensors and may be NULL when only the
+ * workspace is wanted.  seg_ws receives the device-side segment table the
+ * LoRA and permute calls read; it must stay alive and unmodified while they run.
+ * Keys outside [0, num_groups) are clamped for memory safety and counted;
+ * tk_segment_bad_keys() reports the count.
+ * Limits: num_groups <= TK_MAX_GROUPS, rows < 2^31.
+ * ------------------------------------------------------------------------ */
+int64_t tk_segment_workspace_bytes(int64_t rows, int32_t num_groups);
+int tk_segment_build(const void* keys_device, int32_t key_dtype, int64_t rows, int32_t num_groups,
+                     int64_t* perm_out_device, int64_t* offsets_out_device, void* seg_ws_device,
+                     int64_t seg_ws_bytes, tk_stream_t stream);
+/* Synchronises the stream and copies one counter back: number of out-of-range keys. */
+int tk_segment_bad_keys(const void* seg_ws_device, tk_stream_t stream, int64_t* count_out_host);
+
+/* ---------------------------------------------------------------------------
+ * Row gather / weighted scatter-back in segment order.
+ *
+ * tk_permute_rows replaces ep_utils.py:99-118 (`permute`: index_select by the
+ * masked_select order): dst[j] = src[perm[j] mod num_tokens] (* w[token, k] when
+ * weights is non-NULL; that form is the backward of tk_unpermute_rows).
+ * tk_unpermute_rows replaces ep_utils.py:121-149 / :280-287 (`unpermute`:
+ * zero-init + scatter_add_ with routing weights):
+ *   out[t] = sum_{k ascending} rows[pos(k*T + t)] * w[t, k]
+ * computed as a gather with a fixed summation order (deterministic, unlike
+ * the reference's atomics).  weights is [num_tokens, top_k] in `dtype`, or NULL
+ * for unit weights.  rows == num_tokens * top_k.
+ * ------------------------------------------------------------------------ */
+int tk_permute_rows(const void* src_device, int64_t ld_src, void* dst_device, int64_t ld_dst,
+                    const void* weights_device, const void* seg_ws_device, int64_t rows, int64_t num_tokens,
+                    int32_t width, int32_t num_groups, int32_t dtype, tk_stream_t stream);
+int tk_unpermute_rows(const void* rows_device, int64_t ld_rows, void* out_device, int64_t ld_out,
+                      const void* weights_device, const void* seg_ws_device, int64_t rows, int64_t num_tokens,
+                      int32_t width, int32_t num_groups, int32_t dtype, tk_stream_t stream);
+/* dw[t, k] = <dout[t, :], rows[pos(k*T + t), :]>   (gradient of the routing weights, fp32 out) */
+int tk_unpermute_weight_grad(const void* dout_device, int64_t ld_dout, const void* rows_device, int64_t ld_rows,
+                             float* dw_device, const void* seg_ws_device, int64_t rows, int64_t num_tokens,
+                             int32_t width, int32_t num_groups, int32_t dtype, tk_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Segmented LoRA linear.
+ *
+ * Replaces the body of the patched LoraLayer forward
+ *   src/twinkle/model/multi_lora.py:315-326
+ *     h = linear(x, A[:r]); u = linear(h, B[:, :r]); result = result + u * scaling
+ * and the autograd of those two F.linear calls, for every adapter of a mixed
+ * batch in one pass; and, with per-(expert, tenant) groups, the effect of the
+ * merged expert weights of
+ *   src/twinkle/model/multi_lora_target_parameters.py:158-179 inside the per-expert loop
+ *   src/twinkle/model/transformers/moe/expert_parallel.py:347-371
+ * without materialising the [E, out, in] delta.
+ *
+ * Group g uses A_g = lora_A[g] ([>= rank[g], in_features], row stride lda) and
+ * B_g = lora_B[g] ([out_features, >= rank[g]], row stride ldb): the slot
+ * tensors of the reference at their physical strides; only the leading
+ * rank[g] rows / columns are read or written.  rank[g] == 0 skips the group.
+ * ------------------------------------------------------------------------ */
+typedef struct tk_lora_desc {
+  int64_t rows;         /* rows covered by the segment table */
+  int32_t in_features;  /* K */
+  int32_t out_features; /* M */
+  int32_t num_groups;   /* G, as given to tk_segment_build */
+  int32_t max_rank;     /* host-side upper bound of rank[g], <= TK_MAX_RANK */
+  int32_t dtype;        /* TK_DTYPE_* of x, y, A, B, h and the gradients */
+  int32_t map_rows;     /* 1: sorted position p touches row perm[p] of x / y (dense LoRA);
+                           0: rows are already in segment order (after tk_permute_rows) */
+  const void* seg_ws;          /* device, from tk_segment_build */
+  const void* const* lora_A;   /* device array [G] of device pointers */
+  const void* const* lora_B;   /* device array [G] of device pointers */
+  int64_t lda;                 /* elements */
+  int64_t ldb;                 /* elements */
+  const int32_t* rank;         /* device [G] */
+  const float* scale;          /* device [G]: alpha/r or alpha/sqrt(r) */
+} tk_lora_desc;
+
+/* Bytes of the saved shrink output h (scale * x A^T per row, kept for backward). */
+int64_t tk_lora_h_bytes(const tk_lora_desc* desc);
+int64_t tk_lora_bwd_workspace_bytes(const tk_lora_desc* desc);
+
+/* y[row] += scale_g * (x[row] A_g^T) B_g^T in place on the base output; h_device is written. */
+int tk_lora_fwd(const tk_lora_desc* desc, const void* x_device, int64_t ldx, void* y_device, int64_t ldy,
+                void* h_device, tk_stream_t stream);
+
+/* dx[row] += scale_g * (dy[row] B_g) A_g        (skipped when dx_device is NULL)
+ * dA_g[:r] (+)= (scale_g * dy B_g)^T x          (skipped when grad_A is NULL)
+ * dB_g[:, :r] (+)= dy^T h                       (skipped when grad_B is NULL)
+ * grad_A / grad_B are device arrays [G] of device pointers with the strides lda / ldb;
+ * accumulate != 0 adds onto their contents, 0 overwrites the live [:r] block.  Elements
+ * outside the live block are never touched.  Weight gradients are reduced over
+ * row chunks in a fixed order: results are bitwise repeatable. */
+int tk_lora_bwd(const tk_lora_desc* desc, const void* dy_device, int64_t lddy, const void* x_device, int64_t ldx,
+                const void* h_device, void* dx_device, int64_t lddx, void* const* grad_A, void* const* grad_B,
+                int32_t accumulate, void* workspace_device, int64_t workspace_bytes, tk_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TWINKLE_AMD_H */

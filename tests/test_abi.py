@@ -1,0 +1,55 @@
+"""The shared library loads and exports every entry point the header declares (no GPU needed)."""
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, 'include', 'twinkle_amd.h')).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(tk_[a-z_0-9]+)\s*\(', text)))
+
+
+def test_header_declares_entry_points():
+    names = _declared()
+    assert 'tk_segment_build' in names and 'tk_lora_fwd' in names and 'tk_lora_bwd' in names
+    assert len(names) >= 10
+
+
+def test_library_exports_every_declared_symbol():
+    from twinkle_amd import _lib
+    if not os.path.exists(_lib.library_path()):
+        pytest.fail(f'{_lib.library_path()} is not built (run __graft_entry__.build())')
+    lib = _lib.load()
+    for name in _declared():
+        assert hasattr(lib, name), f'{name} declared in the header but not exported'
+    assert set(_lib.EXPORTS) == set(_declared()), 'ctypes table and header disagree'
+    assert lib.tk_version().startswith(b'twinkle_amd')
+    assert lib.tk_error_string(-2) == b'workspace too small'
+
+
+def test_size_queries_run_on_the_host():
+    import ctypes
+    from twinkle_amd import _lib
+    lib = _lib.load()
+    small = lib.tk_segment_workspace_bytes(1024, 4)
+    big = lib.tk_segment_workspace_bytes(65536, 512)
+    assert 0 < small < big
+    assert lib.tk_segment_workspace_bytes(-1, 4) == _lib.TK_ERR_INVALID
+    d = _lib.LoraDesc()
+    d.rows, d.in_features, d.out_features, d.num_groups, d.max_rank, d.dtype = 16384, 4096, 4096, 16, 16, 1
+    h = lib.tk_lora_h_bytes(ctypes.byref(d))
+    assert h == 16 * 16384 * 2
+    assert lib.tk_lora_bwd_workspace_bytes(ctypes.byref(d)) > h
+    d.max_rank = 1000
+    assert lib.tk_lora_h_bytes(ctypes.byref(d)) == _lib.TK_ERR_INVALID
+
+
+def test_ops_refuse_cpu_tensors():
+    import torch
+    from twinkle_amd import build_segments
+    with pytest.raises(RuntimeError):
+        build_segments(torch.zeros(8, dtype=torch.int32), 2)

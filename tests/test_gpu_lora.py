@@ -1,0 +1,244 @@
+"""Segmented LoRA forward/backward through the C ABI against the CPU oracle.
+
+Bars (BASELINE.json): fp32 within 1e-5 relative, bf16 within 2e-2 max relative error against a
+float32-or-better reference; here the reference is the oracle in float64 on the same (rounded) inputs,
+and "relative" is max|got - ref| / max|ref|.
+"""
+import pytest
+import torch
+
+import oracle
+from conftest import max_rel_err
+from twinkle_amd import AdapterGroups, build_segments, lora_bwd_, lora_fwd_, multi_lora_delta, multi_lora_linear
+from twinkle_amd import workloads
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-2}
+
+
+def _problem(t, k, m, n, max_r, ranks, seed, ids=None):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(t, k, generator=g)
+    base = torch.randn(t, m, generator=g)
+    dy = torch.randn(t, m, generator=g)
+    a = [(torch.rand(max_r, k, generator=g) * 2 - 1) / k**0.5 for _ in range(n)]
+    b = [torch.randn(m, max_r, generator=g) * 0.05 for _ in range(n)]
+    if ids is None:
+        ids = torch.randint(0, n, (t,), generator=g)
+    scales = [2.0 if i % 2 == 0 else 0.5 for i in range(n)]
+    return x, base, dy, a, b, ids, list(ranks), scales
+
+
+def _run(dev, dtype, x, base, dy, a, b, ids, ranks, scales, check_zero_beyond_rank=True):
+    """GPU through autograd vs oracle in float64 on the same rounded inputs."""
+    cast = lambda t: t.to(dtype)  # noqa: E731
+    xd = cast(x).to(dev).requires_grad_(True)
+    yd = cast(base).to(dev).requires_grad_(True)
+    ad = [cast(t).to(dev).requires_grad_(True) for t in a]
+    bd = [cast(t).to(dev).requires_grad_(True) for t in b]
+    seg = build_segments(ids.to(torch.int32).to(dev), len(a), check=True)
+    groups = AdapterGroups(ad, bd, ranks, scales)
+    y = multi_lora_delta(xd, yd * 1.0, seg, groups)
+    y.backward(cast(dy).to(dev))
+    f64 = lambda t: cast(t).double()  # noqa: E731
+    yo, dxo, dao, dbo = oracle.multi_lora_linear_grads(f64(x), f64(base), ids, [f64(t) for t in a],
+                                                        [f64(t) for t in b], ranks, scales, f64(dy))
+    tol = TOL[dtype]
+    assert max_rel_err(y, yo) < tol, 'Y'
+    assert max_rel_err(xd.grad, dxo) < tol, 'dX'
+    assert torch.equal(yd.grad.cpu(), cast(dy)), 'dY passes through to the base output unchanged'
+    for g in range(len(a)):
+        assert max_rel_err(ad[g].grad, dao[g]) < tol, f'dA[{g}]'
+        assert max_rel_err(bd[g].grad, dbo[g]) < tol, f'dB[{g}]'
+        if check_zero_beyond_rank:
+            assert torch.count_nonzero(ad[g].grad[ranks[g]:]) == 0
+            assert torch.count_nonzero(bd[g].grad[:, ranks[g]:]) == 0
+    return y, xd.grad, [t.grad for t in ad], [t.grad for t in bd]
+
+
+def test_config1_fp32_plumbing(dev):
+    """BASELINE config 1: T=512, 1024->1024, 4 adapters rank 8 alpha 16, contiguous segments; Y, dX, dA, dB."""
+    w = workloads.config1_plumbing()
+    _run(dev, torch.float32, w.x, w.base_out, w.dy, w.lora_A, w.lora_B, w.ids, w.ranks, w.scales)
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize('t,k,m,n,max_r,ranks', [
+    (1, 8, 8, 1, 4, [4]),
+    (33, 40, 24, 3, 8, [2, 8, 5]),                 # odd widths: generic kernels
+    (257, 128, 256, 4, 16, [16, 8, 16, 1]),
+    (700, 256, 128, 5, 32, [32, 0, 16, 8, 24]),   # a rank-0 (skipped) adapter
+    (1500, 384, 640, 6, 64, [64, 8, 16, 32, 64, 4]),
+])
+def test_small_shapes(dev, dtype, t, k, m, n, max_r, ranks):
+    _run(dev, dtype, *_problem(t, k, m, n, max_r, ranks, seed=t))
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_empty_and_huge_segments(dev, dtype):
+    t, n = 2100, 6
+    ids = torch.zeros(t, dtype=torch.long)
+    ids[:40] = 3          # one tiny segment, adapters 1, 2, 4, 5 empty, adapter 0 spans several chunks
+    ids = ids[torch.randperm(t, generator=torch.Generator().manual_seed(0))]
+    x, base, dy, a, b, _, ranks, scales = _problem(t, 256, 128, n, 16, [16] * n, seed=3)
+    _, _, da, db = _run(dev, dtype, x, base, dy, a, b, ids, ranks, scales)
+    for g in (1, 2, 4, 5):
+        assert torch.count_nonzero(da[g]) == 0 and torch.count_nonzero(db[g]) == 0
+
+
+def test_results_are_bitwise_repeatable(dev):
+    p = _problem(3000, 512, 256, 4, 16, [16, 8, 16, 16], seed=5)
+    r1 = _run(dev, torch.bfloat16, *p)
+    r2 = _run(dev, torch.bfloat16, *p)
+    assert torch.equal(r1[0], r2[0]) and torch.equal(r1[1], r2[1])
+    for u, v in zip(r1[2] + r1[3], r2[2] + r2[3]):
+        assert torch.equal(u, v)
+
+
+def test_my_gradients_ignore_other_tenants_rows(dev):
+    """Reference invariant: only the active adapter is updated (tests/model/test_multi_lora_target_parameters.py:78-100)."""
+    x, base, dy, a, b, ids, ranks, scales = _problem(900, 256, 256, 3, 16, [16, 16, 8], seed=6)
+    _, _, da, db = _run(dev, torch.bfloat16, x, base, dy, a, b, ids, ranks, scales)
+    x2 = x.clone()
+    x2[ids != 0] = 7.0
+    _, _, da2, db2 = _run(dev, torch.bfloat16, x2, base, dy, a, b, ids, ranks, scales)
+    assert torch.equal(da[0], da2[0]) and torch.equal(db[0], db2[0])
+
+
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_fused_base_linear_node(dev, dtype):
+    """F.linear + LoRA as one autograd node: dX of the base GEMM updated in place."""
+    t, k, m, n = 600, 256, 384, 3
+    x, _, dy, a, b, ids, ranks, scales = _problem(t, k, m, n, 16, [16, 4, 8], seed=7)
+    w = torch.randn(m, k, generator=torch.Generator().manual_seed(8)) * 0.05
+    bias = torch.randn(m, generator=torch.Generator().manual_seed(9))
+    cast = lambda v: v.to(dtype)  # noqa: E731
+    xd = cast(x).to(dev).requires_grad_(True)
+    ad = [cast(v).to(dev).requires_grad_(True) for v in a]
+    bd = [cast(v).to(dev).requires_grad_(True) for v in b]
+    seg = build_segments(ids.to(torch.int32).to(dev), n)
+    y = multi_lora_linear(xd, cast(w).to(dev), cast(bias).to(dev), seg, AdapterGroups(ad, bd, ranks, scales))
+    y.backward(cast(dy).to(dev))
+    f64 = lambda v: cast(v).double()  # noqa: E731
+    x64 = f64(x).requires_grad_(True)
+    a64 = [f64(v).requires_grad_(True) for v in a]
+    b64 = [f64(v).requires_grad_(True) for v in b]
+    base64 = torch.nn.functional.linear(x64, f64(w), f64(bias))
+    if dtype == torch.bfloat16:
+        base64 = base64.detach().bfloat16().double() + (base64 - base64.detach())  # base GEMM output is stored in bf16
+    yo = oracle.multi_lora_linear(x64, base64, ids, a64, b64, ranks, scales)
+    yo.backward(f64(dy))
+    tol = TOL[dtype] * (2 if dtype == torch.bfloat16 else 20)   # the base GEMM runs in the library's own order
+    assert max_rel_err(y, yo) < tol
+    assert max_rel_err(xd.grad, x64.grad) < tol
+    for g in range(n):
+        assert max_rel_err(ad[g].grad, a64[g].grad) < TOL[dtype]
+        assert max_rel_err(bd[g].grad, b64[g].grad) < TOL[dtype]
+
+
+def test_rows_already_in_segment_order_and_packed_expert_weights(dev):
+    """map_rows=0 with (expert, tenant) groups reading blocks of packed [E, max_r, in] tensors (config 4 shape, small)."""
+    e, nt, t, k_in, m_out, max_r, r = 6, 2, 500, 128, 256, 8, 4
+    g = torch.Generator().manual_seed(10)
+    keys = torch.randint(0, e * nt, (t,), generator=g)
+    a = [torch.randn(e, max_r, k_in, generator=g) * 0.1 for _ in range(nt)]
+    b = [torch.randn(e, m_out, max_r, generator=g) * 0.1 for _ in range(nt)]
+    x = torch.randn(t, k_in, generator=g)
+    base = torch.randn(t, m_out, generator=g)
+    dy = torch.randn(t, m_out, generator=g)
+    dtype = torch.bfloat16
+    cast = lambda v: v.to(dtype)  # noqa: E731
+    seg = build_segments(keys.to(torch.int32).to(dev), e * nt)
+    perm = seg.perm
+    xs = cast(x).to(dev)[perm].requires_grad_(True)           # rows physically in segment order
+    ys = cast(base).to(dev)[perm]
+    ad = [cast(v).to(dev).requires_grad_(True) for v in a]
+    bd = [cast(v).to(dev).requires_grad_(True) for v in b]
+    groups = AdapterGroups(ad, bd, [r] * (e * nt), [2.0] * (e * nt),
+                           a_index=[i % nt for i in range(e * nt)], a_offset=[(i // nt) * max_r * k_in for i in range(e * nt)],
+                           b_index=[i % nt for i in range(e * nt)], b_offset=[(i // nt) * m_out * max_r for i in range(e * nt)])
+    y = multi_lora_delta(xs, ys * 1.0, seg, groups, map_rows=False)
+    y.backward(cast(dy).to(dev)[perm])
+    # oracle: group i = (expert i // nt, tenant i % nt)
+    f64 = lambda v: cast(v).double()  # noqa: E731
+    a_list = [f64(a[i % nt][i // nt]) for i in range(e * nt)]
+    b_list = [f64(b[i % nt][i // nt]) for i in range(e * nt)]
+    yo, dxo, dao, dbo = oracle.multi_lora_linear_grads(f64(x), f64(base), keys, a_list, b_list, [r] * (e * nt),
+                                                        [2.0] * (e * nt), f64(dy))
+    pc = perm.cpu()
+    assert max_rel_err(y, yo[pc]) < 2e-2
+    assert max_rel_err(xs.grad, dxo[pc]) < 2e-2
+    for i in range(e * nt):
+        assert max_rel_err(ad[i % nt].grad[i // nt], dao[i]) < 2e-2
+        assert max_rel_err(bd[i % nt].grad[i // nt], dbo[i]) < 2e-2
+    # the same thing as the reference's merged-weight expert loop (W + dW)
+    offsets = seg.offsets.cpu()
+    for i in (0, 5, e * nt - 1):
+        s, t_ = int(offsets[i]), int(offsets[i + 1])
+        if s == t_:
+            continue
+        dw = oracle.expert_delta_weight(f64(a[i % nt]), f64(b[i % nt]), r, 2.0)[i // nt]
+        want = f64(base)[pc][s:t_] + f64(x)[pc][s:t_] @ dw.t()
+        assert max_rel_err(y[s:t_], want) < 2e-2
+
+
+def test_accumulate_and_strided_inputs(dev):
+    """C ABI directly: row strides larger than the width, accumulate=1 adds onto existing gradients."""
+    t, k, m, n, max_r = 400, 256, 128, 2, 16
+    x, base, dy, a, b, ids, ranks, scales = _problem(t, k, m, n, max_r, [16, 8], seed=11)
+    dt = torch.bfloat16
+    xbuf = torch.zeros(t, k + 64, dtype=dt, device=dev)
+    ybuf = torch.zeros(t, m + 128, dtype=dt, device=dev)
+    dybuf = torch.zeros(t, m + 8, dtype=dt, device=dev)
+    xbuf[:, :k] = x.to(dt).to(dev)
+    ybuf[:, :m] = base.to(dt).to(dev)
+    dybuf[:, :m] = dy.to(dt).to(dev)
+    xv, yv, dyv = xbuf[:, :k], ybuf[:, :m], dybuf[:, :m]
+    ad = [v.to(dt).to(dev) for v in a]
+    bd = [v.to(dt).to(dev) for v in b]
+    seg = build_segments(ids.to(torch.int32).to(dev), n)
+    groups = AdapterGroups(ad, bd, ranks, scales)
+    h = lora_fwd_(xv, yv, seg, groups)
+    ga = [torch.ones_like(v) for v in ad]
+    gb = [torch.ones_like(v) for v in bd]
+    pa = torch.tensor([v.data_ptr() for v in ga], dtype=torch.int64, device=dev)
+    pb = torch.tensor([v.data_ptr() for v in gb], dtype=torch.int64, device=dev)
+    dx = torch.ones(t, k, dtype=dt, device=dev)
+    lora_bwd_(dyv, xv, h, dx, pa, pb, seg, groups, accumulate=True)
+    f64 = lambda v: v.to(dt).double()  # noqa: E731
+    yo, dxo, dao, dbo = oracle.multi_lora_linear_grads(f64(x), f64(base), ids, [f64(v) for v in a],
+                                                        [f64(v) for v in b], ranks, scales, f64(dy))
+    assert max_rel_err(yv, yo) < 2e-2
+    assert torch.count_nonzero(ybuf[:, m:]) == 0, 'padding columns untouched'
+    assert max_rel_err(dx, dxo + 1.0) < 2e-2
+    for g in range(n):
+        r = ranks[g]
+        assert max_rel_err(ga[g][:r], dao[g][:r] + 1.0) < 2e-2
+        assert max_rel_err(gb[g][:, :r], dbo[g][:, :r] + 1.0) < 2e-2
+        assert torch.all(ga[g][r:] == 1) and torch.all(gb[g][:, r:] == 1), 'outside the live block: untouched'
+
+
+def test_argument_errors(dev):
+    x, base, dy, a, b, ids, ranks, scales = _problem(64, 32, 32, 2, 8, [8, 8], seed=12)
+    ad = [v.to(dev) for v in a]
+    bd = [v.to(dev) for v in b]
+    seg = build_segments(ids.to(torch.int32).to(dev), 2)
+    groups = AdapterGroups(ad, bd, ranks, scales)
+    with pytest.raises(ValueError):
+        lora_fwd_(x.to(dev)[:, :16], base.to(dev), seg, groups)            # wrong width
+    with pytest.raises(ValueError):
+        lora_fwd_(x.bfloat16().to(dev), base.to(dev), seg, groups)          # dtype mismatch
+    with pytest.raises(RuntimeError):
+        lora_fwd_(x, base, seg, groups)                                     # CPU tensors
+    with pytest.raises(RuntimeError):
+        AdapterGroups(ad, bd, [9, 8], scales)                               # rank above the slot size
+    seg3 = build_segments(ids.to(torch.int32).to(dev), 3)
+    with pytest.raises(ValueError):
+        lora_fwd_(x.to(dev), base.to(dev), seg3, groups)                    # group count mismatch
+
+
+def test_config2_full_size_bf16(dev):
+    """BASELINE config 2 at full size: 4096->4096, T=16384, 16 adapters rank 16, Zipf ids, shuffled."""
+    w = workloads.config2_qproj()
+    _run(dev, torch.bfloat16, w.x, w.base_out, w.dy, w.lora_A, w.lora_B, w.ids, w.ranks, w.scales)

@@ -1,0 +1,16 @@
+"""twinkle_amd: the multi-LoRA hot path of modelscope/twinkle on MI355X (gfx950).
+
+Segment builder, segmented LoRA linear forward/backward and the row
+permute/unpermute around them run in hand-written HIP kernels behind a C ABI
+(``include/twinkle_amd.h``); this package binds them to PyTorch-ROCm tensors
+and mirrors the reference's ``MultiLora`` interface on top.  There is no CPU
+path: every op raises if the HIP library is missing or a tensor is not on the GPU.
+"""
+from .lora_layer import LoraConfig, LoraLinear, LoraModel, inject_adapter  # noqa: F401
+from .multi_lora import LoraTenant, MultiLora  # noqa: F401
+from .ops import (AdapterGroups, lora_bwd_, lora_bwd_workspace_bytes, lora_fwd_, lora_h_bytes,  # noqa: F401
+                  multi_lora_delta, multi_lora_linear)
+from .segments import (SegmentTable, build_segments, flat_keys_from_topk, packed_cu_seqlens, permute,  # noqa: F401
+                       token_groups_from_sequences, unpermute)
+
+__version__ = '0.1.0'

@@ -1,0 +1,197 @@
+// C ABI of the library: argument checks, workspace carving, kernel choice.
+#include "tk_common.h"
+
+using namespace tk;
+
+namespace {
+
+bool desc_ok(const tk_lora_desc* d) {
+  if (!d) return false;
+  if (d->rows < 0 || d->rows >= (1ll << 31)) return false;
+  if (d->in_features <= 0 || d->out_features <= 0) return false;
+  if (d->num_groups <= 0 || d->num_groups > TK_MAX_GROUPS) return false;
+  if (d->max_rank < 0 || d->max_rank > TK_MAX_RANK) return false;
+  if (d->dtype != TK_DTYPE_F32 && d->dtype != TK_DTYPE_BF16) return false;
+  if (!d->seg_ws || !d->lora_A || !d->lora_B || !d->rank || !d->scale) return false;
+  if (d->lda < d->in_features || d->ldb < d->max_rank) return false;
+  return true;
+}
+
+int run_pass(const PassArgs& a, const SegView& V, const SegLayout& L, int dtype, hipStream_t s) {
+  if (dtype == TK_DTYPE_BF16 && pass_mfma_supported(a)) return launch_pass_mfma(a, V, L, s);
+  return launch_pass_generic(a, V, L, dtype, s);
+}
+
+int run_wgrad(const WgradArgs& a, const SegView& V, const SegLayout& L, int dtype, hipStream_t s) {
+  int rc;
+  if (dtype == TK_DTYPE_BF16 && wgrad_mfma_supported(a))
+    rc = launch_wgrad_mfma(a, V, L, s);
+  else
+    rc = launch_wgrad_generic(a, V, L, dtype, s);
+  if (rc != TK_OK) return rc;
+  return launch_wgrad_reduce(a, V, L, dtype, s);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* tk_version(void) { return "twinkle_amd 0.1 (gfx950)"; }
+
+const char* tk_error_string(int code) {
+  switch (code) {
+    case TK_OK: return "ok";
+    case TK_ERR_INVALID: return "invalid argument";
+    case TK_ERR_WORKSPACE: return "workspace too small";
+    case TK_ERR_UNSUPPORTED: return "unsupported shape";
+    case TK_ERR_LAUNCH: return "HIP launch error";
+    default: return "unknown error";
+  }
+}
+
+int64_t tk_segment_workspace_bytes(int64_t rows, int32_t num_groups) {
+  if (rows < 0 || num_groups <= 0) return TK_ERR_INVALID;
+  return SegLayout(rows, num_groups).total;
+}
+
+int tk_segment_build(const void* keys, int32_t key_dtype, int64_t rows, int32_t num_groups, int64_t* perm_out,
+                     int64_t* offsets_out, void* seg_ws, int64_t seg_ws_bytes, tk_stream_t stream) {
+  if (rows < 0 || num_groups <= 0 || !seg_ws || (rows > 0 && !keys)) return TK_ERR_INVALID;
+  if (key_dtype != TK_KEY_I32 && key_dtype != TK_KEY_I64) return TK_ERR_INVALID;
+  if (num_groups > TK_MAX_GROUPS || rows >= (1ll << 31)) return TK_ERR_UNSUPPORTED;
+  if (seg_ws_bytes < SegLayout(rows, num_groups).total) return TK_ERR_WORKSPACE;
+  return launch_segment_build(keys, key_dtype, rows, num_groups, perm_out, offsets_out, seg_ws,
+                              (hipStream_t)stream);
+}
+
+int tk_segment_bad_keys(const void* seg_ws, tk_stream_t stream, int64_t* count_out) {
+  if (!seg_ws || !count_out) return TK_ERR_INVALID;
+  SegHeader h;
+  if (hipMemcpyAsync(&h, seg_ws, sizeof(h), hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess)
+    return TK_ERR_LAUNCH;
+  if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return TK_ERR_LAUNCH;
+  if (h.magic != kSegMagic) return TK_ERR_INVALID;
+  *count_out = h.bad_keys;
+  return TK_OK;
+}
+
+static bool rows_args_ok(const void* a, const void* b, const void* ws, int64_t rows, int64_t tokens, int32_t width,
+                         int32_t groups, int32_t dtype) {
+  if (!ws || rows < 0 || tokens < 0 || width <= 0 || groups <= 0) return false;
+  if (rows > 0 && (!a || !b || tokens == 0 || rows % tokens != 0)) return false;
+  return dtype == TK_DTYPE_F32 || dtype == TK_DTYPE_BF16;
+}
+
+int tk_permute_rows(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, const void* weights,
+                    const void* seg_ws, int64_t rows, int64_t num_tokens, int32_t width, int32_t num_groups,
+                    int32_t dtype, tk_stream_t stream) {
+  if (!rows_args_ok(src, dst, seg_ws, rows, num_tokens, width, num_groups, dtype)) return TK_ERR_INVALID;
+  if (ld_src < width || ld_dst < width) return TK_ERR_INVALID;
+  return launch_permute(src, ld_src, dst, ld_dst, weights, seg_ws, rows, num_tokens, width, num_groups, dtype,
+                        (hipStream_t)stream);
+}
+
+int tk_unpermute_rows(const void* rows_p, int64_t ld_rows, void* out, int64_t ld_out, const void* weights,
+                      const void* seg_ws, int64_t rows, int64_t num_tokens, int32_t width, int32_t num_groups,
+                      int32_t dtype, tk_stream_t stream) {
+  if (!rows_args_ok(rows_p, out, seg_ws, rows, num_tokens, width, num_groups, dtype)) return TK_ERR_INVALID;
+  if (ld_rows < width || ld_out < width) return TK_ERR_INVALID;
+  return launch_unpermute(rows_p, ld_rows, out, ld_out, weights, seg_ws, rows, num_tokens, width, num_groups, dtype,
+                          (hipStream_t)stream);
+}
+
+int tk_unpermute_weight_grad(const void* dout, int64_t ld_dout, const void* rows_p, int64_t ld_rows, float* dw,
+                             const void* seg_ws, int64_t rows, int64_t num_tokens, int32_t width,
+                             int32_t num_groups, int32_t dtype, tk_stream_t stream) {
+  if (!rows_args_ok(dout, rows_p, seg_ws, rows, num_tokens, width, num_groups, dtype) || (rows > 0 && !dw))
+    return TK_ERR_INVALID;
+  if (ld_dout < width || ld_rows < width) return TK_ERR_INVALID;
+  return launch_unpermute_wgrad(dout, ld_dout, rows_p, ld_rows, dw, seg_ws, rows, num_tokens, width, num_groups,
+                                dtype, (hipStream_t)stream);
+}
+
+int64_t tk_lora_h_bytes(const tk_lora_desc* d) {
+  if (!d || d->rows < 0 || d->max_rank < 0 || d->max_rank > TK_MAX_RANK) return TK_ERR_INVALID;
+  return round_up((int64_t)rank_pad(d->max_rank) * h_ld(d->rows) * elt_bytes(d->dtype), 256);
+}
+
+int64_t tk_lora_bwd_workspace_bytes(const tk_lora_desc* d) {
+  if (!d || d->rows < 0 || d->num_groups <= 0 || d->max_rank < 0 || d->max_rank > TK_MAX_RANK) return TK_ERR_INVALID;
+  return BwdLayout(*d).total;
+}
+
+int tk_lora_fwd(const tk_lora_desc* d, const void* x, int64_t ldx, void* y, int64_t ldy, void* h,
+                tk_stream_t stream) {
+  if (!desc_ok(d) || !h) return TK_ERR_INVALID;
+  if (d->rows == 0 || d->max_rank == 0) return TK_OK;
+  if (!x || !y || ldx < d->in_features || ldy < d->out_features) return TK_ERR_INVALID;
+  SegLayout L(d->rows, d->num_groups);
+  SegView V(d->seg_ws, L);
+  PassArgs a{};
+  a.src = x;  a.ld_src = ldx;
+  a.dst = y;  a.ld_dst = ldy;
+  a.hT = h;   a.ldh = h_ld(d->rows);
+  a.w_shrink = d->lora_A;  a.ld_shrink = d->lda;
+  a.w_expand = d->lora_B;  a.ld_expand = d->ldb;
+  a.rank = d->rank;  a.scale = d->scale;
+  a.width_src = d->in_features;  a.width_dst = d->out_features;
+  a.map_rows = d->map_rows;  a.rpad = rank_pad(d->max_rank);
+  return run_pass(a, V, L, d->dtype, (hipStream_t)stream);
+}
+
+int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void* x, int64_t ldx, const void* h,
+                void* dx, int64_t lddx, void* const* grad_A, void* const* grad_B, int32_t accumulate, void* ws,
+                int64_t ws_bytes, tk_stream_t stream) {
+  if (!desc_ok(d)) return TK_ERR_INVALID;
+  if (d->rows == 0 || d->max_rank == 0) return TK_OK;
+  if (!dy || lddy < d->out_features || !ws) return TK_ERR_INVALID;
+  if (dx && lddx < d->in_features) return TK_ERR_INVALID;
+  if (grad_A && (!x || ldx < d->in_features)) return TK_ERR_INVALID;
+  if (grad_B && !h) return TK_ERR_INVALID;
+  BwdLayout B(*d);
+  if (ws_bytes < B.total) return TK_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  SegLayout L(d->rows, d->num_groups);
+  SegView V(d->seg_ws, L);
+  char* w = (char*)ws;
+  void* dh = w + B.off_dh;
+  int rc;
+  if (dx || grad_A) {
+    void* bT = w + B.off_wT_shrink;
+    void* aT = w + B.off_wT_expand;
+    if ((rc = launch_transpose_weights(*d, bT, aT, s)) != TK_OK) return rc;
+    PassArgs a{};
+    a.src = dy;  a.ld_src = lddy;
+    a.dst = dx;  a.ld_dst = lddx;
+    a.hT = dh;   a.ldh = B.ldh;
+    a.w_shrink_base = bT;  a.ld_shrink = d->out_features;  a.shrink_group_stride = B.rpad * d->out_features;
+    a.w_expand_base = aT;  a.ld_expand = B.rpad;           a.expand_group_stride = B.rpad * d->in_features;
+    a.rank = d->rank;  a.scale = d->scale;
+    a.width_src = d->out_features;  a.width_dst = d->in_features;
+    a.map_rows = d->map_rows;  a.rpad = (int32_t)B.rpad;
+    if ((rc = run_pass(a, V, L, d->dtype, s)) != TK_OK) return rc;
+  }
+  if (grad_A) {
+    WgradArgs g{};
+    g.src = x;  g.ld_src = ldx;
+    g.hT = dh;  g.ldh = B.ldh;
+    g.partial = (float*)(w + B.off_part_a);
+    g.grad = grad_A;  g.ld_grad = d->lda;
+    g.rank = d->rank;  g.width = d->in_features;  g.transposed = 0;
+    g.accumulate = accumulate;  g.map_rows = d->map_rows;  g.rpad = (int32_t)B.rpad;
+    if ((rc = run_wgrad(g, V, L, d->dtype, s)) != TK_OK) return rc;
+  }
+  if (grad_B) {
+    WgradArgs g{};
+    g.src = dy;  g.ld_src = lddy;
+    g.hT = h;    g.ldh = B.ldh;
+    g.partial = (float*)(w + B.off_part_b);
+    g.grad = grad_B;  g.ld_grad = d->ldb;
+    g.rank = d->rank;  g.width = d->out_features;  g.transposed = 1;
+    g.accumulate = accumulate;  g.map_rows = d->map_rows;  g.rpad = (int32_t)B.rpad;
+    if ((rc = run_wgrad(g, V, L, d->dtype, s)) != TK_OK) return rc;
+  }
+  return TK_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,274 @@
+// Shape-agnostic kernels for the segmented LoRA pass: fp32 or bf16 storage,
+// fp32 accumulation on the vector ALUs, any width / stride / rank <= 128.
+// They carry the fp32 configuration and every shape the MFMA kernels do not
+// take (odd widths, unaligned strides), and share all buffers and tables with
+// them, so the two families are interchangeable per launch.
+#include <algorithm>
+
+#include "tk_device.h"
+
+namespace tk {
+
+namespace {
+
+constexpr int kKC = 64;   // source columns staged per step in the shrink kernel
+
+// hT[n][p] = scale_g * sum_k src[row(p)][k] * W_g[n][k]   for the rows of one tile
+template <typename T>
+__global__ __launch_bounds__(256) void k_shrink_generic(PassArgs a, const TileInfo* __restrict__ tiles,
+                                                        const int32_t* __restrict__ perm, const SegHeader* hdr) {
+  extern __shared__ float lds_f[];
+  const int tile_id = blockIdx.x;
+  if (tile_id >= hdr->num_tiles) return;
+  const TileInfo ti = tiles[tile_id];
+  const int g = ti.group;
+  const int r = min(a.rank[g], a.rpad);
+  const int rpad = a.rpad;
+  float* xs = lds_f;                          // [32][kKC + 1]
+  float* ws = lds_f + kTileRows * (kKC + 1);  // [rpad][kKC + 1]
+  __shared__ int rows_s[kTileRows];
+  const int tid = threadIdx.x;
+  if (tid < kTileRows) {
+    const int p = ti.start + min(tid, ti.count - 1);
+    rows_s[tid] = a.map_rows ? perm[p] : p;
+  }
+  __syncthreads();
+  const T* src = (const T*)a.src;
+  const T* W = group_weight<T>(a.w_shrink, a.w_shrink_base, a.shrink_group_stride, g);
+  const int row = tid & 31;   // tile row this thread accumulates
+  const int ng = tid >> 5;    // rank indices ng, ng + 8, ...
+  float acc[TK_MAX_RANK / 8];
+#pragma unroll
+  for (int j = 0; j < TK_MAX_RANK / 8; ++j) acc[j] = 0.f;
+  const int nacc = (rpad + 7) / 8;
+  for (int k0 = 0; k0 < a.width_src; k0 += kKC) {
+    for (int i = tid; i < kTileRows * kKC; i += 256) {
+      const int rr = i / kKC, kk = i % kKC;
+      const int k = k0 + kk;
+      xs[rr * (kKC + 1) + kk] = k < a.width_src ? to_f32(src[(int64_t)rows_s[rr] * a.ld_src + k]) : 0.f;
+    }
+    for (int i = tid; i < rpad * kKC; i += 256) {
+      const int n = i / kKC, kk = i % kKC;
+      const int k = k0 + kk;
+      ws[n * (kKC + 1) + kk] = (n < r && k < a.width_src) ? to_f32(W[(int64_t)n * a.ld_shrink + k]) : 0.f;
+    }
+    __syncthreads();
+    for (int kk = 0; kk < kKC; ++kk) {
+      const float xv = xs[row * (kKC + 1) + kk];
+#pragma unroll
+      for (int j = 0; j < TK_MAX_RANK / 8; ++j)
+        if (j < nacc) acc[j] += xv * ws[(ng + 8 * j) * (kKC + 1) + kk];
+    }
+    __syncthreads();
+  }
+  const float sc = a.scale[g];
+  T* hT = (T*)a.hT;
+  if (row < ti.count) {
+#pragma unroll
+    for (int j = 0; j < TK_MAX_RANK / 8; ++j) {
+      const int n = ng + 8 * j;
+      if (n < rpad) from_f32(n < r ? acc[j] * sc : 0.f, &hT[(int64_t)n * a.ldh + ti.start + row]);
+    }
+  }
+}
+
+// dst[row(p)][c] += sum_n hT[n][p] * W_g[c][n]   for the rows of one tile
+template <typename T>
+__global__ __launch_bounds__(256) void k_expand_generic(PassArgs a, const TileInfo* __restrict__ tiles,
+                                                        const int32_t* __restrict__ perm, const SegHeader* hdr) {
+  extern __shared__ float lds_f[];  // hs[rpad][32]
+  const int tile_id = blockIdx.x;
+  if (tile_id >= hdr->num_tiles) return;
+  const TileInfo ti = tiles[tile_id];
+  const int g = ti.group;
+  const int r = min(a.rank[g], a.rpad);
+  if (r <= 0) return;
+  __shared__ int rows_s[kTileRows];
+  const int tid = threadIdx.x;
+  if (tid < kTileRows) {
+    const int p = ti.start + min(tid, ti.count - 1);
+    rows_s[tid] = a.map_rows ? perm[p] : p;
+  }
+  const T* hT = (const T*)a.hT;
+  for (int i = tid; i < r * kTileRows; i += 256) {
+    const int n = i / kTileRows, rr = i % kTileRows;
+    lds_f[i] = rr < ti.count ? to_f32(hT[(int64_t)n * a.ldh + ti.start + rr]) : 0.f;
+  }
+  __syncthreads();
+  const T* W = group_weight<T>(a.w_expand, a.w_expand_base, a.expand_group_stride, g);
+  T* dst = (T*)a.dst;
+  for (int c = tid; c < a.width_dst; c += 256) {
+    float acc[kTileRows];
+#pragma unroll
+    for (int rr = 0; rr < kTileRows; ++rr) acc[rr] = 0.f;
+    const T* wrow = W + (int64_t)c * a.ld_expand;
+    for (int n = 0; n < r; ++n) {
+      const float b = to_f32(wrow[n]);
+#pragma unroll
+      for (int rr = 0; rr < kTileRows; ++rr) acc[rr] += lds_f[n * kTileRows + rr] * b;
+    }
+#pragma unroll
+    for (int rr = 0; rr < kTileRows; ++rr) {
+      if (rr < ti.count) {
+        T* o = dst + (int64_t)rows_s[rr] * a.ld_dst + c;
+        from_f32(to_f32(*o) + acc[rr], o);
+      }
+    }
+  }
+}
+
+template <typename T>
+__device__ inline void store_grad(const WgradArgs& a, int g, int n, int c, float v) {
+  T* gp = (T*)a.grad[g];
+  T* o = a.transposed ? gp + (int64_t)c * a.ld_grad + n : gp + (int64_t)n * a.ld_grad + c;
+  if (a.accumulate) v += to_f32(*o);
+  from_f32(v, o);
+}
+
+// One chunk of rows of one group, 256 columns per block:
+// out[n][c] = sum_{p in chunk} hT[n][p] * src[row(p)][c], p ascending.
+template <typename T>
+__global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkInfo* __restrict__ chunks,
+                                                       const int32_t* __restrict__ perm, const SegHeader* hdr) {
+  __shared__ float hs[16][kChunkRows];
+  __shared__ int rows_s[kChunkRows];
+  const int chunk_id = blockIdx.x;
+  if (chunk_id >= hdr->num_chunks) return;
+  const ChunkInfo ci = chunks[chunk_id];
+  const int g = ci.group;
+  const int r = min(a.rank[g], a.rpad);
+  if (r <= 0) return;
+  const int tid = threadIdx.x;
+  const int c = blockIdx.y * 256 + tid;
+  const int len = ci.end - ci.start;
+  for (int i = tid; i < len; i += 256) rows_s[i] = a.map_rows ? perm[ci.start + i] : ci.start + i;
+  const T* src = (const T*)a.src;
+  const T* hT = (const T*)a.hT;
+  for (int n0 = 0; n0 < r; n0 += 16) {
+    __syncthreads();
+    for (int i = tid; i < 16 * len; i += 256) {
+      const int j = i / len, pp = i % len;
+      hs[j][pp] = (n0 + j) < r ? to_f32(hT[(int64_t)(n0 + j) * a.ldh + ci.start + pp]) : 0.f;
+    }
+    __syncthreads();
+    if (c < a.width) {
+      float acc[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+      for (int pp = 0; pp < len; ++pp) {
+        const float xv = to_f32(src[(int64_t)rows_s[pp] * a.ld_src + c]);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[j] += hs[j][pp] * xv;
+      }
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int n = n0 + j;
+        if (n < r) {
+          if (ci.partial >= 0)
+            a.partial[((int64_t)ci.partial * a.rpad + n) * a.width + c] = acc[j];
+          else
+            store_grad<T>(a, g, n, c, acc[j]);
+        }
+      }
+    }
+  }
+}
+
+// Groups with several chunks: sum their partials in chunk order.  Groups with
+// no rows: clear the live block when overwriting.
+template <typename T>
+__global__ __launch_bounds__(256) void k_wgrad_reduce(WgradArgs a, const int32_t* __restrict__ chunk_first,
+                                                      const int32_t* __restrict__ partial_first) {
+  const int g = blockIdx.x;
+  const int r = min(a.rank[g], a.rpad);
+  if (r <= 0) return;
+  const int nchunk = chunk_first[g + 1] - chunk_first[g];
+  if (nchunk == 1) return;
+  if (nchunk == 0 && a.accumulate) return;
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= a.width) return;
+  const int p0 = partial_first[g];
+  for (int n = 0; n < r; ++n) {
+    float acc = 0.f;
+    for (int j = 0; j < nchunk; ++j) acc += a.partial[((int64_t)(p0 + j) * a.rpad + n) * a.width + c];
+    store_grad<T>(a, g, n, c, acc);
+  }
+}
+
+// bT_g[n][m] = B_g[m][n], aT_g[k][n] = A_g[n][k]; zero for n >= rank[g].
+template <typename T>
+__global__ __launch_bounds__(256) void k_transpose_weights(tk_lora_desc d, int rpad, T* __restrict__ bT,
+                                                           T* __restrict__ aT) {
+  const int g = blockIdx.y;
+  const int r = min(d.rank[g], rpad);
+  const T* A = (const T*)d.lora_A[g];
+  const T* B = (const T*)d.lora_B[g];
+  const int64_t nb = (int64_t)rpad * d.out_features, na = (int64_t)rpad * d.in_features;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nb + na; i += (int64_t)gridDim.x * 256) {
+    if (i < nb) {
+      const int n = (int)(i / d.out_features), m = (int)(i % d.out_features);
+      bT[(int64_t)g * nb + i] = n < r ? B[(int64_t)m * d.ldb + n] : (T)0;
+    } else {
+      const int64_t q = i - nb;
+      const int k = (int)(q / rpad), n = (int)(q % rpad);
+      aT[(int64_t)g * na + q] = n < r ? A[(int64_t)n * d.lda + k] : (T)0;
+    }
+  }
+}
+
+}  // namespace
+
+int launch_pass_generic(const PassArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s) {
+  if (L.rows == 0) return TK_OK;
+  const unsigned grid = (unsigned)L.max_tiles;
+  const size_t lds_shrink = sizeof(float) * (size_t)(kTileRows + a.rpad) * (kKC + 1);
+  const size_t lds_expand = sizeof(float) * (size_t)a.rpad * kTileRows;
+  if (dtype == TK_DTYPE_F32) {
+    hipLaunchKernelGGL(k_shrink_generic<float>, dim3(grid), dim3(256), lds_shrink, s, a, seg.tiles, seg.perm,
+                       seg.header);
+    if (a.dst)
+      hipLaunchKernelGGL(k_expand_generic<float>, dim3(grid), dim3(256), lds_expand, s, a, seg.tiles, seg.perm,
+                         seg.header);
+  } else {
+    hipLaunchKernelGGL(k_shrink_generic<bf16_t>, dim3(grid), dim3(256), lds_shrink, s, a, seg.tiles, seg.perm,
+                       seg.header);
+    if (a.dst)
+      hipLaunchKernelGGL(k_expand_generic<bf16_t>, dim3(grid), dim3(256), lds_expand, s, a, seg.tiles, seg.perm,
+                         seg.header);
+  }
+  return check_launch();
+}
+
+int launch_wgrad_generic(const WgradArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s) {
+  if (L.rows == 0) return TK_OK;
+  const dim3 grid((unsigned)L.max_chunks, (unsigned)ceil_div(a.width, 256));
+  if (dtype == TK_DTYPE_F32)
+    hipLaunchKernelGGL(k_wgrad_generic<float>, grid, dim3(256), 0, s, a, seg.chunks, seg.perm, seg.header);
+  else
+    hipLaunchKernelGGL(k_wgrad_generic<bf16_t>, grid, dim3(256), 0, s, a, seg.chunks, seg.perm, seg.header);
+  return check_launch();
+}
+
+int launch_wgrad_reduce(const WgradArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s) {
+  if (L.groups == 0) return TK_OK;
+  const dim3 grid((unsigned)L.groups, (unsigned)ceil_div(a.width, 256));
+  if (dtype == TK_DTYPE_F32)
+    hipLaunchKernelGGL(k_wgrad_reduce<float>, grid, dim3(256), 0, s, a, seg.chunk_first, seg.partial_first);
+  else
+    hipLaunchKernelGGL(k_wgrad_reduce<bf16_t>, grid, dim3(256), 0, s, a, seg.chunk_first, seg.partial_first);
+  return check_launch();
+}
+
+int launch_transpose_weights(const tk_lora_desc& d, void* bT, void* aT, hipStream_t s) {
+  if (d.num_groups == 0) return TK_OK;
+  const int rpad = rank_pad(d.max_rank);
+  const int64_t per_group = (int64_t)rpad * (d.out_features + d.in_features);
+  const dim3 grid((unsigned)std::min<int64_t>(ceil_div(per_group, 256), 64), (unsigned)d.num_groups);
+  if (d.dtype == TK_DTYPE_F32)
+    hipLaunchKernelGGL(k_transpose_weights<float>, grid, dim3(256), 0, s, d, rpad, (float*)bT, (float*)aT);
+  else
+    hipLaunchKernelGGL(k_transpose_weights<bf16_t>, grid, dim3(256), 0, s, d, rpad, (bf16_t*)bT, (bf16_t*)aT);
+  return check_launch();
+}
+
+}  // namespace tk

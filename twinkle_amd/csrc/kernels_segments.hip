@@ -1,0 +1,355 @@
+// Segment builder (stable counting sort of rows by group) and the row
+// gather / scatter-back kernels that use its table.  Integer work, HBM-light:
+// the table is built once per batch and read by every LoRA layer.
+//
+// Pipeline (no host synchronisation anywhere):
+//   k_seg_hist    one wave per 512 rows: LDS histogram -> hist[block][group]
+//   k_seg_scan    one block: per-group totals, exclusive scans -> offsets,
+//                 tile/chunk tables' firsts, per-block bases (in place in hist)
+//   k_seg_scatter one wave per 512 rows: stable rank inside the wave by
+//                 bit-sliced ballots, cursor per group in LDS -> perm, inv
+//   k_seg_fill    one thread per tile / chunk slot: binary search of its group
+#include "tk_device.h"
+
+namespace tk {
+
+namespace {
+
+template <typename KeyT>
+__device__ inline int load_key(const KeyT* keys, int64_t f, int groups, int* bad) {
+  long long k = (long long)keys[f];
+  if (k < 0 || k >= groups) {
+    *bad += 1;
+    k = k < 0 ? 0 : groups - 1;
+  }
+  return (int)k;
+}
+
+template <typename KeyT>
+__global__ __launch_bounds__(64) void k_seg_hist(const KeyT* __restrict__ keys, int rows, int groups,
+                                                 int32_t* __restrict__ hist, SegHeader* hdr) {
+  extern __shared__ int32_t lds[];
+  const int lane = threadIdx.x;
+  const int blk = blockIdx.x;
+  for (int g = lane; g < groups; g += 64) lds[g] = 0;
+  __syncthreads();
+  int bad = 0;
+  const int64_t base = (int64_t)blk * kSortBlockRows;
+#pragma unroll
+  for (int s = 0; s < kSortBlockRows / 64; ++s) {
+    const int64_t f = base + s * 64 + lane;
+    if (f < rows) atomicAdd(&lds[load_key(keys, f, groups, &bad)], 1);
+  }
+  __syncthreads();
+  for (int g = lane; g < groups; g += 64) hist[(int64_t)blk * groups + g] = lds[g];
+  if (bad) atomicAdd(&hdr->bad_keys, bad);
+}
+
+// Exclusive scan of one value per thread over a 1024-thread block.
+__device__ inline int block_exclusive_scan(int v, int* wave_sums, int* total) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int incl = v;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    int o = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += o;
+  }
+  if (lane == 63) wave_sums[wave] = incl;
+  __syncthreads();
+  if (wave == 0) {
+    int w = lane < 16 ? wave_sums[lane] : 0;
+    int wi = w;
+#pragma unroll
+    for (int d = 1; d < 16; d <<= 1) {
+      int o = __shfl_up(wi, d, 64);
+      if (lane >= d) wi += o;
+    }
+    if (lane < 16) wave_sums[lane] = wi - w;  // exclusive base of each wave
+    if (lane == 15) wave_sums[16] = wi;        // block total
+  }
+  __syncthreads();
+  const int res = wave_sums[wave] + incl - v;
+  *total = wave_sums[16];
+  __syncthreads();
+  return res;
+}
+
+__global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sort_blocks, int32_t* __restrict__ hist,
+                                                   int32_t* __restrict__ offsets, int32_t* __restrict__ tile_first,
+                                                   int32_t* __restrict__ chunk_first,
+                                                   int32_t* __restrict__ partial_first,
+                                                   int64_t* __restrict__ offsets_out, SegHeader* hdr) {
+  __shared__ int wave_sums[17];
+  int carry_rows = 0, carry_tiles = 0, carry_chunks = 0, carry_part = 0;
+  for (int g0 = 0; g0 < groups; g0 += 1024) {
+    const int g = g0 + threadIdx.x;
+    int count = 0;
+    if (g < groups) {
+      // per-block counts -> per-block exclusive bases (relative to the group's start)
+      for (int b = 0; b < sort_blocks; ++b) {
+        const int64_t i = (int64_t)b * groups + g;
+        const int c = hist[i];
+        hist[i] = count;
+        count += c;
+      }
+    }
+    const int ntile = (count + kTileRows - 1) / kTileRows;
+    const int nchunk = (count + kChunkRows - 1) / kChunkRows;
+    const int npart = nchunk > 1 ? nchunk : 0;
+    int tot;
+    const int e_rows = block_exclusive_scan(count, wave_sums, &tot) + carry_rows;
+    carry_rows += tot;
+    const int e_tiles = block_exclusive_scan(ntile, wave_sums, &tot) + carry_tiles;
+    carry_tiles += tot;
+    const int e_chunks = block_exclusive_scan(nchunk, wave_sums, &tot) + carry_chunks;
+    carry_chunks += tot;
+    const int e_part = block_exclusive_scan(npart, wave_sums, &tot) + carry_part;
+    carry_part += tot;
+    if (g < groups) {
+      offsets[g] = e_rows;
+      tile_first[g] = e_tiles;
+      chunk_first[g] = e_chunks;
+      partial_first[g] = e_part;
+      if (offsets_out) offsets_out[g] = e_rows;
+    }
+  }
+  if (threadIdx.x == 0) {
+    offsets[groups] = carry_rows;
+    tile_first[groups] = carry_tiles;
+    chunk_first[groups] = carry_chunks;
+    partial_first[groups] = carry_part;
+    if (offsets_out) offsets_out[groups] = carry_rows;
+    hdr->magic = kSegMagic;
+    hdr->rows = rows;
+    hdr->groups = groups;
+    hdr->num_tiles = carry_tiles;
+    hdr->num_chunks = carry_chunks;
+    hdr->num_partials = carry_part;
+  }
+}
+
+template <typename KeyT>
+__global__ __launch_bounds__(64) void k_seg_scatter(const KeyT* __restrict__ keys, int rows, int groups, int key_bits,
+                                                    const int32_t* __restrict__ hist,
+                                                    const int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
+                                                    int32_t* __restrict__ inv, int64_t* __restrict__ perm_out) {
+  extern __shared__ int32_t cursor[];
+  const int lane = threadIdx.x;
+  const int blk = blockIdx.x;
+  for (int g = lane; g < groups; g += 64) cursor[g] = offsets[g] + hist[(int64_t)blk * groups + g];
+  __syncthreads();
+  const int64_t base = (int64_t)blk * kSortBlockRows;
+  int unused = 0;
+  for (int s = 0; s < kSortBlockRows / 64; ++s) {
+    const int64_t f = base + s * 64 + lane;
+    const bool valid = f < rows;
+    const int key = valid ? load_key(keys, f, groups, &unused) : 0;
+    // lanes of this wave that hold the same key
+    unsigned long long same = __ballot(valid);
+    for (int b = 0; b < key_bits; ++b) {
+      const bool bit = (key >> b) & 1;
+      const unsigned long long m = __ballot(valid && bit);
+      same &= bit ? m : ~m;
+    }
+    const unsigned long long below = same & ((1ull << lane) - 1ull);
+    const int rank = __popcll(below);
+    int pos = 0;
+    if (valid) pos = cursor[key] + rank;
+    __syncthreads();
+    if (valid && rank == 0) cursor[key] += __popcll(same);
+    __syncthreads();
+    if (valid) {
+      perm[pos] = (int32_t)f;
+      inv[f] = pos;
+      if (perm_out) perm_out[pos] = f;
+    }
+  }
+}
+
+__device__ inline int group_of(const int32_t* first, int groups, int i) {
+  // largest g with first[g] <= i (first is non-decreasing, first[groups] > i)
+  int lo = 0, hi = groups;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (first[mid] <= i) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+__global__ __launch_bounds__(256) void k_seg_fill(int groups, int max_tiles, int max_chunks,
+                                                  const int32_t* __restrict__ offsets,
+                                                  const int32_t* __restrict__ tile_first,
+                                                  const int32_t* __restrict__ chunk_first,
+                                                  const int32_t* __restrict__ partial_first,
+                                                  TileInfo* __restrict__ tiles, ChunkInfo* __restrict__ chunks) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < max_tiles) {
+    TileInfo t{-1, 0, 0, 0};
+    if (i < tile_first[groups]) {
+      const int g = group_of(tile_first, groups, i);
+      const int j = i - tile_first[g];
+      t.group = g;
+      t.start = offsets[g] + j * kTileRows;
+      t.count = min(kTileRows, offsets[g + 1] - t.start);
+    }
+    tiles[i] = t;
+  }
+  if (i < max_chunks) {
+    ChunkInfo c{-1, 0, 0, -1};
+    if (i < chunk_first[groups]) {
+      const int g = group_of(chunk_first, groups, i);
+      const int j = i - chunk_first[g];
+      const int n = chunk_first[g + 1] - chunk_first[g];
+      c.group = g;
+      c.start = offsets[g] + j * kChunkRows;
+      c.end = min(c.start + kChunkRows, offsets[g + 1]);
+      c.partial = n > 1 ? partial_first[g] + j : -1;
+    }
+    chunks[i] = c;
+  }
+}
+
+__global__ void k_seg_clear(SegHeader* hdr) {
+  if (threadIdx.x < 64) ((int32_t*)hdr)[threadIdx.x] = 0;
+}
+
+// ---- row gather / scatter-back -------------------------------------------------
+
+// dst[j] = src[perm[j] mod tokens] * w[token, k]
+template <typename T>
+__global__ __launch_bounds__(256) void k_permute(const T* __restrict__ src, int64_t ld_src, T* __restrict__ dst,
+                                                 int64_t ld_dst, const T* __restrict__ w,
+                                                 const int32_t* __restrict__ perm, int rows, int tokens, int top_k,
+                                                 int width) {
+  const int j = blockIdx.x;
+  if (j >= rows) return;
+  const int f = perm[j];
+  const int t = f % tokens, k = f / tokens;
+  const T* s = src + (int64_t)t * ld_src;
+  T* d = dst + (int64_t)j * ld_dst;
+  if (w) {
+    const float wt = to_f32(w[(int64_t)t * top_k + k]);
+    for (int c = threadIdx.x; c < width; c += 256) from_f32(to_f32(s[c]) * wt, &d[c]);
+  } else {
+    for (int c = threadIdx.x; c < width; c += 256) d[c] = s[c];
+  }
+}
+
+// out[t] = sum_k rows[inv[k * tokens + t]] * w[t, k], k ascending, fp32 accumulation
+template <typename T>
+__global__ __launch_bounds__(256) void k_unpermute(const T* __restrict__ rows_, int64_t ld_rows, T* __restrict__ out,
+                                                   int64_t ld_out, const T* __restrict__ w,
+                                                   const int32_t* __restrict__ inv, int tokens, int top_k, int width) {
+  const int t = blockIdx.x;
+  if (t >= tokens) return;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float acc = 0.f;
+    for (int k = 0; k < top_k; ++k) {
+      const int j = inv[(int64_t)k * tokens + t];
+      float v = to_f32(rows_[(int64_t)j * ld_rows + c]);
+      if (w) {
+        // the reference scales the row in the activation dtype before adding (ep_utils.py:142)
+        T r;
+        from_f32(v * to_f32(w[(int64_t)t * top_k + k]), &r);
+        v = to_f32(r);
+      }
+      acc += v;
+    }
+    from_f32(acc, &out[(int64_t)t * ld_out + c]);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(64) void k_unpermute_wgrad(const T* __restrict__ dout, int64_t ld_dout,
+                                                        const T* __restrict__ rows_, int64_t ld_rows,
+                                                        float* __restrict__ dw, const int32_t* __restrict__ inv,
+                                                        int tokens, int top_k, int width) {
+  const int f = blockIdx.x;  // flat row k * tokens + t
+  const int t = f % tokens, k = f / tokens;
+  const int j = inv[f];
+  float acc = 0.f;
+  for (int c = threadIdx.x; c < width; c += 64)
+    acc += to_f32(dout[(int64_t)t * ld_dout + c]) * to_f32(rows_[(int64_t)j * ld_rows + c]);
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d, 64);
+  if (threadIdx.x == 0) dw[(int64_t)t * top_k + k] = acc;
+}
+
+}  // namespace
+
+int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t groups, int64_t* perm_out,
+                         int64_t* offsets_out, void* ws, hipStream_t s) {
+  SegLayout L(rows, groups);
+  SegView V(ws, L);
+  const int nblk = (int)L.sort_blocks;
+  const size_t lds = sizeof(int32_t) * (size_t)groups;
+  int key_bits = 0;
+  while ((1 << key_bits) < groups) ++key_bits;
+  hipLaunchKernelGGL(k_seg_clear, dim3(1), dim3(64), 0, s, V.header);
+  if (key_dtype == TK_KEY_I32)
+    hipLaunchKernelGGL(k_seg_hist<int32_t>, dim3(nblk), dim3(64), lds, s, (const int32_t*)keys, (int)rows, groups,
+                       V.hist, V.header);
+  else
+    hipLaunchKernelGGL(k_seg_hist<int64_t>, dim3(nblk), dim3(64), lds, s, (const int64_t*)keys, (int)rows, groups,
+                       V.hist, V.header);
+  hipLaunchKernelGGL(k_seg_scan, dim3(1), dim3(1024), 0, s, (int)rows, groups, nblk, V.hist, V.offsets, V.tile_first,
+                     V.chunk_first, V.partial_first, offsets_out, V.header);
+  if (key_dtype == TK_KEY_I32)
+    hipLaunchKernelGGL(k_seg_scatter<int32_t>, dim3(nblk), dim3(64), lds, s, (const int32_t*)keys, (int)rows, groups,
+                       key_bits, V.hist, V.offsets, V.perm, V.inv, perm_out);
+  else
+    hipLaunchKernelGGL(k_seg_scatter<int64_t>, dim3(nblk), dim3(64), lds, s, (const int64_t*)keys, (int)rows, groups,
+                       key_bits, V.hist, V.offsets, V.perm, V.inv, perm_out);
+  const int fill = (int)(L.max_tiles > L.max_chunks ? L.max_tiles : L.max_chunks);
+  hipLaunchKernelGGL(k_seg_fill, dim3((fill + 255) / 256), dim3(256), 0, s, groups, (int)L.max_tiles,
+                     (int)L.max_chunks, V.offsets, V.tile_first, V.chunk_first, V.partial_first, V.tiles, V.chunks);
+  return check_launch();
+}
+
+int launch_permute(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, const void* w, const void* ws,
+                   int64_t rows, int64_t tokens, int32_t width, int32_t groups, int dtype, hipStream_t s) {
+  if (rows == 0) return TK_OK;
+  SegLayout L(rows, groups);
+  SegView V(ws, L);
+  const int top_k = (int)(rows / tokens);
+  if (dtype == TK_DTYPE_F32)
+    hipLaunchKernelGGL(k_permute<float>, dim3((unsigned)rows), dim3(256), 0, s, (const float*)src, ld_src,
+                       (float*)dst, ld_dst, (const float*)w, V.perm, (int)rows, (int)tokens, top_k, width);
+  else
+    hipLaunchKernelGGL(k_permute<uint16_t>, dim3((unsigned)rows), dim3(256), 0, s, (const uint16_t*)src, ld_src,
+                       (uint16_t*)dst, ld_dst, (const uint16_t*)w, V.perm, (int)rows, (int)tokens, top_k, width);
+  return check_launch();
+}
+
+int launch_unpermute(const void* rows_, int64_t ld_rows, void* out, int64_t ld_out, const void* w, const void* ws,
+                     int64_t rows, int64_t tokens, int32_t width, int32_t groups, int dtype, hipStream_t s) {
+  if (tokens == 0) return TK_OK;
+  SegLayout L(rows, groups);
+  SegView V(ws, L);
+  const int top_k = (int)(rows / tokens);
+  if (dtype == TK_DTYPE_F32)
+    hipLaunchKernelGGL(k_unpermute<float>, dim3((unsigned)tokens), dim3(256), 0, s, (const float*)rows_, ld_rows,
+                       (float*)out, ld_out, (const float*)w, V.inv, (int)tokens, top_k, width);
+  else
+    hipLaunchKernelGGL(k_unpermute<uint16_t>, dim3((unsigned)tokens), dim3(256), 0, s, (const uint16_t*)rows_,
+                       ld_rows, (uint16_t*)out, ld_out, (const uint16_t*)w, V.inv, (int)tokens, top_k, width);
+  return check_launch();
+}
+
+int launch_unpermute_wgrad(const void* dout, int64_t ld_dout, const void* rows_, int64_t ld_rows, float* dw,
+                           const void* ws, int64_t rows, int64_t tokens, int32_t width, int32_t groups, int dtype,
+                           hipStream_t s) {
+  if (rows == 0) return TK_OK;
+  SegLayout L(rows, groups);
+  SegView V(ws, L);
+  const int top_k = (int)(rows / tokens);
+  if (dtype == TK_DTYPE_F32)
+    hipLaunchKernelGGL(k_unpermute_wgrad<float>, dim3((unsigned)rows), dim3(64), 0, s, (const float*)dout, ld_dout,
+                       (const float*)rows_, ld_rows, dw, V.inv, (int)tokens, top_k, width);
+  else
+    hipLaunchKernelGGL(k_unpermute_wgrad<uint16_t>, dim3((unsigned)rows), dim3(64), 0, s, (const uint16_t*)dout,
+                       ld_dout, (const uint16_t*)rows_, ld_rows, dw, V.inv, (int)tokens, top_k, width);
+  return check_launch();
+}
+
+}  // namespace tk

@@ -1,0 +1,189 @@
+// Internal definitions shared by the gfx950 kernels and the C-ABI glue.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "twinkle_amd.h"
+
+namespace tk {
+
+constexpr int kWave = 64;
+constexpr int kTileRows = TK_TILE_ROWS;    // rows per forward tile (two 16-row MFMA tiles)
+constexpr int kChunkRows = TK_CHUNK_ROWS;  // rows per weight-gradient chunk (split over rows)
+constexpr int kSortBlockRows = 512;        // rows one single-wave block orders in the scatter pass
+
+static inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---------------------------------------------------------------------------
+// Device-side segment table.  One allocation, carved by SegLayout from
+// (rows, groups) alone, so producer and consumers agree without a host copy.
+// ---------------------------------------------------------------------------
+struct SegHeader {       // 64 x int32, at the start of the workspace
+  int32_t magic;
+  int32_t rows;
+  int32_t groups;
+  int32_t num_tiles;     // filled on the device
+  int32_t num_chunks;    // filled on the device
+  int32_t num_partials;  // chunks that belong to multi-chunk groups
+  int32_t bad_keys;      // keys outside [0, groups), clamped
+  int32_t pad[57];
+};
+
+struct TileInfo {   // one forward tile: rows [start, start + count) of group `group`
+  int32_t group;
+  int32_t start;
+  int32_t count;
+  int32_t pad;
+};
+
+struct ChunkInfo {  // one weight-gradient chunk: sorted rows [start, end) of group `group`
+  int32_t group;
+  int32_t start;
+  int32_t end;
+  int32_t partial;  // slot in the partial buffer, or -1 when the chunk is its group's only one
+};
+
+struct SegLayout {
+  int64_t rows, groups;
+  int64_t sort_blocks;   // ceil(rows / kSortBlockRows)
+  int64_t max_tiles, max_chunks, max_partials;
+  // byte offsets from the workspace base
+  int64_t off_perm, off_inv, off_offsets, off_tiles, off_chunks, off_tile_first, off_chunk_first, off_partial_first,
+      off_hist, total;
+
+  SegLayout(int64_t rows_, int64_t groups_) : rows(rows_), groups(groups_) {
+    sort_blocks = ceil_div(rows > 0 ? rows : 1, kSortBlockRows);
+    max_tiles = ceil_div(rows, kTileRows) + groups;
+    max_chunks = ceil_div(rows, kChunkRows) + groups;
+    max_partials = 2 * ceil_div(rows, kChunkRows) + 1;
+    int64_t o = round_up(sizeof(SegHeader), 256);
+    off_perm = o;         o += round_up(4 * (rows + 64), 256);
+    off_inv = o;          o += round_up(4 * (rows + 64), 256);
+    off_offsets = o;      o += round_up(4 * (groups + 1), 256);
+    off_tiles = o;        o += round_up(16 * (max_tiles + 1), 256);
+    off_chunks = o;       o += round_up(16 * (max_chunks + 1), 256);
+    off_tile_first = o;   o += round_up(4 * (groups + 1), 256);
+    off_chunk_first = o;  o += round_up(4 * (groups + 1), 256);
+    off_partial_first = o; o += round_up(4 * (groups + 1), 256);
+    off_hist = o;         o += round_up(4 * groups * sort_blocks, 256);
+    total = o;
+  }
+};
+
+struct SegView {  // typed device pointers into a segment workspace
+  SegHeader* header;
+  int32_t* perm;         // [rows]   sorted position -> flat row
+  int32_t* inv;          // [rows]   flat row -> sorted position
+  int32_t* offsets;      // [G + 1]
+  TileInfo* tiles;       // [max_tiles]
+  ChunkInfo* chunks;     // [max_chunks]
+  int32_t* tile_first;     // [G + 1]  first tile of each group
+  int32_t* chunk_first;    // [G + 1]  first chunk of each group
+  int32_t* partial_first;  // [G + 1]  first partial slot of each multi-chunk group
+  int32_t* hist;           // [sort_blocks][G]  per-block histogram, then per-block exclusive bases
+  SegView(const void* base, const SegLayout& L) {
+    char* b = (char*)base;
+    header = (SegHeader*)b;
+    perm = (int32_t*)(b + L.off_perm);
+    inv = (int32_t*)(b + L.off_inv);
+    offsets = (int32_t*)(b + L.off_offsets);
+    tiles = (TileInfo*)(b + L.off_tiles);
+    chunks = (ChunkInfo*)(b + L.off_chunks);
+    tile_first = (int32_t*)(b + L.off_tile_first);
+    chunk_first = (int32_t*)(b + L.off_chunk_first);
+    partial_first = (int32_t*)(b + L.off_partial_first);
+    hist = (int32_t*)(b + L.off_hist);
+  }
+};
+
+constexpr int32_t kSegMagic = 0x544b5347;  // "TKSG"
+
+// ---------------------------------------------------------------------------
+// Saved shrink output.  hT[n][p]: rank index major, sorted position minor, so
+// the row-contraction kernels read 8 consecutive positions per lane.
+// ---------------------------------------------------------------------------
+static inline int64_t h_ld(int64_t rows) { return round_up(rows > 0 ? rows : 1, 64); }
+static inline int32_t rank_pad(int32_t max_rank) { return (int32_t)round_up(max_rank > 0 ? max_rank : 1, 16); }
+static inline int elt_bytes(int dtype) { return dtype == TK_DTYPE_BF16 ? 2 : 4; }
+
+// Backward workspace carving.
+struct BwdLayout {
+  int64_t off_dh, off_wT_shrink, off_wT_expand, off_part_a, off_part_b, total;
+  int64_t rpad, ldh;
+  BwdLayout(const tk_lora_desc& d) {
+    SegLayout S(d.rows, d.num_groups);
+    rpad = rank_pad(d.max_rank);
+    ldh = h_ld(d.rows);
+    const int64_t e = elt_bytes(d.dtype);
+    int64_t o = 0;
+    off_dh = o;         o += round_up(rpad * ldh * e, 256);
+    // B^T per group [rpad][M]  (shrink weight of the backward pass)
+    off_wT_shrink = o;  o += round_up((int64_t)d.num_groups * rpad * d.out_features * e, 256);
+    // A^T per group [K][rpad]  (expand weight of the backward pass)
+    off_wT_expand = o;  o += round_up((int64_t)d.num_groups * rpad * d.in_features * e, 256);
+    off_part_a = o;     o += round_up(S.max_partials * rpad * (int64_t)d.in_features * 4, 256);
+    off_part_b = o;     o += round_up(S.max_partials * rpad * (int64_t)d.out_features * 4, 256);
+    total = o;
+  }
+};
+
+// Everything one pass of the (shrink, expand) pair needs.  The forward pass
+// and the input-gradient pass are the same computation with the roles of the
+// weights swapped, so both are described by this one struct.
+struct PassArgs {
+  const void* src;   int64_t ld_src;   // rows that are shrunk     (x  | dy)
+  void* dst;         int64_t ld_dst;   // rows that are updated    (y  | dx), may be null
+  void* hT;          int64_t ldh;      // shrink output            (h  | dh), written
+  // shrink weight of group g: rank-major [r][width_src]
+  const void* const* w_shrink;  const void* w_shrink_base;  int64_t ld_shrink;  int64_t shrink_group_stride;
+  // expand weight of group g: column-major-by-output [width_dst][r]
+  const void* const* w_expand;  const void* w_expand_base;  int64_t ld_expand;  int64_t expand_group_stride;
+  const int32_t* rank;
+  const float* scale;
+  int32_t width_src;  // K | M
+  int32_t width_dst;  // M | K
+  int32_t map_rows;
+  int32_t rpad;
+};
+
+// Row-contraction (weight gradient) pass: out_g[n][c] = sum_p hT[n][p] * src[row(p)][c].
+struct WgradArgs {
+  const void* src;  int64_t ld_src;   // x | dy
+  const void* hT;   int64_t ldh;      // dh | h
+  float* partial;                     // [max_partials][rpad][width]
+  void* const* grad;                  // device array [G]
+  int64_t ld_grad;
+  const int32_t* rank;
+  int32_t width;       // K | M
+  int32_t transposed;  // 0: grad_g is [r][width] (dA); 1: grad_g is [width][r] (dB)
+  int32_t accumulate;
+  int32_t map_rows;
+  int32_t rpad;
+};
+
+// kernels_segments.hip
+int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t groups, int64_t* perm_out,
+                         int64_t* offsets_out, void* ws, hipStream_t s);
+int launch_permute(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, const void* w, const void* ws,
+                   int64_t rows, int64_t tokens, int32_t width, int32_t groups, int dtype, hipStream_t s);
+int launch_unpermute(const void* rows_, int64_t ld_rows, void* out, int64_t ld_out, const void* w, const void* ws,
+                     int64_t rows, int64_t tokens, int32_t width, int32_t groups, int dtype, hipStream_t s);
+int launch_unpermute_wgrad(const void* dout, int64_t ld_dout, const void* rows_, int64_t ld_rows, float* dw,
+                           const void* ws, int64_t rows, int64_t tokens, int32_t width, int32_t groups, int dtype,
+                           hipStream_t s);
+
+// kernels_generic.hip : any shape / stride, fp32 and bf16, VALU
+int launch_pass_generic(const PassArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s);
+int launch_wgrad_generic(const WgradArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s);
+int launch_wgrad_reduce(const WgradArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s);
+int launch_transpose_weights(const tk_lora_desc& d, void* bT, void* aT, hipStream_t s);
+
+// kernels_mfma.hip : bf16, aligned shapes, MFMA
+bool pass_mfma_supported(const PassArgs& a);
+int launch_pass_mfma(const PassArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
+bool wgrad_mfma_supported(const WgradArgs& a);
+int launch_wgrad_mfma(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
+
+}  // namespace tk

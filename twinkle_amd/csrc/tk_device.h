@@ -1,0 +1,31 @@
+// Device-side helpers shared by the kernel translation units.
+#pragma once
+
+#include "tk_common.h"
+
+namespace tk {
+
+typedef uint16_t bf16_t;  // raw bfloat16 bits
+
+__device__ inline float to_f32(float v) { return v; }
+__device__ inline float to_f32(bf16_t v) { return __uint_as_float((uint32_t)v << 16); }
+
+__device__ inline bf16_t f32_to_bf16(float v) {
+  uint32_t u = __float_as_uint(v);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);  // NaN stays NaN
+  u += 0x7fffu + ((u >> 16) & 1u);                                         // round to nearest even
+  return (bf16_t)(u >> 16);
+}
+__device__ inline void from_f32(float v, float* o) { *o = v; }
+__device__ inline void from_f32(float v, bf16_t* o) { *o = f32_to_bf16(v); }
+
+// Weight of group g: either a per-group pointer (caller-owned slot tensors)
+// or base + g * stride (a packed copy inside a workspace).
+template <typename T>
+__device__ inline const T* group_weight(const void* const* ptrs, const void* base, int64_t stride, int g) {
+  return ptrs ? (const T*)ptrs[g] : (const T*)base + (int64_t)g * stride;
+}
+
+inline int check_launch() { return hipGetLastError() == hipSuccess ? TK_OK : TK_ERR_LAUNCH; }
+
+}  // namespace tk

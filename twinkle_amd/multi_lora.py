@@ -1,0 +1,399 @@
+"""Slot pool, tenant bookkeeping and the patched LoRA forward, on the HIP kernels.
+
+Host-side mirror of ``twinkle.model.multi_lora.MultiLora``
+(src/twinkle/model/multi_lora.py): same method names, argument meaning and
+exceptions, so that code written against the reference's class runs unchanged.
+Two things differ underneath:
+
+* the LoRA arithmetic of the patched forward (reference :315-326) runs in the
+  segmented HIP kernels instead of two ``F.linear`` calls, and
+* :meth:`MultiLora.batch` widens :meth:`MultiLora.adapter` from one adapter per
+  call to one adapter per row, so that many tenants share one forward/backward.
+  ``adapter(name)`` is the one-segment special case and needs no change in callers.
+"""
+from __future__ import annotations
+
+import re
+from contextlib import contextmanager
+from dataclasses import dataclass, field
+from types import MethodType
+from typing import Any, Dict, List, Optional, Sequence, Union
+
+import torch
+
+from .lora_layer import LoraConfig, LoraLinear, LoraModel, inject_adapter
+from .ops import AdapterGroups, multi_lora_delta, multi_lora_linear
+from .segments import SegmentTable, build_segments
+
+
+@dataclass
+class LoraTenant:
+    """One pre-allocated slot and the tenant that holds it (reference :20-28)."""
+    index: int
+    adapter_name: str
+    config: Any
+    tenant_adapter_name: Optional[str] = None
+    tenant_config: Optional[Any] = None
+    lora_A_weights: Dict[str, torch.Tensor] = field(default_factory=dict)
+
+
+def _is_lora_layer(module) -> bool:
+    return all(hasattr(module, a) for a in ('base_layer', 'lora_A', 'lora_B', 'lora_dropout'))
+
+
+class MultiLora:
+
+    def __init__(self, max_loras=5, max_r=32, max_length: int = 8192):
+        self.max_loras = max_loras
+        self.max_r = max_r
+        self.max_length = max_length
+        self.loras: List[LoraTenant] = []
+        self.module = None
+        self._version = 0                 # bumped whenever slot ownership changes
+        self._layer_groups: Dict[int, tuple] = {}
+        self._batch_table: Optional[SegmentTable] = None
+        self._uniform_tables: Dict[tuple, SegmentTable] = {}
+
+    # ------------------------------------------------------------------ slots
+    def _get_available_lora(self) -> Optional[LoraTenant]:
+        return next((t for t in self.loras if t.tenant_adapter_name is None), None)
+
+    def _count_available_loras(self) -> int:
+        return sum(1 for t in self.loras if t.tenant_adapter_name is None)
+
+    def has_lora(self, adapter_name: str) -> bool:
+        return any(t.tenant_adapter_name == adapter_name for t in self.loras)
+
+    def find_lora_by_tenant(self, tenant_adapter_name) -> LoraTenant:
+        for t in self.loras:
+            if t.tenant_adapter_name == tenant_adapter_name:
+                return t
+        raise ValueError(f'No lora found for tenant {tenant_adapter_name}')
+
+    def find_lora(self, adapter_name) -> LoraTenant:
+        for t in self.loras:
+            if t.adapter_name == adapter_name:
+                return t
+        raise ValueError(f'No lora found for real adapter_name {adapter_name}')
+
+    def acquire_lora(self, tenant_adapter_name: str, config) -> str:
+        """Give the tenant the first free slot (reference :209-226; same exceptions)."""
+        if self.has_lora(tenant_adapter_name):
+            raise ValueError(f'Lora {tenant_adapter_name} already exists')
+        slot = self._get_available_lora()
+        if slot is None:
+            raise RuntimeError(f'No lora available for tenant {tenant_adapter_name}. Max loras: {self.max_loras}')
+        if config.r > self.max_r:
+            raise RuntimeError(f'Too big rank for lora: {config.r}')
+        slot.tenant_config = config
+        slot.tenant_adapter_name = tenant_adapter_name
+        self._version += 1
+        return slot.adapter_name
+
+    def release_lora(self, tenant_adapter_name: str) -> Optional[str]:
+        """Free the tenant's slot: A back to its saved initial values, B to zero (reference :228-237)."""
+        try:
+            slot = self.find_lora_by_tenant(tenant_adapter_name)
+        except ValueError:
+            return None
+        slot.tenant_config = None
+        slot.tenant_adapter_name = None
+        self._load_initial_weights(slot.adapter_name)
+        self._version += 1
+        return None
+
+    def check_length(self, inputs) -> None:
+        total_length = sum(len(i['input_ids']) for i in inputs)
+        if total_length > self.max_length:
+            raise ValueError(f'Max length exceeds {self.max_length}')
+
+    # ------------------------------------------------------- target matching
+    @staticmethod
+    def match_target_modules(module_name: str, target_modules: Optional[Union[List[str], str]]) -> bool:
+        """Does a tenant's ``target_modules`` select this layer?  Same rules as reference :256-287."""
+        if target_modules is None:
+            return False
+        many = isinstance(target_modules, (list, set))
+        if many and len(target_modules) == 0:
+            return False
+        if target_modules == 'all-linear' or (many and len(target_modules) == 1
+                                              and next(iter(target_modules)) == 'all-linear'):
+            return True
+        name = module_name
+        if '.lora_' in name:  # a parameter name such as "...proj.lora_A.default.weight"
+            name = re.sub(r'\.lora_\w+(\.[\w-]+)*$', '', name)
+        if isinstance(target_modules, str):
+            return re.fullmatch(target_modules, name) is not None
+        if many:
+            return any(name.endswith(t) for t in target_modules)
+        return False
+
+    # --------------------------------------------------------- activation
+    def _modules(self):
+        return self.module if isinstance(self.module, list) else [self.module]
+
+    def activate_adapter(self, tenant_adapter_name: str, call_enable=False):
+        if not self.has_lora(tenant_adapter_name):
+            raise ValueError(f'Adapter {tenant_adapter_name} does not exist')
+        adapter_name = self.find_lora_by_tenant(tenant_adapter_name).adapter_name
+        for m in self._modules():
+            if call_enable:
+                m.enable_adapter_layers()
+            if getattr(m, 'active_adapter', None) != adapter_name:
+                m.set_adapter(adapter_name)
+
+    def deactivate_adapter(self):
+        for m in self._modules():
+            m.disable_adapter_layers()
+
+    def reset_adapter_status(self):
+        for m in self._modules():
+            m.set_adapter('lora_0')
+
+    @contextmanager
+    def adapter(self, tenant_adapter_name: str, disable_lora: bool = False):
+        """One tenant for every row of the calls inside (reference :154-163)."""
+        self.activate_adapter(tenant_adapter_name)
+        try:
+            if disable_lora:
+                with self._disable_lora_context(tenant_adapter_name):
+                    yield self.find_lora_by_tenant(tenant_adapter_name).adapter_name
+            else:
+                yield self.find_lora_by_tenant(tenant_adapter_name).adapter_name
+        finally:
+            self._uniform_tables.clear()
+
+    @contextmanager
+    def _disable_lora_context(self, tenant_adapter_name):
+        self.deactivate_adapter()
+        try:
+            yield
+        finally:
+            self.activate_adapter(tenant_adapter_name, call_enable=True)
+
+    @contextmanager
+    def batch(self, tenant_adapter_names: Sequence[str], row_tenant: torch.Tensor):
+        """Many tenants in one forward/backward: row ``i`` uses ``tenant_adapter_names[row_tenant[i]]``.
+
+        ``row_tenant`` is an integer GPU tensor with one entry per row of the
+        flattened ``[rows, features]`` activations (so ``batch * seq`` entries for
+        ``[batch, seq, features]`` inputs).  The segment table is built once here
+        and shared by every patched layer called inside the context.
+        """
+        slots = [self.find_lora_by_tenant(n).index for n in tenant_adapter_names]
+        lut = torch.tensor(slots, dtype=torch.int32, device=row_tenant.device)
+        keys = lut[row_tenant.reshape(-1).long()]
+        table = build_segments(keys, self.max_loras, want_perm=False, want_offsets=False)
+        previous, self._batch_table = self._batch_table, table
+        try:
+            yield table
+        finally:
+            self._batch_table = previous
+
+    def _table_for(self, rows: int, slot_index: int, device) -> SegmentTable:
+        key = (rows, slot_index, str(device))
+        table = self._uniform_tables.get(key)
+        if table is None:
+            keys = torch.full((rows,), slot_index, dtype=torch.int32, device=device)
+            table = build_segments(keys, self.max_loras, want_perm=False, want_offsets=False)
+            self._uniform_tables[key] = table
+        return table
+
+    # ------------------------------------------------------------- patching
+    def _groups_for(self, layer, only_slot: Optional[str]) -> Optional[AdapterGroups]:
+        """Rank/scale table of a layer: slots whose tenant targets this layer are live, the rest rank 0."""
+        key = (id(layer), only_slot)
+        cached = self._layer_groups.get(key)
+        if cached is not None and cached[0] == self._version:
+            return cached[1]
+        a, b, ranks, scales = [], [], [], []
+        for slot in self.loras:
+            name = slot.adapter_name
+            if name not in layer.lora_A.keys():
+                raise ValueError(f'layer {layer.layer_name} has no slot {name}')
+            a.append(layer.lora_A[name].weight)
+            b.append(layer.lora_B[name].weight)
+            cfg = slot.tenant_config
+            live = (cfg is not None and (only_slot is None or only_slot == name)
+                    and self.match_target_modules(layer.layer_name, cfg.target_modules))
+            if live:
+                ranks.append(cfg.r)
+                scales.append(cfg.lora_alpha / (cfg.r**0.5 if getattr(cfg, 'use_rslora', False) else cfg.r))
+            else:
+                ranks.append(0)
+                scales.append(0.0)
+        groups = AdapterGroups(a, b, ranks, scales) if max(ranks) > 0 else None
+        self._layer_groups[key] = (self._version, groups)
+        return groups
+
+    def _patch_lora_forward(_self, name, base_layer):
+        """Rebind ``forward`` on one LoRA layer (reference :289-331, Linear branch)."""
+        if not (_is_lora_layer(base_layer) and hasattr(base_layer, 'in_features')):
+            return
+
+        def _linear_forward(self, x: torch.Tensor, *args, **kwargs) -> torch.Tensor:
+            self._check_forward_args(x, *args, **kwargs)
+            table = _self._batch_table
+            only_slot = None
+            if table is None:
+                # one adapter per call: the active slot, if this layer has it (reference :306-309)
+                active = [n for n in self.active_adapters if n in self.lora_A.keys()]
+                only_slot = active[0] if active else None
+            skip = self.disable_adapters or (table is None and only_slot is None)
+            groups = None if skip else _self._groups_for(self, only_slot)
+            if groups is None:
+                return self.base_layer(x, *args, **kwargs)
+
+            wdtype = groups.dtype
+            xw = self._cast_input_dtype(x, wdtype)
+            slot_for_dropout = only_slot if only_slot is not None else _self.loras[0].adapter_name
+            xw = self.lora_dropout[slot_for_dropout](xw)
+            x2 = xw.reshape(-1, xw.shape[-1])
+            if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
+                x2 = x2.contiguous()
+            if table is None:
+                table = _self._table_for(x2.shape[0], _self.find_lora(only_slot).index, x2.device)
+            elif table.rows != x2.shape[0]:
+                raise ValueError(f'batch() was given {table.rows} rows but layer {self.layer_name} sees {x2.shape[0]}')
+
+            base = self.base_layer
+            plain = (type(base) is torch.nn.Linear and not args and not kwargs and xw is x and x.dtype == wdtype
+                     and base.weight.dtype == wdtype and not base._forward_hooks and not base._forward_pre_hooks)
+            if plain:
+                y2 = multi_lora_linear(x2, base.weight, base.bias, table, groups)
+                return y2.reshape(*x.shape[:-1], y2.shape[-1])
+
+            result = base(x, *args, **kwargs)
+            result_dtype = result.dtype
+            if result_dtype == wdtype and result.is_contiguous():
+                y2 = multi_lora_delta(x2, result.view(-1, result.shape[-1]), table, groups)
+                return y2.view(result.shape)
+            delta = multi_lora_delta(x2, torch.zeros(x2.shape[0], groups.out_features, dtype=wdtype, device=x2.device),
+                                     table, groups)
+            return (result + delta.view(*result.shape[:-1], -1)).to(result_dtype)
+
+        base_layer.forward = MethodType(_linear_forward, base_layer)
+        base_layer.layer_name = name
+
+    def patch(self, module, target_modules='all-linear', *args, **kwargs):
+        """Pre-allocate ``max_loras`` slots of rank ``max_r`` on ``module`` and patch every LoRA layer.
+
+        Follows reference :477-556: slots are named ``lora_0 .. lora_{max_loras-1}``,
+        built from ``lora_config`` (default ``r=max_r, lora_alpha=32``), every LoRA
+        parameter is trainable.  With PEFT installed a ``PeftModel`` can be passed
+        and is used as is; otherwise the in-tree container is injected.
+        """
+        for i in range(self.max_loras):
+            config = kwargs.get('lora_config', None)
+            if config is None:
+                config = LoraConfig(r=self.max_r, target_modules=target_modules, lora_alpha=32,
+                                    exclude_modules=['o_a_proj'])
+            slot = LoraTenant(index=i, adapter_name=f'lora_{i}', config=config)
+            self.loras.append(slot)
+            if hasattr(module, 'add_adapter') and hasattr(module, 'peft_config'):
+                module.add_adapter(slot.adapter_name, config)
+            else:
+                module = inject_adapter(module, config, slot.adapter_name)
+            for name, sub in module.named_modules():
+                if _is_lora_layer(sub):
+                    self._patch_lora_forward(name, sub)
+        for name, param in module.named_parameters():
+            if 'lora_' in name and not param.requires_grad:
+                param.requires_grad_(True)
+        self.module = module
+        return module
+
+    # --------------------------------------------------- weights and state
+    @staticmethod
+    def _slice_rank_tensor(name: str, tensor, rank: int):
+        if tensor is None:
+            return None
+        if 'embedding_A' in name:
+            return tensor[:, :rank]
+        if 'embedding_B' in name:
+            return tensor[:rank, :]
+        if '_A' in name:
+            return tensor[:rank, :]
+        if '_B' in name:
+            return tensor[:, :rank]
+        return tensor
+
+    @staticmethod
+    def _copy_rank_tensor(name: str, target, value):
+        if target is None or value is None:
+            return None
+        if 'embedding_A' in name:
+            target[:, :value.shape[1]].copy_(value)
+        elif 'embedding_B' in name:
+            target[:value.shape[0], :].copy_(value)
+        elif '_A' in name:
+            target[:value.shape[0], :].copy_(value)
+        elif '_B' in name:
+            target[:, :value.shape[1]].copy_(value)
+        else:
+            target.copy_(value)
+        return target
+
+    def _named_parameters(self):
+        for m in self._modules():
+            yield from m.named_parameters()
+
+    def save_initial_weights(self):
+        """Keep a CPU copy of every slot's initial A (reference :558-574)."""
+        for slot in self.loras:
+            pattern = re.compile(rf'\.lora_(?:A|embedding_A)\.{re.escape(slot.adapter_name)}\.')
+            for name, p in self._named_parameters():
+                if pattern.search(name):
+                    slot.lora_A_weights[name] = p.detach().clone().to('cpu')
+
+    def _load_initial_weights(self, origin_adapter_name):
+        slot = self.find_lora(origin_adapter_name)
+        pat_a = re.compile(rf'\.lora_(?:A|embedding_A)\.{re.escape(origin_adapter_name)}\.')
+        pat_b = re.compile(rf'\.lora_(?:B|embedding_B)\.{re.escape(origin_adapter_name)}\.')
+        if self.module is None:
+            return
+        with torch.no_grad():
+            for name, p in self._named_parameters():
+                if pat_a.search(name) and name in slot.lora_A_weights:
+                    p.copy_(slot.lora_A_weights[name].to(device=p.device, dtype=p.dtype))
+                if pat_b.search(name):
+                    p.zero_()
+
+    def set_state_dict(self, tenant_adapter_name, state_dict):
+        """Load rank-sliced tensors into the prefix of the tenant's slot (reference :676-699)."""
+        slot = self.find_lora_by_tenant(tenant_adapter_name)
+        pattern = re.compile(rf'\.lora_\w+\.{re.escape(slot.adapter_name)}\.')
+        with torch.no_grad():
+            for name, p in self._named_parameters():
+                if pattern.search(name) and self.match_target_modules(name, slot.tenant_config.target_modules):
+                    key = name.replace(f'.{slot.adapter_name}.', '.')
+                    src = state_dict[key].to(dtype=p.dtype, device=p.device)
+                    self._copy_rank_tensor(name, p.data, src)
+
+    def get_state_dict(self, tenant_adapter_name):
+        """Tenant's live ``[:r]`` blocks under slot-free names (reference :701-729)."""
+        slot = self.find_lora_by_tenant(tenant_adapter_name)
+        pattern = re.compile(rf'\.lora_\w+\.{re.escape(slot.adapter_name)}\.')
+        out = {}
+        for name, p in self._named_parameters():
+            if pattern.search(name) and self.match_target_modules(name, slot.tenant_config.target_modules):
+                out[name.replace(f'.{slot.adapter_name}.', '.')] = self._slice_rank_tensor(name, p.detach(),
+                                                                                           slot.tenant_config.r)
+        return out
+
+    def get_nb_trainable_parameters(self, tenant_adapter_name):
+        """(trainable, all) parameter counts as the tenant sees them (reference :756-813)."""
+        slot = self.find_lora_by_tenant(tenant_adapter_name)
+        pattern = re.compile(rf'\.lora_\w+\.{re.escape(slot.adapter_name)}\.')
+        trainable = total = 0
+        for name, p in self._named_parameters():
+            mine = pattern.search(name) is not None
+            if not mine and 'lora_' in name:
+                continue
+            if mine and not self.match_target_modules(name, slot.tenant_config.target_modules):
+                continue
+            n = self._slice_rank_tensor(name, p, slot.tenant_config.r).numel() if mine else p.numel()
+            total += n
+            if p.requires_grad:
+                trainable += n
+        return trainable, total

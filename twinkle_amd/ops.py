@@ -1,0 +1,269 @@
+"""Segmented multi-LoRA linear: torch custom ops over the C ABI, plus autograd.
+
+``y[row] += scale_g * (x[row] A_g^T) B_g^T`` for every adapter ``g`` of a mixed
+batch in one pass, and the matching backward.  For the rows of one adapter this
+is what the reference's patched forward computes with two ``F.linear`` calls
+(src/twinkle/model/multi_lora.py:315-326) and what autograd derives from them.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import _lib
+from .segments import SegmentTable
+
+
+class AdapterGroups:
+    """Which weight block, rank and scale every group of a layer uses.
+
+    ``a_tensors`` / ``b_tensors`` are the caller-owned parameters (slot tensors
+    ``[max_r, K]`` / ``[M, max_r]``, or packed expert tensors ``[E, max_r, K]`` /
+    ``[E, M, max_r]``).  Group ``g`` reads ``a_tensors[a_index[g]]`` starting
+    ``a_offset[g]`` elements in (likewise for B); the defaults give one tensor
+    per group.  Only pointers are kept: the parameters stay where they are.
+    """
+
+    def __init__(self, a_tensors: Sequence[torch.Tensor], b_tensors: Sequence[torch.Tensor], ranks: Sequence[int],
+                 scales: Sequence[float], a_index: Optional[Sequence[int]] = None,
+                 a_offset: Optional[Sequence[int]] = None, b_index: Optional[Sequence[int]] = None,
+                 b_offset: Optional[Sequence[int]] = None):
+        self.a_tensors = list(a_tensors)
+        self.b_tensors = list(b_tensors)
+        self.num_groups = len(ranks)
+        if self.num_groups == 0:
+            raise ValueError('at least one group is needed')
+        g = self.num_groups
+        self.a_index = list(a_index) if a_index is not None else list(range(g))
+        self.b_index = list(b_index) if b_index is not None else list(range(g))
+        self.a_offset = list(a_offset) if a_offset is not None else [0] * g
+        self.b_offset = list(b_offset) if b_offset is not None else [0] * g
+        self.ranks = [int(r) for r in ranks]
+        self.scales = [float(s) for s in scales]
+        if not (len(self.a_index) == len(self.b_index) == len(self.a_offset) == len(self.b_offset) == len(self.scales)
+                == g):
+            raise ValueError('per-group lists must have one entry per group')
+        a0, b0 = self.a_tensors[0], self.b_tensors[0]
+        self.dtype = a0.dtype
+        self.device = a0.device
+        self.in_features = a0.shape[-1]
+        self.out_features = b0.shape[-2]
+        self.lda = a0.stride(-2)
+        self.ldb = b0.stride(-2)
+        for t in self.a_tensors:
+            if t.dtype != self.dtype or t.shape[-1] != self.in_features or t.stride(-1) != 1 or t.stride(-2) != self.lda:
+                raise ValueError('all lora_A tensors of a layer must share dtype, width and row stride')
+        for t in self.b_tensors:
+            if t.dtype != self.dtype or t.shape[-2] != self.out_features or t.stride(-1) != 1 or \
+                    t.stride(-2) != self.ldb:
+                raise ValueError('all lora_B tensors of a layer must share dtype, height and row stride')
+        self.max_rank = max(self.ranks)
+        if self.max_rank > _lib.TK_MAX_RANK:
+            raise RuntimeError(f'Too big rank for lora: {self.max_rank}')
+        for i, r in enumerate(self.ranks):
+            if r < 0 or r > self.a_tensors[self.a_index[i]].shape[-2] or r > self.b_tensors[self.b_index[i]].shape[-1]:
+                raise RuntimeError(f'Too big rank for lora: {r}')
+        dev = self.device
+        self.rank_dev = torch.tensor(self.ranks, dtype=torch.int32, device=dev)
+        self.scale_dev = torch.tensor(self.scales, dtype=torch.float32, device=dev)
+        # gradient arena: one flat buffer per side, every tensor at a fixed element offset
+        self._a_arena_off, self.a_arena_elems = self._arena(self.a_tensors)
+        self._b_arena_off, self.b_arena_elems = self._arena(self.b_tensors)
+        esz = a0.element_size()
+        self._grad_a_rel = torch.tensor([(self._a_arena_off[self.a_index[i]] + self.a_offset[i]) * esz
+                                         for i in range(g)], dtype=torch.int64, device=dev)
+        self._grad_b_rel = torch.tensor([(self._b_arena_off[self.b_index[i]] + self.b_offset[i]) * esz
+                                         for i in range(g)], dtype=torch.int64, device=dev)
+        self._ptr_key = None
+        self.a_ptrs = self.b_ptrs = None
+        self.refresh()
+
+    @staticmethod
+    def _arena(tensors):
+        offs, total = [], 0
+        for t in tensors:
+            offs.append(total)
+            total += (t.numel() + 127) // 128 * 128
+        return offs, total
+
+    def refresh(self) -> None:
+        """Rebuild the device pointer arrays if a parameter's storage moved."""
+        key = tuple(t.data_ptr() for t in self.a_tensors) + tuple(t.data_ptr() for t in self.b_tensors)
+        if key == self._ptr_key:
+            return
+        esz = self.a_tensors[0].element_size()
+        g = self.num_groups
+        self.a_ptrs = torch.tensor([self.a_tensors[self.a_index[i]].data_ptr() + self.a_offset[i] * esz
+                                    for i in range(g)], dtype=torch.int64, device=self.device)
+        self.b_ptrs = torch.tensor([self.b_tensors[self.b_index[i]].data_ptr() + self.b_offset[i] * esz
+                                    for i in range(g)], dtype=torch.int64, device=self.device)
+        self._ptr_key = key
+
+    def grad_views(self, arena: torch.Tensor, side: str) -> List[torch.Tensor]:
+        tensors, offs = (self.a_tensors, self._a_arena_off) if side == 'a' else (self.b_tensors, self._b_arena_off)
+        return [arena[o:o + t.numel()].view(t.shape) for t, o in zip(tensors, offs)]
+
+
+def _desc(seg: SegmentTable, groups: AdapterGroups, map_rows: bool) -> _lib.LoraDesc:
+    groups.refresh()
+    d = _lib.LoraDesc()
+    d.rows = seg.rows
+    d.in_features = groups.in_features
+    d.out_features = groups.out_features
+    d.num_groups = groups.num_groups
+    d.max_rank = groups.max_rank
+    d.dtype = _lib.dtype_code(groups.dtype)
+    d.map_rows = 1 if map_rows else 0
+    d.seg_ws = seg.workspace.data_ptr()
+    d.lora_A = groups.a_ptrs.data_ptr()
+    d.lora_B = groups.b_ptrs.data_ptr()
+    d.lda = groups.lda
+    d.ldb = groups.ldb
+    d.rank = groups.rank_dev.data_ptr()
+    d.scale = groups.scale_dev.data_ptr()
+    return d
+
+
+def _check_rows(t: torch.Tensor, name: str, rows: int, width: int, dtype: torch.dtype):
+    if not t.is_cuda:
+        raise RuntimeError(f'{name} must live on the GPU: this path has no CPU implementation')
+    if t.dim() != 2 or t.shape[0] != rows or t.shape[1] != width or t.stride(1) != 1:
+        raise ValueError(f'{name} must be [{rows}, {width}] with unit inner stride, got {tuple(t.shape)} '
+                         f'strides {t.stride()}')
+    if t.dtype != dtype:
+        raise ValueError(f'{name} has dtype {t.dtype}, adapters have {dtype}')
+
+
+def lora_h_bytes(seg: SegmentTable, groups: AdapterGroups) -> int:
+    n = _lib.load().tk_lora_h_bytes(ctypes.byref(_desc(seg, groups, True)))
+    _lib.check(n, 'tk_lora_h_bytes')
+    return n
+
+
+def lora_bwd_workspace_bytes(seg: SegmentTable, groups: AdapterGroups) -> int:
+    n = _lib.load().tk_lora_bwd_workspace_bytes(ctypes.byref(_desc(seg, groups, True)))
+    _lib.check(n, 'tk_lora_bwd_workspace_bytes')
+    return n
+
+
+def lora_fwd_(x: torch.Tensor, y: torch.Tensor, seg: SegmentTable, groups: AdapterGroups, map_rows: bool = True,
+              h: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """In place ``y += lora(x)``; returns the saved shrink output ``h`` (opaque bytes)."""
+    if groups.num_groups != seg.num_groups:
+        raise ValueError(f'segment table has {seg.num_groups} groups, adapters have {groups.num_groups}')
+    _check_rows(x, 'x', seg.rows, groups.in_features, groups.dtype)
+    _check_rows(y, 'y', seg.rows, groups.out_features, groups.dtype)
+    d = _desc(seg, groups, map_rows)
+    lib = _lib.load()
+    if h is None:
+        h = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=x.device)
+    code = lib.tk_lora_fwd(ctypes.byref(d), x.data_ptr(), x.stride(0), y.data_ptr(), y.stride(0), h.data_ptr(),
+                           _lib.stream_ptr())
+    _lib.check(code, 'tk_lora_fwd')
+    return h
+
+
+def lora_bwd_(dy: torch.Tensor, x: Optional[torch.Tensor], h: Optional[torch.Tensor], dx: Optional[torch.Tensor],
+              grad_a_ptrs: Optional[torch.Tensor], grad_b_ptrs: Optional[torch.Tensor], seg: SegmentTable,
+              groups: AdapterGroups, map_rows: bool = True, accumulate: bool = False,
+              workspace: Optional[torch.Tensor] = None) -> None:
+    """``dx += ...`` in place, weight gradients through the pointer arrays (see ``tk_lora_bwd``)."""
+    _check_rows(dy, 'dy', seg.rows, groups.out_features, groups.dtype)
+    if x is not None:
+        _check_rows(x, 'x', seg.rows, groups.in_features, groups.dtype)
+    if dx is not None:
+        _check_rows(dx, 'dx', seg.rows, groups.in_features, groups.dtype)
+    d = _desc(seg, groups, map_rows)
+    lib = _lib.load()
+    if workspace is None:
+        workspace = torch.empty(lora_bwd_workspace_bytes(seg, groups), dtype=torch.uint8, device=dy.device)
+    code = lib.tk_lora_bwd(ctypes.byref(d), dy.data_ptr(), dy.stride(0), x.data_ptr() if x is not None else None,
+                           x.stride(0) if x is not None else 0, h.data_ptr() if h is not None else None,
+                           dx.data_ptr() if dx is not None else None, dx.stride(0) if dx is not None else 0,
+                           grad_a_ptrs.data_ptr() if grad_a_ptrs is not None else None,
+                           grad_b_ptrs.data_ptr() if grad_b_ptrs is not None else None, 1 if accumulate else 0,
+                           workspace.data_ptr(), workspace.numel(), _lib.stream_ptr())
+    _lib.check(code, 'tk_lora_bwd')
+
+
+def _weight_grads(ctx_groups: AdapterGroups, needs_a: bool, needs_b: bool, device):
+    groups = ctx_groups
+    arena_a = arena_b = pa = pb = None
+    if needs_a:
+        arena_a = torch.zeros(groups.a_arena_elems, dtype=groups.dtype, device=device)
+        pa = groups._grad_a_rel + arena_a.data_ptr()
+    if needs_b:
+        arena_b = torch.zeros(groups.b_arena_elems, dtype=groups.dtype, device=device)
+        pb = groups._grad_b_rel + arena_b.data_ptr()
+    return arena_a, arena_b, pa, pb
+
+
+class _LoraDelta(torch.autograd.Function):
+    """``y`` (base output) updated in place; gradients for ``x``, ``y`` and every adapter tensor."""
+
+    @staticmethod
+    def forward(ctx, x, y, seg, groups, map_rows, *weights):
+        h = lora_fwd_(x, y, seg, groups, map_rows)
+        ctx.mark_dirty(y)
+        ctx.save_for_backward(x, h)
+        ctx.seg, ctx.groups, ctx.map_rows = seg, groups, map_rows
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, h = ctx.saved_tensors
+        seg, groups = ctx.seg, ctx.groups
+        dy = dy.contiguous()
+        na, nb = len(groups.a_tensors), len(groups.b_tensors)
+        needs_a = any(ctx.needs_input_grad[5:5 + na])
+        needs_b = any(ctx.needs_input_grad[5 + na:5 + na + nb])
+        dx = torch.zeros_like(x) if ctx.needs_input_grad[0] else None
+        arena_a, arena_b, pa, pb = _weight_grads(groups, needs_a, needs_b, dy.device)
+        lora_bwd_(dy, x, h, dx, pa, pb, seg, groups, ctx.map_rows, accumulate=False)
+        ga = groups.grad_views(arena_a, 'a') if needs_a else [None] * na
+        gb = groups.grad_views(arena_b, 'b') if needs_b else [None] * nb
+        return (dx, dy, None, None, None, *ga, *gb)
+
+
+class _LoraLinear(torch.autograd.Function):
+    """Base ``F.linear`` and the LoRA update as one node: ``dx`` of the base GEMM is updated in place."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, seg, groups, map_rows, *weights):
+        y = torch.nn.functional.linear(x, weight, bias)
+        h = lora_fwd_(x, y, seg, groups, map_rows)
+        ctx.save_for_backward(x, weight, h)
+        ctx.has_bias = bias is not None
+        ctx.seg, ctx.groups, ctx.map_rows = seg, groups, map_rows
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight, h = ctx.saved_tensors
+        seg, groups = ctx.seg, ctx.groups
+        dy = dy.contiguous()
+        na, nb = len(groups.a_tensors), len(groups.b_tensors)
+        needs_a = any(ctx.needs_input_grad[6:6 + na])
+        needs_b = any(ctx.needs_input_grad[6 + na:6 + na + nb])
+        dx = dy @ weight if ctx.needs_input_grad[0] else None
+        dw = dy.t() @ x if ctx.needs_input_grad[1] else None
+        db = dy.sum(0) if ctx.has_bias and ctx.needs_input_grad[2] else None
+        arena_a, arena_b, pa, pb = _weight_grads(groups, needs_a, needs_b, dy.device)
+        lora_bwd_(dy, x, h, dx, pa, pb, seg, groups, ctx.map_rows, accumulate=False)
+        ga = groups.grad_views(arena_a, 'a') if needs_a else [None] * na
+        gb = groups.grad_views(arena_b, 'b') if needs_b else [None] * nb
+        return (dx, dw, db, None, None, None, *ga, *gb)
+
+
+def multi_lora_delta(x: torch.Tensor, base_out: torch.Tensor, seg: SegmentTable, groups: AdapterGroups,
+                     map_rows: bool = True) -> torch.Tensor:
+    """``base_out`` with every adapter's LoRA term added to its own rows (in place, differentiable)."""
+    return _LoraDelta.apply(x, base_out, seg, groups, map_rows, *groups.a_tensors, *groups.b_tensors)
+
+
+def multi_lora_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], seg: SegmentTable,
+                      groups: AdapterGroups, map_rows: bool = True) -> torch.Tensor:
+    """``F.linear(x, weight, bias)`` plus the segmented LoRA update as one autograd node."""
+    return _LoraLinear.apply(x, weight, bias, seg, groups, map_rows, *groups.a_tensors, *groups.b_tensors)
