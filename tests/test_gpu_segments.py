@@ -10,8 +10,8 @@ from twinkle_amd import workloads
 pytestmark = pytest.mark.gpu
 
 
-def _check(keys_cpu, groups, dev, dtype=torch.int32):
-    seg = build_segments(keys_cpu.to(dtype).to(dev), groups, check=True)
+def _check(keys_cpu, groups, dev, dtype=torch.int32, num_tokens=None):
+    seg = build_segments(keys_cpu.to(dtype).to(dev), groups, num_tokens=num_tokens, check=True)
     perm, counts, offsets = oracle.segment_build_sort(keys_cpu, groups)
     assert seg.perm.dtype == torch.int64 and seg.offsets.dtype == torch.int64
     assert torch.equal(seg.perm.cpu(), perm)
@@ -70,11 +70,11 @@ def test_config4_expert_tenant_grouping_matches_reference_mask_order(dev):
     sel, w, tenant = workloads.moe_routing()
     t, k = sel.shape
     keys = oracle.flat_keys_from_topk(sel, tenant, 4)
-    seg = _check(keys, 512, dev)
+    seg = _check(keys, 512, dev, num_tokens=t)
     assert torch.equal(flat_keys_from_topk(sel.to(dev), tenant.to(dev), 4).cpu().long(), keys)
     # one tenant: identical to the masked_select order of the reference
     keys1 = oracle.flat_keys_from_topk(sel)
-    seg1 = _check(keys1, 128, dev)
+    seg1 = _check(keys1, 128, dev, num_tokens=t)
     mask = oracle.expert_mask_from_topk(sel.long(), 128)
     _, sorted_indices = oracle.permute_by_mask(torch.zeros(t, 1), mask)
     assert torch.equal(seg1.row_token.cpu(), sorted_indices)
