@@ -1,0 +1,187 @@
+#!/usr/bin/env python3
+"""Benchmark of the multi-LoRA hot path on one MI355X.
+
+One step = segment build + segmented LoRA forward + segmented LoRA backward (dX, dA, dB) over one
+batch of BASELINE.json's config 2: Llama-3-8B q_proj shape (4096 -> 4096), 16384 tokens, 16 adapters of
+rank 16 / alpha 32, adapter ids Zipf(1.1)-distributed and shuffled, bf16 with fp32 accumulation.  The
+frozen base GEMM is not part of the step (it is timed once and reported separately).  Inputs are
+resident in HBM before the timed region; three buffer sets are rotated so that no activation is served
+from the 256 MB last-level cache across steps (the backward of a step runs on the set whose forward ran
+one full step earlier).
+
+Prints one JSON line (see the keys below).  `roofline` describes the dominant kernel, the fused
+shrink->expand pass, on its forward launches: algorithmic bytes of one launch over its mean duration
+between HIP events on the launch stream.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def cpu_baseline(w, budget_s=15.0):
+    """The reference's CPU path (per-adapter F.linear pairs + autograd, restated in oracle/) on this host."""
+    import torch
+    import oracle
+    threads = torch.get_num_threads()
+    x = w.x.bfloat16().float()
+    base = w.base_out.bfloat16().float()
+    dy = w.dy.bfloat16().float()
+    a = [t.bfloat16().float() for t in w.lora_A]
+    b = [t.bfloat16().float() for t in w.lora_B]
+    oracle.multi_lora_linear_grads(x[:2048], base[:2048], w.ids[:2048], a, b, w.ranks, w.scales, dy[:2048])  # warm-up
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        oracle.multi_lora_linear_grads(x, base, w.ids, a, b, w.ranks, w.scales, dy)
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or reps >= 20:
+            break
+    return {
+        'value': w.tokens * reps / el, 'unit': 'tokens/s', 'cores': threads, 'kind': 'port',
+        'sample': f'{reps} x the full {w.name} batch ({w.tokens} tokens), bf16-rounded inputs, fp32 math, '
+                  f'torch {torch.__version__} CPU, per-adapter F.linear pairs + autograd',
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--sets', type=int, default=3, help='rotated buffer sets')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print('bench.py measures one GPU: this path has no multi-GPU part (rows shard trivially; see DESIGN.md). '
+              'Run with --gpus 1.', file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from twinkle_amd import (AdapterGroups, _lib, build_segments, lora_bwd_, lora_bwd_workspace_bytes, lora_fwd_,
+                             lora_h_bytes, workloads)
+    if not torch.cuda.is_available():
+        print('bench.py needs a GPU', file=sys.stderr)
+        sys.exit(2)
+    _lib.load()
+    dev = torch.device('cuda:0')
+    w = workloads.config2_qproj()
+    dt = torch.bfloat16
+    elt = 2
+    T, K, M, G = w.tokens, w.in_features, w.out_features, w.num_adapters
+
+    ids = w.ids.to(dev)
+    A = [t.to(dt).to(dev) for t in w.lora_A]
+    B = [t.to(dt).to(dev) for t in w.lora_B]
+    groups = AdapterGroups(A, B, w.ranks, w.scales)
+    grad_a = [torch.zeros_like(t) for t in A]
+    grad_b = [torch.zeros_like(t) for t in B]
+    pa = torch.tensor([t.data_ptr() for t in grad_a], dtype=torch.int64, device=dev)
+    pb = torch.tensor([t.data_ptr() for t in grad_b], dtype=torch.int64, device=dev)
+    sets = []
+    for i in range(args.sets):
+        sets.append({
+            'x': (w.x if i == 0 else torch.roll(w.x, i, 0)).to(dt).to(dev),
+            'y': w.base_out.to(dt).to(dev),
+            'dy': (w.dy if i == 0 else torch.roll(w.dy, i, 0)).to(dt).to(dev),
+            'dx': torch.zeros(T, K, dtype=dt, device=dev),
+            'h': None,
+        })
+    seg = build_segments(ids, G, want_perm=False, want_offsets=False)
+    for s in sets:
+        s['h'] = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=dev)
+    ws = torch.empty(lora_bwd_workspace_bytes(seg, groups), dtype=torch.uint8, device=dev)
+    seg_holder = {'seg': seg}
+
+    def step(i, ev=None):
+        f = sets[i % len(sets)]
+        b = sets[(i + 1) % len(sets)]
+        seg_i = build_segments(ids, G, want_perm=False, want_offsets=False)
+        seg_holder['seg'] = seg_i
+        if ev is not None:
+            ev[0].record()
+        lora_fwd_(f['x'], f['y'], seg_i, groups, h=f['h'])
+        if ev is not None:
+            ev[1].record()
+        lora_bwd_(b['dy'], b['x'], b['h'], b['dx'], pa, pb, seg_i, groups, accumulate=False, workspace=ws)
+        if ev is not None:
+            ev[2].record()
+
+    # every set needs a forward before its first backward
+    for i in range(len(sets)):
+        lora_fwd_(sets[i]['x'], sets[i]['y'], seg, groups, h=sets[i]['h'])
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i, events[i])
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
+
+    # base GEMM, reported separately and not part of the step
+    wbase = torch.randn(M, K, device=dev, dtype=dt) * 0.02
+    xs = sets[0]['x']
+    for _ in range(3):
+        torch.nn.functional.linear(xs, wbase)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        torch.nn.functional.linear(xs, wbase)
+    e1.record()
+    torch.cuda.synchronize()
+    base_ms = e0.elapsed_time(e1) / 10
+
+    w_live = sum(r * (K + M) for r in w.ranks)
+    step_bytes = w.algorithmic_bytes(elt)
+    fwd_bytes = elt * T * (K + 2 * M) + elt * w_live           # one launch of the fused pass (forward instance)
+    flops = w.flops()
+    achieved = fwd_bytes / (fwd_ms * 1e-3) / 1e9
+    out = {
+        'metric': 'multi-LoRA fwd+bwd tokens/s + % roofline (HBM/MFMA), 8B proj, 16 adapters',
+        'value': T / (ms_per_step * 1e-3),
+        'unit': 'tokens/s',
+        'n_gpus': 1,
+        'steps': args.steps,
+        'warmup': args.warmup,
+        'ms_per_step': ms_per_step,
+        'higher_is_better': True,
+        'scaling': 'weak',
+        'vs_baseline': None,
+        'dtype': 'bf16',
+        'data': 'synthetic',
+        'config': {'workload': 'BASELINE config 2: Llama-3-8B q_proj 4096->4096, T=16384, 16 adapters rank 16 alpha 32, '
+                               'Zipf(1.1) ids shuffled; step = segment build + LoRA fwd + LoRA bwd (dX, dA, dB); '
+                               'base GEMM excluded', 'tokens': T, 'in': K, 'out': M, 'adapters': G, 'rank': 16},
+        'roofline': {'bound': 'hbm', 'achieved': achieved, 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+                     'frac': achieved / HBM_PEAK_GBS, 'traffic': None,
+                     'kernel': 'k_pass_mfma<1,8> (fused shrink->expand), forward launch',
+                     'algorithmic_bytes_per_launch': fwd_bytes, 'avg_launch_ms': fwd_ms},
+        'step_detail': {'fwd_ms': fwd_ms, 'bwd_ms': bwd_ms, 'segment_build_and_gaps_ms': ms_per_step - fwd_ms - bwd_ms,
+                        'algorithmic_bytes_per_step': step_bytes, 'flops_per_step': flops,
+                        'tflops': flops / (ms_per_step * 1e-3) / 1e12,
+                        'hbm_frac_step': step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                        'hbm_frac_fwd_plus_bwd_kernels': step_bytes / ((fwd_ms + bwd_ms) * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                        'mfma_frac_step': flops / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                        'base_gemm_ms_excluded': base_ms},
+    }
+    if not args.no_cpu_baseline:
+        out['cpu_baseline'] = cpu_baseline(w)
+    print(json.dumps(out))
+
+
+if __name__ == '__main__':
+    main()

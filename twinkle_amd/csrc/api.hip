@@ -1,4 +1,6 @@
 // C ABI of the library: argument checks, workspace carving, kernel choice.
+#include <stdlib.h>
+
 #include "tk_common.h"
 
 using namespace tk;
@@ -17,14 +19,24 @@ bool desc_ok(const tk_lora_desc* d) {
   return true;
 }
 
+// TK_FORCE_GENERIC=1 in the environment routes every launch to the shape-agnostic kernels
+// (an A/B switch for debugging; both families are HIP kernels on the GPU).
+bool force_generic() {
+  static const bool v = [] {
+    const char* e = getenv("TK_FORCE_GENERIC");
+    return e && e[0] == '1';
+  }();
+  return v;
+}
+
 int run_pass(const PassArgs& a, const SegView& V, const SegLayout& L, int dtype, hipStream_t s) {
-  if (dtype == TK_DTYPE_BF16 && pass_mfma_supported(a)) return launch_pass_mfma(a, V, L, s);
+  if (dtype == TK_DTYPE_BF16 && !force_generic() && pass_mfma_supported(a)) return launch_pass_mfma(a, V, L, s);
   return launch_pass_generic(a, V, L, dtype, s);
 }
 
 int run_wgrad(const WgradArgs& a, const SegView& V, const SegLayout& L, int dtype, hipStream_t s) {
   int rc;
-  if (dtype == TK_DTYPE_BF16 && wgrad_mfma_supported(a))
+  if (dtype == TK_DTYPE_BF16 && !force_generic() && wgrad_mfma_supported(a))
     rc = launch_wgrad_mfma(a, V, L, s);
   else
     rc = launch_wgrad_generic(a, V, L, dtype, s);

@@ -105,7 +105,12 @@ constexpr int32_t kSegMagic = 0x544b5347;  // "TKSG"
 // the row-contraction kernels read 8 consecutive positions per lane.
 // ---------------------------------------------------------------------------
 static inline int64_t h_ld(int64_t rows) { return round_up(rows > 0 ? rows : 1, 64); }
-static inline int32_t rank_pad(int32_t max_rank) { return (int32_t)round_up(max_rank > 0 ? max_rank : 1, 16); }
+// Padded rank: 16, 32, 64 or 128 (the kernels are instantiated per padded rank).
+static inline int32_t rank_pad(int32_t max_rank) {
+  int32_t p = 16;
+  while (p < max_rank) p <<= 1;
+  return p;
+}
 static inline int elt_bytes(int dtype) { return dtype == TK_DTYPE_BF16 ? 2 : 4; }
 
 // Backward workspace carving.
