@@ -124,7 +124,8 @@ int tk_unpermute_weight_grad(const void* dout, int64_t ld_dout, const void* rows
 
 int64_t tk_lora_h_bytes(const tk_lora_desc* d) {
   if (!d || d->rows < 0 || d->max_rank < 0 || d->max_rank > TK_MAX_RANK) return TK_ERR_INVALID;
-  return round_up((int64_t)rank_pad(d->max_rank) * h_ld(d->rows) * elt_bytes(d->dtype), 256);
+  // rank-major copy hT[rpad][ld] followed by the position-major copy hrow[ld][rpad]
+  return round_up(2 * (int64_t)rank_pad(d->max_rank) * h_ld(d->rows) * elt_bytes(d->dtype), 256);
 }
 
 int64_t tk_lora_bwd_workspace_bytes(const tk_lora_desc* d) {

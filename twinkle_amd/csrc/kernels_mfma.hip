@@ -64,48 +64,38 @@ __device__ inline uint4 keep_range(uint4 v, int lo, int hi) {
 }
 
 // ---------------------------------------------------------------------------
-// Fused pass: one workgroup owns one tile of up to 32 rows of one group.
-//   phase 1 (shrink)  the NW waves split the source width; each wave streams
-//                     its 64-column pieces of the 32 rows once and keeps
-//                     h[32][rank] partial sums in MFMA accumulators;
-//   reduce            partials meet in LDS and are summed in wave order
-//                     (fixed order: bitwise repeatable), scaled, rounded to
-//                     bf16, kept in LDS and written to hT for the backward;
-//   phase 2 (expand)  the waves split the destination width in 128-column
-//                     groups: dst[row] += h[row] W2^T, read-modify-write in place.
+// Shrink: h[p][n] = scale_g * sum_k src[row(p)][k] * W1_g[n][k] for one tile of up
+// to 32 rows of one group per workgroup.  The NW waves split the source width
+// in 64-column steps (interleaved, so the workgroup reads 64*NW contiguous
+// columns of each row at a time); every wave keeps its partial h[32][rank] in
+// MFMA accumulators, issuing the loads of PF steps before the first MFMA so
+// that ~PF*6 KB per wave are in flight.  Partials meet in LDS and are summed
+// in wave order (fixed order: bitwise repeatable), scaled, rounded to bf16
+// and written twice: position-major (hrow, the expand kernel's A operand) and
+// rank-major (hT, read by the weight-gradient kernel).
 // ---------------------------------------------------------------------------
-template <int NB, int NW>
-__global__ __launch_bounds__(NW * 64) void k_pass_mfma(PassArgs a, const TileInfo* __restrict__ tiles,
-                                                       const int32_t* __restrict__ perm, const SegHeader* hdr) {
-  constexpr int RP = 16 * NB;          // padded rank
-  constexpr int PR = RP + 1;           // row stride of the partial sums (floats; odd: conflict-free column reads)
-  constexpr int HS = RP + 8;           // row stride of h in LDS (bf16; keeps 16-byte alignment)
-  constexpr int NKS = (RP + 31) / 32;  // contraction steps of the expand MFMAs
+template <int NB, int NW, int PF>
+__global__ __launch_bounds__(NW * 64) void k_shrink_mfma(PassArgs a, bf16_t* __restrict__ hrow,
+                                                         const TileInfo* __restrict__ tiles,
+                                                         const int32_t* __restrict__ perm, const SegHeader* hdr) {
+  constexpr int RP = 16 * NB;  // padded rank
+  constexpr int PR = RP + 1;   // row stride of the partial sums (floats; odd: conflict-free column reads)
   __shared__ float part[NW][kTileRows][PR];
-  __shared__ __attribute__((aligned(16))) bf16_t hs[kTileRows][HS];
-  __shared__ int rows_s[kTileRows];
 
-  // consecutive tiles (same group, same weights) go to the same XCD: workgroups are dealt to the 8 XCDs round-robin
-  const int per_xcd = gridDim.x >> 3;
-  const int tile_id = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  const int tile_id = blockIdx.x;
   if (tile_id >= hdr->num_tiles) return;
   const TileInfo ti = tiles[tile_id];
   const int g = ti.group;
   const int r = min(a.rank[g], RP);
+  if (r <= 0) return;  // adapter not live on this layer
   const int cnt = ti.count;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
 
-  if (tid < kTileRows) {
-    const int p = ti.start + min(tid, cnt - 1);
-    rows_s[tid] = a.map_rows ? perm[p] : p;
-  }
-  __syncthreads();
-  if (r <= 0) return;  // adapter not live on this layer: rows keep the base output
-
-  // ---- phase 1 ----
+  const int pa = ti.start + min(li, cnt - 1), pb = ti.start + min(16 + li, cnt - 1);
+  const int64_t ra = a.map_rows ? perm[pa] : pa, rb = a.map_rows ? perm[pb] : pb;
   const bf16_t* src = (const bf16_t*)a.src;
-  const bf16_t* xa = src + (int64_t)rows_s[li] * a.ld_src + 16 * kb;
-  const bf16_t* xb = src + (int64_t)rows_s[16 + li] * a.ld_src + 16 * kb;
+  const bf16_t* xa = src + ra * a.ld_src + 16 * kb;
+  const bf16_t* xb = src + rb * a.ld_src + 16 * kb;
   const bf16_t* W1 = group_weight<bf16_t>(a.w_shrink, a.w_shrink_base, a.shrink_group_stride, g);
   const bf16_t* wp[NB];
   bool wv[NB];
@@ -122,24 +112,32 @@ __global__ __launch_bounds__(NW * 64) void k_pass_mfma(PassArgs a, const TileInf
     acc[1][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const int nsteps = a.width_src >> 6;
-#pragma unroll 4
-  for (int s = wave; s < nsteps; s += NW) {
-    const int c = s << 6;
-    const uint4 xa0 = ld16(xa + c), xa1 = ld16(xa + c + 8);
-    const uint4 xb0 = ld16(xb + c), xb1 = ld16(xb + c + 8);
-    uint4 w0[NB], w1[NB];
+  for (int s0 = wave; s0 < nsteps; s0 += NW * PF) {
+    uint4 xa0[PF], xa1[PF], xb0[PF], xb1[PF], w0[PF][NB], w1[PF][NB];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      w0[nb] = wv[nb] ? ld16(wp[nb] + c) : zero4();
-      w1[nb] = wv[nb] ? ld16(wp[nb] + c + 8) : zero4();
+    for (int j = 0; j < PF; ++j) {
+      const int s = s0 + j * NW;
+      const bool ok = s < nsteps;  // wave-uniform
+      const int c = (ok ? s : s0) << 6;
+      xa0[j] = ld16(xa + c);
+      xa1[j] = ld16(xa + c + 8);
+      xb0[j] = ld16(xb + c);
+      xb1[j] = ld16(xb + c + 8);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        w0[j][nb] = (wv[nb] && ok) ? ld16(wp[nb] + c) : zero4();
+        w1[j][nb] = (wv[nb] && ok) ? ld16(wp[nb] + c + 8) : zero4();
+      }
     }
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      acc[0][nb] = mfma16(xa0, w0[nb], acc[0][nb]);
-      acc[1][nb] = mfma16(xb0, w0[nb], acc[1][nb]);
-      acc[0][nb] = mfma16(xa1, w1[nb], acc[0][nb]);
-      acc[1][nb] = mfma16(xb1, w1[nb], acc[1][nb]);
-    }
+    for (int j = 0; j < PF; ++j)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        acc[0][nb] = mfma16(xa0[j], w0[j][nb], acc[0][nb]);
+        acc[1][nb] = mfma16(xb0[j], w0[j][nb], acc[1][nb]);
+        acc[0][nb] = mfma16(xa1[j], w1[j][nb], acc[0][nb]);
+        acc[1][nb] = mfma16(xb1[j], w1[j][nb], acc[1][nb]);
+      }
   }
 #pragma unroll
   for (int tt = 0; tt < 2; ++tt)
@@ -149,43 +147,100 @@ __global__ __launch_bounds__(NW * 64) void k_pass_mfma(PassArgs a, const TileInf
       for (int v = 0; v < 4; ++v) part[wave][16 * tt + 4 * kb + v][16 * nb + li] = acc[tt][nb][v];
   __syncthreads();
 
-  // ---- reduce over waves, scale, round, publish ----
   const float sc = a.scale[g];
   bf16_t* hT = (bf16_t*)a.hT;
+  // position-major copy: consecutive threads -> consecutive rank indices of one row
+  for (int idx = tid; idx < kTileRows * RP; idx += NW * 64) {
+    const int row = idx / RP, n = idx % RP;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) sum += part[w][row][n];
+    if (row < cnt) hrow[(int64_t)(ti.start + row) * RP + n] = (bf16_t)(pack_bf16(sum * sc, 0.f) & 0xffffu);
+  }
+  // rank-major copy: consecutive threads -> consecutive rows of one rank index
   for (int idx = tid; idx < kTileRows * RP; idx += NW * 64) {
     const int n = idx >> 5, row = idx & 31;
     float sum = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) sum += part[w][row][n];
-    const uint32_t hb = pack_bf16(sum * sc, 0.f) & 0xffffu;
-    hs[row][n] = (bf16_t)hb;
-    if (row < cnt) hT[(int64_t)n * a.ldh + ti.start + row] = (bf16_t)hb;
+    if (row < cnt) hT[(int64_t)n * a.ldh + ti.start + row] = (bf16_t)(pack_bf16(sum * sc, 0.f) & 0xffffu);
   }
-  if (a.dst == nullptr) return;
-  __syncthreads();
+}
 
-  // ---- phase 2 ----
+// ---------------------------------------------------------------------------
+// Expand: dst[row(p)][c] += sum_n h[p][n] * W2_g[c][n], read-modify-write in
+// place.  Work is flat: one wave owns CPW adjacent 128-column groups of one
+// 32-row tile and nothing is shared between waves, so the grid is thousands
+// of independent streams.  Column c0 + 8 j + q of a group is output column j
+// of MFMA q, which makes each lane's 8 results of one row 16 contiguous
+// bytes and each wave-wide access 4 rows x 256 B.
+// ---------------------------------------------------------------------------
+template <int NB, int CPW>
+__global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* __restrict__ hrow,
+                                                     const TileInfo* __restrict__ tiles,
+                                                     const int32_t* __restrict__ perm, const SegHeader* hdr) {
+  constexpr int RP = 16 * NB;
+  constexpr int NKS = (RP + 31) / 32;  // contraction steps of the MFMAs
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  const int ngroups = a.width_dst >> 7;
+  const int items_per_tile = (ngroups + CPW - 1) / CPW;
+  const int item = blockIdx.x * 4 + wave;
+  const int tile_id = item / items_per_tile;
+  if (tile_id >= hdr->num_tiles) return;
+  const int cg0 = (item - tile_id * items_per_tile) * CPW;
+  const TileInfo ti = tiles[tile_id];
+  const int g = ti.group;
+  const int r = min(a.rank[g], RP);
+  if (r <= 0) return;
+  const int cnt = ti.count;
+
+  // rows this lane updates: 16 tt + 4 kb + v
+  bf16_t* yp[2][4];
+  bool yok[2][4];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int row = 16 * tt + 4 * kb + v;
+      yok[tt][v] = row < cnt;
+      const int p = ti.start + min(row, cnt - 1);
+      const int64_t rr = a.map_rows ? perm[p] : p;
+      yp[tt][v] = (bf16_t*)a.dst + rr * a.ld_dst + 8 * li;
+    }
   uint4 hop[2][NKS];
 #pragma unroll
   for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
       const int n0 = 32 * ks + 8 * kb;
-      hop[tt][ks] = n0 < RP ? *reinterpret_cast<const uint4*>(&hs[16 * tt + li][n0]) : zero4();
+      const int p = ti.start + min(16 * tt + li, cnt - 1);
+      hop[tt][ks] = n0 < RP ? ld16(hrow + (int64_t)p * RP + n0) : zero4();
     }
   const bf16_t* W2 = group_weight<bf16_t>(a.w_expand, a.w_expand_base, a.expand_group_stride, g);
-  bf16_t* dst = (bf16_t*)a.dst;
-  const int ngroups = a.width_dst >> 7;
-  for (int cg = wave; cg < ngroups; cg += NW) {
-    const int c0 = cg << 7;
-    uint4 bq[8][NKS];
+
+  uint4 y[CPW][2][4];
+  uint4 bq[CPW][8][NKS];
+#pragma unroll
+  for (int u = 0; u < CPW; ++u) {
+    const bool gok = cg0 + u < ngroups;  // wave-uniform
+    const int c0 = (gok ? cg0 + u : cg0) << 7;
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) y[u][tt][v] = (yok[tt][v] && gok) ? ld16(yp[tt][v] + c0) : zero4();
 #pragma unroll
     for (int q = 0; q < 8; ++q)
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
         const int n0 = 32 * ks + 8 * kb;
-        bq[q][ks] = n0 < r ? keep_first(ld16(W2 + (int64_t)(c0 + 8 * li + q) * a.ld_expand + n0), r - n0) : zero4();
+        bq[u][q][ks] =
+            n0 < r ? keep_first(ld16(W2 + (int64_t)(c0 + 8 * li + q) * a.ld_expand + n0), r - n0) : zero4();
       }
+  }
+#pragma unroll
+  for (int u = 0; u < CPW; ++u) {
+    if (cg0 + u >= ngroups) break;
+    const int c0 = (cg0 + u) << 7;
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
       f32x4 d[8];
@@ -193,21 +248,18 @@ __global__ __launch_bounds__(NW * 64) void k_pass_mfma(PassArgs a, const TileInf
       for (int q = 0; q < 8; ++q) {
         d[q] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) d[q] = mfma16(hop[tt][ks], bq[q][ks], d[q]);
+        for (int ks = 0; ks < NKS; ++ks) d[q] = mfma16(hop[tt][ks], bq[u][q][ks], d[q]);
       }
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const int row = 16 * tt + 4 * kb + v;
-        if (row < cnt) {
-          bf16_t* yp = dst + (int64_t)rows_s[row] * a.ld_dst + c0 + 8 * li;
-          const uint4 y = ld16(yp);
-          uint4 o;
-          o.x = pack_bf16(bf16_lo(y.x) + d[0][v], bf16_hi(y.x) + d[1][v]);
-          o.y = pack_bf16(bf16_lo(y.y) + d[2][v], bf16_hi(y.y) + d[3][v]);
-          o.z = pack_bf16(bf16_lo(y.z) + d[4][v], bf16_hi(y.z) + d[5][v]);
-          o.w = pack_bf16(bf16_lo(y.w) + d[6][v], bf16_hi(y.w) + d[7][v]);
-          st16(yp, o);
-        }
+        if (!yok[tt][v]) continue;
+        const uint4 yy = y[u][tt][v];
+        uint4 o;
+        o.x = pack_bf16(bf16_lo(yy.x) + d[0][v], bf16_hi(yy.x) + d[1][v]);
+        o.y = pack_bf16(bf16_lo(yy.y) + d[2][v], bf16_hi(yy.y) + d[3][v]);
+        o.z = pack_bf16(bf16_lo(yy.z) + d[4][v], bf16_hi(yy.z) + d[5][v]);
+        o.w = pack_bf16(bf16_lo(yy.w) + d[6][v], bf16_hi(yy.w) + d[7][v]);
+        st16(yp[tt][v] + c0, o);
       }
     }
   }
@@ -329,10 +381,16 @@ __global__ __launch_bounds__(256) void k_wgrad_mfma(WgradArgs a, const ChunkInfo
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-template <int NB, int NW>
+template <int NB, int NW, int PF, int CPW>
 void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
-  const unsigned grid = (unsigned)round_up(L.max_tiles, 8);
-  hipLaunchKernelGGL((k_pass_mfma<NB, NW>), dim3(grid), dim3(NW * 64), 0, s, a, seg.tiles, seg.perm, seg.header);
+  bf16_t* hrow = (bf16_t*)a.hT + (int64_t)a.rpad * a.ldh;  // second half of the h buffer
+  hipLaunchKernelGGL((k_shrink_mfma<NB, NW, PF>), dim3((unsigned)L.max_tiles), dim3(NW * 64), 0, s, a, hrow,
+                     seg.tiles, seg.perm, seg.header);
+  if (!a.dst) return;
+  const int64_t ngroups = a.width_dst >> 7;
+  const int64_t items = L.max_tiles * ceil_div(ngroups, CPW);
+  hipLaunchKernelGGL((k_expand_mfma<NB, CPW>), dim3((unsigned)ceil_div(items, 4)), dim3(256), 0, s, a, hrow,
+                     seg.tiles, seg.perm, seg.header);
 }
 
 template <int NB>
@@ -355,9 +413,9 @@ bool pass_mfma_supported(const PassArgs& a) {
 
 int launch_pass_mfma(const PassArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
   if (L.rows == 0) return TK_OK;
-  if (a.rpad <= 16) launch_pass<1, 8>(a, seg, L, s);
-  else if (a.rpad <= 32) launch_pass<2, 8>(a, seg, L, s);
-  else launch_pass<4, 4>(a, seg, L, s);
+  if (a.rpad <= 16) launch_pass<1, 4, 4, 2>(a, seg, L, s);
+  else if (a.rpad <= 32) launch_pass<2, 4, 4, 2>(a, seg, L, s);
+  else launch_pass<4, 4, 2, 1>(a, seg, L, s);
   return check_launch();
 }
 

@@ -123,7 +123,7 @@ struct BwdLayout {
     ldh = h_ld(d.rows);
     const int64_t e = elt_bytes(d.dtype);
     int64_t o = 0;
-    off_dh = o;         o += round_up(rpad * ldh * e, 256);
+    off_dh = o;         o += round_up(2 * rpad * ldh * e, 256);  // rank-major + position-major copies
     // B^T per group [rpad][M]  (shrink weight of the backward pass)
     off_wT_shrink = o;  o += round_up((int64_t)d.num_groups * rpad * d.out_features * e, 256);
     // A^T per group [K][rpad]  (expand weight of the backward pass)
