@@ -123,9 +123,11 @@ int tk_unpermute_weight_grad(const void* dout, int64_t ld_dout, const void* rows
 }
 
 int64_t tk_lora_h_bytes(const tk_lora_desc* d) {
-  if (!d || d->rows < 0 || d->max_rank < 0 || d->max_rank > TK_MAX_RANK) return TK_ERR_INVALID;
-  // rank-major copy hT[rpad][ld] followed by the position-major copy hrow[ld][rpad]
-  return round_up(2 * (int64_t)rank_pad(d->max_rank) * h_ld(d->rows) * elt_bytes(d->dtype), 256);
+  if (!d || d->rows < 0 || d->num_groups <= 0 || d->max_rank < 0 || d->max_rank > TK_MAX_RANK) return TK_ERR_INVALID;
+  // rank-major copy hT[rpad][ld], slot-major copy hrow[ld][rpad], then the partial sums of a split shrink
+  const int rpad = rank_pad(d->max_rank);
+  return round_up(2 * (int64_t)rpad * h_ld(d->rows, d->num_groups) * elt_bytes(d->dtype), 256) +
+         shrink_partial_bytes(d->rows, d->num_groups, d->in_features, rpad);
 }
 
 int64_t tk_lora_bwd_workspace_bytes(const tk_lora_desc* d) {
@@ -143,12 +145,15 @@ int tk_lora_fwd(const tk_lora_desc* d, const void* x, int64_t ldx, void* y, int6
   PassArgs a{};
   a.src = x;  a.ld_src = ldx;
   a.dst = y;  a.ld_dst = ldy;
-  a.hT = h;   a.ldh = h_ld(d->rows);
+  a.hT = h;   a.ldh = h_ld(d->rows, d->num_groups);
   a.w_shrink = d->lora_A;  a.ld_shrink = d->lda;
   a.w_expand = d->lora_B;  a.ld_expand = d->ldb;
   a.rank = d->rank;  a.scale = d->scale;
   a.width_src = d->in_features;  a.width_dst = d->out_features;
-  a.map_rows = d->map_rows;  a.rpad = rank_pad(d->max_rank);
+  a.map_rows = d->map_rows;  a.rpad = rank_pad(d->max_rank);  a.src_rows = (int32_t)d->rows;
+  a.hpart = (float*)((char*)h + round_up(2 * (int64_t)a.rpad * a.ldh * elt_bytes(d->dtype), 256));
+  a.tile_ticket = V.tile_ticket;
+  a.kslices = shrink_kslices(d->in_features, a.rpad);
   return run_pass(a, V, L, d->dtype, (hipStream_t)stream);
 }
 
@@ -181,7 +186,10 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
     a.w_expand_base = aT;  a.ld_expand = B.rpad;           a.expand_group_stride = B.rpad * d->in_features;
     a.rank = d->rank;  a.scale = d->scale;
     a.width_src = d->out_features;  a.width_dst = d->in_features;
-    a.map_rows = d->map_rows;  a.rpad = (int32_t)B.rpad;
+    a.map_rows = d->map_rows;  a.rpad = (int32_t)B.rpad;  a.src_rows = (int32_t)d->rows;
+    a.hpart = (float*)(w + B.off_hpart);
+    a.tile_ticket = V.tile_ticket;
+    a.kslices = shrink_kslices(d->out_features, a.rpad);
     if ((rc = run_pass(a, V, L, d->dtype, s)) != TK_OK) return rc;
   }
   if (grad_A) {

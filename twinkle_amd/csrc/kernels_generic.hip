@@ -13,25 +13,22 @@ namespace {
 
 constexpr int kKC = 64;   // source columns staged per step in the shrink kernel
 
-// hT[n][p] = scale_g * sum_k src[row(p)][k] * W_g[n][k]   for the rows of one tile
+// hT[n][slot] = scale_g * sum_k src[row(slot)][k] * W_g[n][k]   for the 32 slots of one tile
 template <typename T>
-__global__ __launch_bounds__(256) void k_shrink_generic(PassArgs a, const TileInfo* __restrict__ tiles,
-                                                        const int32_t* __restrict__ perm, const SegHeader* hdr) {
+__global__ __launch_bounds__(256) void k_shrink_generic(PassArgs a, const int32_t* __restrict__ tile_group,
+                                                        const int32_t* __restrict__ slot_rows) {
   extern __shared__ float lds_f[];
   const int tile_id = blockIdx.x;
-  if (tile_id >= hdr->num_tiles) return;
-  const TileInfo ti = tiles[tile_id];
-  const int g = ti.group;
+  const int g = tile_group[tile_id];
+  if (g < 0) return;
   const int r = min(a.rank[g], a.rpad);
   const int rpad = a.rpad;
   float* xs = lds_f;                          // [32][kKC + 1]
   float* ws = lds_f + kTileRows * (kKC + 1);  // [rpad][kKC + 1]
   __shared__ int rows_s[kTileRows];
   const int tid = threadIdx.x;
-  if (tid < kTileRows) {
-    const int p = ti.start + min(tid, ti.count - 1);
-    rows_s[tid] = a.map_rows ? perm[p] : p;
-  }
+  const int slot0 = tile_id * kTileRows;
+  if (tid < kTileRows) rows_s[tid] = slot_rows[slot0 + tid];
   __syncthreads();
   const T* src = (const T*)a.src;
   const T* W = group_weight<T>(a.w_shrink, a.w_shrink_base, a.shrink_group_stride, g);
@@ -45,7 +42,8 @@ __global__ __launch_bounds__(256) void k_shrink_generic(PassArgs a, const TileIn
     for (int i = tid; i < kTileRows * kKC; i += 256) {
       const int rr = i / kKC, kk = i % kKC;
       const int k = k0 + kk;
-      xs[rr * (kKC + 1) + kk] = k < a.width_src ? to_f32(src[(int64_t)rows_s[rr] * a.ld_src + k]) : 0.f;
+      xs[rr * (kKC + 1) + kk] =
+          (k < a.width_src && rows_s[rr] >= 0) ? to_f32(src[(int64_t)rows_s[rr] * a.ld_src + k]) : 0.f;
     }
     for (int i = tid; i < rpad * kKC; i += 256) {
       const int n = i / kKC, kk = i % kKC;
@@ -61,38 +59,40 @@ __global__ __launch_bounds__(256) void k_shrink_generic(PassArgs a, const TileIn
     }
     __syncthreads();
   }
-  const float sc = a.scale[g];
+  const float sc = r > 0 ? a.scale[g] : 0.f;
   T* hT = (T*)a.hT;
-  if (row < ti.count) {
+  T* hrow = hT + (int64_t)rpad * a.ldh;
+  // padding slots hold exact zeros so that the row-contraction kernels need no masks
 #pragma unroll
-    for (int j = 0; j < TK_MAX_RANK / 8; ++j) {
-      const int n = ng + 8 * j;
-      if (n < rpad) from_f32(n < r ? acc[j] * sc : 0.f, &hT[(int64_t)n * a.ldh + ti.start + row]);
+  for (int j = 0; j < TK_MAX_RANK / 8; ++j) {
+    const int n = ng + 8 * j;
+    if (n < rpad) {
+      T hv;
+      from_f32((n < r && rows_s[row] >= 0) ? acc[j] * sc : 0.f, &hv);
+      hT[(int64_t)n * a.ldh + slot0 + row] = hv;
+      hrow[(int64_t)(slot0 + row) * rpad + n] = hv;
     }
   }
 }
 
-// dst[row(p)][c] += sum_n hT[n][p] * W_g[c][n]   for the rows of one tile
+// dst[row(slot)][c] += sum_n hT[n][slot] * W_g[c][n]   for the 32 slots of one tile
 template <typename T>
-__global__ __launch_bounds__(256) void k_expand_generic(PassArgs a, const TileInfo* __restrict__ tiles,
-                                                        const int32_t* __restrict__ perm, const SegHeader* hdr) {
+__global__ __launch_bounds__(256) void k_expand_generic(PassArgs a, const int32_t* __restrict__ tile_group,
+                                                        const int32_t* __restrict__ slot_rows) {
   extern __shared__ float lds_f[];  // hs[rpad][32]
   const int tile_id = blockIdx.x;
-  if (tile_id >= hdr->num_tiles) return;
-  const TileInfo ti = tiles[tile_id];
-  const int g = ti.group;
+  const int g = tile_group[tile_id];
+  if (g < 0) return;
   const int r = min(a.rank[g], a.rpad);
   if (r <= 0) return;
   __shared__ int rows_s[kTileRows];
   const int tid = threadIdx.x;
-  if (tid < kTileRows) {
-    const int p = ti.start + min(tid, ti.count - 1);
-    rows_s[tid] = a.map_rows ? perm[p] : p;
-  }
+  const int slot0 = tile_id * kTileRows;
+  if (tid < kTileRows) rows_s[tid] = slot_rows[slot0 + tid];
   const T* hT = (const T*)a.hT;
   for (int i = tid; i < r * kTileRows; i += 256) {
     const int n = i / kTileRows, rr = i % kTileRows;
-    lds_f[i] = rr < ti.count ? to_f32(hT[(int64_t)n * a.ldh + ti.start + rr]) : 0.f;
+    lds_f[i] = to_f32(hT[(int64_t)n * a.ldh + slot0 + rr]);
   }
   __syncthreads();
   const T* W = group_weight<T>(a.w_expand, a.w_expand_base, a.expand_group_stride, g);
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(256) void k_expand_generic(PassArgs a, const TileIn
     }
 #pragma unroll
     for (int rr = 0; rr < kTileRows; ++rr) {
-      if (rr < ti.count) {
+      if (rows_s[rr] >= 0) {
         T* o = dst + (int64_t)rows_s[rr] * a.ld_dst + c;
         from_f32(to_f32(*o) + acc[rr], o);
       }
@@ -125,30 +125,30 @@ __device__ inline void store_grad(const WgradArgs& a, int g, int n, int c, float
   from_f32(v, o);
 }
 
-// One chunk of rows of one group, 256 columns per block:
-// out[n][c] = sum_{p in chunk} hT[n][p] * src[row(p)][c], p ascending.
+// One chunk (up to 16 tiles) of one group, 256 columns per block:
+// out[n][c] = sum_{slot in chunk} hT[n][slot] * src[row(slot)][c], slots ascending.
 template <typename T>
 __global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkInfo* __restrict__ chunks,
-                                                       const int32_t* __restrict__ perm, const SegHeader* hdr) {
+                                                       const int32_t* __restrict__ slot_rows) {
   __shared__ float hs[16][kChunkRows];
   __shared__ int rows_s[kChunkRows];
-  const int chunk_id = blockIdx.x;
-  if (chunk_id >= hdr->num_chunks) return;
-  const ChunkInfo ci = chunks[chunk_id];
+  const ChunkInfo ci = chunks[blockIdx.x];
   const int g = ci.group;
+  if (g < 0) return;
   const int r = min(a.rank[g], a.rpad);
   if (r <= 0) return;
   const int tid = threadIdx.x;
   const int c = blockIdx.y * 256 + tid;
-  const int len = ci.end - ci.start;
-  for (int i = tid; i < len; i += 256) rows_s[i] = a.map_rows ? perm[ci.start + i] : ci.start + i;
+  const int slot0 = ci.tile0 * kTileRows;
+  const int len = ci.ntiles * kTileRows;
+  for (int i = tid; i < len; i += 256) rows_s[i] = slot_rows[slot0 + i];
   const T* src = (const T*)a.src;
   const T* hT = (const T*)a.hT;
   for (int n0 = 0; n0 < r; n0 += 16) {
     __syncthreads();
     for (int i = tid; i < 16 * len; i += 256) {
       const int j = i / len, pp = i % len;
-      hs[j][pp] = (n0 + j) < r ? to_f32(hT[(int64_t)(n0 + j) * a.ldh + ci.start + pp]) : 0.f;
+      hs[j][pp] = (n0 + j) < r ? to_f32(hT[(int64_t)(n0 + j) * a.ldh + slot0 + pp]) : 0.f;
     }
     __syncthreads();
     if (c < a.width) {
@@ -156,6 +156,7 @@ __global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkI
 #pragma unroll
       for (int j = 0; j < 16; ++j) acc[j] = 0.f;
       for (int pp = 0; pp < len; ++pp) {
+        if (rows_s[pp] < 0) continue;
         const float xv = to_f32(src[(int64_t)rows_s[pp] * a.ld_src + c]);
 #pragma unroll
         for (int j = 0; j < 16; ++j) acc[j] += hs[j][pp] * xv;
@@ -175,24 +176,32 @@ __global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkI
 }
 
 // Groups with several chunks: sum their partials in chunk order.  Groups with
-// no rows: clear the live block when overwriting.
+// no rows: clear the live block when overwriting.  One (group, rank index,
+// 256 columns) per block.
 template <typename T>
 __global__ __launch_bounds__(256) void k_wgrad_reduce(WgradArgs a, const int32_t* __restrict__ chunk_first,
                                                       const int32_t* __restrict__ partial_first) {
   const int g = blockIdx.x;
-  const int r = min(a.rank[g], a.rpad);
-  if (r <= 0) return;
+  const int n = blockIdx.z;
+  if (n >= min(a.rank[g], a.rpad)) return;
   const int nchunk = chunk_first[g + 1] - chunk_first[g];
   if (nchunk == 1) return;
   if (nchunk == 0 && a.accumulate) return;
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= a.width) return;
-  const int p0 = partial_first[g];
-  for (int n = 0; n < r; ++n) {
-    float acc = 0.f;
-    for (int j = 0; j < nchunk; ++j) acc += a.partial[((int64_t)(p0 + j) * a.rpad + n) * a.width + c];
-    store_grad<T>(a, g, n, c, acc);
+  const float* p = a.partial + ((int64_t)partial_first[g] * a.rpad + n) * a.width + c;
+  const int64_t stride = (int64_t)a.rpad * a.width;
+  float acc = 0.f;
+  int j = 0;
+  for (; j + 4 <= nchunk; j += 4) {
+    const float v0 = p[(j + 0) * stride], v1 = p[(j + 1) * stride], v2 = p[(j + 2) * stride], v3 = p[(j + 3) * stride];
+    acc += v0;
+    acc += v1;
+    acc += v2;
+    acc += v3;
   }
+  for (; j < nchunk; ++j) acc += p[j * stride];
+  store_grad<T>(a, g, n, c, acc);
 }
 
 // bT_g[n][m] = B_g[m][n], aT_g[k][n] = A_g[n][k]; zero for n >= rank[g].
@@ -221,20 +230,17 @@ __global__ __launch_bounds__(256) void k_transpose_weights(tk_lora_desc d, int r
 int launch_pass_generic(const PassArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s) {
   if (L.rows == 0) return TK_OK;
   const unsigned grid = (unsigned)L.max_tiles;
+  const int32_t* rows = seg.slot_table(a.map_rows);
   const size_t lds_shrink = sizeof(float) * (size_t)(kTileRows + a.rpad) * (kKC + 1);
   const size_t lds_expand = sizeof(float) * (size_t)a.rpad * kTileRows;
   if (dtype == TK_DTYPE_F32) {
-    hipLaunchKernelGGL(k_shrink_generic<float>, dim3(grid), dim3(256), lds_shrink, s, a, seg.tiles, seg.perm,
-                       seg.header);
+    hipLaunchKernelGGL(k_shrink_generic<float>, dim3(grid), dim3(256), lds_shrink, s, a, seg.tile_group, rows);
     if (a.dst)
-      hipLaunchKernelGGL(k_expand_generic<float>, dim3(grid), dim3(256), lds_expand, s, a, seg.tiles, seg.perm,
-                         seg.header);
+      hipLaunchKernelGGL(k_expand_generic<float>, dim3(grid), dim3(256), lds_expand, s, a, seg.tile_group, rows);
   } else {
-    hipLaunchKernelGGL(k_shrink_generic<bf16_t>, dim3(grid), dim3(256), lds_shrink, s, a, seg.tiles, seg.perm,
-                       seg.header);
+    hipLaunchKernelGGL(k_shrink_generic<bf16_t>, dim3(grid), dim3(256), lds_shrink, s, a, seg.tile_group, rows);
     if (a.dst)
-      hipLaunchKernelGGL(k_expand_generic<bf16_t>, dim3(grid), dim3(256), lds_expand, s, a, seg.tiles, seg.perm,
-                         seg.header);
+      hipLaunchKernelGGL(k_expand_generic<bf16_t>, dim3(grid), dim3(256), lds_expand, s, a, seg.tile_group, rows);
   }
   return check_launch();
 }
@@ -243,15 +249,15 @@ int launch_wgrad_generic(const WgradArgs& a, const SegView& seg, const SegLayout
   if (L.rows == 0) return TK_OK;
   const dim3 grid((unsigned)L.max_chunks, (unsigned)ceil_div(a.width, 256));
   if (dtype == TK_DTYPE_F32)
-    hipLaunchKernelGGL(k_wgrad_generic<float>, grid, dim3(256), 0, s, a, seg.chunks, seg.perm, seg.header);
+    hipLaunchKernelGGL(k_wgrad_generic<float>, grid, dim3(256), 0, s, a, seg.chunks, seg.slot_table(a.map_rows));
   else
-    hipLaunchKernelGGL(k_wgrad_generic<bf16_t>, grid, dim3(256), 0, s, a, seg.chunks, seg.perm, seg.header);
+    hipLaunchKernelGGL(k_wgrad_generic<bf16_t>, grid, dim3(256), 0, s, a, seg.chunks, seg.slot_table(a.map_rows));
   return check_launch();
 }
 
 int launch_wgrad_reduce(const WgradArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s) {
   if (L.groups == 0) return TK_OK;
-  const dim3 grid((unsigned)L.groups, (unsigned)ceil_div(a.width, 256));
+  const dim3 grid((unsigned)L.groups, (unsigned)ceil_div(a.width, 256), (unsigned)a.rpad);
   if (dtype == TK_DTYPE_F32)
     hipLaunchKernelGGL(k_wgrad_reduce<float>, grid, dim3(256), 0, s, a, seg.chunk_first, seg.partial_first);
   else

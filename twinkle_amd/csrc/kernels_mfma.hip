@@ -52,50 +52,78 @@ __device__ inline uint4 keep_first(uint4 v, int keep) {
   }
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
-// keep elements [lo, hi) of a quad
-__device__ inline uint4 keep_range(uint4 v, int lo, int hi) {
-  uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-  for (int d = 0; d < 4; ++d) {
-    const bool e0 = (2 * d) >= lo && (2 * d) < hi, e1 = (2 * d + 1) >= lo && (2 * d + 1) < hi;
-    w[d] &= (e0 ? 0xffffu : 0u) | (e1 ? 0xffff0000u : 0u);
+// Scales, rounds and writes one tile of h from `planes` partial planes in LDS ([plane][32][RP + 1]):
+// slot-major (hrow) and rank-major (hT); padding slots (row >= cnt) get exact zeros.
+template <int RP, int THREADS>
+__device__ inline void shrink_epilogue(const float* part, int planes, const PassArgs& a, bf16_t* __restrict__ hrow,
+                                       int slot0, int cnt, float sc) {
+  constexpr int PR = RP + 1;
+  const int tid = threadIdx.x;
+  bf16_t* hT = (bf16_t*)a.hT;
+  // slot-major copy: consecutive threads -> consecutive rank indices of one slot
+  for (int idx = tid; idx < kTileRows * RP; idx += THREADS) {
+    const int row = idx / RP, n = idx % RP;
+    float sum = 0.f;
+    for (int w = 0; w < planes; ++w) sum += part[(w * kTileRows + row) * PR + n];
+    hrow[(int64_t)(slot0 + row) * RP + n] = row < cnt ? (bf16_t)(pack_bf16(sum * sc, 0.f) & 0xffffu) : (bf16_t)0;
   }
-  return make_uint4(w[0], w[1], w[2], w[3]);
+  // rank-major copy: consecutive threads -> consecutive slots of one rank index
+  for (int idx = tid; idx < kTileRows * RP; idx += THREADS) {
+    const int n = idx >> 5, row = idx & 31;
+    float sum = 0.f;
+    for (int w = 0; w < planes; ++w) sum += part[(w * kTileRows + row) * PR + n];
+    hT[(int64_t)n * a.ldh + slot0 + row] = row < cnt ? (bf16_t)(pack_bf16(sum * sc, 0.f) & 0xffffu) : (bf16_t)0;
+  }
 }
 
 // ---------------------------------------------------------------------------
-// Shrink: h[p][n] = scale_g * sum_k src[row(p)][k] * W1_g[n][k] for one tile of up
-// to 32 rows of one group per workgroup.  The NW waves split the source width
-// in 64-column steps (interleaved, so the workgroup reads 64*NW contiguous
-// columns of each row at a time); every wave keeps its partial h[32][rank] in
-// MFMA accumulators, issuing the loads of PF steps before the first MFMA so
-// that ~PF*6 KB per wave are in flight.  Partials meet in LDS and are summed
-// in wave order (fixed order: bitwise repeatable), scaled, rounded to bf16
-// and written twice: position-major (hrow, the expand kernel's A operand) and
-// rank-major (hT, read by the weight-gradient kernel).
+// Shrink: h[slot][n] = scale_g * sum_k src[row(slot)][k] * W1_g[n][k].
+//
+// Work item = (tile of 32 padded slots, slice of 512*NW source columns), one
+// block of NW waves each; slices of one tile are consecutive blocks, so
+// neighbouring waves read neighbouring 1 KB pieces of the same rows.  The
+// grid is thousands of short independent streams: the hardware dispatcher
+// keeps every CU equally loaded, which a tile-per-workgroup split does not
+// (2.03 workgroups per CU leaves most CUs waiting for the few that got 3).
+// A wave takes 64-column steps, interleaved with the other waves of its
+// block, keeps its partial h[32][rank] in MFMA accumulators and issues the
+// loads of 4 steps before the first MFMA of the batch.  The waves' partials
+// meet in LDS; if the source is wider than one block the block sums go to a
+// global buffer and k_shrink_finish adds the slices in slice order (a device-
+// scope fence per block, the alternative, costs a cache write-back on this
+// multi-die part).  Summation order is fixed throughout: results are bitwise
+// repeatable.  The result is scaled, rounded
+// to bf16 and written twice: slot-major (hrow, the expand kernel's A operand)
+// and rank-major (hT, read by the weight-gradient kernel); padding slots get
+// exact zeros.  Nothing branches before the source loads are in flight.
 // ---------------------------------------------------------------------------
-template <int NB, int NW, int PF>
+template <int NB, int NW>
 __global__ __launch_bounds__(NW * 64) void k_shrink_mfma(PassArgs a, bf16_t* __restrict__ hrow,
-                                                         const TileInfo* __restrict__ tiles,
-                                                         const int32_t* __restrict__ perm, const SegHeader* hdr) {
+                                                         const int32_t* __restrict__ tile_group,
+                                                         const int32_t* __restrict__ slot_rows) {
   constexpr int RP = 16 * NB;  // padded rank
   constexpr int PR = RP + 1;   // row stride of the partial sums (floats; odd: conflict-free column reads)
+  constexpr int PF = 4;        // steps whose loads are issued together
   __shared__ float part[NW][kTileRows][PR];
 
-  const int tile_id = blockIdx.x;
-  if (tile_id >= hdr->num_tiles) return;
-  const TileInfo ti = tiles[tile_id];
-  const int g = ti.group;
-  const int r = min(a.rank[g], RP);
-  if (r <= 0) return;  // adapter not live on this layer
-  const int cnt = ti.count;
+  const int kslices = a.kslices;
+  const int tile_id = blockIdx.x / kslices, ks = blockIdx.x - tile_id * kslices;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  const int slot0 = tile_id * kTileRows;
+  // independent first loads (a tile of an unused table entry or of an adapter that is not live
+  // computes zeros and is dropped below)
+  const int g_raw = tile_group[tile_id];
+  int ra = slot_rows[slot0 + li], rb = slot_rows[slot0 + 16 + li];
+  const int g = max(g_raw, 0);
+  // padding is always at the end of a tile: count the valid slots
+  const int cnt = g_raw < 0 ? 0 : __popcll(__ballot(ra >= 0) & 0xffffull) + __popcll(__ballot(rb >= 0) & 0xffffull);
+  ra = min(max(ra, 0), a.src_rows - 1);
+  rb = min(max(rb, 0), a.src_rows - 1);
+  const int r = g_raw < 0 ? 0 : min(a.rank[g], RP);
 
-  const int pa = ti.start + min(li, cnt - 1), pb = ti.start + min(16 + li, cnt - 1);
-  const int64_t ra = a.map_rows ? perm[pa] : pa, rb = a.map_rows ? perm[pb] : pb;
   const bf16_t* src = (const bf16_t*)a.src;
-  const bf16_t* xa = src + ra * a.ld_src + 16 * kb;
-  const bf16_t* xb = src + rb * a.ld_src + 16 * kb;
+  const bf16_t* xa = src + (int64_t)ra * a.ld_src + 16 * kb;
+  const bf16_t* xb = src + (int64_t)rb * a.ld_src + 16 * kb;
   const bf16_t* W1 = group_weight<bf16_t>(a.w_shrink, a.w_shrink_base, a.shrink_group_stride, g);
   const bf16_t* wp[NB];
   bool wv[NB];
@@ -105,20 +133,25 @@ __global__ __launch_bounds__(NW * 64) void k_shrink_mfma(PassArgs a, bf16_t* __r
     wv[nb] = n < r;
     wp[nb] = W1 + (int64_t)(wv[nb] ? n : 0) * a.ld_shrink + 16 * kb;
   }
-  f32x4 acc[2][NB];
+  // two accumulators per output tile so that consecutive MFMAs are independent
+  f32x4 acc[2][NB][2];
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    acc[0][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
-    acc[1][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      acc[0][nb][e] = f32x4{0.f, 0.f, 0.f, 0.f};
+      acc[1][nb][e] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
   const int nsteps = a.width_src >> 6;
-  for (int s0 = wave; s0 < nsteps; s0 += NW * PF) {
+  const int s_first = ks * (kShrinkSteps * NW) + wave;
+#pragma unroll
+  for (int b = 0; b < kShrinkSteps / PF; ++b) {
     uint4 xa0[PF], xa1[PF], xb0[PF], xb1[PF], w0[PF][NB], w1[PF][NB];
 #pragma unroll
     for (int j = 0; j < PF; ++j) {
-      const int s = s0 + j * NW;
+      const int s = s_first + (b * PF + j) * NW;
       const bool ok = s < nsteps;  // wave-uniform
-      const int c = (ok ? s : s0) << 6;
+      const int c = (ok ? s : 0) << 6;
       xa0[j] = ld16(xa + c);
       xa1[j] = ld16(xa + c + 8);
       xb0[j] = ld16(xb + c);
@@ -133,89 +166,111 @@ __global__ __launch_bounds__(NW * 64) void k_shrink_mfma(PassArgs a, bf16_t* __r
     for (int j = 0; j < PF; ++j)
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
-        acc[0][nb] = mfma16(xa0[j], w0[j][nb], acc[0][nb]);
-        acc[1][nb] = mfma16(xb0[j], w0[j][nb], acc[1][nb]);
-        acc[0][nb] = mfma16(xa1[j], w1[j][nb], acc[0][nb]);
-        acc[1][nb] = mfma16(xb1[j], w1[j][nb], acc[1][nb]);
+        acc[0][nb][0] = mfma16(xa0[j], w0[j][nb], acc[0][nb][0]);
+        acc[1][nb][0] = mfma16(xb0[j], w0[j][nb], acc[1][nb][0]);
+        acc[0][nb][1] = mfma16(xa1[j], w1[j][nb], acc[0][nb][1]);
+        acc[1][nb][1] = mfma16(xb1[j], w1[j][nb], acc[1][nb][1]);
       }
   }
+  if (r <= 0) return;  // unused tile, or adapter not live on this layer (uniform over the tile's blocks)
 #pragma unroll
   for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) part[wave][16 * tt + 4 * kb + v][16 * nb + li] = acc[tt][nb][v];
+      for (int v = 0; v < 4; ++v)
+        part[wave][16 * tt + 4 * kb + v][16 * nb + li] = acc[tt][nb][0][v] + acc[tt][nb][1][v];
   __syncthreads();
 
-  const float sc = a.scale[g];
-  bf16_t* hT = (bf16_t*)a.hT;
-  // position-major copy: consecutive threads -> consecutive rank indices of one row
-  for (int idx = tid; idx < kTileRows * RP; idx += NW * 64) {
-    const int row = idx / RP, n = idx % RP;
-    float sum = 0.f;
+  if (a.kslices > 1) {
+    // the source is wider than one block: leave this block's sums for k_shrink_finish
+    float* mine = a.hpart + ((int64_t)tile_id * kslices + ks) * (kTileRows * RP);
+    for (int idx = tid; idx < kTileRows * RP; idx += NW * 64) {
+      const int row = idx / RP, n = idx % RP;
+      float sum = 0.f;
 #pragma unroll
-    for (int w = 0; w < NW; ++w) sum += part[w][row][n];
-    if (row < cnt) hrow[(int64_t)(ti.start + row) * RP + n] = (bf16_t)(pack_bf16(sum * sc, 0.f) & 0xffffu);
+      for (int w = 0; w < NW; ++w) sum += part[w][row][n];
+      mine[idx] = sum;
+    }
+    return;
   }
-  // rank-major copy: consecutive threads -> consecutive rows of one rank index
-  for (int idx = tid; idx < kTileRows * RP; idx += NW * 64) {
-    const int n = idx >> 5, row = idx & 31;
+  shrink_epilogue<RP, NW * 64>(&part[0][0][0], NW, a, hrow, slot0, cnt, a.scale[g]);
+}
+
+// Adds the slices of a split shrink in slice order and writes h (one block per tile).
+template <int NB>
+__global__ __launch_bounds__(256) void k_shrink_finish(PassArgs a, bf16_t* __restrict__ hrow,
+                                                       const int32_t* __restrict__ tile_group,
+                                                       const int32_t* __restrict__ slot_rows) {
+  constexpr int RP = 16 * NB, PR = RP + 1;
+  __shared__ float part[kTileRows][PR];
+  const int tile_id = blockIdx.x, tid = threadIdx.x;
+  const int g = tile_group[tile_id];
+  if (g < 0) return;
+  if (a.rank[g] <= 0) return;
+  const int slot0 = tile_id * kTileRows;
+  int cnt = 0;
+  for (int i = 0; i < kTileRows; ++i) cnt += slot_rows[slot0 + i] >= 0;
+  const float* tile_part = a.hpart + (int64_t)tile_id * a.kslices * (kTileRows * RP);
+  for (int idx = tid; idx < kTileRows * RP; idx += 256) {
     float sum = 0.f;
-#pragma unroll
-    for (int w = 0; w < NW; ++w) sum += part[w][row][n];
-    if (row < cnt) hT[(int64_t)n * a.ldh + ti.start + row] = (bf16_t)(pack_bf16(sum * sc, 0.f) & 0xffffu);
+    for (int k = 0; k < a.kslices; ++k) sum += tile_part[(int64_t)k * (kTileRows * RP) + idx];
+    part[idx / RP][idx % RP] = sum;
   }
+  __syncthreads();
+  shrink_epilogue<RP, 256>(&part[0][0], 1, a, hrow, slot0, cnt, a.scale[g]);
 }
 
 // ---------------------------------------------------------------------------
-// Expand: dst[row(p)][c] += sum_n h[p][n] * W2_g[c][n], read-modify-write in
-// place.  Work is flat: one wave owns CPW adjacent 128-column groups of one
-// 32-row tile and nothing is shared between waves, so the grid is thousands
-// of independent streams.  Column c0 + 8 j + q of a group is output column j
-// of MFMA q, which makes each lane's 8 results of one row 16 contiguous
-// bytes and each wave-wide access 4 rows x 256 B.
+// Expand: dst[row(slot)][c] += sum_n h[slot][n] * W2_g[c][n], read-modify-write
+// in place.  Work is flat: one wave owns CPW adjacent 128-column groups of one
+// tile and nothing is shared between waves, so the grid is thousands of
+// independent streams.  Column c0 + 8 j + q of a group is output column j of
+// MFMA q, which makes each lane's 8 results of one row 16 contiguous bytes and
+// each wave-wide access 4 rows x 256 B.  Row indices, h and the group id are
+// addressed from the work-item number alone, so the destination loads are one
+// dependent step away from the start of the wave.
 // ---------------------------------------------------------------------------
 template <int NB, int CPW>
 __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* __restrict__ hrow,
-                                                     const TileInfo* __restrict__ tiles,
-                                                     const int32_t* __restrict__ perm, const SegHeader* hdr) {
+                                                     const int32_t* __restrict__ tile_group,
+                                                     const int32_t* __restrict__ slot_rows, int num_items) {
   constexpr int RP = 16 * NB;
   constexpr int NKS = (RP + 31) / 32;  // contraction steps of the MFMAs
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
   const int ngroups = a.width_dst >> 7;
   const int items_per_tile = (ngroups + CPW - 1) / CPW;
   const int item = blockIdx.x * 4 + wave;
+  if (item >= num_items) return;
   const int tile_id = item / items_per_tile;
-  if (tile_id >= hdr->num_tiles) return;
   const int cg0 = (item - tile_id * items_per_tile) * CPW;
-  const TileInfo ti = tiles[tile_id];
-  const int g = ti.group;
-  const int r = min(a.rank[g], RP);
-  if (r <= 0) return;
-  const int cnt = ti.count;
-
-  // rows this lane updates: 16 tt + 4 kb + v
-  bf16_t* yp[2][4];
-  bool yok[2][4];
-#pragma unroll
-  for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const int row = 16 * tt + 4 * kb + v;
-      yok[tt][v] = row < cnt;
-      const int p = ti.start + min(row, cnt - 1);
-      const int64_t rr = a.map_rows ? perm[p] : p;
-      yp[tt][v] = (bf16_t*)a.dst + rr * a.ld_dst + 8 * li;
-    }
+  const int slot0 = tile_id * kTileRows;
+  // independent first loads: group id, row indices, h operand (nothing branches before the
+  // destination loads are in flight)
+  const int g_raw = tile_group[tile_id];
+  // rows this lane updates: slots 16 tt + 4 kb + v
+  const int4 r0 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 4 * kb);
+  const int4 r1 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 16 + 4 * kb);
   uint4 hop[2][NKS];
 #pragma unroll
   for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
       const int n0 = 32 * ks + 8 * kb;
-      const int p = ti.start + min(16 * tt + li, cnt - 1);
-      hop[tt][ks] = n0 < RP ? ld16(hrow + (int64_t)p * RP + n0) : zero4();
+      hop[tt][ks] = n0 < RP ? ld16(hrow + (int64_t)(slot0 + 16 * tt + li) * RP + n0) : zero4();
     }
+  const int g = max(g_raw, 0);
+  const int rows[2][4] = {{r0.x, r0.y, r0.z, r0.w}, {r1.x, r1.y, r1.z, r1.w}};
+  bool rok[2][4];
+  bf16_t* yp[2][4];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      rok[tt][v] = g_raw >= 0 && rows[tt][v] >= 0;
+      yp[tt][v] = (bf16_t*)a.dst + (int64_t)(rok[tt][v] ? rows[tt][v] : 0) * a.ld_dst + 8 * li;
+    }
+  const int r = g_raw < 0 ? 0 : min(a.rank[g], RP);
   const bf16_t* W2 = group_weight<bf16_t>(a.w_expand, a.w_expand_base, a.expand_group_stride, g);
 
   uint4 y[CPW][2][4];
@@ -227,7 +282,7 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) y[u][tt][v] = (yok[tt][v] && gok) ? ld16(yp[tt][v] + c0) : zero4();
+      for (int v = 0; v < 4; ++v) y[u][tt][v] = (rok[tt][v] && gok) ? ld16(yp[tt][v] + c0) : zero4();
 #pragma unroll
     for (int q = 0; q < 8; ++q)
 #pragma unroll
@@ -237,6 +292,7 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
             n0 < r ? keep_first(ld16(W2 + (int64_t)(c0 + 8 * li + q) * a.ld_expand + n0), r - n0) : zero4();
       }
   }
+  if (r <= 0) return;  // unused tile, or adapter not live on this layer (uniform over the wave)
 #pragma unroll
   for (int u = 0; u < CPW; ++u) {
     if (cg0 + u >= ngroups) break;
@@ -252,7 +308,7 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
       }
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        if (!yok[tt][v]) continue;
+        if (!rok[tt][v]) continue;
         const uint4 yy = y[u][tt][v];
         uint4 o;
         o.x = pack_bf16(bf16_lo(yy.x) + d[0][v], bf16_hi(yy.x) + d[1][v]);
@@ -266,68 +322,70 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
 }
 
 // ---------------------------------------------------------------------------
-// Row contraction (weight gradients): out[n][c] = sum_p hT[n][p] * src[row(p)][c]
-// over the rows of one chunk of one group.  One wave owns 128 columns; it
-// walks the chunk in 32-row windows aligned to absolute multiples of 32 (so
-// the hT loads are 16-byte aligned).  Each lane loads 8 rows x 8 columns
-// (eight fully coalesced wave loads of 4 x 256 B), transposes its 8x8 block in
-// registers with v_perm_b32 so that rows become the MFMA contraction index,
-// and accumulates 128 columns x rank in MFMA registers for the whole chunk.
+// Row contraction (weight gradients): out[n][c] = sum_slot hT[n][slot] * src[row(slot)][c]
+// over the tiles of one chunk of one group, for 128 columns per block.  The
+// NW waves of a block take the chunk's tiles in turn (wave w: tiles w, w+NW,
+// ...), so a chunk is many short streams, and add their accumulators in LDS in
+// wave order at the end.  Each lane loads 8 rows x 8 columns (eight fully
+// coalesced wave loads of 4 x 256 B), transposes its 8x8 block in registers
+// with v_perm_b32 so that rows become the MFMA contraction index, and
+// accumulates 128 columns x rank in MFMA registers.  The loads of a wave's
+// next tile are issued before its current tile is consumed.  Padding slots
+// contribute nothing: their h is exactly zero and their rows are not loaded.
 // ---------------------------------------------------------------------------
-template <int NB>
-__global__ __launch_bounds__(256) void k_wgrad_mfma(WgradArgs a, const ChunkInfo* __restrict__ chunks,
-                                                    const int32_t* __restrict__ perm, const SegHeader* hdr) {
-  const int chunk_id = blockIdx.x;
-  if (chunk_id >= hdr->num_chunks) return;
+template <int NB, int NW>
+__global__ __launch_bounds__(NW * 64) void k_wgrad_mfma(WgradArgs a, const ChunkInfo* __restrict__ chunks,
+                                                        const int32_t* __restrict__ slot_rows) {
+  __shared__ float red[NW > 1 ? NW - 1 : 1][8 * NB * 4][64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
-  const int c0 = (blockIdx.y * 4 + wave) * 128;
-  if (c0 >= a.width) return;
-  const ChunkInfo ci = chunks[chunk_id];
+  const int c0 = blockIdx.y * 128;
+  const ChunkInfo ci = chunks[blockIdx.x];
   const int g = ci.group;
+  if (g < 0) return;
   const int r = min(a.rank[g], 16 * NB);
   if (r <= 0) return;
 
   const bf16_t* src = (const bf16_t*)a.src + c0 + 8 * li;
   const bf16_t* hT = (const bf16_t*)a.hT + 8 * kb;
+  const int32_t* rows_p = slot_rows + ci.tile0 * kTileRows + 8 * kb;  // this lane's 8 slots of the chunk's first tile
   f32x4 acc[8][NB];
 #pragma unroll
   for (int q = 0; q < 8; ++q)
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) acc[q][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int w0 = ci.start & ~31; w0 < ci.end; w0 += 32) {
-    const int p0 = w0 + 8 * kb;  // first of this lane's 8 rows
-    const bool interior = w0 >= ci.start && w0 + 32 <= ci.end;
-    int rows[8];
-    if (a.map_rows) {
-      const int4 ra = *reinterpret_cast<const int4*>(perm + p0);
-      const int4 rb = *reinterpret_cast<const int4*>(perm + p0 + 4);
-      rows[0] = ra.x; rows[1] = ra.y; rows[2] = ra.z; rows[3] = ra.w;
-      rows[4] = rb.x; rows[5] = rb.y; rows[6] = rb.z; rows[7] = rb.w;
-    } else {
+  int4 ra = make_int4(-1, -1, -1, -1), rb = ra;
+  uint4 xn[8];
+  if (wave < ci.ntiles) {
+    ra = *reinterpret_cast<const int4*>(rows_p + wave * kTileRows);
+    rb = *reinterpret_cast<const int4*>(rows_p + wave * kTileRows + 4);
+    const int rows[8] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w};
 #pragma unroll
-      for (int q = 0; q < 8; ++q) rows[q] = p0 + q;
+    for (int q = 0; q < 8; ++q) xn[q] = rows[q] >= 0 ? ld16(src + (int64_t)rows[q] * a.ld_src) : zero4();
+    if (wave + NW < ci.ntiles) {
+      ra = *reinterpret_cast<const int4*>(rows_p + (wave + NW) * kTileRows);
+      rb = *reinterpret_cast<const int4*>(rows_p + (wave + NW) * kTileRows + 4);
     }
+  }
+  for (int t = wave; t < ci.ntiles; t += NW) {
+    const int w0 = (ci.tile0 + t) * kTileRows;
     uint4 x[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) x[q] = xn[q];
     uint4 h[NB];
-    if (interior) {
 #pragma unroll
-      for (int q = 0; q < 8; ++q) x[q] = ld16(src + (int64_t)rows[q] * a.ld_src);
+    for (int nb = 0; nb < NB; ++nb) h[nb] = ld16(hT + (int64_t)(16 * nb + li) * a.ldh + w0);
+    if (t + NW < ci.ntiles) {
+      const int rows[8] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w};
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) h[nb] = ld16(hT + (int64_t)(16 * nb + li) * a.ldh + w0);
-    } else {
-      // first / last window of the chunk: rows outside [start, end) belong to other groups
-#pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        const bool ok = p0 + q >= ci.start && p0 + q < ci.end;
-        x[q] = ok ? ld16(src + (int64_t)rows[q] * a.ld_src) : zero4();
+      for (int q = 0; q < 8; ++q) xn[q] = rows[q] >= 0 ? ld16(src + (int64_t)rows[q] * a.ld_src) : zero4();
+      if (t + 2 * NW < ci.ntiles) {
+        ra = *reinterpret_cast<const int4*>(rows_p + (t + 2 * NW) * kTileRows);
+        rb = *reinterpret_cast<const int4*>(rows_p + (t + 2 * NW) * kTileRows + 4);
       }
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        h[nb] = keep_range(ld16(hT + (int64_t)(16 * nb + li) * a.ldh + w0), ci.start - p0, ci.end - p0);
     }
-    // 8x8 transpose inside the lane: t[q] holds column q of the 8 rows
-    uint4 t[8];
+    // 8x8 transpose inside the lane: tr[q] holds column q of the 8 rows
+    uint4 tr[8];
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
       const int d = q >> 1;
@@ -338,15 +396,36 @@ __global__ __launch_bounds__(256) void k_wgrad_mfma(WgradArgs a, const ChunkInfo
         const uint32_t wsrc[4] = {x[i].x, x[i].y, x[i].z, x[i].w};
         e[i] = wsrc[d];
       }
-      t[q].x = __builtin_amdgcn_perm(e[1], e[0], sel);
-      t[q].y = __builtin_amdgcn_perm(e[3], e[2], sel);
-      t[q].z = __builtin_amdgcn_perm(e[5], e[4], sel);
-      t[q].w = __builtin_amdgcn_perm(e[7], e[6], sel);
+      tr[q].x = __builtin_amdgcn_perm(e[1], e[0], sel);
+      tr[q].y = __builtin_amdgcn_perm(e[3], e[2], sel);
+      tr[q].z = __builtin_amdgcn_perm(e[5], e[4], sel);
+      tr[q].w = __builtin_amdgcn_perm(e[7], e[6], sel);
     }
 #pragma unroll
     for (int q = 0; q < 8; ++q)
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) acc[q][nb] = mfma16(t[q], h[nb], acc[q][nb]);
+      for (int nb = 0; nb < NB; ++nb) acc[q][nb] = mfma16(tr[q], h[nb], acc[q][nb]);
+  }
+
+  // add the waves' accumulators in wave order; wave 0 writes the result
+  if (NW > 1) {
+    if (wave > 0) {
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) red[wave - 1][(q * NB + nb) * 4 + v][lane] = acc[q][nb][v];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    for (int w = 0; w < NW - 1; ++w)
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[q][nb][v] += red[w][(q * NB + nb) * 4 + v][lane];
   }
 
   // lane holds out[n = 16 nb + li][c0 + 32 kb + 8 v + q], q = 0..7, v = 0..3: 32 consecutive columns per n
@@ -381,22 +460,27 @@ __global__ __launch_bounds__(256) void k_wgrad_mfma(WgradArgs a, const ChunkInfo
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-template <int NB, int NW, int PF, int CPW>
+template <int NB, int CPW>
 void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
   bf16_t* hrow = (bf16_t*)a.hT + (int64_t)a.rpad * a.ldh;  // second half of the h buffer
-  hipLaunchKernelGGL((k_shrink_mfma<NB, NW, PF>), dim3((unsigned)L.max_tiles), dim3(NW * 64), 0, s, a, hrow,
-                     seg.tiles, seg.perm, seg.header);
+  const int32_t* rows = seg.slot_table(a.map_rows);
+  constexpr int NW = NB == 1 ? 1 : (NB == 2 ? 2 : 4);  // shrink_waves(16 * NB)
+  hipLaunchKernelGGL((k_shrink_mfma<NB, NW>), dim3((unsigned)(L.max_tiles * a.kslices)), dim3(NW * 64), 0, s, a, hrow,
+                     seg.tile_group, rows);
+  if (a.kslices > 1)
+    hipLaunchKernelGGL((k_shrink_finish<NB>), dim3((unsigned)L.max_tiles), dim3(256), 0, s, a, hrow, seg.tile_group,
+                       rows);
   if (!a.dst) return;
   const int64_t ngroups = a.width_dst >> 7;
   const int64_t items = L.max_tiles * ceil_div(ngroups, CPW);
   hipLaunchKernelGGL((k_expand_mfma<NB, CPW>), dim3((unsigned)ceil_div(items, 4)), dim3(256), 0, s, a, hrow,
-                     seg.tiles, seg.perm, seg.header);
+                     seg.tile_group, rows, (int)items);
 }
 
-template <int NB>
+template <int NB, int NW>
 void launch_wgrad(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
-  const dim3 grid((unsigned)L.max_chunks, (unsigned)ceil_div(a.width, 512));
-  hipLaunchKernelGGL((k_wgrad_mfma<NB>), grid, dim3(256), 0, s, a, seg.chunks, seg.perm, seg.header);
+  const dim3 grid((unsigned)L.max_chunks, (unsigned)(a.width / 128));
+  hipLaunchKernelGGL((k_wgrad_mfma<NB, NW>), grid, dim3(NW * 64), 0, s, a, seg.chunks, seg.slot_table(a.map_rows));
 }
 
 }  // namespace
@@ -413,9 +497,9 @@ bool pass_mfma_supported(const PassArgs& a) {
 
 int launch_pass_mfma(const PassArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
   if (L.rows == 0) return TK_OK;
-  if (a.rpad <= 16) launch_pass<1, 4, 4, 2>(a, seg, L, s);
-  else if (a.rpad <= 32) launch_pass<2, 4, 4, 2>(a, seg, L, s);
-  else launch_pass<4, 4, 2, 1>(a, seg, L, s);
+  if (a.rpad <= 16) launch_pass<1, 1>(a, seg, L, s);
+  else if (a.rpad <= 32) launch_pass<2, 1>(a, seg, L, s);
+  else launch_pass<4, 1>(a, seg, L, s);
   return check_launch();
 }
 
@@ -427,9 +511,9 @@ bool wgrad_mfma_supported(const WgradArgs& a) {
 
 int launch_wgrad_mfma(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
   if (L.rows == 0) return TK_OK;
-  if (a.rpad <= 16) launch_wgrad<1>(a, seg, L, s);
-  else if (a.rpad <= 32) launch_wgrad<2>(a, seg, L, s);
-  else launch_wgrad<4>(a, seg, L, s);
+  if (a.rpad <= 16) launch_wgrad<1, 4>(a, seg, L, s);
+  else if (a.rpad <= 32) launch_wgrad<2, 4>(a, seg, L, s);
+  else launch_wgrad<4, 2>(a, seg, L, s);
   return check_launch();
 }
 

@@ -4,11 +4,13 @@
 //
 // Pipeline (no host synchronisation anywhere):
 //   k_seg_hist    one wave per 512 rows: LDS histogram -> hist[block][group]
-//   k_seg_scan    one block: per-group totals, exclusive scans -> offsets,
-//                 tile/chunk tables' firsts, per-block bases (in place in hist)
+//   k_seg_scan    one block: per-group totals, exclusive scans -> offsets and
+//                 the firsts of the tile / chunk / partial tables, per-block
+//                 bases (in place in hist); then fills tile_group, the chunk
+//                 table and the -1 padding of each group's last tile
 //   k_seg_scatter one wave per 512 rows: stable rank inside the wave by
-//                 bit-sliced ballots, cursor per group in LDS -> perm, inv
-//   k_seg_fill    one thread per tile / chunk slot: binary search of its group
+//                 bit-sliced ballots, cursor per group in LDS -> perm, inv and
+//                 the padded slot tables
 #include "tk_device.h"
 
 namespace tk {
@@ -27,7 +29,7 @@ __device__ inline int load_key(const KeyT* keys, int64_t f, int groups, int* bad
 
 template <typename KeyT>
 __global__ __launch_bounds__(64) void k_seg_hist(const KeyT* __restrict__ keys, int rows, int groups,
-                                                 int32_t* __restrict__ hist, SegHeader* hdr) {
+                                                 int32_t* __restrict__ hist, int32_t* __restrict__ bad_out) {
   extern __shared__ int32_t lds[];
   const int lane = threadIdx.x;
   const int blk = blockIdx.x;
@@ -42,7 +44,9 @@ __global__ __launch_bounds__(64) void k_seg_hist(const KeyT* __restrict__ keys, 
   }
   __syncthreads();
   for (int g = lane; g < groups; g += 64) hist[(int64_t)blk * groups + g] = lds[g];
-  if (bad) atomicAdd(&hdr->bad_keys, bad);
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) bad += __shfl_xor(bad, d, 64);
+  if (lane == 0) bad_out[blk] = bad;
 }
 
 // Exclusive scan of one value per thread over a 1024-thread block.
@@ -74,27 +78,25 @@ __device__ inline int block_exclusive_scan(int v, int* wave_sums, int* total) {
   return res;
 }
 
-__global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sort_blocks, int32_t* __restrict__ hist,
-                                                   int32_t* __restrict__ offsets, int32_t* __restrict__ tile_first,
-                                                   int32_t* __restrict__ chunk_first,
-                                                   int32_t* __restrict__ partial_first,
-                                                   int64_t* __restrict__ offsets_out, SegHeader* hdr) {
+__global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sort_blocks, int max_tiles,
+                                                   int max_chunks, SegView V, int64_t* __restrict__ offsets_out) {
   __shared__ int wave_sums[17];
+  const int tid = threadIdx.x;
   int carry_rows = 0, carry_tiles = 0, carry_chunks = 0, carry_part = 0;
   for (int g0 = 0; g0 < groups; g0 += 1024) {
-    const int g = g0 + threadIdx.x;
+    const int g = g0 + tid;
     int count = 0;
     if (g < groups) {
       // per-block counts -> per-block exclusive bases (relative to the group's start)
       for (int b = 0; b < sort_blocks; ++b) {
         const int64_t i = (int64_t)b * groups + g;
-        const int c = hist[i];
-        hist[i] = count;
+        const int c = V.hist[i];
+        V.hist[i] = count;
         count += c;
       }
     }
     const int ntile = (count + kTileRows - 1) / kTileRows;
-    const int nchunk = (count + kChunkRows - 1) / kChunkRows;
+    const int nchunk = (ntile + kChunkTiles - 1) / kChunkTiles;
     const int npart = nchunk > 1 ? nchunk : 0;
     int tot;
     const int e_rows = block_exclusive_scan(count, wave_sums, &tot) + carry_rows;
@@ -106,37 +108,59 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
     const int e_part = block_exclusive_scan(npart, wave_sums, &tot) + carry_part;
     carry_part += tot;
     if (g < groups) {
-      offsets[g] = e_rows;
-      tile_first[g] = e_tiles;
-      chunk_first[g] = e_chunks;
-      partial_first[g] = e_part;
+      V.offsets[g] = e_rows;
+      V.tile_first[g] = e_tiles;
+      V.chunk_first[g] = e_chunks;
+      V.partial_first[g] = e_part;
       if (offsets_out) offsets_out[g] = e_rows;
+      // this group's tiles, chunks and the padding of its last tile
+      for (int j = 0; j < ntile; ++j) V.tile_group[e_tiles + j] = g;
+      for (int j = 0; j < nchunk; ++j) {
+        ChunkInfo c;
+        c.group = g;
+        c.tile0 = e_tiles + j * kChunkTiles;
+        c.ntiles = min(kChunkTiles, ntile - j * kChunkTiles);
+        c.partial = nchunk > 1 ? e_part + j : -1;
+        V.chunks[e_chunks + j] = c;
+      }
+      for (int j = count; j < ntile * kTileRows; ++j) {
+        V.slot_row[e_tiles * kTileRows + j] = -1;
+        V.slot_pos[e_tiles * kTileRows + j] = -1;
+      }
     }
   }
-  if (threadIdx.x == 0) {
-    offsets[groups] = carry_rows;
-    tile_first[groups] = carry_tiles;
-    chunk_first[groups] = carry_chunks;
-    partial_first[groups] = carry_part;
+  // unused tail of the tile and chunk tables
+  for (int i = carry_tiles + tid; i < max_tiles; i += 1024) V.tile_group[i] = -1;
+  for (int i = tid; i < max_tiles; i += 1024) V.tile_ticket[i] = 0;
+  for (int i = carry_chunks + tid; i < max_chunks; i += 1024) V.chunks[i] = ChunkInfo{-1, 0, 0, -1};
+  int bad = 0;
+  for (int b = tid; b < sort_blocks; b += 1024) bad += V.bad[b];
+  int bad_total;
+  block_exclusive_scan(bad, wave_sums, &bad_total);
+  if (tid == 0) {
+    V.offsets[groups] = carry_rows;
+    V.tile_first[groups] = carry_tiles;
+    V.chunk_first[groups] = carry_chunks;
+    V.partial_first[groups] = carry_part;
     if (offsets_out) offsets_out[groups] = carry_rows;
+    SegHeader* hdr = V.header;
     hdr->magic = kSegMagic;
     hdr->rows = rows;
     hdr->groups = groups;
     hdr->num_tiles = carry_tiles;
     hdr->num_chunks = carry_chunks;
     hdr->num_partials = carry_part;
+    hdr->bad_keys = bad_total;
   }
 }
 
 template <typename KeyT>
 __global__ __launch_bounds__(64) void k_seg_scatter(const KeyT* __restrict__ keys, int rows, int groups, int key_bits,
-                                                    const int32_t* __restrict__ hist,
-                                                    const int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
-                                                    int32_t* __restrict__ inv, int64_t* __restrict__ perm_out) {
+                                                    SegView V, int64_t* __restrict__ perm_out) {
   extern __shared__ int32_t cursor[];
   const int lane = threadIdx.x;
   const int blk = blockIdx.x;
-  for (int g = lane; g < groups; g += 64) cursor[g] = offsets[g] + hist[(int64_t)blk * groups + g];
+  for (int g = lane; g < groups; g += 64) cursor[g] = V.offsets[g] + V.hist[(int64_t)blk * groups + g];
   __syncthreads();
   const int64_t base = (int64_t)blk * kSortBlockRows;
   int unused = 0;
@@ -159,61 +183,15 @@ __global__ __launch_bounds__(64) void k_seg_scatter(const KeyT* __restrict__ key
     if (valid && rank == 0) cursor[key] += __popcll(same);
     __syncthreads();
     if (valid) {
-      perm[pos] = (int32_t)f;
-      inv[f] = pos;
+      V.perm[pos] = (int32_t)f;
+      V.inv[f] = pos;
       if (perm_out) perm_out[pos] = f;
+      const int slot = V.tile_first[key] * kTileRows + (pos - V.offsets[key]);
+      V.slot_row[slot] = (int32_t)f;
+      V.slot_pos[slot] = pos;
     }
   }
 }
-
-__device__ inline int group_of(const int32_t* first, int groups, int i) {
-  // largest g with first[g] <= i (first is non-decreasing, first[groups] > i)
-  int lo = 0, hi = groups;
-  while (hi - lo > 1) {
-    const int mid = (lo + hi) >> 1;
-    if (first[mid] <= i) lo = mid; else hi = mid;
-  }
-  return lo;
-}
-
-__global__ __launch_bounds__(256) void k_seg_fill(int groups, int max_tiles, int max_chunks,
-                                                  const int32_t* __restrict__ offsets,
-                                                  const int32_t* __restrict__ tile_first,
-                                                  const int32_t* __restrict__ chunk_first,
-                                                  const int32_t* __restrict__ partial_first,
-                                                  TileInfo* __restrict__ tiles, ChunkInfo* __restrict__ chunks) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i < max_tiles) {
-    TileInfo t{-1, 0, 0, 0};
-    if (i < tile_first[groups]) {
-      const int g = group_of(tile_first, groups, i);
-      const int j = i - tile_first[g];
-      t.group = g;
-      t.start = offsets[g] + j * kTileRows;
-      t.count = min(kTileRows, offsets[g + 1] - t.start);
-    }
-    tiles[i] = t;
-  }
-  if (i < max_chunks) {
-    ChunkInfo c{-1, 0, 0, -1};
-    if (i < chunk_first[groups]) {
-      const int g = group_of(chunk_first, groups, i);
-      const int j = i - chunk_first[g];
-      const int n = chunk_first[g + 1] - chunk_first[g];
-      c.group = g;
-      c.start = offsets[g] + j * kChunkRows;
-      c.end = min(c.start + kChunkRows, offsets[g + 1]);
-      c.partial = n > 1 ? partial_first[g] + j : -1;
-    }
-    chunks[i] = c;
-  }
-}
-
-__global__ void k_seg_clear(SegHeader* hdr) {
-  if (threadIdx.x < 64) ((int32_t*)hdr)[threadIdx.x] = 0;
-}
-
-// ---- row gather / scatter-back -------------------------------------------------
 
 // dst[j] = src[perm[j] mod tokens] * w[token, k]
 template <typename T>
@@ -285,24 +263,20 @@ int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t 
   const size_t lds = sizeof(int32_t) * (size_t)groups;
   int key_bits = 0;
   while ((1 << key_bits) < groups) ++key_bits;
-  hipLaunchKernelGGL(k_seg_clear, dim3(1), dim3(64), 0, s, V.header);
   if (key_dtype == TK_KEY_I32)
     hipLaunchKernelGGL(k_seg_hist<int32_t>, dim3(nblk), dim3(64), lds, s, (const int32_t*)keys, (int)rows, groups,
-                       V.hist, V.header);
+                       V.hist, V.bad);
   else
     hipLaunchKernelGGL(k_seg_hist<int64_t>, dim3(nblk), dim3(64), lds, s, (const int64_t*)keys, (int)rows, groups,
-                       V.hist, V.header);
-  hipLaunchKernelGGL(k_seg_scan, dim3(1), dim3(1024), 0, s, (int)rows, groups, nblk, V.hist, V.offsets, V.tile_first,
-                     V.chunk_first, V.partial_first, offsets_out, V.header);
+                       V.hist, V.bad);
+  hipLaunchKernelGGL(k_seg_scan, dim3(1), dim3(1024), 0, s, (int)rows, groups, nblk, (int)L.max_tiles,
+                     (int)L.max_chunks, V, offsets_out);
   if (key_dtype == TK_KEY_I32)
     hipLaunchKernelGGL(k_seg_scatter<int32_t>, dim3(nblk), dim3(64), lds, s, (const int32_t*)keys, (int)rows, groups,
-                       key_bits, V.hist, V.offsets, V.perm, V.inv, perm_out);
+                       key_bits, V, perm_out);
   else
     hipLaunchKernelGGL(k_seg_scatter<int64_t>, dim3(nblk), dim3(64), lds, s, (const int64_t*)keys, (int)rows, groups,
-                       key_bits, V.hist, V.offsets, V.perm, V.inv, perm_out);
-  const int fill = (int)(L.max_tiles > L.max_chunks ? L.max_tiles : L.max_chunks);
-  hipLaunchKernelGGL(k_seg_fill, dim3((fill + 255) / 256), dim3(256), 0, s, groups, (int)L.max_tiles,
-                     (int)L.max_chunks, V.offsets, V.tile_first, V.chunk_first, V.partial_first, V.tiles, V.chunks);
+                       key_bits, V, perm_out);
   return check_launch();
 }
 

@@ -19,6 +19,11 @@ static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // ---------------------------------------------------------------------------
 // Device-side segment table.  One allocation, carved by SegLayout from
 // (rows, groups) alone, so producer and consumers agree without a host copy.
+//
+// Kernels work in a *padded* sorted order: every group starts at a multiple of
+// 32 slots, so tile i is slots [32 i, 32 i + 32) and a workgroup finds its
+// rows from blockIdx with one load (no dependent table walk at kernel start).
+// Slots past a group's last row hold -1.
 // ---------------------------------------------------------------------------
 struct SegHeader {       // 64 x int32, at the start of the workspace
   int32_t magic;
@@ -31,80 +36,92 @@ struct SegHeader {       // 64 x int32, at the start of the workspace
   int32_t pad[57];
 };
 
-struct TileInfo {   // one forward tile: rows [start, start + count) of group `group`
+struct ChunkInfo {  // one weight-gradient chunk: tiles [tile0, tile0 + ntiles) of group `group`
   int32_t group;
-  int32_t start;
-  int32_t count;
-  int32_t pad;
-};
-
-struct ChunkInfo {  // one weight-gradient chunk: sorted rows [start, end) of group `group`
-  int32_t group;
-  int32_t start;
-  int32_t end;
+  int32_t tile0;
+  int32_t ntiles;
   int32_t partial;  // slot in the partial buffer, or -1 when the chunk is its group's only one
 };
+
+constexpr int kChunkTiles = kChunkRows / kTileRows;
 
 struct SegLayout {
   int64_t rows, groups;
   int64_t sort_blocks;   // ceil(rows / kSortBlockRows)
   int64_t max_tiles, max_chunks, max_partials;
+  int64_t slots;         // padded sorted length: 32 * max_tiles
   // byte offsets from the workspace base
-  int64_t off_perm, off_inv, off_offsets, off_tiles, off_chunks, off_tile_first, off_chunk_first, off_partial_first,
-      off_hist, total;
+  int64_t off_perm, off_inv, off_slot_row, off_slot_pos, off_offsets, off_tile_group, off_chunks, off_tile_first,
+      off_chunk_first, off_partial_first, off_hist, off_bad, off_ticket, total;
 
   SegLayout(int64_t rows_, int64_t groups_) : rows(rows_), groups(groups_) {
     sort_blocks = ceil_div(rows > 0 ? rows : 1, kSortBlockRows);
     max_tiles = ceil_div(rows, kTileRows) + groups;
     max_chunks = ceil_div(rows, kChunkRows) + groups;
     max_partials = 2 * ceil_div(rows, kChunkRows) + 1;
+    slots = max_tiles * kTileRows;
     int64_t o = round_up(sizeof(SegHeader), 256);
-    off_perm = o;         o += round_up(4 * (rows + 64), 256);
-    off_inv = o;          o += round_up(4 * (rows + 64), 256);
-    off_offsets = o;      o += round_up(4 * (groups + 1), 256);
-    off_tiles = o;        o += round_up(16 * (max_tiles + 1), 256);
-    off_chunks = o;       o += round_up(16 * (max_chunks + 1), 256);
-    off_tile_first = o;   o += round_up(4 * (groups + 1), 256);
-    off_chunk_first = o;  o += round_up(4 * (groups + 1), 256);
+    off_perm = o;          o += round_up(4 * (rows + 64), 256);
+    off_inv = o;           o += round_up(4 * (rows + 64), 256);
+    off_slot_row = o;      o += round_up(4 * slots, 256);
+    off_slot_pos = o;      o += round_up(4 * slots, 256);
+    off_offsets = o;       o += round_up(4 * (groups + 1), 256);
+    off_tile_group = o;    o += round_up(4 * (max_tiles + 1), 256);
+    off_chunks = o;        o += round_up(16 * (max_chunks + 1), 256);
+    off_tile_first = o;    o += round_up(4 * (groups + 1), 256);
+    off_chunk_first = o;   o += round_up(4 * (groups + 1), 256);
     off_partial_first = o; o += round_up(4 * (groups + 1), 256);
-    off_hist = o;         o += round_up(4 * groups * sort_blocks, 256);
+    off_hist = o;          o += round_up(4 * groups * sort_blocks, 256);
+    off_bad = o;           o += round_up(4 * sort_blocks, 256);
+    off_ticket = o;        o += round_up(4 * (max_tiles + 1), 256);
     total = o;
   }
 };
 
 struct SegView {  // typed device pointers into a segment workspace
   SegHeader* header;
-  int32_t* perm;         // [rows]   sorted position -> flat row
-  int32_t* inv;          // [rows]   flat row -> sorted position
-  int32_t* offsets;      // [G + 1]
-  TileInfo* tiles;       // [max_tiles]
-  ChunkInfo* chunks;     // [max_chunks]
+  int32_t* perm;           // [rows]    sorted position -> flat row
+  int32_t* inv;            // [rows]    flat row -> sorted position
+  int32_t* slot_row;       // [slots]   padded slot -> flat row (perm), -1 in padding
+  int32_t* slot_pos;       // [slots]   padded slot -> sorted position, -1 in padding
+  int32_t* offsets;        // [G + 1]
+  int32_t* tile_group;     // [max_tiles]  group of each tile, -1 past the last tile
+  ChunkInfo* chunks;       // [max_chunks]
   int32_t* tile_first;     // [G + 1]  first tile of each group
   int32_t* chunk_first;    // [G + 1]  first chunk of each group
   int32_t* partial_first;  // [G + 1]  first partial slot of each multi-chunk group
   int32_t* hist;           // [sort_blocks][G]  per-block histogram, then per-block exclusive bases
+  int32_t* bad;            // [sort_blocks]  out-of-range keys seen by each block
+  int32_t* tile_ticket;    // [max_tiles]  arrival counters of the split shrink (zero between launches)
   SegView(const void* base, const SegLayout& L) {
     char* b = (char*)base;
     header = (SegHeader*)b;
     perm = (int32_t*)(b + L.off_perm);
     inv = (int32_t*)(b + L.off_inv);
+    slot_row = (int32_t*)(b + L.off_slot_row);
+    slot_pos = (int32_t*)(b + L.off_slot_pos);
     offsets = (int32_t*)(b + L.off_offsets);
-    tiles = (TileInfo*)(b + L.off_tiles);
+    tile_group = (int32_t*)(b + L.off_tile_group);
     chunks = (ChunkInfo*)(b + L.off_chunks);
     tile_first = (int32_t*)(b + L.off_tile_first);
     chunk_first = (int32_t*)(b + L.off_chunk_first);
     partial_first = (int32_t*)(b + L.off_partial_first);
     hist = (int32_t*)(b + L.off_hist);
+    bad = (int32_t*)(b + L.off_bad);
+    tile_ticket = (int32_t*)(b + L.off_ticket);
   }
+  // rows of the activation tensors, by padded slot
+  const int32_t* slot_table(int map_rows) const { return map_rows ? slot_row : slot_pos; }
 };
 
 constexpr int32_t kSegMagic = 0x544b5347;  // "TKSG"
 
 // ---------------------------------------------------------------------------
-// Saved shrink output.  hT[n][p]: rank index major, sorted position minor, so
-// the row-contraction kernels read 8 consecutive positions per lane.
+// Saved shrink output, indexed by padded slot.  hT[n][slot]: rank index major,
+// so the row-contraction kernels read 8 consecutive slots per lane; followed
+// by hrow[slot][n], the expand kernel's operand.
 // ---------------------------------------------------------------------------
-static inline int64_t h_ld(int64_t rows) { return round_up(rows > 0 ? rows : 1, 64); }
+static inline int64_t h_ld(int64_t rows, int64_t groups) { return round_up(SegLayout(rows, groups).slots, 64); }
 // Padded rank: 16, 32, 64 or 128 (the kernels are instantiated per padded rank).
 static inline int32_t rank_pad(int32_t max_rank) {
   int32_t p = 16;
@@ -113,17 +130,31 @@ static inline int32_t rank_pad(int32_t max_rank) {
 }
 static inline int elt_bytes(int dtype) { return dtype == TK_DTYPE_BF16 ? 2 : 4; }
 
+// The MFMA shrink kernel covers the source width with blocks of shrink_waves() waves, each wave
+// taking kShrinkSteps steps of 64 columns; wider sources are split over several blocks whose
+// partial sums meet in a global buffer.
+constexpr int kShrinkSteps = 8;
+static inline int shrink_waves(int rpad) { return rpad <= 16 ? 1 : (rpad <= 32 ? 2 : 4); }
+static inline int shrink_kslices(int width, int rpad) {
+  return (int)ceil_div(ceil_div(width, 64), (int64_t)kShrinkSteps * shrink_waves(rpad));
+}
+static inline int64_t shrink_partial_bytes(int64_t rows, int64_t groups, int width, int rpad) {
+  const int ks = shrink_kslices(width, rpad);
+  return ks > 1 ? round_up(SegLayout(rows, groups).max_tiles * ks * (int64_t)kTileRows * rpad * 4, 256) : 0;
+}
+
 // Backward workspace carving.
 struct BwdLayout {
-  int64_t off_dh, off_wT_shrink, off_wT_expand, off_part_a, off_part_b, total;
+  int64_t off_dh, off_hpart, off_wT_shrink, off_wT_expand, off_part_a, off_part_b, total;
   int64_t rpad, ldh;
   BwdLayout(const tk_lora_desc& d) {
     SegLayout S(d.rows, d.num_groups);
     rpad = rank_pad(d.max_rank);
-    ldh = h_ld(d.rows);
+    ldh = h_ld(d.rows, d.num_groups);
     const int64_t e = elt_bytes(d.dtype);
     int64_t o = 0;
-    off_dh = o;         o += round_up(2 * rpad * ldh * e, 256);  // rank-major + position-major copies
+    off_dh = o;         o += round_up(2 * rpad * ldh * e, 256);  // rank-major + slot-major copies
+    off_hpart = o;      o += shrink_partial_bytes(d.rows, d.num_groups, d.out_features, (int)rpad);
     // B^T per group [rpad][M]  (shrink weight of the backward pass)
     off_wT_shrink = o;  o += round_up((int64_t)d.num_groups * rpad * d.out_features * e, 256);
     // A^T per group [K][rpad]  (expand weight of the backward pass)
@@ -151,6 +182,10 @@ struct PassArgs {
   int32_t width_dst;  // M | K
   int32_t map_rows;
   int32_t rpad;
+  int32_t src_rows;  // rows of src / dst (bound for speculative row addresses)
+  float* hpart;          // partial sums of the split shrink, [tile][slice][32][rpad]
+  int32_t* tile_ticket;  // arrival counter per tile
+  int32_t kslices;       // blocks per tile of the MFMA shrink
 };
 
 // Row-contraction (weight gradient) pass: out_g[n][c] = sum_p hT[n][p] * src[row(p)][c].
