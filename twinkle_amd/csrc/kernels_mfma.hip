@@ -205,17 +205,27 @@ __global__ __launch_bounds__(256) void k_shrink_finish(PassArgs a, bf16_t* __res
   constexpr int RP = 16 * NB, PR = RP + 1;
   __shared__ float part[kTileRows][PR];
   const int tile_id = blockIdx.x, tid = threadIdx.x;
+  const int slot0 = tile_id * kTileRows;
+  // independent loads first: group id, this tile's row indices, the slices themselves
   const int g = tile_group[tile_id];
+  const int my_row = slot_rows[slot0 + (tid & 31)];
+  const float* tile_part = a.hpart + (int64_t)tile_id * a.kslices * (kTileRows * RP);
+  float sums[(kTileRows * RP + 255) / 256];
+#pragma unroll
+  for (int i = 0; i < (kTileRows * RP + 255) / 256; ++i) {
+    const int idx = tid + 256 * i;
+    float sum = 0.f;
+    if (idx < kTileRows * RP)
+      for (int k = 0; k < a.kslices; ++k) sum += tile_part[(int64_t)k * (kTileRows * RP) + idx];
+    sums[i] = sum;
+  }
   if (g < 0) return;
   if (a.rank[g] <= 0) return;
-  const int slot0 = tile_id * kTileRows;
-  int cnt = 0;
-  for (int i = 0; i < kTileRows; ++i) cnt += slot_rows[slot0 + i] >= 0;
-  const float* tile_part = a.hpart + (int64_t)tile_id * a.kslices * (kTileRows * RP);
-  for (int idx = tid; idx < kTileRows * RP; idx += 256) {
-    float sum = 0.f;
-    for (int k = 0; k < a.kslices; ++k) sum += tile_part[(int64_t)k * (kTileRows * RP) + idx];
-    part[idx / RP][idx % RP] = sum;
+  const int cnt = __popcll(__ballot(my_row >= 0) & 0xffffffffull);  // padding is at the end of a tile
+#pragma unroll
+  for (int i = 0; i < (kTileRows * RP + 255) / 256; ++i) {
+    const int idx = tid + 256 * i;
+    if (idx < kTileRows * RP) part[idx / RP][idx % RP] = sums[i];
   }
   __syncthreads();
   shrink_epilogue<RP, 256>(&part[0][0], 1, a, hrow, slot0, cnt, a.scale[g]);
@@ -324,22 +334,23 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
 // ---------------------------------------------------------------------------
 // Row contraction (weight gradients): out[n][c] = sum_slot hT[n][slot] * src[row(slot)][c]
 // over the tiles of one chunk of one group, for 128 columns per block.  The
-// NW waves of a block take the chunk's tiles in turn (wave w: tiles w, w+NW,
-// ...), so a chunk is many short streams, and add their accumulators in LDS in
+// NW waves of a block split the chunk's tiles (wave w: tiles w*16/NW ...), so
+// a chunk is several short streams, and add their accumulators in LDS in
 // wave order at the end.  Each lane loads 8 rows x 8 columns (eight fully
 // coalesced wave loads of 4 x 256 B), transposes its 8x8 block in registers
 // with v_perm_b32 so that rows become the MFMA contraction index, and
-// accumulates 128 columns x rank in MFMA registers.  The loads of a wave's
-// next tile are issued before its current tile is consumed.  Padding slots
-// contribute nothing: their h is exactly zero and their rows are not loaded.
+// accumulates 128 columns x rank in MFMA registers.  A wave issues the loads
+// of all its tiles before it consumes the first.  Padding slots contribute
+// nothing: their h is exactly zero and their rows are not loaded.
 // ---------------------------------------------------------------------------
-template <int NB, int NW>
+template <int NB, int NW, int TB>
 __global__ __launch_bounds__(NW * 64) void k_wgrad_mfma(WgradArgs a, const ChunkInfo* __restrict__ chunks,
                                                         const int32_t* __restrict__ slot_rows) {
   __shared__ float red[NW > 1 ? NW - 1 : 1][8 * NB * 4][64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
-  const int c0 = blockIdx.y * 128;
-  const ChunkInfo ci = chunks[blockIdx.x];
+  // column block fastest: blocks that run together read neighbouring pieces of the same rows
+  const int c0 = blockIdx.x * 128;
+  const ChunkInfo ci = chunks[blockIdx.y];
   const int g = ci.group;
   if (g < 0) return;
   const int r = min(a.rank[g], 16 * NB);
@@ -354,57 +365,51 @@ __global__ __launch_bounds__(NW * 64) void k_wgrad_mfma(WgradArgs a, const Chunk
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) acc[q][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  int4 ra = make_int4(-1, -1, -1, -1), rb = ra;
-  uint4 xn[8];
-  if (wave < ci.ntiles) {
-    ra = *reinterpret_cast<const int4*>(rows_p + wave * kTileRows);
-    rb = *reinterpret_cast<const int4*>(rows_p + wave * kTileRows + 4);
-    const int rows[8] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w};
+  // A wave owns tiles wave*TPW .. wave*TPW+TPW-1 of the chunk and issues the loads of up to four of
+  // them before it consumes the first (32 KB per wave in flight).
+  constexpr int TPW = kChunkTiles / NW;       // tiles per wave
+  static_assert(TPW % TB == 0, "TB (tiles whose loads are issued together) must divide the tiles per wave");
+  for (int tb = wave * TPW; tb < wave * TPW + TPW && tb < ci.ntiles; tb += TB) {
+    uint4 x[TB][8];
+    uint4 h[TB][NB];
 #pragma unroll
-    for (int q = 0; q < 8; ++q) xn[q] = rows[q] >= 0 ? ld16(src + (int64_t)rows[q] * a.ld_src) : zero4();
-    if (wave + NW < ci.ntiles) {
-      ra = *reinterpret_cast<const int4*>(rows_p + (wave + NW) * kTileRows);
-      rb = *reinterpret_cast<const int4*>(rows_p + (wave + NW) * kTileRows + 4);
-    }
-  }
-  for (int t = wave; t < ci.ntiles; t += NW) {
-    const int w0 = (ci.tile0 + t) * kTileRows;
-    uint4 x[8];
-#pragma unroll
-    for (int q = 0; q < 8; ++q) x[q] = xn[q];
-    uint4 h[NB];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) h[nb] = ld16(hT + (int64_t)(16 * nb + li) * a.ldh + w0);
-    if (t + NW < ci.ntiles) {
+    for (int u = 0; u < TB; ++u) {
+      const bool tok = tb + u < ci.ntiles;  // wave-uniform
+      const int t = tok ? tb + u : 0;
+      const int4 ra = *reinterpret_cast<const int4*>(rows_p + t * kTileRows);
+      const int4 rb = *reinterpret_cast<const int4*>(rows_p + t * kTileRows + 4);
       const int rows[8] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w};
 #pragma unroll
-      for (int q = 0; q < 8; ++q) xn[q] = rows[q] >= 0 ? ld16(src + (int64_t)rows[q] * a.ld_src) : zero4();
-      if (t + 2 * NW < ci.ntiles) {
-        ra = *reinterpret_cast<const int4*>(rows_p + (t + 2 * NW) * kTileRows);
-        rb = *reinterpret_cast<const int4*>(rows_p + (t + 2 * NW) * kTileRows + 4);
-      }
-    }
-    // 8x8 transpose inside the lane: tr[q] holds column q of the 8 rows
-    uint4 tr[8];
+      for (int q = 0; q < 8; ++q)
+        x[u][q] = (tok && rows[q] >= 0) ? ld16(src + (int64_t)rows[q] * a.ld_src) : zero4();
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      const int d = q >> 1;
-      const uint32_t sel = (q & 1) ? 0x07060302u : 0x05040100u;
-      uint32_t e[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const uint32_t wsrc[4] = {x[i].x, x[i].y, x[i].z, x[i].w};
-        e[i] = wsrc[d];
-      }
-      tr[q].x = __builtin_amdgcn_perm(e[1], e[0], sel);
-      tr[q].y = __builtin_amdgcn_perm(e[3], e[2], sel);
-      tr[q].z = __builtin_amdgcn_perm(e[5], e[4], sel);
-      tr[q].w = __builtin_amdgcn_perm(e[7], e[6], sel);
+      for (int nb = 0; nb < NB; ++nb)
+        h[u][nb] = tok ? ld16(hT + (int64_t)(16 * nb + li) * a.ldh + (ci.tile0 + t) * kTileRows) : zero4();
     }
 #pragma unroll
-    for (int q = 0; q < 8; ++q)
+    for (int u = 0; u < TB; ++u) {
+      // 8x8 transpose inside the lane: tr[q] holds column q of the 8 rows
+      uint4 tr[8];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) acc[q][nb] = mfma16(tr[q], h[nb], acc[q][nb]);
+      for (int q = 0; q < 8; ++q) {
+        const int d = q >> 1;
+        const uint32_t sel = (q & 1) ? 0x07060302u : 0x05040100u;
+        uint32_t e[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const uint32_t wsrc[4] = {x[u][i].x, x[u][i].y, x[u][i].z, x[u][i].w};
+          e[i] = wsrc[d];
+        }
+        tr[q].x = __builtin_amdgcn_perm(e[1], e[0], sel);
+        tr[q].y = __builtin_amdgcn_perm(e[3], e[2], sel);
+        tr[q].z = __builtin_amdgcn_perm(e[5], e[4], sel);
+        tr[q].w = __builtin_amdgcn_perm(e[7], e[6], sel);
+      }
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[q][nb] = mfma16(tr[q], h[u][nb], acc[q][nb]);
+    }
   }
 
   // add the waves' accumulators in wave order; wave 0 writes the result
@@ -477,10 +482,10 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, hipS
                      seg.tile_group, rows, (int)items);
 }
 
-template <int NB, int NW>
+template <int NB, int NW, int TB>
 void launch_wgrad(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
-  const dim3 grid((unsigned)L.max_chunks, (unsigned)(a.width / 128));
-  hipLaunchKernelGGL((k_wgrad_mfma<NB, NW>), grid, dim3(NW * 64), 0, s, a, seg.chunks, seg.slot_table(a.map_rows));
+  const dim3 grid((unsigned)(a.width / 128), (unsigned)L.max_chunks);
+  hipLaunchKernelGGL((k_wgrad_mfma<NB, NW, TB>), grid, dim3(NW * 64), 0, s, a, seg.chunks, seg.slot_table(a.map_rows));
 }
 
 }  // namespace
@@ -511,9 +516,9 @@ bool wgrad_mfma_supported(const WgradArgs& a) {
 
 int launch_wgrad_mfma(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
   if (L.rows == 0) return TK_OK;
-  if (a.rpad <= 16) launch_wgrad<1, 4>(a, seg, L, s);
-  else if (a.rpad <= 32) launch_wgrad<2, 4>(a, seg, L, s);
-  else launch_wgrad<4, 2>(a, seg, L, s);
+  if (a.rpad <= 16) launch_wgrad<1, 2, 2>(a, seg, L, s);
+  else if (a.rpad <= 32) launch_wgrad<2, 2, 2>(a, seg, L, s);
+  else launch_wgrad<4, 2, 2>(a, seg, L, s);
   return check_launch();
 }
 

@@ -2,20 +2,23 @@
 // gather / scatter-back kernels that use its table.  Integer work, HBM-light:
 // the table is built once per batch and read by every LoRA layer.
 //
-// Pipeline (no host synchronisation anywhere):
-//   k_seg_hist    one wave per 512 rows: LDS histogram -> hist[block][group]
+// Pipeline (three launches, no host synchronisation anywhere):
+//   k_seg_hist    one wave per 512 rows: per-key counts by bit-sliced ballots
+//                 (no contended atomics) -> hist[block][group]
 //   k_seg_scan    one block: per-group totals, exclusive scans -> offsets and
 //                 the firsts of the tile / chunk / partial tables, per-block
-//                 bases (in place in hist); then fills tile_group, the chunk
-//                 table and the -1 padding of each group's last tile
+//                 bases (in place in hist); then, in parallel over tiles and
+//                 slots, tile_group, the chunk table, slot_pos and the -1
+//                 padding of slot_row
 //   k_seg_scatter one wave per 512 rows: stable rank inside the wave by
-//                 bit-sliced ballots, cursor per group in LDS -> perm, inv and
-//                 the padded slot tables
+//                 bit-sliced ballots, cursor per group in LDS -> inv, slot_row
 #include "tk_device.h"
 
 namespace tk {
 
 namespace {
+
+constexpr int kKeysPerLane = kSortBlockRows / 64;
 
 template <typename KeyT>
 __device__ inline int load_key(const KeyT* keys, int64_t f, int groups, int* bad) {
@@ -27,8 +30,19 @@ __device__ inline int load_key(const KeyT* keys, int64_t f, int groups, int* bad
   return (int)k;
 }
 
+// lanes of this wave that are valid and hold the same key as the calling lane
+__device__ inline unsigned long long same_key_lanes(bool valid, int key, int key_bits) {
+  unsigned long long same = __ballot(valid);
+  for (int b = 0; b < key_bits; ++b) {
+    const bool bit = (key >> b) & 1;
+    const unsigned long long m = __ballot(valid && bit);
+    same &= bit ? m : ~m;
+  }
+  return same;
+}
+
 template <typename KeyT>
-__global__ __launch_bounds__(64) void k_seg_hist(const KeyT* __restrict__ keys, int rows, int groups,
+__global__ __launch_bounds__(64) void k_seg_hist(const KeyT* __restrict__ keys, int rows, int groups, int key_bits,
                                                  int32_t* __restrict__ hist, int32_t* __restrict__ bad_out) {
   extern __shared__ int32_t lds[];
   const int lane = threadIdx.x;
@@ -37,10 +51,19 @@ __global__ __launch_bounds__(64) void k_seg_hist(const KeyT* __restrict__ keys, 
   __syncthreads();
   int bad = 0;
   const int64_t base = (int64_t)blk * kSortBlockRows;
+  int k[kKeysPerLane];
 #pragma unroll
-  for (int s = 0; s < kSortBlockRows / 64; ++s) {
-    const int64_t f = base + s * 64 + lane;
-    if (f < rows) atomicAdd(&lds[load_key(keys, f, groups, &bad)], 1);
+  for (int j = 0; j < kKeysPerLane; ++j) {  // all loads first: they overlap
+    const int64_t f = base + j * 64 + lane;
+    k[j] = f < rows ? load_key(keys, f, groups, &bad) : -1;
+  }
+#pragma unroll
+  for (int j = 0; j < kKeysPerLane; ++j) {
+    const bool valid = k[j] >= 0;
+    const unsigned long long same = same_key_lanes(valid, k[j], key_bits);
+    const bool leader = valid && (same & ((1ull << lane) - 1ull)) == 0;
+    if (leader) lds[k[j]] += __popcll(same);  // one lane per distinct key: no conflicts
+    __builtin_amdgcn_wave_barrier();
   }
   __syncthreads();
   for (int g = lane; g < groups; g += 64) hist[(int64_t)blk * groups + g] = lds[g];
@@ -78,21 +101,44 @@ __device__ inline int block_exclusive_scan(int v, int* wave_sums, int* total) {
   return res;
 }
 
+// largest g in [0, groups) with first[g] <= i, for a non-decreasing `first` with first[groups] > i
+__device__ inline int group_of(const int32_t* first, int groups, int i) {
+  int lo = 0, hi = groups;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (first[mid] <= i) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+constexpr int kScanLdsGroups = 2048;  // up to this many groups the scan keeps its four prefix tables in LDS
+
 __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sort_blocks, int max_tiles,
                                                    int max_chunks, SegView V, int64_t* __restrict__ offsets_out) {
   __shared__ int wave_sums[17];
+  __shared__ int32_t lds_first[4][kScanLdsGroups + 1];  // offsets, tile_first, chunk_first, partial_first
   const int tid = threadIdx.x;
+  const bool in_lds = groups <= kScanLdsGroups;
+  int bad = 0;
+  for (int b = tid; b < sort_blocks; b += 1024) bad += V.bad[b];
+  int bad_total;
+  block_exclusive_scan(bad, wave_sums, &bad_total);
   int carry_rows = 0, carry_tiles = 0, carry_chunks = 0, carry_part = 0;
   for (int g0 = 0; g0 < groups; g0 += 1024) {
     const int g = g0 + tid;
     int count = 0;
     if (g < groups) {
-      // per-block counts -> per-block exclusive bases (relative to the group's start)
-      for (int b = 0; b < sort_blocks; ++b) {
-        const int64_t i = (int64_t)b * groups + g;
-        const int c = V.hist[i];
-        V.hist[i] = count;
-        count += c;
+      // per-block counts -> per-block exclusive bases (relative to the group's start); loads are
+      // issued eight at a time so that their latencies overlap
+      for (int b0 = 0; b0 < sort_blocks; b0 += 8) {
+        int c[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) c[j] = b0 + j < sort_blocks ? V.hist[(int64_t)(b0 + j) * groups + g] : 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if (b0 + j < sort_blocks) V.hist[(int64_t)(b0 + j) * groups + g] = count;
+          count += c[j];
+        }
       }
     }
     const int ntile = (count + kTileRows - 1) / kTileRows;
@@ -113,36 +159,26 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
       V.chunk_first[g] = e_chunks;
       V.partial_first[g] = e_part;
       if (offsets_out) offsets_out[g] = e_rows;
-      // this group's tiles, chunks and the padding of its last tile
-      for (int j = 0; j < ntile; ++j) V.tile_group[e_tiles + j] = g;
-      for (int j = 0; j < nchunk; ++j) {
-        ChunkInfo c;
-        c.group = g;
-        c.tile0 = e_tiles + j * kChunkTiles;
-        c.ntiles = min(kChunkTiles, ntile - j * kChunkTiles);
-        c.partial = nchunk > 1 ? e_part + j : -1;
-        V.chunks[e_chunks + j] = c;
-      }
-      for (int j = count; j < ntile * kTileRows; ++j) {
-        V.slot_row[e_tiles * kTileRows + j] = -1;
-        V.slot_pos[e_tiles * kTileRows + j] = -1;
+      if (in_lds) {
+        lds_first[0][g] = e_rows;
+        lds_first[1][g] = e_tiles;
+        lds_first[2][g] = e_chunks;
+        lds_first[3][g] = e_part;
       }
     }
   }
-  // unused tail of the tile and chunk tables
-  for (int i = carry_tiles + tid; i < max_tiles; i += 1024) V.tile_group[i] = -1;
-  for (int i = tid; i < max_tiles; i += 1024) V.tile_ticket[i] = 0;
-  for (int i = carry_chunks + tid; i < max_chunks; i += 1024) V.chunks[i] = ChunkInfo{-1, 0, 0, -1};
-  int bad = 0;
-  for (int b = tid; b < sort_blocks; b += 1024) bad += V.bad[b];
-  int bad_total;
-  block_exclusive_scan(bad, wave_sums, &bad_total);
   if (tid == 0) {
     V.offsets[groups] = carry_rows;
     V.tile_first[groups] = carry_tiles;
     V.chunk_first[groups] = carry_chunks;
     V.partial_first[groups] = carry_part;
     if (offsets_out) offsets_out[groups] = carry_rows;
+    if (in_lds) {
+      lds_first[0][groups] = carry_rows;
+      lds_first[1][groups] = carry_tiles;
+      lds_first[2][groups] = carry_chunks;
+      lds_first[3][groups] = carry_part;
+    }
     SegHeader* hdr = V.header;
     hdr->magic = kSegMagic;
     hdr->rows = rows;
@@ -152,6 +188,44 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
     hdr->num_partials = carry_part;
     hdr->bad_keys = bad_total;
   }
+  // the firsts were written by this block: make them visible to all of its threads, then fill the
+  // per-tile (with its 32 slots) and per-chunk tables in parallel
+  __threadfence_block();
+  __syncthreads();
+  const int32_t* offs = in_lds ? lds_first[0] : V.offsets;
+  const int32_t* tfirst = in_lds ? lds_first[1] : V.tile_first;
+  const int32_t* cfirst = in_lds ? lds_first[2] : V.chunk_first;
+  const int32_t* pfirst = in_lds ? lds_first[3] : V.partial_first;
+  for (int i = tid; i < max_tiles; i += 1024) {
+    int g = -1, pos0 = 0, valid = 0;
+    if (i < carry_tiles) {
+      g = group_of(tfirst, groups, i);
+      pos0 = offs[g] + (i - tfirst[g]) * kTileRows;   // sorted position of the tile's first slot
+      valid = min(kTileRows, offs[g + 1] - pos0);       // padding is at the end of a group's last tile
+    }
+    V.tile_group[i] = g;
+    V.tile_ticket[i] = 0;
+    int4* sp = reinterpret_cast<int4*>(V.slot_pos + (int64_t)i * kTileRows);
+#pragma unroll
+    for (int j = 0; j < kTileRows; j += 4)
+      sp[j / 4] = make_int4(j < valid ? pos0 + j : -1, j + 1 < valid ? pos0 + j + 1 : -1,
+                            j + 2 < valid ? pos0 + j + 2 : -1, j + 3 < valid ? pos0 + j + 3 : -1);
+    // slot_row: only the padding is written here, the rows come from k_seg_scatter
+    for (int j = valid; j < kTileRows; ++j) V.slot_row[(int64_t)i * kTileRows + j] = -1;
+  }
+  for (int i = tid; i < max_chunks; i += 1024) {
+    ChunkInfo c{-1, 0, 0, -1};
+    if (i < carry_chunks) {
+      const int g = group_of(cfirst, groups, i);
+      const int j = i - cfirst[g];
+      const int ntile = tfirst[g + 1] - tfirst[g];
+      c.group = g;
+      c.tile0 = tfirst[g] + j * kChunkTiles;
+      c.ntiles = min(kChunkTiles, ntile - j * kChunkTiles);
+      c.partial = cfirst[g + 1] - cfirst[g] > 1 ? pfirst[g] + j : -1;
+    }
+    V.chunks[i] = c;
+  }
 }
 
 template <typename KeyT>
@@ -160,48 +234,48 @@ __global__ __launch_bounds__(64) void k_seg_scatter(const KeyT* __restrict__ key
   extern __shared__ int32_t cursor[];
   const int lane = threadIdx.x;
   const int blk = blockIdx.x;
-  for (int g = lane; g < groups; g += 64) cursor[g] = V.offsets[g] + V.hist[(int64_t)blk * groups + g];
-  __syncthreads();
   const int64_t base = (int64_t)blk * kSortBlockRows;
   int unused = 0;
-  for (int s = 0; s < kSortBlockRows / 64; ++s) {
-    const int64_t f = base + s * 64 + lane;
-    const bool valid = f < rows;
-    const int key = valid ? load_key(keys, f, groups, &unused) : 0;
-    // lanes of this wave that hold the same key
-    unsigned long long same = __ballot(valid);
-    for (int b = 0; b < key_bits; ++b) {
-      const bool bit = (key >> b) & 1;
-      const unsigned long long m = __ballot(valid && bit);
-      same &= bit ? m : ~m;
-    }
-    const unsigned long long below = same & ((1ull << lane) - 1ull);
-    const int rank = __popcll(below);
+  int k[kKeysPerLane];
+#pragma unroll
+  for (int j = 0; j < kKeysPerLane; ++j) {  // all loads first: they overlap
+    const int64_t f = base + j * 64 + lane;
+    k[j] = f < rows ? load_key(keys, f, groups, &unused) : -1;
+  }
+  for (int g = lane; g < groups; g += 64) cursor[g] = V.offsets[g] + V.hist[(int64_t)blk * groups + g];
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kKeysPerLane; ++j) {
+    const int64_t f = base + j * 64 + lane;
+    const bool valid = k[j] >= 0;
+    const int key = max(k[j], 0);
+    // rows with equal keys keep their lane order
+    const unsigned long long same = same_key_lanes(valid, key, key_bits);
+    const int rank = __popcll(same & ((1ull << lane) - 1ull));
     int pos = 0;
     if (valid) pos = cursor[key] + rank;
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();
     if (valid && rank == 0) cursor[key] += __popcll(same);
-    __syncthreads();
+    __builtin_amdgcn_wave_barrier();
     if (valid) {
-      V.perm[pos] = (int32_t)f;
       V.inv[f] = pos;
       if (perm_out) perm_out[pos] = f;
-      const int slot = V.tile_first[key] * kTileRows + (pos - V.offsets[key]);
-      V.slot_row[slot] = (int32_t)f;
-      V.slot_pos[slot] = pos;
+      // padded slot = 32 * first tile of the group + position inside the group
+      V.slot_row[V.tile_first[key] * kTileRows + (pos - V.offsets[key])] = (int32_t)f;
     }
   }
 }
 
-// dst[j] = src[perm[j] mod tokens] * w[token, k]
+// dst[j] = src[perm[j] mod tokens] * w[token, k], one block per padded slot (slot_row is perm in padded order)
 template <typename T>
 __global__ __launch_bounds__(256) void k_permute(const T* __restrict__ src, int64_t ld_src, T* __restrict__ dst,
                                                  int64_t ld_dst, const T* __restrict__ w,
-                                                 const int32_t* __restrict__ perm, int rows, int tokens, int top_k,
+                                                 const int32_t* __restrict__ slot_row,
+                                                 const int32_t* __restrict__ slot_pos, int tokens, int top_k,
                                                  int width) {
-  const int j = blockIdx.x;
-  if (j >= rows) return;
-  const int f = perm[j];
+  const int f = slot_row[blockIdx.x];
+  const int j = slot_pos[blockIdx.x];
+  if (f < 0 || j < 0) return;
   const int t = f % tokens, k = f / tokens;
   const T* s = src + (int64_t)t * ld_src;
   T* d = dst + (int64_t)j * ld_dst;
@@ -265,10 +339,10 @@ int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t 
   while ((1 << key_bits) < groups) ++key_bits;
   if (key_dtype == TK_KEY_I32)
     hipLaunchKernelGGL(k_seg_hist<int32_t>, dim3(nblk), dim3(64), lds, s, (const int32_t*)keys, (int)rows, groups,
-                       V.hist, V.bad);
+                       key_bits, V.hist, V.bad);
   else
     hipLaunchKernelGGL(k_seg_hist<int64_t>, dim3(nblk), dim3(64), lds, s, (const int64_t*)keys, (int)rows, groups,
-                       V.hist, V.bad);
+                       key_bits, V.hist, V.bad);
   hipLaunchKernelGGL(k_seg_scan, dim3(1), dim3(1024), 0, s, (int)rows, groups, nblk, (int)L.max_tiles,
                      (int)L.max_chunks, V, offsets_out);
   if (key_dtype == TK_KEY_I32)
@@ -287,11 +361,11 @@ int launch_permute(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, c
   SegView V(ws, L);
   const int top_k = (int)(rows / tokens);
   if (dtype == TK_DTYPE_F32)
-    hipLaunchKernelGGL(k_permute<float>, dim3((unsigned)rows), dim3(256), 0, s, (const float*)src, ld_src,
-                       (float*)dst, ld_dst, (const float*)w, V.perm, (int)rows, (int)tokens, top_k, width);
+    hipLaunchKernelGGL(k_permute<float>, dim3((unsigned)L.slots), dim3(256), 0, s, (const float*)src, ld_src,
+                       (float*)dst, ld_dst, (const float*)w, V.slot_row, V.slot_pos, (int)tokens, top_k, width);
   else
-    hipLaunchKernelGGL(k_permute<uint16_t>, dim3((unsigned)rows), dim3(256), 0, s, (const uint16_t*)src, ld_src,
-                       (uint16_t*)dst, ld_dst, (const uint16_t*)w, V.perm, (int)rows, (int)tokens, top_k, width);
+    hipLaunchKernelGGL(k_permute<uint16_t>, dim3((unsigned)L.slots), dim3(256), 0, s, (const uint16_t*)src, ld_src,
+                       (uint16_t*)dst, ld_dst, (const uint16_t*)w, V.slot_row, V.slot_pos, (int)tokens, top_k, width);
   return check_launch();
 }
 

@@ -51,7 +51,7 @@ struct SegLayout {
   int64_t max_tiles, max_chunks, max_partials;
   int64_t slots;         // padded sorted length: 32 * max_tiles
   // byte offsets from the workspace base
-  int64_t off_perm, off_inv, off_slot_row, off_slot_pos, off_offsets, off_tile_group, off_chunks, off_tile_first,
+  int64_t off_inv, off_slot_row, off_slot_pos, off_offsets, off_tile_group, off_chunks, off_tile_first,
       off_chunk_first, off_partial_first, off_hist, off_bad, off_ticket, total;
 
   SegLayout(int64_t rows_, int64_t groups_) : rows(rows_), groups(groups_) {
@@ -61,7 +61,6 @@ struct SegLayout {
     max_partials = 2 * ceil_div(rows, kChunkRows) + 1;
     slots = max_tiles * kTileRows;
     int64_t o = round_up(sizeof(SegHeader), 256);
-    off_perm = o;          o += round_up(4 * (rows + 64), 256);
     off_inv = o;           o += round_up(4 * (rows + 64), 256);
     off_slot_row = o;      o += round_up(4 * slots, 256);
     off_slot_pos = o;      o += round_up(4 * slots, 256);
@@ -80,7 +79,6 @@ struct SegLayout {
 
 struct SegView {  // typed device pointers into a segment workspace
   SegHeader* header;
-  int32_t* perm;           // [rows]    sorted position -> flat row
   int32_t* inv;            // [rows]    flat row -> sorted position
   int32_t* slot_row;       // [slots]   padded slot -> flat row (perm), -1 in padding
   int32_t* slot_pos;       // [slots]   padded slot -> sorted position, -1 in padding
@@ -96,7 +94,6 @@ struct SegView {  // typed device pointers into a segment workspace
   SegView(const void* base, const SegLayout& L) {
     char* b = (char*)base;
     header = (SegHeader*)b;
-    perm = (int32_t*)(b + L.off_perm);
     inv = (int32_t*)(b + L.off_inv);
     slot_row = (int32_t*)(b + L.off_slot_row);
     slot_pos = (int32_t*)(b + L.off_slot_pos);
