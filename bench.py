@@ -9,9 +9,9 @@ resident in HBM before the timed region; three buffer sets are rotated so that n
 from the 256 MB last-level cache across steps (the backward of a step runs on the set whose forward ran
 one full step earlier).
 
-Prints one JSON line (see the keys below).  `roofline` describes the dominant kernel, the fused
-shrink->expand pass, on its forward launches: algorithmic bytes of one launch over its mean duration
-between HIP events on the launch stream.
+Prints one JSON line (see the keys below).  `roofline` describes the dominant kernel, the expand
+kernel (y += h B^T, a read-modify-write of the whole output), on its forward launches: algorithmic
+bytes of one launch over its mean duration between HIP events on the launch stream.
 """
 import argparse
 import json
@@ -66,8 +66,8 @@ def main():
         sys.exit(2)
 
     import torch
-    from twinkle_amd import (AdapterGroups, _lib, build_segments, lora_bwd_, lora_bwd_workspace_bytes, lora_fwd_,
-                             lora_h_bytes, workloads)
+    from twinkle_amd import (AdapterGroups, _lib, build_segments, lora_bwd_, lora_bwd_workspace_bytes, lora_expand_,
+                             lora_fwd_, lora_h_bytes, lora_shrink_, workloads)
     if not torch.cuda.is_available():
         print('bench.py needs a GPU', file=sys.stderr)
         sys.exit(2)
@@ -108,12 +108,15 @@ def main():
         seg_holder['seg'] = seg_i
         if ev is not None:
             ev[0].record()
-        lora_fwd_(f['x'], f['y'], seg_i, groups, h=f['h'])
+        lora_shrink_(f['x'], seg_i, groups, f['h'])     # tk_lora_fwd == these two calls
         if ev is not None:
             ev[1].record()
-        lora_bwd_(b['dy'], b['x'], b['h'], b['dx'], pa, pb, seg_i, groups, accumulate=False, workspace=ws)
+        lora_expand_(f['h'], f['y'], seg_i, groups)
         if ev is not None:
             ev[2].record()
+        lora_bwd_(b['dy'], b['x'], b['h'], b['dx'], pa, pb, seg_i, groups, accumulate=False, workspace=ws)
+        if ev is not None:
+            ev[3].record()
 
     # every set needs a forward before its first backward
     for i in range(len(sets)):
@@ -121,7 +124,7 @@ def main():
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
@@ -129,8 +132,10 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
+    shrink_ms = sum(e[0].elapsed_time(e[1]) for e in events) / args.steps
+    expand_ms = sum(e[1].elapsed_time(e[2]) for e in events) / args.steps
+    fwd_ms = shrink_ms + expand_ms
+    bwd_ms = sum(e[2].elapsed_time(e[3]) for e in events) / args.steps
 
     # base GEMM, reported separately and not part of the step
     wbase = torch.randn(M, K, device=dev, dtype=dt) * 0.02
@@ -145,11 +150,11 @@ def main():
     torch.cuda.synchronize()
     base_ms = e0.elapsed_time(e1) / 10
 
-    w_live = sum(r * (K + M) for r in w.ranks)
     step_bytes = w.algorithmic_bytes(elt)
-    fwd_bytes = elt * T * (K + 2 * M) + elt * w_live           # one launch of the fused pass (forward instance)
+    # one forward launch of the expand kernel: read + write y, read the live columns of every B
+    expand_bytes = elt * T * 2 * M + elt * sum(r * M for r in w.ranks)
     flops = w.flops()
-    achieved = fwd_bytes / (fwd_ms * 1e-3) / 1e9
+    achieved = expand_bytes / (expand_ms * 1e-3) / 1e9
     out = {
         'metric': 'multi-LoRA fwd+bwd tokens/s + % roofline (HBM/MFMA), 8B proj, 16 adapters',
         'value': T / (ms_per_step * 1e-3),
@@ -168,9 +173,9 @@ def main():
                                'base GEMM excluded', 'tokens': T, 'in': K, 'out': M, 'adapters': G, 'rank': 16},
         'roofline': {'bound': 'hbm', 'achieved': achieved, 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
                      'frac': achieved / HBM_PEAK_GBS, 'traffic': None,
-                     'kernel': 'k_pass_mfma<1,8> (fused shrink->expand), forward launch',
-                     'algorithmic_bytes_per_launch': fwd_bytes, 'avg_launch_ms': fwd_ms},
-        'step_detail': {'fwd_ms': fwd_ms, 'bwd_ms': bwd_ms, 'segment_build_and_gaps_ms': ms_per_step - fwd_ms - bwd_ms,
+                     'kernel': 'k_expand_mfma<1,1> (y += h B^T in place), forward launch',
+                     'algorithmic_bytes_per_launch': expand_bytes, 'avg_launch_ms': expand_ms},
+        'step_detail': {'shrink_ms': shrink_ms, 'expand_ms': expand_ms, 'fwd_ms': fwd_ms, 'bwd_ms': bwd_ms, 'segment_build_and_gaps_ms': ms_per_step - fwd_ms - bwd_ms,
                         'algorithmic_bytes_per_step': step_bytes, 'flops_per_step': flops,
                         'tflops': flops / (ms_per_step * 1e-3) / 1e12,
                         'hbm_frac_step': step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,

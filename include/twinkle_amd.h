@@ -140,6 +140,12 @@ int64_t tk_lora_bwd_workspace_bytes(const tk_lora_desc* desc);
 int tk_lora_fwd(const tk_lora_desc* desc, const void* x_device, int64_t ldx, void* y_device, int64_t ldy,
                 void* h_device, tk_stream_t stream);
 
+/* The two halves of tk_lora_fwd, for callers that time or schedule them separately:
+ * tk_lora_shrink writes h = scale_g * x A_g^T (reference: multi_lora.py:322-323, the first F.linear),
+ * tk_lora_expand adds h B_g^T onto y in place (reference: multi_lora.py:324-326). */
+int tk_lora_shrink(const tk_lora_desc* desc, const void* x_device, int64_t ldx, void* h_device, tk_stream_t stream);
+int tk_lora_expand(const tk_lora_desc* desc, const void* h_device, void* y_device, int64_t ldy, tk_stream_t stream);
+
 /* dx[row] += scale_g * (dy[row] B_g) A_g        (skipped when dx_device is NULL)
  * dA_g[:r] (+)= (scale_g * dy B_g)^T x          (skipped when grad_A is NULL)
  * dB_g[:, :r] (+)= dy^T h                       (skipped when grad_B is NULL)

@@ -65,6 +65,8 @@ EXPORTS = {
     'tk_lora_h_bytes': (c_int64, [POINTER(LoraDesc)]),
     'tk_lora_bwd_workspace_bytes': (c_int64, [POINTER(LoraDesc)]),
     'tk_lora_fwd': (c_int32, [POINTER(LoraDesc), c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
+    'tk_lora_shrink': (c_int32, [POINTER(LoraDesc), c_void_p, c_int64, c_void_p, c_void_p]),
+    'tk_lora_expand': (c_int32, [POINTER(LoraDesc), c_void_p, c_void_p, c_int64, c_void_p]),
     'tk_lora_bwd': (c_int32, [POINTER(LoraDesc), c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                               c_void_p, c_void_p, c_int32, c_void_p, c_int64, c_void_p]),
 }

@@ -29,9 +29,10 @@ bool force_generic() {
   return v;
 }
 
-int run_pass(const PassArgs& a, const SegView& V, const SegLayout& L, int dtype, hipStream_t s) {
-  if (dtype == TK_DTYPE_BF16 && !force_generic() && pass_mfma_supported(a)) return launch_pass_mfma(a, V, L, s);
-  return launch_pass_generic(a, V, L, dtype, s);
+int run_pass(const PassArgs& a, const SegView& V, const SegLayout& L, int dtype, int phases, hipStream_t s) {
+  if (dtype == TK_DTYPE_BF16 && !force_generic() && pass_mfma_supported(a))
+    return launch_pass_mfma(a, V, L, phases, s);
+  return launch_pass_generic(a, V, L, dtype, phases, s);
 }
 
 int run_wgrad(const WgradArgs& a, const SegView& V, const SegLayout& L, int dtype, hipStream_t s) {
@@ -135,16 +136,18 @@ int64_t tk_lora_bwd_workspace_bytes(const tk_lora_desc* d) {
   return BwdLayout(*d).total;
 }
 
-int tk_lora_fwd(const tk_lora_desc* d, const void* x, int64_t ldx, void* y, int64_t ldy, void* h,
-                tk_stream_t stream) {
+static int lora_pass_fwd(const tk_lora_desc* d, const void* x, int64_t ldx, void* y, int64_t ldy, void* h,
+                         int phases, tk_stream_t stream) {
   if (!desc_ok(d) || !h) return TK_ERR_INVALID;
   if (d->rows == 0 || d->max_rank == 0) return TK_OK;
-  if (!x || !y || ldx < d->in_features || ldy < d->out_features) return TK_ERR_INVALID;
+  if ((phases & 1) && (!x || ldx < d->in_features)) return TK_ERR_INVALID;
+  if ((phases & 2) && (!y || ldy < d->out_features)) return TK_ERR_INVALID;
   SegLayout L(d->rows, d->num_groups);
   SegView V(d->seg_ws, L);
   PassArgs a{};
-  a.src = x;  a.ld_src = ldx;
-  a.dst = y;  a.ld_dst = ldy;
+  // shapes are checked against what both phases need, so that the two halves of one forward pick the same kernels
+  a.src = x ? x : h;  a.ld_src = x ? ldx : d->in_features;
+  a.dst = y ? y : h;  a.ld_dst = y ? ldy : d->out_features;
   a.hT = h;   a.ldh = h_ld(d->rows, d->num_groups);
   a.w_shrink = d->lora_A;  a.ld_shrink = d->lda;
   a.w_expand = d->lora_B;  a.ld_expand = d->ldb;
@@ -154,7 +157,20 @@ int tk_lora_fwd(const tk_lora_desc* d, const void* x, int64_t ldx, void* y, int6
   a.hpart = (float*)((char*)h + round_up(2 * (int64_t)a.rpad * a.ldh * elt_bytes(d->dtype), 256));
   a.tile_ticket = V.tile_ticket;
   a.kslices = shrink_kslices(d->in_features, a.rpad);
-  return run_pass(a, V, L, d->dtype, (hipStream_t)stream);
+  return run_pass(a, V, L, d->dtype, phases, (hipStream_t)stream);
+}
+
+int tk_lora_fwd(const tk_lora_desc* d, const void* x, int64_t ldx, void* y, int64_t ldy, void* h,
+                tk_stream_t stream) {
+  return lora_pass_fwd(d, x, ldx, y, ldy, h, 3, stream);
+}
+
+int tk_lora_shrink(const tk_lora_desc* d, const void* x, int64_t ldx, void* h, tk_stream_t stream) {
+  return lora_pass_fwd(d, x, ldx, nullptr, 0, h, 1, stream);
+}
+
+int tk_lora_expand(const tk_lora_desc* d, const void* h, void* y, int64_t ldy, tk_stream_t stream) {
+  return lora_pass_fwd(d, nullptr, 0, y, ldy, const_cast<void*>(h), 2, stream);
 }
 
 int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void* x, int64_t ldx, const void* h,
@@ -190,7 +206,7 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
     a.hpart = (float*)(w + B.off_hpart);
     a.tile_ticket = V.tile_ticket;
     a.kslices = shrink_kslices(d->out_features, a.rpad);
-    if ((rc = run_pass(a, V, L, d->dtype, s)) != TK_OK) return rc;
+    if ((rc = run_pass(a, V, L, d->dtype, 3, s)) != TK_OK) return rc;
   }
   if (grad_A) {
     WgradArgs g{};

@@ -227,19 +227,22 @@ __global__ __launch_bounds__(256) void k_transpose_weights(tk_lora_desc d, int r
 
 }  // namespace
 
-int launch_pass_generic(const PassArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s) {
+int launch_pass_generic(const PassArgs& a, const SegView& seg, const SegLayout& L, int dtype, int phases,
+                        hipStream_t s) {
   if (L.rows == 0) return TK_OK;
   const unsigned grid = (unsigned)L.max_tiles;
   const int32_t* rows = seg.slot_table(a.map_rows);
   const size_t lds_shrink = sizeof(float) * (size_t)(kTileRows + a.rpad) * (kKC + 1);
   const size_t lds_expand = sizeof(float) * (size_t)a.rpad * kTileRows;
   if (dtype == TK_DTYPE_F32) {
-    hipLaunchKernelGGL(k_shrink_generic<float>, dim3(grid), dim3(256), lds_shrink, s, a, seg.tile_group, rows);
-    if (a.dst)
+    if (phases & 1)
+      hipLaunchKernelGGL(k_shrink_generic<float>, dim3(grid), dim3(256), lds_shrink, s, a, seg.tile_group, rows);
+    if (a.dst && (phases & 2))
       hipLaunchKernelGGL(k_expand_generic<float>, dim3(grid), dim3(256), lds_expand, s, a, seg.tile_group, rows);
   } else {
-    hipLaunchKernelGGL(k_shrink_generic<bf16_t>, dim3(grid), dim3(256), lds_shrink, s, a, seg.tile_group, rows);
-    if (a.dst)
+    if (phases & 1)
+      hipLaunchKernelGGL(k_shrink_generic<bf16_t>, dim3(grid), dim3(256), lds_shrink, s, a, seg.tile_group, rows);
+    if (a.dst && (phases & 2))
       hipLaunchKernelGGL(k_expand_generic<bf16_t>, dim3(grid), dim3(256), lds_expand, s, a, seg.tile_group, rows);
   }
   return check_launch();

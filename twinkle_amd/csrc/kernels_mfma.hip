@@ -466,16 +466,18 @@ __global__ __launch_bounds__(NW * 64) void k_wgrad_mfma(WgradArgs a, const Chunk
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <int NB, int CPW>
-void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
+void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int phases, hipStream_t s) {
   bf16_t* hrow = (bf16_t*)a.hT + (int64_t)a.rpad * a.ldh;  // second half of the h buffer
   const int32_t* rows = seg.slot_table(a.map_rows);
   constexpr int NW = NB == 1 ? 1 : (NB == 2 ? 2 : 4);  // shrink_waves(16 * NB)
-  hipLaunchKernelGGL((k_shrink_mfma<NB, NW>), dim3((unsigned)(L.max_tiles * a.kslices)), dim3(NW * 64), 0, s, a, hrow,
-                     seg.tile_group, rows);
-  if (a.kslices > 1)
-    hipLaunchKernelGGL((k_shrink_finish<NB>), dim3((unsigned)L.max_tiles), dim3(256), 0, s, a, hrow, seg.tile_group,
-                       rows);
-  if (!a.dst) return;
+  if (phases & 1) {
+    hipLaunchKernelGGL((k_shrink_mfma<NB, NW>), dim3((unsigned)(L.max_tiles * a.kslices)), dim3(NW * 64), 0, s, a,
+                       hrow, seg.tile_group, rows);
+    if (a.kslices > 1)
+      hipLaunchKernelGGL((k_shrink_finish<NB>), dim3((unsigned)L.max_tiles), dim3(256), 0, s, a, hrow,
+                         seg.tile_group, rows);
+  }
+  if (!a.dst || !(phases & 2)) return;
   const int64_t ngroups = a.width_dst >> 7;
   const int64_t items = L.max_tiles * ceil_div(ngroups, CPW);
   hipLaunchKernelGGL((k_expand_mfma<NB, CPW>), dim3((unsigned)ceil_div(items, 4)), dim3(256), 0, s, a, hrow,
@@ -500,11 +502,11 @@ bool pass_mfma_supported(const PassArgs& a) {
   return true;
 }
 
-int launch_pass_mfma(const PassArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
+int launch_pass_mfma(const PassArgs& a, const SegView& seg, const SegLayout& L, int phases, hipStream_t s) {
   if (L.rows == 0) return TK_OK;
-  if (a.rpad <= 16) launch_pass<1, 1>(a, seg, L, s);
-  else if (a.rpad <= 32) launch_pass<2, 1>(a, seg, L, s);
-  else launch_pass<4, 1>(a, seg, L, s);
+  if (a.rpad <= 16) launch_pass<1, 1>(a, seg, L, phases, s);
+  else if (a.rpad <= 32) launch_pass<2, 1>(a, seg, L, phases, s);
+  else launch_pass<4, 1>(a, seg, L, phases, s);
   return check_launch();
 }
 

@@ -212,14 +212,16 @@ int launch_unpermute_wgrad(const void* dout, int64_t ld_dout, const void* rows_,
                            hipStream_t s);
 
 // kernels_generic.hip : any shape / stride, fp32 and bf16, VALU
-int launch_pass_generic(const PassArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s);
+int launch_pass_generic(const PassArgs& a, const SegView& seg, const SegLayout& L, int dtype, int phases,
+                        hipStream_t s);
 int launch_wgrad_generic(const WgradArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s);
 int launch_wgrad_reduce(const WgradArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s);
 int launch_transpose_weights(const tk_lora_desc& d, void* bT, void* aT, hipStream_t s);
 
 // kernels_mfma.hip : bf16, aligned shapes, MFMA
 bool pass_mfma_supported(const PassArgs& a);
-int launch_pass_mfma(const PassArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
+// `phases`: 1 = shrink only, 2 = expand only (h already written), 3 = both
+int launch_pass_mfma(const PassArgs& a, const SegView& seg, const SegLayout& L, int phases, hipStream_t s);
 bool wgrad_mfma_supported(const WgradArgs& a);
 int launch_wgrad_mfma(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
 

@@ -165,6 +165,24 @@ def lora_fwd_(x: torch.Tensor, y: torch.Tensor, seg: SegmentTable, groups: Adapt
     return h
 
 
+def lora_shrink_(x: torch.Tensor, seg: SegmentTable, groups: AdapterGroups, h: torch.Tensor,
+                 map_rows: bool = True) -> None:
+    """First half of :func:`lora_fwd_`: ``h = scale * x A^T`` (see ``tk_lora_shrink``)."""
+    _check_rows(x, 'x', seg.rows, groups.in_features, groups.dtype)
+    d = _desc(seg, groups, map_rows)
+    _lib.check(_lib.load().tk_lora_shrink(ctypes.byref(d), x.data_ptr(), x.stride(0), h.data_ptr(), _lib.stream_ptr()),
+               'tk_lora_shrink')
+
+
+def lora_expand_(h: torch.Tensor, y: torch.Tensor, seg: SegmentTable, groups: AdapterGroups,
+                 map_rows: bool = True) -> None:
+    """Second half of :func:`lora_fwd_`: ``y += h B^T`` in place (see ``tk_lora_expand``)."""
+    _check_rows(y, 'y', seg.rows, groups.out_features, groups.dtype)
+    d = _desc(seg, groups, map_rows)
+    _lib.check(_lib.load().tk_lora_expand(ctypes.byref(d), h.data_ptr(), y.data_ptr(), y.stride(0), _lib.stream_ptr()),
+               'tk_lora_expand')
+
+
 def lora_bwd_(dy: torch.Tensor, x: Optional[torch.Tensor], h: Optional[torch.Tensor], dx: Optional[torch.Tensor],
               grad_a_ptrs: Optional[torch.Tensor], grad_b_ptrs: Optional[torch.Tensor], seg: SegmentTable,
               groups: AdapterGroups, map_rows: bool = True, accumulate: bool = False,
