@@ -1,0 +1,216 @@
+"""The MultiLora mirror on the GPU: mixed-tenant batches equal each tenant run alone, and both equal the oracle."""
+import pytest
+import torch
+from torch import nn
+
+import oracle
+from conftest import max_rel_err
+from twinkle_amd import LoraConfig, LoraLinear, MultiLora
+
+pytestmark = pytest.mark.gpu
+
+
+class Block(nn.Module):
+
+    def __init__(self, d=128, f=256):
+        super().__init__()
+        self.q_proj = nn.Linear(d, d, bias=False)
+        self.up_proj = nn.Linear(d, f, bias=True)
+        self.down_proj = nn.Linear(f, d, bias=False)
+
+    def forward(self, x):
+        return self.down_proj(torch.nn.functional.silu(self.up_proj(self.q_proj(x))))
+
+
+def _setup(dev, dtype, max_loras=4, max_r=16):
+    torch.manual_seed(0)
+    ml = MultiLora(max_loras=max_loras, max_r=max_r)
+    model = ml.patch(Block().to(dtype).to(dev), target_modules='all-linear')
+    ml.save_initial_weights()
+    cfgs = {
+        'alice': LoraConfig(r=8, lora_alpha=16, target_modules='all-linear'),
+        'bob': LoraConfig(r=16, lora_alpha=32, target_modules=['q_proj', 'down_proj']),       # up_proj not targeted
+        'carol': LoraConfig(r=4, lora_alpha=16, target_modules='all-linear', use_rslora=True),
+    }
+    for name, cfg in cfgs.items():
+        ml.acquire_lora(name, cfg)
+    g = torch.Generator().manual_seed(1)
+    with torch.no_grad():
+        for n, p in model.named_parameters():
+            if '.lora_B.' in n:                   # B starts at zero: give it values so the LoRA term is visible
+                p.copy_((torch.randn(p.shape, generator=g) * 0.05).to(dtype))
+    return ml, model, cfgs
+
+
+def _oracle_block(model, x64, tenant_of_row, cfgs, ml, dtype):
+    """The block evaluated per layer with the oracle's per-adapter loop, in float64 on the rounded weights."""
+    names = list(cfgs)
+    slot = {n: ml.find_lora_by_tenant(n).adapter_name for n in names}
+
+    def lora_layer(layer, name, h):
+        w = layer.base_layer.weight.detach().double().cpu()
+        b = layer.base_layer.bias.detach().double().cpu() if layer.base_layer.bias is not None else None
+        base = torch.nn.functional.linear(h, w, b)
+        a_list, b_list, ranks, scales = [], [], [], []
+        for n in names:
+            cfg = cfgs[n]
+            live = oracle.match_target_modules(name, cfg.target_modules)
+            a_list.append(layer.lora_A[slot[n]].weight.detach().double().cpu())
+            b_list.append(layer.lora_B[slot[n]].weight.detach().double().cpu())
+            ranks.append(cfg.r if live else 0)
+            scales.append(oracle.lora_scaling(cfg.lora_alpha, cfg.r, cfg.use_rslora))
+        return oracle.multi_lora_linear(h, base, tenant_of_row, a_list, b_list, ranks, scales)
+
+    m = model.model
+    h = lora_layer(m.q_proj, 'model.q_proj', x64)
+    h = torch.nn.functional.silu(lora_layer(m.up_proj, 'model.up_proj', h))
+    return lora_layer(m.down_proj, 'model.down_proj', h)
+
+
+@pytest.mark.parametrize('dtype,tol', [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+def test_mixed_batch_equals_each_tenant_alone_and_the_oracle(dev, dtype, tol):
+    ml, model, cfgs = _setup(dev, dtype)
+    names = list(cfgs)
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(3, 70, 128, generator=g).to(dtype)                      # [batch, seq, features]
+    row_tenant = torch.randint(0, 3, (3 * 70,), generator=g)
+    xd = x.to(dev)
+    with ml.batch(names, row_tenant.to(dev)):
+        y_mixed = model(xd)
+    # every tenant alone through the reference-style one-adapter context
+    y_single = torch.empty_like(y_mixed)
+    for i, n in enumerate(names):
+        with ml.adapter(n):
+            yi = model(xd)
+        mask = (row_tenant == i).view(3, 70).to(dev)
+        y_single[mask] = yi[mask]
+    assert max_rel_err(y_mixed, y_single) < (1e-6 if dtype == torch.float32 else 1e-2)
+    want = _oracle_block(model, x.double().view(-1, 128), row_tenant, cfgs, ml, dtype).view(3, 70, 128)
+    assert max_rel_err(y_mixed, want) < tol
+
+
+def test_only_the_tenants_in_the_batch_get_gradients(dev):
+    """Reference invariant: updates only the active adapter (tests/model/test_multi_lora_target_parameters.py:78-100)."""
+    ml, model, cfgs = _setup(dev, torch.float32)
+    x = torch.randn(50, 128, generator=torch.Generator().manual_seed(3)).to(dev)
+    row_tenant = (torch.arange(50) % 2).to(dev)                             # alice and bob only
+    with ml.batch(['alice', 'bob'], row_tenant):
+        model(x).pow(2).mean().backward()
+    params = dict(model.named_parameters())
+    for n, p in params.items():
+        if 'lora_' not in n:
+            assert p.grad is None                                            # base stays frozen
+            continue
+        slot = n.split('.')[-2]
+        if slot in ('lora_2', 'lora_3'):                                     # carol's slot and the free slot
+            assert p.grad is None or torch.count_nonzero(p.grad) == 0, n
+    ga = params['model.q_proj.lora_A.lora_0.weight'].grad
+    assert torch.count_nonzero(ga[:8]) > 0 and torch.count_nonzero(ga[8:]) == 0   # alice: rank 8 of a 16-row slot
+    assert params['model.up_proj.lora_A.lora_1.weight'].grad is None or \
+        torch.count_nonzero(params['model.up_proj.lora_A.lora_1.weight'].grad) == 0  # bob does not target up_proj
+
+
+def test_gradients_match_the_oracle_through_the_whole_block(dev):
+    ml, model, cfgs = _setup(dev, torch.float32)
+    names = list(cfgs)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(90, 128, generator=g)
+    row_tenant = torch.randint(0, 3, (90,), generator=g)
+    xd = x.to(dev).requires_grad_(True)
+    with ml.batch(names, row_tenant.to(dev)):
+        model(xd).pow(2).sum().backward()
+    # oracle: same block in float64 with autograd
+    x64 = x.double().requires_grad_(True)
+    m = model.model
+    slot = {n: ml.find_lora_by_tenant(n).adapter_name for n in names}
+    leaves = {}
+
+    def layer64(layer, name, h):
+        base = torch.nn.functional.linear(h, layer.base_layer.weight.detach().double().cpu(),
+                                          None if layer.base_layer.bias is None else layer.base_layer.bias.detach().double().cpu())
+        a_list, b_list, ranks, scales = [], [], [], []
+        for n in names:
+            cfg = cfgs[n]
+            a = layer.lora_A[slot[n]].weight.detach().double().cpu().requires_grad_(True)
+            b = layer.lora_B[slot[n]].weight.detach().double().cpu().requires_grad_(True)
+            leaves[(name, n, 'A')], leaves[(name, n, 'B')] = a, b
+            a_list.append(a)
+            b_list.append(b)
+            ranks.append(cfg.r if oracle.match_target_modules(name, cfg.target_modules) else 0)
+            scales.append(oracle.lora_scaling(cfg.lora_alpha, cfg.r, cfg.use_rslora))
+        return oracle.multi_lora_linear(h, base, row_tenant, a_list, b_list, ranks, scales)
+
+    h = layer64(m.q_proj, 'model.q_proj', x64)
+    h = torch.nn.functional.silu(layer64(m.up_proj, 'model.up_proj', h))
+    layer64(m.down_proj, 'model.down_proj', h).pow(2).sum().backward()
+    assert max_rel_err(xd.grad, x64.grad) < 1e-4
+    params = dict(model.named_parameters())
+    for (lname, tenant, side), leaf in leaves.items():
+        got = params[f'{lname}.lora_{side}.{slot[tenant]}.weight'].grad
+        want = leaf.grad if leaf.grad is not None else torch.zeros_like(leaf)
+        if got is None:
+            assert torch.count_nonzero(want) == 0
+        else:
+            assert max_rel_err(got, want) < 1e-4, (lname, tenant, side)
+
+
+def test_disable_lora_and_unmatched_layers_return_the_base_output(dev):
+    ml, model, _ = _setup(dev, torch.float32)
+    x = torch.randn(10, 128, generator=torch.Generator().manual_seed(5)).to(dev)
+    m = model.model
+    base = m.down_proj.base_layer(torch.nn.functional.silu(m.up_proj.base_layer(m.q_proj.base_layer(x))))
+    with ml.adapter('alice', disable_lora=True):
+        assert torch.equal(model(x), base)
+    with ml.adapter('bob'):                        # bob does not target up_proj: that layer must be the base layer
+        q = m.q_proj(x)
+        assert torch.equal(m.up_proj(q), m.up_proj.base_layer(q))
+    # after release B is zero again: the tenant's rows are the base output exactly (reference :745-748)
+    ml.release_lora('alice')
+    ml.acquire_lora('dave', LoraConfig(r=8, lora_alpha=16, target_modules='all-linear'))
+    with ml.adapter('dave'):
+        assert torch.equal(model(x), base)
+
+
+def test_activation_checkpointing_recompute_is_bitwise_identical(dev):
+    """The reference runs with gradient checkpointing on (multi_lora_transformers.py:85): forward runs twice."""
+    from torch.utils.checkpoint import checkpoint
+    ml, model, cfgs = _setup(dev, torch.bfloat16)
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(200, 128, generator=g).bfloat16().to(dev).requires_grad_(True)
+    row_tenant = torch.randint(0, 3, (200,), generator=g).to(dev)
+    with ml.batch(list(cfgs), row_tenant):
+        y1 = model(x)
+        y1.float().pow(2).sum().backward()
+        g1 = {n: p.grad.clone() for n, p in model.named_parameters() if p.grad is not None}
+        gx1 = x.grad.clone()
+        model.zero_grad()
+        x.grad = None
+        y2 = checkpoint(model, x, use_reentrant=False)
+        y2.float().pow(2).sum().backward()
+    assert torch.equal(y1, y2) and torch.equal(gx1, x.grad)
+    for n, p in model.named_parameters():
+        if p.grad is not None:
+            assert torch.equal(p.grad, g1[n]), n
+
+
+def test_mixed_dtype_base_bf16_adapters_fp32(dev):
+    """x is cast to the adapter dtype and the sum back to the base output dtype (multi_lora.py:320, :327)."""
+    torch.manual_seed(0)
+    ml = MultiLora(max_loras=2, max_r=8)
+    base = nn.Sequential(nn.Linear(64, 128, bias=False)).bfloat16().to(dev)
+    model = ml.patch(base, target_modules='all-linear')
+    for n, p in model.named_parameters():
+        if 'lora_' in n:
+            p.data = p.data.float()
+    ml.acquire_lora('alice', LoraConfig(r=8, lora_alpha=16, target_modules='all-linear'))
+    layer = [m for m in model.modules() if isinstance(m, LoraLinear)][0]
+    with torch.no_grad():
+        layer.lora_B['lora_0'].weight.normal_(0, 0.05)
+    x = torch.randn(33, 64, generator=torch.Generator().manual_seed(7)).bfloat16().to(dev)
+    with ml.adapter('alice'):
+        y = model(x)
+    assert y.dtype == torch.bfloat16
+    want = oracle.lora_linear_forward(x.cpu(), layer.base_layer(x).cpu(), layer.lora_A['lora_0'].weight.detach().cpu(),
+                                      layer.lora_B['lora_0'].weight.detach().cpu(), 8, 2.0)
+    assert want.dtype == torch.bfloat16
+    assert max_rel_err(y, want) < 1e-2

@@ -1,0 +1,176 @@
+"""Host-side mirror of the reference's MultiLora / target-parameter LoRA bookkeeping (no GPU needed)."""
+import pytest
+import torch
+from torch import nn
+
+import oracle
+from twinkle_amd import LoraConfig, LoraLinear, MultiLora
+from twinkle_amd.expert_lora import ExpertLoraSlots
+
+
+class TinyBlock(nn.Module):
+
+    def __init__(self, d=16, f=24):
+        super().__init__()
+        self.q_proj = nn.Linear(d, d, bias=False)
+        self.up_proj = nn.Linear(d, f, bias=True)
+        self.down_proj = nn.Linear(f, d, bias=False)
+
+    def forward(self, x):
+        return self.down_proj(torch.relu(self.up_proj(self.q_proj(x))))
+
+
+def _patched(max_loras=3, max_r=8):
+    torch.manual_seed(0)
+    ml = MultiLora(max_loras=max_loras, max_r=max_r)
+    model = ml.patch(TinyBlock(), target_modules='all-linear')
+    ml.save_initial_weights()
+    return ml, model
+
+
+def test_patch_preallocates_slots_at_max_rank():
+    ml, model = _patched()
+    assert [t.adapter_name for t in ml.loras] == ['lora_0', 'lora_1', 'lora_2']
+    layers = [m for m in model.modules() if isinstance(m, LoraLinear)]
+    assert len(layers) == 3
+    for layer in layers:
+        assert set(layer.lora_A.keys()) == {'lora_0', 'lora_1', 'lora_2'}
+        assert layer.lora_A['lora_1'].weight.shape == (8, layer.in_features)
+        assert layer.lora_B['lora_1'].weight.shape == (layer.out_features, 8)
+        assert torch.count_nonzero(layer.lora_B['lora_2'].weight) == 0       # B starts at zero
+        assert hasattr(layer, 'layer_name')
+    assert all(p.requires_grad for n, p in model.named_parameters() if 'lora_' in n)
+    assert not any(p.requires_grad for n, p in model.named_parameters() if 'lora_' not in n)
+
+
+def test_acquire_release_and_errors():
+    """Same exceptions as the reference (multi_lora.py:128, :211-216, :247)."""
+    ml, _ = _patched(max_loras=2, max_r=8)
+    cfg = LoraConfig(r=4, lora_alpha=8, target_modules='all-linear')
+    assert ml.acquire_lora('alice', cfg) == 'lora_0'
+    assert ml.acquire_lora('bob', cfg) == 'lora_1'
+    with pytest.raises(ValueError):
+        ml.acquire_lora('alice', cfg)                      # duplicate tenant
+    with pytest.raises(RuntimeError):
+        ml.acquire_lora('carol', cfg)                      # no free slot
+    ml.release_lora('alice')
+    with pytest.raises(RuntimeError):
+        ml.acquire_lora('carol', LoraConfig(r=16, lora_alpha=8, target_modules='all-linear'))   # r > max_r
+    assert ml.acquire_lora('carol', cfg) == 'lora_0'       # first free slot is reused
+    with pytest.raises(ValueError):
+        ml.find_lora_by_tenant('alice')
+    with pytest.raises(ValueError):
+        ml.activate_adapter('nobody')
+    assert ml.release_lora('nobody') is None               # unknown tenant: silently ignored, as in the reference
+    with pytest.raises(ValueError):
+        ml.check_length([{'input_ids': [0] * 5000}, {'input_ids': [0] * 5000}])
+
+
+def test_release_restores_initial_a_and_zeroes_b():
+    """Reference invariant (tests/model/test_multi_lora_target_parameters.py:103-134, and multi_lora.py:731-754)."""
+    ml, model = _patched()
+    ml.acquire_lora('alice', LoraConfig(r=4, lora_alpha=8, target_modules='all-linear'))
+    before = {n: p.detach().clone() for n, p in model.named_parameters() if '.lora_0.' in n}
+    with torch.no_grad():
+        for n, p in model.named_parameters():
+            if '.lora_0.' in n:
+                p.add_(1.0)
+    ml.release_lora('alice')
+    for n, p in model.named_parameters():
+        if '.lora_A.lora_0.' in n:
+            assert torch.equal(p, before[n])
+        if '.lora_B.lora_0.' in n:
+            assert torch.count_nonzero(p) == 0
+
+
+def test_state_dict_is_rank_sliced_renamed_and_round_trips():
+    """Slicing / renaming of multi_lora.py:85-113, :676-729; round trip as in the reference test :188-213."""
+    ml, model = _patched()
+    ml.acquire_lora('alice', LoraConfig(r=4, lora_alpha=8, target_modules=['q_proj', 'down_proj']))
+    with torch.no_grad():
+        for n, p in model.named_parameters():
+            if '.lora_0.' in n:
+                p.uniform_(-0.1, 0.1)
+    sd = ml.get_state_dict('alice')
+    assert set(sd) == {'model.q_proj.lora_A.weight', 'model.q_proj.lora_B.weight', 'model.down_proj.lora_A.weight',
+                       'model.down_proj.lora_B.weight'}
+    assert sd['model.q_proj.lora_A.weight'].shape == (4, 16) and sd['model.q_proj.lora_B.weight'].shape == (16, 4)
+    ml2, model2 = _patched()
+    ml2.acquire_lora('zed', LoraConfig(r=4, lora_alpha=8, target_modules='all-linear'))
+    ml2.acquire_lora('alice', LoraConfig(r=4, lora_alpha=8, target_modules=['q_proj', 'down_proj']))   # lands in lora_1
+    ml2.set_state_dict('alice', sd)
+    sd2 = ml2.get_state_dict('alice')
+    for k in sd:
+        assert torch.equal(sd[k], sd2[k])
+    # only the live [:r] block of the slot was written
+    a_full = dict(model2.named_parameters())['model.q_proj.lora_A.lora_1.weight']
+    assert torch.equal(a_full[:4], sd['model.q_proj.lora_A.weight'])
+    for name, t in [('m.lora_A.weight', torch.randn(8, 5)), ('m.lora_B.weight', torch.randn(5, 8))]:
+        assert torch.equal(MultiLora._slice_rank_tensor(name, t, 3), oracle.slice_rank_tensor(name, t, 3))
+    trainable, total = ml.get_nb_trainable_parameters('alice')
+    assert trainable == 4 * 16 + 16 * 4 + 4 * 24 + 16 * 4
+
+
+def test_match_target_modules_agrees_with_oracle():
+    cases = [('model.layers.0.q_proj', None), ('x', []), ('a', 'all-linear'), ('a', ['all-linear']),
+             ('model.layers.0.attn.proj', ['attn.proj']), ('model.layers.0.attn.proj', ['mlp.up']),
+             ('model.layers.0.attn.proj.lora_A.default.weight', ['attn.proj']), ('model.layers.3.q_proj', r'.*\.q_proj'),
+             ('model.layers.3.k_proj', r'.*\.q_proj'), ('m.q_proj', {'q_proj'})]
+    for name, tm in cases:
+        assert MultiLora.match_target_modules(name, tm) == oracle.match_target_modules(name, tm)
+
+
+def test_adapter_context_selects_the_slot():
+    ml, model = _patched()
+    ml.acquire_lora('alice', LoraConfig(r=4, lora_alpha=8, target_modules='all-linear'))
+    ml.acquire_lora('bob', LoraConfig(r=8, lora_alpha=8, target_modules='all-linear'))
+    with ml.adapter('bob') as slot:
+        assert slot == 'lora_1' and model.active_adapter == 'lora_1'
+        assert all(m.active_adapters == ['lora_1'] for m in model.modules() if isinstance(m, LoraLinear))
+    with ml.adapter('alice', disable_lora=True):
+        assert all(m.disable_adapters for m in model.modules() if isinstance(m, LoraLinear))
+        x = torch.randn(3, 16)
+        assert torch.equal(model(x), model.model.down_proj.base_layer(
+            torch.relu(model.model.up_proj.base_layer(model.model.q_proj.base_layer(x)))))   # base only, runs on CPU
+    assert not any(m.disable_adapters for m in model.modules() if isinstance(m, LoraLinear))
+
+
+def test_expert_slots_follow_the_reference_rules():
+    """Checks of multi_lora_target_parameters.py:136-156 and the state-dict shape rules :232-278."""
+    torch.manual_seed(0)
+    slots = ExpertLoraSlots(num_experts=2, in_features=4, out_features=12, max_loras=2, max_r=4, key_prefix='m.experts')
+    assert slots.lora_A['lora_0'].shape == (2, 4, 4) and slots.lora_B['lora_1'].shape == (2, 12, 4)
+    assert torch.count_nonzero(slots.lora_B['lora_0']) == 0
+    assert slots.lora_A['lora_0'].abs().max() <= 1.0
+    with pytest.raises(ValueError):
+        slots.configure_slot('lora_9', LoraConfig(r=2, lora_alpha=4))
+    with pytest.raises(ValueError):
+        slots.configure_slot('lora_0', LoraConfig(r=0, lora_alpha=4))
+    with pytest.raises(ValueError):
+        slots.configure_slot('lora_0', LoraConfig(r=8, lora_alpha=4))
+    for bad in (dict(lora_dropout=0.1), dict(fan_in_fan_out=True), dict(use_dora=True), dict(lora_bias=True)):
+        with pytest.raises(ValueError):
+            slots.configure_slot('lora_0', LoraConfig(r=2, lora_alpha=4, **bad))
+    slots.configure_slot('lora_0', LoraConfig(r=2, lora_alpha=4))
+    slots.configure_slot('lora_1', LoraConfig(r=4, lora_alpha=4, use_rslora=True))
+    assert slots.scaling['lora_0'] == 2.0 and slots.scaling['lora_1'] == 2.0 and slots.r['lora_0'] == 2
+    with torch.no_grad():
+        slots.lora_A['lora_0'].uniform_(-0.1, 0.1)
+        slots.lora_B['lora_0'].uniform_(-0.1, 0.1)
+    dw = slots.get_delta_weight('lora_0')
+    want = oracle.expert_delta_weight(slots.lora_A['lora_0'].detach(), slots.lora_B['lora_0'].detach(), 2, 2.0)
+    assert torch.allclose(dw, want) and dw.shape == (2, 12, 4)
+    assert slots.get_delta_weight('lora_0', out_in_layout=False).shape == (2, 4, 12)
+    sd = slots.get_state_dict('lora_0')
+    assert sd['m.experts.lora_A.weight'].shape == (2, 2, 4) and sd['m.experts.lora_B.weight'].shape == (2, 12, 2)
+    other = ExpertLoraSlots(2, 4, 12, 2, 4, key_prefix='m.experts')
+    other.configure_slot('lora_1', LoraConfig(r=2, lora_alpha=4))
+    assert other.set_state_dict('lora_1', sd) == set(sd)
+    assert torch.allclose(other.get_delta_weight('lora_1'), dw, atol=1e-6)       # reference round-trip bar: atol 1e-6
+    with pytest.raises(KeyError):
+        other.set_state_dict('lora_1', {'m.experts.lora_A.weight': sd['m.experts.lora_A.weight']})
+    with pytest.raises(ValueError):
+        other.set_state_dict('lora_1', {k: v[:1] for k, v in sd.items()})
+    a0 = slots._initial_lora_A['lora_0'].clone()
+    slots.reset_slot('lora_0')
+    assert torch.equal(slots.lora_A['lora_0'].detach(), a0) and torch.count_nonzero(slots.lora_B['lora_0']) == 0

@@ -164,12 +164,13 @@ def inject_adapter(model: nn.Module, config: LoraConfig, adapter_name: str) -> L
     if isinstance(exclude, str):
         exclude = [exclude]
     wrapped = 0
+    inside = tuple(n + '.' for n, m in root.named_modules() if isinstance(m, LoraLinear))
     for name, module in list(root.named_modules()):
         if isinstance(module, LoraLinear):
             module.update_layer(adapter_name, config.r, config.lora_alpha, config.lora_dropout)
             wrapped += 1
             continue
-        if not isinstance(module, nn.Linear) or name.endswith('base_layer'):
+        if not isinstance(module, nn.Linear) or name.startswith(inside):   # base layers and slot weights stay as they are
             continue
         if not _name_matches(name, config.target_modules) or any(name.endswith(e) for e in exclude):
             continue
