@@ -27,6 +27,19 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
+def measured_traffic(kernel):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 --pmc summary (None if it is not there)."""
+    path = os.path.join(ROOT, 'profiles', 'bench_cfg2_hbm_traffic_pmc.txt')
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.startswith(f'traffic_bytes_per_launch[{kernel}]:'):
+                    return float(line.split(':')[1])
+    except OSError:
+        pass
+    return None
+
+
 def cpu_baseline(w, budget_s=15.0):
     """The reference's CPU path (per-adapter F.linear pairs + autograd, restated in oracle/) on this host."""
     import torch
@@ -59,6 +72,9 @@ def main():
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--sets', type=int, default=3, help='rotated buffer sets')
+    ap.add_argument('--calibrate-copy', action='store_true',
+                    help='also run five plain 128 MiB device copies (a known-size kernel to scale rocprofv3 --pmc '
+                         'FETCH_SIZE / WRITE_SIZE readings by)')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py measures one GPU: this path has no multi-GPU part (rows shard trivially; see DESIGN.md). '
@@ -137,6 +153,11 @@ def main():
     fwd_ms = shrink_ms + expand_ms
     bwd_ms = sum(e[2].elapsed_time(e[3]) for e in events) / args.steps
 
+    if args.calibrate_copy:
+        for _ in range(5):
+            sets[0]['dx'].copy_(sets[1]['x'])      # reads T*K*2 bytes, writes T*K*2 bytes
+        torch.cuda.synchronize()
+
     # base GEMM, reported separately and not part of the step
     wbase = torch.randn(M, K, device=dev, dtype=dt) * 0.02
     xs = sets[0]['x']
@@ -172,7 +193,7 @@ def main():
                                'Zipf(1.1) ids shuffled; step = segment build + LoRA fwd + LoRA bwd (dX, dA, dB); '
                                'base GEMM excluded', 'tokens': T, 'in': K, 'out': M, 'adapters': G, 'rank': 16},
         'roofline': {'bound': 'hbm', 'achieved': achieved, 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                     'frac': achieved / HBM_PEAK_GBS, 'traffic': None,
+                     'frac': achieved / HBM_PEAK_GBS, 'traffic': measured_traffic('k_expand_mfma<1, 1>'),
                      'kernel': 'k_expand_mfma<1,1> (y += h B^T in place), forward launch',
                      'algorithmic_bytes_per_launch': expand_bytes, 'avg_launch_ms': expand_ms},
         'step_detail': {'shrink_ms': shrink_ms, 'expand_ms': expand_ms, 'fwd_ms': fwd_ms, 'bwd_ms': bwd_ms, 'segment_build_and_gaps_ms': ms_per_step - fwd_ms - bwd_ms,
