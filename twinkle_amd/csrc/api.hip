@@ -41,8 +41,7 @@ int run_wgrad(const WgradArgs& a, const SegView& V, const SegLayout& L, int dtyp
     rc = launch_wgrad_mfma(a, V, L, s);
   else
     rc = launch_wgrad_generic(a, V, L, dtype, s);
-  if (rc != TK_OK) return rc;
-  return launch_wgrad_reduce(a, V, L, dtype, s);
+  return rc;
 }
 
 }  // namespace
@@ -190,6 +189,19 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
   char* w = (char*)ws;
   void* dh = w + B.off_dh;
   int rc;
+  WgradArgs ga{}, gb{};
+  // dB first: the two passes over dy (this one and the shrink below) run back to back, so the second
+  // one is served from the 256 MB last-level cache instead of HBM
+  if (grad_B) {
+    WgradArgs& g = gb;
+    g.src = dy;  g.ld_src = lddy;
+    g.hT = h;    g.ldh = B.ldh;
+    g.partial = (float*)(w + B.off_part_b);
+    g.grad = grad_B;  g.ld_grad = d->ldb;
+    g.rank = d->rank;  g.width = d->out_features;  g.transposed = 1;
+    g.accumulate = accumulate;  g.map_rows = d->map_rows;  g.rpad = (int32_t)B.rpad;
+    if ((rc = run_wgrad(g, V, L, d->dtype, s)) != TK_OK) return rc;
+  }
   if (dx || grad_A) {
     void* bT = w + B.off_wT_shrink;
     void* aT = w + B.off_wT_expand;
@@ -209,7 +221,7 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
     if ((rc = run_pass(a, V, L, d->dtype, 3, s)) != TK_OK) return rc;
   }
   if (grad_A) {
-    WgradArgs g{};
+    WgradArgs& g = ga;
     g.src = x;  g.ld_src = ldx;
     g.hT = dh;  g.ldh = B.ldh;
     g.partial = (float*)(w + B.off_part_a);
@@ -218,17 +230,8 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
     g.accumulate = accumulate;  g.map_rows = d->map_rows;  g.rpad = (int32_t)B.rpad;
     if ((rc = run_wgrad(g, V, L, d->dtype, s)) != TK_OK) return rc;
   }
-  if (grad_B) {
-    WgradArgs g{};
-    g.src = dy;  g.ld_src = lddy;
-    g.hT = h;    g.ldh = B.ldh;
-    g.partial = (float*)(w + B.off_part_b);
-    g.grad = grad_B;  g.ld_grad = d->ldb;
-    g.rank = d->rank;  g.width = d->out_features;  g.transposed = 1;
-    g.accumulate = accumulate;  g.map_rows = d->map_rows;  g.rpad = (int32_t)B.rpad;
-    if ((rc = run_wgrad(g, V, L, d->dtype, s)) != TK_OK) return rc;
-  }
-  return TK_OK;
+  // the chunk partials of both contractions are summed by one launch
+  return launch_wgrad_reduce(grad_A ? &ga : nullptr, grad_B ? &gb : nullptr, V, L, d->dtype, s);
 }
 
 }  // extern "C"

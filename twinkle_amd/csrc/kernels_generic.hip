@@ -177,12 +177,17 @@ __global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkI
 
 // Groups with several chunks: sum their partials in chunk order.  Groups with
 // no rows: clear the live block when overwriting.  One (group, rank index,
-// 256 columns) per block.
+// 256 columns) per block; blockIdx.z >= rpad selects the second argument set,
+// so that the reductions of dA and dB share one launch.
 template <typename T>
-__global__ __launch_bounds__(256) void k_wgrad_reduce(WgradArgs a, const int32_t* __restrict__ chunk_first,
+__global__ __launch_bounds__(256) void k_wgrad_reduce(WgradArgs a0, WgradArgs a1, int rpad,
+                                                      const int32_t* __restrict__ chunk_first,
                                                       const int32_t* __restrict__ partial_first) {
+  const bool second = (int)blockIdx.z >= rpad;
+  const WgradArgs& a = second ? a1 : a0;
+  if (a.grad == nullptr) return;
   const int g = blockIdx.x;
-  const int n = blockIdx.z;
+  const int n = second ? blockIdx.z - rpad : blockIdx.z;
   if (n >= min(a.rank[g], a.rpad)) return;
   const int nchunk = chunk_first[g + 1] - chunk_first[g];
   if (nchunk == 1) return;
@@ -258,13 +263,20 @@ int launch_wgrad_generic(const WgradArgs& a, const SegView& seg, const SegLayout
   return check_launch();
 }
 
-int launch_wgrad_reduce(const WgradArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s) {
-  if (L.groups == 0) return TK_OK;
-  const dim3 grid((unsigned)L.groups, (unsigned)ceil_div(a.width, 256), (unsigned)a.rpad);
+int launch_wgrad_reduce(const WgradArgs* a0, const WgradArgs* a1, const SegView& seg, const SegLayout& L, int dtype,
+                        hipStream_t s) {
+  if (L.groups == 0 || (!a0 && !a1)) return TK_OK;
+  WgradArgs none{};
+  const WgradArgs& x0 = a0 ? *a0 : none;
+  const WgradArgs& x1 = a1 ? *a1 : none;
+  const int rpad = a0 ? a0->rpad : a1->rpad;
+  const int width = std::max(a0 ? a0->width : 0, a1 ? a1->width : 0);
+  const dim3 grid((unsigned)L.groups, (unsigned)ceil_div(width, 256), (unsigned)(a1 ? 2 * rpad : rpad));
   if (dtype == TK_DTYPE_F32)
-    hipLaunchKernelGGL(k_wgrad_reduce<float>, grid, dim3(256), 0, s, a, seg.chunk_first, seg.partial_first);
+    hipLaunchKernelGGL(k_wgrad_reduce<float>, grid, dim3(256), 0, s, x0, x1, rpad, seg.chunk_first, seg.partial_first);
   else
-    hipLaunchKernelGGL(k_wgrad_reduce<bf16_t>, grid, dim3(256), 0, s, a, seg.chunk_first, seg.partial_first);
+    hipLaunchKernelGGL(k_wgrad_reduce<bf16_t>, grid, dim3(256), 0, s, x0, x1, rpad, seg.chunk_first,
+                       seg.partial_first);
   return check_launch();
 }
 

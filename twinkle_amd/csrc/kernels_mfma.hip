@@ -283,29 +283,33 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
   const int r = g_raw < 0 ? 0 : min(a.rank[g], RP);
   const bf16_t* W2 = group_weight<bf16_t>(a.w_expand, a.w_expand_base, a.expand_group_stride, g);
 
-  uint4 y[CPW][2][4];
-  uint4 bq[CPW][8][NKS];
-#pragma unroll
-  for (int u = 0; u < CPW; ++u) {
+  // Two register buffers: the loads of column group u + 1 are issued before group u is consumed, so a
+  // wave always has a group's worth of loads (8 KB of dst, 4 KB of weights) in flight.
+  uint4 y[2][2][4];
+  uint4 bq[2][8][NKS];
+  auto issue = [&](int u, int buf) {
     const bool gok = cg0 + u < ngroups;  // wave-uniform
     const int c0 = (gok ? cg0 + u : cg0) << 7;
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) y[u][tt][v] = (rok[tt][v] && gok) ? ld16(yp[tt][v] + c0) : zero4();
+      for (int v = 0; v < 4; ++v) y[buf][tt][v] = (rok[tt][v] && gok) ? ld16(yp[tt][v] + c0) : zero4();
 #pragma unroll
     for (int q = 0; q < 8; ++q)
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
         const int n0 = 32 * ks + 8 * kb;
-        bq[u][q][ks] =
+        bq[buf][q][ks] =
             n0 < r ? keep_first(ld16(W2 + (int64_t)(c0 + 8 * li + q) * a.ld_expand + n0), r - n0) : zero4();
       }
-  }
+  };
+  issue(0, 0);
   if (r <= 0) return;  // unused tile, or adapter not live on this layer (uniform over the wave)
 #pragma unroll
   for (int u = 0; u < CPW; ++u) {
     if (cg0 + u >= ngroups) break;
+    const int buf = u & 1;
+    if (u + 1 < CPW) issue(u + 1, buf ^ 1);
     const int c0 = (cg0 + u) << 7;
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
@@ -314,12 +318,12 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
       for (int q = 0; q < 8; ++q) {
         d[q] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) d[q] = mfma16(hop[tt][ks], bq[u][q][ks], d[q]);
+        for (int ks = 0; ks < NKS; ++ks) d[q] = mfma16(hop[tt][ks], bq[buf][q][ks], d[q]);
       }
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         if (!rok[tt][v]) continue;
-        const uint4 yy = y[u][tt][v];
+        const uint4 yy = y[buf][tt][v];
         uint4 o;
         o.x = pack_bf16(bf16_lo(yy.x) + d[0][v], bf16_hi(yy.x) + d[1][v]);
         o.y = pack_bf16(bf16_lo(yy.y) + d[2][v], bf16_hi(yy.y) + d[3][v]);

@@ -215,7 +215,9 @@ int launch_unpermute_wgrad(const void* dout, int64_t ld_dout, const void* rows_,
 int launch_pass_generic(const PassArgs& a, const SegView& seg, const SegLayout& L, int dtype, int phases,
                         hipStream_t s);
 int launch_wgrad_generic(const WgradArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s);
-int launch_wgrad_reduce(const WgradArgs& a, const SegView& seg, const SegLayout& L, int dtype, hipStream_t s);
+// sums the chunk partials of up to two contractions (dA, dB; either may be null) in one launch
+int launch_wgrad_reduce(const WgradArgs* a0, const WgradArgs* a1, const SegView& seg, const SegLayout& L, int dtype,
+                        hipStream_t s);
 int launch_transpose_weights(const tk_lora_desc& d, void* bT, void* aT, hipStream_t s);
 
 // kernels_mfma.hip : bf16, aligned shapes, MFMA
