@@ -36,7 +36,9 @@ enum { TK_KEY_I32 = 0, TK_KEY_I64 = 1 };
 
 /* Rows per forward tile and per weight-gradient chunk (fixed at build time). */
 #define TK_TILE_ROWS 32
+#ifndef TK_CHUNK_ROWS
 #define TK_CHUNK_ROWS 512
+#endif
 #define TK_MAX_GROUPS 16384
 #define TK_MAX_RANK 128
 

@@ -467,6 +467,195 @@ __global__ __launch_bounds__(NW * 64) void k_wgrad_mfma(WgradArgs a, const Chunk
   }
 }
 
+// Eight consecutive bf16 results: one 16-byte store when `vec`, element stores otherwise; `keep` (1..8)
+// elements are written, the rest of the destination is left alone.
+__device__ inline void store_bf16x8(bf16_t* o, const float (&v)[8], int keep, bool accumulate, bool vec) {
+  if (vec && keep >= 8) {
+    float f[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = v[i];
+    if (accumulate) {
+      const uint4 old = ld16(o);
+      f[0] += bf16_lo(old.x); f[1] += bf16_hi(old.x); f[2] += bf16_lo(old.y); f[3] += bf16_hi(old.y);
+      f[4] += bf16_lo(old.z); f[5] += bf16_hi(old.z); f[6] += bf16_lo(old.w); f[7] += bf16_hi(old.w);
+    }
+    st16(o, make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7])));
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    if (i >= keep) break;
+    float val = v[i];
+    if (accumulate) val += to_f32(o[i]);
+    o[i] = (bf16_t)(pack_bf16(val, 0.f) & 0xffffu);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Weight gradient: out_g[n][c] = sum over the rows of group g of hT[n][slot] * src[row(slot)][c].
+//
+// Work item = (chunk of up to 16 tiles of one group, 128 source columns), one block of NW waves; wave w
+// owns tiles w*TPW .. of the chunk.  The loads run as a software pipeline over the wave's tiles: the row
+// indices of tile t+DEPTH+1 and the source rows of tile t+DEPTH are requested before tile t is consumed,
+// so a wave never waits on an index load and always has DEPTH tiles (8 KB each) in flight.  A lane loads
+// 16 B of eight rows, transposes the 8x8 block in registers (v_perm_b32) and feeds it as the MFMA A
+// operand with the rows as contraction index.  The waves' sums are added in wave order in LDS, staged
+// there in [n][column] order and leave as whole 512-byte rows: into the chunk's slot of the partial
+// buffer (groups that span several chunks; k_wgrad_reduce adds the chunks in order) or straight into the
+// gradient (single-chunk groups).  No atomics: the result is bitwise repeatable.
+// ---------------------------------------------------------------------------
+template <int NB, int NW, int DEPTH>
+__global__ __launch_bounds__(NW * 64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo* __restrict__ chunks,
+                                                        const int32_t* __restrict__ slot_rows) {
+  constexpr int TPW = kChunkTiles / NW;  // tiles per wave
+  constexpr int RP = 16 * NB;
+  constexpr int OS = 132;  // row stride of the staged result in floats (4 mod 32: conflict-free 16-byte accesses)
+  constexpr int RED = (NW - 1) * 32 * NB * 64;
+  constexpr int OUT = RP * OS;
+  __shared__ __attribute__((aligned(16))) float lds[RED > OUT ? RED : OUT];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  // column block fastest: blocks that run together read neighbouring pieces of the same rows
+  const int c0 = blockIdx.x * 128;
+  const ChunkInfo ci = chunks[blockIdx.y];
+  const int g = ci.group;
+  if (g < 0) return;
+  const int r = min(a.rank[g], RP);
+  if (r <= 0) return;
+
+  const bf16_t* src = (const bf16_t*)a.src + c0 + 8 * li;
+  const bf16_t* hT = (const bf16_t*)a.hT + 8 * kb;
+  const int32_t* rows_p = slot_rows + ci.tile0 * kTileRows + 8 * kb;  // this lane's 8 slots of the chunk's first tile
+  f32x4 acc[8][NB];
+#pragma unroll
+  for (int q = 0; q < 8; ++q)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[q][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int t0 = wave * TPW;
+  if (t0 < ci.ntiles) {
+    int4 ra[TPW], rb[TPW];
+    uint4 x[TPW][8], h[TPW][NB];
+    auto load_rows = [&](int u) {
+      const int t = min(t0 + u, ci.ntiles - 1);  // tiles past the end re-read the last one and are masked below
+      ra[u] = *reinterpret_cast<const int4*>(rows_p + t * kTileRows);
+      rb[u] = *reinterpret_cast<const int4*>(rows_p + t * kTileRows + 4);
+    };
+    auto issue = [&](int u) {
+      const bool tok = t0 + u < ci.ntiles;  // wave-uniform
+      const int t = tok ? t0 + u : 0;
+      const int rows[8] = {ra[u].x, ra[u].y, ra[u].z, ra[u].w, rb[u].x, rb[u].y, rb[u].z, rb[u].w};
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+        x[u][q] = (tok && rows[q] >= 0) ? ld16(src + (int64_t)rows[q] * a.ld_src) : zero4();
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        h[u][nb] = tok ? ld16(hT + (int64_t)(16 * nb + li) * a.ldh + (ci.tile0 + t) * kTileRows) : zero4();
+    };
+    auto consume = [&](int u) {
+      // 8x8 transpose inside the lane: tr[q] holds column q of the 8 rows
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const int d = q >> 1;
+        const uint32_t sel = (q & 1) ? 0x07060302u : 0x05040100u;
+        uint32_t e[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const uint32_t wsrc[4] = {x[u][i].x, x[u][i].y, x[u][i].z, x[u][i].w};
+          e[i] = wsrc[d];
+        }
+        uint4 tr;
+        tr.x = __builtin_amdgcn_perm(e[1], e[0], sel);
+        tr.y = __builtin_amdgcn_perm(e[3], e[2], sel);
+        tr.z = __builtin_amdgcn_perm(e[5], e[4], sel);
+        tr.w = __builtin_amdgcn_perm(e[7], e[6], sel);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[q][nb] = mfma16(tr, h[u][nb], acc[q][nb]);
+      }
+    };
+#pragma unroll
+    for (int u = 0; u <= DEPTH && u < TPW; ++u) load_rows(u);
+#pragma unroll
+    for (int u = 0; u < DEPTH && u < TPW; ++u) issue(u);
+#pragma unroll
+    for (int u = 0; u < TPW; ++u) {
+      if (u + DEPTH < TPW) issue(u + DEPTH);
+      if (u + DEPTH + 1 < TPW) load_rows(u + DEPTH + 1);
+      consume(u);
+    }
+  }
+
+  // add the waves' accumulators in wave order; wave 0 keeps the result
+  if (NW > 1) {
+    if (wave > 0) {
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) lds[((wave - 1) * 32 * NB + (q * NB + nb) * 4 + v) * 64 + lane] = acc[q][nb][v];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+    for (int w = 0; w < NW - 1; ++w)
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[q][nb][v] += lds[(w * 32 * NB + (q * NB + nb) * 4 + v) * 64 + lane];
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");  // the sums are read before the staging below overwrites them
+  }
+
+  // lane holds out[n = 16 nb + li][32 kb + 8 v + q]; stage it as out[n][0..127]
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      float* o = lds + (16 * nb + li) * OS + 32 * kb + 8 * v;
+      *reinterpret_cast<float4*>(o) = make_float4(acc[0][nb][v], acc[1][nb][v], acc[2][nb][v], acc[3][nb][v]);
+      *reinterpret_cast<float4*>(o + 4) = make_float4(acc[4][nb][v], acc[5][nb][v], acc[6][nb][v], acc[7][nb][v]);
+    }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+
+  if (ci.partial >= 0) {
+    float* part = a.partial + (int64_t)ci.partial * a.rpad * a.width + c0;
+#pragma unroll
+    for (int i = 0; i < RP / 2; ++i) {
+      const int n = 2 * i + (lane >> 5), c = 4 * (lane & 31);
+      if (n < r) *reinterpret_cast<float4*>(part + (int64_t)n * a.width + c) = *reinterpret_cast<const float4*>(lds + n * OS + c);
+    }
+    return;
+  }
+  bf16_t* gp = (bf16_t*)a.grad[g];
+  const bool vec = (reinterpret_cast<uintptr_t>(gp) & 15u) == 0 && (a.ld_grad & 7) == 0;
+  if (!a.transposed) {
+    // grad[n][c0 + c]: four rows of 128 columns per step
+#pragma unroll
+    for (int i = 0; i < RP / 4; ++i) {
+      const int n = 4 * i + kb, c = 8 * li;
+      if (n >= r) continue;
+      const float4 lo = *reinterpret_cast<const float4*>(lds + n * OS + c);
+      const float4 hi = *reinterpret_cast<const float4*>(lds + n * OS + c + 4);
+      const float v8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      store_bf16x8(gp + (int64_t)n * a.ld_grad + c0 + c, v8, 8, a.accumulate != 0, vec);
+    }
+  } else {
+    // grad[c0 + c][n]: a lane owns columns c = lane and lane + 64
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int c = lane + 64 * half;
+#pragma unroll
+      for (int n8 = 0; n8 < RP; n8 += 8) {
+        if (n8 >= r) break;
+        float v8[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v8[i] = lds[(n8 + i) * OS + c];
+        store_bf16x8(gp + (int64_t)(c0 + c) * a.ld_grad + n8, v8, min(8, r - n8), a.accumulate != 0, vec);
+      }
+    }
+  }
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <int NB, int CPW>
@@ -492,6 +681,12 @@ template <int NB, int NW, int TB>
 void launch_wgrad(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
   const dim3 grid((unsigned)(a.width / 128), (unsigned)L.max_chunks);
   hipLaunchKernelGGL((k_wgrad_mfma<NB, NW, TB>), grid, dim3(NW * 64), 0, s, a, seg.chunks, seg.slot_table(a.map_rows));
+}
+
+template <int NB, int NW, int DEPTH>
+void launch_wgrad_pipe(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
+  const dim3 grid((unsigned)(a.width / 128), (unsigned)L.max_chunks);
+  hipLaunchKernelGGL((k_wgrad_pipe<NB, NW, DEPTH>), grid, dim3(NW * 64), 0, s, a, seg.chunks, seg.slot_table(a.map_rows));
 }
 
 }  // namespace
@@ -522,9 +717,9 @@ bool wgrad_mfma_supported(const WgradArgs& a) {
 
 int launch_wgrad_mfma(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
   if (L.rows == 0) return TK_OK;
-  if (a.rpad <= 16) launch_wgrad<1, 2, 2>(a, seg, L, s);
-  else if (a.rpad <= 32) launch_wgrad<2, 2, 2>(a, seg, L, s);
-  else launch_wgrad<4, 2, 2>(a, seg, L, s);
+  if (a.rpad <= 16) launch_wgrad_pipe<1, 1, 2>(a, seg, L, s);
+  else if (a.rpad <= 32) launch_wgrad_pipe<2, 1, 2>(a, seg, L, s);
+  else launch_wgrad_pipe<4, 2, 1>(a, seg, L, s);
   return check_launch();
 }
 

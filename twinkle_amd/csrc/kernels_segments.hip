@@ -2,7 +2,8 @@
 // gather / scatter-back kernels that use its table.  Integer work, HBM-light:
 // the table is built once per batch and read by every LoRA layer.
 //
-// Pipeline (three launches, no host synchronisation anywhere):
+// Small inputs take one launch (k_seg_one, below).  General pipeline (three
+// launches, no host synchronisation anywhere):
 //   k_seg_hist    one wave per 512 rows: per-key counts by bit-sliced ballots
 //                 (no contended atomics) -> hist[block][group]
 //   k_seg_scan    one block: per-group totals, exclusive scans -> offsets and
@@ -266,6 +267,186 @@ __global__ __launch_bounds__(64) void k_seg_scatter(const KeyT* __restrict__ key
   }
 }
 
+// ---------------------------------------------------------------------------
+// Single-launch builder for the common small case (at most kOneGroups groups and kOneBlocks * 512
+// rows, i.e. one micro-batch of tokens over a handful of adapters).  Three dependent launches cost
+// more than the work itself there, so every block redundantly counts *all* keys (a few hundred KB,
+// served from L2), which gives it the group totals and the number of equal keys ahead of its own 512
+// rows without any communication.  Counting is one LDS add per key into one of 16 sub-histograms
+// (lane % 16, rows of 65 words: equal keys of different lanes fall into different banks).  The
+// block's own 512 rows are ranked by its first 8 waves, one 64-row round each: rank inside the round
+// from bit-sliced ballots, rounds before it from a small per-round table.  All threads then fill
+// the block's share of the tile / chunk tables.  Integer adds only: the result does not depend on
+// the order in which the adds land.
+// ---------------------------------------------------------------------------
+constexpr int kOneGroups = 64;
+constexpr int kOneBlocks = 64;
+constexpr int kOneWaves = 16;
+constexpr int kOneSubs = 16;
+constexpr int kOneBatch = kOneBlocks / kOneWaves;  // sort blocks whose keys a wave requests together
+
+template <typename KeyT>
+__global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restrict__ keys, int rows, int groups,
+                                                            int key_bits, int sort_blocks, int max_tiles,
+                                                            int max_chunks, SegView V, int64_t* __restrict__ perm_out,
+                                                            int64_t* __restrict__ offsets_out) {
+  __shared__ int32_t cnt[2][kOneSubs][kOneGroups + 1];  // keys ahead of this block / in it and after it
+  __shared__ int32_t round_cnt[kKeysPerLane][kOneGroups];  // this block's keys per 64-row round
+  __shared__ int32_t first[4][kOneGroups + 1];          // offsets, tile_first, chunk_first, partial_first
+  __shared__ int32_t cursor[kOneGroups];                // sorted position of the block's first row of each group
+  __shared__ int32_t bad_s[kOneWaves];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, blk = blockIdx.x;
+  const int64_t base = (int64_t)blk * kSortBlockRows;
+
+  // all key loads first: the block's own rows (one round per wave), then this wave's share of all rows
+  int unused = 0, bad = 0;
+  int mine = -1;
+  if (wave < kKeysPerLane) {
+    const int64_t f = base + wave * 64 + lane;
+    mine = f < rows ? load_key(keys, f, groups, &unused) : -1;
+  }
+  int k[kOneBatch][kKeysPerLane];
+#pragma unroll
+  for (int u = 0; u < kOneBatch; ++u)
+#pragma unroll
+    for (int j = 0; j < kKeysPerLane; ++j) {
+      const int64_t f = (int64_t)(wave + u * kOneWaves) * kSortBlockRows + j * 64 + lane;
+      k[u][j] = f < rows ? load_key(keys, f, groups, &bad) : -1;
+    }
+  for (int i = tid; i < 2 * kOneSubs * (kOneGroups + 1); i += kOneWaves * 64) (&cnt[0][0][0])[i] = 0;
+  for (int i = tid; i < kKeysPerLane * kOneGroups; i += kOneWaves * 64) (&round_cnt[0][0])[i] = 0;
+  __syncthreads();
+
+#pragma unroll
+  for (int u = 0; u < kOneBatch; ++u) {
+    if (wave + u * kOneWaves >= sort_blocks) break;  // wave-uniform
+    int32_t* c = cnt[wave + u * kOneWaves < blk ? 0 : 1][lane & (kOneSubs - 1)];
+#pragma unroll
+    for (int j = 0; j < kKeysPerLane; ++j)
+      if (k[u][j] >= 0) atomicAdd(&c[k[u][j]], 1);
+  }
+  int rank_in_round = 0;
+  if (wave < kKeysPerLane) {
+    const bool valid = mine >= 0;
+    const unsigned long long same = same_key_lanes(valid, max(mine, 0), key_bits);
+    rank_in_round = __popcll(same & ((1ull << lane) - 1ull));  // rows with equal keys keep their lane order
+    if (valid && rank_in_round == 0) round_cnt[wave][mine] = __popcll(same);
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) bad += __shfl_xor(bad, d, 64);
+  if (lane == 0) bad_s[wave] = bad;
+  __syncthreads();
+
+  if (wave == 0) {
+    int before = 0, rest = 0;
+    if (lane < groups) {
+#pragma unroll
+      for (int sub = 0; sub < kOneSubs; ++sub) {
+        before += cnt[0][sub][lane];
+        rest += cnt[1][sub][lane];
+      }
+    }
+    const int count = before + rest;
+    const int ntile = (count + kTileRows - 1) / kTileRows;
+    const int nchunk = (ntile + kChunkTiles - 1) / kChunkTiles;
+    const int npart = nchunk > 1 ? nchunk : 0;
+    int v[4] = {count, ntile, nchunk, npart}, excl[4], total[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      int incl = v[t];
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int o = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += o;
+      }
+      excl[t] = incl - v[t];
+      total[t] = __shfl(incl, 63, 64);
+    }
+    if (lane < groups) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) first[t][lane] = excl[t];
+      cursor[lane] = excl[0] + before;
+    }
+    if (lane == 0) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) first[t][groups] = total[t];
+    }
+    if (blk == 0) {
+      if (lane < groups) {
+        V.offsets[lane] = excl[0];
+        V.tile_first[lane] = excl[1];
+        V.chunk_first[lane] = excl[2];
+        V.partial_first[lane] = excl[3];
+        if (offsets_out) offsets_out[lane] = excl[0];
+      }
+      if (lane == 0) {
+        V.offsets[groups] = total[0];
+        V.tile_first[groups] = total[1];
+        V.chunk_first[groups] = total[2];
+        V.partial_first[groups] = total[3];
+        if (offsets_out) offsets_out[groups] = total[0];
+        int bad_total = 0;
+        for (int w = 0; w < kOneWaves; ++w) bad_total += bad_s[w];
+        SegHeader* hdr = V.header;
+        hdr->magic = kSegMagic;
+        hdr->rows = rows;
+        hdr->groups = groups;
+        hdr->num_tiles = total[1];
+        hdr->num_chunks = total[2];
+        hdr->num_partials = total[3];
+        hdr->bad_keys = bad_total;
+      }
+    }
+  }
+  __syncthreads();
+
+  const int32_t* offs = first[0];
+  const int32_t* tfirst = first[1];
+  const int32_t* cfirst = first[2];
+  const int32_t* pfirst = first[3];
+  if (wave < kKeysPerLane && mine >= 0) {
+    const int64_t f = base + wave * 64 + lane;
+    int pos = cursor[mine] + rank_in_round;
+    for (int w = 0; w < wave; ++w) pos += round_cnt[w][mine];
+    V.inv[f] = pos;
+    if (perm_out) perm_out[pos] = f;
+    // padded slot = 32 * first tile of the group + position inside the group
+    V.slot_row[tfirst[mine] * kTileRows + (pos - offs[mine])] = (int32_t)f;
+  }
+
+  const int num_tiles = tfirst[groups], num_chunks = cfirst[groups];
+  const int stride = sort_blocks * kOneWaves * 64;
+  for (int i = blk * kOneWaves * 64 + tid; i < max_tiles; i += stride) {
+    int g = -1, pos0 = 0, valid = 0;
+    if (i < num_tiles) {
+      g = group_of(tfirst, groups, i);
+      pos0 = offs[g] + (i - tfirst[g]) * kTileRows;  // sorted position of the tile's first slot
+      valid = min(kTileRows, offs[g + 1] - pos0);      // padding is at the end of a group's last tile
+    }
+    V.tile_group[i] = g;
+    V.tile_ticket[i] = 0;
+    int4* sp = reinterpret_cast<int4*>(V.slot_pos + (int64_t)i * kTileRows);
+#pragma unroll
+    for (int j = 0; j < kTileRows; j += 4)
+      sp[j / 4] = make_int4(j < valid ? pos0 + j : -1, j + 1 < valid ? pos0 + j + 1 : -1,
+                            j + 2 < valid ? pos0 + j + 2 : -1, j + 3 < valid ? pos0 + j + 3 : -1);
+    for (int j = valid; j < kTileRows; ++j) V.slot_row[(int64_t)i * kTileRows + j] = -1;
+  }
+  for (int i = blk * kOneWaves * 64 + tid; i < max_chunks; i += stride) {
+    ChunkInfo c{-1, 0, 0, -1};
+    if (i < num_chunks) {
+      const int g = group_of(cfirst, groups, i);
+      const int j = i - cfirst[g];
+      const int ntile = tfirst[g + 1] - tfirst[g];
+      c.group = g;
+      c.tile0 = tfirst[g] + j * kChunkTiles;
+      c.ntiles = min(kChunkTiles, ntile - j * kChunkTiles);
+      c.partial = cfirst[g + 1] - cfirst[g] > 1 ? pfirst[g] + j : -1;
+    }
+    V.chunks[i] = c;
+  }
+}
+
 // dst[j] = src[perm[j] mod tokens] * w[token, k], one block per padded slot (slot_row is perm in padded order)
 template <typename T>
 __global__ __launch_bounds__(256) void k_permute(const T* __restrict__ src, int64_t ld_src, T* __restrict__ dst,
@@ -337,6 +518,15 @@ int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t 
   const size_t lds = sizeof(int32_t) * (size_t)groups;
   int key_bits = 0;
   while ((1 << key_bits) < groups) ++key_bits;
+  if (groups <= kOneGroups && nblk <= kOneBlocks) {
+    if (key_dtype == TK_KEY_I32)
+      hipLaunchKernelGGL(k_seg_one<int32_t>, dim3(nblk), dim3(kOneWaves * 64), 0, s, (const int32_t*)keys, (int)rows,
+                         groups, key_bits, nblk, (int)L.max_tiles, (int)L.max_chunks, V, perm_out, offsets_out);
+    else
+      hipLaunchKernelGGL(k_seg_one<int64_t>, dim3(nblk), dim3(kOneWaves * 64), 0, s, (const int64_t*)keys, (int)rows,
+                         groups, key_bits, nblk, (int)L.max_tiles, (int)L.max_chunks, V, perm_out, offsets_out);
+    return check_launch();
+  }
   if (key_dtype == TK_KEY_I32)
     hipLaunchKernelGGL(k_seg_hist<int32_t>, dim3(nblk), dim3(64), lds, s, (const int32_t*)keys, (int)rows, groups,
                        key_bits, V.hist, V.bad);
