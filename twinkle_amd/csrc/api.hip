@@ -190,6 +190,10 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
   void* dh = w + B.off_dh;
   int rc;
   WgradArgs ga{}, gb{};
+  const bool need_wT = dx || grad_A;
+  void* bT = w + B.off_wT_shrink;
+  void* aT = w + B.off_wT_expand;
+  bool wT_done = false;
   // dB first: the two passes over dy (this one and the shrink below) run back to back, so the second
   // one is served from the 256 MB last-level cache instead of HBM
   if (grad_B) {
@@ -200,12 +204,20 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
     g.grad = grad_B;  g.ld_grad = d->ldb;
     g.rank = d->rank;  g.width = d->out_features;  g.transposed = 1;
     g.accumulate = accumulate;  g.map_rows = d->map_rows;  g.rpad = (int32_t)B.rpad;
+    if (need_wT && d->dtype == TK_DTYPE_BF16 && !force_generic() && wgrad_mfma_supported(g) &&
+        d->out_features % 8 == 0) {
+      // the MFMA launch also writes the transposed weight copies of the pass below
+      g.tr.lora_A = d->lora_A;  g.tr.lda = d->lda;
+      g.tr.lora_B = d->lora_B;  g.tr.ldb = d->ldb;
+      g.tr.aT = aT;  g.tr.bT = bT;
+      g.tr.in_features = d->in_features;  g.tr.out_features = d->out_features;  g.tr.groups = d->num_groups;
+      wT_done = true;
+    }
     if ((rc = run_wgrad(g, V, L, d->dtype, s)) != TK_OK) return rc;
+    g.tr = TransposeJob{};
   }
-  if (dx || grad_A) {
-    void* bT = w + B.off_wT_shrink;
-    void* aT = w + B.off_wT_expand;
-    if ((rc = launch_transpose_weights(*d, bT, aT, s)) != TK_OK) return rc;
+  if (need_wT) {
+    if (!wT_done && (rc = launch_transpose_weights(*d, bT, aT, s)) != TK_OK) return rc;
     PassArgs a{};
     a.src = dy;  a.ld_src = lddy;
     a.dst = dx;  a.ld_dst = lddx;

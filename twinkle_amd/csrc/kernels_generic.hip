@@ -188,24 +188,25 @@ __global__ __launch_bounds__(256) void k_wgrad_reduce(WgradArgs a0, WgradArgs a1
   if (a.grad == nullptr) return;
   const int g = blockIdx.x;
   const int n = second ? blockIdx.z - rpad : blockIdx.z;
-  if (n >= min(a.rank[g], a.rpad)) return;
-  const int nchunk = chunk_first[g + 1] - chunk_first[g];
+  // independent loads first
+  const int rk = a.rank[g], cf0 = chunk_first[g], cf1 = chunk_first[g + 1], pf = partial_first[g];
+  if (n >= min(rk, a.rpad)) return;
+  const int nchunk = cf1 - cf0;
   if (nchunk == 1) return;
   if (nchunk == 0 && a.accumulate) return;
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= a.width) return;
-  const float* p = a.partial + ((int64_t)partial_first[g] * a.rpad + n) * a.width + c;
+  const float* p = a.partial + ((int64_t)pf * a.rpad + n) * a.width + c;
   const int64_t stride = (int64_t)a.rpad * a.width;
   float acc = 0.f;
-  int j = 0;
-  for (; j + 4 <= nchunk; j += 4) {
-    const float v0 = p[(j + 0) * stride], v1 = p[(j + 1) * stride], v2 = p[(j + 2) * stride], v3 = p[(j + 3) * stride];
-    acc += v0;
-    acc += v1;
-    acc += v2;
-    acc += v3;
+  // eight chunks are requested together (their latencies overlap) and added in chunk order
+  for (int j0 = 0; j0 < nchunk; j0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = j0 + j < nchunk ? p[(j0 + j) * stride] : 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc += v[j];
   }
-  for (; j < nchunk; ++j) acc += p[j * stride];
   store_grad<T>(a, g, n, c, acc);
 }
 

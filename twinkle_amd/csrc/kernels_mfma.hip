@@ -12,6 +12,8 @@
 // The contraction index k may be permuted freely as long as A and B agree, and
 // the output indices i, j may be mapped to any rows / columns: both freedoms
 // are used to make the global accesses contiguous.
+#include <algorithm>
+
 #include "tk_device.h"
 
 namespace tk {
@@ -210,17 +212,29 @@ __global__ __launch_bounds__(256) void k_shrink_finish(PassArgs a, bf16_t* __res
   const int g = tile_group[tile_id];
   const int my_row = slot_rows[slot0 + (tid & 31)];
   const float* tile_part = a.hpart + (int64_t)tile_id * a.kslices * (kTileRows * RP);
-  float sums[(kTileRows * RP + 255) / 256];
+  constexpr int NI = (kTileRows * RP + 255) / 256;
+  float sums[NI];
 #pragma unroll
-  for (int i = 0; i < (kTileRows * RP + 255) / 256; ++i) {
-    const int idx = tid + 256 * i;
-    float sum = 0.f;
-    if (idx < kTileRows * RP)
-      for (int k = 0; k < a.kslices; ++k) sum += tile_part[(int64_t)k * (kTileRows * RP) + idx];
-    sums[i] = sum;
+  for (int i = 0; i < NI; ++i) sums[i] = 0.f;
+  // eight slices are requested together (their latencies overlap) and added in slice order
+  for (int k0 = 0; k0 < a.kslices; k0 += 8) {
+    float v[NI][8];
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int idx = tid + 256 * i;
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        v[i][k] = (idx < kTileRows * RP && k0 + k < a.kslices) ? tile_part[(int64_t)(k0 + k) * (kTileRows * RP) + idx] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) sums[i] += v[i][k];
   }
-  if (g < 0) return;
-  if (a.rank[g] <= 0) return;
+  const int gg = max(g, 0);
+  const int rk = a.rank[gg];
+  const float sc = a.scale[gg];
+  if (g < 0 || rk <= 0) return;
   const int cnt = __popcll(__ballot(my_row >= 0) & 0xffffffffull);  // padding is at the end of a tile
 #pragma unroll
   for (int i = 0; i < (kTileRows * RP + 255) / 256; ++i) {
@@ -228,7 +242,7 @@ __global__ __launch_bounds__(256) void k_shrink_finish(PassArgs a, bf16_t* __res
     if (idx < kTileRows * RP) part[idx / RP][idx % RP] = sums[i];
   }
   __syncthreads();
-  shrink_epilogue<RP, 256>(&part[0][0], 1, a, hrow, slot0, cnt, a.scale[g]);
+  shrink_epilogue<RP, 256>(&part[0][0], 1, a, hrow, slot0, cnt, sc);
 }
 
 // ---------------------------------------------------------------------------
@@ -335,138 +349,6 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
   }
 }
 
-// ---------------------------------------------------------------------------
-// Row contraction (weight gradients): out[n][c] = sum_slot hT[n][slot] * src[row(slot)][c]
-// over the tiles of one chunk of one group, for 128 columns per block.  The
-// NW waves of a block split the chunk's tiles (wave w: tiles w*16/NW ...), so
-// a chunk is several short streams, and add their accumulators in LDS in
-// wave order at the end.  Each lane loads 8 rows x 8 columns (eight fully
-// coalesced wave loads of 4 x 256 B), transposes its 8x8 block in registers
-// with v_perm_b32 so that rows become the MFMA contraction index, and
-// accumulates 128 columns x rank in MFMA registers.  A wave issues the loads
-// of all its tiles before it consumes the first.  Padding slots contribute
-// nothing: their h is exactly zero and their rows are not loaded.
-// ---------------------------------------------------------------------------
-template <int NB, int NW, int TB>
-__global__ __launch_bounds__(NW * 64) void k_wgrad_mfma(WgradArgs a, const ChunkInfo* __restrict__ chunks,
-                                                        const int32_t* __restrict__ slot_rows) {
-  __shared__ float red[NW > 1 ? NW - 1 : 1][8 * NB * 4][64];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
-  // column block fastest: blocks that run together read neighbouring pieces of the same rows
-  const int c0 = blockIdx.x * 128;
-  const ChunkInfo ci = chunks[blockIdx.y];
-  const int g = ci.group;
-  if (g < 0) return;
-  const int r = min(a.rank[g], 16 * NB);
-  if (r <= 0) return;
-
-  const bf16_t* src = (const bf16_t*)a.src + c0 + 8 * li;
-  const bf16_t* hT = (const bf16_t*)a.hT + 8 * kb;
-  const int32_t* rows_p = slot_rows + ci.tile0 * kTileRows + 8 * kb;  // this lane's 8 slots of the chunk's first tile
-  f32x4 acc[8][NB];
-#pragma unroll
-  for (int q = 0; q < 8; ++q)
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) acc[q][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-  // A wave owns tiles wave*TPW .. wave*TPW+TPW-1 of the chunk and issues the loads of up to four of
-  // them before it consumes the first (32 KB per wave in flight).
-  constexpr int TPW = kChunkTiles / NW;       // tiles per wave
-  static_assert(TPW % TB == 0, "TB (tiles whose loads are issued together) must divide the tiles per wave");
-  for (int tb = wave * TPW; tb < wave * TPW + TPW && tb < ci.ntiles; tb += TB) {
-    uint4 x[TB][8];
-    uint4 h[TB][NB];
-#pragma unroll
-    for (int u = 0; u < TB; ++u) {
-      const bool tok = tb + u < ci.ntiles;  // wave-uniform
-      const int t = tok ? tb + u : 0;
-      const int4 ra = *reinterpret_cast<const int4*>(rows_p + t * kTileRows);
-      const int4 rb = *reinterpret_cast<const int4*>(rows_p + t * kTileRows + 4);
-      const int rows[8] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w};
-#pragma unroll
-      for (int q = 0; q < 8; ++q)
-        x[u][q] = (tok && rows[q] >= 0) ? ld16(src + (int64_t)rows[q] * a.ld_src) : zero4();
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        h[u][nb] = tok ? ld16(hT + (int64_t)(16 * nb + li) * a.ldh + (ci.tile0 + t) * kTileRows) : zero4();
-    }
-#pragma unroll
-    for (int u = 0; u < TB; ++u) {
-      // 8x8 transpose inside the lane: tr[q] holds column q of the 8 rows
-      uint4 tr[8];
-#pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        const int d = q >> 1;
-        const uint32_t sel = (q & 1) ? 0x07060302u : 0x05040100u;
-        uint32_t e[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const uint32_t wsrc[4] = {x[u][i].x, x[u][i].y, x[u][i].z, x[u][i].w};
-          e[i] = wsrc[d];
-        }
-        tr[q].x = __builtin_amdgcn_perm(e[1], e[0], sel);
-        tr[q].y = __builtin_amdgcn_perm(e[3], e[2], sel);
-        tr[q].z = __builtin_amdgcn_perm(e[5], e[4], sel);
-        tr[q].w = __builtin_amdgcn_perm(e[7], e[6], sel);
-      }
-#pragma unroll
-      for (int q = 0; q < 8; ++q)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) acc[q][nb] = mfma16(tr[q], h[u][nb], acc[q][nb]);
-    }
-  }
-
-  // add the waves' accumulators in wave order; wave 0 writes the result
-  if (NW > 1) {
-    if (wave > 0) {
-#pragma unroll
-      for (int q = 0; q < 8; ++q)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int v = 0; v < 4; ++v) red[wave - 1][(q * NB + nb) * 4 + v][lane] = acc[q][nb][v];
-    }
-    __syncthreads();
-    if (wave > 0) return;
-    for (int w = 0; w < NW - 1; ++w)
-#pragma unroll
-      for (int q = 0; q < 8; ++q)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int v = 0; v < 4; ++v) acc[q][nb][v] += red[w][(q * NB + nb) * 4 + v][lane];
-  }
-
-  // lane holds out[n = 16 nb + li][c0 + 32 kb + 8 v + q], q = 0..7, v = 0..3: 32 consecutive columns per n
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    const int n = 16 * nb + li;
-    if (n >= r) continue;
-    const int cb = c0 + 32 * kb;
-    if (ci.partial >= 0) {
-      float* o = a.partial + ((int64_t)ci.partial * a.rpad + n) * a.width + cb;
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        *reinterpret_cast<float4*>(o + 8 * v) = make_float4(acc[0][nb][v], acc[1][nb][v], acc[2][nb][v], acc[3][nb][v]);
-        *reinterpret_cast<float4*>(o + 8 * v + 4) =
-            make_float4(acc[4][nb][v], acc[5][nb][v], acc[6][nb][v], acc[7][nb][v]);
-      }
-    } else {
-      bf16_t* gp = (bf16_t*)a.grad[g];
-#pragma unroll
-      for (int v = 0; v < 4; ++v)
-#pragma unroll
-        for (int q = 0; q < 8; ++q) {
-          const int c = cb + 8 * v + q;
-          bf16_t* o = a.transposed ? gp + (int64_t)c * a.ld_grad + n : gp + (int64_t)n * a.ld_grad + c;
-          float val = acc[q][nb][v];
-          if (a.accumulate) val += to_f32(*o);
-          *o = (bf16_t)(pack_bf16(val, 0.f) & 0xffffu);
-        }
-    }
-  }
-}
-
 // Eight consecutive bf16 results: one 16-byte store when `vec`, element stores otherwise; `keep` (1..8)
 // elements are written, the rest of the destination is left alone.
 __device__ inline void store_bf16x8(bf16_t* o, const float (&v)[8], int keep, bool accumulate, bool vec) {
@@ -488,6 +370,40 @@ __device__ inline void store_bf16x8(bf16_t* o, const float (&v)[8], int keep, bo
     float val = v[i];
     if (accumulate) val += to_f32(o[i]);
     o[i] = (bf16_t)(pack_bf16(val, 0.f) & 0xffffu);
+  }
+}
+
+// Transposed weight copies (see TransposeJob): a thread writes 8 consecutive outputs with one 16-byte
+// store and gathers them with 8 element loads (the weights are L2 resident and small).
+__device__ inline void transpose_weights_job(const TransposeJob& t, const int32_t* __restrict__ rank, int rpad,
+                                             int64_t thread, int64_t threads) {
+  const int m8 = t.out_features >> 3, n8 = rpad >> 3;
+  const int64_t units_b = (int64_t)t.groups * m8 * rpad;           // (g, m-octet, n), n fastest
+  const int64_t units_a = (int64_t)t.groups * n8 * t.in_features;  // (g, n-octet, k), k fastest
+  for (int64_t u = thread; u < units_b + units_a; u += threads) {
+    uint32_t e[8];
+    bf16_t* out;
+    if (u < units_b) {
+      const int n = (int)(u % rpad);
+      const int64_t q = u / rpad;
+      const int mo = (int)(q % m8), g = (int)(q / m8);
+      const bf16_t* B = (const bf16_t*)t.lora_B[g] + (int64_t)(8 * mo) * t.ldb + n;
+      const bool live = n < rank[g];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) e[i] = live ? B[(int64_t)i * t.ldb] : 0;
+      out = (bf16_t*)t.bT + ((int64_t)g * rpad + n) * t.out_features + 8 * mo;
+    } else {
+      const int64_t v = u - units_b;
+      const int k = (int)(v % t.in_features);
+      const int64_t q = v / t.in_features;
+      const int no = (int)(q % n8), g = (int)(q / n8);
+      const bf16_t* A = (const bf16_t*)t.lora_A[g] + (int64_t)(8 * no) * t.lda + k;
+      const int r = rank[g];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) e[i] = 8 * no + i < r ? A[(int64_t)i * t.lda] : 0;
+      out = (bf16_t*)t.aT + ((int64_t)g * t.in_features + k) * rpad + 8 * no;
+    }
+    st16(out, make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)));
   }
 }
 
@@ -514,9 +430,14 @@ __global__ __launch_bounds__(NW * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
   constexpr int OUT = RP * OS;
   __shared__ __attribute__((aligned(16))) float lds[RED > OUT ? RED : OUT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  if ((int)blockIdx.y < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
+    transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (NW * 64) + tid,
+                          (int64_t)a.tr.y_blocks * gridDim.x * (NW * 64));
+    return;
+  }
   // column block fastest: blocks that run together read neighbouring pieces of the same rows
   const int c0 = blockIdx.x * 128;
-  const ChunkInfo ci = chunks[blockIdx.y];
+  const ChunkInfo ci = chunks[blockIdx.y - a.tr.y_blocks];
   const int g = ci.group;
   if (g < 0) return;
   const int r = min(a.rank[g], RP);
@@ -677,15 +598,15 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
                      seg.tile_group, rows, (int)items);
 }
 
-template <int NB, int NW, int TB>
-void launch_wgrad(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
-  const dim3 grid((unsigned)(a.width / 128), (unsigned)L.max_chunks);
-  hipLaunchKernelGGL((k_wgrad_mfma<NB, NW, TB>), grid, dim3(NW * 64), 0, s, a, seg.chunks, seg.slot_table(a.map_rows));
-}
-
 template <int NB, int NW, int DEPTH>
-void launch_wgrad_pipe(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
-  const dim3 grid((unsigned)(a.width / 128), (unsigned)L.max_chunks);
+void launch_wgrad_pipe(const WgradArgs& a0, const SegView& seg, const SegLayout& L, hipStream_t s) {
+  WgradArgs a = a0;
+  a.tr.y_blocks = 0;
+  if (a.tr.aT) {  // about four 16-byte outputs per thread of the side job
+    const int64_t units = (int64_t)a.tr.groups * a.rpad * ((a.tr.out_features + a.tr.in_features) / 8);
+    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 128) * (NW * 64))));
+  }
+  const dim3 grid((unsigned)(a.width / 128), (unsigned)(L.max_chunks + a.tr.y_blocks));
   hipLaunchKernelGGL((k_wgrad_pipe<NB, NW, DEPTH>), grid, dim3(NW * 64), 0, s, a, seg.chunks, seg.slot_table(a.map_rows));
 }
 

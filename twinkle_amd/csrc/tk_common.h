@@ -185,6 +185,18 @@ struct PassArgs {
   int32_t kslices;       // blocks per tile of the MFMA shrink
 };
 
+// Optional side job of a weight-gradient launch (bf16 MFMA path): the first `y_blocks` rows of the
+// grid write the transposed weight copies the input-gradient pass reads, bT_g[n][m] = B_g[m][n] and
+// aT_g[k][n] = A_g[n][k] (zero for n >= rank[g]), instead of spending a launch of their own on them.
+struct TransposeJob {
+  const void* const* lora_A;  int64_t lda;
+  const void* const* lora_B;  int64_t ldb;
+  void* aT;  // [groups][in_features][rpad]
+  void* bT;  // [groups][rpad][out_features]
+  int32_t in_features, out_features, groups;
+  int32_t y_blocks;  // 0: no job
+};
+
 // Row-contraction (weight gradient) pass: out_g[n][c] = sum_p hT[n][p] * src[row(p)][c].
 struct WgradArgs {
   const void* src;  int64_t ld_src;   // x | dy
@@ -198,6 +210,7 @@ struct WgradArgs {
   int32_t accumulate;
   int32_t map_rows;
   int32_t rpad;
+  TransposeJob tr;
 };
 
 // kernels_segments.hip
@@ -225,6 +238,7 @@ bool pass_mfma_supported(const PassArgs& a);
 // `phases`: 1 = shrink only, 2 = expand only (h already written), 3 = both
 int launch_pass_mfma(const PassArgs& a, const SegView& seg, const SegLayout& L, int phases, hipStream_t s);
 bool wgrad_mfma_supported(const WgradArgs& a);
+// a.tr.y_blocks is chosen by the launcher when a.tr.aT is set
 int launch_wgrad_mfma(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
 
 }  // namespace tk
