@@ -176,38 +176,71 @@ __global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkI
 }
 
 // Groups with several chunks: sum their partials in chunk order.  Groups with
-// no rows: clear the live block when overwriting.  One (group, rank index,
-// 256 columns) per block; blockIdx.z >= rpad selects the second argument set,
+// no rows: clear the live block when overwriting.  One (group, 8 rank
+// indices, 256 columns) per block, a thread owns one column of the eight, so
+// that a transposed gradient ([width][r], dB) leaves as 16-byte pieces instead
+// of single elements; blockIdx.z >= rpad / 8 selects the second argument set,
 // so that the reductions of dA and dB share one launch.
 template <typename T>
 __global__ __launch_bounds__(256) void k_wgrad_reduce(WgradArgs a0, WgradArgs a1, int rpad,
                                                       const int32_t* __restrict__ chunk_first,
                                                       const int32_t* __restrict__ partial_first) {
-  const bool second = (int)blockIdx.z >= rpad;
+  const int zsets = rpad >> 3;
+  const bool second = (int)blockIdx.z >= zsets;
   const WgradArgs& a = second ? a1 : a0;
   if (a.grad == nullptr) return;
   const int g = blockIdx.x;
-  const int n = second ? blockIdx.z - rpad : blockIdx.z;
+  const int n0 = 8 * (second ? blockIdx.z - zsets : blockIdx.z);
   // independent loads first
   const int rk = a.rank[g], cf0 = chunk_first[g], cf1 = chunk_first[g + 1], pf = partial_first[g];
-  if (n >= min(rk, a.rpad)) return;
+  const int r = min(rk, a.rpad);
+  if (n0 >= r) return;
   const int nchunk = cf1 - cf0;
   if (nchunk == 1) return;
   if (nchunk == 0 && a.accumulate) return;
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= a.width) return;
-  const float* p = a.partial + ((int64_t)pf * a.rpad + n) * a.width + c;
+  const float* p = a.partial + ((int64_t)pf * a.rpad + n0) * a.width + c;
   const int64_t stride = (int64_t)a.rpad * a.width;
-  float acc = 0.f;
-  // eight chunks are requested together (their latencies overlap) and added in chunk order
-  for (int j0 = 0; j0 < nchunk; j0 += 8) {
-    float v[8];
+  float acc[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = j0 + j < nchunk ? p[(j0 + j) * stride] : 0.f;
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  // two chunks (16 loads) are requested together; every sum adds its chunks in chunk order
+  for (int j0 = 0; j0 < nchunk; j0 += 2) {
+    float v[2][8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc += v[j];
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        v[j][i] = (j0 + j < nchunk && n0 + i < r) ? p[(j0 + j) * stride + (int64_t)i * a.width] : 0.f;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] += v[j][i];
   }
-  store_grad<T>(a, g, n, c, acc);
+  T* gp = (T*)a.grad[g];
+  if (sizeof(T) == 2 && a.transposed && n0 + 8 <= r && (a.ld_grad & 7) == 0 &&
+      (reinterpret_cast<uintptr_t>(gp) & 15u) == 0) {
+    uint4* o = reinterpret_cast<uint4*>(gp + (int64_t)c * a.ld_grad + n0);
+    if (a.accumulate) {
+      const uint4 old = *o;
+      const uint32_t w[4] = {old.x, old.y, old.z, old.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[2 * i] += __uint_as_float(w[i] << 16);
+        acc[2 * i + 1] += __uint_as_float(w[i] & 0xffff0000u);
+      }
+    }
+    uint16_t h[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) from_f32(acc[i], &h[i]);
+    *o = make_uint4(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16), h[4] | ((uint32_t)h[5] << 16),
+                    h[6] | ((uint32_t)h[7] << 16));
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    if (n0 + i < r) store_grad<T>(a, g, n0 + i, c, acc[i]);
 }
 
 // bT_g[n][m] = B_g[m][n], aT_g[k][n] = A_g[n][k]; zero for n >= rank[g].
@@ -272,7 +305,7 @@ int launch_wgrad_reduce(const WgradArgs* a0, const WgradArgs* a1, const SegView&
   const WgradArgs& x1 = a1 ? *a1 : none;
   const int rpad = a0 ? a0->rpad : a1->rpad;
   const int width = std::max(a0 ? a0->width : 0, a1 ? a1->width : 0);
-  const dim3 grid((unsigned)L.groups, (unsigned)ceil_div(width, 256), (unsigned)(a1 ? 2 * rpad : rpad));
+  const dim3 grid((unsigned)L.groups, (unsigned)ceil_div(width, 256), (unsigned)(a1 ? 2 * (rpad / 8) : rpad / 8));
   if (dtype == TK_DTYPE_F32)
     hipLaunchKernelGGL(k_wgrad_reduce<float>, grid, dim3(256), 0, s, x0, x1, rpad, seg.chunk_first, seg.partial_first);
   else
