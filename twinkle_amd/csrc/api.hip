@@ -1,6 +1,8 @@
 // C ABI of the library: argument checks, workspace carving, kernel choice.
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "tk_common.h"
 
 using namespace tk;
@@ -27,6 +29,40 @@ bool force_generic() {
     return e && e[0] == '1';
   }();
   return v;
+}
+
+// The backward pass has two independent chains that meet only at the end (dB needs dy and h; dX and
+// dA need the dy shrink), and no single kernel of either reaches the memory system's peak, so the
+// library runs them on two streams: the caller's and one of its own per device (default priority,
+// non-blocking), forked and joined with events.  TK_BWD_STREAMS=0 keeps everything on the caller's stream.
+struct SideStream {
+  hipStream_t stream = nullptr;
+  hipEvent_t fork = nullptr, mid = nullptr, join = nullptr;
+  int state = 0;  // 0: not created yet, 1: ready, -1: creation failed (single-stream fallback)
+};
+
+SideStream* side_stream() {
+  static const bool enabled = [] {
+    const char* e = getenv("TK_BWD_STREAMS");
+    return !(e && e[0] == '0');
+  }();
+  if (!enabled) return nullptr;
+  constexpr int kMaxDevices = 64;
+  static SideStream side[kMaxDevices];
+  static std::mutex mu;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  SideStream& x = side[dev];
+  if (x.state == 0) {
+    const bool ok = hipStreamCreateWithFlags(&x.stream, hipStreamNonBlocking) == hipSuccess &&
+                    hipEventCreateWithFlags(&x.fork, hipEventDisableTiming) == hipSuccess &&
+                    hipEventCreateWithFlags(&x.mid, hipEventDisableTiming) == hipSuccess &&
+                    hipEventCreateWithFlags(&x.join, hipEventDisableTiming) == hipSuccess;
+    x.state = ok ? 1 : -1;
+    if (!ok) (void)hipGetLastError();
+  }
+  return x.state == 1 ? &x : nullptr;
 }
 
 int run_pass(const PassArgs& a, const SegView& V, const SegLayout& L, int dtype, int phases, hipStream_t s) {
@@ -189,61 +225,93 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
   char* w = (char*)ws;
   void* dh = w + B.off_dh;
   int rc;
-  WgradArgs ga{}, gb{};
   const bool need_wT = dx || grad_A;
   void* bT = w + B.off_wT_shrink;
   void* aT = w + B.off_wT_expand;
+  WgradArgs ga{}, gb{};
+  if (grad_B) {  // dB[m][n] = sum_rows dy[row][m] * h[row][n]
+    gb.src = dy;  gb.ld_src = lddy;
+    gb.hT = h;    gb.ldh = B.ldh;
+    gb.partial = (float*)(w + B.off_part_b);
+    gb.grad = grad_B;  gb.ld_grad = d->ldb;
+    gb.rank = d->rank;  gb.width = d->out_features;  gb.transposed = 1;
+    gb.accumulate = accumulate;  gb.map_rows = d->map_rows;  gb.rpad = (int32_t)B.rpad;
+  }
+  if (grad_A) {  // dA[n][k] = sum_rows dh[row][n] * x[row][k]
+    ga.src = x;  ga.ld_src = ldx;
+    ga.hT = dh;  ga.ldh = B.ldh;
+    ga.partial = (float*)(w + B.off_part_a);
+    ga.grad = grad_A;  ga.ld_grad = d->lda;
+    ga.rank = d->rank;  ga.width = d->in_features;  ga.transposed = 0;
+    ga.accumulate = accumulate;  ga.map_rows = d->map_rows;  ga.rpad = (int32_t)B.rpad;
+  }
+  PassArgs a{};  // dh = scale * dy B, dx += dh A
+  a.src = dy;  a.ld_src = lddy;
+  a.dst = dx;  a.ld_dst = lddx;
+  a.hT = dh;   a.ldh = B.ldh;
+  a.w_shrink_base = bT;  a.ld_shrink = d->out_features;  a.shrink_group_stride = B.rpad * d->out_features;
+  a.w_expand_base = aT;  a.ld_expand = B.rpad;           a.expand_group_stride = B.rpad * d->in_features;
+  a.rank = d->rank;  a.scale = d->scale;
+  a.width_src = d->out_features;  a.width_dst = d->in_features;
+  a.map_rows = d->map_rows;  a.rpad = (int32_t)B.rpad;  a.src_rows = (int32_t)d->rows;
+  a.hpart = (float*)(w + B.off_hpart);
+  a.tile_ticket = V.tile_ticket;
+  a.kslices = shrink_kslices(d->out_features, a.rpad);
+  const bool mfma = d->dtype == TK_DTYPE_BF16 && !force_generic();
+  TransposeJob tr{};
+  tr.lora_A = d->lora_A;  tr.lda = d->lda;
+  tr.lora_B = d->lora_B;  tr.ldb = d->ldb;
+  tr.aT = aT;  tr.bT = bT;
+  tr.in_features = d->in_features;  tr.out_features = d->out_features;  tr.groups = d->num_groups;
+
+  if (grad_B && need_wT && mfma && pass_mfma_supported(a) && dy_fused_supported(gb, a.kslices)) {
+    // One pass over dy yields dB and the slices of dh (and, on the side, the A^T copy for dX).
+    gb.tr = tr;
+    gb.tr.bT = nullptr;
+    rc = launch_dy_fused(gb, d->lora_B, d->ldb, a.hpart, a.kslices, V, L, s);
+    gb.tr = TransposeJob{};
+    if (rc != TK_OK) return rc;
+    if ((rc = launch_pass_mfma(a, V, L, dx ? 4 | 2 : 4, s)) != TK_OK) return rc;
+    if (grad_A && (rc = run_wgrad(ga, V, L, d->dtype, s)) != TK_OK) return rc;
+    return launch_wgrad_reduce(grad_A ? &ga : nullptr, &gb, V, L, d->dtype, s);
+  }
+
+  // Separate kernels.  Two chains that meet only at the end: dB (reads dy and h) runs on a side stream,
+  // the dy shrink -> dX on the caller's; dA follows the shrink on the side stream, next to the expand.
+  // Without a side stream everything runs in the same order on the caller's stream.
+  SideStream* side = (grad_B && need_wT) ? side_stream() : nullptr;
+  hipStream_t s2 = side ? side->stream : s;
+  if (side) {
+    if (hipEventRecord(side->fork, s) != hipSuccess || hipStreamWaitEvent(s2, side->fork, 0) != hipSuccess)
+      return TK_ERR_LAUNCH;
+  }
   bool wT_done = false;
-  // dB first: the two passes over dy (this one and the shrink below) run back to back, so the second
-  // one is served from the 256 MB last-level cache instead of HBM
   if (grad_B) {
-    WgradArgs& g = gb;
-    g.src = dy;  g.ld_src = lddy;
-    g.hT = h;    g.ldh = B.ldh;
-    g.partial = (float*)(w + B.off_part_b);
-    g.grad = grad_B;  g.ld_grad = d->ldb;
-    g.rank = d->rank;  g.width = d->out_features;  g.transposed = 1;
-    g.accumulate = accumulate;  g.map_rows = d->map_rows;  g.rpad = (int32_t)B.rpad;
-    if (need_wT && d->dtype == TK_DTYPE_BF16 && !force_generic() && wgrad_mfma_supported(g) &&
-        d->out_features % 8 == 0) {
-      // the MFMA launch also writes the transposed weight copies of the pass below
-      g.tr.lora_A = d->lora_A;  g.tr.lda = d->lda;
-      g.tr.lora_B = d->lora_B;  g.tr.ldb = d->ldb;
-      g.tr.aT = aT;  g.tr.bT = bT;
-      g.tr.in_features = d->in_features;  g.tr.out_features = d->out_features;  g.tr.groups = d->num_groups;
+    if (!side && need_wT && mfma && wgrad_mfma_supported(gb) && d->out_features % 8 == 0) {
+      gb.tr = tr;  // one stream: the MFMA launch also writes the transposed weight copies of the pass below
       wT_done = true;
     }
-    if ((rc = run_wgrad(g, V, L, d->dtype, s)) != TK_OK) return rc;
-    g.tr = TransposeJob{};
+    rc = run_wgrad(gb, V, L, d->dtype, s2);
+    gb.tr = TransposeJob{};
+    if (rc != TK_OK) return rc;
   }
   if (need_wT) {
     if (!wT_done && (rc = launch_transpose_weights(*d, bT, aT, s)) != TK_OK) return rc;
-    PassArgs a{};
-    a.src = dy;  a.ld_src = lddy;
-    a.dst = dx;  a.ld_dst = lddx;
-    a.hT = dh;   a.ldh = B.ldh;
-    a.w_shrink_base = bT;  a.ld_shrink = d->out_features;  a.shrink_group_stride = B.rpad * d->out_features;
-    a.w_expand_base = aT;  a.ld_expand = B.rpad;           a.expand_group_stride = B.rpad * d->in_features;
-    a.rank = d->rank;  a.scale = d->scale;
-    a.width_src = d->out_features;  a.width_dst = d->in_features;
-    a.map_rows = d->map_rows;  a.rpad = (int32_t)B.rpad;  a.src_rows = (int32_t)d->rows;
-    a.hpart = (float*)(w + B.off_hpart);
-    a.tile_ticket = V.tile_ticket;
-    a.kslices = shrink_kslices(d->out_features, a.rpad);
-    if ((rc = run_pass(a, V, L, d->dtype, 3, s)) != TK_OK) return rc;
+    if ((rc = run_pass(a, V, L, d->dtype, 1, s)) != TK_OK) return rc;
+    if (side && grad_A) {  // dh is complete: the side stream may start dA while dX runs here
+      if (hipEventRecord(side->mid, s) != hipSuccess || hipStreamWaitEvent(s2, side->mid, 0) != hipSuccess)
+        return TK_ERR_LAUNCH;
+    }
+    if (dx && (rc = run_pass(a, V, L, d->dtype, 2, s)) != TK_OK) return rc;
   }
-  if (grad_A) {
-    WgradArgs& g = ga;
-    g.src = x;  g.ld_src = ldx;
-    g.hT = dh;  g.ldh = B.ldh;
-    g.partial = (float*)(w + B.off_part_a);
-    g.grad = grad_A;  g.ld_grad = d->lda;
-    g.rank = d->rank;  g.width = d->in_features;  g.transposed = 0;
-    g.accumulate = accumulate;  g.map_rows = d->map_rows;  g.rpad = (int32_t)B.rpad;
-    if ((rc = run_wgrad(g, V, L, d->dtype, s)) != TK_OK) return rc;
-  }
+  if (grad_A && (rc = run_wgrad(ga, V, L, d->dtype, s2)) != TK_OK) return rc;
   // the chunk partials of both contractions are summed by one launch
-  return launch_wgrad_reduce(grad_A ? &ga : nullptr, grad_B ? &gb : nullptr, V, L, d->dtype, s);
+  rc = launch_wgrad_reduce(grad_A ? &ga : nullptr, grad_B ? &gb : nullptr, V, L, d->dtype, s2);
+  if (side) {
+    if (hipEventRecord(side->join, s2) != hipSuccess || hipStreamWaitEvent(s, side->join, 0) != hipSuccess)
+      return TK_ERR_LAUNCH;
+  }
+  return rc;
 }
 
 }  // extern "C"

@@ -42,6 +42,14 @@ __device__ inline uint32_t pack_bf16(float lo, float hi) {
 __device__ inline float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
 __device__ inline float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 
+// Block barrier that orders LDS traffic only: unlike __syncthreads() it does not wait for the global
+// loads a wave has in flight, so software-pipelined loads stay outstanding across it.
+__device__ inline void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 // keep the first `keep` (0..8) bf16 elements of a quad, zero the rest
 __device__ inline uint4 keep_first(uint4 v, int keep) {
   if (keep >= 8) return v;
@@ -373,12 +381,71 @@ __device__ inline void store_bf16x8(bf16_t* o, const float (&v)[8], int keep, bo
   }
 }
 
+// One wave's weight-gradient block out[n][c0 .. c0 + 127] (lane holds out[16 nb + li][32 kb + 8 v + q] in
+// acc[q][nb][v]) leaves through `lds` (RP rows of kWgradStageStride floats, private to the wave) as whole
+// 512-byte rows: into the chunk's slot of the partial buffer, or straight into the gradient when the
+// chunk is its group's only one.
+constexpr int kWgradStageStride = 132;  // 4 mod 32: conflict-free 16-byte accesses
+template <int NB>
+__device__ inline void wgrad_store(const f32x4 (&acc)[8][NB], float* lds, const WgradArgs& a, const ChunkInfo& ci,
+                                   int g, int r, int c0, int lane) {
+  constexpr int RP = 16 * NB, OS = kWgradStageStride;
+  const int li = lane & 15, kb = lane >> 4;
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      float* o = lds + (16 * nb + li) * OS + 32 * kb + 8 * v;
+      *reinterpret_cast<float4*>(o) = make_float4(acc[0][nb][v], acc[1][nb][v], acc[2][nb][v], acc[3][nb][v]);
+      *reinterpret_cast<float4*>(o + 4) = make_float4(acc[4][nb][v], acc[5][nb][v], acc[6][nb][v], acc[7][nb][v]);
+    }
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+
+  if (ci.partial >= 0) {
+    float* part = a.partial + (int64_t)ci.partial * a.rpad * a.width + c0;
+#pragma unroll
+    for (int i = 0; i < RP / 2; ++i) {
+      const int n = 2 * i + (lane >> 5), c = 4 * (lane & 31);
+      if (n < r) *reinterpret_cast<float4*>(part + (int64_t)n * a.width + c) = *reinterpret_cast<const float4*>(lds + n * OS + c);
+    }
+    return;
+  }
+  bf16_t* gp = (bf16_t*)a.grad[g];
+  const bool vec = (reinterpret_cast<uintptr_t>(gp) & 15u) == 0 && (a.ld_grad & 7) == 0;
+  if (!a.transposed) {
+    // grad[n][c0 + c]: four rows of 128 columns per step
+#pragma unroll
+    for (int i = 0; i < RP / 4; ++i) {
+      const int n = 4 * i + kb, c = 8 * li;
+      if (n >= r) continue;
+      const float4 lo = *reinterpret_cast<const float4*>(lds + n * OS + c);
+      const float4 hi = *reinterpret_cast<const float4*>(lds + n * OS + c + 4);
+      const float v8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+      store_bf16x8(gp + (int64_t)n * a.ld_grad + c0 + c, v8, 8, a.accumulate != 0, vec);
+    }
+  } else {
+    // grad[c0 + c][n]: a lane owns columns c = lane and lane + 64
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int c = lane + 64 * half;
+#pragma unroll
+      for (int n8 = 0; n8 < RP; n8 += 8) {
+        if (n8 >= r) break;
+        float v8[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v8[i] = lds[(n8 + i) * OS + c];
+        store_bf16x8(gp + (int64_t)(c0 + c) * a.ld_grad + n8, v8, min(8, r - n8), a.accumulate != 0, vec);
+      }
+    }
+  }
+}
+
 // Transposed weight copies (see TransposeJob): a thread writes 8 consecutive outputs with one 16-byte
 // store and gathers them with 8 element loads (the weights are L2 resident and small).
 __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_t* __restrict__ rank, int rpad,
                                              int64_t thread, int64_t threads) {
   const int m8 = t.out_features >> 3, n8 = rpad >> 3;
-  const int64_t units_b = (int64_t)t.groups * m8 * rpad;           // (g, m-octet, n), n fastest
+  const int64_t units_b = t.bT ? (int64_t)t.groups * m8 * rpad : 0;  // (g, m-octet, n), n fastest
   const int64_t units_a = (int64_t)t.groups * n8 * t.in_features;  // (g, n-octet, k), k fastest
   for (int64_t u = thread; u < units_b + units_a; u += threads) {
     uint32_t e[8];
@@ -425,7 +492,7 @@ __global__ __launch_bounds__(NW * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
                                                         const int32_t* __restrict__ slot_rows) {
   constexpr int TPW = kChunkTiles / NW;  // tiles per wave
   constexpr int RP = 16 * NB;
-  constexpr int OS = 132;  // row stride of the staged result in floats (4 mod 32: conflict-free 16-byte accesses)
+  constexpr int OS = kWgradStageStride;
   constexpr int RED = (NW - 1) * 32 * NB * 64;
   constexpr int OUT = RP * OS;
   __shared__ __attribute__((aligned(16))) float lds[RED > OUT ? RED : OUT];
@@ -527,54 +594,137 @@ __global__ __launch_bounds__(NW * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");  // the sums are read before the staging below overwrites them
   }
 
-  // lane holds out[n = 16 nb + li][32 kb + 8 v + q]; stage it as out[n][0..127]
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      float* o = lds + (16 * nb + li) * OS + 32 * kb + 8 * v;
-      *reinterpret_cast<float4*>(o) = make_float4(acc[0][nb][v], acc[1][nb][v], acc[2][nb][v], acc[3][nb][v]);
-      *reinterpret_cast<float4*>(o + 4) = make_float4(acc[4][nb][v], acc[5][nb][v], acc[6][nb][v], acc[7][nb][v]);
-    }
-  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+  wgrad_store<NB>(acc, lds, a, ci, g, r, c0, lane);
+}
 
-  if (ci.partial >= 0) {
-    float* part = a.partial + (int64_t)ci.partial * a.rpad * a.width + c0;
-#pragma unroll
-    for (int i = 0; i < RP / 2; ++i) {
-      const int n = 2 * i + (lane >> 5), c = 4 * (lane & 31);
-      if (n < r) *reinterpret_cast<float4*>(part + (int64_t)n * a.width + c) = *reinterpret_cast<const float4*>(lds + n * OS + c);
-    }
+// ---------------------------------------------------------------------------
+// Backward, both uses of dy in one pass (rank <= 16, width a multiple of 512): a block of four waves owns
+// (chunk of up to 16 tiles of one group, 512 columns), wave w the columns [128 w, 128 w + 128) of it.
+// Per tile a wave loads its 32 x 128 piece once, in the weight-gradient layout (a lane holds 8 rows x 8
+// columns), and uses it twice:
+//   dB:  the piece, transposed in registers, is the MFMA A operand with the rows as contraction index,
+//        accumulated over the chunk's tiles exactly like k_wgrad_pipe does;
+//   dh:  the piece goes through a per-wave LDS buffer to come back in the row-major operand layout and
+//        is multiplied with the wave's 128 x rank block of B (loaded once per chunk, straight from the
+//        adapter's [out][r] layout); the four waves' partial dh[32][rank] meet in LDS after a block
+//        barrier and one of them writes the sum as slice `blockIdx.x` of the split-shrink buffer, which
+//        k_shrink_finish turns into dh like after a separate shrink.
+// dy crosses the memory system once instead of twice.  Sums are formed in a fixed order.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void k_dy_fused(WgradArgs a, const void* const* __restrict__ lora_B, int64_t ldb,
+                                                  float* __restrict__ hpart, int kslices,
+                                                  const ChunkInfo* __restrict__ chunks,
+                                                  const int32_t* __restrict__ slot_rows) {
+  constexpr int SS = 136;  // row stride of the staged piece in bf16 (272 B)
+  constexpr int PR = 17;   // row stride of the partial dh in floats
+  __shared__ int32_t rows_s[kChunkRows];
+  __shared__ __attribute__((aligned(16))) bf16_t stage[4][kTileRows * SS];
+  __shared__ float part[2][4][kTileRows * PR];
+  static_assert(sizeof(bf16_t) * kTileRows * SS >= sizeof(float) * 16 * kWgradStageStride, "stage holds the dB block too");
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  if ((int)blockIdx.y < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
+    transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + tid,
+                          (int64_t)a.tr.y_blocks * gridDim.x * 256);
     return;
   }
-  bf16_t* gp = (bf16_t*)a.grad[g];
-  const bool vec = (reinterpret_cast<uintptr_t>(gp) & 15u) == 0 && (a.ld_grad & 7) == 0;
-  if (!a.transposed) {
-    // grad[n][c0 + c]: four rows of 128 columns per step
+  const ChunkInfo ci = chunks[blockIdx.y - a.tr.y_blocks];
+  const int g = ci.group;
+  if (g < 0) return;
+  const int r = min(a.rank[g], 16);
+  if (r <= 0) return;
+  const int slab = blockIdx.x;
+  const int c0 = slab * 512 + wave * 128;
+  const int nt = ci.ntiles;
+  for (int i = tid; i < nt * kTileRows; i += 256) rows_s[i] = slot_rows[ci.tile0 * kTileRows + i];
+  // this wave's block of B as MFMA B operand: lane (n = li, kb) holds B[c0 + 32 s + 8 kb + i][n], i = 0..7
+  uint4 wB[4];
+  {
+    const bf16_t* Bg = (const bf16_t*)lora_B[g] + (int64_t)(c0 + 8 * kb) * ldb + li;
 #pragma unroll
-    for (int i = 0; i < RP / 4; ++i) {
-      const int n = 4 * i + kb, c = 8 * li;
-      if (n >= r) continue;
-      const float4 lo = *reinterpret_cast<const float4*>(lds + n * OS + c);
-      const float4 hi = *reinterpret_cast<const float4*>(lds + n * OS + c + 4);
-      const float v8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-      store_bf16x8(gp + (int64_t)n * a.ld_grad + c0 + c, v8, 8, a.accumulate != 0, vec);
-    }
-  } else {
-    // grad[c0 + c][n]: a lane owns columns c = lane and lane + 64
+    for (int s4 = 0; s4 < 4; ++s4) {
+      uint32_t e[8];
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      const int c = lane + 64 * half;
-#pragma unroll
-      for (int n8 = 0; n8 < RP; n8 += 8) {
-        if (n8 >= r) break;
-        float v8[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v8[i] = lds[(n8 + i) * OS + c];
-        store_bf16x8(gp + (int64_t)(c0 + c) * a.ld_grad + n8, v8, min(8, r - n8), a.accumulate != 0, vec);
-      }
+      for (int i = 0; i < 8; ++i) e[i] = li < r ? Bg[(int64_t)(32 * s4 + i) * ldb] : 0;
+      wB[s4] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
     }
   }
+  __syncthreads();
+
+  const bf16_t* src = (const bf16_t*)a.src + c0 + 8 * li;
+  const bf16_t* hT = (const bf16_t*)a.hT + (int64_t)li * a.ldh + (int64_t)ci.tile0 * kTileRows + 8 * kb;
+  bf16_t* my_stage = stage[wave];
+  f32x4 acc[8][1];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) acc[q][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  auto issue = [&](int t, uint4 (&x)[8], uint4& h) {
+    const bool tok = t < nt;  // block-uniform
+    const int4 ra = tok ? *reinterpret_cast<const int4*>(rows_s + t * kTileRows + 8 * kb) : make_int4(-1, -1, -1, -1);
+    const int4 rb = tok ? *reinterpret_cast<const int4*>(rows_s + t * kTileRows + 8 * kb + 4) : make_int4(-1, -1, -1, -1);
+    const int rows[8] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w};
+#pragma unroll
+    for (int q = 0; q < 8; ++q) x[q] = rows[q] >= 0 ? ld16(src + (int64_t)rows[q] * a.ld_src) : zero4();
+    h = tok ? ld16(hT + t * kTileRows) : zero4();
+  };
+  auto consume = [&](int t, const uint4 (&x)[8], const uint4& h) {
+    // the piece in row-major order for the dh product
+#pragma unroll
+    for (int q = 0; q < 8; ++q) st16(my_stage + (8 * kb + q) * SS + 8 * li, x[q]);
+    // dB: 8x8 transpose inside the lane, rows become the contraction index
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int d = q >> 1;
+      const uint32_t sel = (q & 1) ? 0x07060302u : 0x05040100u;
+      uint32_t e[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t wsrc[4] = {x[i].x, x[i].y, x[i].z, x[i].w};
+        e[i] = wsrc[d];
+      }
+      uint4 tr;
+      tr.x = __builtin_amdgcn_perm(e[1], e[0], sel);
+      tr.y = __builtin_amdgcn_perm(e[3], e[2], sel);
+      tr.z = __builtin_amdgcn_perm(e[5], e[4], sel);
+      tr.w = __builtin_amdgcn_perm(e[7], e[6], sel);
+      acc[q][0] = mfma16(tr, h, acc[q][0]);
+    }
+    // dh: partial over this wave's 128 columns (LDS operations of one wave complete in order)
+    float* mine = part[t & 1][wave];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      f32x4 d = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s4 = 0; s4 < 4; ++s4) d = mfma16(ld16(my_stage + (16 * tt + li) * SS + 32 * s4 + 8 * kb), wB[s4], d);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) mine[(16 * tt + 4 * kb + v) * PR + li] = d[v];
+    }
+    lds_barrier();
+    if (wave == (t & 3)) {
+      float* o = hpart + ((int64_t)(ci.tile0 + t) * kslices + slab) * (kTileRows * 16);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int idx = lane + 64 * i, row = idx >> 4, n = idx & 15;
+        float sum = part[t & 1][0][row * PR + n];
+        sum += part[t & 1][1][row * PR + n];
+        sum += part[t & 1][2][row * PR + n];
+        sum += part[t & 1][3][row * PR + n];
+        o[idx] = sum;
+      }
+    }
+  };
+
+  uint4 xa[8], xb[8], ha, hb;
+  issue(0, xa, ha);
+  for (int t = 0; t < nt; t += 2) {
+    issue(t + 1, xb, hb);
+    consume(t, xa, ha);
+    if (t + 1 < nt) {
+      issue(t + 2, xa, ha);
+      consume(t + 1, xb, hb);
+    }
+  }
+  // every wave has its own 128 columns of dB
+  wgrad_store<1>(acc, reinterpret_cast<float*>(my_stage), a, ci, g, r, c0, lane);
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -584,13 +734,12 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
   bf16_t* hrow = (bf16_t*)a.hT + (int64_t)a.rpad * a.ldh;  // second half of the h buffer
   const int32_t* rows = seg.slot_table(a.map_rows);
   constexpr int NW = NB == 1 ? 1 : (NB == 2 ? 2 : 4);  // shrink_waves(16 * NB)
-  if (phases & 1) {
+  if (phases & 1)
     hipLaunchKernelGGL((k_shrink_mfma<NB, NW>), dim3((unsigned)(L.max_tiles * a.kslices)), dim3(NW * 64), 0, s, a,
                        hrow, seg.tile_group, rows);
-    if (a.kslices > 1)
-      hipLaunchKernelGGL((k_shrink_finish<NB>), dim3((unsigned)L.max_tiles), dim3(256), 0, s, a, hrow,
-                         seg.tile_group, rows);
-  }
+  if ((phases & 5) && a.kslices > 1)
+    hipLaunchKernelGGL((k_shrink_finish<NB>), dim3((unsigned)L.max_tiles), dim3(256), 0, s, a, hrow, seg.tile_group,
+                       rows);
   if (!a.dst || !(phases & 2)) return;
   const int64_t ngroups = a.width_dst >> 7;
   const int64_t items = L.max_tiles * ceil_div(ngroups, CPW);
@@ -611,6 +760,25 @@ void launch_wgrad_pipe(const WgradArgs& a0, const SegView& seg, const SegLayout&
 }
 
 }  // namespace
+
+bool dy_fused_supported(const WgradArgs& a, int kslices) {
+  return a.rpad == 16 && a.width % 512 == 0 && kslices >= 2 && kslices == a.width / 512 && wgrad_mfma_supported(a);
+}
+
+int launch_dy_fused(const WgradArgs& a0, const void* const* lora_B, int64_t ldb, float* hpart, int kslices,
+                    const SegView& seg, const SegLayout& L, hipStream_t s) {
+  if (L.rows == 0) return TK_OK;
+  WgradArgs a = a0;
+  a.tr.y_blocks = 0;
+  if (a.tr.aT) {
+    const int64_t units = (int64_t)a.tr.groups * a.rpad * ((a.tr.bT ? a.tr.out_features : 0) + a.tr.in_features) / 8;
+    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 512) * 256)));
+  }
+  const dim3 grid((unsigned)(a.width / 512), (unsigned)(L.max_chunks + a.tr.y_blocks));
+  hipLaunchKernelGGL(k_dy_fused, grid, dim3(256), 0, s, a, lora_B, ldb, hpart, kslices, seg.chunks,
+                     seg.slot_table(a.map_rows));
+  return check_launch();
+}
 
 bool pass_mfma_supported(const PassArgs& a) {
   if (a.rpad > 64) return false;

@@ -235,10 +235,15 @@ int launch_transpose_weights(const tk_lora_desc& d, void* bT, void* aT, hipStrea
 
 // kernels_mfma.hip : bf16, aligned shapes, MFMA
 bool pass_mfma_supported(const PassArgs& a);
-// `phases`: 1 = shrink only, 2 = expand only (h already written), 3 = both
+// `phases` (bit mask): 1 = shrink, 2 = expand (h already written), 4 = only the last step of a split shrink
+// (its slices are already in a.hpart)
 int launch_pass_mfma(const PassArgs& a, const SegView& seg, const SegLayout& L, int phases, hipStream_t s);
 bool wgrad_mfma_supported(const WgradArgs& a);
 // a.tr.y_blocks is chosen by the launcher when a.tr.aT is set
 int launch_wgrad_mfma(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
+// dB and the slices of the dy shrink from one pass over dy (a: the dB contraction; a.tr may carry the aT copy)
+bool dy_fused_supported(const WgradArgs& a, int kslices);
+int launch_dy_fused(const WgradArgs& a, const void* const* lora_B, int64_t ldb, float* hpart, int kslices,
+                    const SegView& seg, const SegLayout& L, hipStream_t s);
 
 }  // namespace tk
