@@ -70,6 +70,8 @@ def test_config1_fp32_plumbing(dev):
     (257, 128, 256, 4, 16, [16, 8, 16, 1]),
     (700, 256, 128, 5, 32, [32, 0, 16, 8, 24]),   # a rank-0 (skipped) adapter
     (1500, 384, 640, 6, 64, [64, 8, 16, 32, 64, 4]),
+    (900, 256, 1024, 5, 16, [16, 3, 0, 9, 16]),    # rank <= 16, out width a multiple of 512: one pass over dy
+    (2100, 128, 1536, 4, 8, [8, 8, 1, 5]),         # ... with groups that span several chunks
 ])
 def test_small_shapes(dev, dtype, t, k, m, n, max_r, ranks):
     _run(dev, dtype, *_problem(t, k, m, n, max_r, ranks, seed=t))
