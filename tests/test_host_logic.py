@@ -174,3 +174,23 @@ def test_expert_slots_follow_the_reference_rules():
     a0 = slots._initial_lora_A['lora_0'].clone()
     slots.reset_slot('lora_0')
     assert torch.equal(slots.lora_A['lora_0'].detach(), a0) and torch.count_nonzero(slots.lora_B['lora_0']) == 0
+
+
+def test_custom_ops_are_registered_and_traceable():
+    """torch.ops.twinkle_amd.* exist, declare their mutations, and their fake kernels give exact shapes."""
+    import twinkle_amd  # noqa: F401
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from twinkle_amd import _lib
+    for name in ('segment_build', 'lora_fwd', 'lora_bwd'):
+        assert hasattr(torch.ops.twinkle_amd, name)
+    schema = str(torch.ops.twinkle_amd.lora_fwd.default._schema)
+    assert 'Tensor(a1!) y' in schema and 'Tensor(a2!) h' in schema
+    schema = str(torch.ops.twinkle_amd.lora_bwd.default._schema)
+    for arg in ('dx', 'grad_a', 'grad_b', 'workspace'):
+        assert f'!) {arg}' in schema
+    with FakeTensorMode():
+        keys = torch.empty(1000, dtype=torch.int32)
+        ws = torch.ops.twinkle_amd.segment_build(keys, 7)
+    assert ws.dtype == torch.uint8 and ws.numel() == _lib.load().tk_segment_workspace_bytes(1000, 7)
+    with pytest.raises(RuntimeError, match='GPU'):
+        torch.ops.twinkle_amd.segment_build(torch.zeros(4, dtype=torch.int32), 2)

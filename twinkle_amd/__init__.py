@@ -6,6 +6,7 @@ permute/unpermute around them run in hand-written HIP kernels behind a C ABI
 and mirrors the reference's ``MultiLora`` interface on top.  There is no CPU
 path: every op raises if the HIP library is missing or a tensor is not on the GPU.
 """
+from . import custom_ops  # noqa: F401  (registers torch.ops.twinkle_amd.*)
 from .lora_layer import LoraConfig, LoraLinear, LoraModel, inject_adapter  # noqa: F401
 from .multi_lora import LoraTenant, MultiLora  # noqa: F401
 from .ops import (AdapterGroups, lora_bwd_, lora_bwd_workspace_bytes, lora_expand_, lora_fwd_,  # noqa: F401
