@@ -75,12 +75,16 @@ def main():
     ap.add_argument('--event-every', type=int, default=4,
                     help='bracket the kernels with HIP events on every n-th timed step (an event record costs a few '
                          'microseconds of idle queue, so not every step carries them)')
+    ap.add_argument('--workload', default='cfg2', choices=['cfg2', 'cfg3_up', 'cfg3_down', 'cfg5_q'],
+                    help='cfg2 is the headline configuration; the others are the wider BASELINE shapes '
+                         '(cfg3: 4096<->14336, T=32768, 32 adapters of rank 8..64; cfg5_q: 4096->4096, T=32768, 8 tenants '
+                         'of rank 64, one per packed 4096-token sequence) for additional measurements')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run five plain 128 MiB device copies (a known-size kernel to scale rocprofv3 --pmc '
                          'FETCH_SIZE / WRITE_SIZE readings by)')
     args = ap.parse_args()
     if args.gpus != 1:
-        print('bench.py measures one GPU: this path has no multi-GPU part (rows shard trivially; see DESIGN.md). '
+        print('bench.py measures one GPU: this path has no multi-GPU part (rows are independent and would shard trivially). '
               'Run with --gpus 1.', file=sys.stderr)
         sys.exit(2)
 
@@ -92,7 +96,16 @@ def main():
         sys.exit(2)
     _lib.load()
     dev = torch.device('cuda:0')
-    w = workloads.config2_qproj()
+    if args.workload == 'cfg2':
+        w = workloads.config2_qproj()
+    elif args.workload == 'cfg5_q':
+        w = workloads.config2_qproj(tokens=32768, n=8, r=64)
+        w.ids = torch.repeat_interleave(torch.arange(8, dtype=torch.int32), 4096)
+        w.name = 'cfg5_llama8b_q_rank64'
+    else:
+        w = workloads.config3_mlp('up' if args.workload == 'cfg3_up' else 'down')
+    if args.workload != 'cfg2':
+        args.sets = min(args.sets, 2)
     dt = torch.bfloat16
     elt = 2
     T, K, M, G = w.tokens, w.in_features, w.out_features, w.num_adapters
@@ -195,12 +208,14 @@ def main():
         'vs_baseline': None,
         'dtype': 'bf16',
         'data': 'synthetic',
-        'config': {'workload': 'BASELINE config 2: Llama-3-8B q_proj 4096->4096, T=16384, 16 adapters rank 16 alpha 32, '
-                               'Zipf(1.1) ids shuffled; step = segment build + LoRA fwd + LoRA bwd (dX, dA, dB); '
-                               'base GEMM excluded', 'tokens': T, 'in': K, 'out': M, 'adapters': G, 'rank': 16},
+        'config': {'workload': ('BASELINE config 2: Llama-3-8B q_proj 4096->4096, T=16384, 16 adapters rank 16 alpha 32, '
+                                'Zipf(1.1) ids shuffled' if args.workload == 'cfg2' else w.name) +
+                               '; step = segment build + LoRA fwd + LoRA bwd (dX, dA, dB); base GEMM excluded',
+                   'tokens': T, 'in': K, 'out': M, 'adapters': G, 'rank': max(w.ranks)},
         'roofline': {'bound': 'hbm', 'achieved': achieved, 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                     'frac': achieved / HBM_PEAK_GBS, 'traffic': measured_traffic('k_expand_mfma<1, 1>'),
-                     'kernel': 'k_expand_mfma<1,1> (y += h B^T in place), forward launch',
+                     'frac': achieved / HBM_PEAK_GBS, 'traffic': measured_traffic('k_expand_mfma<1, 1>') if args.workload == 'cfg2' else None,
+                     'kernel': f'k_expand_mfma<{max(1, (max(w.ranks) + 15) // 16 if max(w.ranks) <= 32 else 4)},1> '
+                               '(y += h B^T in place), forward launch',
                      'algorithmic_bytes_per_launch': expand_bytes, 'avg_launch_ms': expand_ms,
                      'launches_timed': len(events)},
         'step_detail': {'shrink_ms': shrink_ms, 'expand_ms': expand_ms, 'fwd_ms': fwd_ms, 'bwd_ms': bwd_ms, 'segment_build_and_gaps_ms': ms_per_step - fwd_ms - bwd_ms,

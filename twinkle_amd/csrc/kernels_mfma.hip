@@ -370,6 +370,108 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
   }
 }
 
+// ---------------------------------------------------------------------------
+// Expand for padded ranks above 16.  There a wave's block of W2 (128 columns x rank) is as large as
+// its piece of a 32-row tile (16 KB at rank 64), so re-reading it for every tile doubles the traffic
+// between L2 and the CUs.  Here a wave keeps the block in registers and walks TPI consecutive tiles
+// of one chunk (same group, hence the same weights): work item = (chunk, part of TPI tiles, 128
+// columns).  The next tile's rows, h operand and destination rows are requested before the current
+// tile is consumed.
+// ---------------------------------------------------------------------------
+template <int NB, int TPI>
+__global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* __restrict__ hrow,
+                                                      const ChunkInfo* __restrict__ chunks,
+                                                      const int32_t* __restrict__ slot_rows) {
+  constexpr int RP = 16 * NB;
+  constexpr int NKS = (RP + 31) / 32;
+  constexpr int PARTS = kChunkTiles / TPI;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  const int ngroups = a.width_dst >> 7;
+  const int nbt = (ngroups + 3) >> 2;  // blocks per (chunk, part): column block fastest
+  const int cb = blockIdx.x % nbt, rest = blockIdx.x / nbt;
+  const int part = rest % PARTS, chunk = rest / PARTS;
+  const int cg = cb * 4 + wave;
+  if (cg >= ngroups) return;
+  const ChunkInfo ci = chunks[chunk];
+  const int g = ci.group;
+  if (g < 0) return;
+  const int nt = min(TPI, ci.ntiles - part * TPI);
+  if (nt <= 0) return;
+  const int r = min(a.rank[g], RP);
+  if (r <= 0) return;
+  const int tile0 = ci.tile0 + part * TPI;
+  const int c0 = cg << 7;
+  const bf16_t* W2 = group_weight<bf16_t>(a.w_expand, a.w_expand_base, a.expand_group_stride, g);
+  uint4 bq[8][NKS];
+#pragma unroll
+  for (int q = 0; q < 8; ++q)
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      const int n0 = 32 * ks + 8 * kb;
+      bq[q][ks] = n0 < r ? keep_first(ld16(W2 + (int64_t)(c0 + 8 * li + q) * a.ld_expand + n0), r - n0) : zero4();
+    }
+
+  struct Tile {
+    int rows[2][4];
+    uint4 hop[2][NKS];
+    uint4 y[2][4];
+  };
+  bf16_t* dst = (bf16_t*)a.dst + c0 + 8 * li;
+  auto issue = [&](int t, Tile& T) {
+    const bool tok = t < nt;  // wave-uniform
+    const int slot0 = (tile0 + (tok ? t : 0)) * kTileRows;
+    const int4 r0 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 4 * kb);
+    const int4 r1 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 16 + 4 * kb);
+    const int rr[2][4] = {{r0.x, r0.y, r0.z, r0.w}, {r1.x, r1.y, r1.z, r1.w}};
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        const int n0 = 32 * ks + 8 * kb;
+        T.hop[tt][ks] = (tok && n0 < RP) ? ld16(hrow + (int64_t)(slot0 + 16 * tt + li) * RP + n0) : zero4();
+      }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        T.rows[tt][v] = tok ? rr[tt][v] : -1;
+        T.y[tt][v] = T.rows[tt][v] >= 0 ? ld16_nt(dst + (int64_t)T.rows[tt][v] * a.ld_dst) : zero4();
+      }
+    }
+  };
+  auto consume = [&](const Tile& T) {
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      f32x4 d[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        d[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) d[q] = mfma16(T.hop[tt][ks], bq[q][ks], d[q]);
+      }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        if (T.rows[tt][v] < 0) continue;
+        const uint4 yy = T.y[tt][v];
+        uint4 o;
+        o.x = pack_bf16(bf16_lo(yy.x) + d[0][v], bf16_hi(yy.x) + d[1][v]);
+        o.y = pack_bf16(bf16_lo(yy.y) + d[2][v], bf16_hi(yy.y) + d[3][v]);
+        o.z = pack_bf16(bf16_lo(yy.z) + d[4][v], bf16_hi(yy.z) + d[5][v]);
+        o.w = pack_bf16(bf16_lo(yy.w) + d[6][v], bf16_hi(yy.w) + d[7][v]);
+        st16_nt(dst + (int64_t)T.rows[tt][v] * a.ld_dst, o);
+      }
+    }
+  };
+  Tile A, B;
+  issue(0, A);
+  for (int t = 0; t < nt; t += 2) {
+    issue(t + 1, B);
+    consume(A);
+    if (t + 1 < nt) {
+      issue(t + 2, A);
+      consume(B);
+    }
+  }
+}
+
 // Eight consecutive bf16 results: one 16-byte store when `vec`, element stores otherwise; `keep` (1..8)
 // elements are written, the rest of the destination is left alone.
 __device__ inline void store_bf16x8(bf16_t* o, const float (&v)[8], int keep, bool accumulate, bool vec) {
@@ -755,6 +857,12 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
                        rows);
   if (!a.dst || !(phases & 2)) return;
   const int64_t ngroups = a.width_dst >> 7;
+  if (NB > 1) {
+    constexpr int TPI = 4;
+    const int64_t blocks = L.max_chunks * (kChunkTiles / TPI) * ceil_div(ngroups, 4);
+    hipLaunchKernelGGL((k_expand_multi<NB, TPI>), dim3((unsigned)blocks), dim3(256), 0, s, a, hrow, seg.chunks, rows);
+    return;
+  }
   const int64_t items = L.max_tiles * ceil_div(ngroups, CPW);
   hipLaunchKernelGGL((k_expand_mfma<NB, CPW>), dim3((unsigned)ceil_div(items, 4)), dim3(256), 0, s, a, hrow,
                      seg.tile_group, rows, (int)items);
