@@ -503,7 +503,8 @@ __device__ inline void store_bf16x8(bf16_t* o, const float (&v)[8], int keep, bo
 constexpr int kWgradStageStride = 132;  // 4 mod 32: conflict-free 16-byte accesses
 template <int NB>
 __device__ inline void wgrad_store(const f32x4 (&acc)[8][NB], float* lds, const WgradArgs& a, const ChunkInfo& ci,
-                                   int g, int r, int c0, int lane) {
+                                   int g, int r_all, int c0, int lane, int n_base = 0) {
+  const int r = r_all - n_base;  // live rows of this block of 16 NB rank indices, which starts at n_base
   constexpr int RP = 16 * NB, OS = kWgradStageStride;
   const int li = lane & 15, kb = lane >> 4;
 #pragma unroll
@@ -517,7 +518,7 @@ __device__ inline void wgrad_store(const f32x4 (&acc)[8][NB], float* lds, const 
   __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
 
   if (ci.partial >= 0) {
-    float* part = a.partial + (int64_t)ci.partial * a.rpad * a.width + c0;
+    float* part = a.partial + ((int64_t)ci.partial * a.rpad + n_base) * a.width + c0;
 #pragma unroll
     for (int i = 0; i < RP / 2; ++i) {
       const int n = 2 * i + (lane >> 5), c = 4 * (lane & 31);
@@ -536,7 +537,7 @@ __device__ inline void wgrad_store(const f32x4 (&acc)[8][NB], float* lds, const 
       const float4 lo = *reinterpret_cast<const float4*>(lds + n * OS + c);
       const float4 hi = *reinterpret_cast<const float4*>(lds + n * OS + c + 4);
       const float v8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-      store_bf16x8(gp + (int64_t)n * a.ld_grad + c0 + c, v8, 8, a.accumulate != 0, vec);
+      store_bf16x8(gp + (int64_t)(n_base + n) * a.ld_grad + c0 + c, v8, 8, a.accumulate != 0, vec);
     }
   } else {
     // grad[c0 + c][n]: a lane owns columns c = lane and lane + 64
@@ -549,7 +550,7 @@ __device__ inline void wgrad_store(const f32x4 (&acc)[8][NB], float* lds, const 
         float v8[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) v8[i] = lds[(n8 + i) * OS + c];
-        store_bf16x8(gp + (int64_t)(c0 + c) * a.ld_grad + n8, v8, min(8, r - n8), a.accumulate != 0, vec);
+        store_bf16x8(gp + (int64_t)(c0 + c) * a.ld_grad + n_base + n8, v8, min(8, r - n8), a.accumulate != 0, vec);
       }
     }
   }
@@ -602,19 +603,27 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
 // buffer (groups that span several chunks; k_wgrad_reduce adds the chunks in order) or straight into the
 // gradient (single-chunk groups).  No atomics: the result is bitwise repeatable.
 // ---------------------------------------------------------------------------
-template <int NB, int NW, int DEPTH>
-__global__ __launch_bounds__(NW * 64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo* __restrict__ chunks,
-                                                        const int32_t* __restrict__ slot_rows) {
+//
+// RS > 1 (padded ranks above 32, where 128 columns x rank of accumulators would leave one wave per SIMD):
+// the block has RS waves that walk the same tiles and each own 1/RS of the rank indices; the second
+// reader of a tile finds it in the CU's cache.
+template <int NB, int NW, int DEPTH, int RS = 1>
+__global__ __launch_bounds__(NW * RS * 64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo* __restrict__ chunks,
+                                                             const int32_t* __restrict__ slot_rows) {
+  static_assert(RS == 1 || NW == 1, "either the tiles or the rank indices are split over the waves");
+  static_assert(NB % RS == 0, "rank blocks must divide evenly");
+  constexpr int NBW = NB / RS;           // blocks of 16 rank indices per wave
   constexpr int TPW = kChunkTiles / NW;  // tiles per wave
   constexpr int RP = 16 * NB;
   constexpr int OS = kWgradStageStride;
   constexpr int RED = (NW - 1) * 32 * NB * 64;
   constexpr int OUT = RP * OS;
   __shared__ __attribute__((aligned(16))) float lds[RED > OUT ? RED : OUT];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kb = lane >> 4;
+  const int wave = (tid >> 6) / RS, rs = (tid >> 6) % RS;
   if ((int)blockIdx.y < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
-    transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (NW * 64) + tid,
-                          (int64_t)a.tr.y_blocks * gridDim.x * (NW * 64));
+    transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (NW * RS * 64) + tid,
+                          (int64_t)a.tr.y_blocks * gridDim.x * (NW * RS * 64));
     return;
   }
   // column block fastest: blocks that run together read neighbouring pieces of the same rows
@@ -623,21 +632,22 @@ __global__ __launch_bounds__(NW * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
   const int g = ci.group;
   if (g < 0) return;
   const int r = min(a.rank[g], RP);
-  if (r <= 0) return;
+  const int n_base = rs * NBW * 16;  // first rank index of this wave
+  if (r <= n_base) return;           // covers r <= 0; with RS > 1 there is no block barrier below
 
   const bf16_t* src = (const bf16_t*)a.src + c0 + 8 * li;
-  const bf16_t* hT = (const bf16_t*)a.hT + 8 * kb;
+  const bf16_t* hT = (const bf16_t*)a.hT + (int64_t)n_base * a.ldh + 8 * kb;
   const int32_t* rows_p = slot_rows + ci.tile0 * kTileRows + 8 * kb;  // this lane's 8 slots of the chunk's first tile
-  f32x4 acc[8][NB];
+  f32x4 acc[8][NBW];
 #pragma unroll
   for (int q = 0; q < 8; ++q)
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) acc[q][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int nb = 0; nb < NBW; ++nb) acc[q][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   const int t0 = wave * TPW;
   if (t0 < ci.ntiles) {
     int4 ra[TPW], rb[TPW];
-    uint4 x[TPW][8], h[TPW][NB];
+    uint4 x[TPW][8], h[TPW][NBW];
     auto load_rows = [&](int u) {
       const int t = min(t0 + u, ci.ntiles - 1);  // tiles past the end re-read the last one and are masked below
       ra[u] = *reinterpret_cast<const int4*>(rows_p + t * kTileRows);
@@ -651,7 +661,7 @@ __global__ __launch_bounds__(NW * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
       for (int q = 0; q < 8; ++q)
         x[u][q] = (tok && rows[q] >= 0) ? ld16(src + (int64_t)rows[q] * a.ld_src) : zero4();
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
+      for (int nb = 0; nb < NBW; ++nb)
         h[u][nb] = tok ? ld16(hT + (int64_t)(16 * nb + li) * a.ldh + (ci.tile0 + t) * kTileRows) : zero4();
     };
     auto consume = [&](int u) {
@@ -672,7 +682,7 @@ __global__ __launch_bounds__(NW * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
         tr.z = __builtin_amdgcn_perm(e[5], e[4], sel);
         tr.w = __builtin_amdgcn_perm(e[7], e[6], sel);
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) acc[q][nb] = mfma16(tr, h[u][nb], acc[q][nb]);
+        for (int nb = 0; nb < NBW; ++nb) acc[q][nb] = mfma16(tr, h[u][nb], acc[q][nb]);
       }
     };
 #pragma unroll
@@ -693,7 +703,7 @@ __global__ __launch_bounds__(NW * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
 #pragma unroll
       for (int q = 0; q < 8; ++q)
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
+        for (int nb = 0; nb < NBW; ++nb)
 #pragma unroll
           for (int v = 0; v < 4; ++v) lds[((wave - 1) * 32 * NB + (q * NB + nb) * 4 + v) * 64 + lane] = acc[q][nb][v];
     }
@@ -703,13 +713,13 @@ __global__ __launch_bounds__(NW * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
 #pragma unroll
       for (int q = 0; q < 8; ++q)
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
+        for (int nb = 0; nb < NBW; ++nb)
 #pragma unroll
           for (int v = 0; v < 4; ++v) acc[q][nb][v] += lds[(w * 32 * NB + (q * NB + nb) * 4 + v) * 64 + lane];
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");  // the sums are read before the staging below overwrites them
   }
 
-  wgrad_store<NB>(acc, lds, a, ci, g, r, c0, lane);
+  wgrad_store<NBW>(acc, lds + n_base * OS, a, ci, g, r, c0, lane, n_base);
 }
 
 // ---------------------------------------------------------------------------
@@ -868,16 +878,17 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
                      seg.tile_group, rows, (int)items);
 }
 
-template <int NB, int NW, int DEPTH>
+template <int NB, int NW, int DEPTH, int RS = 1>
 void launch_wgrad_pipe(const WgradArgs& a0, const SegView& seg, const SegLayout& L, hipStream_t s) {
   WgradArgs a = a0;
   a.tr.y_blocks = 0;
   if (a.tr.aT) {  // about four 16-byte outputs per thread of the side job
     const int64_t units = (int64_t)a.tr.groups * a.rpad * ((a.tr.out_features + a.tr.in_features) / 8);
-    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 128) * (NW * 64))));
+    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 128) * (NW * RS * 64))));
   }
   const dim3 grid((unsigned)(a.width / 128), (unsigned)(L.max_chunks + a.tr.y_blocks));
-  hipLaunchKernelGGL((k_wgrad_pipe<NB, NW, DEPTH>), grid, dim3(NW * 64), 0, s, a, seg.chunks, seg.slot_table(a.map_rows));
+  hipLaunchKernelGGL((k_wgrad_pipe<NB, NW, DEPTH, RS>), grid, dim3(NW * RS * 64), 0, s, a, seg.chunks,
+                     seg.slot_table(a.map_rows));
 }
 
 }  // namespace
@@ -929,7 +940,7 @@ int launch_wgrad_mfma(const WgradArgs& a, const SegView& seg, const SegLayout& L
   if (L.rows == 0) return TK_OK;
   if (a.rpad <= 16) launch_wgrad_pipe<1, 1, 2>(a, seg, L, s);
   else if (a.rpad <= 32) launch_wgrad_pipe<2, 1, 2>(a, seg, L, s);
-  else launch_wgrad_pipe<4, 2, 1>(a, seg, L, s);
+  else launch_wgrad_pipe<4, 1, 2, 2>(a, seg, L, s);
   return check_launch();
 }
 
