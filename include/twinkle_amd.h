@@ -34,7 +34,8 @@ enum {
 enum { TK_DTYPE_F32 = 0, TK_DTYPE_BF16 = 1 };
 enum { TK_KEY_I32 = 0, TK_KEY_I64 = 1 };
 
-/* Rows per forward tile and per weight-gradient chunk (fixed at build time). */
+/* Rows per forward tile and per smallest weight-gradient chunk (fixed at build time; chunks grow with the
+ * batch: 512 rows up to 16384 rows, then doubling with the row count up to 4096). */
 #define TK_TILE_ROWS 32
 #ifndef TK_CHUNK_ROWS
 #define TK_CHUNK_ROWS 512

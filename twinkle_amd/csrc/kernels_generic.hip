@@ -125,13 +125,14 @@ __device__ inline void store_grad(const WgradArgs& a, int g, int n, int c, float
   from_f32(v, o);
 }
 
-// One chunk (up to 16 tiles) of one group, 256 columns per block:
+// One chunk of one group, 256 columns per block, walked in passes of 512 slots:
 // out[n][c] = sum_{slot in chunk} hT[n][slot] * src[row(slot)][c], slots ascending.
 template <typename T>
 __global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkInfo* __restrict__ chunks,
                                                        const int32_t* __restrict__ slot_rows) {
-  __shared__ float hs[16][kChunkRows];
-  __shared__ int rows_s[kChunkRows];
+  constexpr int kPass = kChunkTilesMin * kTileRows;
+  __shared__ float hs[16][kPass];
+  __shared__ int rows_s[kPass];
   const ChunkInfo ci = chunks[blockIdx.x];
   const int g = ci.group;
   if (g < 0) return;
@@ -139,28 +140,33 @@ __global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkI
   if (r <= 0) return;
   const int tid = threadIdx.x;
   const int c = blockIdx.y * 256 + tid;
-  const int slot0 = ci.tile0 * kTileRows;
-  const int len = ci.ntiles * kTileRows;
-  for (int i = tid; i < len; i += 256) rows_s[i] = slot_rows[slot0 + i];
+  const int total = ci.ntiles * kTileRows;
   const T* src = (const T*)a.src;
   const T* hT = (const T*)a.hT;
   for (int n0 = 0; n0 < r; n0 += 16) {
-    __syncthreads();
-    for (int i = tid; i < 16 * len; i += 256) {
-      const int j = i / len, pp = i % len;
-      hs[j][pp] = (n0 + j) < r ? to_f32(hT[(int64_t)(n0 + j) * a.ldh + slot0 + pp]) : 0.f;
-    }
-    __syncthreads();
-    if (c < a.width) {
-      float acc[16];
+    float acc[16];
 #pragma unroll
-      for (int j = 0; j < 16; ++j) acc[j] = 0.f;
-      for (int pp = 0; pp < len; ++pp) {
-        if (rows_s[pp] < 0) continue;
-        const float xv = to_f32(src[(int64_t)rows_s[pp] * a.ld_src + c]);
-#pragma unroll
-        for (int j = 0; j < 16; ++j) acc[j] += hs[j][pp] * xv;
+    for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+    for (int p0 = 0; p0 < total; p0 += kPass) {
+      const int slot0 = ci.tile0 * kTileRows + p0;
+      const int len = min(kPass, total - p0);
+      __syncthreads();
+      for (int i = tid; i < len; i += 256) rows_s[i] = slot_rows[slot0 + i];
+      for (int i = tid; i < 16 * len; i += 256) {
+        const int j = i / len, pp = i % len;
+        hs[j][pp] = (n0 + j) < r ? to_f32(hT[(int64_t)(n0 + j) * a.ldh + slot0 + pp]) : 0.f;
       }
+      __syncthreads();
+      if (c < a.width) {
+        for (int pp = 0; pp < len; ++pp) {
+          if (rows_s[pp] < 0) continue;
+          const float xv = to_f32(src[(int64_t)rows_s[pp] * a.ld_src + c]);
+#pragma unroll
+          for (int j = 0; j < 16; ++j) acc[j] += hs[j][pp] * xv;
+        }
+      }
+    }
+    if (c < a.width) {
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         const int n = n0 + j;

@@ -373,50 +373,35 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
 // ---------------------------------------------------------------------------
 // Expand for padded ranks above 16.  There a wave's block of W2 (128 columns x rank) is as large as
 // its piece of a 32-row tile (16 KB at rank 64), so re-reading it for every tile doubles the traffic
-// between L2 and the CUs.  Here a wave keeps the block in registers and walks TPI consecutive tiles
-// of one chunk (same group, hence the same weights): work item = (chunk, part of TPI tiles, 128
-// columns).  The next tile's rows, h operand and destination rows are requested before the current
-// tile is consumed.
+// between L2 and the CUs.  Here a wave keeps the block in registers and walks TPI consecutive tiles:
+// work item = (TPI tiles, 128 columns).  Consecutive tiles almost always belong to the same group;
+// where the group changes inside an item the wave reloads the block.  The next tile's rows, h operand
+// and destination rows are requested before the current tile is consumed.
 // ---------------------------------------------------------------------------
 template <int NB, int TPI>
 __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* __restrict__ hrow,
-                                                      const ChunkInfo* __restrict__ chunks,
-                                                      const int32_t* __restrict__ slot_rows) {
+                                                      const int32_t* __restrict__ tile_group,
+                                                      const int32_t* __restrict__ slot_rows, int max_tiles) {
   constexpr int RP = 16 * NB;
   constexpr int NKS = (RP + 31) / 32;
-  constexpr int PARTS = kChunkTiles / TPI;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
   const int ngroups = a.width_dst >> 7;
-  const int nbt = (ngroups + 3) >> 2;  // blocks per (chunk, part): column block fastest
-  const int cb = blockIdx.x % nbt, rest = blockIdx.x / nbt;
-  const int part = rest % PARTS, chunk = rest / PARTS;
+  const int nbt = (ngroups + 3) >> 2;  // blocks per tile set: column block fastest
+  const int cb = blockIdx.x % nbt, tile0 = (blockIdx.x / nbt) * TPI;
   const int cg = cb * 4 + wave;
   if (cg >= ngroups) return;
-  const ChunkInfo ci = chunks[chunk];
-  const int g = ci.group;
-  if (g < 0) return;
-  const int nt = min(TPI, ci.ntiles - part * TPI);
-  if (nt <= 0) return;
-  const int r = min(a.rank[g], RP);
-  if (r <= 0) return;
-  const int tile0 = ci.tile0 + part * TPI;
+  const int nt = min(TPI, max_tiles - tile0);
+  int gt[TPI];
+#pragma unroll
+  for (int t = 0; t < TPI; ++t) gt[t] = t < nt ? tile_group[tile0 + t] : -1;
   const int c0 = cg << 7;
-  const bf16_t* W2 = group_weight<bf16_t>(a.w_expand, a.w_expand_base, a.expand_group_stride, g);
-  uint4 bq[8][NKS];
-#pragma unroll
-  for (int q = 0; q < 8; ++q)
-#pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) {
-      const int n0 = 32 * ks + 8 * kb;
-      bq[q][ks] = n0 < r ? keep_first(ld16(W2 + (int64_t)(c0 + 8 * li + q) * a.ld_expand + n0), r - n0) : zero4();
-    }
+  bf16_t* dst = (bf16_t*)a.dst + c0 + 8 * li;
 
   struct Tile {
     int rows[2][4];
     uint4 hop[2][NKS];
     uint4 y[2][4];
   };
-  bf16_t* dst = (bf16_t*)a.dst + c0 + 8 * li;
   auto issue = [&](int t, Tile& T) {
     const bool tok = t < nt;  // wave-uniform
     const int slot0 = (tile0 + (tok ? t : 0)) * kTileRows;
@@ -436,6 +421,19 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
         T.y[tt][v] = T.rows[tt][v] >= 0 ? ld16_nt(dst + (int64_t)T.rows[tt][v] * a.ld_dst) : zero4();
       }
     }
+  };
+  uint4 bq[8][NKS];
+  int r = 0;
+  auto load_weights = [&](int g) {  // this wave's block of W2 for group g
+    r = min(a.rank[g], RP);
+    const bf16_t* W2 = group_weight<bf16_t>(a.w_expand, a.w_expand_base, a.expand_group_stride, g);
+#pragma unroll
+    for (int q = 0; q < 8; ++q)
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) {
+        const int n0 = 32 * ks + 8 * kb;
+        bq[q][ks] = n0 < r ? keep_first(ld16(W2 + (int64_t)(c0 + 8 * li + q) * a.ld_expand + n0), r - n0) : zero4();
+      }
   };
   auto consume = [&](const Tile& T) {
 #pragma unroll
@@ -460,15 +458,35 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
       }
     }
   };
+  // tiles past the last one of the table carry -1 and come last
+  bool uniform = true;
+#pragma unroll
+  for (int t = 1; t < TPI; ++t) uniform = uniform && (gt[t] == gt[0] || gt[t] < 0);
   Tile A, B;
-  issue(0, A);
-  for (int t = 0; t < nt; t += 2) {
-    issue(t + 1, B);
-    consume(A);
-    if (t + 1 < nt) {
-      issue(t + 2, A);
-      consume(B);
+  if (uniform) {  // the usual case: one group, one block of W2, loads pipelined over the tiles
+    if (gt[0] < 0) return;
+    int nv = 0;
+#pragma unroll
+    for (int t = 0; t < TPI; ++t) nv += gt[t] >= 0;
+    load_weights(gt[0]);
+    if (r <= 0) return;  // adapter not live on this layer
+    issue(0, A);
+    for (int t = 0; t < nv; t += 2) {
+      issue(t + 1 < nv ? t + 1 : nt, B);
+      consume(A);
+      if (t + 1 < nv) {
+        issue(t + 2 < nv ? t + 2 : nt, A);
+        consume(B);
+      }
     }
+    return;
+  }
+  for (int t = 0; t < nt; ++t) {  // a group boundary inside the item: tile by tile
+    if (gt[t] < 0) continue;
+    load_weights(gt[t]);
+    if (r <= 0) continue;
+    issue(t, A);
+    consume(A);
   }
 }
 
@@ -593,37 +611,30 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
 // ---------------------------------------------------------------------------
 // Weight gradient: out_g[n][c] = sum over the rows of group g of hT[n][slot] * src[row(slot)][c].
 //
-// Work item = (chunk of up to 16 tiles of one group, 128 source columns), one block of NW waves; wave w
-// owns tiles w*TPW .. of the chunk.  The loads run as a software pipeline over the wave's tiles: the row
-// indices of tile t+DEPTH+1 and the source rows of tile t+DEPTH are requested before tile t is consumed,
-// so a wave never waits on an index load and always has DEPTH tiles (8 KB each) in flight.  A lane loads
-// 16 B of eight rows, transposes the 8x8 block in registers (v_perm_b32) and feeds it as the MFMA A
-// operand with the rows as contraction index.  The waves' sums are added in wave order in LDS, staged
-// there in [n][column] order and leave as whole 512-byte rows: into the chunk's slot of the partial
-// buffer (groups that span several chunks; k_wgrad_reduce adds the chunks in order) or straight into the
-// gradient (single-chunk groups).  No atomics: the result is bitwise repeatable.
-// ---------------------------------------------------------------------------
+// Work item = (chunk of one group, 128 source columns), one block of RS waves.  A wave walks all tiles of
+// the chunk with a three-stage software pipeline: the row indices of tile t+3 and the source rows of
+// tile t+2 are requested before tile t is consumed, so a wave never waits on an index load and has two
+// tiles (8 KB each) in flight.  A lane loads 16 B of eight rows, transposes the 8x8 block in registers
+// (v_perm_b32) and feeds it as the MFMA A operand with the rows as contraction index.  The result is
+// staged in LDS in [n][column] order and leaves as whole 512-byte rows: into the chunk's slot of the
+// partial buffer (groups that span several chunks; k_wgrad_reduce adds the chunks in order) or straight
+// into the gradient (single-chunk groups).  No atomics: the result is bitwise repeatable.
 //
-// RS > 1 (padded ranks above 32, where 128 columns x rank of accumulators would leave one wave per SIMD):
-// the block has RS waves that walk the same tiles and each own 1/RS of the rank indices; the second
-// reader of a tile finds it in the CU's cache.
-template <int NB, int NW, int DEPTH, int RS = 1>
-__global__ __launch_bounds__(NW * RS * 64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo* __restrict__ chunks,
-                                                             const int32_t* __restrict__ slot_rows) {
-  static_assert(RS == 1 || NW == 1, "either the tiles or the rank indices are split over the waves");
+// RS > 1 (padded rank 64, where 128 columns x rank of accumulators would leave one wave per SIMD): the
+// RS waves of a block walk the same tiles and each own 1/RS of the rank indices; the second reader of a
+// tile finds it in the CU's cache.
+// ---------------------------------------------------------------------------
+template <int NB, int RS>
+__global__ __launch_bounds__(RS * 64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo* __restrict__ chunks,
+                                                        const int32_t* __restrict__ slot_rows) {
   static_assert(NB % RS == 0, "rank blocks must divide evenly");
-  constexpr int NBW = NB / RS;           // blocks of 16 rank indices per wave
-  constexpr int TPW = kChunkTiles / NW;  // tiles per wave
-  constexpr int RP = 16 * NB;
+  constexpr int NBW = NB / RS;  // blocks of 16 rank indices per wave
   constexpr int OS = kWgradStageStride;
-  constexpr int RED = (NW - 1) * 32 * NB * 64;
-  constexpr int OUT = RP * OS;
-  __shared__ __attribute__((aligned(16))) float lds[RED > OUT ? RED : OUT];
-  const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kb = lane >> 4;
-  const int wave = (tid >> 6) / RS, rs = (tid >> 6) % RS;
+  __shared__ __attribute__((aligned(16))) float lds[16 * NB * OS];
+  const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kb = lane >> 4, rs = tid >> 6;
   if ((int)blockIdx.y < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
-    transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (NW * RS * 64) + tid,
-                          (int64_t)a.tr.y_blocks * gridDim.x * (NW * RS * 64));
+    transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (RS * 64) + tid,
+                          (int64_t)a.tr.y_blocks * gridDim.x * (RS * 64));
     return;
   }
   // column block fastest: blocks that run together read neighbouring pieces of the same rows
@@ -631,12 +642,13 @@ __global__ __launch_bounds__(NW * RS * 64) void k_wgrad_pipe(WgradArgs a, const 
   const ChunkInfo ci = chunks[blockIdx.y - a.tr.y_blocks];
   const int g = ci.group;
   if (g < 0) return;
-  const int r = min(a.rank[g], RP);
+  const int r = min(a.rank[g], 16 * NB);
   const int n_base = rs * NBW * 16;  // first rank index of this wave
-  if (r <= n_base) return;           // covers r <= 0; with RS > 1 there is no block barrier below
+  if (r <= n_base) return;           // covers r <= 0; the waves of a block never meet at a barrier
 
+  const int nt = ci.ntiles;
   const bf16_t* src = (const bf16_t*)a.src + c0 + 8 * li;
-  const bf16_t* hT = (const bf16_t*)a.hT + (int64_t)n_base * a.ldh + 8 * kb;
+  const bf16_t* hT = (const bf16_t*)a.hT + (int64_t)(n_base + li) * a.ldh + (int64_t)ci.tile0 * kTileRows + 8 * kb;
   const int32_t* rows_p = slot_rows + ci.tile0 * kTileRows + 8 * kb;  // this lane's 8 slots of the chunk's first tile
   f32x4 acc[8][NBW];
 #pragma unroll
@@ -644,87 +656,88 @@ __global__ __launch_bounds__(NW * RS * 64) void k_wgrad_pipe(WgradArgs a, const 
 #pragma unroll
     for (int nb = 0; nb < NBW; ++nb) acc[q][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const int t0 = wave * TPW;
-  if (t0 < ci.ntiles) {
-    int4 ra[TPW], rb[TPW];
-    uint4 x[TPW][8], h[TPW][NBW];
-    auto load_rows = [&](int u) {
-      const int t = min(t0 + u, ci.ntiles - 1);  // tiles past the end re-read the last one and are masked below
-      ra[u] = *reinterpret_cast<const int4*>(rows_p + t * kTileRows);
-      rb[u] = *reinterpret_cast<const int4*>(rows_p + t * kTileRows + 4);
-    };
-    auto issue = [&](int u) {
-      const bool tok = t0 + u < ci.ntiles;  // wave-uniform
-      const int t = tok ? t0 + u : 0;
-      const int rows[8] = {ra[u].x, ra[u].y, ra[u].z, ra[u].w, rb[u].x, rb[u].y, rb[u].z, rb[u].w};
+  // The loop body below is straight-line code: every load is unconditional (tiles past the end re-read the
+  // last tile, padding slots read row 0) and what must not count is zeroed when it is consumed.  With no
+  // branch between a load and its use the compiler can wait for exactly the loads it needs and leave the
+  // younger ones in flight.
+  struct Tile {
+    uint4 x[8];
+    uint4 h[NBW];
+    uint32_t live;  // bit q: row q of this lane is a real row of a tile inside the chunk
+  };
+  int4 ra, rb;  // row indices of the tile that is issued next
+  auto load_rows = [&](int t) {
+    const int tc = min(t, nt - 1);
+    ra = *reinterpret_cast<const int4*>(rows_p + tc * kTileRows);
+    rb = *reinterpret_cast<const int4*>(rows_p + tc * kTileRows + 4);
+  };
+  auto issue = [&](int t, Tile& T) {
+    const int tc = min(t, nt - 1);
+    const int rows[8] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w};
+    T.live = 0;
 #pragma unroll
-      for (int q = 0; q < 8; ++q)
-        x[u][q] = (tok && rows[q] >= 0) ? ld16(src + (int64_t)rows[q] * a.ld_src) : zero4();
+    for (int q = 0; q < 8; ++q) {
+      T.x[q] = ld16(src + (int64_t)max(rows[q], 0) * a.ld_src);
+      T.live |= (t < nt && rows[q] >= 0) ? (1u << q) : 0u;
+    }
 #pragma unroll
-      for (int nb = 0; nb < NBW; ++nb)
-        h[u][nb] = tok ? ld16(hT + (int64_t)(16 * nb + li) * a.ldh + (ci.tile0 + t) * kTileRows) : zero4();
-    };
-    auto consume = [&](int u) {
-      // 8x8 transpose inside the lane: tr[q] holds column q of the 8 rows
+    for (int nb = 0; nb < NBW; ++nb) T.h[nb] = ld16(hT + (int64_t)(16 * nb) * a.ldh + tc * kTileRows);
+  };
+  auto consume = [&](const Tile& T) {
+    // 8x8 transpose inside the lane: tr holds column q of the 8 rows
 #pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        const int d = q >> 1;
-        const uint32_t sel = (q & 1) ? 0x07060302u : 0x05040100u;
-        uint32_t e[8];
+    for (int q = 0; q < 8; ++q) {
+      const int d = q >> 1;
+      const uint32_t sel = (q & 1) ? 0x07060302u : 0x05040100u;
+      uint32_t e[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const uint32_t wsrc[4] = {x[u][i].x, x[u][i].y, x[u][i].z, x[u][i].w};
-          e[i] = wsrc[d];
-        }
-        uint4 tr;
-        tr.x = __builtin_amdgcn_perm(e[1], e[0], sel);
-        tr.y = __builtin_amdgcn_perm(e[3], e[2], sel);
-        tr.z = __builtin_amdgcn_perm(e[5], e[4], sel);
-        tr.w = __builtin_amdgcn_perm(e[7], e[6], sel);
-#pragma unroll
-        for (int nb = 0; nb < NBW; ++nb) acc[q][nb] = mfma16(tr, h[u][nb], acc[q][nb]);
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t wsrc[4] = {T.x[i].x, T.x[i].y, T.x[i].z, T.x[i].w};
+        e[i] = (T.live >> i) & 1u ? wsrc[d] : 0u;
       }
-    };
+      uint4 tr;
+      tr.x = __builtin_amdgcn_perm(e[1], e[0], sel);
+      tr.y = __builtin_amdgcn_perm(e[3], e[2], sel);
+      tr.z = __builtin_amdgcn_perm(e[5], e[4], sel);
+      tr.w = __builtin_amdgcn_perm(e[7], e[6], sel);
 #pragma unroll
-    for (int u = 0; u <= DEPTH && u < TPW; ++u) load_rows(u);
-#pragma unroll
-    for (int u = 0; u < DEPTH && u < TPW; ++u) issue(u);
-#pragma unroll
-    for (int u = 0; u < TPW; ++u) {
-      if (u + DEPTH < TPW) issue(u + DEPTH);
-      if (u + DEPTH + 1 < TPW) load_rows(u + DEPTH + 1);
-      consume(u);
+      for (int nb = 0; nb < NBW; ++nb) acc[q][nb] = mfma16(tr, T.h[nb], acc[q][nb]);
     }
+  };
+  Tile A, B, C;
+  load_rows(0);
+  issue(0, A);
+  load_rows(1);
+  issue(1, B);
+  load_rows(2);
+  int t = 0;
+  for (; t + 4 < nt; t += 3) {  // every tile touched in here exists
+    issue(t + 2, C);
+    load_rows(t + 3);
+    consume(A);
+    issue(t + 3, A);
+    load_rows(t + 4);
+    consume(B);
+    issue(t + 4, B);
+    load_rows(t + 5);
+    consume(C);
   }
-
-  // add the waves' accumulators in wave order; wave 0 keeps the result
-  if (NW > 1) {
-    if (wave > 0) {
-#pragma unroll
-      for (int q = 0; q < 8; ++q)
-#pragma unroll
-        for (int nb = 0; nb < NBW; ++nb)
-#pragma unroll
-          for (int v = 0; v < 4; ++v) lds[((wave - 1) * 32 * NB + (q * NB + nb) * 4 + v) * 64 + lane] = acc[q][nb][v];
-    }
-    __syncthreads();
-    if (wave > 0) return;
-    for (int w = 0; w < NW - 1; ++w)
-#pragma unroll
-      for (int q = 0; q < 8; ++q)
-#pragma unroll
-        for (int nb = 0; nb < NBW; ++nb)
-#pragma unroll
-          for (int v = 0; v < 4; ++v) acc[q][nb][v] += lds[(w * 32 * NB + (q * NB + nb) * 4 + v) * 64 + lane];
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");  // the sums are read before the staging below overwrites them
+  // drain: one to four tiles are left, t and t + 1 already on their way (tiles past the end count as zeros)
+  issue(t + 2, C);
+  load_rows(t + 3);
+  consume(A);
+  consume(B);
+  consume(C);
+  if (t + 3 < nt) {
+    issue(t + 3, A);
+    consume(A);
   }
-
   wgrad_store<NBW>(acc, lds + n_base * OS, a, ci, g, r, c0, lane, n_base);
 }
 
 // ---------------------------------------------------------------------------
 // Backward, both uses of dy in one pass (rank <= 16, width a multiple of 512): a block of four waves owns
-// (chunk of up to 16 tiles of one group, 512 columns), wave w the columns [128 w, 128 w + 128) of it.
+// (chunk of one group, 512 columns), wave w the columns [128 w, 128 w + 128) of it.
 // Per tile a wave loads its 32 x 128 piece once, in the weight-gradient layout (a lane holds 8 rows x 8
 // columns), and uses it twice:
 //   dB:  the piece, transposed in registers, is the MFMA A operand with the rows as contraction index,
@@ -742,7 +755,7 @@ __global__ __launch_bounds__(256) void k_dy_fused(WgradArgs a, const void* const
                                                   const int32_t* __restrict__ slot_rows) {
   constexpr int SS = 136;  // row stride of the staged piece in bf16 (272 B)
   constexpr int PR = 17;   // row stride of the partial dh in floats
-  __shared__ int32_t rows_s[kChunkRows];
+  __shared__ int32_t rows_s[kChunkTilesMax * kTileRows];
   __shared__ __attribute__((aligned(16))) bf16_t stage[4][kTileRows * SS];
   __shared__ float part[2][4][kTileRows * PR];
   static_assert(sizeof(bf16_t) * kTileRows * SS >= sizeof(float) * 16 * kWgradStageStride, "stage holds the dB block too");
@@ -869,8 +882,9 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
   const int64_t ngroups = a.width_dst >> 7;
   if (NB > 1) {
     constexpr int TPI = 4;
-    const int64_t blocks = L.max_chunks * (kChunkTiles / TPI) * ceil_div(ngroups, 4);
-    hipLaunchKernelGGL((k_expand_multi<NB, TPI>), dim3((unsigned)blocks), dim3(256), 0, s, a, hrow, seg.chunks, rows);
+    const int64_t blocks = ceil_div(L.max_tiles, TPI) * ceil_div(ngroups, 4);
+    hipLaunchKernelGGL((k_expand_multi<NB, TPI>), dim3((unsigned)blocks), dim3(256), 0, s, a, hrow, seg.tile_group,
+                       rows, (int)L.max_tiles);
     return;
   }
   const int64_t items = L.max_tiles * ceil_div(ngroups, CPW);
@@ -878,17 +892,16 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
                      seg.tile_group, rows, (int)items);
 }
 
-template <int NB, int NW, int DEPTH, int RS = 1>
+template <int NB, int RS>
 void launch_wgrad_pipe(const WgradArgs& a0, const SegView& seg, const SegLayout& L, hipStream_t s) {
   WgradArgs a = a0;
   a.tr.y_blocks = 0;
   if (a.tr.aT) {  // about four 16-byte outputs per thread of the side job
     const int64_t units = (int64_t)a.tr.groups * a.rpad * ((a.tr.out_features + a.tr.in_features) / 8);
-    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 128) * (NW * RS * 64))));
+    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 128) * (RS * 64))));
   }
   const dim3 grid((unsigned)(a.width / 128), (unsigned)(L.max_chunks + a.tr.y_blocks));
-  hipLaunchKernelGGL((k_wgrad_pipe<NB, NW, DEPTH, RS>), grid, dim3(NW * RS * 64), 0, s, a, seg.chunks,
-                     seg.slot_table(a.map_rows));
+  hipLaunchKernelGGL((k_wgrad_pipe<NB, RS>), grid, dim3(RS * 64), 0, s, a, seg.chunks, seg.slot_table(a.map_rows));
 }
 
 }  // namespace
@@ -938,9 +951,9 @@ bool wgrad_mfma_supported(const WgradArgs& a) {
 
 int launch_wgrad_mfma(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
   if (L.rows == 0) return TK_OK;
-  if (a.rpad <= 16) launch_wgrad_pipe<1, 1, 2>(a, seg, L, s);
-  else if (a.rpad <= 32) launch_wgrad_pipe<2, 1, 2>(a, seg, L, s);
-  else launch_wgrad_pipe<4, 1, 2, 2>(a, seg, L, s);
+  if (a.rpad <= 16) launch_wgrad_pipe<1, 1>(a, seg, L, s);
+  else if (a.rpad <= 32) launch_wgrad_pipe<2, 1>(a, seg, L, s);
+  else launch_wgrad_pipe<4, 2>(a, seg, L, s);
   return check_launch();
 }
 

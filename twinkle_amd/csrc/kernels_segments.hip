@@ -115,7 +115,8 @@ __device__ inline int group_of(const int32_t* first, int groups, int i) {
 constexpr int kScanLdsGroups = 2048;  // up to this many groups the scan keeps its four prefix tables in LDS
 
 __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sort_blocks, int max_tiles,
-                                                   int max_chunks, SegView V, int64_t* __restrict__ offsets_out) {
+                                                   int max_chunks, int chunk_tiles, SegView V,
+                                                   int64_t* __restrict__ offsets_out) {
   __shared__ int wave_sums[17];
   __shared__ int32_t lds_first[4][kScanLdsGroups + 1];  // offsets, tile_first, chunk_first, partial_first
   const int tid = threadIdx.x;
@@ -143,7 +144,7 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
       }
     }
     const int ntile = (count + kTileRows - 1) / kTileRows;
-    const int nchunk = (ntile + kChunkTiles - 1) / kChunkTiles;
+    const int nchunk = (ntile + chunk_tiles - 1) / chunk_tiles;
     const int npart = nchunk > 1 ? nchunk : 0;
     int tot;
     const int e_rows = block_exclusive_scan(count, wave_sums, &tot) + carry_rows;
@@ -221,8 +222,8 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
       const int j = i - cfirst[g];
       const int ntile = tfirst[g + 1] - tfirst[g];
       c.group = g;
-      c.tile0 = tfirst[g] + j * kChunkTiles;
-      c.ntiles = min(kChunkTiles, ntile - j * kChunkTiles);
+      c.tile0 = tfirst[g] + j * chunk_tiles;
+      c.ntiles = min(chunk_tiles, ntile - j * chunk_tiles);
       c.partial = cfirst[g + 1] - cfirst[g] > 1 ? pfirst[g] + j : -1;
     }
     V.chunks[i] = c;
@@ -288,7 +289,8 @@ constexpr int kOneBatch = kOneBlocks / kOneWaves;  // sort blocks whose keys a w
 template <typename KeyT>
 __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restrict__ keys, int rows, int groups,
                                                             int key_bits, int sort_blocks, int max_tiles,
-                                                            int max_chunks, SegView V, int64_t* __restrict__ perm_out,
+                                                            int max_chunks, int chunk_tiles, SegView V,
+                                                            int64_t* __restrict__ perm_out,
                                                             int64_t* __restrict__ offsets_out) {
   __shared__ int32_t cnt[2][kOneSubs][kOneGroups + 1];  // keys ahead of this block / in it and after it
   __shared__ int32_t round_cnt[kKeysPerLane][kOneGroups];  // this block's keys per 64-row round
@@ -348,7 +350,7 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
     }
     const int count = before + rest;
     const int ntile = (count + kTileRows - 1) / kTileRows;
-    const int nchunk = (ntile + kChunkTiles - 1) / kChunkTiles;
+    const int nchunk = (ntile + chunk_tiles - 1) / chunk_tiles;
     const int npart = nchunk > 1 ? nchunk : 0;
     int v[4] = {count, ntile, nchunk, npart}, excl[4], total[4];
 #pragma unroll
@@ -439,8 +441,8 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
       const int j = i - cfirst[g];
       const int ntile = tfirst[g + 1] - tfirst[g];
       c.group = g;
-      c.tile0 = tfirst[g] + j * kChunkTiles;
-      c.ntiles = min(kChunkTiles, ntile - j * kChunkTiles);
+      c.tile0 = tfirst[g] + j * chunk_tiles;
+      c.ntiles = min(chunk_tiles, ntile - j * chunk_tiles);
       c.partial = cfirst[g + 1] - cfirst[g] > 1 ? pfirst[g] + j : -1;
     }
     V.chunks[i] = c;
@@ -521,10 +523,12 @@ int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t 
   if (groups <= kOneGroups && nblk <= kOneBlocks) {
     if (key_dtype == TK_KEY_I32)
       hipLaunchKernelGGL(k_seg_one<int32_t>, dim3(nblk), dim3(kOneWaves * 64), 0, s, (const int32_t*)keys, (int)rows,
-                         groups, key_bits, nblk, (int)L.max_tiles, (int)L.max_chunks, V, perm_out, offsets_out);
+                         groups, key_bits, nblk, (int)L.max_tiles, (int)L.max_chunks, (int)L.chunk_tiles, V, perm_out,
+                         offsets_out);
     else
       hipLaunchKernelGGL(k_seg_one<int64_t>, dim3(nblk), dim3(kOneWaves * 64), 0, s, (const int64_t*)keys, (int)rows,
-                         groups, key_bits, nblk, (int)L.max_tiles, (int)L.max_chunks, V, perm_out, offsets_out);
+                         groups, key_bits, nblk, (int)L.max_tiles, (int)L.max_chunks, (int)L.chunk_tiles, V, perm_out,
+                         offsets_out);
     return check_launch();
   }
   if (key_dtype == TK_KEY_I32)
@@ -534,7 +538,7 @@ int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t 
     hipLaunchKernelGGL(k_seg_hist<int64_t>, dim3(nblk), dim3(64), lds, s, (const int64_t*)keys, (int)rows, groups,
                        key_bits, V.hist, V.bad);
   hipLaunchKernelGGL(k_seg_scan, dim3(1), dim3(1024), 0, s, (int)rows, groups, nblk, (int)L.max_tiles,
-                     (int)L.max_chunks, V, offsets_out);
+                     (int)L.max_chunks, (int)L.chunk_tiles, V, offsets_out);
   if (key_dtype == TK_KEY_I32)
     hipLaunchKernelGGL(k_seg_scatter<int32_t>, dim3(nblk), dim3(64), lds, s, (const int32_t*)keys, (int)rows, groups,
                        key_bits, V, perm_out);

@@ -10,7 +10,8 @@ namespace tk {
 
 constexpr int kWave = 64;
 constexpr int kTileRows = TK_TILE_ROWS;    // rows per forward tile (two 16-row MFMA tiles)
-constexpr int kChunkRows = TK_CHUNK_ROWS;  // rows per weight-gradient chunk (split over rows)
+constexpr int kChunkTilesMin = TK_CHUNK_ROWS / TK_TILE_ROWS;  // smallest weight-gradient chunk: 16 tiles (512 rows)
+constexpr int kChunkTilesMax = 128;                             // largest: 4096 rows
 constexpr int kSortBlockRows = 512;        // rows one single-wave block orders in the scatter pass
 
 static inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
@@ -36,18 +37,28 @@ struct SegHeader {       // 64 x int32, at the start of the workspace
   int32_t pad[57];
 };
 
-struct ChunkInfo {  // one weight-gradient chunk: tiles [tile0, tile0 + ntiles) of group `group`
+struct ChunkInfo {  // one weight-gradient chunk: tiles [tile0, tile0 + ntiles) of group `group`, ntiles <= chunk_tiles
   int32_t group;
   int32_t tile0;
   int32_t ntiles;
   int32_t partial;  // slot in the partial buffer, or -1 when the chunk is its group's only one
 };
 
-constexpr int kChunkTiles = kChunkRows / kTileRows;
+// A chunk is the unit the row contractions (dA, dB) are split into: up to `chunk_tiles` tiles of one
+// group.  Every chunk of a multi-chunk group costs one fp32 partial of rank x width, so the chunk
+// grows with the batch (about 32 chunks over all rows): the partial traffic stays a fixed small
+// fraction of the activations while the number of work items stays in the thousands.  A function
+// of the row count alone, so producer and consumers agree.
+static inline int chunk_tiles_for(int64_t rows) {
+  int t = kChunkTilesMin;
+  while (t < kChunkTilesMax && (int64_t)t * kTileRows * 32 < rows) t <<= 1;
+  return t;
+}
 
 struct SegLayout {
   int64_t rows, groups;
   int64_t sort_blocks;   // ceil(rows / kSortBlockRows)
+  int64_t chunk_tiles;   // tiles per weight-gradient chunk (chunk_tiles_for(rows))
   int64_t max_tiles, max_chunks, max_partials;
   int64_t slots;         // padded sorted length: 32 * max_tiles
   // byte offsets from the workspace base
@@ -57,8 +68,9 @@ struct SegLayout {
   SegLayout(int64_t rows_, int64_t groups_) : rows(rows_), groups(groups_) {
     sort_blocks = ceil_div(rows > 0 ? rows : 1, kSortBlockRows);
     max_tiles = ceil_div(rows, kTileRows) + groups;
-    max_chunks = ceil_div(rows, kChunkRows) + groups;
-    max_partials = 2 * ceil_div(rows, kChunkRows) + 1;
+    chunk_tiles = chunk_tiles_for(rows);
+    max_chunks = ceil_div(rows, chunk_tiles * kTileRows) + groups;
+    max_partials = 2 * ceil_div(rows, chunk_tiles * kTileRows) + 1;
     slots = max_tiles * kTileRows;
     int64_t o = round_up(sizeof(SegHeader), 256);
     off_inv = o;           o += round_up(4 * (rows + 64), 256);
