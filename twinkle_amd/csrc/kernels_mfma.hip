@@ -795,16 +795,25 @@ __global__ __launch_bounds__(256) void k_dy_fused(WgradArgs a, const void* const
 #pragma unroll
   for (int q = 0; q < 8; ++q) acc[q][0] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  auto issue = [&](int t, uint4 (&x)[8], uint4& h) {
-    const bool tok = t < nt;  // block-uniform
-    const int4 ra = tok ? *reinterpret_cast<const int4*>(rows_s + t * kTileRows + 8 * kb) : make_int4(-1, -1, -1, -1);
-    const int4 rb = tok ? *reinterpret_cast<const int4*>(rows_s + t * kTileRows + 8 * kb + 4) : make_int4(-1, -1, -1, -1);
+  // loads are unconditional (tiles past the end re-read the last one, padding slots read row 0) and what
+  // must not count is zeroed when it is consumed: no branch between a load and its use
+  auto issue = [&](int t, uint4 (&x)[8], uint4& h, uint32_t& live) {
+    const int tc = min(t, nt - 1);
+    const int4 ra = *reinterpret_cast<const int4*>(rows_s + tc * kTileRows + 8 * kb);
+    const int4 rb = *reinterpret_cast<const int4*>(rows_s + tc * kTileRows + 8 * kb + 4);
     const int rows[8] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w};
+    live = 0;
 #pragma unroll
-    for (int q = 0; q < 8; ++q) x[q] = rows[q] >= 0 ? ld16(src + (int64_t)rows[q] * a.ld_src) : zero4();
-    h = tok ? ld16(hT + t * kTileRows) : zero4();
+    for (int q = 0; q < 8; ++q) {
+      x[q] = ld16(src + (int64_t)max(rows[q], 0) * a.ld_src);
+      live |= (t < nt && rows[q] >= 0) ? (1u << q) : 0u;
+    }
+    h = ld16(hT + tc * kTileRows);
   };
-  auto consume = [&](int t, const uint4 (&x)[8], const uint4& h) {
+  auto consume = [&](int t, uint4 (&x)[8], const uint4& h, uint32_t live) {
+#pragma unroll
+    for (int q = 0; q < 8; ++q)
+      if (!((live >> q) & 1u)) x[q] = zero4();
     // the piece in row-major order for the dh product
 #pragma unroll
     for (int q = 0; q < 8; ++q) st16(my_stage + (8 * kb + q) * SS + 8 * li, x[q]);
@@ -852,15 +861,19 @@ __global__ __launch_bounds__(256) void k_dy_fused(WgradArgs a, const void* const
   };
 
   uint4 xa[8], xb[8], ha, hb;
-  issue(0, xa, ha);
-  for (int t = 0; t < nt; t += 2) {
-    issue(t + 1, xb, hb);
-    consume(t, xa, ha);
-    if (t + 1 < nt) {
-      issue(t + 2, xa, ha);
-      consume(t + 1, xb, hb);
-    }
+  uint32_t la, lb;
+  issue(0, xa, ha, la);
+  int t = 0;
+  for (; t + 2 < nt; t += 2) {  // every tile touched in here exists
+    issue(t + 1, xb, hb, lb);
+    consume(t, xa, ha, la);
+    issue(t + 2, xa, ha, la);
+    consume(t + 1, xb, hb, lb);
   }
+  // one or two tiles are left
+  issue(t + 1, xb, hb, lb);
+  consume(t, xa, ha, la);
+  if (t + 1 < nt) consume(t + 1, xb, hb, lb);
   // every wave has its own 128 columns of dB
   wgrad_store<1>(acc, reinterpret_cast<float*>(my_stage), a, ci, g, r, c0, lane);
 }
