@@ -126,7 +126,7 @@ __global__ __launch_bounds__(NW * 64) void k_shrink_mfma(PassArgs a, bf16_t* __r
                                                          const int32_t* __restrict__ slot_rows) {
   constexpr int RP = 16 * NB;  // padded rank
   constexpr int PR = RP + 1;   // row stride of the partial sums (floats; odd: conflict-free column reads)
-  constexpr int PF = 4;        // steps whose loads are issued together
+  constexpr int PF = NB >= 4 ? 2 : 4;  // steps whose loads are issued together (fewer at rank 64: registers)
   __shared__ float part[NW][kTileRows][PR];
 
   const int kslices = a.kslices;
