@@ -213,9 +213,9 @@ def main():
                                '; step = segment build + LoRA fwd + LoRA bwd (dX, dA, dB); base GEMM excluded',
                    'tokens': T, 'in': K, 'out': M, 'adapters': G, 'rank': max(w.ranks)},
         'roofline': {'bound': 'hbm', 'achieved': achieved, 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                     'frac': achieved / HBM_PEAK_GBS, 'traffic': measured_traffic('k_expand_mfma<1, 1>') if args.workload == 'cfg2' else None,
-                     'kernel': f'k_expand_mfma<{max(1, (max(w.ranks) + 15) // 16 if max(w.ranks) <= 32 else 4)},1> '
-                               '(y += h B^T in place), forward launch',
+                     'frac': achieved / HBM_PEAK_GBS, 'traffic': measured_traffic('k_expand_mfma<1>') if args.workload == 'cfg2' else None,
+                     'kernel': ('k_expand_mfma<1>' if max(w.ranks) <= 16 else
+                                f'k_expand_multi<{2 if max(w.ranks) <= 32 else 4},4>') + ' (y += h B^T in place), forward launch',
                      'algorithmic_bytes_per_launch': expand_bytes, 'avg_launch_ms': expand_ms,
                      'launches_timed': len(events)},
         'step_detail': {'shrink_ms': shrink_ms, 'expand_ms': expand_ms, 'fwd_ms': fwd_ms, 'bwd_ms': bwd_ms, 'segment_build_and_gaps_ms': ms_per_step - fwd_ms - bwd_ms,

@@ -190,7 +190,6 @@ static int lora_pass_fwd(const tk_lora_desc* d, const void* x, int64_t ldx, void
   a.width_src = d->in_features;  a.width_dst = d->out_features;
   a.map_rows = d->map_rows;  a.rpad = rank_pad(d->max_rank);  a.src_rows = (int32_t)d->rows;
   a.hpart = (float*)((char*)h + round_up(2 * (int64_t)a.rpad * a.ldh * elt_bytes(d->dtype), 256));
-  a.tile_ticket = V.tile_ticket;
   a.kslices = shrink_kslices(d->in_features, a.rpad);
   return run_pass(a, V, L, d->dtype, phases, (hipStream_t)stream);
 }
@@ -255,7 +254,6 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
   a.width_src = d->out_features;  a.width_dst = d->in_features;
   a.map_rows = d->map_rows;  a.rpad = (int32_t)B.rpad;  a.src_rows = (int32_t)d->rows;
   a.hpart = (float*)(w + B.off_hpart);
-  a.tile_ticket = V.tile_ticket;
   a.kslices = shrink_kslices(d->out_features, a.rpad);
   const bool mfma = d->dtype == TK_DTYPE_BF16 && !force_generic();
   TransposeJob tr{};

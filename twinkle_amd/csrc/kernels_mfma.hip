@@ -268,15 +268,16 @@ __global__ __launch_bounds__(256) void k_shrink_finish(PassArgs a, bf16_t* __res
 
 // ---------------------------------------------------------------------------
 // Expand: dst[row(slot)][c] += sum_n h[slot][n] * W2_g[c][n], read-modify-write
-// in place.  Work is flat: one wave owns CPW adjacent 128-column groups of one
-// tile and nothing is shared between waves, so the grid is thousands of
-// independent streams.  Column c0 + 8 j + q of a group is output column j of
-// MFMA q, which makes each lane's 8 results of one row 16 contiguous bytes and
-// each wave-wide access 4 rows x 256 B.  Row indices, h and the group id are
-// addressed from the work-item number alone, so the destination loads are one
-// dependent step away from the start of the wave.
+// in place.  Work is flat: one wave owns one 128-column group of one tile and
+// nothing is shared between waves, so the grid is thousands of independent
+// streams.  Column c0 + 8 j + q of a group is output column j of MFMA q, which
+// makes each lane's 8 results of one row 16 contiguous bytes and each wave-wide
+// access 4 rows x 256 B.  Row indices, h and the group id are addressed from the
+// work-item number alone, so the destination loads are one dependent step away
+// from the start of the wave.  (Used for padded rank 16; above that
+// k_expand_multi shares the weight block between tiles.)
 // ---------------------------------------------------------------------------
-template <int NB, int CPW>
+template <int NB>
 __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* __restrict__ hrow,
                                                      const int32_t* __restrict__ tile_group,
                                                      const int32_t* __restrict__ slot_rows, int num_items) {
@@ -284,11 +285,10 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
   constexpr int NKS = (RP + 31) / 32;  // contraction steps of the MFMAs
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
   const int ngroups = a.width_dst >> 7;
-  const int items_per_tile = (ngroups + CPW - 1) / CPW;
   const int item = blockIdx.x * 4 + wave;
   if (item >= num_items) return;
-  const int tile_id = item / items_per_tile;
-  const int cg0 = (item - tile_id * items_per_tile) * CPW;
+  const int tile_id = item / ngroups;
+  const int c0 = (item - tile_id * ngroups) << 7;
   const int slot0 = tile_id * kTileRows;
   // independent first loads: group id, row indices, h operand (nothing branches before the
   // destination loads are in flight)
@@ -308,64 +308,45 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
   const int rows[2][4] = {{r0.x, r0.y, r0.z, r0.w}, {r1.x, r1.y, r1.z, r1.w}};
   bool rok[2][4];
   bf16_t* yp[2][4];
+  uint4 y[2][4];
 #pragma unroll
   for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       rok[tt][v] = g_raw >= 0 && rows[tt][v] >= 0;
-      yp[tt][v] = (bf16_t*)a.dst + (int64_t)(rok[tt][v] ? rows[tt][v] : 0) * a.ld_dst + 8 * li;
+      yp[tt][v] = (bf16_t*)a.dst + (int64_t)(rok[tt][v] ? rows[tt][v] : 0) * a.ld_dst + 8 * li + c0;
+      y[tt][v] = rok[tt][v] ? ld16_nt(yp[tt][v]) : zero4();
     }
   const int r = g_raw < 0 ? 0 : min(a.rank[g], RP);
   const bf16_t* W2 = group_weight<bf16_t>(a.w_expand, a.w_expand_base, a.expand_group_stride, g);
-
-  // Two register buffers: the loads of column group u + 1 are issued before group u is consumed, so a
-  // wave always has a group's worth of loads (8 KB of dst, 4 KB of weights) in flight.
-  uint4 y[2][2][4];
-  uint4 bq[2][8][NKS];
-  auto issue = [&](int u, int buf) {
-    const bool gok = cg0 + u < ngroups;  // wave-uniform
-    const int c0 = (gok ? cg0 + u : cg0) << 7;
+  uint4 bq[8][NKS];
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
+  for (int q = 0; q < 8; ++q)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) y[buf][tt][v] = (rok[tt][v] && gok) ? ld16_nt(yp[tt][v] + c0) : zero4();
-#pragma unroll
-    for (int q = 0; q < 8; ++q)
-#pragma unroll
-      for (int ks = 0; ks < NKS; ++ks) {
-        const int n0 = 32 * ks + 8 * kb;
-        bq[buf][q][ks] =
-            n0 < r ? keep_first(ld16(W2 + (int64_t)(c0 + 8 * li + q) * a.ld_expand + n0), r - n0) : zero4();
-      }
-  };
-  issue(0, 0);
+    for (int ks = 0; ks < NKS; ++ks) {
+      const int n0 = 32 * ks + 8 * kb;
+      bq[q][ks] = n0 < r ? keep_first(ld16(W2 + (int64_t)(c0 + 8 * li + q) * a.ld_expand + n0), r - n0) : zero4();
+    }
   if (r <= 0) return;  // unused tile, or adapter not live on this layer (uniform over the wave)
 #pragma unroll
-  for (int u = 0; u < CPW; ++u) {
-    if (cg0 + u >= ngroups) break;
-    const int buf = u & 1;
-    if (u + 1 < CPW) issue(u + 1, buf ^ 1);
-    const int c0 = (cg0 + u) << 7;
+  for (int tt = 0; tt < 2; ++tt) {
+    f32x4 d[8];
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-      f32x4 d[8];
+    for (int q = 0; q < 8; ++q) {
+      d[q] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        d[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int ks = 0; ks < NKS; ++ks) d[q] = mfma16(hop[tt][ks], bq[q][ks], d[q]);
+    }
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) d[q] = mfma16(hop[tt][ks], bq[buf][q][ks], d[q]);
-      }
-#pragma unroll
-      for (int v = 0; v < 4; ++v) {
-        if (!rok[tt][v]) continue;
-        const uint4 yy = y[buf][tt][v];
-        uint4 o;
-        o.x = pack_bf16(bf16_lo(yy.x) + d[0][v], bf16_hi(yy.x) + d[1][v]);
-        o.y = pack_bf16(bf16_lo(yy.y) + d[2][v], bf16_hi(yy.y) + d[3][v]);
-        o.z = pack_bf16(bf16_lo(yy.z) + d[4][v], bf16_hi(yy.z) + d[5][v]);
-        o.w = pack_bf16(bf16_lo(yy.w) + d[6][v], bf16_hi(yy.w) + d[7][v]);
-        st16_nt(yp[tt][v] + c0, o);
-      }
+    for (int v = 0; v < 4; ++v) {
+      if (!rok[tt][v]) continue;
+      const uint4 yy = y[tt][v];
+      uint4 o;
+      o.x = pack_bf16(bf16_lo(yy.x) + d[0][v], bf16_hi(yy.x) + d[1][v]);
+      o.y = pack_bf16(bf16_lo(yy.y) + d[2][v], bf16_hi(yy.y) + d[3][v]);
+      o.z = pack_bf16(bf16_lo(yy.z) + d[4][v], bf16_hi(yy.z) + d[5][v]);
+      o.w = pack_bf16(bf16_lo(yy.w) + d[6][v], bf16_hi(yy.w) + d[7][v]);
+      st16_nt(yp[tt][v], o);
     }
   }
 }
@@ -880,7 +861,7 @@ __global__ __launch_bounds__(256) void k_dy_fused(WgradArgs a, const void* const
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-template <int NB, int CPW>
+template <int NB>
 void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int phases, hipStream_t s) {
   bf16_t* hrow = (bf16_t*)a.hT + (int64_t)a.rpad * a.ldh;  // second half of the h buffer
   const int32_t* rows = seg.slot_table(a.map_rows);
@@ -893,16 +874,16 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
                        rows);
   if (!a.dst || !(phases & 2)) return;
   const int64_t ngroups = a.width_dst >> 7;
-  if (NB > 1) {
+  if constexpr (NB > 1) {
     constexpr int TPI = 4;
     const int64_t blocks = ceil_div(L.max_tiles, TPI) * ceil_div(ngroups, 4);
     hipLaunchKernelGGL((k_expand_multi<NB, TPI>), dim3((unsigned)blocks), dim3(256), 0, s, a, hrow, seg.tile_group,
                        rows, (int)L.max_tiles);
-    return;
+  } else {
+    const int64_t items = L.max_tiles * ngroups;
+    hipLaunchKernelGGL((k_expand_mfma<NB>), dim3((unsigned)ceil_div(items, 4)), dim3(256), 0, s, a, hrow,
+                       seg.tile_group, rows, (int)items);
   }
-  const int64_t items = L.max_tiles * ceil_div(ngroups, CPW);
-  hipLaunchKernelGGL((k_expand_mfma<NB, CPW>), dim3((unsigned)ceil_div(items, 4)), dim3(256), 0, s, a, hrow,
-                     seg.tile_group, rows, (int)items);
 }
 
 template <int NB, int RS>
@@ -950,9 +931,9 @@ bool pass_mfma_supported(const PassArgs& a) {
 
 int launch_pass_mfma(const PassArgs& a, const SegView& seg, const SegLayout& L, int phases, hipStream_t s) {
   if (L.rows == 0) return TK_OK;
-  if (a.rpad <= 16) launch_pass<1, 1>(a, seg, L, phases, s);
-  else if (a.rpad <= 32) launch_pass<2, 1>(a, seg, L, phases, s);
-  else launch_pass<4, 1>(a, seg, L, phases, s);
+  if (a.rpad <= 16) launch_pass<1>(a, seg, L, phases, s);
+  else if (a.rpad <= 32) launch_pass<2>(a, seg, L, phases, s);
+  else launch_pass<4>(a, seg, L, phases, s);
   return check_launch();
 }
 

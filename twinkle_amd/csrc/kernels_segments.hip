@@ -206,7 +206,6 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
       valid = min(kTileRows, offs[g + 1] - pos0);       // padding is at the end of a group's last tile
     }
     V.tile_group[i] = g;
-    V.tile_ticket[i] = 0;
     int4* sp = reinterpret_cast<int4*>(V.slot_pos + (int64_t)i * kTileRows);
 #pragma unroll
     for (int j = 0; j < kTileRows; j += 4)
@@ -426,7 +425,6 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
       valid = min(kTileRows, offs[g + 1] - pos0);      // padding is at the end of a group's last tile
     }
     V.tile_group[i] = g;
-    V.tile_ticket[i] = 0;
     int4* sp = reinterpret_cast<int4*>(V.slot_pos + (int64_t)i * kTileRows);
 #pragma unroll
     for (int j = 0; j < kTileRows; j += 4)

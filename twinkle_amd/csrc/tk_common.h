@@ -63,7 +63,7 @@ struct SegLayout {
   int64_t slots;         // padded sorted length: 32 * max_tiles
   // byte offsets from the workspace base
   int64_t off_inv, off_slot_row, off_slot_pos, off_offsets, off_tile_group, off_chunks, off_tile_first,
-      off_chunk_first, off_partial_first, off_hist, off_bad, off_ticket, total;
+      off_chunk_first, off_partial_first, off_hist, off_bad, total;
 
   SegLayout(int64_t rows_, int64_t groups_) : rows(rows_), groups(groups_) {
     sort_blocks = ceil_div(rows > 0 ? rows : 1, kSortBlockRows);
@@ -84,7 +84,6 @@ struct SegLayout {
     off_partial_first = o; o += round_up(4 * (groups + 1), 256);
     off_hist = o;          o += round_up(4 * groups * sort_blocks, 256);
     off_bad = o;           o += round_up(4 * sort_blocks, 256);
-    off_ticket = o;        o += round_up(4 * (max_tiles + 1), 256);
     total = o;
   }
 };
@@ -102,7 +101,6 @@ struct SegView {  // typed device pointers into a segment workspace
   int32_t* partial_first;  // [G + 1]  first partial slot of each multi-chunk group
   int32_t* hist;           // [sort_blocks][G]  per-block histogram, then per-block exclusive bases
   int32_t* bad;            // [sort_blocks]  out-of-range keys seen by each block
-  int32_t* tile_ticket;    // [max_tiles]  arrival counters of the split shrink (zero between launches)
   SegView(const void* base, const SegLayout& L) {
     char* b = (char*)base;
     header = (SegHeader*)b;
@@ -117,7 +115,6 @@ struct SegView {  // typed device pointers into a segment workspace
     partial_first = (int32_t*)(b + L.off_partial_first);
     hist = (int32_t*)(b + L.off_hist);
     bad = (int32_t*)(b + L.off_bad);
-    tile_ticket = (int32_t*)(b + L.off_ticket);
   }
   // rows of the activation tensors, by padded slot
   const int32_t* slot_table(int map_rows) const { return map_rows ? slot_row : slot_pos; }
@@ -193,7 +190,6 @@ struct PassArgs {
   int32_t rpad;
   int32_t src_rows;  // rows of src / dst (bound for speculative row addresses)
   float* hpart;          // partial sums of the split shrink, [tile][slice][32][rpad]
-  int32_t* tile_ticket;  // arrival counter per tile
   int32_t kslices;       // blocks per tile of the MFMA shrink
 };
 
