@@ -308,18 +308,21 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
   const int rows[2][4] = {{r0.x, r0.y, r0.z, r0.w}, {r1.x, r1.y, r1.z, r1.w}};
   bool rok[2][4];
   bf16_t* yp[2][4];
-  uint4 y[2][4];
 #pragma unroll
   for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       rok[tt][v] = g_raw >= 0 && rows[tt][v] >= 0;
       yp[tt][v] = (bf16_t*)a.dst + (int64_t)(rok[tt][v] ? rows[tt][v] : 0) * a.ld_dst + 8 * li + c0;
-      y[tt][v] = rok[tt][v] ? ld16_nt(yp[tt][v]) : zero4();
     }
   const int r = g_raw < 0 ? 0 : min(a.rank[g], RP);
   const bf16_t* W2 = group_weight<bf16_t>(a.w_expand, a.w_expand_base, a.expand_group_stride, g);
+  uint4 y[2][4];
   uint4 bq[8][NKS];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) y[tt][v] = rok[tt][v] ? ld16_nt(yp[tt][v]) : zero4();
 #pragma unroll
   for (int q = 0; q < 8; ++q)
 #pragma unroll
