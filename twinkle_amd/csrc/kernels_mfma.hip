@@ -220,6 +220,138 @@ __global__ __launch_bounds__(NW * 64) void k_shrink_mfma(PassArgs a, bf16_t* __r
   shrink_epilogue<RP, NW * 64>(&part[0][0][0], NW, a, hrow, slot0, cnt, a.scale[g]);
 }
 
+// ---------------------------------------------------------------------------
+// Shrink for padded ranks above 16.  There the weight operands outnumber the source operands (at rank
+// 64 a 64-column step takes 8 weight loads for 4 source loads), and with one tile per block the load
+// pipeline, not memory, sets the pace.  A block here owns two consecutive tiles and the same slice of
+// columns, and every weight operand it loads feeds both tiles.  Consecutive tiles almost always
+// belong to the same group; a pair that straddles a group boundary is done one tile at a time.  Sums,
+// slices and the h layout are exactly those of k_shrink_mfma.
+// ---------------------------------------------------------------------------
+template <int NB, int NW, int TT>
+__device__ inline void shrink_tiles(const PassArgs& a, bf16_t* __restrict__ hrow, const int32_t* __restrict__ slot_rows,
+                                    const int (&tiles)[TT], int g, int ks, float (*part)[kTileRows][16 * NB + 1]) {
+  constexpr int RP = 16 * NB;
+  constexpr int PF = 2;  // steps whose loads are issued together
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  const bf16_t* src = (const bf16_t*)a.src;
+  const bf16_t *xa[TT], *xb[TT];
+  int cnt[TT];
+#pragma unroll
+  for (int u = 0; u < TT; ++u) {
+    const int slot0 = tiles[u] * kTileRows;
+    int ra = slot_rows[slot0 + li], rb = slot_rows[slot0 + 16 + li];
+    // padding is always at the end of a tile: count the valid slots
+    cnt[u] = __popcll(__ballot(ra >= 0) & 0xffffull) + __popcll(__ballot(rb >= 0) & 0xffffull);
+    ra = min(max(ra, 0), a.src_rows - 1);
+    rb = min(max(rb, 0), a.src_rows - 1);
+    xa[u] = src + (int64_t)ra * a.ld_src + 16 * kb;
+    xb[u] = src + (int64_t)rb * a.ld_src + 16 * kb;
+  }
+  const int r = min(a.rank[g], RP);
+  const bf16_t* W1 = group_weight<bf16_t>(a.w_shrink, a.w_shrink_base, a.shrink_group_stride, g);
+  const bf16_t* wp[NB];
+  bool wv[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int n = 16 * nb + li;
+    wv[nb] = n < r;
+    wp[nb] = W1 + (int64_t)(wv[nb] ? n : 0) * a.ld_shrink + 16 * kb;
+  }
+  f32x4 acc[TT][2][NB];
+#pragma unroll
+  for (int u = 0; u < TT; ++u)
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) acc[u][tt][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int nsteps = a.width_src >> 6;
+  const int s_first = ks * (kShrinkSteps * NW) + wave;
+#pragma unroll
+  for (int b = 0; b < kShrinkSteps / PF; ++b) {
+    uint4 x0[PF][TT][2], x1[PF][TT][2], w0[PF][NB], w1[PF][NB];
+#pragma unroll
+    for (int j = 0; j < PF; ++j) {
+      const int s = s_first + (b * PF + j) * NW;
+      const bool ok = s < nsteps;  // wave-uniform
+      const int c = (ok ? s : 0) << 6;
+#pragma unroll
+      for (int u = 0; u < TT; ++u) {
+        x0[j][u][0] = ld16(xa[u] + c);
+        x1[j][u][0] = ld16(xa[u] + c + 8);
+        x0[j][u][1] = ld16(xb[u] + c);
+        x1[j][u][1] = ld16(xb[u] + c + 8);
+      }
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        w0[j][nb] = (wv[nb] && ok) ? ld16(wp[nb] + c) : zero4();
+        w1[j][nb] = (wv[nb] && ok) ? ld16(wp[nb] + c + 8) : zero4();
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < PF; ++j)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int u = 0; u < TT; ++u)
+#pragma unroll
+          for (int tt = 0; tt < 2; ++tt) {
+            acc[u][tt][nb] = mfma16(x0[j][u][tt], w0[j][nb], acc[u][tt][nb]);
+            acc[u][tt][nb] = mfma16(x1[j][u][tt], w1[j][nb], acc[u][tt][nb]);
+          }
+  }
+  if (r <= 0) return;  // adapter not live on this layer (uniform over the block)
+  const float sc = a.scale[g];
+#pragma unroll
+  for (int u = 0; u < TT; ++u) {
+    __syncthreads();  // the previous tile's sums have been read
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) part[wave][16 * tt + 4 * kb + v][16 * nb + li] = acc[u][tt][nb][v];
+    __syncthreads();
+    if (a.kslices > 1) {
+      // the source is wider than one block: leave this block's sums for k_shrink_finish
+      float* mine = a.hpart + ((int64_t)tiles[u] * a.kslices + ks) * (kTileRows * RP);
+      for (int idx = tid; idx < kTileRows * RP; idx += NW * 64) {
+        const int row = idx / RP, n = idx % RP;
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) sum += part[w][row][n];
+        mine[idx] = sum;
+      }
+    } else {
+      shrink_epilogue<RP, NW * 64>(&part[0][0][0], NW, a, hrow, tiles[u] * kTileRows, cnt[u], sc);
+    }
+  }
+}
+
+template <int NB, int NW>
+__global__ __launch_bounds__(NW * 64) void k_shrink_pair(PassArgs a, bf16_t* __restrict__ hrow,
+                                                         const int32_t* __restrict__ tile_group,
+                                                         const int32_t* __restrict__ slot_rows, int max_tiles) {
+  __shared__ float part[NW][kTileRows][16 * NB + 1];
+  const int pair = blockIdx.x / a.kslices, ks = blockIdx.x - pair * a.kslices;
+  const int t0 = 2 * pair, t1 = t0 + 1;
+  const int g0 = tile_group[t0];
+  const int g1 = t1 < max_tiles ? tile_group[t1] : -1;
+  if (g0 >= 0 && g1 == g0) {
+    const int tiles[2] = {t0, t1};
+    shrink_tiles<NB, NW, 2>(a, hrow, slot_rows, tiles, g0, ks, part);
+    return;
+  }
+  if (g0 >= 0) {
+    const int tiles[1] = {t0};
+    shrink_tiles<NB, NW, 1>(a, hrow, slot_rows, tiles, g0, ks, part);
+  }
+  if (g1 >= 0) {
+    const int tiles[1] = {t1};
+    shrink_tiles<NB, NW, 1>(a, hrow, slot_rows, tiles, g1, ks, part);
+  }
+}
+
 // Adds the slices of a split shrink in slice order and writes h (one block per tile).
 template <int NB>
 __global__ __launch_bounds__(256) void k_shrink_finish(PassArgs a, bf16_t* __restrict__ hrow,
@@ -869,9 +1001,14 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
   bf16_t* hrow = (bf16_t*)a.hT + (int64_t)a.rpad * a.ldh;  // second half of the h buffer
   const int32_t* rows = seg.slot_table(a.map_rows);
   constexpr int NW = NB == 1 ? 1 : (NB == 2 ? 2 : 4);  // shrink_waves(16 * NB)
-  if (phases & 1)
-    hipLaunchKernelGGL((k_shrink_mfma<NB, NW>), dim3((unsigned)(L.max_tiles * a.kslices)), dim3(NW * 64), 0, s, a,
-                       hrow, seg.tile_group, rows);
+  if (phases & 1) {
+    if constexpr (NB > 1)
+      hipLaunchKernelGGL((k_shrink_pair<NB, NW>), dim3((unsigned)(ceil_div(L.max_tiles, 2) * a.kslices)), dim3(NW * 64),
+                         0, s, a, hrow, seg.tile_group, rows, (int)L.max_tiles);
+    else
+      hipLaunchKernelGGL((k_shrink_mfma<NB, NW>), dim3((unsigned)(L.max_tiles * a.kslices)), dim3(NW * 64), 0, s, a,
+                         hrow, seg.tile_group, rows);
+  }
   if ((phases & 5) && a.kslices > 1)
     hipLaunchKernelGGL((k_shrink_finish<NB>), dim3((unsigned)L.max_tiles), dim3(256), 0, s, a, hrow, seg.tile_group,
                        rows);
