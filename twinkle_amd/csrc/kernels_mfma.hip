@@ -102,131 +102,22 @@ __device__ inline void shrink_epilogue(const float* part, int planes, const Pass
 // ---------------------------------------------------------------------------
 // Shrink: h[slot][n] = scale_g * sum_k src[row(slot)][k] * W1_g[n][k].
 //
-// Work item = (tile of 32 padded slots, slice of 512*NW source columns), one
-// block of NW waves each; slices of one tile are consecutive blocks, so
-// neighbouring waves read neighbouring 1 KB pieces of the same rows.  The
-// grid is thousands of short independent streams: the hardware dispatcher
-// keeps every CU equally loaded, which a tile-per-workgroup split does not
-// (2.03 workgroups per CU leaves most CUs waiting for the few that got 3).
-// A wave takes 64-column steps, interleaved with the other waves of its
-// block, keeps its partial h[32][rank] in MFMA accumulators and issues the
-// loads of 4 steps before the first MFMA of the batch.  The waves' partials
-// meet in LDS; if the source is wider than one block the block sums go to a
-// global buffer and k_shrink_finish adds the slices in slice order (a device-
-// scope fence per block, the alternative, costs a cache write-back on this
-// multi-die part).  Summation order is fixed throughout: results are bitwise
-// repeatable.  The result is scaled, rounded
-// to bf16 and written twice: slot-major (hrow, the expand kernel's A operand)
-// and rank-major (hT, read by the weight-gradient kernel); padding slots get
-// exact zeros.  Nothing branches before the source loads are in flight.
-// ---------------------------------------------------------------------------
-template <int NB, int NW>
-__global__ __launch_bounds__(NW * 64) void k_shrink_mfma(PassArgs a, bf16_t* __restrict__ hrow,
-                                                         const int32_t* __restrict__ tile_group,
-                                                         const int32_t* __restrict__ slot_rows) {
-  constexpr int RP = 16 * NB;  // padded rank
-  constexpr int PR = RP + 1;   // row stride of the partial sums (floats; odd: conflict-free column reads)
-  constexpr int PF = NB >= 4 ? 2 : 4;  // steps whose loads are issued together (fewer at rank 64: registers)
-  __shared__ float part[NW][kTileRows][PR];
-
-  const int kslices = a.kslices;
-  const int tile_id = blockIdx.x / kslices, ks = blockIdx.x - tile_id * kslices;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
-  const int slot0 = tile_id * kTileRows;
-  // independent first loads (a tile of an unused table entry or of an adapter that is not live
-  // computes zeros and is dropped below)
-  const int g_raw = tile_group[tile_id];
-  int ra = slot_rows[slot0 + li], rb = slot_rows[slot0 + 16 + li];
-  const int g = max(g_raw, 0);
-  // padding is always at the end of a tile: count the valid slots
-  const int cnt = g_raw < 0 ? 0 : __popcll(__ballot(ra >= 0) & 0xffffull) + __popcll(__ballot(rb >= 0) & 0xffffull);
-  ra = min(max(ra, 0), a.src_rows - 1);
-  rb = min(max(rb, 0), a.src_rows - 1);
-  const int r = g_raw < 0 ? 0 : min(a.rank[g], RP);
-
-  const bf16_t* src = (const bf16_t*)a.src;
-  const bf16_t* xa = src + (int64_t)ra * a.ld_src + 16 * kb;
-  const bf16_t* xb = src + (int64_t)rb * a.ld_src + 16 * kb;
-  const bf16_t* W1 = group_weight<bf16_t>(a.w_shrink, a.w_shrink_base, a.shrink_group_stride, g);
-  const bf16_t* wp[NB];
-  bool wv[NB];
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb) {
-    const int n = 16 * nb + li;
-    wv[nb] = n < r;
-    wp[nb] = W1 + (int64_t)(wv[nb] ? n : 0) * a.ld_shrink + 16 * kb;
-  }
-  // two accumulators per output tile so that consecutive MFMAs are independent
-  f32x4 acc[2][NB][2];
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-      acc[0][nb][e] = f32x4{0.f, 0.f, 0.f, 0.f};
-      acc[1][nb][e] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-  const int nsteps = a.width_src >> 6;
-  const int s_first = ks * (kShrinkSteps * NW) + wave;
-#pragma unroll
-  for (int b = 0; b < kShrinkSteps / PF; ++b) {
-    uint4 xa0[PF], xa1[PF], xb0[PF], xb1[PF], w0[PF][NB], w1[PF][NB];
-#pragma unroll
-    for (int j = 0; j < PF; ++j) {
-      const int s = s_first + (b * PF + j) * NW;
-      const bool ok = s < nsteps;  // wave-uniform
-      const int c = (ok ? s : 0) << 6;
-      xa0[j] = ld16(xa + c);
-      xa1[j] = ld16(xa + c + 8);
-      xb0[j] = ld16(xb + c);
-      xb1[j] = ld16(xb + c + 8);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        w0[j][nb] = (wv[nb] && ok) ? ld16(wp[nb] + c) : zero4();
-        w1[j][nb] = (wv[nb] && ok) ? ld16(wp[nb] + c + 8) : zero4();
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < PF; ++j)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        acc[0][nb][0] = mfma16(xa0[j], w0[j][nb], acc[0][nb][0]);
-        acc[1][nb][0] = mfma16(xb0[j], w0[j][nb], acc[1][nb][0]);
-        acc[0][nb][1] = mfma16(xa1[j], w1[j][nb], acc[0][nb][1]);
-        acc[1][nb][1] = mfma16(xb1[j], w1[j][nb], acc[1][nb][1]);
-      }
-  }
-  if (r <= 0) return;  // unused tile, or adapter not live on this layer (uniform over the tile's blocks)
-#pragma unroll
-  for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int v = 0; v < 4; ++v)
-        part[wave][16 * tt + 4 * kb + v][16 * nb + li] = acc[tt][nb][0][v] + acc[tt][nb][1][v];
-  __syncthreads();
-
-  if (a.kslices > 1) {
-    // the source is wider than one block: leave this block's sums for k_shrink_finish
-    float* mine = a.hpart + ((int64_t)tile_id * kslices + ks) * (kTileRows * RP);
-    for (int idx = tid; idx < kTileRows * RP; idx += NW * 64) {
-      const int row = idx / RP, n = idx % RP;
-      float sum = 0.f;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) sum += part[w][row][n];
-      mine[idx] = sum;
-    }
-    return;
-  }
-  shrink_epilogue<RP, NW * 64>(&part[0][0][0], NW, a, hrow, slot0, cnt, a.scale[g]);
-}
-
-// ---------------------------------------------------------------------------
-// Shrink for padded ranks above 16.  There the weight operands outnumber the source operands (at rank
-// 64 a 64-column step takes 8 weight loads for 4 source loads), and with one tile per block the load
-// pipeline, not memory, sets the pace.  A block here owns two consecutive tiles and the same slice of
-// columns, and every weight operand it loads feeds both tiles.  Consecutive tiles almost always
-// belong to the same group; a pair that straddles a group boundary is done one tile at a time.  Sums,
-// slices and the h layout are exactly those of k_shrink_mfma.
+// Work item = (two consecutive tiles of 32 padded slots, slice of 512*NW source columns), one block of
+// NW waves; the slices of a tile pair are consecutive blocks, so neighbouring waves read neighbouring
+// 1 KB pieces of the same rows.  The grid is thousands of short independent streams: the hardware
+// dispatcher keeps every CU equally loaded, which a tile-per-workgroup split does not (2.03 workgroups
+// per CU leaves most CUs waiting for the few that got 3).  A wave takes 64-column steps, interleaved
+// with the other waves of its block, keeps its partial h[32][rank] of both tiles in MFMA accumulators
+// and issues the loads of two steps before the first MFMA of the batch.  Every weight operand feeds both
+// tiles: at rank 64 a step has 8 weight loads for 4 source loads per tile, and with one tile per block the
+// load pipeline, not memory, set the pace (rank 64: 129 -> 87 us; rank 16: 2 us).  Consecutive tiles
+// almost always belong to the same group; a pair that straddles a group boundary is done one tile at a
+// time.  The waves' partials meet in LDS; if the source is wider than one block the block sums go to
+// a global buffer and k_shrink_finish adds the slices in slice order (a device-scope fence per block,
+// the alternative, costs a cache write-back on this multi-die part).  Summation order is fixed
+// throughout: results are bitwise repeatable.  The result is scaled, rounded to bf16 and written
+// twice: slot-major (hrow, the expand kernel's A operand) and rank-major (hT, read by the
+// weight-gradient kernels); padding slots get exact zeros.
 // ---------------------------------------------------------------------------
 template <int NB, int NW, int TT>
 __device__ inline void shrink_tiles(const PassArgs& a, bf16_t* __restrict__ hrow, const int32_t* __restrict__ slot_rows,
@@ -1001,14 +892,9 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
   bf16_t* hrow = (bf16_t*)a.hT + (int64_t)a.rpad * a.ldh;  // second half of the h buffer
   const int32_t* rows = seg.slot_table(a.map_rows);
   constexpr int NW = NB == 1 ? 1 : (NB == 2 ? 2 : 4);  // shrink_waves(16 * NB)
-  if (phases & 1) {
-    if constexpr (NB > 1)
-      hipLaunchKernelGGL((k_shrink_pair<NB, NW>), dim3((unsigned)(ceil_div(L.max_tiles, 2) * a.kslices)), dim3(NW * 64),
-                         0, s, a, hrow, seg.tile_group, rows, (int)L.max_tiles);
-    else
-      hipLaunchKernelGGL((k_shrink_mfma<NB, NW>), dim3((unsigned)(L.max_tiles * a.kslices)), dim3(NW * 64), 0, s, a,
-                         hrow, seg.tile_group, rows);
-  }
+  if (phases & 1)
+    hipLaunchKernelGGL((k_shrink_pair<NB, NW>), dim3((unsigned)(ceil_div(L.max_tiles, 2) * a.kslices)), dim3(NW * 64), 0,
+                       s, a, hrow, seg.tile_group, rows, (int)L.max_tiles);
   if ((phases & 5) && a.kslices > 1)
     hipLaunchKernelGGL((k_shrink_finish<NB>), dim3((unsigned)L.max_tiles), dim3(256), 0, s, a, hrow, seg.tile_group,
                        rows);
