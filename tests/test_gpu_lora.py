@@ -340,3 +340,19 @@ def test_hip_graph_replay_matches_eager(dev, max_r, ranks):
             got_a, ref_a = groups.grad_views(ga, 'a')[g], groups.grad_views(want[2], 'a')[g]
             got_b, ref_b = groups.grad_views(gb, 'b')[g], groups.grad_views(want[3], 'b')[g]
             assert torch.equal(got_a[:r], ref_a[:r]) and torch.equal(got_b[:, :r], ref_b[:, :r])
+
+
+@pytest.mark.parametrize('dtype,t,k,m,max_r,ranks', [
+    (torch.bfloat16, 20000, 128, 1024, 16, [16, 5, 16]),    # 32-tile chunks, single pass over dy
+    (torch.bfloat16, 40000, 128, 256, 64, [64, 17, 40]),    # 64-tile chunks, rank indices split over two waves
+    (torch.float32, 17000, 24, 40, 8, [8, 3]),              # generic kernels walk a chunk in passes of 512 slots
+])
+def test_chunks_larger_than_512_rows(dev, dtype, t, k, m, max_r, ranks):
+    """Above 16384 rows a chunk of the row contractions holds 32 or more tiles; groups span several such chunks."""
+    n = len(ranks)
+    x, base, dy, a, b, _, _, scales = _problem(t, k, m, n, max_r, ranks, seed=t)
+    ids = torch.zeros(t, dtype=torch.long)
+    ids[: t // 7] = 1 % n
+    ids[t // 7: t // 7 + 50] = n - 1          # one group far smaller than a chunk
+    ids = ids[torch.randperm(t, generator=torch.Generator().manual_seed(1))]
+    _run(dev, dtype, x, base, dy, a, b, ids, ranks, scales)
