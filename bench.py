@@ -65,6 +65,42 @@ def cpu_baseline(w, budget_s=15.0):
     }
 
 
+def torch_gpu_loop(w, dev, dt, steps=5):
+    """What the reference does today, on the same GPU: tenants one after the other, two F.linear per tenant on the
+    tenant's rows (index_select / index_add_) and stock autograd.  Plain torch ops, no kernel of this library."""
+    import torch
+    import torch.nn.functional as F
+    x = w.x.to(dt).to(dev).requires_grad_(True)
+    base = w.base_out.to(dt).to(dev)
+    dy = w.dy.to(dt).to(dev)
+    ids = w.ids.to(dev)
+    a = [t.to(dt).to(dev).requires_grad_(True) for t in w.lora_A]
+    b = [t.to(dt).to(dev).requires_grad_(True) for t in w.lora_B]
+    rows = [torch.nonzero(ids == g).flatten() for g in range(w.num_adapters)]
+
+    def one():
+        y = base.clone()
+        for g in range(w.num_adapters):
+            r = w.ranks[g]
+            if rows[g].numel() == 0 or r == 0:
+                continue
+            xg = x.index_select(0, rows[g])
+            y = y.index_add(0, rows[g], F.linear(F.linear(xg, a[g][:r]), b[g][:, :r]) * w.scales[g])
+        y.backward(dy)
+        for t in [x] + a + b:
+            t.grad = None
+
+    one()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / steps
+    return {'value': w.tokens / (ms * 1e-3), 'unit': 'tokens/s', 'ms_per_step': ms,
+            'kind': 'per-adapter F.linear loop with index_select / index_add_ and autograd on the same GPU (torch ops only)'}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -227,6 +263,7 @@ def main():
                         'base_gemm_ms_excluded': base_ms},
     }
     if not args.no_cpu_baseline:
+        out['torch_gpu_loop'] = torch_gpu_loop(w, dev, dt)
         out['cpu_baseline'] = cpu_baseline(w)
     print(json.dumps(out))
 
