@@ -160,6 +160,58 @@ int tk_lora_bwd(const tk_lora_desc* desc, const void* dy_device, int64_t lddy, c
                 const void* h_device, void* dx_device, int64_t lddx, void* const* grad_A, void* const* grad_B,
                 int32_t accumulate, void* workspace_device, int64_t workspace_bytes, tk_stream_t stream);
 
+/* ---------------------------------------------------------------------------
+ * Multi-tenant optimizer step over adapter tensors (one launch set for all tenants).
+ *
+ * What the reference does per tenant, one tenant at a time (src/twinkle/model/transformers/transformers.py):
+ * clip_grad_norm (:732-778) divides the tenant's gradients by its token count and clips their total norm
+ * (src/twinkle/utils/grad_clip.py:31-96, torch.nn.utils.clip_grad_norm_ on one GPU), step (:835-876) runs
+ * torch.optim.AdamW / Adam with per-call lr / weight_decay / eps / betas, zero_grad (:879-894) clears the
+ * gradients.  Here every tensor carries its tenant's index and the tenants' numbers sit in one table.
+ * ------------------------------------------------------------------------- */
+typedef struct tk_opt_tensor { /* one contiguous parameter tensor of one tenant (device pointers) */
+  void* param;                 /* dtype given per call */
+  void* grad;                  /* same dtype and size */
+  float* exp_avg;              /* fp32 first moment, numel floats */
+  float* exp_avg_sq;           /* fp32 second moment */
+  int64_t numel;
+  int32_t tenant;              /* row of the tenant table */
+  int32_t reserved;
+} tk_opt_tensor;
+
+typedef struct tk_opt_tenant { /* one row of the tenant table */
+  float lr, beta1, beta2, eps, weight_decay;
+  float one_minus_beta1;       /* 1 - beta1 and 1 - beta2, rounded from double by the caller: formed in fp32 from */
+  float one_minus_beta2;       /* the rounded betas they would be off by 1e-5 relative (beta2 = 0.999) */
+  float bias_correction1;      /* 1 - beta1^step, computed in double by the caller (as torch does) */
+  float bias_correction2_sqrt; /* sqrt(1 - beta2^step) */
+  float grad_scale;            /* 1 / num_tokens (grad_clip.py:81-96: gradients are divided by the token count) */
+  float max_grad_norm;         /* <= 0: no clipping */
+  float norm_type;             /* 2, or +infinity for the max norm */
+  int32_t active;              /* 0: the tenant's tensors are skipped (no step for it this time) */
+  int32_t reserved;
+} tk_opt_tenant;
+
+#define TK_OPT_WRITE_GRADS 1 /* leave the normalised, clipped gradients in grad (what the reference's grads hold) */
+#define TK_OPT_ZERO_GRADS 2  /* clear grad in the same pass (the reference's zero_grad after step) */
+
+/* Bytes of scratch for tk_opt_grad_norm. */
+int64_t tk_opt_workspace_bytes(int32_t num_tensors, int64_t max_numel);
+
+/* norm_out[t] = norm of tenant t's gradients after division by its token count, before clipping (the value
+ * clip_grad_norm returns); clip_out[t] = min(1, max_grad_norm / (norm + 1e-6)), 1 without clipping.  Both are
+ * device arrays [num_tenants]; tensors_device / tenants_device are device arrays; no host synchronisation.
+ * Sums run in a fixed order: bitwise repeatable. */
+int tk_opt_grad_norm(const tk_opt_tensor* tensors_device, int32_t num_tensors, const tk_opt_tenant* tenants_device,
+                     int32_t num_tenants, int64_t max_numel, int32_t dtype, float* norm_out, float* clip_out,
+                     void* workspace_device, int64_t workspace_bytes, tk_stream_t stream);
+
+/* AdamW (decoupled weight decay; weight_decay = 0 gives Adam) on every active tenant's tensors with
+ * g' = grad * grad_scale * clip[t] (clip_device may be NULL: no clipping).  fp32 arithmetic and moments. */
+int tk_opt_adamw_step(const tk_opt_tensor* tensors_device, int32_t num_tensors, const tk_opt_tenant* tenants_device,
+                      int32_t num_tenants, int64_t max_numel, int32_t dtype, const float* clip_device, int32_t flags,
+                      tk_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

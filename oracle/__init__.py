@@ -28,6 +28,9 @@ expert_delta_weight / expert_lora_low_rank                 : pinned
 packed_cu_seqlens                                          : pinned (brute force)
 slice_rank_tensor / copy_rank_tensor / match_target_modules : pinned
     (round-trip + hand-written cases from the reference's comments)
+normalize_and_clip_grad_norm / TenantAdamW (oracle/optim.py)  : pinned
+    (they are torch.nn.utils.clip_grad_norm_ and torch.optim.AdamW themselves, the
+    library routines the reference calls; one step also checked against the closed form)
 PEFT-side container behaviour (attribute names, adapter dtype autocast)
     : parity unpinned — PEFT is absent from this image; affects dtypes at the
     boundary, not the arithmetic.
@@ -43,6 +46,7 @@ from .segments import (  # noqa: F401
     unpermute,
     unpermute_rows,
 )
+from .optim import TenantAdamW, normalize_and_clip_grad_norm, trainable_parameter_names  # noqa: F401
 from .lora import (  # noqa: F401
     copy_rank_tensor,
     expert_delta_weight,

@@ -11,6 +11,7 @@ from .lora_layer import LoraConfig, LoraLinear, LoraModel, inject_adapter  # noq
 from .multi_lora import LoraTenant, MultiLora  # noqa: F401
 from .ops import (AdapterGroups, lora_bwd_, lora_bwd_workspace_bytes, lora_expand_, lora_fwd_,  # noqa: F401
                   lora_h_bytes, lora_shrink_, multi_lora_delta, multi_lora_linear)
+from .optim import MultiTenantAdamW, trainable_parameters  # noqa: F401
 from .segments import (SegmentTable, build_segments, flat_keys_from_topk, packed_cu_seqlens, permute,  # noqa: F401
                        token_groups_from_sequences, unpermute)
 

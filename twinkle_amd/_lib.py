@@ -69,6 +69,11 @@ EXPORTS = {
     'tk_lora_expand': (c_int32, [POINTER(LoraDesc), c_void_p, c_void_p, c_int64, c_void_p]),
     'tk_lora_bwd': (c_int32, [POINTER(LoraDesc), c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                               c_void_p, c_void_p, c_int32, c_void_p, c_int64, c_void_p]),
+    'tk_opt_workspace_bytes': (c_int64, [c_int32, c_int64]),
+    'tk_opt_grad_norm': (c_int32, [c_void_p, c_int32, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p,
+                                   c_int64, c_void_p]),
+    'tk_opt_adamw_step': (c_int32, [c_void_p, c_int32, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_int32,
+                                    c_void_p]),
 }
 
 _lib = None

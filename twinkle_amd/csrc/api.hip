@@ -312,4 +312,35 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
   return rc;
 }
 
+int64_t tk_opt_workspace_bytes(int32_t num_tensors, int64_t max_numel) {
+  if (num_tensors < 0 || max_numel < 0) return TK_ERR_INVALID;
+  return round_up(4 * opt_partial_floats(num_tensors, max_numel) + 4, 256);
+}
+
+static bool opt_args_ok(const tk_opt_tensor* tensors, int32_t num_tensors, const tk_opt_tenant* tenants,
+                        int32_t num_tenants, int64_t max_numel, int32_t dtype) {
+  if (num_tensors < 0 || num_tenants <= 0 || max_numel < 0) return false;
+  if (num_tensors > 0 && (!tensors || !tenants)) return false;
+  if (num_tensors > 65535) return false;  // grid.y
+  return dtype == TK_DTYPE_F32 || dtype == TK_DTYPE_BF16;
+}
+
+int tk_opt_grad_norm(const tk_opt_tensor* tensors, int32_t num_tensors, const tk_opt_tenant* tenants,
+                     int32_t num_tenants, int64_t max_numel, int32_t dtype, float* norm_out, float* clip_out,
+                     void* ws, int64_t ws_bytes, tk_stream_t stream) {
+  if (!opt_args_ok(tensors, num_tensors, tenants, num_tenants, max_numel, dtype) || !tenants || !norm_out || !clip_out)
+    return TK_ERR_INVALID;
+  if (!ws || ws_bytes < tk_opt_workspace_bytes(num_tensors, max_numel)) return TK_ERR_WORKSPACE;
+  return launch_opt_grad_norm(tensors, num_tensors, tenants, num_tenants, max_numel > 0 ? max_numel : 1, dtype, norm_out,
+                              clip_out, (float*)ws, (hipStream_t)stream);
+}
+
+int tk_opt_adamw_step(const tk_opt_tensor* tensors, int32_t num_tensors, const tk_opt_tenant* tenants,
+                      int32_t num_tenants, int64_t max_numel, int32_t dtype, const float* clip, int32_t flags,
+                      tk_stream_t stream) {
+  if (!opt_args_ok(tensors, num_tensors, tenants, num_tenants, max_numel, dtype)) return TK_ERR_INVALID;
+  if (num_tensors == 0 || max_numel == 0) return TK_OK;
+  return launch_opt_adamw(tensors, num_tensors, tenants, max_numel, dtype, clip, flags, (hipStream_t)stream);
+}
+
 }  // extern "C"

@@ -241,6 +241,13 @@ int launch_wgrad_reduce(const WgradArgs* a0, const WgradArgs* a1, const SegView&
                         hipStream_t s);
 int launch_transpose_weights(const tk_lora_desc& d, void* bT, void* aT, hipStream_t s);
 
+// kernels_optim.hip : multi-tenant gradient norm and AdamW
+int launch_opt_grad_norm(const tk_opt_tensor* tensors, int n_tensors, const tk_opt_tenant* tenants, int n_tenants,
+                         int64_t max_numel, int dtype, float* norm_out, float* clip_out, float* partial, hipStream_t s);
+int launch_opt_adamw(const tk_opt_tensor* tensors, int n_tensors, const tk_opt_tenant* tenants, int64_t max_numel,
+                     int dtype, const float* clip, int flags, hipStream_t s);
+int64_t opt_partial_floats(int n_tensors, int64_t max_numel);
+
 // kernels_mfma.hip : bf16, aligned shapes, MFMA
 bool pass_mfma_supported(const PassArgs& a);
 // `phases` (bit mask): 1 = shrink, 2 = expand (h already written), 4 = only the last step of a split shrink

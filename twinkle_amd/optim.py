@@ -1,0 +1,216 @@
+"""Per-tenant gradient normalisation, clipping and AdamW, stepped for all tenants at once.
+
+The reference keeps one ``torch.optim`` optimizer per tenant and walks the tenants one
+after the other: ``clip_grad_norm`` divides the tenant's gradients by its token count and
+clips their norm, ``step`` applies per-call lr / weight decay / eps / betas, ``zero_grad``
+clears them (src/twinkle/model/transformers/transformers.py:732-894,
+src/twinkle/utils/grad_clip.py:31-96).  With many small adapters that is thousands of tiny
+launches per training step.  Here every tenant's adapter tensors sit in one device table and
+three launches (two for the norms, one for the update) serve all tenants, each with its own
+token count, threshold and hyper-parameters (``tk_opt_grad_norm``, ``tk_opt_adamw_step``).
+Moments are fp32 whatever the parameter dtype; arithmetic is fp32.
+"""
+from __future__ import annotations
+
+import math
+import re
+from typing import Dict, Iterable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from . import _lib
+
+_TENSOR_DTYPE = np.dtype([('param', '<u8'), ('grad', '<u8'), ('exp_avg', '<u8'), ('exp_avg_sq', '<u8'),
+                          ('numel', '<i8'), ('tenant', '<i4'), ('reserved', '<i4')])
+_TENANT_DTYPE = np.dtype([('lr', '<f4'), ('beta1', '<f4'), ('beta2', '<f4'), ('eps', '<f4'), ('weight_decay', '<f4'),
+                          ('one_minus_beta1', '<f4'), ('one_minus_beta2', '<f4'), ('bias_correction1', '<f4'),
+                          ('bias_correction2_sqrt', '<f4'), ('grad_scale', '<f4'),
+                          ('max_grad_norm', '<f4'), ('norm_type', '<f4'), ('active', '<i4'), ('reserved', '<i4')])
+TK_OPT_WRITE_GRADS = 1
+TK_OPT_ZERO_GRADS = 2
+
+
+def trainable_parameters(model: torch.nn.Module, adapter_name: str) -> Dict[str, torch.nn.Parameter]:
+    """The parameters of one tenant's slot: names matching ``.lora_<x>.<adapter_name>`` (transformers.py:962-972)."""
+    pattern = re.compile(rf'\.lora_\w+\.{re.escape(adapter_name)}')
+    return {n: p for n, p in model.named_parameters() if p.requires_grad and pattern.search(n)}
+
+
+class _Tenant:
+
+    def __init__(self, index, params, lr, betas, eps, weight_decay):
+        self.index = index
+        self.params: List[torch.nn.Parameter] = list(params)
+        self.lr, self.betas, self.eps, self.weight_decay = float(lr), (float(betas[0]), float(betas[1])), float(eps), \
+            float(weight_decay)
+        self.step = 0
+        self.exp_avg: List[Optional[torch.Tensor]] = [None] * len(self.params)
+        self.exp_avg_sq: List[Optional[torch.Tensor]] = [None] * len(self.params)
+
+
+class MultiTenantAdamW:
+    """AdamW (``weight_decay=0``: Adam) for many tenants, one launch set per step."""
+
+    def __init__(self):
+        self._tenants: Dict[str, _Tenant] = {}
+        self._last_clip: Dict[torch.dtype, torch.Tensor] = {}
+        self._last_tables = None
+
+    # ---- tenant management -------------------------------------------------------------------------------
+    def add_tenant(self, name: str, params: Iterable[torch.nn.Parameter], lr: float = 1e-3, betas=(0.9, 0.999),
+                   eps: float = 1e-8, weight_decay: float = 1e-2) -> None:
+        """Register a tenant with its optimizer defaults (``torch.optim.AdamW``'s)."""
+        if name in self._tenants:
+            raise ValueError(f'tenant {name} already has an optimizer')
+        params = list(params)
+        for p in params:
+            if not p.is_cuda:
+                raise RuntimeError('optimizer parameters must live on the GPU: this path has no CPU implementation')
+            if p.dtype not in (torch.float32, torch.bfloat16):
+                raise ValueError(f'parameters must be float32 or bfloat16, got {p.dtype}')
+            if not p.is_contiguous():
+                raise ValueError('parameters must be contiguous')
+        self._tenants[name] = _Tenant(len(self._tenants), params, lr, betas, eps, weight_decay)
+
+    def remove_tenant(self, name: str) -> None:
+        """Drop a tenant and its state (slot released); the remaining tenants keep their rows."""
+        self._tenants.pop(name)
+        for i, t in enumerate(self._tenants.values()):
+            t.index = i
+
+    def tenants(self) -> List[str]:
+        return list(self._tenants)
+
+    def state(self, name: str):
+        t = self._tenants[name]
+        return {'step': t.step, 'exp_avg': t.exp_avg, 'exp_avg_sq': t.exp_avg_sq}
+
+    # ---- the step ----------------------------------------------------------------------------------------
+    def _tables(self, names: Sequence[str], num_tokens, max_grad_norm, norm_type, optim_params, advance: bool):
+        """Device tables per parameter dtype for the tenants in ``names``."""
+        names = list(names)
+        tenant_rows = np.zeros(len(self._tenants), dtype=_TENANT_DTYPE)
+        per_dtype: Dict[torch.dtype, list] = {}
+        keep = []
+        device = None
+        for name in names:
+            t = self._tenants[name]
+            over = (optim_params or {}).get(name) or {}
+            lr = float(over['lr']) if 'lr' in over else t.lr
+            # the reference only overrides a weight decay that was positive (transformers.py:862-863)
+            wd = float(over['weight_decay']) if (t.weight_decay > 0.0 and over.get('weight_decay') is not None) \
+                else t.weight_decay
+            eps = float(over['eps']) if over.get('eps') is not None else t.eps
+            b1, b2 = over['betas'] if over.get('betas') is not None else t.betas
+            step = t.step + 1 if advance else max(t.step, 1)
+            tokens = int(num_tokens.get(name, 1)) if isinstance(num_tokens, dict) else int(num_tokens)
+            row = tenant_rows[t.index]
+            row['lr'], row['beta1'], row['beta2'], row['eps'], row['weight_decay'] = lr, b1, b2, eps, wd
+            row['one_minus_beta1'], row['one_minus_beta2'] = 1.0 - float(b1), 1.0 - float(b2)
+            row['bias_correction1'] = 1.0 - float(b1)**step
+            row['bias_correction2_sqrt'] = math.sqrt(1.0 - float(b2)**step)
+            row['grad_scale'] = 1.0 / tokens if tokens > 0 else 1.0   # grad_clip.py:83-84
+            row['max_grad_norm'] = max_grad_norm if max_grad_norm is not None else 0.0
+            row['norm_type'] = norm_type
+            row['active'] = 1
+            for i, p in enumerate(t.params):
+                if p.grad is None:
+                    continue  # torch optimizers skip parameters without a gradient
+                g = p.grad
+                if g.dtype != p.dtype or not g.is_contiguous() or g.shape != p.shape:
+                    g = g.to(p.dtype).contiguous()
+                    p.grad = g
+                if t.exp_avg[i] is None:
+                    t.exp_avg[i] = torch.zeros(p.shape, dtype=torch.float32, device=p.device)
+                    t.exp_avg_sq[i] = torch.zeros(p.shape, dtype=torch.float32, device=p.device)
+                device = p.device
+                per_dtype.setdefault(p.dtype, []).append(
+                    (p.data_ptr(), g.data_ptr(), t.exp_avg[i].data_ptr(), t.exp_avg_sq[i].data_ptr(), p.numel(),
+                     t.index, 0))
+                keep.append(g)
+        out = {}
+        if device is None:
+            return out, tenant_rows
+        tenants_dev = torch.from_numpy(tenant_rows.view(np.uint8).copy()).to(device)
+        for dtype, rows in per_dtype.items():
+            arr = np.array(rows, dtype=_TENSOR_DTYPE)
+            out[dtype] = (torch.from_numpy(arr.view(np.uint8).copy()).to(device), len(rows),
+                          int(arr['numel'].max()), tenants_dev, keep)
+        return out, tenant_rows
+
+    def clip_grad_norm(self, num_tokens, max_grad_norm: float = 1.0, norm_type: float = 2.0,
+                       names: Optional[Sequence[str]] = None) -> Dict[str, torch.Tensor]:
+        """Norm of every tenant's gradients after division by its token count (device scalars, no host
+        synchronisation), as ``clip_grad_norm`` returns it per tenant; the division and the clipping themselves
+        are applied inside :meth:`step`, which must follow (``clip_grad_and_step`` does both)."""
+        names = list(names) if names is not None else self.tenants()
+        tables, _ = self._tables(names, num_tokens, max_grad_norm, float(norm_type), None, advance=False)
+        lib = _lib.load()
+        norms: Dict[str, torch.Tensor] = {}
+        self._last_clip = {}
+        per_dtype_norms = []
+        for dtype, (tensors_dev, n, max_numel, tenants_dev, _keep) in tables.items():
+            nt = len(self._tenants)
+            norm = torch.empty(nt, dtype=torch.float32, device=tensors_dev.device)
+            clip = torch.empty(nt, dtype=torch.float32, device=tensors_dev.device)
+            nbytes = lib.tk_opt_workspace_bytes(n, max_numel)
+            _lib.check(nbytes, 'tk_opt_workspace_bytes')
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=tensors_dev.device)
+            code = lib.tk_opt_grad_norm(tensors_dev.data_ptr(), n, tenants_dev.data_ptr(), nt, max_numel,
+                                        _lib.dtype_code(dtype), norm.data_ptr(), clip.data_ptr(), ws.data_ptr(),
+                                        ws.numel(), _lib.stream_ptr())
+            _lib.check(code, 'tk_opt_grad_norm')
+            per_dtype_norms.append(norm)
+            self._last_clip[dtype] = clip
+        if len(per_dtype_norms) > 1:
+            # a tenant with parameters of both dtypes: combine the two partial norms and redo the coefficient
+            inf = math.isinf(float(norm_type))
+            total = torch.maximum(*per_dtype_norms) if inf else torch.sqrt(sum(v * v for v in per_dtype_norms))
+            clip = torch.clamp(max_grad_norm / (total + 1e-6), max=1.0) if max_grad_norm and max_grad_norm > 0 \
+                else torch.ones_like(total)
+            self._last_clip = {dtype: clip for dtype in self._last_clip}
+            per_dtype_norms = [total]
+        if per_dtype_norms:
+            for name in names:
+                norms[name] = per_dtype_norms[0][self._tenants[name].index]
+        return norms
+
+    def step(self, num_tokens=1, optim_params: Optional[Dict[str, dict]] = None,
+             names: Optional[Sequence[str]] = None, zero_grad: bool = False, write_grads: bool = False,
+             use_clip: bool = True) -> None:
+        """AdamW for the tenants in ``names`` (default: all), gradients divided by ``num_tokens`` (an int or a
+        dict per tenant) and scaled by the coefficients of the preceding :meth:`clip_grad_norm`.
+        ``optim_params[name]`` may carry ``lr``, ``weight_decay``, ``eps``, ``betas`` for this call
+        (transformers.py:857-868)."""
+        names = list(names) if names is not None else self.tenants()
+        tables, _ = self._tables(names, num_tokens, 0.0, 2.0, optim_params, advance=True)
+        lib = _lib.load()
+        flags = (TK_OPT_ZERO_GRADS if zero_grad else 0) | (TK_OPT_WRITE_GRADS if write_grads else 0)
+        for dtype, (tensors_dev, n, max_numel, tenants_dev, _keep) in tables.items():
+            clip = self._last_clip.get(dtype) if use_clip else None
+            code = lib.tk_opt_adamw_step(tensors_dev.data_ptr(), n, tenants_dev.data_ptr(), len(self._tenants),
+                                         max_numel, _lib.dtype_code(dtype),
+                                         clip.data_ptr() if clip is not None else None, flags, _lib.stream_ptr())
+            _lib.check(code, 'tk_opt_adamw_step')
+        self._last_tables = tables  # keeps the device tables alive until the next call (stream-ordered use)
+        self._last_clip = {}
+        for name in names:
+            self._tenants[name].step += 1
+
+    def clip_grad_and_step(self, num_tokens, max_grad_norm: float = 1.0, norm_type: float = 2.0,
+                           optim_params: Optional[Dict[str, dict]] = None,
+                           names: Optional[Sequence[str]] = None) -> Dict[str, torch.Tensor]:
+        """clip_grad_norm, step and zero_grad for every tenant in one go (transformers.py:781-785)."""
+        norms = self.clip_grad_norm(num_tokens, max_grad_norm, norm_type, names)
+        self.step(num_tokens, optim_params, names, zero_grad=True)
+        return norms
+
+    def zero_grad(self, names: Optional[Sequence[str]] = None, set_to_none: bool = True) -> None:
+        for name in (names if names is not None else self.tenants()):
+            for p in self._tenants[name].params:
+                if p.grad is not None:
+                    if set_to_none:
+                        p.grad = None
+                    else:
+                        p.grad.zero_()
