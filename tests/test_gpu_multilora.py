@@ -214,3 +214,52 @@ def test_mixed_dtype_base_bf16_adapters_fp32(dev):
                                       layer.lora_B['lora_0'].weight.detach().cpu(), 8, 2.0)
     assert want.dtype == torch.bfloat16
     assert max_rel_err(y, want) < 1e-2
+
+
+def test_batched_training_step_equals_tenants_one_after_the_other(dev):
+    """One mixed-tenant forward/backward and one multi-tenant optimizer launch set against the reference's
+    schedule: every tenant alone (adapter context, its own rows), grads divided by its token count, clipped,
+    torch.optim.AdamW per tenant."""
+    from twinkle_amd import MultiTenantAdamW, trainable_parameters
+    dtype = torch.float32
+    names = ['alice', 'bob', 'carol']
+    hyper = {'alice': dict(lr=1e-2, weight_decay=0.01), 'bob': dict(lr=5e-3, weight_decay=0.0),
+             'carol': dict(lr=2e-2, weight_decay=0.1)}
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(2, 90, 128, generator=g)
+    target = torch.randn(2, 90, 128, generator=g)
+    row_tenant = torch.randint(0, 3, (180,), generator=g)
+    tokens = {n: int((row_tenant == i).sum()) for i, n in enumerate(names)}
+
+    # (a) batched: one forward/backward, sum-of-squares loss per token, then one optimizer step for all tenants
+    ml, model, cfgs = _setup(dev, dtype)
+    opt = MultiTenantAdamW()
+    slot = {n: ml.find_lora_by_tenant(n).adapter_name for n in names}
+    for n in names:
+        opt.add_tenant(n, trainable_parameters(model, slot[n]).values(), **hyper[n])
+    with ml.batch(names, row_tenant.to(dev)):
+        y = model(x.to(dev))
+    ((y - target.to(dev))**2).sum().backward()
+    norms = opt.clip_grad_and_step(tokens, max_grad_norm=1.0)
+    got = {n: {k: p.detach().clone() for k, p in trainable_parameters(model, slot[n]).items()} for n in names}
+
+    # (b) the reference's schedule on a fresh copy: tenants one after the other, each on its own rows
+    ml2, model2, _ = _setup(dev, dtype)
+    for i, n in enumerate(names):
+        params = trainable_parameters(model2, slot[n])
+        rows = (row_tenant == i).nonzero().flatten().to(dev)
+        xs = x.to(dev).reshape(180, 128).index_select(0, rows)
+        ts = target.to(dev).reshape(180, 128).index_select(0, rows)
+        with ml2.adapter(n):
+            ys = model2(xs)
+        ((ys - ts)**2).sum().backward()
+        tenant_params = [p for p in params.values() if p.grad is not None]
+        for p in tenant_params:
+            p.grad.div_(tokens[n])                                   # grad_clip.py:81-96
+        want_norm = torch.nn.utils.clip_grad_norm_(tenant_params, 1.0)
+        torch.optim.AdamW(tenant_params, **hyper[n]).step()
+        assert abs(float(norms[n]) - float(want_norm)) < 1e-4 * float(want_norm)
+        for k, p in params.items():
+            assert max_rel_err(got[n][k], p.detach()) < 2e-5, (n, k)
+        for p in model2.parameters():
+            p.grad = None

@@ -54,20 +54,42 @@ __global__ __launch_bounds__(kOptThreads) void k_opt_norm_partial(const tk_opt_t
   const bool inf = isinf(h.norm_type);
   const T* g = (const T*)t.grad;
   float acc = 0.f;
-#pragma unroll 4
-  for (int j = 0; j < kOptPerThread; ++j) {
-    const int64_t i = i0 + (int64_t)j * kOptThreads + threadIdx.x;
-    if (i < t.numel) {
-      const float v = load_f32(g, i) * h.grad_scale;
-      acc = inf ? fmaxf(acc, fabsf(v)) : acc + v * v;
+  constexpr int V = 16 / sizeof(T);  // elements per 16-byte load
+  const int64_t i1 = min(i0 + kOptPerBlock, t.numel);
+  if ((reinterpret_cast<uintptr_t>(g) & 15u) == 0 && ((i1 - i0) % V) == 0) {
+    // 16-byte loads, consecutive threads on consecutive pieces
+    for (int64_t i = i0 + (int64_t)threadIdx.x * V; i < i1; i += (int64_t)kOptThreads * V) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(g + i);
+      float v[8];
+      if (sizeof(T) == 2) {
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          v[2 * k] = __uint_as_float(w[k] << 16);
+          v[2 * k + 1] = __uint_as_float(w[k] & 0xffff0000u);
+        }
+      } else {
+        v[0] = __uint_as_float(raw.x); v[1] = __uint_as_float(raw.y);
+        v[2] = __uint_as_float(raw.z); v[3] = __uint_as_float(raw.w);
+      }
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        const float x = v[k] * h.grad_scale;
+        acc = inf ? fmaxf(acc, fabsf(x)) : acc + x * x;
+      }
+    }
+  } else {
+    for (int64_t i = i0 + threadIdx.x; i < i1; i += kOptThreads) {
+      const float x = load_f32(g, i) * h.grad_scale;
+      acc = inf ? fmaxf(acc, fabsf(x)) : acc + x * x;
     }
   }
   acc = inf ? block_reduce<true>(acc, scratch) : block_reduce<false>(acc, scratch);
   if (threadIdx.x == 0) partial[(int64_t)blockIdx.y * blocks_per_tensor + blockIdx.x] = acc;
 }
 
-// One block per tenant: walks the tenant's partials in (tensor, block) order, every thread a fixed strided
-// share, then the block tree.  norm[tenant] = total norm after normalisation, before clipping;
+// One block per tenant: every thread adds the partials of a fixed share of the tenant's tensors in a fixed
+// order, then the block tree.  norm[tenant] = total norm after normalisation, before clipping;
 // clip[tenant] = min(1, max_grad_norm / (norm + 1e-6)) (torch.nn.utils.clip_grad_norm_'s coefficient).
 __global__ __launch_bounds__(kOptThreads) void k_opt_norm_final(const tk_opt_tensor* __restrict__ tensors, int n_tensors,
                                                                 const tk_opt_tenant* __restrict__ tenants,
@@ -86,13 +108,12 @@ __global__ __launch_bounds__(kOptThreads) void k_opt_norm_final(const tk_opt_ten
   }
   const bool inf = isinf(h.norm_type);
   float acc = 0.f;
-  for (int ti = 0; ti < n_tensors; ++ti) {
-    if (tensors[ti].tenant != tenant) continue;  // uniform over the block
+  // a thread takes every 256th tensor and adds that tensor's blocks in block order
+  for (int ti = threadIdx.x; ti < n_tensors; ti += kOptThreads) {
+    if (tensors[ti].tenant != tenant) continue;
     const int nb = (int)((tensors[ti].numel + kOptPerBlock - 1) / kOptPerBlock);
-    for (int b = threadIdx.x; b < nb; b += kOptThreads) {
-      const float v = partial[(int64_t)ti * blocks_per_tensor + b];
-      acc = inf ? fmaxf(acc, v) : acc + v;
-    }
+    const float* p = partial + (int64_t)ti * blocks_per_tensor;
+    for (int b = 0; b < nb; ++b) acc = inf ? fmaxf(acc, p[b]) : acc + p[b];
   }
   acc = inf ? block_reduce<true>(acc, scratch) : block_reduce<false>(acc, scratch);
   if (threadIdx.x == 0) {

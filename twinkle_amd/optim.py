@@ -56,6 +56,7 @@ class MultiTenantAdamW:
         self._tenants: Dict[str, _Tenant] = {}
         self._last_clip: Dict[torch.dtype, torch.Tensor] = {}
         self._last_tables = None
+        self._table_cache: Dict[torch.dtype, tuple] = {}
 
     # ---- tenant management -------------------------------------------------------------------------------
     def add_tenant(self, name: str, params: Iterable[torch.nn.Parameter], lr: float = 1e-3, betas=(0.9, 0.999),
@@ -88,10 +89,14 @@ class MultiTenantAdamW:
 
     # ---- the step ----------------------------------------------------------------------------------------
     def _tables(self, names: Sequence[str], num_tokens, max_grad_norm, norm_type, optim_params, advance: bool):
-        """Device tables per parameter dtype for the tenants in ``names``."""
+        """Device tables per parameter dtype for the tenants in ``names``.
+
+        The tensor table only changes when a gradient tensor was replaced (autograd accumulates in place and the
+        in-kernel zeroing keeps the tensors), so it is cached on the pointers it holds; the small tenant table
+        carries this call's numbers and is rebuilt every time."""
         names = list(names)
         tenant_rows = np.zeros(len(self._tenants), dtype=_TENANT_DTYPE)
-        per_dtype: Dict[torch.dtype, list] = {}
+        rows: Dict[torch.dtype, list] = {}
         keep = []
         device = None
         for name in names:
@@ -115,9 +120,9 @@ class MultiTenantAdamW:
             row['norm_type'] = norm_type
             row['active'] = 1
             for i, p in enumerate(t.params):
-                if p.grad is None:
-                    continue  # torch optimizers skip parameters without a gradient
                 g = p.grad
+                if g is None:
+                    continue  # torch optimizers skip parameters without a gradient
                 if g.dtype != p.dtype or not g.is_contiguous() or g.shape != p.shape:
                     g = g.to(p.dtype).contiguous()
                     p.grad = g
@@ -125,33 +130,29 @@ class MultiTenantAdamW:
                     t.exp_avg[i] = torch.zeros(p.shape, dtype=torch.float32, device=p.device)
                     t.exp_avg_sq[i] = torch.zeros(p.shape, dtype=torch.float32, device=p.device)
                 device = p.device
-                per_dtype.setdefault(p.dtype, []).append(
-                    (p.data_ptr(), g.data_ptr(), t.exp_avg[i].data_ptr(), t.exp_avg_sq[i].data_ptr(), p.numel(),
-                     t.index, 0))
+                rows.setdefault(p.dtype, []).append((p.data_ptr(), g.data_ptr(), t.exp_avg[i].data_ptr(),
+                                                     t.exp_avg_sq[i].data_ptr(), p.numel(), t.index, 0))
                 keep.append(g)
         out = {}
         if device is None:
             return out, tenant_rows
         tenants_dev = torch.from_numpy(tenant_rows.view(np.uint8).copy()).to(device)
-        for dtype, rows in per_dtype.items():
-            arr = np.array(rows, dtype=_TENSOR_DTYPE)
-            out[dtype] = (torch.from_numpy(arr.view(np.uint8).copy()).to(device), len(rows),
-                          int(arr['numel'].max()), tenants_dev, keep)
+        for dtype, lst in rows.items():
+            cached = self._table_cache.get(dtype)
+            if cached is None or cached[0] != lst:
+                arr = np.array(lst, dtype=_TENSOR_DTYPE)
+                cached = (lst, torch.from_numpy(arr.view(np.uint8).copy()).to(device), int(arr['numel'].max()))
+                self._table_cache[dtype] = cached
+            out[dtype] = (cached[1], len(lst), cached[2], tenants_dev, keep)
         return out, tenant_rows
 
-    def clip_grad_norm(self, num_tokens, max_grad_norm: float = 1.0, norm_type: float = 2.0,
-                       names: Optional[Sequence[str]] = None) -> Dict[str, torch.Tensor]:
-        """Norm of every tenant's gradients after division by its token count (device scalars, no host
-        synchronisation), as ``clip_grad_norm`` returns it per tenant; the division and the clipping themselves
-        are applied inside :meth:`step`, which must follow (``clip_grad_and_step`` does both)."""
-        names = list(names) if names is not None else self.tenants()
-        tables, _ = self._tables(names, num_tokens, max_grad_norm, float(norm_type), None, advance=False)
+    def _run_norm(self, tables, names, max_grad_norm, norm_type) -> Dict[str, torch.Tensor]:
         lib = _lib.load()
         norms: Dict[str, torch.Tensor] = {}
         self._last_clip = {}
         per_dtype_norms = []
+        nt = len(self._tenants)
         for dtype, (tensors_dev, n, max_numel, tenants_dev, _keep) in tables.items():
-            nt = len(self._tenants)
             norm = torch.empty(nt, dtype=torch.float32, device=tensors_dev.device)
             clip = torch.empty(nt, dtype=torch.float32, device=tensors_dev.device)
             nbytes = lib.tk_opt_workspace_bytes(n, max_numel)
@@ -176,17 +177,8 @@ class MultiTenantAdamW:
                 norms[name] = per_dtype_norms[0][self._tenants[name].index]
         return norms
 
-    def step(self, num_tokens=1, optim_params: Optional[Dict[str, dict]] = None,
-             names: Optional[Sequence[str]] = None, zero_grad: bool = False, write_grads: bool = False,
-             use_clip: bool = True) -> None:
-        """AdamW for the tenants in ``names`` (default: all), gradients divided by ``num_tokens`` (an int or a
-        dict per tenant) and scaled by the coefficients of the preceding :meth:`clip_grad_norm`.
-        ``optim_params[name]`` may carry ``lr``, ``weight_decay``, ``eps``, ``betas`` for this call
-        (transformers.py:857-868)."""
-        names = list(names) if names is not None else self.tenants()
-        tables, _ = self._tables(names, num_tokens, 0.0, 2.0, optim_params, advance=True)
+    def _run_step(self, tables, names, flags: int, use_clip: bool) -> None:
         lib = _lib.load()
-        flags = (TK_OPT_ZERO_GRADS if zero_grad else 0) | (TK_OPT_WRITE_GRADS if write_grads else 0)
         for dtype, (tensors_dev, n, max_numel, tenants_dev, _keep) in tables.items():
             clip = self._last_clip.get(dtype) if use_clip else None
             code = lib.tk_opt_adamw_step(tensors_dev.data_ptr(), n, tenants_dev.data_ptr(), len(self._tenants),
@@ -198,12 +190,36 @@ class MultiTenantAdamW:
         for name in names:
             self._tenants[name].step += 1
 
+    def clip_grad_norm(self, num_tokens, max_grad_norm: float = 1.0, norm_type: float = 2.0,
+                       names: Optional[Sequence[str]] = None) -> Dict[str, torch.Tensor]:
+        """Norm of every tenant's gradients after division by its token count (device scalars, no host
+        synchronisation), as ``clip_grad_norm`` returns it per tenant; the division and the clipping themselves
+        are applied inside :meth:`step`, which must follow (``clip_grad_and_step`` does both)."""
+        names = list(names) if names is not None else self.tenants()
+        tables, _ = self._tables(names, num_tokens, max_grad_norm, float(norm_type), None, advance=False)
+        return self._run_norm(tables, names, max_grad_norm, norm_type)
+
+    def step(self, num_tokens=1, optim_params: Optional[Dict[str, dict]] = None,
+             names: Optional[Sequence[str]] = None, zero_grad: bool = False, write_grads: bool = False,
+             use_clip: bool = True) -> None:
+        """AdamW for the tenants in ``names`` (default: all), gradients divided by ``num_tokens`` (an int or a
+        dict per tenant) and scaled by the coefficients of the preceding :meth:`clip_grad_norm`.
+        ``optim_params[name]`` may carry ``lr``, ``weight_decay``, ``eps``, ``betas`` for this call
+        (transformers.py:857-868)."""
+        names = list(names) if names is not None else self.tenants()
+        tables, _ = self._tables(names, num_tokens, 0.0, 2.0, optim_params, advance=True)
+        flags = (TK_OPT_ZERO_GRADS if zero_grad else 0) | (TK_OPT_WRITE_GRADS if write_grads else 0)
+        self._run_step(tables, names, flags, use_clip)
+
     def clip_grad_and_step(self, num_tokens, max_grad_norm: float = 1.0, norm_type: float = 2.0,
                            optim_params: Optional[Dict[str, dict]] = None,
                            names: Optional[Sequence[str]] = None) -> Dict[str, torch.Tensor]:
-        """clip_grad_norm, step and zero_grad for every tenant in one go (transformers.py:781-785)."""
-        norms = self.clip_grad_norm(num_tokens, max_grad_norm, norm_type, names)
-        self.step(num_tokens, optim_params, names, zero_grad=True)
+        """clip_grad_norm, step and zero_grad for every tenant in one go (transformers.py:781-785); the device
+        tables are built once and serve both passes."""
+        names = list(names) if names is not None else self.tenants()
+        tables, _ = self._tables(names, num_tokens, max_grad_norm, float(norm_type), optim_params, advance=True)
+        norms = self._run_norm(tables, names, max_grad_norm, norm_type)
+        self._run_step(tables, names, TK_OPT_ZERO_GRADS, use_clip=True)
         return norms
 
     def zero_grad(self, names: Optional[Sequence[str]] = None, set_to_none: bool = True) -> None:
