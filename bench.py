@@ -170,6 +170,8 @@ def main():
                     help='cfg2 is the headline configuration; the others are the wider BASELINE shapes '
                          '(cfg3: 4096<->14336, T=32768, 32 adapters of rank 8..64; cfg5_q: 4096->4096, T=32768, 8 tenants '
                          'of rank 64, one per packed 4096-token sequence) for additional measurements')
+    ap.add_argument('--optimizer-only', action='store_true',
+                    help='run only the multi-tenant optimizer micro-benchmark and print its JSON (for profiling)')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run five plain 128 MiB device copies (a known-size kernel to scale rocprofv3 --pmc '
                          'FETCH_SIZE / WRITE_SIZE readings by)')
@@ -187,6 +189,9 @@ def main():
         sys.exit(2)
     _lib.load()
     dev = torch.device('cuda:0')
+    if args.optimizer_only:
+        print(json.dumps({'optimizer_step': optimizer_step_bench(dev)}))
+        return
     if args.workload == 'cfg2':
         w = workloads.config2_qproj()
     elif args.workload == 'cfg5_q':
