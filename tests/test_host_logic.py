@@ -194,3 +194,55 @@ def test_custom_ops_are_registered_and_traceable():
     assert ws.dtype == torch.uint8 and ws.numel() == _lib.load().tk_segment_workspace_bytes(1000, 7)
     with pytest.raises(RuntimeError, match='GPU'):
         torch.ops.twinkle_amd.segment_build(torch.zeros(4, dtype=torch.int32), 2)
+
+
+def test_adapter_checkpoint_round_trip_in_peft_format(tmp_path):
+    """adapter_model.safetensors holds the tenant's [:r] blocks under slot-free, PEFT-prefixed keys; loading into
+    another slot (even of another MultiLora) reproduces them and leaves the rest of the slot alone."""
+    import json
+
+    from safetensors.torch import load_file
+
+    class Tiny(nn.Module):
+
+        def __init__(self):
+            super().__init__()
+            self.q_proj = nn.Linear(12, 12, bias=False)
+            self.up_proj = nn.Linear(12, 20, bias=False)
+
+        def forward(self, x):
+            return self.up_proj(self.q_proj(x))
+
+    torch.manual_seed(0)
+    ml = MultiLora(max_loras=3, max_r=8)
+    model = ml.patch(Tiny(), target_modules='all-linear')
+    ml.save_initial_weights()
+    ml.acquire_lora('alice', LoraConfig(r=4, lora_alpha=8, target_modules=['q_proj']))
+    with torch.no_grad():
+        for n, p in model.named_parameters():
+            if 'lora_' in n:
+                p.copy_(torch.randn(p.shape))
+    out = ml.save_adapter('alice', str(tmp_path / 'ckpt'))
+    saved = load_file(f'{out}/adapter_model.safetensors')
+    # key and shape KAT: PEFT layout, rank-sliced, only the targeted module
+    assert sorted(saved) == ['base_model.model.q_proj.lora_A.weight', 'base_model.model.q_proj.lora_B.weight']
+    assert saved['base_model.model.q_proj.lora_A.weight'].shape == (4, 12)
+    assert saved['base_model.model.q_proj.lora_B.weight'].shape == (12, 4)
+    cfg = json.load(open(f'{out}/adapter_config.json'))
+    assert cfg['peft_type'] == 'LORA' and cfg['r'] == 4 and cfg['lora_alpha'] == 8 and cfg['target_modules'] == ['q_proj']
+    slot = ml.find_lora_by_tenant('alice').adapter_name
+    a_src = dict(model.named_parameters())[f'model.q_proj.lora_A.{slot}.weight'].detach().clone()
+    assert torch.equal(saved['base_model.model.q_proj.lora_A.weight'], a_src[:4])
+
+    ml2 = MultiLora(max_loras=2, max_r=8)
+    model2 = ml2.patch(Tiny(), target_modules='all-linear')
+    ml2.save_initial_weights()
+    ml2.acquire_lora('x', LoraConfig(r=2, lora_alpha=4, target_modules='all-linear'))     # takes the first slot
+    ml2.acquire_lora('alice', LoraConfig(r=4, lora_alpha=8, target_modules=['q_proj']))
+    slot2 = ml2.find_lora_by_tenant('alice').adapter_name
+    before = dict(model2.named_parameters())[f'model.q_proj.lora_A.{slot2}.weight'].detach().clone()
+    ml2.load_adapter('alice', out)
+    after = dict(model2.named_parameters())[f'model.q_proj.lora_A.{slot2}.weight'].detach()
+    assert torch.equal(after[:4], a_src[:4]) and torch.equal(after[4:], before[4:])
+    for k, v in ml2.get_state_dict('alice').items():
+        assert torch.equal(v, saved['base_model.' + k])

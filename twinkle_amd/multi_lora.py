@@ -381,6 +381,51 @@ class MultiLora:
                                                                                            slot.tenant_config.r)
         return out
 
+    # ---- adapter checkpoints in PEFT's on-disk format -----------------------------------------------------------
+    _PEFT_PREFIX = 'base_model.'
+
+    def save_adapter(self, tenant_adapter_name: str, checkpoint_dir: str) -> str:
+        """Write the tenant's adapter as ``adapter_model.safetensors`` + ``adapter_config.json``.
+
+        Same content as the reference's save for a tenant (transformers.py:1001-1033 with the state dict of
+        multi_lora_transformers.py:265-267): the live ``[:r]`` blocks, slot name removed from the keys, on the
+        CPU, contiguous.  The holder returned by ``patch`` takes the place of ``PeftModel.base_model``, so keys
+        get the ``base_model.`` prefix PEFT's files carry and load with ``peft.utils.load_peft_weights``."""
+        import json
+        import os
+
+        from safetensors.torch import save_file
+        slot = self.find_lora_by_tenant(tenant_adapter_name)
+        state = {self._PEFT_PREFIX + k: v.detach().to('cpu').contiguous()
+                 for k, v in self.get_state_dict(tenant_adapter_name).items()}
+        os.makedirs(checkpoint_dir, exist_ok=True)
+        save_file(state, os.path.join(checkpoint_dir, 'adapter_model.safetensors'))
+        cfg = slot.tenant_config
+        target = cfg.target_modules
+        config = {
+            'peft_type': 'LORA', 'task_type': 'CAUSAL_LM', 'base_model_name_or_path': None, 'inference_mode': True,
+            'r': cfg.r, 'lora_alpha': cfg.lora_alpha, 'lora_dropout': getattr(cfg, 'lora_dropout', 0.0),
+            'target_modules': sorted(target) if isinstance(target, (set, list, tuple)) else target,
+            'exclude_modules': getattr(cfg, 'exclude_modules', None), 'use_rslora': bool(getattr(cfg, 'use_rslora', False)),
+            'use_dora': False, 'fan_in_fan_out': False, 'bias': 'none',
+            'target_parameters': getattr(cfg, 'target_parameters', None),
+        }
+        with open(os.path.join(checkpoint_dir, 'adapter_config.json'), 'w') as f:
+            json.dump(config, f, indent=2, sort_keys=True)
+        return checkpoint_dir
+
+    def load_adapter(self, tenant_adapter_name: str, checkpoint_dir: str) -> None:
+        """Read ``adapter_model.safetensors`` into the prefix of the tenant's slot (the reference's load,
+        multi_lora_transformers.py:280-300: weights to the CPU first, then ``set_state_dict``); tensors saved at a
+        rank below the slot's are padded by leaving the rest of the slot untouched."""
+        import os
+
+        from safetensors.torch import load_file
+        state = load_file(os.path.join(checkpoint_dir, 'adapter_model.safetensors'), device='cpu')
+        n = len(self._PEFT_PREFIX)
+        state = {(k[n:] if k.startswith(self._PEFT_PREFIX) else k): v for k, v in state.items()}
+        self.set_state_dict(tenant_adapter_name, state)
+
     def get_nb_trainable_parameters(self, tenant_adapter_name):
         """(trainable, all) parameter counts as the tenant sees them (reference :756-813)."""
         slot = self.find_lora_by_tenant(tenant_adapter_name)
