@@ -283,28 +283,35 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
     if (hipEventRecord(side->fork, s) != hipSuccess || hipStreamWaitEvent(s2, side->fork, 0) != hipSuccess)
       return TK_ERR_LAUNCH;
   }
-  bool wT_done = false;
-  if (grad_B) {
-    if (!side && need_wT && mfma && wgrad_mfma_supported(gb) && d->out_features % 8 == 0) {
-      gb.tr = tr;  // one stream: the MFMA launch also writes the transposed weight copies of the pass below
-      wT_done = true;
+  // once forked, every path joins again, also after an error: the side stream must not be left attached to
+  // the caller's stream (or to a graph capture of it)
+  rc = TK_OK;
+  do {
+    bool wT_done = false;
+    if (grad_B) {
+      if (!side && need_wT && mfma && wgrad_mfma_supported(gb) && d->out_features % 8 == 0) {
+        gb.tr = tr;  // one stream: the MFMA launch also writes the transposed weight copies of the pass below
+        wT_done = true;
+      }
+      rc = run_wgrad(gb, V, L, d->dtype, s2);
+      gb.tr = TransposeJob{};
+      if (rc != TK_OK) break;
     }
-    rc = run_wgrad(gb, V, L, d->dtype, s2);
-    gb.tr = TransposeJob{};
-    if (rc != TK_OK) return rc;
-  }
-  if (need_wT) {
-    if (!wT_done && (rc = launch_transpose_weights(*d, bT, aT, s)) != TK_OK) return rc;
-    if ((rc = run_pass(a, V, L, d->dtype, 1, s)) != TK_OK) return rc;
-    if (side && grad_A) {  // dh is complete: the side stream may start dA while dX runs here
-      if (hipEventRecord(side->mid, s) != hipSuccess || hipStreamWaitEvent(s2, side->mid, 0) != hipSuccess)
-        return TK_ERR_LAUNCH;
+    if (need_wT) {
+      if (!wT_done && (rc = launch_transpose_weights(*d, bT, aT, s)) != TK_OK) break;
+      if ((rc = run_pass(a, V, L, d->dtype, 1, s)) != TK_OK) break;
+      if (side && grad_A) {  // dh is complete: the side stream may start dA while dX runs here
+        if (hipEventRecord(side->mid, s) != hipSuccess || hipStreamWaitEvent(s2, side->mid, 0) != hipSuccess) {
+          rc = TK_ERR_LAUNCH;
+          break;
+        }
+      }
+      if (dx && (rc = run_pass(a, V, L, d->dtype, 2, s)) != TK_OK) break;
     }
-    if (dx && (rc = run_pass(a, V, L, d->dtype, 2, s)) != TK_OK) return rc;
-  }
-  if (grad_A && (rc = run_wgrad(ga, V, L, d->dtype, s2)) != TK_OK) return rc;
-  // the chunk partials of both contractions are summed by one launch
-  rc = launch_wgrad_reduce(grad_A ? &ga : nullptr, grad_B ? &gb : nullptr, V, L, d->dtype, s2);
+    if (grad_A && (rc = run_wgrad(ga, V, L, d->dtype, s2)) != TK_OK) break;
+    // the chunk partials of both contractions are summed by one launch
+    rc = launch_wgrad_reduce(grad_A ? &ga : nullptr, grad_B ? &gb : nullptr, V, L, d->dtype, s2);
+  } while (false);
   if (side) {
     if (hipEventRecord(side->join, s2) != hipSuccess || hipStreamWaitEvent(s, side->join, 0) != hipSuccess)
       return TK_ERR_LAUNCH;
