@@ -166,7 +166,7 @@ def main():
     ap.add_argument('--event-every', type=int, default=4,
                     help='bracket the kernels with HIP events on every n-th timed step (an event record costs a few '
                          'microseconds of idle queue, so not every step carries them)')
-    ap.add_argument('--workload', default='cfg2', choices=['cfg2', 'cfg3_up', 'cfg3_down', 'cfg5_q'],
+    ap.add_argument('--workload', default='cfg2', choices=['cfg2', 'cfg3_up', 'cfg3_down', 'cfg5_q', 'cfg4_gate_up'],
                     help='cfg2 is the headline configuration; the others are the wider BASELINE shapes '
                          '(cfg3: 4096<->14336, T=32768, 32 adapters of rank 8..64; cfg5_q: 4096->4096, T=32768, 8 tenants '
                          'of rank 64, one per packed 4096-token sequence) for additional measurements')
@@ -198,6 +198,14 @@ def main():
         w = workloads.config2_qproj(tokens=32768, n=8, r=64)
         w.ids = torch.repeat_interleave(torch.arange(8, dtype=torch.int32), 4096)
         w.name = 'cfg5_llama8b_q_rank64'
+    elif args.workload == 'cfg4_gate_up':
+        # expert LoRA shape: 8192 tokens x top-8 = 65536 routed rows, 128 experts x 4 tenants = 512 groups of rank 8,
+        # hidden 2048 -> fused gate_up 1536; rows arrive sorted by (expert, tenant) like after the routing permute
+        w = workloads.config2_qproj(tokens=65536, features=2048, n=512, r=8)
+        w.ids = torch.sort(torch.randint(0, 512, (65536,), generator=torch.Generator().manual_seed(6)).to(torch.int32)).values
+        w.lora_B = [b[:1536].contiguous() for b in w.lora_B]
+        w.base_out, w.dy, w.out_features = w.base_out[:, :1536].contiguous(), w.dy[:, :1536].contiguous(), 1536
+        w.name = 'cfg4_qwen3moe_gate_up_rank8'
     else:
         w = workloads.config3_mlp('up' if args.workload == 'cfg3_up' else 'down')
     if args.workload != 'cfg2':
