@@ -171,16 +171,10 @@ int64_t tk_lora_bwd_workspace_bytes(const tk_lora_desc* d) {
   return BwdLayout(*d).total;
 }
 
-static int lora_pass_fwd(const tk_lora_desc* d, const void* x, int64_t ldx, void* y, int64_t ldy, void* h,
-                         int phases, tk_stream_t stream) {
-  if (!desc_ok(d) || !h) return TK_ERR_INVALID;
-  if (d->rows == 0 || d->max_rank == 0) return TK_OK;
-  if ((phases & 1) && (!x || ldx < d->in_features)) return TK_ERR_INVALID;
-  if ((phases & 2) && (!y || ldy < d->out_features)) return TK_ERR_INVALID;
-  SegLayout L(d->rows, d->num_groups);
-  SegView V(d->seg_ws, L);
+// Arguments of the forward pass h = scale x A^T, y += h B^T.  Null x / y are replaced by placeholders: shapes are
+// checked against what both phases need, so that the two halves of one forward pick the same kernels.
+static PassArgs fwd_pass_args(const tk_lora_desc* d, const void* x, int64_t ldx, void* y, int64_t ldy, void* h) {
   PassArgs a{};
-  // shapes are checked against what both phases need, so that the two halves of one forward pick the same kernels
   a.src = x ? x : h;  a.ld_src = x ? ldx : d->in_features;
   a.dst = y ? y : h;  a.ld_dst = y ? ldy : d->out_features;
   a.hT = h;   a.ldh = h_ld(d->rows, d->num_groups);
@@ -191,6 +185,73 @@ static int lora_pass_fwd(const tk_lora_desc* d, const void* x, int64_t ldx, void
   a.map_rows = d->map_rows;  a.rpad = rank_pad(d->max_rank);  a.src_rows = (int32_t)d->rows;
   a.hpart = (float*)((char*)h + round_up(2 * (int64_t)a.rpad * a.ldh * elt_bytes(d->dtype), 256));
   a.kslices = shrink_kslices(d->in_features, a.rpad);
+  return a;
+}
+
+// Everything the backward of one projection needs, carved from its workspace.
+struct BwdPlan {
+  WgradArgs ga{}, gb{};  // dA[n][k] = sum_rows dh[row][n] x[row][k];  dB[m][n] = sum_rows dy[row][m] h[row][n]
+  PassArgs a{};          // dh = scale * dy B, dx += dh A
+  TransposeJob tr{};     // B^T, A^T copies
+  void* dh = nullptr;
+  void* bT = nullptr;
+  void* aT = nullptr;
+};
+
+static BwdPlan bwd_plan(const tk_lora_desc* d, const BwdLayout& B, const void* dy, int64_t lddy, const void* x,
+                        int64_t ldx, const void* h, void* dx, int64_t lddx, void* const* grad_A, void* const* grad_B,
+                        int32_t accumulate, void* ws) {
+  BwdPlan p;
+  char* w = (char*)ws;
+  p.dh = w + B.off_dh;
+  p.bT = w + B.off_wT_shrink;
+  p.aT = w + B.off_wT_expand;
+  if (grad_B) {
+    WgradArgs& g = p.gb;
+    g.src = dy;  g.ld_src = lddy;
+    g.hT = h;    g.ldh = B.ldh;
+    g.partial = (float*)(w + B.off_part_b);
+    g.grad = grad_B;  g.ld_grad = d->ldb;
+    g.rank = d->rank;  g.width = d->out_features;  g.transposed = 1;
+    g.accumulate = accumulate;  g.map_rows = d->map_rows;  g.rpad = (int32_t)B.rpad;
+  }
+  if (grad_A) {
+    WgradArgs& g = p.ga;
+    g.src = x;  g.ld_src = ldx;
+    g.hT = p.dh;  g.ldh = B.ldh;
+    g.partial = (float*)(w + B.off_part_a);
+    g.grad = grad_A;  g.ld_grad = d->lda;
+    g.rank = d->rank;  g.width = d->in_features;  g.transposed = 0;
+    g.accumulate = accumulate;  g.map_rows = d->map_rows;  g.rpad = (int32_t)B.rpad;
+  }
+  PassArgs& a = p.a;
+  a.src = dy;  a.ld_src = lddy;
+  a.dst = dx;  a.ld_dst = lddx;
+  a.hT = p.dh;   a.ldh = B.ldh;
+  a.w_shrink_base = p.bT;  a.ld_shrink = d->out_features;  a.shrink_group_stride = B.rpad * d->out_features;
+  a.w_expand_base = p.aT;  a.ld_expand = B.rpad;           a.expand_group_stride = B.rpad * d->in_features;
+  a.rank = d->rank;  a.scale = d->scale;
+  a.width_src = d->out_features;  a.width_dst = d->in_features;
+  a.map_rows = d->map_rows;  a.rpad = (int32_t)B.rpad;  a.src_rows = (int32_t)d->rows;
+  a.hpart = (float*)(w + B.off_hpart);
+  a.kslices = shrink_kslices(d->out_features, a.rpad);
+  TransposeJob& tr = p.tr;
+  tr.lora_A = d->lora_A;  tr.lda = d->lda;
+  tr.lora_B = d->lora_B;  tr.ldb = d->ldb;
+  tr.aT = p.aT;  tr.bT = p.bT;
+  tr.in_features = d->in_features;  tr.out_features = d->out_features;  tr.groups = d->num_groups;
+  return p;
+}
+
+static int lora_pass_fwd(const tk_lora_desc* d, const void* x, int64_t ldx, void* y, int64_t ldy, void* h,
+                         int phases, tk_stream_t stream) {
+  if (!desc_ok(d) || !h) return TK_ERR_INVALID;
+  if (d->rows == 0 || d->max_rank == 0) return TK_OK;
+  if ((phases & 1) && (!x || ldx < d->in_features)) return TK_ERR_INVALID;
+  if ((phases & 2) && (!y || ldy < d->out_features)) return TK_ERR_INVALID;
+  SegLayout L(d->rows, d->num_groups);
+  SegView V(d->seg_ws, L);
+  const PassArgs a = fwd_pass_args(d, x, ldx, y, ldy, h);
   return run_pass(a, V, L, d->dtype, phases, (hipStream_t)stream);
 }
 
@@ -221,46 +282,14 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
   hipStream_t s = (hipStream_t)stream;
   SegLayout L(d->rows, d->num_groups);
   SegView V(d->seg_ws, L);
-  char* w = (char*)ws;
-  void* dh = w + B.off_dh;
   int rc;
   const bool need_wT = dx || grad_A;
-  void* bT = w + B.off_wT_shrink;
-  void* aT = w + B.off_wT_expand;
-  WgradArgs ga{}, gb{};
-  if (grad_B) {  // dB[m][n] = sum_rows dy[row][m] * h[row][n]
-    gb.src = dy;  gb.ld_src = lddy;
-    gb.hT = h;    gb.ldh = B.ldh;
-    gb.partial = (float*)(w + B.off_part_b);
-    gb.grad = grad_B;  gb.ld_grad = d->ldb;
-    gb.rank = d->rank;  gb.width = d->out_features;  gb.transposed = 1;
-    gb.accumulate = accumulate;  gb.map_rows = d->map_rows;  gb.rpad = (int32_t)B.rpad;
-  }
-  if (grad_A) {  // dA[n][k] = sum_rows dh[row][n] * x[row][k]
-    ga.src = x;  ga.ld_src = ldx;
-    ga.hT = dh;  ga.ldh = B.ldh;
-    ga.partial = (float*)(w + B.off_part_a);
-    ga.grad = grad_A;  ga.ld_grad = d->lda;
-    ga.rank = d->rank;  ga.width = d->in_features;  ga.transposed = 0;
-    ga.accumulate = accumulate;  ga.map_rows = d->map_rows;  ga.rpad = (int32_t)B.rpad;
-  }
-  PassArgs a{};  // dh = scale * dy B, dx += dh A
-  a.src = dy;  a.ld_src = lddy;
-  a.dst = dx;  a.ld_dst = lddx;
-  a.hT = dh;   a.ldh = B.ldh;
-  a.w_shrink_base = bT;  a.ld_shrink = d->out_features;  a.shrink_group_stride = B.rpad * d->out_features;
-  a.w_expand_base = aT;  a.ld_expand = B.rpad;           a.expand_group_stride = B.rpad * d->in_features;
-  a.rank = d->rank;  a.scale = d->scale;
-  a.width_src = d->out_features;  a.width_dst = d->in_features;
-  a.map_rows = d->map_rows;  a.rpad = (int32_t)B.rpad;  a.src_rows = (int32_t)d->rows;
-  a.hpart = (float*)(w + B.off_hpart);
-  a.kslices = shrink_kslices(d->out_features, a.rpad);
+  BwdPlan plan = bwd_plan(d, B, dy, lddy, x, ldx, h, dx, lddx, grad_A, grad_B, accumulate, ws);
+  WgradArgs &ga = plan.ga, &gb = plan.gb;
+  PassArgs& a = plan.a;
+  const TransposeJob& tr = plan.tr;
+  void *bT = plan.bT, *aT = plan.aT;
   const bool mfma = d->dtype == TK_DTYPE_BF16 && !force_generic();
-  TransposeJob tr{};
-  tr.lora_A = d->lora_A;  tr.lda = d->lda;
-  tr.lora_B = d->lora_B;  tr.ldb = d->ldb;
-  tr.aT = aT;  tr.bT = bT;
-  tr.in_features = d->in_features;  tr.out_features = d->out_features;  tr.groups = d->num_groups;
 
   if (grad_B && need_wT && mfma && pass_mfma_supported(a) && dy_fused_supported(gb, a.kslices)) {
     // One pass over dy yields dB and the slices of dh (and, on the side, the A^T copy for dX).
