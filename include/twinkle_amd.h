@@ -212,6 +212,26 @@ int tk_opt_adamw_step(const tk_opt_tensor* tensors_device, int32_t num_tensors, 
                       int32_t num_tenants, int64_t max_numel, int32_t dtype, const float* clip_device, int32_t flags,
                       tk_stream_t stream);
 
+/* ---------------------------------------------------------------------------
+ * Projections that share their input (q / k / v, gate / up): one call for all of them, with the shared
+ * tensors crossing memory once.  Same results contract as one tk_lora_fwd / tk_lora_bwd per projection, which
+ * is also what runs when the shapes are outside the shared kernels (bf16, every max_rank <= 16, 2..4
+ * projections, in_features a multiple of 1024 .. see the single-projection fast-path limits): forward reads
+ * x once instead of once per projection; backward reads x once for all dA and updates dx once with the sum
+ * over the projections (one rounding instead of one per projection).  The descriptors must agree in rows,
+ * in_features, num_groups, dtype, map_rows and seg_ws.  Arrays indexed by projection are host arrays.
+ * No counterpart in the reference, which runs every projection's two F.linear calls on its own
+ * (multi_lora.py:322-326).
+ * ------------------------------------------------------------------------- */
+#define TK_MAX_SHARED 4
+int tk_lora_fwd_shared(const tk_lora_desc* const* descs, int32_t num_proj, const void* x_device, int64_t ldx,
+                       void* const* y_device, const int64_t* ldy, void* const* h_device, tk_stream_t stream);
+int tk_lora_bwd_shared(const tk_lora_desc* const* descs, int32_t num_proj, const void* const* dy_device,
+                       const int64_t* lddy, const void* x_device, int64_t ldx, const void* const* h_device,
+                       void* dx_device, int64_t lddx, void* const* const* grad_A, void* const* const* grad_B,
+                       int32_t accumulate, void* const* workspace_device, const int64_t* workspace_bytes,
+                       tk_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -69,6 +69,10 @@ EXPORTS = {
     'tk_lora_expand': (c_int32, [POINTER(LoraDesc), c_void_p, c_void_p, c_int64, c_void_p]),
     'tk_lora_bwd': (c_int32, [POINTER(LoraDesc), c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                               c_void_p, c_void_p, c_int32, c_void_p, c_int64, c_void_p]),
+    # arrays indexed by projection are host arrays: pointers to descriptors / device pointers / strides
+    'tk_lora_fwd_shared': (c_int32, [c_void_p, c_int32, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    'tk_lora_bwd_shared': (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
+                                     c_int64, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p]),
     'tk_opt_workspace_bytes': (c_int64, [c_int32, c_int64]),
     'tk_opt_grad_norm': (c_int32, [c_void_p, c_int32, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p,
                                    c_int64, c_void_p]),

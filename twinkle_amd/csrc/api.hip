@@ -348,6 +348,124 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
   return rc;
 }
 
+// ---- projections that share their input ------------------------------------------------------------------------
+
+static bool shared_descs_ok(const tk_lora_desc* const* descs, int32_t n) {
+  if (!descs || n < 1 || n > TK_MAX_SHARED) return false;
+  for (int p = 0; p < n; ++p) {
+    if (!desc_ok(descs[p])) return false;
+    const tk_lora_desc *a = descs[0], *b = descs[p];
+    if (a->rows != b->rows || a->in_features != b->in_features || a->num_groups != b->num_groups ||
+        a->dtype != b->dtype || a->map_rows != b->map_rows || a->seg_ws != b->seg_ws)
+      return false;
+  }
+  return true;
+}
+
+// the kernels of kernels_shared.hip apply: bf16, 2..4 projections of padded rank 16, a split shrink
+static bool shared_fast_path(const tk_lora_desc* const* descs, int32_t n) {
+  if (n < 2 || descs[0]->dtype != TK_DTYPE_BF16 || force_generic()) return false;
+  for (int p = 0; p < n; ++p)
+    if (descs[p]->max_rank < 1 || descs[p]->max_rank > 16) return false;
+  return shrink_kslices(descs[0]->in_features, 16) > 1;
+}
+
+int tk_lora_fwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* x, int64_t ldx, void* const* y,
+                       const int64_t* ldy, void* const* h, tk_stream_t stream) {
+  if (!shared_descs_ok(descs, n) || !y || !ldy || !h) return TK_ERR_INVALID;
+  const tk_lora_desc* d0 = descs[0];
+  if (d0->rows == 0) return TK_OK;
+  if (!x || ldx < d0->in_features) return TK_ERR_INVALID;
+  for (int p = 0; p < n; ++p)
+    if (!y[p] || !h[p] || ldy[p] < descs[p]->out_features) return TK_ERR_INVALID;
+  hipStream_t s = (hipStream_t)stream;
+  SegLayout L(d0->rows, d0->num_groups);
+  SegView V(d0->seg_ws, L);
+  PassArgs a[TK_MAX_SHARED];
+  bool fast = shared_fast_path(descs, n);
+  for (int p = 0; p < n; ++p) {
+    a[p] = fwd_pass_args(descs[p], x, ldx, y[p], ldy[p], h[p]);
+    fast = fast && pass_mfma_supported(a[p]);
+  }
+  int rc;
+  if (!fast) {
+    for (int p = 0; p < n; ++p)
+      if ((rc = tk_lora_fwd(descs[p], x, ldx, y[p], ldy[p], h[p], stream)) != TK_OK) return rc;
+    return TK_OK;
+  }
+  SharedShrinkArgs sa{};
+  sa.src = x;  sa.ld_src = ldx;
+  sa.width_src = d0->in_features;  sa.src_rows = (int32_t)d0->rows;  sa.map_rows = d0->map_rows;
+  sa.kslices = a[0].kslices;  sa.nproj = n;
+  for (int p = 0; p < n; ++p) {
+    sa.w[p] = descs[p]->lora_A;  sa.ld_w[p] = descs[p]->lda;
+    sa.rank[p] = descs[p]->rank;  sa.hpart[p] = a[p].hpart;
+  }
+  if ((rc = launch_shrink_shared(sa, V, L, s)) != TK_OK) return rc;
+  for (int p = 0; p < n; ++p)  // per projection: add the slices (h_p), then y_p += h_p B_p^T
+    if ((rc = launch_pass_mfma(a[p], V, L, 4 | 2, s)) != TK_OK) return rc;
+  return TK_OK;
+}
+
+int tk_lora_bwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* const* dy, const int64_t* lddy,
+                       const void* x, int64_t ldx, const void* const* h, void* dx, int64_t lddx,
+                       void* const* const* grad_A, void* const* const* grad_B, int32_t accumulate, void* const* ws,
+                       const int64_t* ws_bytes, tk_stream_t stream) {
+  if (!shared_descs_ok(descs, n) || !dy || !lddy || !h || !grad_A || !grad_B || !ws || !ws_bytes) return TK_ERR_INVALID;
+  const tk_lora_desc* d0 = descs[0];
+  if (d0->rows == 0) return TK_OK;
+  if (!x || ldx < d0->in_features || !dx || lddx < d0->in_features) return TK_ERR_INVALID;
+  hipStream_t s = (hipStream_t)stream;
+  SegLayout L(d0->rows, d0->num_groups);
+  SegView V(d0->seg_ws, L);
+  BwdPlan plan[TK_MAX_SHARED];
+  bool fast = shared_fast_path(descs, n);
+  for (int p = 0; p < n; ++p) {
+    const tk_lora_desc* d = descs[p];
+    if (!dy[p] || lddy[p] < d->out_features || !h[p] || !grad_A[p] || !grad_B[p] || !ws[p]) return TK_ERR_INVALID;
+    BwdLayout B(*d);
+    if (ws_bytes[p] < B.total) return TK_ERR_WORKSPACE;
+    if (d->max_rank == 0) {
+      fast = false;
+      continue;
+    }
+    plan[p] = bwd_plan(d, B, dy[p], lddy[p], x, ldx, h[p], dx, lddx, grad_A[p], grad_B[p], accumulate, ws[p]);
+    fast = fast && pass_mfma_supported(plan[p].a) && dy_fused_supported(plan[p].gb, plan[p].a.kslices) &&
+           wgrad_mfma_supported(plan[p].ga);
+  }
+  int rc;
+  if (!fast) {
+    for (int p = 0; p < n; ++p)
+      if ((rc = tk_lora_bwd(descs[p], dy[p], lddy[p], x, ldx, h[p], dx, lddx, grad_A[p], grad_B[p], accumulate, ws[p],
+                            ws_bytes[p], stream)) != TK_OK)
+        return rc;
+    return TK_OK;
+  }
+  SharedExpandArgs ea{};
+  ea.dst = dx;  ea.ld_dst = lddx;  ea.width_dst = d0->in_features;  ea.map_rows = d0->map_rows;  ea.nproj = n;
+  SharedWgradArgs wa{};
+  wa.nproj = n;
+  for (int p = 0; p < n; ++p) {
+    BwdPlan& P = plan[p];
+    // dy_p once: dB_p, the slices of dh_p and the A_p^T copy; then dh_p
+    P.gb.tr = P.tr;
+    P.gb.tr.bT = nullptr;
+    rc = launch_dy_fused(P.gb, descs[p]->lora_B, descs[p]->ldb, P.a.hpart, P.a.kslices, V, L, s);
+    P.gb.tr = TransposeJob{};
+    if (rc != TK_OK) return rc;
+    if ((rc = launch_pass_mfma(P.a, V, L, 4, s)) != TK_OK) return rc;
+    ea.hrow[p] = (const char*)P.dh + (int64_t)P.a.rpad * P.a.ldh * 2;  // slot-major half of the dh buffer (bf16)
+    ea.aT[p] = P.aT;
+    ea.rank[p] = descs[p]->rank;
+    wa.w[p] = P.ga;
+  }
+  if ((rc = launch_expand_shared(ea, V, L, s)) != TK_OK) return rc;  // dx += sum_p dh_p A_p
+  if ((rc = launch_wgrad_shared(wa, V, L, s)) != TK_OK) return rc;   // dA_p for all p, x read once
+  for (int p = 0; p < n; ++p)
+    if ((rc = launch_wgrad_reduce(&plan[p].ga, &plan[p].gb, V, L, d0->dtype, s)) != TK_OK) return rc;
+  return TK_OK;
+}
+
 int64_t tk_opt_workspace_bytes(int32_t num_tensors, int64_t max_numel) {
   if (num_tensors < 0 || max_numel < 0) return TK_ERR_INVALID;
   return round_up(4 * opt_partial_floats(num_tensors, max_numel) + 4, 256);

@@ -1,0 +1,396 @@
+// Projections that share their input (q / k / v, gate / up): the parts of the forward and backward
+// passes that touch the shared tensors, done once for all of them.
+//
+//   forward   k_shrink_shared   x is read once and multiplied with every projection's A (the per-projection
+//                               finish and expand kernels follow unchanged)
+//   backward  k_expand_shared   dx += sum_p dh_p A_p in one read-modify-write of dx instead of one per projection
+//             k_wgrad_shared    dA_p = dh_p^T x for every projection from one pass over x
+//
+// Each projection has padded rank 16 here, so projection p is simply block p of 16 rank indices of the
+// single-projection kernels: same operand layouts, same order of every sum, hence the same h, dA and dB bit
+// for bit; only dx differs (one rounding to bf16 instead of one per projection).
+#include "tk_mfma.h"
+
+namespace tk {
+
+namespace {
+
+template <typename T>
+__device__ inline T pick(const T (&v)[kMaxShared], int i) {  // v[i] without a register-indexed array
+  T r = v[0];
+#pragma unroll
+  for (int j = 1; j < kMaxShared; ++j) r = i == j ? v[j] : r;
+  return r;
+}
+
+// ---------------------------------------------------------------------------
+// Shrink of P projections: work item = (two consecutive tiles, 512 source columns), one wave, exactly like
+// k_shrink_pair<1, 1>; the wave keeps one accumulator block per projection and writes one slice of every
+// projection's split-shrink buffer ([tile][slice][32][16] each), which that projection's k_shrink_finish
+// turns into its h.
+// ---------------------------------------------------------------------------
+template <int P, int TT>
+__device__ inline void shrink_tiles_shared(const SharedShrinkArgs& a, const int32_t* __restrict__ slot_rows,
+                                           const int (&tiles)[TT], int g, int ks, float (*part)[16 * P + 1]) {
+  constexpr int PF = 2;  // steps whose loads are issued together
+  const int lane = threadIdx.x & 63, li = lane & 15, kb = lane >> 4;
+  const bf16_t* src = (const bf16_t*)a.src;
+  const bf16_t *xa[TT], *xb[TT];
+#pragma unroll
+  for (int u = 0; u < TT; ++u) {
+    const int slot0 = tiles[u] * kTileRows;
+    int ra = slot_rows[slot0 + li], rb = slot_rows[slot0 + 16 + li];
+    ra = min(max(ra, 0), a.src_rows - 1);  // padding slots read a real row; their h is zeroed by the finish kernel
+    rb = min(max(rb, 0), a.src_rows - 1);
+    xa[u] = src + (int64_t)ra * a.ld_src + 16 * kb;
+    xb[u] = src + (int64_t)rb * a.ld_src + 16 * kb;
+  }
+  const bf16_t* wp[P];
+  bool wv[P];
+  int r[P];
+  bool any = false;
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    r[p] = min(a.rank[p][g], 16);
+    any = any || r[p] > 0;
+    wv[p] = li < r[p];
+    wp[p] = (const bf16_t*)a.w[p][g] + (int64_t)(wv[p] ? li : 0) * a.ld_w[p] + 16 * kb;
+  }
+  f32x4 acc[TT][2][P];
+#pragma unroll
+  for (int u = 0; u < TT; ++u)
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int p = 0; p < P; ++p) acc[u][tt][p] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int nsteps = a.width_src >> 6;
+  const int s_first = ks * kShrinkSteps;
+#pragma unroll
+  for (int b = 0; b < kShrinkSteps / PF; ++b) {
+    uint4 x0[PF][TT][2], x1[PF][TT][2], w0[PF][P], w1[PF][P];
+#pragma unroll
+    for (int j = 0; j < PF; ++j) {
+      const int s = s_first + b * PF + j;
+      const bool ok = s < nsteps;  // wave-uniform
+      const int c = (ok ? s : 0) << 6;
+#pragma unroll
+      for (int u = 0; u < TT; ++u) {
+        x0[j][u][0] = ld16(xa[u] + c);
+        x1[j][u][0] = ld16(xa[u] + c + 8);
+        x0[j][u][1] = ld16(xb[u] + c);
+        x1[j][u][1] = ld16(xb[u] + c + 8);
+      }
+#pragma unroll
+      for (int p = 0; p < P; ++p) {
+        w0[j][p] = (wv[p] && ok) ? ld16(wp[p] + c) : zero4();
+        w1[j][p] = (wv[p] && ok) ? ld16(wp[p] + c + 8) : zero4();
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < PF; ++j)
+#pragma unroll
+      for (int p = 0; p < P; ++p)
+#pragma unroll
+        for (int u = 0; u < TT; ++u)
+#pragma unroll
+          for (int tt = 0; tt < 2; ++tt) {
+            acc[u][tt][p] = mfma16(x0[j][u][tt], w0[j][p], acc[u][tt][p]);
+            acc[u][tt][p] = mfma16(x1[j][u][tt], w1[j][p], acc[u][tt][p]);
+          }
+  }
+  if (!any) return;  // no projection's adapter is live on this layer (uniform over the block)
+#pragma unroll
+  for (int u = 0; u < TT; ++u) {
+    __syncthreads();  // the previous tile's sums have been read
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int p = 0; p < P; ++p)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) part[16 * tt + 4 * kb + v][16 * p + li] = acc[u][tt][p][v];
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      if (r[p] <= 0) continue;
+      float* mine = a.hpart[p] + ((int64_t)tiles[u] * a.kslices + ks) * (kTileRows * 16);
+      for (int idx = lane; idx < kTileRows * 16; idx += 64) mine[idx] = part[idx >> 4][16 * p + (idx & 15)];
+    }
+  }
+}
+
+template <int P>
+__global__ __launch_bounds__(64) void k_shrink_shared(SharedShrinkArgs a, const int32_t* __restrict__ tile_group,
+                                                      const int32_t* __restrict__ slot_rows, int max_tiles) {
+  __shared__ float part[kTileRows][16 * P + 1];
+  const int pair = blockIdx.x / a.kslices, ks = blockIdx.x - pair * a.kslices;
+  const int t0 = 2 * pair, t1 = t0 + 1;
+  const int g0 = tile_group[t0];
+  const int g1 = t1 < max_tiles ? tile_group[t1] : -1;
+  if (g0 >= 0 && g1 == g0) {
+    const int tiles[2] = {t0, t1};
+    shrink_tiles_shared<P, 2>(a, slot_rows, tiles, g0, ks, part);
+    return;
+  }
+  if (g0 >= 0) {
+    const int tiles[1] = {t0};
+    shrink_tiles_shared<P, 1>(a, slot_rows, tiles, g0, ks, part);
+  }
+  if (g1 >= 0) {
+    const int tiles[1] = {t1};
+    shrink_tiles_shared<P, 1>(a, slot_rows, tiles, g1, ks, part);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// dx[row] += sum_p dh_p[row] A_p: the flat expand kernel (one wave = one tile x 128 columns) with the
+// contraction running over the P projections' blocks of 16 rank indices; lane group kb reads block
+// 2 ks + kb / 2 of h (slot-major, [slots][16] per projection) and of the transposed weight copies
+// ([G][K][16] per projection).
+// ---------------------------------------------------------------------------
+template <int P>
+__global__ __launch_bounds__(256) void k_expand_shared(SharedExpandArgs a, const int32_t* __restrict__ tile_group,
+                                                       const int32_t* __restrict__ slot_rows, int num_items) {
+  constexpr int NKS = (16 * P + 31) / 32;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  const int ngroups = a.width_dst >> 7;
+  const int item = blockIdx.x * 4 + wave;
+  if (item >= num_items) return;
+  const int tile_id = item / ngroups;
+  const int c0 = (item - tile_id * ngroups) << 7;
+  const int slot0 = tile_id * kTileRows;
+  const int g_raw = tile_group[tile_id];
+  const int4 r0 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 4 * kb);
+  const int4 r1 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 16 + 4 * kb);
+  const int off = 8 * (kb & 1);  // first rank index of this lane inside its block
+  uint4 hop[2][NKS];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+    const int blk = 2 * ks + (kb >> 1);
+    const bf16_t* hp = (const bf16_t*)pick(a.hrow, blk);
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+      hop[tt][ks] = blk < P ? ld16(hp + (int64_t)(slot0 + 16 * tt + li) * 16 + off) : zero4();
+  }
+  const int g = max(g_raw, 0);
+  const int rows[2][4] = {{r0.x, r0.y, r0.z, r0.w}, {r1.x, r1.y, r1.z, r1.w}};
+  bool rok[2][4];
+  bf16_t* yp[2][4];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      rok[tt][v] = g_raw >= 0 && rows[tt][v] >= 0;
+      yp[tt][v] = (bf16_t*)a.dst + (int64_t)(rok[tt][v] ? rows[tt][v] : 0) * a.ld_dst + 8 * li + c0;
+    }
+  int rblk[NKS];
+  bool any = false;
+#pragma unroll
+  for (int p = 0; p < P; ++p) any = any || (g_raw >= 0 && a.rank[p][g] > 0);
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+    const int blk = 2 * ks + (kb >> 1);
+    rblk[ks] = (blk < P && g_raw >= 0) ? min(pick(a.rank, blk)[g], 16) : 0;
+  }
+  uint4 y[2][4];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) y[tt][v] = rok[tt][v] ? ld16_nt(yp[tt][v]) : zero4();
+  uint4 bq[8][NKS];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+    const int blk = 2 * ks + (kb >> 1);
+    const bf16_t* wt = (const bf16_t*)pick(a.aT, blk) + ((int64_t)g * a.width_dst + c0 + 8 * li) * 16 + off;
+#pragma unroll
+    for (int q = 0; q < 8; ++q)
+      bq[q][ks] = off < rblk[ks] ? keep_first(ld16(wt + (int64_t)q * 16), rblk[ks] - off) : zero4();
+  }
+  if (!any) return;  // unused tile, or no projection live on this layer (uniform over the wave)
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks)  // a projection without this adapter has no dh: never multiply what is there
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) hop[tt][ks] = rblk[ks] > 0 ? hop[tt][ks] : zero4();
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) {
+    f32x4 d[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      d[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks) d[q] = mfma16(hop[tt][ks], bq[q][ks], d[q]);
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      if (!rok[tt][v]) continue;
+      const uint4 yy = y[tt][v];
+      uint4 o;
+      o.x = pack_bf16(bf16_lo(yy.x) + d[0][v], bf16_hi(yy.x) + d[1][v]);
+      o.y = pack_bf16(bf16_lo(yy.y) + d[2][v], bf16_hi(yy.y) + d[3][v]);
+      o.z = pack_bf16(bf16_lo(yy.z) + d[4][v], bf16_hi(yy.z) + d[5][v]);
+      o.w = pack_bf16(bf16_lo(yy.w) + d[6][v], bf16_hi(yy.w) + d[7][v]);
+      st16_nt(yp[tt][v], o);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// dA_p[n][c] = sum over the rows of dh_p[n][slot] x[row(slot)][c] for all projections from one pass over x:
+// k_wgrad_pipe's pipeline and operand layouts with one accumulator block per projection; every block
+// leaves through the same staging buffer into its own projection's partial buffer or gradient.
+// ---------------------------------------------------------------------------
+template <int P>
+__global__ __launch_bounds__(64) void k_wgrad_shared(SharedWgradArgs a, const ChunkInfo* __restrict__ chunks,
+                                                     const int32_t* __restrict__ slot_rows) {
+  constexpr int OS = kWgradStageStride;
+  __shared__ __attribute__((aligned(16))) float lds[16 * OS];
+  const int lane = threadIdx.x & 63, li = lane & 15, kb = lane >> 4;
+  const int c0 = blockIdx.x * 128;
+  const ChunkInfo ci = chunks[blockIdx.y];
+  const int g = ci.group;
+  if (g < 0) return;
+  int r[P];
+  bool any = false;
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    r[p] = min(a.w[p].rank[g], 16);
+    any = any || r[p] > 0;
+  }
+  if (!any) return;
+  const WgradArgs& a0 = a.w[0];
+  const int nt = ci.ntiles;
+  const bf16_t* src = (const bf16_t*)a0.src + c0 + 8 * li;
+  const bf16_t* hT[P];
+#pragma unroll
+  for (int p = 0; p < P; ++p)
+    hT[p] = (const bf16_t*)a.w[p].hT + (int64_t)li * a.w[p].ldh + (int64_t)ci.tile0 * kTileRows + 8 * kb;
+  const int32_t* rows_p = slot_rows + ci.tile0 * kTileRows + 8 * kb;
+  f32x4 acc[8][P];
+#pragma unroll
+  for (int q = 0; q < 8; ++q)
+#pragma unroll
+    for (int p = 0; p < P; ++p) acc[q][p] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  struct Tile {
+    uint4 x[8];
+    uint4 h[P];
+    uint32_t live;
+  };
+  int4 ra, rb;
+  auto load_rows = [&](int t) {
+    const int tc = min(t, nt - 1);
+    ra = *reinterpret_cast<const int4*>(rows_p + tc * kTileRows);
+    rb = *reinterpret_cast<const int4*>(rows_p + tc * kTileRows + 4);
+  };
+  auto issue = [&](int t, Tile& T) {
+    const int tc = min(t, nt - 1);
+    const int rows[8] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w};
+    T.live = 0;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      T.x[q] = ld16(src + (int64_t)max(rows[q], 0) * a0.ld_src);
+      T.live |= (t < nt && rows[q] >= 0) ? (1u << q) : 0u;
+    }
+#pragma unroll
+    for (int p = 0; p < P; ++p) T.h[p] = ld16(hT[p] + tc * kTileRows);
+  };
+  auto consume = [&](const Tile& T) {
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int d = q >> 1;
+      const uint32_t sel = (q & 1) ? 0x07060302u : 0x05040100u;
+      uint32_t e[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t wsrc[4] = {T.x[i].x, T.x[i].y, T.x[i].z, T.x[i].w};
+        e[i] = (T.live >> i) & 1u ? wsrc[d] : 0u;
+      }
+      uint4 tr;
+      tr.x = __builtin_amdgcn_perm(e[1], e[0], sel);
+      tr.y = __builtin_amdgcn_perm(e[3], e[2], sel);
+      tr.z = __builtin_amdgcn_perm(e[5], e[4], sel);
+      tr.w = __builtin_amdgcn_perm(e[7], e[6], sel);
+#pragma unroll
+      for (int p = 0; p < P; ++p) acc[q][p] = mfma16(tr, T.h[p], acc[q][p]);
+    }
+  };
+  Tile A, B, C;
+  load_rows(0);
+  issue(0, A);
+  load_rows(1);
+  issue(1, B);
+  load_rows(2);
+  int t = 0;
+  for (; t + 4 < nt; t += 3) {  // every tile touched in here exists
+    issue(t + 2, C);
+    load_rows(t + 3);
+    consume(A);
+    issue(t + 3, A);
+    load_rows(t + 4);
+    consume(B);
+    issue(t + 4, B);
+    load_rows(t + 5);
+    consume(C);
+  }
+  issue(t + 2, C);
+  load_rows(t + 3);
+  consume(A);
+  consume(B);
+  consume(C);
+  if (t + 3 < nt) {
+    issue(t + 3, A);
+    consume(A);
+  }
+#pragma unroll
+  for (int p = 0; p < P; ++p) {
+    if (r[p] <= 0) continue;
+    f32x4 one[8][1];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) one[q][0] = acc[q][p];
+    wgrad_store<1>(one, lds, a.w[p], ci, g, r[p], c0, lane);
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");  // the staging buffer is read before the next block overwrites it
+  }
+}
+
+}  // namespace
+
+int launch_shrink_shared(const SharedShrinkArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
+  if (L.rows == 0) return TK_OK;
+  const dim3 grid((unsigned)(ceil_div(L.max_tiles, 2) * a.kslices));
+  const int32_t* rows = seg.slot_table(a.map_rows);
+  if (a.nproj == 2)
+    hipLaunchKernelGGL(k_shrink_shared<2>, grid, dim3(64), 0, s, a, seg.tile_group, rows, (int)L.max_tiles);
+  else if (a.nproj == 3)
+    hipLaunchKernelGGL(k_shrink_shared<3>, grid, dim3(64), 0, s, a, seg.tile_group, rows, (int)L.max_tiles);
+  else
+    hipLaunchKernelGGL(k_shrink_shared<4>, grid, dim3(64), 0, s, a, seg.tile_group, rows, (int)L.max_tiles);
+  return check_launch();
+}
+
+int launch_expand_shared(const SharedExpandArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
+  if (L.rows == 0) return TK_OK;
+  const int64_t items = L.max_tiles * (a.width_dst >> 7);
+  const dim3 grid((unsigned)ceil_div(items, 4));
+  const int32_t* rows = seg.slot_table(a.map_rows);
+  if (a.nproj == 2)
+    hipLaunchKernelGGL(k_expand_shared<2>, grid, dim3(256), 0, s, a, seg.tile_group, rows, (int)items);
+  else if (a.nproj == 3)
+    hipLaunchKernelGGL(k_expand_shared<3>, grid, dim3(256), 0, s, a, seg.tile_group, rows, (int)items);
+  else
+    hipLaunchKernelGGL(k_expand_shared<4>, grid, dim3(256), 0, s, a, seg.tile_group, rows, (int)items);
+  return check_launch();
+}
+
+int launch_wgrad_shared(const SharedWgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
+  if (L.rows == 0) return TK_OK;
+  const dim3 grid((unsigned)(a.w[0].width / 128), (unsigned)L.max_chunks);
+  const int32_t* rows = seg.slot_table(a.w[0].map_rows);
+  if (a.nproj == 2)
+    hipLaunchKernelGGL(k_wgrad_shared<2>, grid, dim3(64), 0, s, a, seg.chunks, rows);
+  else if (a.nproj == 3)
+    hipLaunchKernelGGL(k_wgrad_shared<3>, grid, dim3(64), 0, s, a, seg.chunks, rows);
+  else
+    hipLaunchKernelGGL(k_wgrad_shared<4>, grid, dim3(64), 0, s, a, seg.chunks, rows);
+  return check_launch();
+}
+
+}  // namespace tk

@@ -221,6 +221,31 @@ struct WgradArgs {
   TransposeJob tr;
 };
 
+// Projections that share their input (kernels_shared.hip); every projection has padded rank 16 there.
+constexpr int kMaxShared = 4;
+struct SharedShrinkArgs {
+  const void* src;  int64_t ld_src;      // x
+  int32_t width_src, src_rows, map_rows, kslices, nproj;
+  const void* const* w[kMaxShared];      // device pointer tables [G] of A_p, rank-major [r][K]
+  int64_t ld_w[kMaxShared];
+  const int32_t* rank[kMaxShared];       // device [G]
+  float* hpart[kMaxShared];              // split-shrink buffer of projection p, [tile][slice][32][16]
+};
+struct SharedExpandArgs {
+  void* dst;  int64_t ld_dst;            // dx
+  int32_t width_dst, map_rows, nproj;
+  const void* hrow[kMaxShared];          // slot-major dh of projection p, [slots][16]
+  const void* aT[kMaxShared];            // A_p^T copies, [G][K][16]
+  const int32_t* rank[kMaxShared];
+};
+struct SharedWgradArgs {                 // dA_p for all p from one pass over x (w[p].src / ld_src / width agree)
+  int32_t nproj;
+  WgradArgs w[kMaxShared];
+};
+int launch_shrink_shared(const SharedShrinkArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
+int launch_expand_shared(const SharedExpandArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
+int launch_wgrad_shared(const SharedWgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
+
 // kernels_segments.hip
 int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t groups, int64_t* perm_out,
                          int64_t* offsets_out, void* ws, hipStream_t s);

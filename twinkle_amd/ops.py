@@ -8,7 +8,7 @@ is what the reference's patched forward computes with two ``F.linear`` calls
 from __future__ import annotations
 
 import ctypes
-from typing import List, Optional, Sequence
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
@@ -285,3 +285,100 @@ def multi_lora_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torc
                       groups: AdapterGroups, map_rows: bool = True) -> torch.Tensor:
     """``F.linear(x, weight, bias)`` plus the segmented LoRA update as one autograd node."""
     return _LoraLinear.apply(x, weight, bias, seg, groups, map_rows, *groups.a_tensors, *groups.b_tensors)
+
+
+# ---- projections that share their input (q / k / v, gate / up) ----------------------------------------------
+
+def _host_array(ctype, values):
+    return (ctype * len(values))(*values)
+
+
+def _shared_descs(seg: SegmentTable, groups_list: Sequence[AdapterGroups], map_rows: bool):
+    if not 1 <= len(groups_list) <= 4:
+        raise ValueError(f'1 to 4 projections can share an input, got {len(groups_list)}')
+    g0 = groups_list[0]
+    for g in groups_list:
+        if g.num_groups != seg.num_groups:
+            raise ValueError(f'segment table has {seg.num_groups} groups, adapters have {g.num_groups}')
+        if g.in_features != g0.in_features or g.dtype != g0.dtype:
+            raise ValueError('projections that share an input must agree in in_features and dtype')
+    descs = [_desc(seg, g, map_rows) for g in groups_list]
+    table = _host_array(ctypes.c_void_p, [ctypes.addressof(d) for d in descs])
+    return descs, table
+
+
+def lora_fwd_shared_(x: torch.Tensor, ys: Sequence[torch.Tensor], seg: SegmentTable,
+                     groups_list: Sequence[AdapterGroups], map_rows: bool = True) -> List[torch.Tensor]:
+    """In place ``ys[p] += lora_p(x)`` for projections that read the same ``x``; returns their saved ``h``."""
+    descs, table = _shared_descs(seg, groups_list, map_rows)
+    _check_rows(x, 'x', seg.rows, groups_list[0].in_features, groups_list[0].dtype)
+    for y, g in zip(ys, groups_list):
+        _check_rows(y, 'y', seg.rows, g.out_features, g.dtype)
+    hs = [torch.empty(lora_h_bytes(seg, g), dtype=torch.uint8, device=x.device) for g in groups_list]
+    code = _lib.load().tk_lora_fwd_shared(
+        table, len(descs), x.data_ptr(), x.stride(0), _host_array(ctypes.c_void_p, [y.data_ptr() for y in ys]),
+        _host_array(ctypes.c_int64, [y.stride(0) for y in ys]), _host_array(ctypes.c_void_p, [h.data_ptr() for h in hs]),
+        _lib.stream_ptr())
+    _lib.check(code, 'tk_lora_fwd_shared')
+    return hs
+
+
+def lora_bwd_shared_(dys: Sequence[torch.Tensor], x: torch.Tensor, hs: Sequence[torch.Tensor], dx: torch.Tensor,
+                     grad_a_ptrs: Sequence[torch.Tensor], grad_b_ptrs: Sequence[torch.Tensor], seg: SegmentTable,
+                     groups_list: Sequence[AdapterGroups], map_rows: bool = True, accumulate: bool = False) -> None:
+    """``dx += sum_p dx_p`` in place and every projection's weight gradients (see ``tk_lora_bwd_shared``)."""
+    descs, table = _shared_descs(seg, groups_list, map_rows)
+    _check_rows(x, 'x', seg.rows, groups_list[0].in_features, groups_list[0].dtype)
+    _check_rows(dx, 'dx', seg.rows, groups_list[0].in_features, groups_list[0].dtype)
+    for dy, g in zip(dys, groups_list):
+        _check_rows(dy, 'dy', seg.rows, g.out_features, g.dtype)
+    wss = [torch.empty(lora_bwd_workspace_bytes(seg, g), dtype=torch.uint8, device=x.device) for g in groups_list]
+    code = _lib.load().tk_lora_bwd_shared(
+        table, len(descs), _host_array(ctypes.c_void_p, [t.data_ptr() for t in dys]),
+        _host_array(ctypes.c_int64, [t.stride(0) for t in dys]), x.data_ptr(), x.stride(0),
+        _host_array(ctypes.c_void_p, [h.data_ptr() for h in hs]), dx.data_ptr(), dx.stride(0),
+        _host_array(ctypes.c_void_p, [t.data_ptr() for t in grad_a_ptrs]),
+        _host_array(ctypes.c_void_p, [t.data_ptr() for t in grad_b_ptrs]), 1 if accumulate else 0,
+        _host_array(ctypes.c_void_p, [w.data_ptr() for w in wss]), _host_array(ctypes.c_int64, [w.numel() for w in wss]),
+        _lib.stream_ptr())
+    _lib.check(code, 'tk_lora_bwd_shared')
+
+
+class _LoraDeltaShared(torch.autograd.Function):
+    """Several base outputs of one input updated in place by their own adapters, as one node."""
+
+    @staticmethod
+    def forward(ctx, x, seg, groups_list, map_rows, n, *rest):
+        ys = rest[:n]
+        hs = lora_fwd_shared_(x, ys, seg, groups_list, map_rows)
+        ctx.mark_dirty(*ys)
+        ctx.save_for_backward(x, *hs)
+        ctx.seg, ctx.groups_list, ctx.map_rows, ctx.n = seg, groups_list, map_rows, n
+        return tuple(ys)
+
+    @staticmethod
+    def backward(ctx, *dys):
+        x, *hs = ctx.saved_tensors
+        seg, groups_list, n = ctx.seg, ctx.groups_list, ctx.n
+        dys = [torch.zeros(seg.rows, g.out_features, dtype=g.dtype, device=x.device) if dy is None else dy.contiguous()
+               for dy, g in zip(dys, groups_list)]
+        dx = torch.zeros_like(x)
+        arenas = [_weight_grads(g, True, True, x.device) for g in groups_list]
+        lora_bwd_shared_(dys, x, hs, dx, [a[2] for a in arenas], [a[3] for a in arenas], seg, groups_list, ctx.map_rows)
+        grads = []
+        for g, (arena_a, arena_b, _, _) in zip(groups_list, arenas):
+            grads += g.grad_views(arena_a, 'a') + g.grad_views(arena_b, 'b')
+        return (dx if ctx.needs_input_grad[0] else None, None, None, None, None, *dys, *grads)
+
+
+def multi_lora_delta_shared(x: torch.Tensor, base_outs: Sequence[torch.Tensor], seg: SegmentTable,
+                            groups_list: Sequence[AdapterGroups], map_rows: bool = True) -> Tuple[torch.Tensor, ...]:
+    """:func:`multi_lora_delta` for projections that read the same ``x`` (q / k / v, gate / up).
+
+    ``base_outs[p]`` gets the LoRA term of ``groups_list[p]`` added in place.  ``x`` and, in backward, the
+    gradient of ``x`` cross memory once for all projections instead of once per projection.
+    """
+    weights = []
+    for g in groups_list:
+        weights += list(g.a_tensors) + list(g.b_tensors)
+    return _LoraDeltaShared.apply(x, seg, tuple(groups_list), map_rows, len(groups_list), *base_outs, *weights)
