@@ -156,6 +156,63 @@ def optimizer_step_bench(dev, steps=10):
                     'per tenant grad.div_, clip_grad_norm_, fused AdamW (bf16 moments), zero_grad'}
 
 
+def shared_qkv_bench(dev, steps=20):
+    """q / k / v of one attention block (4096 -> 4096, 1024, 1024; config 2's tokens, adapters and ids):
+    one shared call against one call per projection, forward + backward, segment table built once."""
+    import torch
+    from twinkle_amd import (AdapterGroups, build_segments, lora_bwd_, lora_bwd_shared_, lora_bwd_workspace_bytes,
+                             lora_fwd_, lora_fwd_shared_, lora_h_bytes, workloads)
+    w = workloads.config2_qproj()
+    dt, T, K, G = torch.bfloat16, w.tokens, w.in_features, w.num_adapters
+    outs = (4096, 1024, 1024)
+    gen = torch.Generator().manual_seed(11)
+    x = w.x.to(dt).to(dev)
+    seg = build_segments(w.ids.to(dev), G, want_perm=False, want_offsets=False)
+    groups, ys, dys, pas, pbs, keep = [], [], [], [], [], []
+    for m in outs:
+        A = [(torch.randn(16, K, generator=gen) / K**0.5).to(dt).to(dev) for _ in range(G)]
+        B = [(torch.randn(m, 16, generator=gen) * 0.05).to(dt).to(dev) for _ in range(G)]
+        groups.append(AdapterGroups(A, B, w.ranks, w.scales))
+        ys.append(torch.randn(T, m, generator=gen).to(dt).to(dev))
+        dys.append(torch.randn(T, m, generator=gen).to(dt).to(dev))
+        ga, gb = [torch.zeros_like(t) for t in A], [torch.zeros_like(t) for t in B]
+        keep.append((ga, gb))
+        pas.append(torch.tensor([t.data_ptr() for t in ga], dtype=torch.int64, device=dev))
+        pbs.append(torch.tensor([t.data_ptr() for t in gb], dtype=torch.int64, device=dev))
+    dx = torch.zeros(T, K, dtype=dt, device=dev)
+    hs = [torch.empty(lora_h_bytes(seg, g), dtype=torch.uint8, device=dev) for g in groups]
+    wss = [torch.empty(lora_bwd_workspace_bytes(seg, g), dtype=torch.uint8, device=dev) for g in groups]
+
+    def separate():
+        for y, h, g in zip(ys, hs, groups):
+            lora_fwd_(x, y, seg, g, h=h)
+        for dy, h, pa, pb, g, ws in zip(dys, hs, pas, pbs, groups, wss):
+            lora_bwd_(dy, x, h, dx, pa, pb, seg, g, workspace=ws)
+
+    def shared():
+        lora_fwd_shared_(x, ys, seg, groups, hs=hs)
+        lora_bwd_shared_(dys, x, hs, dx, pas, pbs, seg, groups, workspaces=wss)
+
+    res = {}
+    for name, fn in (('one_call_per_projection_ms', separate), ('shared_ms', shared)):
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        res[name] = (time.perf_counter() - t0) * 1e3 / steps
+    elt = 2
+    per_proj = sum(elt * T * (4 * m + 3 * K) for m in outs)            # y rw, dy r | x r (fwd, dA), dx rw
+    joint = sum(elt * T * 4 * m for m in outs) + elt * T * 4 * K       # x r twice, dx rw once
+    res.update({'workload': f'T={T}, {K} -> {outs}, {G} adapters rank 16, fwd + bwd, segment table prebuilt',
+                'algorithmic_bytes_one_call_per_projection': per_proj, 'algorithmic_bytes_shared': joint,
+                'speedup': res['one_call_per_projection_ms'] / res['shared_ms'],
+                'hbm_frac_shared': joint / (res['shared_ms'] * 1e-3) / 1e9 / HBM_PEAK_GBS})
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -172,6 +229,8 @@ def main():
                          'of rank 64, one per packed 4096-token sequence) for additional measurements')
     ap.add_argument('--optimizer-only', action='store_true',
                     help='run only the multi-tenant optimizer micro-benchmark and print its JSON (for profiling)')
+    ap.add_argument('--shared-qkv', action='store_true',
+                    help='run only the q / k / v micro-benchmark (one shared call against one call per projection)')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run five plain 128 MiB device copies (a known-size kernel to scale rocprofv3 --pmc '
                          'FETCH_SIZE / WRITE_SIZE readings by)')
@@ -191,6 +250,9 @@ def main():
     dev = torch.device('cuda:0')
     if args.optimizer_only:
         print(json.dumps({'optimizer_step': optimizer_step_bench(dev)}))
+        return
+    if args.shared_qkv:
+        print(json.dumps({'shared_qkv': shared_qkv_bench(dev)}))
         return
     if args.workload == 'cfg2':
         w = workloads.config2_qproj()

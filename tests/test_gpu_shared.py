@@ -113,3 +113,67 @@ def test_shared_argument_errors(dev):
         multi_lora_delta_shared(x, y * 3, seg, grp * 3)           # more than four projections
     with pytest.raises(ValueError):
         multi_lora_delta_shared(x, [y[0], y[1][:, :256]], seg, grp)  # an output of the wrong width
+
+
+# ---- through the MultiLora mirror: q / k / v of one block routed through forward_shared --------------------
+
+class _QKV(torch.nn.Module):
+
+    def __init__(self, d, kv):
+        super().__init__()
+        self.q_proj = torch.nn.Linear(d, d, bias=True)
+        self.k_proj = torch.nn.Linear(d, kv, bias=False)
+        self.v_proj = torch.nn.Linear(d, kv, bias=False)
+
+    def forward(self, x):
+        return self.q_proj(x), self.k_proj(x), self.v_proj(x)
+
+
+@pytest.mark.parametrize('dtype,d,kv', [(torch.bfloat16, 2048, 512), (torch.float32, 128, 64)])
+def test_forward_shared_equals_layer_by_layer(dev, dtype, d, kv):
+    from twinkle_amd import LoraConfig, MultiLora
+    torch.manual_seed(0)
+    ml = MultiLora(max_loras=4, max_r=16)
+    model = ml.patch(_QKV(d, kv).to(dtype).to(dev), target_modules='all-linear')
+    ml.acquire_lora('alice', LoraConfig(r=8, lora_alpha=16, target_modules='all-linear'))
+    ml.acquire_lora('bob', LoraConfig(r=16, lora_alpha=32, target_modules=['q_proj', 'v_proj']))   # k_proj not targeted
+    ml.acquire_lora('carol', LoraConfig(r=4, lora_alpha=16, target_modules='all-linear', use_rslora=True))
+    g = torch.Generator().manual_seed(1)
+    with torch.no_grad():
+        for n, p in model.named_parameters():
+            if '.lora_B.' in n:
+                p.copy_((torch.randn(p.shape, generator=g) * 0.05).to(dtype))
+    x = torch.randn(2, 150, d, generator=g).to(dtype).to(dev)
+    row_tenant = torch.randint(0, 3, (300,), generator=g).to(dev)
+    wq, wk, wv = (torch.randn(2, 150, n, generator=g).to(dtype).to(dev) for n in (d, kv, kv))
+    m = model.model
+    layers = [m.q_proj, m.k_proj, m.v_proj]
+
+    def run(shared):
+        for p in model.parameters():
+            p.grad = None
+        xi = x.clone().requires_grad_(True)
+        with ml.batch(['alice', 'bob', 'carol'], row_tenant):
+            q, k, v = ml.forward_shared(layers, xi) if shared else model(xi)
+            ((q * wq).sum() + (k * wk).sum() + (v * wv).sum()).backward()
+        grads = {n: p.grad.clone() for n, p in model.named_parameters() if p.grad is not None}
+        return (q, k, v), xi.grad, grads
+
+    (q0, k0, v0), dx0, g0 = run(False)
+    (q1, k1, v1), dx1, g1 = run(True)
+    bf16 = dtype == torch.bfloat16
+    for a, b in ((q0, q1), (k0, k1), (v0, v1)):
+        assert torch.equal(a, b) if bf16 else max_rel_err(b, a) < 1e-6
+    assert g0.keys() == g1.keys()
+    for n in g0:
+        assert (torch.equal(g0[n], g1[n]) if bf16 and 'lora_' in n else max_rel_err(g1[n], g0[n].double()) < 1e-5), n
+    assert max_rel_err(dx1, dx0.double()) < (2e-2 if bf16 else 1e-5)
+    # one adapter per call (the reference's adapter() context) takes the same route
+    with ml.adapter('carol'):
+        a = ml.forward_shared(layers, x)
+        b = model(x)
+    for u, w in zip(a, b):
+        assert torch.equal(u, w) if bf16 else max_rel_err(u, w) < 1e-6
+    with ml.adapter('carol', disable_lora=True):
+        a = ml.forward_shared(layers, x)
+    assert torch.equal(a[1], torch.nn.functional.linear(x, m.k_proj.base_layer.weight))

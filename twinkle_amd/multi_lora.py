@@ -17,12 +17,12 @@ import re
 from contextlib import contextmanager
 from dataclasses import dataclass, field
 from types import MethodType
-from typing import Any, Dict, List, Optional, Sequence, Union
+from typing import Any, Dict, List, Optional, Sequence, Tuple, Union
 
 import torch
 
 from .lora_layer import LoraConfig, LoraLinear, LoraModel, inject_adapter
-from .ops import AdapterGroups, multi_lora_delta, multi_lora_linear
+from .ops import AdapterGroups, multi_lora_delta, multi_lora_linear, multi_lora_linear_shared
 from .segments import SegmentTable, build_segments
 
 
@@ -274,6 +274,51 @@ class MultiLora:
 
         base_layer.forward = MethodType(_linear_forward, base_layer)
         base_layer.layer_name = name
+
+    def forward_shared(self, layers: Sequence, x: torch.Tensor) -> Tuple[torch.Tensor, ...]:
+        """``tuple(layer(x) for layer in layers)`` for patched layers that read the same ``x`` (q / k / v,
+        gate / up), with the LoRA terms of all of them computed by one shared call: ``x`` is read once in
+        forward, and once in backward for every layer's dA, and the gradient of ``x`` is updated once.
+
+        The reference has no per-input entry (every projection runs its own two ``F.linear`` calls, :322-326);
+        a caller opts in by routing such a group of projections through this method.  Falls back to calling
+        the layers one by one whenever one of them would not take the plain in-place path (adapters disabled,
+        a layer without a live adapter, dtype casts, non-``nn.Linear`` base layers).
+        """
+        layers = list(layers)
+        table = self._batch_table
+        only_slot = None
+        ok = 2 <= len(layers) <= 4 and x.is_cuda
+        groups_list = []
+        for layer in layers if ok else ():
+            if table is None:
+                active = [n for n in layer.active_adapters if n in layer.lora_A.keys()]
+                slot = active[0] if active else None
+                if slot is None or (only_slot is not None and slot != only_slot):
+                    ok = False
+                    break
+                only_slot = slot
+            groups = None if layer.disable_adapters else self._groups_for(layer, only_slot)
+            base = layer.base_layer
+            slot_for_dropout = only_slot if only_slot is not None else self.loras[0].adapter_name
+            if (groups is None or groups.dtype != x.dtype or type(base) is not torch.nn.Linear
+                    or base.weight.dtype != x.dtype or base._forward_hooks or base._forward_pre_hooks
+                    or not isinstance(layer.lora_dropout[slot_for_dropout], torch.nn.Identity)):
+                ok = False
+                break
+            groups_list.append(groups)
+        if not ok:
+            return tuple(layer(x) for layer in layers)
+        x2 = x.reshape(-1, x.shape[-1])
+        if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
+            x2 = x2.contiguous()
+        if table is None:
+            table = self._table_for(x2.shape[0], self.find_lora(only_slot).index, x2.device)
+        elif table.rows != x2.shape[0]:
+            raise ValueError(f'batch() was given {table.rows} rows but the shared input has {x2.shape[0]}')
+        outs = multi_lora_linear_shared(x2, [layer.base_layer.weight for layer in layers],
+                                        [layer.base_layer.bias for layer in layers], table, groups_list)
+        return tuple(y.view(*x.shape[:-1], y.shape[-1]) for y in outs)
 
     def patch(self, module, target_modules='all-linear', *args, **kwargs):
         """Pre-allocate ``max_loras`` slots of rank ``max_r`` on ``module`` and patch every LoRA layer.

@@ -308,31 +308,36 @@ def _shared_descs(seg: SegmentTable, groups_list: Sequence[AdapterGroups], map_r
 
 
 def lora_fwd_shared_(x: torch.Tensor, ys: Sequence[torch.Tensor], seg: SegmentTable,
-                     groups_list: Sequence[AdapterGroups], map_rows: bool = True) -> List[torch.Tensor]:
+                     groups_list: Sequence[AdapterGroups], map_rows: bool = True,
+                     hs: Optional[Sequence[torch.Tensor]] = None) -> List[torch.Tensor]:
     """In place ``ys[p] += lora_p(x)`` for projections that read the same ``x``; returns their saved ``h``."""
     descs, table = _shared_descs(seg, groups_list, map_rows)
     _check_rows(x, 'x', seg.rows, groups_list[0].in_features, groups_list[0].dtype)
     for y, g in zip(ys, groups_list):
         _check_rows(y, 'y', seg.rows, g.out_features, g.dtype)
-    hs = [torch.empty(lora_h_bytes(seg, g), dtype=torch.uint8, device=x.device) for g in groups_list]
+    if hs is None:
+        hs = [torch.empty(lora_h_bytes(seg, g), dtype=torch.uint8, device=x.device) for g in groups_list]
     code = _lib.load().tk_lora_fwd_shared(
         table, len(descs), x.data_ptr(), x.stride(0), _host_array(ctypes.c_void_p, [y.data_ptr() for y in ys]),
         _host_array(ctypes.c_int64, [y.stride(0) for y in ys]), _host_array(ctypes.c_void_p, [h.data_ptr() for h in hs]),
         _lib.stream_ptr())
     _lib.check(code, 'tk_lora_fwd_shared')
-    return hs
+    return list(hs)
 
 
 def lora_bwd_shared_(dys: Sequence[torch.Tensor], x: torch.Tensor, hs: Sequence[torch.Tensor], dx: torch.Tensor,
                      grad_a_ptrs: Sequence[torch.Tensor], grad_b_ptrs: Sequence[torch.Tensor], seg: SegmentTable,
-                     groups_list: Sequence[AdapterGroups], map_rows: bool = True, accumulate: bool = False) -> None:
+                     groups_list: Sequence[AdapterGroups], map_rows: bool = True, accumulate: bool = False,
+                     workspaces: Optional[Sequence[torch.Tensor]] = None) -> None:
     """``dx += sum_p dx_p`` in place and every projection's weight gradients (see ``tk_lora_bwd_shared``)."""
     descs, table = _shared_descs(seg, groups_list, map_rows)
     _check_rows(x, 'x', seg.rows, groups_list[0].in_features, groups_list[0].dtype)
     _check_rows(dx, 'dx', seg.rows, groups_list[0].in_features, groups_list[0].dtype)
     for dy, g in zip(dys, groups_list):
         _check_rows(dy, 'dy', seg.rows, g.out_features, g.dtype)
-    wss = [torch.empty(lora_bwd_workspace_bytes(seg, g), dtype=torch.uint8, device=x.device) for g in groups_list]
+    wss = workspaces
+    if wss is None:
+        wss = [torch.empty(lora_bwd_workspace_bytes(seg, g), dtype=torch.uint8, device=x.device) for g in groups_list]
     code = _lib.load().tk_lora_bwd_shared(
         table, len(descs), _host_array(ctypes.c_void_p, [t.data_ptr() for t in dys]),
         _host_array(ctypes.c_int64, [t.stride(0) for t in dys]), x.data_ptr(), x.stride(0),
@@ -382,3 +387,50 @@ def multi_lora_delta_shared(x: torch.Tensor, base_outs: Sequence[torch.Tensor], 
     for g in groups_list:
         weights += list(g.a_tensors) + list(g.b_tensors)
     return _LoraDeltaShared.apply(x, seg, tuple(groups_list), map_rows, len(groups_list), *base_outs, *weights)
+
+
+class _LoraLinearShared(torch.autograd.Function):
+    """Base ``F.linear`` of several projections of one input and their LoRA updates as one node: in backward
+    the base GEMMs accumulate into one ``dx``, which the shared LoRA backward then updates in place."""
+
+    @staticmethod
+    def forward(ctx, x, seg, groups_list, map_rows, n, has_bias, *rest):
+        weights, biases = rest[:n], rest[n:2 * n]
+        ys = [torch.nn.functional.linear(x, w, b if hb else None) for w, b, hb in zip(weights, biases, has_bias)]
+        hs = lora_fwd_shared_(x, ys, seg, groups_list, map_rows)
+        ctx.save_for_backward(x, *weights, *hs)
+        ctx.seg, ctx.groups_list, ctx.map_rows, ctx.n, ctx.has_bias = seg, groups_list, map_rows, n, has_bias
+        return tuple(ys)
+
+    @staticmethod
+    def backward(ctx, *dys):
+        n, seg, groups_list = ctx.n, ctx.seg, ctx.groups_list
+        x, *rest = ctx.saved_tensors
+        weights, hs = rest[:n], rest[n:]
+        dys = [torch.zeros(seg.rows, g.out_features, dtype=g.dtype, device=x.device) if dy is None else dy.contiguous()
+               for dy, g in zip(dys, groups_list)]
+        dx = dys[0] @ weights[0]
+        for dy, w in zip(dys[1:], weights[1:]):
+            dx.addmm_(dy, w)
+        dws = [dy.t() @ x if ctx.needs_input_grad[6 + p] else None for p, dy in enumerate(dys)]
+        dbs = [dy.sum(0) if ctx.has_bias[p] and ctx.needs_input_grad[6 + n + p] else None for p, dy in enumerate(dys)]
+        arenas = [_weight_grads(g, True, True, x.device) for g in groups_list]
+        lora_bwd_shared_(dys, x, hs, dx, [a[2] for a in arenas], [a[3] for a in arenas], seg, groups_list, ctx.map_rows)
+        grads = []
+        for g, (arena_a, arena_b, _, _) in zip(groups_list, arenas):
+            grads += g.grad_views(arena_a, 'a') + g.grad_views(arena_b, 'b')
+        return (dx if ctx.needs_input_grad[0] else None, None, None, None, None, None, *dws, *dbs, *grads)
+
+
+def multi_lora_linear_shared(x: torch.Tensor, weights: Sequence[torch.Tensor],
+                             biases: Sequence[Optional[torch.Tensor]], seg: SegmentTable,
+                             groups_list: Sequence[AdapterGroups], map_rows: bool = True) -> Tuple[torch.Tensor, ...]:
+    """:func:`multi_lora_linear` for projections that read the same ``x``: ``F.linear(x, weights[p], biases[p])``
+    plus the segmented LoRA update of ``groups_list[p]``, all projections in one autograd node."""
+    has_bias = tuple(b is not None for b in biases)
+    dummies = [b if b is not None else x.new_zeros(0) for b in biases]
+    lora = []
+    for g in groups_list:
+        lora += list(g.a_tensors) + list(g.b_tensors)
+    return _LoraLinearShared.apply(x, seg, tuple(groups_list), map_rows, len(groups_list), has_bias, *weights, *dummies,
+                                   *lora)
