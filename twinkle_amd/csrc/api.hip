@@ -402,9 +402,8 @@ int tk_lora_fwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* 
     sa.rank[p] = descs[p]->rank;  sa.hpart[p] = a[p].hpart;
   }
   if ((rc = launch_shrink_shared(sa, V, L, s)) != TK_OK) return rc;
-  for (int p = 0; p < n; ++p)  // per projection: add the slices (h_p), then y_p += h_p B_p^T
-    if ((rc = launch_pass_mfma(a[p], V, L, 4 | 2, s)) != TK_OK) return rc;
-  return TK_OK;
+  // every projection in one launch each: add the slices (h_p), then y_p += h_p B_p^T
+  return launch_pass_multi(a, n, V, L, 4 | 2, s);
 }
 
 int tk_lora_bwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* const* dy, const int64_t* lddy,
@@ -445,25 +444,30 @@ int tk_lora_bwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* 
   ea.dst = dx;  ea.ld_dst = lddx;  ea.width_dst = d0->in_features;  ea.map_rows = d0->map_rows;  ea.nproj = n;
   SharedWgradArgs wa{};
   wa.nproj = n;
+  DyFusedJob dj[TK_MAX_SHARED];
+  PassArgs pa[TK_MAX_SHARED];
+  WgradArgs red[2 * TK_MAX_SHARED];
   for (int p = 0; p < n; ++p) {
     BwdPlan& P = plan[p];
-    // dy_p once: dB_p, the slices of dh_p and the A_p^T copy; then dh_p
-    P.gb.tr = P.tr;
-    P.gb.tr.bT = nullptr;
-    rc = launch_dy_fused(P.gb, descs[p]->lora_B, descs[p]->ldb, P.a.hpart, P.a.kslices, V, L, s);
-    P.gb.tr = TransposeJob{};
-    if (rc != TK_OK) return rc;
-    if ((rc = launch_pass_mfma(P.a, V, L, 4, s)) != TK_OK) return rc;
+    dj[p].a = P.gb;
+    dj[p].a.tr = P.tr;
+    dj[p].a.tr.bT = nullptr;  // the fused kernel reads B_p where it lies
+    dj[p].lora_B = descs[p]->lora_B;  dj[p].ldb = descs[p]->ldb;
+    dj[p].hpart = P.a.hpart;  dj[p].kslices = P.a.kslices;
+    pa[p] = P.a;
     ea.hrow[p] = (const char*)P.dh + (int64_t)P.a.rpad * P.a.ldh * 2;  // slot-major half of the dh buffer (bf16)
     ea.aT[p] = P.aT;
     ea.rank[p] = descs[p]->rank;
     wa.w[p] = P.ga;
+    red[2 * p] = P.ga;
+    red[2 * p + 1] = P.gb;
   }
+  // every dy_p once: dB_p, the slices of dh_p and the A_p^T copies; then every dh_p
+  if ((rc = launch_dy_fused_multi(dj, n, V, L, s)) != TK_OK) return rc;
+  if ((rc = launch_pass_multi(pa, n, V, L, 4, s)) != TK_OK) return rc;
   if ((rc = launch_expand_shared(ea, V, L, s)) != TK_OK) return rc;  // dx += sum_p dh_p A_p
   if ((rc = launch_wgrad_shared(wa, V, L, s)) != TK_OK) return rc;   // dA_p for all p, x read once
-  for (int p = 0; p < n; ++p)
-    if ((rc = launch_wgrad_reduce(&plan[p].ga, &plan[p].gb, V, L, d0->dtype, s)) != TK_OK) return rc;
-  return TK_OK;
+  return launch_wgrad_reduce_multi(red, 2 * n, V, L, s);
 }
 
 int64_t tk_opt_workspace_bytes(int32_t num_tensors, int64_t max_numel) {

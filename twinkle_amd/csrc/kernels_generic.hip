@@ -188,15 +188,10 @@ __global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkI
 // of single elements; blockIdx.z >= rpad / 8 selects the second argument set,
 // so that the reductions of dA and dB share one launch.
 template <typename T>
-__global__ __launch_bounds__(256) void k_wgrad_reduce(WgradArgs a0, WgradArgs a1, int rpad,
-                                                      const int32_t* __restrict__ chunk_first,
-                                                      const int32_t* __restrict__ partial_first) {
-  const int zsets = rpad >> 3;
-  const bool second = (int)blockIdx.z >= zsets;
-  const WgradArgs& a = second ? a1 : a0;
+__device__ __forceinline__ void wgrad_reduce_body(const WgradArgs& a, int n0, const int32_t* __restrict__ chunk_first,
+                                                  const int32_t* __restrict__ partial_first) {
   if (a.grad == nullptr) return;
   const int g = blockIdx.x;
-  const int n0 = 8 * (second ? blockIdx.z - zsets : blockIdx.z);
   // independent loads first
   const int rk = a.rank[g], cf0 = chunk_first[g], cf1 = chunk_first[g + 1], pf = partial_first[g];
   const int r = min(rk, a.rpad);
@@ -247,6 +242,22 @@ __global__ __launch_bounds__(256) void k_wgrad_reduce(WgradArgs a0, WgradArgs a1
 #pragma unroll
   for (int i = 0; i < 8; ++i)
     if (n0 + i < r) store_grad<T>(a, g, n0 + i, c, acc[i]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void k_wgrad_reduce(WgradArgs a0, WgradArgs a1, int rpad,
+                                                      const int32_t* __restrict__ chunk_first,
+                                                      const int32_t* __restrict__ partial_first) {
+  const int zsets = rpad >> 3;
+  const bool second = (int)blockIdx.z >= zsets;
+  wgrad_reduce_body<T>(second ? a1 : a0, 8 * (second ? blockIdx.z - zsets : blockIdx.z), chunk_first, partial_first);
+}
+
+// Any number of argument sets of padded rank 16 (dA and dB of several projections) in one launch:
+// blockIdx.z = 2 * set + octet of rank indices.
+__global__ __launch_bounds__(256) void k_wgrad_reduce_multi(WgradReduceJobs jobs, const int32_t* __restrict__ chunk_first,
+                                                            const int32_t* __restrict__ partial_first) {
+  wgrad_reduce_body<bf16_t>(jobs.a[blockIdx.z >> 1], 8 * (blockIdx.z & 1), chunk_first, partial_first);
 }
 
 // bT_g[n][m] = B_g[m][n], aT_g[k][n] = A_g[n][k]; zero for n >= rank[g].
@@ -317,6 +328,20 @@ int launch_wgrad_reduce(const WgradArgs* a0, const WgradArgs* a1, const SegView&
   else
     hipLaunchKernelGGL(k_wgrad_reduce<bf16_t>, grid, dim3(256), 0, s, x0, x1, rpad, seg.chunk_first,
                        seg.partial_first);
+  return check_launch();
+}
+
+int launch_wgrad_reduce_multi(const WgradArgs* sets, int n, const SegView& seg, const SegLayout& L, hipStream_t s) {
+  if (L.groups == 0 || n == 0) return TK_OK;
+  WgradReduceJobs J{};
+  J.n = n;
+  int width = 0;
+  for (int i = 0; i < n; ++i) {
+    J.a[i] = sets[i];
+    width = std::max(width, sets[i].width);
+  }
+  const dim3 grid((unsigned)L.groups, (unsigned)ceil_div(width, 256), (unsigned)(2 * n));
+  hipLaunchKernelGGL(k_wgrad_reduce_multi, grid, dim3(256), 0, s, J, seg.chunk_first, seg.partial_first);
   return check_launch();
 }
 

@@ -190,12 +190,12 @@ __global__ __launch_bounds__(NW * 64) void k_shrink_pair(PassArgs a, bf16_t* __r
 
 // Adds the slices of a split shrink in slice order and writes h (one block per tile).
 template <int NB>
-__global__ __launch_bounds__(256) void k_shrink_finish(PassArgs a, bf16_t* __restrict__ hrow,
-                                                       const int32_t* __restrict__ tile_group,
-                                                       const int32_t* __restrict__ slot_rows) {
+__device__ __forceinline__ void shrink_finish_body(const PassArgs& a, bf16_t* __restrict__ hrow,
+                                                   const int32_t* __restrict__ tile_group,
+                                                   const int32_t* __restrict__ slot_rows, int tile_id) {
   constexpr int RP = 16 * NB, PR = RP + 1;
   __shared__ float part[kTileRows][PR];
-  const int tile_id = blockIdx.x, tid = threadIdx.x;
+  const int tid = threadIdx.x;
   const int slot0 = tile_id * kTileRows;
   // independent loads first: group id, this tile's row indices, the slices themselves
   const int g = tile_group[tile_id];
@@ -234,6 +234,20 @@ __global__ __launch_bounds__(256) void k_shrink_finish(PassArgs a, bf16_t* __res
   shrink_epilogue<RP, 256>(&part[0][0], 1, a, hrow, slot0, cnt, sc);
 }
 
+template <int NB>
+__global__ __launch_bounds__(256) void k_shrink_finish(PassArgs a, bf16_t* __restrict__ hrow,
+                                                       const int32_t* __restrict__ tile_group,
+                                                       const int32_t* __restrict__ slot_rows) {
+  shrink_finish_body<NB>(a, hrow, tile_group, slot_rows, blockIdx.x);
+}
+
+// The same for up to kMaxShared projections of padded rank 16 in one launch: blockIdx.y selects the projection.
+__global__ __launch_bounds__(256) void k_shrink_finish_multi(PassJobs jobs, const int32_t* __restrict__ tile_group,
+                                                             const int32_t* __restrict__ slot_rows) {
+  const PassArgs& a = jobs.p[blockIdx.y];
+  shrink_finish_body<1>(a, (bf16_t*)a.hT + (int64_t)a.rpad * a.ldh, tile_group, slot_rows, blockIdx.x);
+}
+
 // ---------------------------------------------------------------------------
 // Expand: dst[row(slot)][c] += sum_n h[slot][n] * W2_g[c][n], read-modify-write
 // in place.  Work is flat: one wave owns one 128-column group of one tile and
@@ -246,14 +260,14 @@ __global__ __launch_bounds__(256) void k_shrink_finish(PassArgs a, bf16_t* __res
 // k_expand_multi shares the weight block between tiles.)
 // ---------------------------------------------------------------------------
 template <int NB>
-__global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* __restrict__ hrow,
-                                                     const int32_t* __restrict__ tile_group,
-                                                     const int32_t* __restrict__ slot_rows, int num_items) {
+__device__ __forceinline__ void expand_flat_body(const PassArgs& a, const bf16_t* __restrict__ hrow,
+                                                 const int32_t* __restrict__ tile_group,
+                                                 const int32_t* __restrict__ slot_rows, int num_items, int block) {
   constexpr int RP = 16 * NB;
   constexpr int NKS = (RP + 31) / 32;  // contraction steps of the MFMAs
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
   const int ngroups = a.width_dst >> 7;
-  const int item = blockIdx.x * 4 + wave;
+  const int item = block * 4 + wave;
   if (item >= num_items) return;
   const int tile_id = item / ngroups;
   const int c0 = (item - tile_id * ngroups) << 7;
@@ -320,6 +334,22 @@ __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* _
       st16_nt(yp[tt][v], o);
     }
   }
+}
+
+template <int NB>
+__global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* __restrict__ hrow,
+                                                     const int32_t* __restrict__ tile_group,
+                                                     const int32_t* __restrict__ slot_rows, int num_items) {
+  expand_flat_body<NB>(a, hrow, tile_group, slot_rows, num_items, blockIdx.x);
+}
+
+// Up to kMaxShared projections of padded rank 16 in one launch: blockIdx.y selects the projection; the grid
+// is as wide as the widest projection needs.
+__global__ __launch_bounds__(256) void k_expand_mfma_multi(PassJobs jobs, const int32_t* __restrict__ tile_group,
+                                                           const int32_t* __restrict__ slot_rows, int max_tiles) {
+  const PassArgs& a = jobs.p[blockIdx.y];
+  expand_flat_body<1>(a, (const bf16_t*)a.hT + (int64_t)a.rpad * a.ldh, tile_group, slot_rows,
+                      max_tiles * (a.width_dst >> 7), blockIdx.x);
 }
 
 // ---------------------------------------------------------------------------
@@ -617,10 +647,10 @@ __global__ __launch_bounds__(RS * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
 //        k_shrink_finish turns into dh like after a separate shrink.
 // dy crosses the memory system once instead of twice.  Sums are formed in a fixed order.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void k_dy_fused(WgradArgs a, const void* const* __restrict__ lora_B, int64_t ldb,
-                                                  float* __restrict__ hpart, int kslices,
-                                                  const ChunkInfo* __restrict__ chunks,
-                                                  const int32_t* __restrict__ slot_rows) {
+__device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* const* __restrict__ lora_B, int64_t ldb,
+                                              float* __restrict__ hpart, int kslices,
+                                              const ChunkInfo* __restrict__ chunks,
+                                              const int32_t* __restrict__ slot_rows, int bx, int by, int x_blocks) {
   constexpr int SS = 136;  // row stride of the staged piece in bf16 (272 B)
   constexpr int PR = 17;   // row stride of the partial dh in floats
   __shared__ int32_t rows_s[kChunkTilesMax * kTileRows];
@@ -628,17 +658,17 @@ __global__ __launch_bounds__(256) void k_dy_fused(WgradArgs a, const void* const
   __shared__ float part[2][4][kTileRows * PR];
   static_assert(sizeof(bf16_t) * kTileRows * SS >= sizeof(float) * 16 * kWgradStageStride, "stage holds the dB block too");
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
-  if ((int)blockIdx.y < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
-    transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 256 + tid,
-                          (int64_t)a.tr.y_blocks * gridDim.x * 256);
+  if (by < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
+    transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)by * x_blocks + bx) * 256 + tid,
+                          (int64_t)a.tr.y_blocks * x_blocks * 256);
     return;
   }
-  const ChunkInfo ci = chunks[blockIdx.y - a.tr.y_blocks];
+  const ChunkInfo ci = chunks[by - a.tr.y_blocks];
   const int g = ci.group;
   if (g < 0) return;
   const int r = min(a.rank[g], 16);
   if (r <= 0) return;
-  const int slab = blockIdx.x;
+  const int slab = bx;
   const int c0 = slab * 512 + wave * 128;
   const int nt = ci.ntiles;
   for (int i = tid; i < nt * kTileRows; i += 256) rows_s[i] = slot_rows[ci.tile0 * kTileRows + i];
@@ -746,6 +776,22 @@ __global__ __launch_bounds__(256) void k_dy_fused(WgradArgs a, const void* const
   wgrad_store<1>(acc, reinterpret_cast<float*>(my_stage), a, ci, g, r, c0, lane);
 }
 
+__global__ __launch_bounds__(256) void k_dy_fused(WgradArgs a, const void* const* __restrict__ lora_B, int64_t ldb,
+                                                  float* __restrict__ hpart, int kslices,
+                                                  const ChunkInfo* __restrict__ chunks,
+                                                  const int32_t* __restrict__ slot_rows) {
+  dy_fused_body(a, lora_B, ldb, hpart, kslices, chunks, slot_rows, blockIdx.x, blockIdx.y, gridDim.x);
+}
+
+// Up to kMaxShared projections in one launch (blockIdx.z selects the projection): a narrow projection alone
+// has too few (chunk, 512 columns) blocks to fill the chip.  The grid is as large as the largest job needs.
+__global__ __launch_bounds__(256) void k_dy_fused_multi(DyFusedJobs jobs, const ChunkInfo* __restrict__ chunks,
+                                                        const int32_t* __restrict__ slot_rows, int max_chunks) {
+  const DyFusedJob& j = jobs.j[blockIdx.z];
+  if ((int)blockIdx.x >= j.x_blocks || (int)blockIdx.y >= j.a.tr.y_blocks + max_chunks) return;
+  dy_fused_body(j.a, j.lora_B, j.ldb, j.hpart, j.kslices, chunks, slot_rows, blockIdx.x, blockIdx.y, j.x_blocks);
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <int NB>
@@ -803,6 +849,47 @@ int launch_dy_fused(const WgradArgs& a0, const void* const* lora_B, int64_t ldb,
   const dim3 grid((unsigned)(a.width / 512), (unsigned)(L.max_chunks + a.tr.y_blocks));
   hipLaunchKernelGGL(k_dy_fused, grid, dim3(256), 0, s, a, lora_B, ldb, hpart, kslices, seg.chunks,
                      seg.slot_table(a.map_rows));
+  return check_launch();
+}
+
+int launch_dy_fused_multi(const DyFusedJob* jobs, int n, const SegView& seg, const SegLayout& L, hipStream_t s) {
+  if (L.rows == 0 || n == 0) return TK_OK;
+  DyFusedJobs J{};
+  int gx = 0, gy = 0;
+  for (int p = 0; p < n; ++p) {
+    DyFusedJob& j = J.j[p];
+    j = jobs[p];
+    j.x_blocks = j.a.width / 512;
+    j.a.tr.y_blocks = 0;
+    if (j.a.tr.aT) {
+      const int64_t units =
+          (int64_t)j.a.tr.groups * j.a.rpad * ((j.a.tr.bT ? j.a.tr.out_features : 0) + j.a.tr.in_features) / 8;
+      j.a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * j.x_blocks * 256)));
+    }
+    gx = std::max(gx, j.x_blocks);
+    gy = std::max(gy, (int)L.max_chunks + j.a.tr.y_blocks);
+  }
+  hipLaunchKernelGGL(k_dy_fused_multi, dim3((unsigned)gx, (unsigned)gy, (unsigned)n), dim3(256), 0, s, J, seg.chunks,
+                     seg.slot_table(J.j[0].a.map_rows), (int)L.max_chunks);
+  return check_launch();
+}
+
+// Finish and / or flat expand of several projections of padded rank 16 (phases: 4 finish, 2 expand).
+int launch_pass_multi(const PassArgs* a, int n, const SegView& seg, const SegLayout& L, int phases, hipStream_t s) {
+  if (L.rows == 0 || n == 0) return TK_OK;
+  PassJobs J{};
+  int64_t widest = 0;
+  for (int p = 0; p < n; ++p) {
+    J.p[p] = a[p];
+    widest = std::max<int64_t>(widest, a[p].width_dst >> 7);
+  }
+  const int32_t* rows = seg.slot_table(a[0].map_rows);
+  if (phases & 4)
+    hipLaunchKernelGGL(k_shrink_finish_multi, dim3((unsigned)L.max_tiles, (unsigned)n), dim3(256), 0, s, J,
+                       seg.tile_group, rows);
+  if (phases & 2)
+    hipLaunchKernelGGL(k_expand_mfma_multi, dim3((unsigned)ceil_div(L.max_tiles * widest, 4), (unsigned)n), dim3(256), 0,
+                       s, J, seg.tile_group, rows, (int)L.max_tiles);
   return check_launch();
 }
 

@@ -242,6 +242,26 @@ struct SharedWgradArgs {                 // dA_p for all p from one pass over x 
   int32_t nproj;
   WgradArgs w[kMaxShared];
 };
+struct PassJobs {
+  PassArgs p[kMaxShared];
+};
+struct DyFusedJob {
+  WgradArgs a;                  // dB job of one projection (src = dy_p); a.tr carries the weight transposes
+  const void* const* lora_B;    // device pointer table [G] of B_p
+  int64_t ldb;
+  float* hpart;                 // split-shrink buffer receiving the slices of dh_p
+  int32_t kslices, x_blocks;    // x_blocks is filled in by the launcher
+};
+struct DyFusedJobs {
+  DyFusedJob j[kMaxShared];
+};
+struct WgradReduceJobs {
+  int32_t n;
+  WgradArgs a[2 * kMaxShared];
+};
+int launch_dy_fused_multi(const DyFusedJob* jobs, int n, const SegView& seg, const SegLayout& L, hipStream_t s);
+int launch_pass_multi(const PassArgs* a, int n, const SegView& seg, const SegLayout& L, int phases, hipStream_t s);
+int launch_wgrad_reduce_multi(const WgradArgs* sets, int n, const SegView& seg, const SegLayout& L, hipStream_t s);
 int launch_shrink_shared(const SharedShrinkArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
 int launch_expand_shared(const SharedExpandArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
 int launch_wgrad_shared(const SharedWgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
