@@ -295,6 +295,8 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
     // One pass over dy yields dB and the slices of dh (and, on the side, the A^T copy for dX).
     gb.tr = tr;
     gb.tr.bT = nullptr;
+    gb.tr.swizzle_a = 1;  // written here, read only by the expand below
+    a.expand_swizzled = 1;
     rc = launch_dy_fused(gb, d->lora_B, d->ldb, a.hpart, a.kslices, V, L, s);
     gb.tr = TransposeJob{};
     if (rc != TK_OK) return rc;
@@ -452,6 +454,7 @@ int tk_lora_bwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* 
     dj[p].a = P.gb;
     dj[p].a.tr = P.tr;
     dj[p].a.tr.bT = nullptr;  // the fused kernel reads B_p where it lies
+    dj[p].a.tr.swizzle_a = 1;
     dj[p].lora_B = descs[p]->lora_B;  dj[p].ldb = descs[p]->ldb;
     dj[p].hpart = P.a.hpart;  dj[p].kslices = P.a.kslices;
     pa[p] = P.a;

@@ -310,7 +310,8 @@ __device__ __forceinline__ void expand_flat_body(const PassArgs& a, const bf16_t
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
       const int n0 = 32 * ks + 8 * kb;
-      bq[q][ks] = n0 < r ? keep_first(ld16(W2 + (int64_t)(c0 + 8 * li + q) * a.ld_expand + n0), r - n0) : zero4();
+      const int wrow = a.expand_swizzled ? c0 + 16 * q + li : c0 + 8 * li + q;
+      bq[q][ks] = n0 < r ? keep_first(ld16(W2 + (int64_t)wrow * a.ld_expand + n0), r - n0) : zero4();
     }
   if (r <= 0) return;  // unused tile, or adapter not live on this layer (uniform over the wave)
 #pragma unroll
@@ -493,14 +494,15 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
       out = (bf16_t*)t.bT + ((int64_t)g * rpad + n) * t.out_features + 8 * mo;
     } else {
       const int64_t v = u - units_b;
-      const int k = (int)(v % t.in_features);
+      const int kd = (int)(v % t.in_features);  // row of aT; which column of A lies there:
+      const int k = t.swizzle_a ? ((kd & ~127) | ((kd & 15) << 3) | ((kd >> 4) & 7)) : kd;
       const int64_t q = v / t.in_features;
       const int no = (int)(q % n8), g = (int)(q / n8);
       const bf16_t* A = (const bf16_t*)t.lora_A[g] + (int64_t)(8 * no) * t.lda + k;
       const int r = rank[g];
 #pragma unroll
       for (int i = 0; i < 8; ++i) e[i] = 8 * no + i < r ? A[(int64_t)i * t.lda] : 0;
-      out = (bf16_t*)t.aT + ((int64_t)g * t.in_features + k) * rpad + 8 * no;
+      out = (bf16_t*)t.aT + ((int64_t)g * t.in_features + kd) * rpad + 8 * no;
     }
     st16(out, make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)));
   }
@@ -783,13 +785,18 @@ __global__ __launch_bounds__(256) void k_dy_fused(WgradArgs a, const void* const
   dy_fused_body(a, lora_B, ldb, hpart, kslices, chunks, slot_rows, blockIdx.x, blockIdx.y, gridDim.x);
 }
 
-// Up to kMaxShared projections in one launch (blockIdx.z selects the projection): a narrow projection alone
-// has too few (chunk, 512 columns) blocks to fill the chip.  The grid is as large as the largest job needs.
+// Up to kMaxShared projections in one launch: a narrow projection alone has too few (chunk, 512 columns)
+// blocks to fill the chip.  The jobs' column slabs lie side by side along blockIdx.x, so that the blocks of
+// all projections are dispatched interleaved and run next to each other.
 __global__ __launch_bounds__(256) void k_dy_fused_multi(DyFusedJobs jobs, const ChunkInfo* __restrict__ chunks,
                                                         const int32_t* __restrict__ slot_rows, int max_chunks) {
-  const DyFusedJob& j = jobs.j[blockIdx.z];
-  if ((int)blockIdx.x >= j.x_blocks || (int)blockIdx.y >= j.a.tr.y_blocks + max_chunks) return;
-  dy_fused_body(j.a, j.lora_B, j.ldb, j.hpart, j.kslices, chunks, slot_rows, blockIdx.x, blockIdx.y, j.x_blocks);
+  int p = 0;
+#pragma unroll
+  for (int i = 1; i < kMaxShared; ++i) p += (i < jobs.n && (int)blockIdx.x >= jobs.x_first[i]) ? 1 : 0;
+  const DyFusedJob& j = jobs.j[p];
+  if ((int)blockIdx.y >= j.a.tr.y_blocks + max_chunks) return;
+  dy_fused_body(j.a, j.lora_B, j.ldb, j.hpart, j.kslices, chunks, slot_rows, blockIdx.x - jobs.x_first[p], blockIdx.y,
+                j.x_blocks);
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -855,7 +862,8 @@ int launch_dy_fused(const WgradArgs& a0, const void* const* lora_B, int64_t ldb,
 int launch_dy_fused_multi(const DyFusedJob* jobs, int n, const SegView& seg, const SegLayout& L, hipStream_t s) {
   if (L.rows == 0 || n == 0) return TK_OK;
   DyFusedJobs J{};
-  int gx = 0, gy = 0;
+  J.n = n;
+  int gy = 0;
   for (int p = 0; p < n; ++p) {
     DyFusedJob& j = J.j[p];
     j = jobs[p];
@@ -866,10 +874,10 @@ int launch_dy_fused_multi(const DyFusedJob* jobs, int n, const SegView& seg, con
           (int64_t)j.a.tr.groups * j.a.rpad * ((j.a.tr.bT ? j.a.tr.out_features : 0) + j.a.tr.in_features) / 8;
       j.a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * j.x_blocks * 256)));
     }
-    gx = std::max(gx, j.x_blocks);
+    J.x_first[p + 1] = J.x_first[p] + j.x_blocks;
     gy = std::max(gy, (int)L.max_chunks + j.a.tr.y_blocks);
   }
-  hipLaunchKernelGGL(k_dy_fused_multi, dim3((unsigned)gx, (unsigned)gy, (unsigned)n), dim3(256), 0, s, J, seg.chunks,
+  hipLaunchKernelGGL(k_dy_fused_multi, dim3((unsigned)J.x_first[n], (unsigned)gy), dim3(256), 0, s, J, seg.chunks,
                      seg.slot_table(J.j[0].a.map_rows), (int)L.max_chunks);
   return check_launch();
 }

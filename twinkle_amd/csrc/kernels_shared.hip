@@ -15,6 +15,16 @@ namespace tk {
 
 namespace {
 
+// Blocks go to the XCDs (each with an L2 of its own) round-robin.  This renumbering gives every XCD one
+// contiguous eighth of the work items, so that an XCD's L2 fetches the weights of few groups instead of all.
+__device__ inline int xcd_contiguous(int block, int blocks) {
+#ifdef TK_NO_XCD_MAP
+  return block;
+#endif
+  const int per = blocks >> 3;
+  return block < 8 * per ? (block & 7) * per + (block >> 3) : block;
+}
+
 template <typename T>
 __device__ inline T pick(const T (&v)[kMaxShared], int i) {  // v[i] without a register-indexed array
   T r = v[0];
@@ -32,7 +42,7 @@ __device__ inline T pick(const T (&v)[kMaxShared], int i) {  // v[i] without a r
 template <int P, int TT>
 __device__ inline void shrink_tiles_shared(const SharedShrinkArgs& a, const int32_t* __restrict__ slot_rows,
                                            const int (&tiles)[TT], int g, int ks, float (*part)[16 * P + 1]) {
-  constexpr int PF = 2;  // steps whose loads are issued together
+  constexpr int PF = P <= 2 ? 2 : 1;  // steps whose loads are issued together (what leaves three waves per SIMD)
   const int lane = threadIdx.x & 63, li = lane & 15, kb = lane >> 4;
   const bf16_t* src = (const bf16_t*)a.src;
   const bf16_t *xa[TT], *xb[TT];
@@ -119,10 +129,11 @@ __device__ inline void shrink_tiles_shared(const SharedShrinkArgs& a, const int3
 }
 
 template <int P>
-__global__ __launch_bounds__(64) void k_shrink_shared(SharedShrinkArgs a, const int32_t* __restrict__ tile_group,
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(P <= 3 ? 3 : 2))) void k_shrink_shared(SharedShrinkArgs a, const int32_t* __restrict__ tile_group,
                                                       const int32_t* __restrict__ slot_rows, int max_tiles) {
   __shared__ float part[kTileRows][16 * P + 1];
-  const int pair = blockIdx.x / a.kslices, ks = blockIdx.x - pair * a.kslices;
+  const int block = xcd_contiguous(blockIdx.x, gridDim.x);
+  const int pair = block / a.kslices, ks = block - pair * a.kslices;
   const int t0 = 2 * pair, t1 = t0 + 1;
   const int g0 = tile_group[t0];
   const int g1 = t1 < max_tiles ? tile_group[t1] : -1;
@@ -145,15 +156,15 @@ __global__ __launch_bounds__(64) void k_shrink_shared(SharedShrinkArgs a, const 
 // dx[row] += sum_p dh_p[row] A_p: the flat expand kernel (one wave = one tile x 128 columns) with the
 // contraction running over the P projections' blocks of 16 rank indices; lane group kb reads block
 // 2 ks + kb / 2 of h (slot-major, [slots][16] per projection) and of the transposed weight copies
-// ([G][K][16] per projection).
+// ([G][K][16] per projection, rows permuted inside every 128 as TransposeJob::swizzle_a describes).
 // ---------------------------------------------------------------------------
 template <int P>
-__global__ __launch_bounds__(256) void k_expand_shared(SharedExpandArgs a, const int32_t* __restrict__ tile_group,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void k_expand_shared(SharedExpandArgs a, const int32_t* __restrict__ tile_group,
                                                        const int32_t* __restrict__ slot_rows, int num_items) {
   constexpr int NKS = (16 * P + 31) / 32;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
   const int ngroups = a.width_dst >> 7;
-  const int item = blockIdx.x * 4 + wave;
+  const int item = xcd_contiguous(blockIdx.x, gridDim.x) * 4 + wave;
   if (item >= num_items) return;
   const int tile_id = item / ngroups;
   const int c0 = (item - tile_id * ngroups) << 7;
@@ -200,10 +211,11 @@ __global__ __launch_bounds__(256) void k_expand_shared(SharedExpandArgs a, const
 #pragma unroll
   for (int ks = 0; ks < NKS; ++ks) {
     const int blk = 2 * ks + (kb >> 1);
-    const bf16_t* wt = (const bf16_t*)pick(a.aT, blk) + ((int64_t)g * a.width_dst + c0 + 8 * li) * 16 + off;
+    // rows permuted inside every 128: the row of column c0 + 8 li + q lies at c0 + 16 q + li
+    const bf16_t* wt = (const bf16_t*)pick(a.aT, blk) + ((int64_t)g * a.width_dst + c0 + li) * 16 + off;
 #pragma unroll
     for (int q = 0; q < 8; ++q)
-      bq[q][ks] = off < rblk[ks] ? keep_first(ld16(wt + (int64_t)q * 16), rblk[ks] - off) : zero4();
+      bq[q][ks] = off < rblk[ks] ? keep_first(ld16(wt + (int64_t)q * 256), rblk[ks] - off) : zero4();
   }
   if (!any) return;  // unused tile, or no projection live on this layer (uniform over the wave)
 #pragma unroll
@@ -239,10 +251,12 @@ __global__ __launch_bounds__(256) void k_expand_shared(SharedExpandArgs a, const
 // leaves through the same staging buffer into its own projection's partial buffer or gradient.
 // ---------------------------------------------------------------------------
 template <int P>
-__global__ __launch_bounds__(64) void k_wgrad_shared(SharedWgradArgs a, const ChunkInfo* __restrict__ chunks,
-                                                     const int32_t* __restrict__ slot_rows) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(P <= 3 ? 2 : 1))) void k_wgrad_shared(
+    SharedWgradArgs a, const ChunkInfo* __restrict__ chunks, const int32_t* __restrict__ slot_rows) {
   constexpr int OS = kWgradStageStride;
+  constexpr int STAGES = 2;  // tiles in registers: what fits next to P accumulator blocks at two waves per SIMD
   __shared__ __attribute__((aligned(16))) float lds[16 * OS];
+  extern __shared__ __attribute__((aligned(16))) int32_t rows_s[];  // the chunk's row indices
   const int lane = threadIdx.x & 63, li = lane & 15, kb = lane >> 4;
   const int c0 = blockIdx.x * 128;
   const ChunkInfo ci = chunks[blockIdx.y];
@@ -258,31 +272,31 @@ __global__ __launch_bounds__(64) void k_wgrad_shared(SharedWgradArgs a, const Ch
   if (!any) return;
   const WgradArgs& a0 = a.w[0];
   const int nt = ci.ntiles;
+  // the row indices go through LDS: reading them there does not wait for the tile loads in flight
+  for (int i = lane; i < nt * kTileRows; i += 64) rows_s[i] = slot_rows[ci.tile0 * kTileRows + i];
   const bf16_t* src = (const bf16_t*)a0.src + c0 + 8 * li;
   const bf16_t* hT[P];
 #pragma unroll
   for (int p = 0; p < P; ++p)
     hT[p] = (const bf16_t*)a.w[p].hT + (int64_t)li * a.w[p].ldh + (int64_t)ci.tile0 * kTileRows + 8 * kb;
-  const int32_t* rows_p = slot_rows + ci.tile0 * kTileRows + 8 * kb;
   f32x4 acc[8][P];
 #pragma unroll
   for (int q = 0; q < 8; ++q)
 #pragma unroll
     for (int p = 0; p < P; ++p) acc[q][p] = f32x4{0.f, 0.f, 0.f, 0.f};
+  __syncthreads();
 
   struct Tile {
     uint4 x[8];
     uint4 h[P];
     uint32_t live;
   };
-  int4 ra, rb;
-  auto load_rows = [&](int t) {
-    const int tc = min(t, nt - 1);
-    ra = *reinterpret_cast<const int4*>(rows_p + tc * kTileRows);
-    rb = *reinterpret_cast<const int4*>(rows_p + tc * kTileRows + 4);
-  };
+  // loads are unconditional (tiles past the end re-read the last one, padding slots read row 0); what must
+  // not count is zeroed when it is consumed
   auto issue = [&](int t, Tile& T) {
     const int tc = min(t, nt - 1);
+    const int4 ra = *reinterpret_cast<const int4*>(rows_s + tc * kTileRows + 8 * kb);
+    const int4 rb = *reinterpret_cast<const int4*>(rows_s + tc * kTileRows + 8 * kb + 4);
     const int rows[8] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w};
     T.live = 0;
 #pragma unroll
@@ -313,32 +327,40 @@ __global__ __launch_bounds__(64) void k_wgrad_shared(SharedWgradArgs a, const Ch
       for (int p = 0; p < P; ++p) acc[q][p] = mfma16(tr, T.h[p], acc[q][p]);
     }
   };
-  Tile A, B, C;
-  load_rows(0);
-  issue(0, A);
-  load_rows(1);
-  issue(1, B);
-  load_rows(2);
-  int t = 0;
-  for (; t + 4 < nt; t += 3) {  // every tile touched in here exists
+  if constexpr (STAGES == 3) {
+    Tile A, B, C;
+    issue(0, A);
+    issue(1, B);
+    int t = 0;
+    for (; t + 4 < nt; t += 3) {  // every tile touched in here exists
+      issue(t + 2, C);
+      consume(A);
+      issue(t + 3, A);
+      consume(B);
+      issue(t + 4, B);
+      consume(C);
+    }
     issue(t + 2, C);
-    load_rows(t + 3);
     consume(A);
-    issue(t + 3, A);
-    load_rows(t + 4);
     consume(B);
-    issue(t + 4, B);
-    load_rows(t + 5);
     consume(C);
-  }
-  issue(t + 2, C);
-  load_rows(t + 3);
-  consume(A);
-  consume(B);
-  consume(C);
-  if (t + 3 < nt) {
-    issue(t + 3, A);
+    if (t + 3 < nt) {
+      issue(t + 3, A);
+      consume(A);
+    }
+  } else {
+    Tile A, B;
+    issue(0, A);
+    int t = 0;
+    for (; t + 2 < nt; t += 2) {
+      issue(t + 1, B);
+      consume(A);
+      issue(t + 2, A);
+      consume(B);
+    }
+    issue(t + 1, B);  // one or two tiles are left
     consume(A);
+    consume(B);       // all zeros when tile t + 1 does not exist
   }
 #pragma unroll
   for (int p = 0; p < P; ++p) {
@@ -384,12 +406,13 @@ int launch_wgrad_shared(const SharedWgradArgs& a, const SegView& seg, const SegL
   if (L.rows == 0) return TK_OK;
   const dim3 grid((unsigned)(a.w[0].width / 128), (unsigned)L.max_chunks);
   const int32_t* rows = seg.slot_table(a.w[0].map_rows);
+  const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);  // a chunk's row indices
   if (a.nproj == 2)
-    hipLaunchKernelGGL(k_wgrad_shared<2>, grid, dim3(64), 0, s, a, seg.chunks, rows);
+    hipLaunchKernelGGL(k_wgrad_shared<2>, grid, dim3(64), dyn, s, a, seg.chunks, rows);
   else if (a.nproj == 3)
-    hipLaunchKernelGGL(k_wgrad_shared<3>, grid, dim3(64), 0, s, a, seg.chunks, rows);
+    hipLaunchKernelGGL(k_wgrad_shared<3>, grid, dim3(64), dyn, s, a, seg.chunks, rows);
   else
-    hipLaunchKernelGGL(k_wgrad_shared<4>, grid, dim3(64), 0, s, a, seg.chunks, rows);
+    hipLaunchKernelGGL(k_wgrad_shared<4>, grid, dim3(64), dyn, s, a, seg.chunks, rows);
   return check_launch();
 }
 

@@ -191,6 +191,9 @@ struct PassArgs {
   int32_t src_rows;  // rows of src / dst (bound for speculative row addresses)
   float* hpart;          // partial sums of the split shrink, [tile][slice][32][rpad]
   int32_t kslices;       // blocks per tile of the MFMA shrink
+  // the expand weight's rows are permuted inside every group of 128 (TransposeJob::swizzle_a): the row of
+  // column c0 + 8 i + q lies at c0 + 16 q + i, so that the 16 rows one MFMA operand load touches are adjacent
+  int32_t expand_swizzled;
 };
 
 // Optional side job of a weight-gradient launch (bf16 MFMA path): the first `y_blocks` rows of the
@@ -203,6 +206,7 @@ struct TransposeJob {
   void* bT;  // [groups][rpad][out_features]
   int32_t in_features, out_features, groups;
   int32_t y_blocks;  // 0: no job
+  int32_t swizzle_a; // aT rows permuted inside every 128 (see PassArgs::expand_swizzled); in_features % 128 == 0
 };
 
 // Row-contraction (weight gradient) pass: out_g[n][c] = sum_p hT[n][p] * src[row(p)][c].
@@ -254,6 +258,8 @@ struct DyFusedJob {
 };
 struct DyFusedJobs {
   DyFusedJob j[kMaxShared];
+  int32_t n;
+  int32_t x_first[kMaxShared + 1];  // job p owns the blocks x_first[p] <= blockIdx.x < x_first[p + 1]
 };
 struct WgradReduceJobs {
   int32_t n;
