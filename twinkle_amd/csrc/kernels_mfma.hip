@@ -512,9 +512,11 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
 // Weight gradient: out_g[n][c] = sum over the rows of group g of hT[n][slot] * src[row(slot)][c].
 //
 // Work item = (chunk of one group, 128 source columns), one block of RS waves.  A wave walks all tiles of
-// the chunk with a three-stage software pipeline: the row indices of tile t+3 and the source rows of
-// tile t+2 are requested before tile t is consumed, so a wave never waits on an index load and has two
-// tiles (8 KB each) in flight.  A lane loads 16 B of eight rows, transposes the 8x8 block in registers
+// the chunk with an S-stage software pipeline: the source rows of tile t+S-1 are requested before tile t
+// is consumed, so a wave has S-1 tiles (8 KB each) in flight; the chunk's row indices wait in LDS, where
+// reading them does not have to wait for the tile loads in flight.  A grid of (chunks x 128-column
+// blocks) is small next to the chip, so the depth of the pipeline, not the number of resident waves, is
+// what keeps enough bytes in flight.  A lane loads 16 B of eight rows, transposes the 8x8 block in registers
 // (v_perm_b32) and feeds it as the MFMA A operand with the rows as contraction index.  The result is
 // staged in LDS in [n][column] order and leaves as whole 512-byte rows: into the chunk's slot of the
 // partial buffer (groups that span several chunks; k_wgrad_reduce adds the chunks in order) or straight
@@ -524,13 +526,14 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
 // RS waves of a block walk the same tiles and each own 1/RS of the rank indices; the second reader of a
 // tile finds it in the CU's cache.
 // ---------------------------------------------------------------------------
-template <int NB, int RS>
+template <int NB, int RS, int S>
 __global__ __launch_bounds__(RS * 64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo* __restrict__ chunks,
                                                         const int32_t* __restrict__ slot_rows) {
   static_assert(NB % RS == 0, "rank blocks must divide evenly");
   constexpr int NBW = NB / RS;  // blocks of 16 rank indices per wave
   constexpr int OS = kWgradStageStride;
   __shared__ __attribute__((aligned(16))) float lds[16 * NB * OS];
+  extern __shared__ __attribute__((aligned(16))) int32_t rows_s[];  // the chunk's row indices
   const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kb = lane >> 4, rs = tid >> 6;
   if ((int)blockIdx.y < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
     transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (RS * 64) + tid,
@@ -543,13 +546,15 @@ __global__ __launch_bounds__(RS * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
   const int g = ci.group;
   if (g < 0) return;
   const int r = min(a.rank[g], 16 * NB);
-  const int n_base = rs * NBW * 16;  // first rank index of this wave
-  if (r <= n_base) return;           // covers r <= 0; the waves of a block never meet at a barrier
-
+  if (r <= 0) return;
   const int nt = ci.ntiles;
+  for (int i = tid; i < nt * kTileRows; i += RS * 64) rows_s[i] = slot_rows[ci.tile0 * kTileRows + i];
+  __syncthreads();
+  const int n_base = rs * NBW * 16;  // first rank index of this wave
+  if (r <= n_base) return;           // from here on the waves of a block never meet at a barrier
+
   const bf16_t* src = (const bf16_t*)a.src + c0 + 8 * li;
   const bf16_t* hT = (const bf16_t*)a.hT + (int64_t)(n_base + li) * a.ldh + (int64_t)ci.tile0 * kTileRows + 8 * kb;
-  const int32_t* rows_p = slot_rows + ci.tile0 * kTileRows + 8 * kb;  // this lane's 8 slots of the chunk's first tile
   f32x4 acc[8][NBW];
 #pragma unroll
   for (int q = 0; q < 8; ++q)
@@ -565,14 +570,10 @@ __global__ __launch_bounds__(RS * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
     uint4 h[NBW];
     uint32_t live;  // bit q: row q of this lane is a real row of a tile inside the chunk
   };
-  int4 ra, rb;  // row indices of the tile that is issued next
-  auto load_rows = [&](int t) {
-    const int tc = min(t, nt - 1);
-    ra = *reinterpret_cast<const int4*>(rows_p + tc * kTileRows);
-    rb = *reinterpret_cast<const int4*>(rows_p + tc * kTileRows + 4);
-  };
   auto issue = [&](int t, Tile& T) {
     const int tc = min(t, nt - 1);
+    const int4 ra = *reinterpret_cast<const int4*>(rows_s + tc * kTileRows + 8 * kb);
+    const int4 rb = *reinterpret_cast<const int4*>(rows_s + tc * kTileRows + 8 * kb + 4);
     const int rows[8] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w};
     T.live = 0;
 #pragma unroll
@@ -604,34 +605,20 @@ __global__ __launch_bounds__(RS * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
       for (int nb = 0; nb < NBW; ++nb) acc[q][nb] = mfma16(tr, T.h[nb], acc[q][nb]);
     }
   };
-  Tile A, B, C;
-  load_rows(0);
-  issue(0, A);
-  load_rows(1);
-  issue(1, B);
-  load_rows(2);
+  Tile T[S];
+#pragma unroll
+  for (int i = 0; i < S - 1; ++i) issue(i, T[i]);
   int t = 0;
-  for (; t + 4 < nt; t += 3) {  // every tile touched in here exists
-    issue(t + 2, C);
-    load_rows(t + 3);
-    consume(A);
-    issue(t + 3, A);
-    load_rows(t + 4);
-    consume(B);
-    issue(t + 4, B);
-    load_rows(t + 5);
-    consume(C);
+  for (; t + S <= nt; t += S) {  // every tile consumed in here exists (the youngest requests may lie past the end)
+#pragma unroll
+    for (int i = 0; i < S; ++i) {
+      issue(t + i + S - 1, T[(i + S - 1) % S]);
+      consume(T[i]);
+    }
   }
-  // drain: one to four tiles are left, t and t + 1 already on their way (tiles past the end count as zeros)
-  issue(t + 2, C);
-  load_rows(t + 3);
-  consume(A);
-  consume(B);
-  consume(C);
-  if (t + 3 < nt) {
-    issue(t + 3, A);
-    consume(A);
-  }
+  // drain: fewer than S tiles are left, all requested already (tiles past the end count as zeros)
+#pragma unroll
+  for (int i = 0; i < S - 1; ++i) consume(T[i]);
   wgrad_store<NBW>(acc, lds + n_base * OS, a, ci, g, r, c0, lane, n_base);
 }
 
@@ -799,6 +786,10 @@ __global__ __launch_bounds__(256) void k_dy_fused_multi(DyFusedJobs jobs, const 
                 j.x_blocks);
 }
 
+#ifndef TK_WGRAD_STAGES
+#define TK_WGRAD_STAGES 3
+#endif
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 template <int NB>
@@ -826,7 +817,7 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
   }
 }
 
-template <int NB, int RS>
+template <int NB, int RS, int S>
 void launch_wgrad_pipe(const WgradArgs& a0, const SegView& seg, const SegLayout& L, hipStream_t s) {
   WgradArgs a = a0;
   a.tr.y_blocks = 0;
@@ -835,7 +826,9 @@ void launch_wgrad_pipe(const WgradArgs& a0, const SegView& seg, const SegLayout&
     a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 128) * (RS * 64))));
   }
   const dim3 grid((unsigned)(a.width / 128), (unsigned)(L.max_chunks + a.tr.y_blocks));
-  hipLaunchKernelGGL((k_wgrad_pipe<NB, RS>), grid, dim3(RS * 64), 0, s, a, seg.chunks, seg.slot_table(a.map_rows));
+  const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);  // a chunk's row indices
+  hipLaunchKernelGGL((k_wgrad_pipe<NB, RS, S>), grid, dim3(RS * 64), dyn, s, a, seg.chunks,
+                     seg.slot_table(a.map_rows));
 }
 
 }  // namespace
@@ -927,9 +920,9 @@ bool wgrad_mfma_supported(const WgradArgs& a) {
 
 int launch_wgrad_mfma(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
   if (L.rows == 0) return TK_OK;
-  if (a.rpad <= 16) launch_wgrad_pipe<1, 1>(a, seg, L, s);
-  else if (a.rpad <= 32) launch_wgrad_pipe<2, 1>(a, seg, L, s);
-  else launch_wgrad_pipe<4, 2>(a, seg, L, s);
+  if (a.rpad <= 16) launch_wgrad_pipe<1, 1, TK_WGRAD_STAGES>(a, seg, L, s);
+  else if (a.rpad <= 32) launch_wgrad_pipe<2, 1, 3>(a, seg, L, s);
+  else launch_wgrad_pipe<4, 2, 3>(a, seg, L, s);
   return check_launch();
 }
 
