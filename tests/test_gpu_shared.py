@@ -177,3 +177,58 @@ def test_forward_shared_equals_layer_by_layer(dev, dtype, d, kv):
     with ml.adapter('carol', disable_lora=True):
         a = ml.forward_shared(layers, x)
     assert torch.equal(a[1], torch.nn.functional.linear(x, m.k_proj.base_layer.weight))
+
+
+def test_shared_calls_replay_from_a_hip_graph(dev):
+    """Segment build + shared forward + shared backward captured once and replayed: every replay equals eager."""
+    from twinkle_amd import (lora_bwd_shared_, lora_bwd_workspace_bytes, lora_fwd_shared_, lora_h_bytes)
+    t, k, outs, n = 1500, 1024, (1024, 512, 512), 4
+    ranks = [(16, 7, 16, 3), (8, 8, 0, 8), (16, 16, 16, 16)]
+    g = torch.Generator().manual_seed(31)
+    dt = torch.bfloat16
+    x = torch.randn(t, k, generator=g).to(dt).to(dev)
+    bases = [torch.randn(t, m, generator=g).to(dt).to(dev) for m in outs]
+    dys = [torch.randn(t, m, generator=g).to(dt).to(dev) for m in outs]
+    keys = torch.randint(0, n, (t,), generator=g).to(torch.int32).to(dev)
+    groups = [grp for grp, _, _ in _groups(_projections(k, outs, n, 16, ranks, 7, dt, dev), dev)]
+    seg0 = build_segments(keys, n, want_perm=False, want_offsets=False)
+    hs = [torch.empty(lora_h_bytes(seg0, grp), dtype=torch.uint8, device=dev) for grp in groups]
+    wss = [torch.empty(lora_bwd_workspace_bytes(seg0, grp), dtype=torch.uint8, device=dev) for grp in groups]
+    gas = [torch.zeros(grp.a_arena_elems, dtype=dt, device=dev) for grp in groups]
+    gbs = [torch.zeros(grp.b_arena_elems, dtype=dt, device=dev) for grp in groups]
+    pas = [grp._grad_a_rel + ga.data_ptr() for grp, ga in zip(groups, gas)]
+    pbs = [grp._grad_b_rel + gb.data_ptr() for grp, gb in zip(groups, gbs)]
+    ys = [torch.empty_like(b) for b in bases]
+    dx = torch.empty_like(x)
+
+    def step():
+        for y, b in zip(ys, bases):
+            y.copy_(b)
+        dx.fill_(0)
+        seg = build_segments(keys, n, want_perm=False, want_offsets=False)
+        lora_fwd_shared_(x, ys, seg, groups, hs=hs)
+        lora_bwd_shared_(dys, x, hs, dx, pas, pbs, seg, groups, workspaces=wss)
+
+    step()
+    torch.cuda.synchronize()
+    want = [v.clone() for v in (*ys, dx, *gas, *gbs)]
+    assert want[3].abs().max() > 0
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        step()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(3):
+        for v in (*ys, dx):
+            v.fill_(1)
+        for v in (*gas, *gbs):
+            v.zero_()                # regions beyond an adapter's rank are never written: keep them comparable
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref in zip((*ys, dx, *gas, *gbs), want):
+            assert torch.equal(got, ref)

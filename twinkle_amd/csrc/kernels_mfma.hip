@@ -16,6 +16,14 @@
 
 #include "tk_mfma.h"
 
+// depths of the software pipelines of k_dy_fused and k_wgrad_pipe<1, 1, S> (tiles in registers per wave)
+#ifndef TK_DY_STAGES
+#define TK_DY_STAGES 2
+#endif
+#ifndef TK_WGRAD_STAGES
+#define TK_WGRAD_STAGES 3
+#endif
+
 namespace tk {
 
 namespace {
@@ -747,20 +755,28 @@ __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* co
     }
   };
 
-  uint4 xa[8], xb[8], ha, hb;
-  uint32_t la, lb;
-  issue(0, xa, ha, la);
+  constexpr int S = TK_DY_STAGES;  // software pipeline: S - 1 tiles in flight while one is consumed
+  struct Tile {
+    uint4 x[8];
+    uint4 h;
+    uint32_t live;
+  };
+  Tile T[S];
+#pragma unroll
+  for (int i = 0; i < S - 1; ++i) issue(i, T[i].x, T[i].h, T[i].live);
   int t = 0;
-  for (; t + 2 < nt; t += 2) {  // every tile touched in here exists
-    issue(t + 1, xb, hb, lb);
-    consume(t, xa, ha, la);
-    issue(t + 2, xa, ha, la);
-    consume(t + 1, xb, hb, lb);
+  for (; t + S <= nt; t += S) {  // every tile consumed in here exists (the youngest requests may lie past the end)
+#pragma unroll
+    for (int i = 0; i < S; ++i) {
+      Tile& Y = T[(i + S - 1) % S];
+      issue(t + i + S - 1, Y.x, Y.h, Y.live);
+      consume(t + i, T[i].x, T[i].h, T[i].live);
+    }
   }
-  // one or two tiles are left
-  issue(t + 1, xb, hb, lb);
-  consume(t, xa, ha, la);
-  if (t + 1 < nt) consume(t + 1, xb, hb, lb);
+  // fewer than S tiles are left, all of them requested already
+#pragma unroll
+  for (int i = 0; i < S - 1; ++i)
+    if (t + i < nt) consume(t + i, T[i].x, T[i].h, T[i].live);
   // every wave has its own 128 columns of dB
   wgrad_store<1>(acc, reinterpret_cast<float*>(my_stage), a, ci, g, r, c0, lane);
 }
@@ -785,10 +801,6 @@ __global__ __launch_bounds__(256) void k_dy_fused_multi(DyFusedJobs jobs, const 
   dy_fused_body(j.a, j.lora_B, j.ldb, j.hpart, j.kslices, chunks, slot_rows, blockIdx.x - jobs.x_first[p], blockIdx.y,
                 j.x_blocks);
 }
-
-#ifndef TK_WGRAD_STAGES
-#define TK_WGRAD_STAGES 3
-#endif
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
