@@ -329,7 +329,12 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
       if (rc != TK_OK) break;
     }
     if (need_wT) {
-      if (!wT_done && (rc = launch_transpose_weights(*d, bT, aT, s)) != TK_OK) break;
+      if (!wT_done) {
+        // both consumers on the MFMA kernels: 16-byte stores, dead rank indices skipped; else the generic copy
+        const bool fast = mfma && pass_mfma_supported(a) && d->out_features % 8 == 0;
+        rc = fast ? launch_transpose_job(tr, d->rank, a.rpad, s) : launch_transpose_weights(*d, bT, aT, s);
+        if (rc != TK_OK) break;
+      }
       if ((rc = run_pass(a, V, L, d->dtype, 1, s)) != TK_OK) break;
       if (side && grad_A) {  // dh is complete: the side stream may start dA while dX runs here
         if (hipEventRecord(side->mid, s) != hipSuccess || hipStreamWaitEvent(s2, side->mid, 0) != hipSuccess) {

@@ -497,6 +497,7 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
       const int mo = (int)(q % m8), g = (int)(q / m8);
       const bf16_t* B = (const bf16_t*)t.lora_B[g] + (int64_t)(8 * mo) * t.ldb + n;
       const bool live = n < rank[g];
+      if (!live && t.skip_dead) continue;
 #pragma unroll
       for (int i = 0; i < 8; ++i) e[i] = live ? B[(int64_t)i * t.ldb] : 0;
       out = (bf16_t*)t.bT + ((int64_t)g * rpad + n) * t.out_features + 8 * mo;
@@ -508,12 +509,18 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
       const int no = (int)(q % n8), g = (int)(q / n8);
       const bf16_t* A = (const bf16_t*)t.lora_A[g] + (int64_t)(8 * no) * t.lda + k;
       const int r = rank[g];
+      if (8 * no >= r && t.skip_dead) continue;
 #pragma unroll
       for (int i = 0; i < 8; ++i) e[i] = 8 * no + i < r ? A[(int64_t)i * t.lda] : 0;
       out = (bf16_t*)t.aT + ((int64_t)g * t.in_features + kd) * rpad + 8 * no;
     }
     st16(out, make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)));
   }
+}
+
+// The transposed copies as a launch of their own (backward paths whose first kernel cannot carry them as a side job).
+__global__ __launch_bounds__(256) void k_transpose_job(TransposeJob t, const int32_t* __restrict__ rank, int rpad) {
+  transpose_weights_job(t, rank, rpad, (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
 }
 
 // ---------------------------------------------------------------------------
@@ -903,6 +910,18 @@ int launch_pass_multi(const PassArgs* a, int n, const SegView& seg, const SegLay
   if (phases & 2)
     hipLaunchKernelGGL(k_expand_mfma_multi, dim3((unsigned)ceil_div(L.max_tiles * widest, 4), (unsigned)n), dim3(256), 0,
                        s, J, seg.tile_group, rows, (int)L.max_tiles);
+  return check_launch();
+}
+
+// B^T / A^T copies for the MFMA shrink and expand of a backward pass (bf16, out_features a multiple of 8).
+// Entries at and beyond a group's rank are left unwritten: those kernels never read them.
+int launch_transpose_job(const TransposeJob& t0, const int32_t* rank, int rpad, hipStream_t s) {
+  if (t0.groups == 0) return TK_OK;
+  TransposeJob t = t0;
+  t.skip_dead = 1;
+  const int64_t units = (int64_t)t.groups * rpad * ((t.bT ? t.out_features : 0) + t.in_features) / 8;
+  const int64_t blocks = std::min<int64_t>(4096, std::max<int64_t>(1, units / (2 * 256)));
+  hipLaunchKernelGGL(k_transpose_job, dim3((unsigned)blocks), dim3(256), 0, s, t, rank, rpad);
   return check_launch();
 }
 

@@ -207,6 +207,7 @@ struct TransposeJob {
   int32_t in_features, out_features, groups;
   int32_t y_blocks;  // 0: no job
   int32_t swizzle_a; // aT rows permuted inside every 128 (see PassArgs::expand_swizzled); in_features % 128 == 0
+  int32_t skip_dead; // leave entries at and beyond a group's rank unwritten (the MFMA kernels never read them)
 };
 
 // Row-contraction (weight gradient) pass: out_g[n][c] = sum_p hT[n][p] * src[row(p)][c].
@@ -265,6 +266,7 @@ struct WgradReduceJobs {
   int32_t n;
   WgradArgs a[2 * kMaxShared];
 };
+int launch_transpose_job(const TransposeJob& t, const int32_t* rank, int rpad, hipStream_t s);
 int launch_dy_fused_multi(const DyFusedJob* jobs, int n, const SegView& seg, const SegLayout& L, hipStream_t s);
 int launch_pass_multi(const PassArgs* a, int n, const SegView& seg, const SegLayout& L, int phases, hipStream_t s);
 int launch_wgrad_reduce_multi(const WgradArgs* sets, int n, const SegView& seg, const SegLayout& L, hipStream_t s);
