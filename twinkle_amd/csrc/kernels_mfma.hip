@@ -20,6 +20,9 @@
 #ifndef TK_DY_STAGES
 #define TK_DY_STAGES 2
 #endif
+#ifndef TK_COOP_STAGES
+#define TK_COOP_STAGES 3
+#endif
 #ifndef TK_WGRAD_STAGES
 #define TK_WGRAD_STAGES 3
 #endif
@@ -638,6 +641,120 @@ __global__ __launch_bounds__(RS * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
 }
 
 // ---------------------------------------------------------------------------
+// Weight gradient at padded rank 64: (chunk, 128 columns), two waves, each owning 32 rank indices and both
+// needing every tile of the source.  Two independent readers of a tile drift apart and the later one misses
+// the CU's cache (measured: 1.66 x the source bytes fetched from memory), so here the tile crosses the
+// memory system once: each wave requests half of it (4 of the 8 rows of every lane's 8 x 8 block), S - 1
+// tiles ahead, the halves meet in a double-buffered LDS tile behind an LDS-only barrier (global loads stay
+// in flight), and every wave reads the whole tile back in the operand layout.  Padding rows are zeroed when
+// they are written to LDS.  One barrier per tile: a wave overwrites a buffer two tiles later, after the
+// barrier that every reader of it has passed.
+// ---------------------------------------------------------------------------
+template <int S>
+__global__ __launch_bounds__(128) void k_wgrad_coop64(WgradArgs a, const ChunkInfo* __restrict__ chunks,
+                                                      const int32_t* __restrict__ slot_rows) {
+  constexpr int NB = 4, RS = 2, NBW = 2;
+  constexpr int OS = kWgradStageStride;
+  constexpr int XS = 136;  // row stride of a staged tile in bf16 (272 B)
+  // the tile buffers are dead when the result is staged: one array serves both
+  __shared__ __attribute__((aligned(16))) float lds[16 * NB * OS];
+  static_assert(sizeof(float) * 16 * NB * OS >= sizeof(bf16_t) * 2 * kTileRows * XS, "two staged tiles fit");
+  extern __shared__ __attribute__((aligned(16))) int32_t rows_s[];  // the chunk's row indices
+  const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kb = lane >> 4, rs = tid >> 6;
+  if ((int)blockIdx.y < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
+    transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (RS * 64) + tid,
+                          (int64_t)a.tr.y_blocks * gridDim.x * (RS * 64));
+    return;
+  }
+  const int c0 = blockIdx.x * 128;
+  const ChunkInfo ci = chunks[blockIdx.y - a.tr.y_blocks];
+  const int g = ci.group;
+  if (g < 0) return;
+  const int r = min(a.rank[g], 16 * NB);
+  if (r <= 0) return;
+  const int nt = ci.ntiles;
+  for (int i = tid; i < nt * kTileRows; i += RS * 64) rows_s[i] = slot_rows[ci.tile0 * kTileRows + i];
+  __syncthreads();
+  const int n_base = rs * NBW * 16;   // first rank index of this wave
+  const bool mine = r > n_base;       // a wave without live rank indices still carries its half of every tile
+
+  bf16_t* tiles = reinterpret_cast<bf16_t*>(lds);
+  const bf16_t* src = (const bf16_t*)a.src + c0 + 8 * li;
+  const bf16_t* hT = (const bf16_t*)a.hT + (int64_t)(n_base + li) * a.ldh + (int64_t)ci.tile0 * kTileRows + 8 * kb;
+  f32x4 acc[8][NBW];
+#pragma unroll
+  for (int q = 0; q < 8; ++q)
+#pragma unroll
+    for (int nb = 0; nb < NBW; ++nb) acc[q][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  struct Piece {
+    uint4 x[4];      // rows 8 kb + 4 rs + i of the tile, columns 8 li .. 8 li + 7
+    uint4 h[NBW];
+    uint32_t live;
+  };
+  auto issue = [&](int t, Piece& P) {
+    const int tc = min(t, nt - 1);
+    const int4 rr = *reinterpret_cast<const int4*>(rows_s + tc * kTileRows + 8 * kb + 4 * rs);
+    const int rows[4] = {rr.x, rr.y, rr.z, rr.w};
+    P.live = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      P.x[i] = ld16(src + (int64_t)max(rows[i], 0) * a.ld_src);
+      P.live |= rows[i] >= 0 ? (1u << i) : 0u;
+    }
+#pragma unroll
+    for (int nb = 0; nb < NBW; ++nb) P.h[nb] = ld16(hT + (int64_t)(16 * nb) * a.ldh + tc * kTileRows);
+  };
+  auto consume = [&](int t, const Piece& P) {
+    bf16_t* buf = tiles + (t & 1) * (kTileRows * XS);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      st16(buf + (8 * kb + 4 * rs + i) * XS + 8 * li, (P.live >> i) & 1u ? P.x[i] : zero4());
+    lds_barrier();
+    if (!mine) return;
+    uint4 x[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = ld16(buf + (8 * kb + i) * XS + 8 * li);
+    // 8x8 transpose inside the lane: tr holds column q of the 8 rows
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int d = q >> 1;
+      const uint32_t sel = (q & 1) ? 0x07060302u : 0x05040100u;
+      uint32_t e[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t wsrc[4] = {x[i].x, x[i].y, x[i].z, x[i].w};
+        e[i] = wsrc[d];
+      }
+      uint4 tr;
+      tr.x = __builtin_amdgcn_perm(e[1], e[0], sel);
+      tr.y = __builtin_amdgcn_perm(e[3], e[2], sel);
+      tr.z = __builtin_amdgcn_perm(e[5], e[4], sel);
+      tr.w = __builtin_amdgcn_perm(e[7], e[6], sel);
+#pragma unroll
+      for (int nb = 0; nb < NBW; ++nb) acc[q][nb] = mfma16(tr, P.h[nb], acc[q][nb]);
+    }
+  };
+  Piece T[S];
+#pragma unroll
+  for (int i = 0; i < S - 1; ++i) issue(i, T[i]);
+  int t = 0;
+  for (; t + S <= nt; t += S) {  // every tile consumed in here exists (the youngest requests may lie past the end)
+#pragma unroll
+    for (int i = 0; i < S; ++i) {
+      issue(t + i + S - 1, T[(i + S - 1) % S]);
+      consume(t + i, T[i]);
+    }
+  }
+  // fewer than S tiles are left, all of them requested already; both waves take the same trips (barriers inside)
+#pragma unroll
+  for (int i = 0; i < S - 1; ++i)
+    if (t + i < nt) consume(t + i, T[i]);
+  __syncthreads();  // the last tile has been read everywhere: its buffer becomes the staging area
+  if (mine) wgrad_store<NBW>(acc, lds + n_base * OS, a, ci, g, r, c0, lane, n_base);
+}
+
+// ---------------------------------------------------------------------------
 // Backward, both uses of dy in one pass (rank <= 16, width a multiple of 512): a block of four waves owns
 // (chunk of one group, 512 columns), wave w the columns [128 w, 128 w + 128) of it.
 // Per tile a wave loads its 32 x 128 piece once, in the weight-gradient layout (a lane holds 8 rows x 8
@@ -850,6 +967,19 @@ void launch_wgrad_pipe(const WgradArgs& a0, const SegView& seg, const SegLayout&
                      seg.slot_table(a.map_rows));
 }
 
+void launch_wgrad_coop64(const WgradArgs& a0, const SegView& seg, const SegLayout& L, hipStream_t s) {
+  constexpr int S = TK_COOP_STAGES;
+  WgradArgs a = a0;
+  a.tr.y_blocks = 0;
+  if (a.tr.aT) {
+    const int64_t units = (int64_t)a.tr.groups * a.rpad * ((a.tr.out_features + a.tr.in_features) / 8);
+    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 128) * 128)));
+  }
+  const dim3 grid((unsigned)(a.width / 128), (unsigned)(L.max_chunks + a.tr.y_blocks));
+  const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);
+  hipLaunchKernelGGL((k_wgrad_coop64<S>), grid, dim3(128), dyn, s, a, seg.chunks, seg.slot_table(a.map_rows));
+}
+
 }  // namespace
 
 bool dy_fused_supported(const WgradArgs& a, int kslices) {
@@ -953,7 +1083,7 @@ int launch_wgrad_mfma(const WgradArgs& a, const SegView& seg, const SegLayout& L
   if (L.rows == 0) return TK_OK;
   if (a.rpad <= 16) launch_wgrad_pipe<1, 1, TK_WGRAD_STAGES>(a, seg, L, s);
   else if (a.rpad <= 32) launch_wgrad_pipe<2, 1, 3>(a, seg, L, s);
-  else launch_wgrad_pipe<4, 2, 3>(a, seg, L, s);
+  else launch_wgrad_coop64(a, seg, L, s);
   return check_launch();
 }
 
