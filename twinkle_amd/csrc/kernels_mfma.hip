@@ -16,7 +16,7 @@
 
 #include "tk_mfma.h"
 
-// depths of the software pipelines of k_dy_fused and k_wgrad_pipe<1, 1, S> (tiles in registers per wave)
+// depths of the software pipelines of k_dy_fused, k_wgrad_pipe<1, S> and k_wgrad_coop64<S> (tiles in registers per wave)
 #ifndef TK_DY_STAGES
 #define TK_DY_STAGES 2
 #endif
@@ -529,7 +529,7 @@ __global__ __launch_bounds__(256) void k_transpose_job(TransposeJob t, const int
 // ---------------------------------------------------------------------------
 // Weight gradient: out_g[n][c] = sum over the rows of group g of hT[n][slot] * src[row(slot)][c].
 //
-// Work item = (chunk of one group, 128 source columns), one block of RS waves.  A wave walks all tiles of
+// Work item = (chunk of one group, 128 source columns), one wave.  The wave walks all tiles of
 // the chunk with an S-stage software pipeline: the source rows of tile t+S-1 are requested before tile t
 // is consumed, so a wave has S-1 tiles (8 KB each) in flight; the chunk's row indices wait in LDS, where
 // reading them does not have to wait for the tile loads in flight.  A grid of (chunks x 128-column
@@ -540,22 +540,19 @@ __global__ __launch_bounds__(256) void k_transpose_job(TransposeJob t, const int
 // partial buffer (groups that span several chunks; k_wgrad_reduce adds the chunks in order) or straight
 // into the gradient (single-chunk groups).  No atomics: the result is bitwise repeatable.
 //
-// RS > 1 (padded rank 64, where 128 columns x rank of accumulators would leave one wave per SIMD): the
-// RS waves of a block walk the same tiles and each own 1/RS of the rank indices; the second reader of a
-// tile finds it in the CU's cache.
+// Padded rank 64 (128 columns x 64 rank indices of accumulators would leave one wave per SIMD) has its own
+// kernel below.
 // ---------------------------------------------------------------------------
-template <int NB, int RS, int S>
-__global__ __launch_bounds__(RS * 64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo* __restrict__ chunks,
+template <int NB, int S>
+__global__ __launch_bounds__(64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo* __restrict__ chunks,
                                                         const int32_t* __restrict__ slot_rows) {
-  static_assert(NB % RS == 0, "rank blocks must divide evenly");
-  constexpr int NBW = NB / RS;  // blocks of 16 rank indices per wave
   constexpr int OS = kWgradStageStride;
   __shared__ __attribute__((aligned(16))) float lds[16 * NB * OS];
   extern __shared__ __attribute__((aligned(16))) int32_t rows_s[];  // the chunk's row indices
-  const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kb = lane >> 4, rs = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kb = lane >> 4;
   if ((int)blockIdx.y < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
-    transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (RS * 64) + tid,
-                          (int64_t)a.tr.y_blocks * gridDim.x * (RS * 64));
+    transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * 64 + tid,
+                          (int64_t)a.tr.y_blocks * gridDim.x * 64);
     return;
   }
   // column block fastest: blocks that run together read neighbouring pieces of the same rows
@@ -566,18 +563,16 @@ __global__ __launch_bounds__(RS * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
   const int r = min(a.rank[g], 16 * NB);
   if (r <= 0) return;
   const int nt = ci.ntiles;
-  for (int i = tid; i < nt * kTileRows; i += RS * 64) rows_s[i] = slot_rows[ci.tile0 * kTileRows + i];
+  for (int i = tid; i < nt * kTileRows; i += 64) rows_s[i] = slot_rows[ci.tile0 * kTileRows + i];
   __syncthreads();
-  const int n_base = rs * NBW * 16;  // first rank index of this wave
-  if (r <= n_base) return;           // from here on the waves of a block never meet at a barrier
 
   const bf16_t* src = (const bf16_t*)a.src + c0 + 8 * li;
-  const bf16_t* hT = (const bf16_t*)a.hT + (int64_t)(n_base + li) * a.ldh + (int64_t)ci.tile0 * kTileRows + 8 * kb;
-  f32x4 acc[8][NBW];
+  const bf16_t* hT = (const bf16_t*)a.hT + (int64_t)li * a.ldh + (int64_t)ci.tile0 * kTileRows + 8 * kb;
+  f32x4 acc[8][NB];
 #pragma unroll
   for (int q = 0; q < 8; ++q)
 #pragma unroll
-    for (int nb = 0; nb < NBW; ++nb) acc[q][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int nb = 0; nb < NB; ++nb) acc[q][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // The loop body below is straight-line code: every load is unconditional (tiles past the end re-read the
   // last tile, padding slots read row 0) and what must not count is zeroed when it is consumed.  With no
@@ -585,7 +580,7 @@ __global__ __launch_bounds__(RS * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
   // younger ones in flight.
   struct Tile {
     uint4 x[8];
-    uint4 h[NBW];
+    uint4 h[NB];
     uint32_t live;  // bit q: row q of this lane is a real row of a tile inside the chunk
   };
   auto issue = [&](int t, Tile& T) {
@@ -600,7 +595,7 @@ __global__ __launch_bounds__(RS * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
       T.live |= (t < nt && rows[q] >= 0) ? (1u << q) : 0u;
     }
 #pragma unroll
-    for (int nb = 0; nb < NBW; ++nb) T.h[nb] = ld16(hT + (int64_t)(16 * nb) * a.ldh + tc * kTileRows);
+    for (int nb = 0; nb < NB; ++nb) T.h[nb] = ld16(hT + (int64_t)(16 * nb) * a.ldh + tc * kTileRows);
   };
   auto consume = [&](const Tile& T) {
     // 8x8 transpose inside the lane: tr holds column q of the 8 rows
@@ -620,7 +615,7 @@ __global__ __launch_bounds__(RS * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
       tr.z = __builtin_amdgcn_perm(e[5], e[4], sel);
       tr.w = __builtin_amdgcn_perm(e[7], e[6], sel);
 #pragma unroll
-      for (int nb = 0; nb < NBW; ++nb) acc[q][nb] = mfma16(tr, T.h[nb], acc[q][nb]);
+      for (int nb = 0; nb < NB; ++nb) acc[q][nb] = mfma16(tr, T.h[nb], acc[q][nb]);
     }
   };
   Tile T[S];
@@ -637,7 +632,7 @@ __global__ __launch_bounds__(RS * 64) void k_wgrad_pipe(WgradArgs a, const Chunk
   // drain: fewer than S tiles are left, all requested already (tiles past the end count as zeros)
 #pragma unroll
   for (int i = 0; i < S - 1; ++i) consume(T[i]);
-  wgrad_store<NBW>(acc, lds + n_base * OS, a, ci, g, r, c0, lane, n_base);
+  wgrad_store<NB>(acc, lds, a, ci, g, r, c0, lane);
 }
 
 // ---------------------------------------------------------------------------
@@ -953,17 +948,17 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
   }
 }
 
-template <int NB, int RS, int S>
+template <int NB, int S>
 void launch_wgrad_pipe(const WgradArgs& a0, const SegView& seg, const SegLayout& L, hipStream_t s) {
   WgradArgs a = a0;
   a.tr.y_blocks = 0;
   if (a.tr.aT) {  // about four 16-byte outputs per thread of the side job
     const int64_t units = (int64_t)a.tr.groups * a.rpad * ((a.tr.out_features + a.tr.in_features) / 8);
-    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 128) * (RS * 64))));
+    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 128) * 64)));
   }
   const dim3 grid((unsigned)(a.width / 128), (unsigned)(L.max_chunks + a.tr.y_blocks));
   const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);  // a chunk's row indices
-  hipLaunchKernelGGL((k_wgrad_pipe<NB, RS, S>), grid, dim3(RS * 64), dyn, s, a, seg.chunks,
+  hipLaunchKernelGGL((k_wgrad_pipe<NB, S>), grid, dim3(64), dyn, s, a, seg.chunks,
                      seg.slot_table(a.map_rows));
 }
 
@@ -1081,8 +1076,8 @@ bool wgrad_mfma_supported(const WgradArgs& a) {
 
 int launch_wgrad_mfma(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
   if (L.rows == 0) return TK_OK;
-  if (a.rpad <= 16) launch_wgrad_pipe<1, 1, TK_WGRAD_STAGES>(a, seg, L, s);
-  else if (a.rpad <= 32) launch_wgrad_pipe<2, 1, 3>(a, seg, L, s);
+  if (a.rpad <= 16) launch_wgrad_pipe<1, TK_WGRAD_STAGES>(a, seg, L, s);
+  else if (a.rpad <= 32) launch_wgrad_pipe<2, 3>(a, seg, L, s);
   else launch_wgrad_coop64(a, seg, L, s);
   return check_launch();
 }
