@@ -55,3 +55,43 @@ def test_ops_refuse_cpu_tensors():
     from twinkle_amd import build_segments
     with pytest.raises(RuntimeError):
         build_segments(torch.zeros(8, dtype=torch.int32), 2)
+
+
+def test_shared_entry_points_reject_malformed_arguments_on_the_host():
+    """Argument checks of tk_lora_fwd_shared / tk_lora_bwd_shared run before any GPU work (fake device pointers)."""
+    import ctypes
+    from twinkle_amd import _lib
+    lib = _lib.load()
+
+    def desc(rows=64, k=2048, m=512):
+        d = _lib.LoraDesc()
+        d.rows, d.in_features, d.out_features, d.num_groups, d.max_rank, d.dtype = rows, k, m, 2, 16, 1
+        d.map_rows, d.lda, d.ldb = 1, k, 16
+        d.seg_ws = d.lora_A = d.lora_B = d.rank = d.scale = 0x1000      # never dereferenced by the checks
+        return d
+
+    def table(descs):
+        return (ctypes.c_void_p * len(descs))(*[ctypes.addressof(d) for d in descs])
+
+    ptrs = (ctypes.c_void_p * 5)(*([0x1000] * 5))
+    lds = (ctypes.c_int64 * 5)(*([4096] * 5))
+    a, b = desc(), desc()
+    bad = _lib.TK_ERR_INVALID
+    fwd = lambda t, n, y=ptrs, ld=lds, h=ptrs: lib.tk_lora_fwd_shared(t, n, 0x1000, 2048, y, ld, h, None)  # noqa: E731
+    assert fwd(None, 2) == bad                                   # no descriptor table
+    assert fwd(table([a, b]), 0) == bad                          # no projection
+    assert fwd(table([a] * 5), 5) == bad                         # more than TK_MAX_SHARED
+    assert fwd(table([a, desc(rows=65)]), 2) == bad              # projections disagree in rows
+    assert fwd(table([a, desc(k=1024)]), 2) == bad               # ... in in_features
+    assert fwd(table([a, b]), 2, y=None) == bad                  # no output table
+    small = (ctypes.c_int64 * 2)(4096, 100)
+    assert fwd(table([a, b]), 2, ld=small) == bad                # a row stride below out_features
+    empty = desc(rows=0)
+    assert fwd(table([empty, desc(rows=0)]), 2) == _lib.TK_OK    # nothing to do
+    assert lib.tk_lora_bwd_shared(table([a, b]), 2, ptrs, lds, 0x1000, 2048, ptrs, 0x1000, 2048, None, ptrs, 0, ptrs,
+                                  lds, None) == bad              # no dA table
+    assert lib.tk_lora_bwd_shared(table([a, b]), 2, ptrs, lds, 0x1000, 100, ptrs, 0x1000, 2048, ptrs, ptrs, 0, ptrs,
+                                  lds, None) == bad              # x row stride below in_features
+    tiny = (ctypes.c_int64 * 2)(16, 16)
+    assert lib.tk_lora_bwd_shared(table([a, b]), 2, ptrs, lds, 0x1000, 2048, ptrs, 0x1000, 2048, ptrs, ptrs, 0, ptrs,
+                                  tiny, None) == _lib.TK_ERR_WORKSPACE

@@ -77,6 +77,7 @@ class AdapterGroups:
         self._grad_b_rel = torch.tensor([(self._b_arena_off[self.b_index[i]] + self.b_offset[i]) * esz
                                          for i in range(g)], dtype=torch.int64, device=dev)
         self._ptr_key = None
+        self._size_cache = {}
         self.a_ptrs = self.b_ptrs = None
         self.refresh()
 
@@ -136,16 +137,26 @@ def _check_rows(t: torch.Tensor, name: str, rows: int, width: int, dtype: torch.
         raise ValueError(f'{name} has dtype {t.dtype}, adapters have {dtype}')
 
 
-def lora_h_bytes(seg: SegmentTable, groups: AdapterGroups) -> int:
-    n = _lib.load().tk_lora_h_bytes(ctypes.byref(_desc(seg, groups, True)))
-    _lib.check(n, 'tk_lora_h_bytes')
+def _cached_size(seg: SegmentTable, groups: AdapterGroups, which: str) -> int:
+    # both sizes are functions of the shapes alone (rows, groups, widths, padded rank, dtype), all of which are
+    # fixed for an AdapterGroups object except the row count
+    key = (which, seg.rows)
+    n = groups._size_cache.get(key)
+    if n is None:
+        n = getattr(_lib.load(), which)(ctypes.byref(_desc(seg, groups, True)))
+        _lib.check(n, which)
+        if len(groups._size_cache) > 64:
+            groups._size_cache.clear()
+        groups._size_cache[key] = n
     return n
+
+
+def lora_h_bytes(seg: SegmentTable, groups: AdapterGroups) -> int:
+    return _cached_size(seg, groups, 'tk_lora_h_bytes')
 
 
 def lora_bwd_workspace_bytes(seg: SegmentTable, groups: AdapterGroups) -> int:
-    n = _lib.load().tk_lora_bwd_workspace_bytes(ctypes.byref(_desc(seg, groups, True)))
-    _lib.check(n, 'tk_lora_bwd_workspace_bytes')
-    return n
+    return _cached_size(seg, groups, 'tk_lora_bwd_workspace_bytes')
 
 
 def lora_fwd_(x: torch.Tensor, y: torch.Tensor, seg: SegmentTable, groups: AdapterGroups, map_rows: bool = True,
