@@ -27,6 +27,10 @@
 #define TK_WGRAD_STAGES 3
 #endif
 
+#ifndef TK_XCD_MAP
+#define TK_XCD_MAP(b, n) xcd_contiguous(b, n)
+#endif
+
 namespace tk {
 
 namespace {
@@ -381,7 +385,8 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
   const int ngroups = a.width_dst >> 7;
   const int nbt = (ngroups + 3) >> 2;  // blocks per tile set: column block fastest
-  const int cb = blockIdx.x % nbt, tile0 = (blockIdx.x / nbt) * TPI;
+  const int block = TK_XCD_MAP(blockIdx.x, gridDim.x);
+  const int cb = block % nbt, tile0 = (block / nbt) * TPI;
   const int cg = cb * 4 + wave;
   if (cg >= ngroups) return;
   const int nt = min(TPI, max_tiles - tile0);

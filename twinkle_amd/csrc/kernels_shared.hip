@@ -15,16 +15,6 @@ namespace tk {
 
 namespace {
 
-// Blocks go to the XCDs (each with an L2 of its own) round-robin.  This renumbering gives every XCD one
-// contiguous eighth of the work items, so that an XCD's L2 fetches the weights of few groups instead of all.
-__device__ inline int xcd_contiguous(int block, int blocks) {
-#ifdef TK_NO_XCD_MAP
-  return block;
-#endif
-  const int per = blocks >> 3;
-  return block < 8 * per ? (block & 7) * per + (block >> 3) : block;
-}
-
 template <typename T>
 __device__ inline T pick(const T (&v)[kMaxShared], int i) {  // v[i] without a register-indexed array
   T r = v[0];

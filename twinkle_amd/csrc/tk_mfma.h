@@ -91,6 +91,13 @@ __device__ inline void store_bf16x8(bf16_t* o, const float (&v)[8], int keep, bo
   }
 }
 
+// Blocks go to the XCDs (each with an L2 of its own) round-robin.  This renumbering gives every XCD one
+// contiguous eighth of the work items, so that an XCD's L2 fetches the weights of few groups instead of all.
+__device__ inline int xcd_contiguous(int block, int blocks) {
+  const int per = blocks >> 3;
+  return block < 8 * per ? (block & 7) * per + (block >> 3) : block;
+}
+
 // One wave's weight-gradient block out[n][c0 .. c0 + 127] (lane holds out[16 nb + li][32 kb + 8 v + q] in
 // acc[q][nb][v]) leaves through `lds` (RP rows of kWgradStageStride floats, private to the wave) as whole
 // 512-byte rows: into the chunk's slot of the partial buffer, or straight into the gradient when the
