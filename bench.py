@@ -227,6 +227,8 @@ def main():
                     help='cfg2 is the headline configuration; the others are the wider BASELINE shapes '
                          '(cfg3: 4096<->14336, T=32768, 32 adapters of rank 8..64; cfg5_q: 4096->4096, T=32768, 8 tenants '
                          'of rank 64, one per packed 4096-token sequence) for additional measurements')
+    ap.add_argument('--tokens', type=int, default=0,
+                    help='cfg2 with another number of tokens (a scaling measurement, not the headline configuration)')
     ap.add_argument('--optimizer-only', action='store_true',
                     help='run only the multi-tenant optimizer micro-benchmark and print its JSON (for profiling)')
     ap.add_argument('--shared-qkv', action='store_true',
@@ -254,7 +256,10 @@ def main():
     if args.shared_qkv:
         print(json.dumps({'shared_qkv': shared_qkv_bench(dev)}))
         return
-    if args.workload == 'cfg2':
+    if args.workload == 'cfg2' and args.tokens:
+        w = workloads.config2_qproj(tokens=args.tokens)
+        w.name = f'cfg2 shape with T={args.tokens}'
+    elif args.workload == 'cfg2':
         w = workloads.config2_qproj()
     elif args.workload == 'cfg5_q':
         w = workloads.config2_qproj(tokens=32768, n=8, r=64)
@@ -375,11 +380,11 @@ def main():
         'dtype': 'bf16',
         'data': 'synthetic',
         'config': {'workload': ('BASELINE config 2: Llama-3-8B q_proj 4096->4096, T=16384, 16 adapters rank 16 alpha 32, '
-                                'Zipf(1.1) ids shuffled' if args.workload == 'cfg2' else w.name) +
+                                'Zipf(1.1) ids shuffled' if args.workload == 'cfg2' and not args.tokens else w.name) +
                                '; step = segment build + LoRA fwd + LoRA bwd (dX, dA, dB); base GEMM excluded',
                    'tokens': T, 'in': K, 'out': M, 'adapters': G, 'rank': max(w.ranks)},
         'roofline': {'bound': 'hbm', 'achieved': achieved, 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                     'frac': achieved / HBM_PEAK_GBS, 'traffic': measured_traffic('k_expand_mfma<1>') if args.workload == 'cfg2' else None,
+                     'frac': achieved / HBM_PEAK_GBS, 'traffic': measured_traffic('k_expand_mfma<1>') if args.workload == 'cfg2' and not args.tokens else None,
                      'kernel': ('k_expand_mfma<1>' if max(w.ranks) <= 16 else
                                 f'k_expand_multi<{2 if max(w.ranks) <= 32 else 4},4>') + ' (y += h B^T in place), forward launch',
                      'algorithmic_bytes_per_launch': expand_bytes, 'avg_launch_ms': expand_ms,
