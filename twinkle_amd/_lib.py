@@ -123,4 +123,6 @@ def dtype_code(dtype: torch.dtype) -> int:
 
 
 def stream_ptr() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """The current HIP stream of the current device as an integer handle."""
+    # the raw accessor costs a fraction of a microsecond; torch.cuda.current_stream() builds a Stream object (8 us)
+    return torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice())

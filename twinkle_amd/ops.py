@@ -78,6 +78,7 @@ class AdapterGroups:
                                          for i in range(g)], dtype=torch.int64, device=dev)
         self._ptr_key = None
         self._size_cache = {}
+        self._desc_template = self._desc_key = None
         self.a_ptrs = self.b_ptrs = None
         self.refresh()
 
@@ -91,7 +92,7 @@ class AdapterGroups:
 
     def refresh(self) -> None:
         """Rebuild the device pointer arrays if a parameter's storage moved."""
-        key = tuple(t.data_ptr() for t in self.a_tensors) + tuple(t.data_ptr() for t in self.b_tensors)
+        key = [t.data_ptr() for t in self.a_tensors] + [t.data_ptr() for t in self.b_tensors]
         if key == self._ptr_key:
             return
         esz = self.a_tensors[0].element_size()
@@ -109,21 +110,27 @@ class AdapterGroups:
 
 def _desc(seg: SegmentTable, groups: AdapterGroups, map_rows: bool) -> _lib.LoraDesc:
     groups.refresh()
-    d = _lib.LoraDesc()
+    # a fresh struct per call (callers keep several alive at once), copied from a template that holds everything
+    # which is fixed for the AdapterGroups object
+    template = groups._desc_template
+    if template is None or groups._desc_key is not groups._ptr_key:
+        template = _lib.LoraDesc()
+        template.in_features = groups.in_features
+        template.out_features = groups.out_features
+        template.num_groups = groups.num_groups
+        template.max_rank = groups.max_rank
+        template.dtype = _lib.dtype_code(groups.dtype)
+        template.lora_A = groups.a_ptrs.data_ptr()
+        template.lora_B = groups.b_ptrs.data_ptr()
+        template.lda = groups.lda
+        template.ldb = groups.ldb
+        template.rank = groups.rank_dev.data_ptr()
+        template.scale = groups.scale_dev.data_ptr()
+        groups._desc_template, groups._desc_key = template, groups._ptr_key
+    d = _lib.LoraDesc.from_buffer_copy(template)
     d.rows = seg.rows
-    d.in_features = groups.in_features
-    d.out_features = groups.out_features
-    d.num_groups = groups.num_groups
-    d.max_rank = groups.max_rank
-    d.dtype = _lib.dtype_code(groups.dtype)
     d.map_rows = 1 if map_rows else 0
     d.seg_ws = seg.workspace.data_ptr()
-    d.lora_A = groups.a_ptrs.data_ptr()
-    d.lora_B = groups.b_ptrs.data_ptr()
-    d.lda = groups.lda
-    d.ldb = groups.ldb
-    d.rank = groups.rank_dev.data_ptr()
-    d.scale = groups.scale_dev.data_ptr()
     return d
 
 
