@@ -35,10 +35,10 @@ enum { TK_DTYPE_F32 = 0, TK_DTYPE_BF16 = 1 };
 enum { TK_KEY_I32 = 0, TK_KEY_I64 = 1 };
 
 /* Rows per forward tile and per smallest weight-gradient chunk (fixed at build time; chunks grow with the
- * batch: 512 rows up to 16384 rows, then doubling with the row count up to 4096). */
+ * batch, about 32 of them over all rows: 128 rows up to 4096 rows, 512 at 16384, up to 4096). */
 #define TK_TILE_ROWS 32
 #ifndef TK_CHUNK_ROWS
-#define TK_CHUNK_ROWS 512
+#define TK_CHUNK_ROWS 128
 #endif
 #define TK_MAX_GROUPS 16384
 #define TK_MAX_RANK 128

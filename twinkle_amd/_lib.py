@@ -24,7 +24,7 @@ TK_DTYPE_BF16 = 1
 TK_KEY_I32 = 0
 TK_KEY_I64 = 1
 TK_TILE_ROWS = 32
-TK_CHUNK_ROWS = 512
+TK_CHUNK_ROWS = 128
 TK_MAX_GROUPS = 16384
 TK_MAX_RANK = 128
 

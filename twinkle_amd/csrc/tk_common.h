@@ -10,7 +10,7 @@ namespace tk {
 
 constexpr int kWave = 64;
 constexpr int kTileRows = TK_TILE_ROWS;    // rows per forward tile (two 16-row MFMA tiles)
-constexpr int kChunkTilesMin = TK_CHUNK_ROWS / TK_TILE_ROWS;  // smallest weight-gradient chunk: 16 tiles (512 rows)
+constexpr int kChunkTilesMin = TK_CHUNK_ROWS / TK_TILE_ROWS;  // smallest weight-gradient chunk: 4 tiles (128 rows)
 constexpr int kChunkTilesMax = 128;                             // largest: 4096 rows
 constexpr int kSortBlockRows = 512;        // rows one single-wave block orders in the scatter pass
 
@@ -47,8 +47,10 @@ struct ChunkInfo {  // one weight-gradient chunk: tiles [tile0, tile0 + ntiles) 
 // A chunk is the unit the row contractions (dA, dB) are split into: up to `chunk_tiles` tiles of one
 // group.  Every chunk of a multi-chunk group costs one fp32 partial of rank x width, so the chunk
 // grows with the batch (about 32 chunks over all rows): the partial traffic stays a fixed small
-// fraction of the activations while the number of work items stays in the thousands.  A function
-// of the row count alone, so producer and consumers agree.
+// fraction of the activations while the number of work items stays in the thousands.  Small batches
+// get small chunks: a block walks its chunk tile by tile, one memory latency each, so there the chunk
+// length sets the duration of the row-contraction kernels.  A function of the row count alone, so
+// producer and consumers agree.
 static inline int chunk_tiles_for(int64_t rows) {
   int t = kChunkTilesMin;
   while (t < kChunkTilesMax && (int64_t)t * kTileRows * 32 < rows) t <<= 1;
