@@ -388,7 +388,7 @@ int tk_lora_fwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* 
   hipStream_t s = (hipStream_t)stream;
   SegLayout L(d0->rows, d0->num_groups);
   SegView V(d0->seg_ws, L);
-  PassArgs a[TK_MAX_SHARED];
+  PassArgs a[TK_MAX_SHARED] = {};
   bool fast = shared_fast_path(descs, n);
   for (int p = 0; p < n; ++p) {
     a[p] = fwd_pass_args(descs[p], x, ldx, y[p], ldy[p], h[p]);
@@ -451,9 +451,9 @@ int tk_lora_bwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* 
   ea.dst = dx;  ea.ld_dst = lddx;  ea.width_dst = d0->in_features;  ea.map_rows = d0->map_rows;  ea.nproj = n;
   SharedWgradArgs wa{};
   wa.nproj = n;
-  DyFusedJob dj[TK_MAX_SHARED];
-  PassArgs pa[TK_MAX_SHARED];
-  WgradArgs red[2 * TK_MAX_SHARED];
+  DyFusedJob dj[TK_MAX_SHARED] = {};
+  PassArgs pa[TK_MAX_SHARED] = {};
+  WgradArgs red[2 * TK_MAX_SHARED] = {};
   for (int p = 0; p < n; ++p) {
     BwdPlan& P = plan[p];
     dj[p].a = P.gb;
