@@ -162,12 +162,27 @@ def test_forward_shared_equals_layer_by_layer(dev, dtype, d, kv):
     (q0, k0, v0), dx0, g0 = run(False)
     (q1, k1, v1), dx1, g1 = run(True)
     bf16 = dtype == torch.bfloat16
-    for a, b in ((q0, q1), (k0, k1), (v0, v1)):
-        assert torch.equal(a, b) if bf16 else max_rel_err(b, a) < 1e-6
-    assert g0.keys() == g1.keys()
-    for n in g0:
-        assert (torch.equal(g0[n], g1[n]) if bf16 and 'lora_' in n else max_rel_err(g1[n], g0[n].double()) < 1e-5), n
-    assert max_rel_err(dx1, dx0.double()) < (2e-2 if bf16 else 1e-5)
+
+    def same(outs, dx, grads):
+        for a, b in zip((q0, k0, v0), outs):
+            assert torch.equal(a, b) if bf16 else max_rel_err(b, a) < 1e-6
+        assert g0.keys() == grads.keys()
+        for n in g0:
+            assert (torch.equal(g0[n], grads[n]) if bf16 and 'lora_' in n
+                    else max_rel_err(grads[n], g0[n].double()) < 1e-5), n
+        assert max_rel_err(dx, dx0.double()) < (2e-2 if bf16 else 1e-5)
+
+    same((q1, k1, v1), dx1, g1)
+    # the module's own forward (q_proj(x), k_proj(x), v_proj(x) one after the other) with the group declared
+    ml.share_inputs([layers])
+    calls = []
+    original = ml.forward_shared
+    ml.forward_shared = lambda ls, t: calls.append(len(ls)) or original(ls, t)
+    outs2, dx2, g2 = run(False)
+    ml.forward_shared = original
+    ml.unshare_inputs()
+    assert calls == [3]
+    same(outs2, dx2, g2)
     # one adapter per call (the reference's adapter() context) takes the same route
     with ml.adapter('carol'):
         a = ml.forward_shared(layers, x)

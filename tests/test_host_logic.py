@@ -246,3 +246,48 @@ def test_adapter_checkpoint_round_trip_in_peft_format(tmp_path):
     assert torch.equal(after[:4], a_src[:4]) and torch.equal(after[4:], before[4:])
     for k, v in ml2.get_state_dict('alice').items():
         assert torch.equal(v, saved['base_model.' + k])
+
+
+def test_share_inputs_bookkeeping_without_a_gpu():
+    """share_inputs: the first sibling that sees a tensor computes the group, the others collect; no stale results."""
+    from torch import nn
+
+    class QKV(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q_proj, self.k_proj, self.v_proj = nn.Linear(16, 16), nn.Linear(16, 8), nn.Linear(16, 8)
+
+        def forward(self, x):
+            return self.q_proj(x), self.k_proj(x), self.v_proj(x)
+
+    torch.manual_seed(0)
+    ml = MultiLora(max_loras=2, max_r=4)
+    model = ml.patch(QKV(), target_modules='all-linear')
+    ml.acquire_lora('alice', LoraConfig(r=4, lora_alpha=8, target_modules='all-linear'))
+    x = torch.randn(5, 16)
+    with ml.adapter('alice', disable_lora=True):                    # base path only: runs on the CPU
+        want = model(x)
+        calls = []
+        original = ml.forward_shared
+        ml.forward_shared = lambda layers, t: calls.append(len(layers)) or original(layers, t)
+        ml.share_inputs([['model.q_proj', 'model.k_proj', 'model.v_proj']])
+        got = model(x)
+        assert calls == [3]                                         # one group computation for three layer calls
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+        m = model.model
+        state = m.q_proj._tk_shared_inputs
+        assert state.source is None and not state.pending           # everything was collected
+        # a sibling called with another tensor starts over instead of handing out a stale result
+        k1 = m.k_proj(x)
+        x2 = torch.randn(5, 16)
+        v2 = m.v_proj(x2)
+        assert torch.equal(k1, want[1]) and torch.equal(v2, torch.nn.functional.linear(x2, m.v_proj.base_layer.weight,
+                                                                                      m.v_proj.base_layer.bias))
+        x2.add_(1.0)                                                # same object, new version: recomputed
+        assert torch.equal(m.q_proj(x2), torch.nn.functional.linear(x2, m.q_proj.base_layer.weight,
+                                                                    m.q_proj.base_layer.bias))
+        ml.unshare_inputs()
+        assert not hasattr(m.q_proj, '_tk_shared_inputs')
+    with pytest.raises(ValueError):
+        ml.share_inputs([['model.q_proj']])

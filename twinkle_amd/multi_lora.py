@@ -37,6 +37,28 @@ class LoraTenant:
     lora_A_weights: Dict[str, torch.Tensor] = field(default_factory=dict)
 
 
+class _SharedInputGroup:
+    """Layers that are called one after the other on the same tensor (q / k / v, gate / up)."""
+
+    def __init__(self, layers):
+        self.layers = list(layers)
+        self.source = None       # the input the pending outputs were computed from
+        self.version = -1
+        self.pending = {}        # id(layer) -> output not handed out yet
+
+    def take(self, layer, x):
+        if self.source is x and self.version == x._version and id(layer) in self.pending:
+            out = self.pending.pop(id(layer))
+            if not self.pending:
+                self.source = None
+            return out
+        return None
+
+    def fill(self, x, outs, first):
+        self.pending = {id(layer): out for layer, out in zip(self.layers, outs) if layer is not first}
+        self.source, self.version = (x, x._version) if self.pending else (None, -1)
+
+
 def _is_lora_layer(module) -> bool:
     return all(hasattr(module, a) for a in ('base_layer', 'lora_A', 'lora_B', 'lora_dropout'))
 
@@ -232,6 +254,20 @@ class MultiLora:
             return
 
         def _linear_forward(self, x: torch.Tensor, *args, **kwargs) -> torch.Tensor:
+            shared = getattr(self, '_tk_shared_inputs', None)
+            if shared is None or args or kwargs:
+                return _forward_one(self, x, *args, **kwargs)
+            # a sibling has computed this layer's output from the same tensor already, or this call computes
+            # the outputs of all siblings (see MultiLora.share_inputs)
+            self._check_forward_args(x)
+            out = shared.take(self, x)
+            if out is None:
+                outs = _self.forward_shared(shared.layers, x)
+                shared.fill(x, outs, self)
+                out = outs[shared.layers.index(self)]
+            return out
+
+        def _forward_one(self, x: torch.Tensor, *args, **kwargs) -> torch.Tensor:
             self._check_forward_args(x, *args, **kwargs)
             table = _self._batch_table
             only_slot = None
@@ -273,7 +309,37 @@ class MultiLora:
             return (result + delta.view(*result.shape[:-1], -1)).to(result_dtype)
 
         base_layer.forward = MethodType(_linear_forward, base_layer)
+        base_layer._tk_forward_one = MethodType(_forward_one, base_layer)   # this layer alone, whatever it shares
         base_layer.layer_name = name
+
+    def share_inputs(self, layer_groups: Sequence[Sequence]) -> None:
+        """Declare groups of patched layers that the model calls one after the other on the same tensor
+        (``[[q_proj, k_proj, v_proj], [gate_proj, up_proj]]`` per block; modules or their names inside the
+        patched module).  Model code stays as it is: the first layer of a group that sees a new input computes
+        the outputs of the whole group through :meth:`forward_shared` and the siblings, called with the same
+        tensor, pick theirs up.  A sibling called with another tensor (or twice) simply starts a new group
+        computation, so results never depend on the call pattern; outputs nobody collects are dropped at the next
+        call.  ``share_inputs([])`` clears nothing: call :meth:`unshare_inputs` for that.
+        """
+        named = {n: sub for m in self._modules() for n, sub in m.named_modules()}
+        for group in layer_groups:
+            layers = [named[m] if isinstance(m, str) else m for m in group]
+            if not 2 <= len(layers) <= 4:
+                raise ValueError(f'a group of shared inputs has 2 to 4 layers, got {len(layers)}')
+            for layer in layers:
+                if not _is_lora_layer(layer) or not hasattr(layer, 'layer_name'):
+                    raise ValueError('share_inputs takes layers that patch() has patched')
+            if len({layer.in_features for layer in layers}) != 1:
+                raise ValueError('layers that share an input must agree in in_features')
+            state = _SharedInputGroup(layers)
+            for layer in layers:
+                layer._tk_shared_inputs = state
+
+    def unshare_inputs(self) -> None:
+        for m in self._modules():
+            for sub in m.modules():
+                if hasattr(sub, '_tk_shared_inputs'):
+                    del sub._tk_shared_inputs
 
     def forward_shared(self, layers: Sequence, x: torch.Tensor) -> Tuple[torch.Tensor, ...]:
         """``tuple(layer(x) for layer in layers)`` for patched layers that read the same ``x`` (q / k / v,
@@ -308,7 +374,7 @@ class MultiLora:
                 break
             groups_list.append(groups)
         if not ok:
-            return tuple(layer(x) for layer in layers)
+            return tuple(getattr(layer, '_tk_forward_one', layer)(x) for layer in layers)
         x2 = x.reshape(-1, x.shape[-1])
         if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
             x2 = x2.contiguous()
