@@ -263,3 +263,116 @@ def test_batched_training_step_equals_tenants_one_after_the_other(dev):
             assert max_rel_err(got[n][k], p.detach()) < 2e-5, (n, k)
         for p in model2.parameters():
             p.grad = None
+
+
+# ---- a Llama-shaped block stack (BASELINE config 5 in miniature): seven projections per layer, packed sequences ----
+
+class _RMSNorm(nn.Module):
+
+    def __init__(self, d):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(d))
+
+    def forward(self, x):
+        v = x.float()
+        return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + 1e-5)).to(x.dtype) * self.weight
+
+
+class _LlamaLayer(nn.Module):
+
+    def __init__(self, d, heads, kv_heads, inter):
+        super().__init__()
+        self.heads, self.kv_heads, self.hd = heads, kv_heads, d // heads
+        self.input_layernorm, self.post_attention_layernorm = _RMSNorm(d), _RMSNorm(d)
+        self.q_proj = nn.Linear(d, d, bias=False)
+        self.k_proj = nn.Linear(d, kv_heads * self.hd, bias=False)
+        self.v_proj = nn.Linear(d, kv_heads * self.hd, bias=False)
+        self.o_proj = nn.Linear(d, d, bias=False)
+        self.gate_proj = nn.Linear(d, inter, bias=False)
+        self.up_proj = nn.Linear(d, inter, bias=False)
+        self.down_proj = nn.Linear(inter, d, bias=False)
+
+    def forward(self, x):                                            # x: [sequences, tokens, d], causal per sequence
+        b, s, _ = x.shape
+        h = self.input_layernorm(x)
+        q = self.q_proj(h).view(b, s, self.heads, self.hd).transpose(1, 2)
+        k = self.k_proj(h).view(b, s, self.kv_heads, self.hd).transpose(1, 2)
+        v = self.v_proj(h).view(b, s, self.kv_heads, self.hd).transpose(1, 2)
+        rep = self.heads // self.kv_heads
+        a = torch.nn.functional.scaled_dot_product_attention(q, k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1),
+                                                             is_causal=True)
+        x = x + self.o_proj(a.transpose(1, 2).reshape(b, s, -1))
+        h = self.post_attention_layernorm(x)
+        return x + self.down_proj(torch.nn.functional.silu(self.gate_proj(h)) * self.up_proj(h))
+
+
+class _LlamaStack(nn.Module):
+
+    def __init__(self, layers=2, d=1024, heads=8, kv_heads=2, inter=2048):
+        super().__init__()
+        self.layers = nn.ModuleList(_LlamaLayer(d, heads, kv_heads, inter) for _ in range(layers))
+
+    def forward(self, x):
+        for layer in self.layers:
+            x = layer(x)
+        return x
+
+
+def test_llama_shaped_stack_packed_sequences_one_tenant_each(dev):
+    """Seven LoRA projections per layer (q/k/v and gate/up through the shared-input path), one tenant per packed
+    sequence: the mixed batch equals every tenant run alone through the reference-style adapter context, outputs
+    and every adapter gradient."""
+    dtype = torch.bfloat16
+    torch.manual_seed(0)
+    ml = MultiLora(max_loras=4, max_r=16)
+    model = ml.patch(_LlamaStack().to(dtype).to(dev), target_modules='all-linear')
+    cfgs = {'alice': LoraConfig(r=16, lora_alpha=32, target_modules='all-linear'),
+            'bob': LoraConfig(r=8, lora_alpha=16, target_modules=['q_proj', 'v_proj', 'down_proj']),
+            'carol': LoraConfig(r=4, lora_alpha=16, target_modules='all-linear', use_rslora=True)}
+    for n, c in cfgs.items():
+        ml.acquire_lora(n, c)
+    g = torch.Generator().manual_seed(1)
+    with torch.no_grad():
+        for n, p in model.named_parameters():
+            if '.lora_B.' in n:
+                p.copy_((torch.randn(p.shape, generator=g) * 0.02).to(dtype))
+    names = list(cfgs)
+    seqs, toks, d = 5, 96, 1024
+    seq_tenant = torch.tensor([0, 1, 2, 1, 0])
+    x = torch.randn(seqs, toks, d, generator=g).to(dtype).to(dev)
+    w = torch.randn(seqs, toks, d, generator=g).to(dtype).to(dev)
+    row_tenant = seq_tenant.repeat_interleave(toks).to(dev)
+    lora = {n: p for n, p in model.named_parameters() if 'lora_' in n}
+
+    def run(mixed, shared):
+        for p in model.parameters():
+            p.grad = None
+        if shared:
+            ml.share_inputs([[f'model.layers.{i}.{a}' for a in grp] for i in range(2)
+                             for grp in (('q_proj', 'k_proj', 'v_proj'), ('gate_proj', 'up_proj'))])
+        try:
+            if mixed:
+                with ml.batch(names, row_tenant):
+                    y = model(x)
+                (y * w).sum().backward()
+            else:
+                y = torch.empty_like(x)
+                for i, n in enumerate(names):                        # the reference's schedule: one tenant per pass
+                    mine = (seq_tenant == i).nonzero().flatten().to(dev)
+                    with ml.adapter(n):
+                        yi = model(x.index_select(0, mine))
+                    (yi * w.index_select(0, mine)).sum().backward()
+                    y[mine] = yi.detach()
+        finally:
+            ml.unshare_inputs()
+        return y.detach().clone(), {n: (p.grad.clone() if p.grad is not None else None) for n, p in lora.items()}
+
+    y_ref, g_ref = run(mixed=False, shared=False)
+    for shared in (False, True):
+        y, grads = run(mixed=True, shared=shared)
+        assert max_rel_err(y, y_ref) < 2e-2, shared
+        for n in lora:
+            if g_ref[n] is None or g_ref[n].abs().max() == 0:
+                assert grads[n] is None or grads[n].abs().max() == 0, n        # free slot, untargeted layer
+            else:
+                assert max_rel_err(grads[n], g_ref[n].double()) < 3e-2, (shared, n)
