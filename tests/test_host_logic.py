@@ -291,3 +291,31 @@ def test_share_inputs_bookkeeping_without_a_gpu():
         assert not hasattr(m.q_proj, '_tk_shared_inputs')
     with pytest.raises(ValueError):
         ml.share_inputs([['model.q_proj']])
+
+
+def test_checkpoint_stream_converters_slice_and_pad():
+    """save_lora_converter cuts to the tenant's rank and renames; load_lora_converter pads back to max_r."""
+    from torch import nn
+    torch.manual_seed(0)
+    ml = MultiLora(max_loras=2, max_r=8)
+    model = ml.patch(nn.Sequential(nn.Linear(12, 6)), target_modules='all-linear')
+    ml.acquire_lora('alice', LoraConfig(r=3, lora_alpha=6, target_modules='all-linear'))
+    slot = ml.find_lora_by_tenant('alice').adapter_name
+    other = 'lora_1' if slot == 'lora_0' else 'lora_0'
+    params = dict(model.named_parameters())
+    name_a = next(n for n in params if f'lora_A.{slot}.' in n)
+    name_b = next(n for n in params if f'lora_B.{slot}.' in n)
+    with torch.no_grad():
+        params[name_b].normal_()
+    key_a, a = ml.save_lora_converter(name_a, params[name_a], slot)
+    key_b, b = ml.save_lora_converter(name_b, params[name_b], slot)
+    assert slot not in key_a and a.shape == (3, 12) and b.shape == (6, 3)
+    assert torch.equal(a, params[name_a][:3]) and torch.equal(b, params[name_b][:, :3])
+    assert ml.save_lora_converter(name_a.replace(slot, other), params[name_a], slot) is None    # another slot's weight
+    assert ml.save_lora_converter('model.0.base_layer.weight', params[name_a], slot) is None    # not a LoRA weight
+    _, a8 = ml.load_lora_converter('x.lora_A.weight', a)
+    _, b8 = ml.load_lora_converter('x.lora_B.weight', b)
+    assert a8.shape == (8, 12) and b8.shape == (6, 8)
+    assert torch.equal(a8[:3], a) and a8[3:].abs().sum() == 0 and torch.equal(b8[:, :3], b) and b8[:, 3:].abs().sum() == 0
+    example = ml.get_trainable_parameters_example('alice')
+    assert 'lora_A.alice' in example and slot not in example

@@ -553,3 +553,44 @@ class MultiLora:
             if p.requires_grad:
                 trainable += n
         return trainable, total
+
+    def get_trainable_parameters_example(self, tenant_adapter_name):
+        """First and last five trainable parameter names of the tenant, slot name replaced by the tenant's
+        (reference :815-837)."""
+        slot = self.find_lora_by_tenant(tenant_adapter_name)
+        pattern = re.compile(rf'\.lora_\w+\.{re.escape(slot.adapter_name)}\.')
+        names = []
+        for name, p in self._named_parameters():
+            if p.requires_grad and pattern.search(name) and \
+                    self.match_target_modules(name, slot.tenant_config.target_modules):
+                for side in ('A', 'B'):
+                    name = name.replace(f'{side}.{slot.adapter_name}', f'{side}.{tenant_adapter_name}')
+                names.append(name)
+        return '\n'.join(names[:5] + ['...'] + names[-5:])
+
+    # ---- per-tensor converters of a checkpoint stream (one parameter at a time) ----------------------------------
+    def save_lora_converter(self, name, parameter, adapter_name):
+        """``(key, tensor)`` to write for one parameter of slot ``adapter_name``, or ``None`` to skip it: other
+        slots' weights are dropped, the slot's own are cut to the tenant's rank and lose the slot name
+        (reference :659-674)."""
+        slot = self.find_lora(adapter_name)
+        if re.search(r'\.lora_\w+\.\w+\.', name) and not re.search(rf'\.lora_\w+\.{re.escape(adapter_name)}\.', name):
+            return None
+        if not re.search(rf'\.lora_\w+\.({re.escape(adapter_name)}|weight)', name):
+            return None
+        tensor = self._slice_rank_tensor(name, parameter.detach() if hasattr(parameter, 'detach') else parameter,
+                                         slot.tenant_config.r)
+        return name.replace(f'.{slot.adapter_name}.', '.'), (tensor.clone() if tensor is not None else None)
+
+    def load_lora_converter(self, name, parameter, **kwargs):
+        """``(name, tensor)`` with a rank-``r`` LoRA tensor zero-padded to the slot's ``max_r`` (reference :576-608,
+        the linear branches: A grows by rows, B by columns)."""
+        if '_A' in name and parameter.shape[0] < self.max_r:
+            pad = torch.zeros(self.max_r - parameter.shape[0], parameter.shape[1], dtype=parameter.dtype,
+                              device=parameter.device)
+            parameter = torch.cat((parameter, pad), dim=0)
+        elif '_B' in name and parameter.shape[1] < self.max_r:
+            pad = torch.zeros(parameter.shape[0], self.max_r - parameter.shape[1], dtype=parameter.dtype,
+                              device=parameter.device)
+            parameter = torch.cat((parameter, pad), dim=1)
+        return name, parameter
