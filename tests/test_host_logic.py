@@ -319,3 +319,97 @@ def test_checkpoint_stream_converters_slice_and_pad():
     assert torch.equal(a8[:3], a) and a8[3:].abs().sum() == 0 and torch.equal(b8[:, :3], b) and b8[:, 3:].abs().sum() == 0
     example = ml.get_trainable_parameters_example('alice')
     assert 'lora_A.alice' in example and slot not in example
+
+
+# ---- packed expert parameters through MultiLora (the reference's tests/model/test_multi_lora_target_parameters.py) ----
+
+class _PackedExperts(torch.nn.Module):
+    """Two experts, hidden 4, intermediate 6; ``[E, out, in]`` storage, or ``[E, in, out]`` with is_transposed."""
+
+    def __init__(self, is_transposed=False):
+        super().__init__()
+        self.is_transposed = is_transposed
+        shape_gu, shape_d = ((2, 4, 12), (2, 6, 4)) if is_transposed else ((2, 12, 4), (2, 4, 6))
+        self.gate_up_proj = torch.nn.Parameter(torch.randn(*shape_gu))
+        self.down_proj = torch.nn.Parameter(torch.randn(*shape_d))
+
+
+def _expert_model(is_transposed=False):
+    from twinkle_amd import LoraTenant
+    model = torch.nn.Module()
+    model.mlp = torch.nn.Module()
+    model.mlp.experts = _PackedExperts(is_transposed)
+    model.active_adapter = 'lora_0'
+    model.set_adapter = lambda name: setattr(model, 'active_adapter', name)
+    model.disable_adapter_layers = lambda: None
+    model.enable_adapter_layers = lambda: None
+    targets = ['mlp.experts.gate_up_proj', 'mlp.experts.down_proj']
+    cfg = lambda r: LoraConfig(r=r, lora_alpha=2 * r, target_modules=[], target_parameters=targets)  # noqa: E731
+    ml = MultiLora(max_loras=2, max_r=4)
+    ml.module = model
+    ml.loras = [LoraTenant(index=i, adapter_name=f'lora_{i}', config=cfg(4)) for i in range(2)]
+    ml.patch_target_parameters(model, targets)
+    return ml, model, cfg
+
+
+@pytest.mark.parametrize('is_transposed', [False, True])
+def test_target_parameter_slots_keys_shapes_release_and_round_trip(is_transposed):
+    torch.manual_seed(0)
+    ml, model, cfg = _expert_model(is_transposed)
+    manager = ml.target_parameter_manager
+    gate_up, down = manager.wrappers
+    assert (gate_up.in_features, gate_up.out_features, down.in_features, down.out_features) == (4, 12, 6, 4)
+    ml.acquire_lora('adapter_a', cfg(2))
+    named = dict(manager.named_slot_parameters('adapter_a'))
+    assert {k: tuple(v.shape) for k, v in named.items()} == {
+        'mlp.experts.gate_up_proj.lora_A.lora_0.weight': (2, 4, 4),
+        'mlp.experts.gate_up_proj.lora_B.lora_0.weight': (2, 12, 4),
+        'mlp.experts.down_proj.lora_A.lora_0.weight': (2, 4, 6),
+        'mlp.experts.down_proj.lora_B.lora_0.weight': (2, 4, 4),
+    }
+    assert ml.get_target_parameter_trainable_parameters('adapter_a').keys() == named.keys()
+    # the first target parameter of a module is the innermost wrapper in PEFT's nesting (reference :321-330)
+    state = ml.get_state_dict('adapter_a')
+    assert {k: tuple(v.shape) for k, v in state.items()} == {
+        'base_model.model.mlp.experts.base_layer.lora_A.weight': (2, 2, 4),
+        'base_model.model.mlp.experts.base_layer.lora_B.weight': (2, 12, 2),
+        'base_model.model.mlp.experts.lora_A.weight': (2, 2, 6),
+        'base_model.model.mlp.experts.lora_B.weight': (2, 4, 2),
+    }
+    # the merged delta has the parameter's own layout
+    assert gate_up.get_delta_weight('lora_0', gate_up.out_in_layout).shape == model.mlp.experts.gate_up_proj.shape
+    # state-dict round trip into a fresh model (reference test :188-213, atol 1e-6)
+    with torch.no_grad():
+        for p in named.values():
+            p.uniform_(-0.1, 0.1)
+    state = ml.get_state_dict('adapter_a')
+    ml2, _, cfg2 = _expert_model(is_transposed)
+    ml2.acquire_lora('adapter_a', cfg2(2))
+    ml2.set_state_dict('adapter_a', state)
+    for w1, w2 in zip(manager.wrappers, ml2.target_parameter_manager.wrappers):
+        assert torch.allclose(w1.get_delta_weight('lora_0'), w2.get_delta_weight('lora_0'), atol=1e-6)
+    # adapter() tells every slot storage which slot is the active one, and restores it
+    with ml.adapter('adapter_a'):
+        assert gate_up.active_adapter == 'lora_0' and not gate_up.disable_adapters
+    assert gate_up.active_adapter is None
+    # release: A back to its first initialisation, B to zero (reference test :103-134)
+    ml3, _, cfg3 = _expert_model(is_transposed)
+    ml3.acquire_lora('adapter_a', cfg3(2))
+    first = {k: v.detach().clone() for k, v in ml3.target_parameter_manager.named_slot_parameters('adapter_a')
+             if '.lora_A.' in k}
+    with torch.no_grad():
+        for _, p in ml3.target_parameter_manager.named_slot_parameters('adapter_a'):
+            p.add_(1.0)
+    ml3.release_lora('adapter_a')
+    for w in ml3.target_parameter_manager.wrappers:
+        for k in ('lora_A', 'lora_B'):
+            p = getattr(w, k)['lora_0'].detach()
+            if k == 'lora_A':
+                assert torch.equal(p, first[f'{w.parameter_key}.lora_A.lora_0.weight'])
+            else:
+                assert torch.count_nonzero(p) == 0
+    with pytest.raises(ValueError):
+        manager.patch(model, ['mlp.experts.down_proj'])              # another target list after patching
+    with pytest.raises(ValueError):
+        ml.acquire_lora('adapter_b', LoraConfig(r=2, lora_alpha=4, target_modules=[], lora_dropout=0.1,
+                                                target_parameters=['mlp.experts.down_proj']))

@@ -14,6 +14,7 @@ delta is never materialised and many tenants share one pass.
 from __future__ import annotations
 
 import math
+from contextlib import contextmanager
 from typing import Dict, List, Optional, Sequence
 
 import torch
@@ -140,3 +141,137 @@ def expert_lora_delta(x_sorted: torch.Tensor, y_sorted: torch.Tensor, seg: Segme
     if groups is None:
         groups = slots.groups(tenant_slots)
     return multi_lora_delta(x_sorted, y_sorted, seg, groups, map_rows=False)
+
+
+class ExpertLoraManager:
+    """Finds packed expert parameters in a model, gives each its slot storage and keeps the tenant -> slot map.
+
+    Host-side mirror of the reference's ``TargetParameterLoraManager``
+    (src/twinkle/model/multi_lora_target_parameters.py:281-383): same method names, arguments and errors.  What
+    differs is how a slot takes effect: the reference merges ``W + B A * scaling`` into the parameter through a
+    parametrization while a tenant is active (:182-209); here the expert forward adds the low-rank term of every
+    (expert, tenant) segment with :func:`expert_lora_delta`, and :meth:`adapter` only records which tenant is the
+    active one for callers that run one tenant per pass.
+
+    The slot tensors have the reference's shapes for both storage layouts (``lora_A [E, max_r, in_features]``,
+    ``lora_B [E, out_features, max_r]`` with the reference's naming of the two trailing dimensions).  The segmented
+    kernels apply ``scale * (x A^T) B^T``, which is the reference's merged form when the expert computes
+    ``F.linear(x, W[e])`` on ``[E, out, in]`` storage (its expert forward, moe/expert_parallel.py:360-371);
+    for modules that compute ``x @ W[e]`` the merged delta of :meth:`ExpertLoraSlots.get_delta_weight` applies.
+    """
+
+    def __init__(self, max_loras: int, max_r: int):
+        self.max_loras = max_loras
+        self.max_r = max_r
+        self.wrappers: List[ExpertLoraSlots] = []
+        self.tenant_to_slot: Dict[str, str] = {}
+        self.tenant_configs: Dict[str, object] = {}
+        self._target_parameters: Optional[tuple] = None
+
+    def patch(self, model: nn.Module, target_parameters) -> None:
+        """Attach slot storage to every parameter named (or suffixed ``.name``) in ``target_parameters``
+        (reference :291-319).  3-D parameters are ``[E, out, in]`` unless the owning module says
+        ``is_transposed`` (then ``[E, in, out]``), 2-D ones ``[out, in]`` with one expert (:47-52)."""
+        target_parameters = tuple(target_parameters)
+        if not target_parameters:
+            return
+        if self._target_parameters is not None:
+            if self._target_parameters != target_parameters:
+                raise ValueError(
+                    f'target_parameters already patched as {self._target_parameters}, got {target_parameters}')
+            return
+        found = []
+        for module_name, module in model.named_modules():
+            for param_name, parameter in module.named_parameters(recurse=False):
+                key = f'{module_name}.{param_name}' if module_name else param_name
+                if key in target_parameters or any(key.endswith(f'.{t}') for t in target_parameters):
+                    if parameter.ndim not in (2, 3):
+                        raise ValueError(
+                            f'target parameter {key} has {parameter.ndim} dimensions; only 2D and 3D are supported')
+                    found.append((module_name, module, param_name, parameter))
+        if not found:
+            raise ValueError(f'target_parameters={target_parameters} were set but no parameter was matched')
+        per_module: Dict[str, List[ExpertLoraSlots]] = {}
+        for module_name, module, param_name, parameter in found:
+            if parameter.ndim == 3:
+                out_in = not getattr(module, 'is_transposed', False)
+                experts = parameter.shape[0]
+                fin, fout = (parameter.shape[-1], parameter.shape[-2]) if out_in else (parameter.shape[-2],
+                                                                                      parameter.shape[-1])
+            else:
+                out_in, experts = True, 1
+                fout, fin = parameter.shape
+            device = 'cpu' if parameter.device.type == 'meta' else parameter.device
+            slots = ExpertLoraSlots(experts, fin, fout, self.max_loras, self.max_r, dtype=parameter.dtype, device=device)
+            slots.parameter_key = f'{module_name}.{param_name}' if module_name else param_name
+            slots.out_in_layout = out_in
+            slots.active_adapter, slots.disable_adapters = None, False
+            module.add_module(f'_twinkle_lora_{param_name}', slots)
+            self.wrappers.append(slots)
+            per_module.setdefault(module_name, []).append(slots)
+        # PEFT nests one wrapper per target parameter of a module: the first one found is the innermost (:321-330)
+        for module_name, group in per_module.items():
+            prefix = f'base_model.model.{module_name}' if module_name else 'base_model.model'
+            for index, slots in enumerate(group):
+                nested = '.'.join(['base_layer'] * (len(group) - index - 1))
+                slots.peft_key_prefix = f'{prefix}.{nested}' if nested else prefix
+        self._target_parameters = target_parameters
+
+    def acquire(self, tenant_adapter_name: str, slot_name: str, config) -> None:
+        if tenant_adapter_name in self.tenant_to_slot:
+            raise ValueError(f'Lora {tenant_adapter_name} already exists')
+        if getattr(config, 'target_parameters', None) and not self.wrappers:
+            raise ValueError('target_parameters LoRA slots must be patched before acquire')
+        self.tenant_to_slot[tenant_adapter_name] = slot_name
+        self.tenant_configs[tenant_adapter_name] = config
+        for slots in self.wrappers:
+            slots.configure_slot(slot_name, config)
+
+    def release(self, tenant_adapter_name: str) -> None:
+        slot_name = self.tenant_to_slot.pop(tenant_adapter_name, None)
+        self.tenant_configs.pop(tenant_adapter_name, None)
+        if slot_name is None:
+            return
+        for slots in self.wrappers:
+            slots.reset_slot(slot_name)
+
+    @contextmanager
+    def adapter(self, tenant_adapter_name: str, disable_lora: bool = False):
+        """One tenant per pass: every slot storage learns which slot is active (``None`` for unknown tenants)."""
+        slot_name = self.tenant_to_slot.get(tenant_adapter_name)
+        previous = [(s.active_adapter, s.disable_adapters) for s in self.wrappers]
+        for s in self.wrappers:
+            s.active_adapter, s.disable_adapters = slot_name, disable_lora
+        try:
+            yield
+        finally:
+            for s, (a, d) in zip(self.wrappers, previous):
+                s.active_adapter, s.disable_adapters = a, d
+
+    def slots_of(self, tenant_adapter_names: Sequence[str]) -> List[str]:
+        """Slot names of the tenants of a mixed batch, in the order their ids appear in the group keys."""
+        return [self.tenant_to_slot[t] for t in tenant_adapter_names]
+
+    def parameters_for_tenant(self, tenant_adapter_name: str) -> List[nn.Parameter]:
+        return [p for _, p in self.named_slot_parameters(tenant_adapter_name)]
+
+    def named_slot_parameters(self, tenant_adapter_name: str):
+        slot_name = self.tenant_to_slot[tenant_adapter_name]
+        for slots in self.wrappers:
+            if slot_name in slots.lora_A:
+                yield f'{slots.parameter_key}.lora_A.{slot_name}.weight', slots.lora_A[slot_name]
+                yield f'{slots.parameter_key}.lora_B.{slot_name}.weight', slots.lora_B[slot_name]
+
+    def get_state_dict(self, tenant_adapter_name: str) -> Dict[str, torch.Tensor]:
+        slot_name = self.tenant_to_slot[tenant_adapter_name]
+        state = {}
+        for slots in self.wrappers:
+            state.update(slots.get_state_dict(slot_name))
+        return state
+
+    def set_state_dict(self, tenant_adapter_name: str, state_dict: Dict[str, torch.Tensor]) -> set:
+        slot_name = self.tenant_to_slot[tenant_adapter_name]
+        consumed = set()
+        for slots in self.wrappers:
+            consumed.update(slots.set_state_dict(slot_name, state_dict))
+        return consumed

@@ -21,6 +21,7 @@ from typing import Any, Dict, List, Optional, Sequence, Tuple, Union
 
 import torch
 
+from .expert_lora import ExpertLoraManager
 from .lora_layer import LoraConfig, LoraLinear, LoraModel, inject_adapter
 from .ops import AdapterGroups, multi_lora_delta, multi_lora_linear, multi_lora_linear_shared
 from .segments import SegmentTable, build_segments
@@ -75,6 +76,19 @@ class MultiLora:
         self._layer_groups: Dict[int, tuple] = {}
         self._batch_table: Optional[SegmentTable] = None
         self._uniform_tables: Dict[tuple, SegmentTable] = {}
+        # packed expert parameters (reference :40): slot storage per target parameter, same tenant -> slot map
+        self.target_parameter_manager = ExpertLoraManager(max_loras=max_loras, max_r=max_r)
+
+    def patch_target_parameters(self, module, target_parameters):
+        """Slot storage for packed expert parameters such as ``gate_up_proj`` / ``down_proj`` (reference :151-152)."""
+        self.target_parameter_manager.patch(module, target_parameters)
+
+    def get_target_parameter_trainable_parameters(self, tenant_adapter_name):
+        return dict(self.target_parameter_manager.named_slot_parameters(tenant_adapter_name))
+
+    @staticmethod
+    def _is_target_parameter_lora_name(name: str) -> bool:
+        return '._twinkle_lora_' in name
 
     # ------------------------------------------------------------------ slots
     def _get_available_lora(self) -> Optional[LoraTenant]:
@@ -109,6 +123,9 @@ class MultiLora:
             raise RuntimeError(f'Too big rank for lora: {config.r}')
         slot.tenant_config = config
         slot.tenant_adapter_name = tenant_adapter_name
+        if getattr(config, 'target_parameters', None):
+            self.target_parameter_manager.acquire(tenant_adapter_name=tenant_adapter_name, slot_name=slot.adapter_name,
+                                                  config=config)
         self._version += 1
         return slot.adapter_name
 
@@ -121,6 +138,7 @@ class MultiLora:
         slot.tenant_config = None
         slot.tenant_adapter_name = None
         self._load_initial_weights(slot.adapter_name)
+        self.target_parameter_manager.release(tenant_adapter_name)
         self._version += 1
         return None
 
@@ -177,11 +195,12 @@ class MultiLora:
         """One tenant for every row of the calls inside (reference :154-163)."""
         self.activate_adapter(tenant_adapter_name)
         try:
-            if disable_lora:
-                with self._disable_lora_context(tenant_adapter_name):
+            with self.target_parameter_manager.adapter(tenant_adapter_name, disable_lora=disable_lora):
+                if disable_lora:
+                    with self._disable_lora_context(tenant_adapter_name):
+                        yield self.find_lora_by_tenant(tenant_adapter_name).adapter_name
+                else:
                     yield self.find_lora_by_tenant(tenant_adapter_name).adapter_name
-            else:
-                yield self.find_lora_by_tenant(tenant_adapter_name).adapter_name
         finally:
             self._uniform_tables.clear()
 
@@ -476,10 +495,14 @@ class MultiLora:
         pattern = re.compile(rf'\.lora_\w+\.{re.escape(slot.adapter_name)}\.')
         with torch.no_grad():
             for name, p in self._named_parameters():
+                if self._is_target_parameter_lora_name(name):
+                    continue
                 if pattern.search(name) and self.match_target_modules(name, slot.tenant_config.target_modules):
                     key = name.replace(f'.{slot.adapter_name}.', '.')
                     src = state_dict[key].to(dtype=p.dtype, device=p.device)
                     self._copy_rank_tensor(name, p.data, src)
+        if tenant_adapter_name in self.target_parameter_manager.tenant_to_slot:
+            self.target_parameter_manager.set_state_dict(tenant_adapter_name, state_dict)
 
     def get_state_dict(self, tenant_adapter_name):
         """Tenant's live ``[:r]`` blocks under slot-free names (reference :701-729)."""
@@ -487,9 +510,17 @@ class MultiLora:
         pattern = re.compile(rf'\.lora_\w+\.{re.escape(slot.adapter_name)}\.')
         out = {}
         for name, p in self._named_parameters():
+            if self._is_target_parameter_lora_name(name):
+                continue
             if pattern.search(name) and self.match_target_modules(name, slot.tenant_config.target_modules):
                 out[name.replace(f'.{slot.adapter_name}.', '.')] = self._slice_rank_tensor(name, p.detach(),
                                                                                            slot.tenant_config.r)
+        if tenant_adapter_name in self.target_parameter_manager.tenant_to_slot:
+            expert_state = self.target_parameter_manager.get_state_dict(tenant_adapter_name)
+            overlap = out.keys() & expert_state.keys()
+            if overlap:
+                raise ValueError(f'Duplicate LoRA state keys: {sorted(overlap)[:5]}')
+            out.update(expert_state)
         return out
 
     # ---- adapter checkpoints in PEFT's on-disk format -----------------------------------------------------------
