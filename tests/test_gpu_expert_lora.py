@@ -104,3 +104,80 @@ def test_config4_shapes_bf16(dev):
     row_w = weights.bfloat16().t().reshape(-1)[perm]
     want = oracle.unpermute_rows((out.cpu().double() * row_w.double()[:, None]).bfloat16().double(), None, perm % t, t)
     assert max_rel_err(final, want) < 2e-2
+
+
+def test_moe_block_with_expert_lora_equals_merged_weights_per_tenant(dev):
+    """Router outputs -> permute -> packed experts (gate_up, SiLU gate, down) with per-(expert, tenant) LoRA ->
+    weighted unpermute, against the reference's form in float64: merged weights W + B A * scaling of every token's
+    own tenant (multi_lora_target_parameters.py:158-209), the per-expert loop, zero-init + index_add."""
+    from twinkle_amd import LoraTenant, MultiLora
+    from twinkle_amd.expert_lora import moe_experts_block
+    torch.manual_seed(0)
+    e, hid, inter, t, k = 6, 128, 256, 300, 2
+
+    class Experts(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.gate_up_proj = torch.nn.Parameter(torch.randn(e, 2 * inter, hid) * 0.05, requires_grad=False)
+            self.down_proj = torch.nn.Parameter(torch.randn(e, hid, inter) * 0.05, requires_grad=False)
+            self.act_fn = torch.nn.functional.silu
+
+    model = torch.nn.Module()
+    model.experts = Experts().to(dev)
+    model.set_adapter = lambda name: None
+    model.disable_adapter_layers = model.enable_adapter_layers = lambda: None
+    targets = ['experts.gate_up_proj', 'experts.down_proj']
+    ml = MultiLora(max_loras=3, max_r=8)
+    ml.module = model
+    ml.loras = [LoraTenant(index=i, adapter_name=f'lora_{i}', config=None) for i in range(3)]
+    ml.patch_target_parameters(model, targets)
+    tenants = ['alice', 'bob']
+    for name, r in zip(tenants, (8, 4)):
+        ml.acquire_lora(name, LoraConfig(r=r, lora_alpha=2 * r, target_modules=[], target_parameters=targets))
+    manager = ml.target_parameter_manager
+    gu_slots, down_slots = manager.wrappers
+    with torch.no_grad():
+        for name in tenants:
+            for key, p in manager.named_slot_parameters(name):
+                if '.lora_B.' in key:
+                    p.normal_(0, 0.05)
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(t, hid, generator=g)
+    logits = torch.randn(t, e, generator=g)
+    weights, sel = torch.topk(torch.softmax(logits, -1), k)
+    tenant = torch.randint(0, 2, (t,), generator=g)
+    xd = x.to(dev).requires_grad_(True)
+    slots = manager.slots_of(tenants)
+    y = moe_experts_block(xd, sel.to(dev), weights.to(dev), tenant.to(dev), model.experts, slots, gu_slots, down_slots)
+    y.pow(2).sum().backward()
+
+    # float64 restatement with merged weights, token by token group
+    x64 = x.double().requires_grad_(True)
+    leaf = {}
+    for s in slots:
+        for w in (gu_slots, down_slots):
+            leaf[(id(w), s, 'a')] = w.lora_A[s].detach().double().cpu().requires_grad_(True)
+            leaf[(id(w), s, 'b')] = w.lora_B[s].detach().double().cpu().requires_grad_(True)
+    out = torch.zeros(t, hid, dtype=torch.float64)
+    for kk in range(k):
+        for ex in range(e):
+            for ti, s in enumerate(slots):
+                idx = ((sel[:, kk] == ex) & (tenant == ti)).nonzero().flatten()
+                if idx.numel() == 0:
+                    continue
+                merged = []
+                for w, base in ((gu_slots, model.experts.gate_up_proj), (down_slots, model.experts.down_proj)):
+                    dw = oracle.expert_delta_weight(leaf[(id(w), s, 'a')], leaf[(id(w), s, 'b')], w.r[s], w.scaling[s])
+                    merged.append(base.detach().double().cpu()[ex] + dw[ex])
+                h = x64[idx] @ merged[0].t()
+                gate, up = h.chunk(2, dim=-1)
+                o = (torch.nn.functional.silu(gate) * up) @ merged[1].t()
+                out = out.index_add(0, idx, o * weights[idx, kk].double()[:, None])
+    out.pow(2).sum().backward()
+    assert max_rel_err(y, out) < 2e-5
+    assert max_rel_err(xd.grad, x64.grad) < 1e-4
+    for s in slots:
+        for w in (gu_slots, down_slots):
+            assert max_rel_err(w.lora_A[s].grad, leaf[(id(w), s, 'a')].grad) < 2e-4
+            assert max_rel_err(w.lora_B[s].grad, leaf[(id(w), s, 'b')].grad) < 2e-4
+    assert gu_slots.lora_A['lora_2'].grad is None                      # the free slot

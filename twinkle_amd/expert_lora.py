@@ -275,3 +275,66 @@ class ExpertLoraManager:
         for slots in self.wrappers:
             consumed.update(slots.set_state_dict(slot_name, state_dict))
         return consumed
+
+
+def experts_forward(experts_mod: nn.Module, rows: torch.Tensor, seg: SegmentTable, tenant_slots: Sequence[str],
+                    gate_up_slots: Optional[ExpertLoraSlots] = None,
+                    down_slots: Optional[ExpertLoraSlots] = None) -> torch.Tensor:
+    """Packed experts on rows in (expert, tenant) segment order, every tenant's LoRA terms included.
+
+    The per-expert loop of the reference's expert forward (moe/expert_parallel.py:333-378: ``F.linear`` with
+    ``gate_up_proj[e]``, gate activation, ``F.linear`` with ``down_proj[e]`` on contiguous chunks), with two
+    differences: the chunk boundaries come from the segment table in one device-to-host copy (the reference
+    synchronises once per expert, :347-349), and the LoRA terms are added per (expert, tenant) segment by the
+    segmented kernels instead of being merged into the weights.  ``seg`` was built from keys
+    ``expert * len(tenant_slots) + tenant`` with ``want_offsets=True``; ``experts_mod`` holds
+    ``gate_up_proj [E, 2 I, H]`` and ``down_proj [E, H, I]`` and either ``_apply_gate`` or ``act_fn``.
+    """
+    if rows.shape[0] == 0:
+        return rows                                                   # keeps the autograd edge (reference :340-344)
+    nt = len(tenant_slots)
+    gate_up, down = experts_mod.gate_up_proj, experts_mod.down_proj
+    experts = gate_up.shape[0]
+    if seg.num_groups != experts * nt or seg.offsets is None:
+        raise ValueError('the segment table must hold offsets for expert * num_tenants + tenant keys')
+    bounds = seg.offsets[::nt].tolist()                               # first sorted position of every expert
+    input_dtype = rows.dtype
+    x = rows if rows.dtype == gate_up.dtype else rows.to(gate_up.dtype)
+
+    def per_expert(inp, weight):
+        chunks = [torch.nn.functional.linear(inp[bounds[e]:bounds[e + 1]], weight[e]) for e in range(experts)
+                  if bounds[e + 1] > bounds[e]]
+        return torch.cat(chunks, dim=0)
+
+    gate_up_out = per_expert(x, gate_up)
+    if gate_up_slots is not None:
+        gate_up_out = expert_lora_delta(x, gate_up_out, seg, gate_up_slots, tenant_slots)
+    if hasattr(experts_mod, '_apply_gate'):
+        hidden = experts_mod._apply_gate(gate_up_out)
+    else:
+        gate, up = gate_up_out.chunk(2, dim=-1)
+        hidden = experts_mod.act_fn(gate) * up
+    hidden = hidden.contiguous()
+    out = per_expert(hidden, down)
+    if down_slots is not None:
+        out = expert_lora_delta(hidden, out, seg, down_slots, tenant_slots)
+    return out if out.dtype == input_dtype else out.to(input_dtype)
+
+
+def moe_experts_block(hidden_states: torch.Tensor, selected_experts: torch.Tensor, routing_weights: torch.Tensor,
+                      tenant: Optional[torch.Tensor], experts_mod: nn.Module, tenant_slots: Sequence[str],
+                      gate_up_slots: Optional[ExpertLoraSlots] = None,
+                      down_slots: Optional[ExpertLoraSlots] = None) -> torch.Tensor:
+    """Routed tokens through the packed experts and back: segment build, permute, :func:`experts_forward`,
+    weighted unpermute (the single-rank part of the reference's patched block forward,
+    moe/expert_parallel.py:253-255 and moe/ep_utils.py:99-149, :280-287).  ``tenant [T]`` gives every token's
+    index into ``tenant_slots`` (``None``: one tenant)."""
+    from .segments import build_segments, flat_keys_from_topk, permute, unpermute
+    nt = len(tenant_slots)
+    experts = experts_mod.gate_up_proj.shape[0]
+    tokens = hidden_states.shape[0]
+    keys = flat_keys_from_topk(selected_experts, tenant if nt > 1 else None, nt)
+    seg = build_segments(keys, experts * nt, num_tokens=tokens)
+    rows, _ = permute(hidden_states, seg)
+    out_rows = experts_forward(experts_mod, rows, seg, tenant_slots, gate_up_slots, down_slots)
+    return unpermute(out_rows, routing_weights.to(hidden_states.dtype), seg)
