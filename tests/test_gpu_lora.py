@@ -356,3 +356,30 @@ def test_chunks_larger_than_512_rows(dev, dtype, t, k, m, max_r, ranks):
     ids[t // 7: t // 7 + 50] = n - 1          # one group far smaller than a chunk
     ids = ids[torch.randperm(t, generator=torch.Generator().manual_seed(1))]
     _run(dev, dtype, x, base, dy, a, b, ids, ranks, scales)
+
+
+def _random_case(seed):
+    g = torch.Generator().manual_seed(1000 + seed)
+    pick = lambda xs: xs[int(torch.randint(0, len(xs), (1,), generator=g))]  # noqa: E731
+    t = pick([1, 7, 32, 33, 100, 257, 1000, 2500])
+    k = pick([64, 128, 192, 256, 512, 1024, 1088])
+    m = pick([128, 256, 384, 512, 640, 1024, 1536])
+    max_r = pick([4, 8, 16, 24, 32, 48, 64])
+    n = pick([1, 2, 5, 17, 40])
+    ranks = [int(torch.randint(0, max_r + 1, (1,), generator=g)) for _ in range(n)]
+    ranks[int(torch.randint(0, n, (1,), generator=g))] = max_r            # at least one adapter at the slot's rank
+    # ids over a random subset of the adapters, so that some stay empty
+    live = torch.randperm(n, generator=g)[:max(1, int(torch.randint(1, n + 1, (1,), generator=g)))]
+    ids = live[torch.randint(0, live.numel(), (t,), generator=g)]
+    return t, k, m, n, max_r, ranks, ids
+
+
+@pytest.mark.parametrize('seed', range(36))
+def test_random_shapes_ranks_and_id_distributions(dev, seed):
+    """Seeded draws over the kernels' boundary sizes (one row, one tile plus one, widths at and off the MFMA
+    kernels' multiples, ranks 0 .. 64, many empty adapters), bf16 and fp32 alternating."""
+    t, k, m, n, max_r, ranks, ids = _random_case(seed)
+    print(f'case {seed}: t={t} k={k} m={m} n={n} max_r={max_r} ranks={ranks}', flush=True)
+    dtype = torch.bfloat16 if seed % 3 else torch.float32
+    x, base, dy, a, b, _, _, scales = _problem(t, k, m, n, max_r, ranks, seed=seed)
+    _run(dev, dtype, x, base, dy, a, b, ids, ranks, scales)

@@ -247,3 +247,18 @@ def test_shared_calls_replay_from_a_hip_graph(dev):
         torch.cuda.synchronize()
         for got, ref in zip((*ys, dx, *gas, *gbs), want):
             assert torch.equal(got, ref)
+
+
+@pytest.mark.parametrize('seed', range(12))
+def test_shared_random_projection_sets(dev, seed):
+    """Seeded draws: 2..4 projections, widths on and off the single-pass backward's multiples, ranks 0..16, few rows."""
+    g = torch.Generator().manual_seed(500 + seed)
+    pick = lambda xs: xs[int(torch.randint(0, len(xs), (1,), generator=g))]  # noqa: E731
+    p = pick([2, 3, 4])
+    t, k, n = pick([1, 33, 500, 2100]), pick([1024, 2048]), pick([1, 3, 9])
+    outs = tuple(pick([256, 512, 1024, 1536]) for _ in range(p))
+    ranks = [tuple(int(torch.randint(0, 17, (1,), generator=g)) for _ in range(n)) for _ in range(p)]
+    ranks = [tuple(16 if i == 0 else r for i, r in enumerate(rs)) for rs in ranks]    # keep every projection live
+    print(f'case {seed}: t={t} k={k} outs={outs} n={n} ranks={ranks}', flush=True)
+    # forward through the shared kernels always; backward too when every width is a multiple of 512
+    _compare(dev, torch.bfloat16, t, k, outs, n, 16, ranks, seed=seed)
