@@ -156,7 +156,7 @@ def optimizer_step_bench(dev, steps=10):
                     'per tenant grad.div_, clip_grad_norm_, fused AdamW (bf16 moments), zero_grad'}
 
 
-def shared_qkv_bench(dev, steps=20):
+def shared_qkv_bench(dev, steps=20, calibrate_copy=False):
     """q / k / v of one attention block (4096 -> 4096, 1024, 1024; config 2's tokens, adapters and ids):
     one shared call against one call per projection, forward + backward, segment table built once."""
     import torch
@@ -203,6 +203,10 @@ def shared_qkv_bench(dev, steps=20):
             fn()
         torch.cuda.synchronize()
         res[name] = (time.perf_counter() - t0) * 1e3 / steps
+    if calibrate_copy:
+        for _ in range(5):
+            dx.copy_(x)                                # a known-size kernel for rocprofv3 --pmc readings
+        torch.cuda.synchronize()
     elt = 2
     per_proj = sum(elt * T * (4 * m + 3 * K) for m in outs)            # y rw, dy r | x r (fwd, dA), dx rw
     joint = sum(elt * T * 4 * m for m in outs) + elt * T * 4 * K       # x r twice, dx rw once
@@ -254,7 +258,7 @@ def main():
         print(json.dumps({'optimizer_step': optimizer_step_bench(dev)}))
         return
     if args.shared_qkv:
-        print(json.dumps({'shared_qkv': shared_qkv_bench(dev)}))
+        print(json.dumps({'shared_qkv': shared_qkv_bench(dev, calibrate_copy=args.calibrate_copy)}))
         return
     if args.workload == 'cfg2' and args.tokens:
         w = workloads.config2_qproj(tokens=args.tokens)
