@@ -217,6 +217,79 @@ def shared_qkv_bench(dev, steps=20, calibrate_copy=False):
     return res
 
 
+def cfg5_layer_bench(dev, steps=5):
+    """The seven projections of one Llama-3-8B-shaped layer (4096 hidden, 1024 k/v, 14336 intermediate) with LoRA
+    rank 64 on all of them, 8 tenants, one per packed 4096-token sequence (T = 32768), bf16: forward + backward
+    of the projection chain with the adapters off, on (one mixed batch), and on with q/k/v and gate/up declared
+    as shared inputs.  The attention core has no adapter and is left out (q stands in for its output)."""
+    import torch
+    from torch import nn
+    from twinkle_amd import LoraConfig, MultiLora
+
+    class Projections(nn.Module):
+        def __init__(self, d=4096, kv=1024, inter=14336):
+            super().__init__()
+            self.q_proj, self.k_proj, self.v_proj = nn.Linear(d, d, bias=False), nn.Linear(d, kv, bias=False), \
+                nn.Linear(d, kv, bias=False)
+            self.o_proj = nn.Linear(d, d, bias=False)
+            self.gate_proj, self.up_proj = nn.Linear(d, inter, bias=False), nn.Linear(d, inter, bias=False)
+            self.down_proj = nn.Linear(inter, d, bias=False)
+
+        def forward(self, x):
+            q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
+            h = x + self.o_proj(q) + (k.sum(-1, keepdim=True) + v.sum(-1, keepdim=True)) * 1e-3
+            return h + self.down_proj(nn.functional.silu(self.gate_proj(h)) * self.up_proj(h))
+
+    dt, seqs, toks, d = torch.bfloat16, 8, 4096, 4096
+    torch.manual_seed(7)
+    ml = MultiLora(max_loras=8, max_r=64, max_length=seqs * toks)
+    model = ml.patch(Projections().to(dt).to(dev), target_modules='all-linear')
+    for n, p in model.named_parameters():
+        if 'lora_' not in n:
+            p.requires_grad_(False)
+        elif '.lora_B.' in n:
+            with torch.no_grad():
+                p.normal_(0, 0.02)
+    names = [f'tenant_{i}' for i in range(8)]
+    for n in names:
+        ml.acquire_lora(n, LoraConfig(r=64, lora_alpha=128, target_modules='all-linear'))
+    x = torch.randn(seqs * toks, d, device=dev, dtype=dt).requires_grad_(True)
+    dy = torch.randn(seqs * toks, d, device=dev, dtype=dt)
+    row_tenant = torch.repeat_interleave(torch.arange(8, device=dev), toks)
+
+    def run(mode):
+        if mode == 'base':
+            with ml.adapter(names[0], disable_lora=True):
+                y = model(x)
+        else:
+            with ml.batch(names, row_tenant):
+                y = model(x)
+        y.backward(dy)
+        x.grad = None
+        for p in model.parameters():
+            p.grad = None
+
+    res = {}
+    for mode in ('base', 'lora', 'lora_shared_inputs'):
+        if mode == 'lora_shared_inputs':
+            ml.share_inputs([['model.q_proj', 'model.k_proj', 'model.v_proj'], ['model.gate_proj', 'model.up_proj']])
+        for _ in range(2):
+            run(mode)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            run(mode)
+        torch.cuda.synchronize()
+        res[mode + '_ms'] = (time.perf_counter() - t0) * 1e3 / steps
+    ml.unshare_inputs()
+    T = seqs * toks
+    res.update({'tokens': T, 'lora_share_of_step': 1 - res['base_ms'] / res['lora_ms'],
+                'tokens_per_s_with_lora': T / (res['lora_ms'] * 1e-3),
+                'workload': 'Llama-3-8B-shaped projections (q, k, v, o, gate, up, down), rank 64, 8 tenants x 4096 packed '
+                            'tokens, fwd + bwd; base weights frozen (dX only), attention core omitted'})
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -237,6 +310,8 @@ def main():
                     help='run only the multi-tenant optimizer micro-benchmark and print its JSON (for profiling)')
     ap.add_argument('--shared-qkv', action='store_true',
                     help='run only the q / k / v micro-benchmark (one shared call against one call per projection)')
+    ap.add_argument('--layer-cfg5', action='store_true',
+                    help='run only the one-layer measurement of BASELINE config 5 (seven projections, rank 64)')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run five plain 128 MiB device copies (a known-size kernel to scale rocprofv3 --pmc '
                          'FETCH_SIZE / WRITE_SIZE readings by)')
@@ -256,6 +331,9 @@ def main():
     dev = torch.device('cuda:0')
     if args.optimizer_only:
         print(json.dumps({'optimizer_step': optimizer_step_bench(dev)}))
+        return
+    if args.layer_cfg5:
+        print(json.dumps({'cfg5_layer': cfg5_layer_bench(dev)}))
         return
     if args.shared_qkv:
         print(json.dumps({'shared_qkv': shared_qkv_bench(dev, calibrate_copy=args.calibrate_copy)}))
