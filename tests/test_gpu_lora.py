@@ -383,3 +383,46 @@ def test_random_shapes_ranks_and_id_distributions(dev, seed):
     dtype = torch.bfloat16 if seed % 3 else torch.float32
     x, base, dy, a, b, _, _, scales = _problem(t, k, m, n, max_r, ranks, seed=seed)
     _run(dev, dtype, x, base, dy, a, b, ids, ranks, scales)
+
+
+_ENV_CHILD = r'''
+import sys, torch
+sys.path.insert(0, sys.argv[1]); sys.path.insert(0, sys.argv[1] + "/tests")
+import oracle
+from twinkle_amd import AdapterGroups, build_segments, multi_lora_delta
+torch.manual_seed(0)
+t, k, m, n, max_r, ranks = 700, 256, 512, 4, 32, [32, 9, 0, 17]
+g = torch.Generator().manual_seed(5)
+bf = lambda v: v.bfloat16()
+x, base, dy = bf(torch.randn(t, k, generator=g)), bf(torch.randn(t, m, generator=g)), bf(torch.randn(t, m, generator=g))
+a = [bf((torch.rand(max_r, k, generator=g) * 2 - 1) / k ** 0.5) for _ in range(n)]
+b = [bf(torch.randn(m, max_r, generator=g) * 0.05) for _ in range(n)]
+ids = torch.randint(0, n, (t,), generator=g)
+scales = [2.0, 0.5, 1.0, 2.0]
+dev = torch.device("cuda:0")
+xd = x.to(dev).requires_grad_(True)
+ad = [v.to(dev).requires_grad_(True) for v in a]; bd = [v.to(dev).requires_grad_(True) for v in b]
+seg = build_segments(ids.to(torch.int32).to(dev), n)
+y = multi_lora_delta(xd, base.to(dev) * 1.0, seg, AdapterGroups(ad, bd, ranks, scales))
+y.backward(dy.to(dev))
+yo, dxo, dao, dbo = oracle.multi_lora_linear_grads(x.double(), base.double(), ids, [v.double() for v in a],
+                                                    [v.double() for v in b], ranks, scales, dy.double())
+err = lambda got, ref: float((got.double().cpu() - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+worst = max([err(y, yo), err(xd.grad, dxo)] + [err(ad[i].grad, dao[i]) for i in (0, 1, 3)] +
+            [err(bd[i].grad, dbo[i]) for i in (0, 1, 3)])
+print("worst", worst)
+sys.exit(0 if worst < 2e-2 else 1)
+'''
+
+
+@pytest.mark.parametrize('env', [{'TK_FORCE_GENERIC': '1'}, {'TK_BWD_STREAMS': '0'}])
+def test_environment_switches_in_a_child_process(dev, env):
+    """TK_FORCE_GENERIC=1 (every launch on the shape-agnostic kernels) and TK_BWD_STREAMS=0 (backward on the
+    caller's stream only) are read once per process, so each runs in a child: same bar against the oracle."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, '-c', _ENV_CHILD, root], env={**os.environ, **env}, capture_output=True,
+                         text=True, timeout=300)
+    assert out.returncode == 0, out.stdout[-2000:] + out.stderr[-2000:]
