@@ -306,6 +306,8 @@ def main():
                          'of rank 64, one per packed 4096-token sequence) for additional measurements')
     ap.add_argument('--tokens', type=int, default=0,
                     help='cfg2 with another number of tokens (a scaling measurement, not the headline configuration)')
+    ap.add_argument('--rank', type=int, default=0,
+                    help='cfg2 with another adapter rank (alpha = 2 x rank; a scaling measurement like --tokens)')
     ap.add_argument('--optimizer-only', action='store_true',
                     help='run only the multi-tenant optimizer micro-benchmark and print its JSON (for profiling)')
     ap.add_argument('--shared-qkv', action='store_true',
@@ -338,9 +340,10 @@ def main():
     if args.shared_qkv:
         print(json.dumps({'shared_qkv': shared_qkv_bench(dev, calibrate_copy=args.calibrate_copy)}))
         return
-    if args.workload == 'cfg2' and args.tokens:
-        w = workloads.config2_qproj(tokens=args.tokens)
-        w.name = f'cfg2 shape with T={args.tokens}'
+    if args.workload == 'cfg2' and (args.tokens or args.rank):
+        w = workloads.config2_qproj(tokens=args.tokens or 16384, r=args.rank or 16)
+        w.name = f'cfg2 shape with T={w.tokens}, rank {max(w.ranks)}'
+        args.tokens = w.tokens
     elif args.workload == 'cfg2':
         w = workloads.config2_qproj()
     elif args.workload == 'cfg5_q':
