@@ -376,3 +376,66 @@ def test_llama_shaped_stack_packed_sequences_one_tenant_each(dev):
                 assert grads[n] is None or grads[n].abs().max() == 0, n        # free slot, untargeted layer
             else:
                 assert max_rel_err(grads[n], g_ref[n].double()) < 3e-2, (shared, n)
+
+
+def test_fp32_adapters_computed_in_bf16_on_request(dev):
+    """lora_compute_dtype=bfloat16: fp32 adapter parameters under a bf16 base run through the bf16 kernels (copies
+    refreshed at every forward), gradients arrive in fp32 on the fp32 parameters, and an in-place update of the
+    masters - by torch or by the multi-tenant optimizer kernel, which bumps no version counter - shows up in the
+    next forward."""
+    from twinkle_amd import MultiTenantAdamW, trainable_parameters
+    torch.manual_seed(0)
+    ml = MultiLora(max_loras=3, max_r=16, lora_compute_dtype=torch.bfloat16)
+    model = ml.patch(Block(d=256, f=512).bfloat16().to(dev), target_modules='all-linear')
+    g = torch.Generator().manual_seed(1)
+    for n, p in model.named_parameters():
+        if 'lora_' in n:
+            p.data = p.data.float()
+            if '.lora_B.' in n:
+                with torch.no_grad():
+                    p.copy_(torch.randn(p.shape, generator=g) * 0.05)
+    cfgs = {'alice': LoraConfig(r=16, lora_alpha=32, target_modules='all-linear'),
+            'bob': LoraConfig(r=8, lora_alpha=16, target_modules='all-linear')}
+    for n, c in cfgs.items():
+        ml.acquire_lora(n, c)
+    names = list(cfgs)
+    x = torch.randn(300, 256, generator=g).bfloat16()
+    row_tenant = torch.randint(0, 2, (300,), generator=g)
+
+    def forward():
+        with ml.batch(names, row_tenant.to(dev)):
+            return model(x.to(dev))
+
+    def reference():
+        # the reference's arithmetic on the fp32 masters, float64, per layer through the oracle's per-adapter loop
+        m = model.model
+        h = x.double()
+        for layer, act in ((m.q_proj, None), (m.up_proj, torch.nn.functional.silu), (m.down_proj, None)):
+            w = layer.base_layer.weight.detach().double().cpu()
+            b = layer.base_layer.bias.detach().double().cpu() if layer.base_layer.bias is not None else None
+            base = torch.nn.functional.linear(h, w, b)
+            a_list = [layer.lora_A[ml.find_lora_by_tenant(n).adapter_name].weight.detach().double().cpu() for n in names]
+            b_list = [layer.lora_B[ml.find_lora_by_tenant(n).adapter_name].weight.detach().double().cpu() for n in names]
+            h = oracle.multi_lora_linear(h, base, row_tenant, a_list, b_list, [cfgs[n].r for n in names], [2.0, 2.0])
+            if act is not None:
+                h = act(h)
+        return h
+
+    y = forward()
+    assert y.dtype == torch.bfloat16 and max_rel_err(y, reference()) < 3e-2
+    y.float().pow(2).mean().backward()
+    slot = ml.find_lora_by_tenant('alice').adapter_name
+    pa = model.model.q_proj.lora_A[slot].weight
+    assert pa.dtype == torch.float32 and pa.grad is not None and pa.grad.dtype == torch.float32
+    assert pa.grad.abs().max() > 0
+    for n, p in model.named_parameters():
+        assert 'lora_' in n or p.grad is None
+    # masters updated by the optimizer kernel: the next forward must see them
+    opt = MultiTenantAdamW()
+    for n in names:
+        opt.add_tenant(n, trainable_parameters(model, ml.find_lora_by_tenant(n).adapter_name).values(), lr=0.05)
+    before = pa.detach().clone()
+    opt.clip_grad_and_step({'alice': 150, 'bob': 150}, max_grad_norm=1.0)
+    assert (pa.detach() - before).abs().max() > 0
+    y2 = forward()
+    assert max_rel_err(y2, reference()) < 3e-2 and (y2.float() - y.float()).abs().max() > 0

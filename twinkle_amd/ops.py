@@ -29,9 +29,19 @@ class AdapterGroups:
     def __init__(self, a_tensors: Sequence[torch.Tensor], b_tensors: Sequence[torch.Tensor], ranks: Sequence[int],
                  scales: Sequence[float], a_index: Optional[Sequence[int]] = None,
                  a_offset: Optional[Sequence[int]] = None, b_index: Optional[Sequence[int]] = None,
-                 b_offset: Optional[Sequence[int]] = None):
+                 b_offset: Optional[Sequence[int]] = None, master_a: Optional[Sequence[torch.Tensor]] = None,
+                 master_b: Optional[Sequence[torch.Tensor]] = None):
         self.a_tensors = list(a_tensors)
         self.b_tensors = list(b_tensors)
+        # mixed precision: the kernels read `a_tensors` / `b_tensors` (compute copies, e.g. bf16) while the
+        # parameters autograd knows are `master_a` / `master_b` (same shapes, e.g. fp32)
+        self.master_a = list(master_a) if master_a is not None else None
+        self.master_b = list(master_b) if master_b is not None else None
+        if (self.master_a is None) != (self.master_b is None):
+            raise ValueError('master_a and master_b come together')
+        if self.master_a is not None and ([t.shape for t in self.master_a] != [t.shape for t in self.a_tensors] or
+                                          [t.shape for t in self.master_b] != [t.shape for t in self.b_tensors]):
+            raise ValueError('master tensors must have the shapes of the compute copies')
         self.num_groups = len(ranks)
         if self.num_groups == 0:
             raise ValueError('at least one group is needed')
@@ -105,7 +115,22 @@ class AdapterGroups:
 
     def grad_views(self, arena: torch.Tensor, side: str) -> List[torch.Tensor]:
         tensors, offs = (self.a_tensors, self._a_arena_off) if side == 'a' else (self.b_tensors, self._b_arena_off)
+        masters = self.master_a if side == 'a' else self.master_b
+        if masters is not None and masters[0].dtype != arena.dtype:
+            arena = arena.to(masters[0].dtype)        # one cast for the whole side; the views below share it
         return [arena[o:o + t.numel()].view(t.shape) for t, o in zip(tensors, offs)]
+
+    def autograd_tensors(self) -> List[torch.Tensor]:
+        """The tensors gradients are reported for: the masters where there are any, else the tensors read."""
+        if self.master_a is not None:
+            return self.master_a + self.master_b
+        return self.a_tensors + self.b_tensors
+
+    def sync_masters(self) -> None:
+        """Refresh the compute copies from the masters (two multi-tensor copies, whatever changed the masters)."""
+        if self.master_a is not None:
+            with torch.no_grad():
+                torch._foreach_copy_(self.a_tensors + self.b_tensors, self.master_a + self.master_b)
 
 
 def _desc(seg: SegmentTable, groups: AdapterGroups, map_rows: bool) -> _lib.LoraDesc:
@@ -296,13 +321,13 @@ class _LoraLinear(torch.autograd.Function):
 def multi_lora_delta(x: torch.Tensor, base_out: torch.Tensor, seg: SegmentTable, groups: AdapterGroups,
                      map_rows: bool = True) -> torch.Tensor:
     """``base_out`` with every adapter's LoRA term added to its own rows (in place, differentiable)."""
-    return _LoraDelta.apply(x, base_out, seg, groups, map_rows, *groups.a_tensors, *groups.b_tensors)
+    return _LoraDelta.apply(x, base_out, seg, groups, map_rows, *groups.autograd_tensors())
 
 
 def multi_lora_linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], seg: SegmentTable,
                       groups: AdapterGroups, map_rows: bool = True) -> torch.Tensor:
     """``F.linear(x, weight, bias)`` plus the segmented LoRA update as one autograd node."""
-    return _LoraLinear.apply(x, weight, bias, seg, groups, map_rows, *groups.a_tensors, *groups.b_tensors)
+    return _LoraLinear.apply(x, weight, bias, seg, groups, map_rows, *groups.autograd_tensors())
 
 
 # ---- projections that share their input (q / k / v, gate / up) ----------------------------------------------
@@ -403,7 +428,7 @@ def multi_lora_delta_shared(x: torch.Tensor, base_outs: Sequence[torch.Tensor], 
     """
     weights = []
     for g in groups_list:
-        weights += list(g.a_tensors) + list(g.b_tensors)
+        weights += g.autograd_tensors()
     return _LoraDeltaShared.apply(x, seg, tuple(groups_list), map_rows, len(groups_list), *base_outs, *weights)
 
 
@@ -449,6 +474,6 @@ def multi_lora_linear_shared(x: torch.Tensor, weights: Sequence[torch.Tensor],
     dummies = [b if b is not None else x.new_zeros(0) for b in biases]
     lora = []
     for g in groups_list:
-        lora += list(g.a_tensors) + list(g.b_tensors)
+        lora += g.autograd_tensors()
     return _LoraLinearShared.apply(x, seg, tuple(groups_list), map_rows, len(groups_list), has_bias, *weights, *dummies,
                                    *lora)
