@@ -1,9 +1,17 @@
 // bf16 kernels for gfx950 built on v_mfma_f32_16x16x32_bf16 (fp32 accumulate).
 //
-// Both kernels are HBM-streaming: the matrix cores are used because the vector
-// ALUs could not keep up with 8 TB/s at these ranks, not because the op is
-// compute bound.  Everything is laid out so that each wave-wide load covers
-// whole 128-byte lines and every activation byte crosses HBM once per pass.
+// All of these kernels stream activations from HBM: the matrix cores are used
+// because the vector ALUs could not keep up with 8 TB/s at these ranks, not
+// because anything is compute bound.  Everything is laid out so that each
+// wave-wide load covers whole 128-byte lines and every activation byte crosses
+// HBM once per pass.
+//
+//   k_shrink_pair / k_shrink_finish      h = scale * x A^T (split over column slices when x is wide)
+//   k_expand_mfma / k_expand_multi       y += h B^T in place (rank <= 16 / above)
+//   k_dy_fused                           backward, rank <= 16: dB and the slices of dh from one pass over dy
+//   k_wgrad_pipe / k_wgrad_coop64        dA, dB: contraction over the rows of a chunk (rank <= 32 / 33..64)
+//   k_transpose_job                      B^T, A^T copies for the backward shrink / expand
+//   *_multi                              the same bodies for several projections in one launch
 //
 // MFMA operand layout used below (l = lane, 64 lanes):
 //   A operand: lane l holds A[i = l % 16][k = 8 * (l / 16) .. + 8]   (8 bf16 = 16 B)
@@ -27,6 +35,7 @@
 #define TK_WGRAD_STAGES 3
 #endif
 
+// block renumbering of the rank > 16 expand (contiguous runs of tiles per XCD)
 #ifndef TK_XCD_MAP
 #define TK_XCD_MAP(b, n) xcd_contiguous(b, n)
 #endif
