@@ -89,6 +89,17 @@ def test_mixed_batch_equals_each_tenant_alone_and_the_oracle(dev, dtype, tol):
     assert max_rel_err(y_mixed, want) < tol
 
 
+def test_batch_check_rejects_rows_without_a_tenant(dev):
+    ml, model, cfgs = _setup(dev, torch.float32)
+    rows = torch.tensor([0, 1, 3], device=dev)
+    with pytest.raises(ValueError):
+        with ml.batch(['alice', 'bob', 'carol'], rows, check=True):
+            pass
+    with pytest.raises(ValueError):
+        with ml.batch(['alice', 'nobody'], rows[:2]):
+            pass
+
+
 def test_only_the_tenants_in_the_batch_get_gradients(dev):
     """Reference invariant: updates only the active adapter (tests/model/test_multi_lora_target_parameters.py:78-100)."""
     ml, model, cfgs = _setup(dev, torch.float32)

@@ -219,15 +219,21 @@ class MultiLora:
             self.activate_adapter(tenant_adapter_name, call_enable=True)
 
     @contextmanager
-    def batch(self, tenant_adapter_names: Sequence[str], row_tenant: torch.Tensor):
+    def batch(self, tenant_adapter_names: Sequence[str], row_tenant: torch.Tensor, check: bool = False):
         """Many tenants in one forward/backward: row ``i`` uses ``tenant_adapter_names[row_tenant[i]]``.
 
         ``row_tenant`` is an integer GPU tensor with one entry per row of the
         flattened ``[rows, features]`` activations (so ``batch * seq`` entries for
         ``[batch, seq, features]`` inputs).  The segment table is built once here
-        and shared by every patched layer called inside the context.
+        and shared by every patched layer called inside the context.  ``check=True`` verifies that every entry
+        of ``row_tenant`` indexes ``tenant_adapter_names`` (one device synchronisation) and raises ``ValueError``
+        otherwise; unchecked, an entry out of range is an out-of-bounds index on the device.
         """
         slots = [self.find_lora_by_tenant(n).index for n in tenant_adapter_names]
+        if check and row_tenant.numel():
+            lo, hi = int(row_tenant.min()), int(row_tenant.max())
+            if lo < 0 or hi >= len(slots):
+                raise ValueError(f'row_tenant holds {lo}..{hi} but the batch has {len(slots)} tenants')
         lut = torch.tensor(slots, dtype=torch.int32, device=row_tenant.device)
         keys = lut[row_tenant.reshape(-1).long()]
         table = build_segments(keys, self.max_loras, want_perm=False, want_offsets=False)
