@@ -95,3 +95,49 @@ def test_shared_entry_points_reject_malformed_arguments_on_the_host():
     tiny = (ctypes.c_int64 * 2)(16, 16)
     assert lib.tk_lora_bwd_shared(table([a, b]), 2, ptrs, lds, 0x1000, 2048, ptrs, 0x1000, 2048, ptrs, ptrs, 0, ptrs,
                                   tiny, None) == _lib.TK_ERR_WORKSPACE
+
+
+def test_entry_points_reject_malformed_arguments_on_the_host():
+    """Every entry point checks its arguments before any GPU work: fake device pointers, only failing calls."""
+    import ctypes
+    from twinkle_amd import _lib
+    lib = _lib.load()
+    bad, small, unsupported = _lib.TK_ERR_INVALID, _lib.TK_ERR_WORKSPACE, _lib.TK_ERR_UNSUPPORTED
+    P = 0x1000
+    # segment builder
+    assert lib.tk_segment_build(P, 0, -1, 4, None, None, P, 1 << 20, None) == bad           # negative row count
+    assert lib.tk_segment_build(P, 0, 64, 0, None, None, P, 1 << 20, None) == bad           # no groups
+    assert lib.tk_segment_build(None, 0, 64, 4, None, None, P, 1 << 20, None) == bad        # no keys
+    assert lib.tk_segment_build(P, 7, 64, 4, None, None, P, 1 << 20, None) == bad           # unknown key type
+    assert lib.tk_segment_build(P, 0, 64, 1 << 20, None, None, P, 1 << 40, None) == unsupported   # too many groups
+    assert lib.tk_segment_build(P, 0, 64, 4, None, None, P, 16, None) == small              # workspace too small
+    # row movers
+    assert lib.tk_permute_rows(P, 64, P, 64, None, None, 64, 64, 64, 4, 1, None) == bad     # no segment table
+    assert lib.tk_permute_rows(P, 64, P, 64, None, P, 65, 64, 64, 4, 1, None) == bad        # rows not k * tokens
+    assert lib.tk_unpermute_rows(P, 64, P, 64, None, P, 64, 64, 0, 4, 1, None) == bad       # zero width
+    assert lib.tk_unpermute_rows(P, 64, P, 64, None, P, 64, 64, 64, 4, 9, None) == bad      # unknown dtype
+    # single-projection LoRA
+    d = _lib.LoraDesc()
+    d.rows, d.in_features, d.out_features, d.num_groups, d.max_rank, d.dtype = 64, 256, 128, 2, 8, 1
+    d.map_rows, d.lda, d.ldb = 1, 256, 8
+    d.seg_ws = d.lora_A = d.lora_B = d.rank = d.scale = P
+    ref = ctypes.byref(d)
+    assert lib.tk_lora_fwd(ref, P, 255, P, 128, P, None) == bad                              # ldx below in_features
+    assert lib.tk_lora_fwd(ref, P, 256, P, 64, P, None) == bad                               # ldy below out_features
+    assert lib.tk_lora_fwd(ref, P, 256, P, 128, None, None) == bad                           # no h buffer
+    assert lib.tk_lora_fwd(None, P, 256, P, 128, P, None) == bad                             # no descriptor
+    assert lib.tk_lora_bwd(ref, None, 128, P, 256, P, P, 256, P, P, 0, P, 1 << 30, None) == bad   # no dy
+    assert lib.tk_lora_bwd(ref, P, 128, None, 256, P, P, 256, P, P, 0, P, 1 << 30, None) == bad   # dA wanted, no x
+    assert lib.tk_lora_bwd(ref, P, 128, P, 256, P, P, 256, P, P, 0, P, 16, None) == small
+    d.lda = 100
+    assert lib.tk_lora_fwd(ref, P, 256, P, 128, P, None) == bad                              # lda below in_features
+    d.lda, d.dtype = 256, 5
+    assert lib.tk_lora_h_bytes(ref) == bad                                                   # unknown dtype
+    # optimizer
+    assert lib.tk_opt_workspace_bytes(-1, 10) == bad
+    assert lib.tk_opt_grad_norm(P, 4, P, 0, 100, 1, P, P, P, 1 << 20, None) == bad           # no tenants
+    assert lib.tk_opt_grad_norm(P, 4, P, 2, 100, 1, None, P, P, 1 << 20, None) == bad        # no norm output
+    assert lib.tk_opt_grad_norm(P, 4, P, 2, 100, 1, P, P, P, 0, None) == small
+    assert lib.tk_opt_adamw_step(None, 4, P, 2, 100, 1, None, 0, None) == bad                # no tensor table
+    assert lib.tk_opt_adamw_step(P, 70000, P, 2, 100, 1, None, 0, None) == bad               # more tensors than a launch takes
+    assert lib.tk_opt_adamw_step(P, 0, P, 2, 100, 1, None, 0, None) == _lib.TK_OK            # nothing to do

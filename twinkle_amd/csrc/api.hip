@@ -158,8 +158,15 @@ int tk_unpermute_weight_grad(const void* dout, int64_t ld_dout, const void* rows
                                 dtype, (hipStream_t)stream);
 }
 
+// what the size queries need of a descriptor: shapes and dtype, no pointers
+static bool desc_shape_ok(const tk_lora_desc* d) {
+  return d && d->rows >= 0 && d->num_groups > 0 && d->num_groups <= TK_MAX_GROUPS && d->max_rank >= 0 &&
+         d->max_rank <= TK_MAX_RANK && d->in_features > 0 && d->out_features > 0 &&
+         (d->dtype == TK_DTYPE_F32 || d->dtype == TK_DTYPE_BF16);
+}
+
 int64_t tk_lora_h_bytes(const tk_lora_desc* d) {
-  if (!d || d->rows < 0 || d->num_groups <= 0 || d->max_rank < 0 || d->max_rank > TK_MAX_RANK) return TK_ERR_INVALID;
+  if (!desc_shape_ok(d)) return TK_ERR_INVALID;
   // rank-major copy hT[rpad][ld], slot-major copy hrow[ld][rpad], then the partial sums of a split shrink
   const int rpad = rank_pad(d->max_rank);
   return round_up(2 * (int64_t)rpad * h_ld(d->rows, d->num_groups) * elt_bytes(d->dtype), 256) +
@@ -167,7 +174,7 @@ int64_t tk_lora_h_bytes(const tk_lora_desc* d) {
 }
 
 int64_t tk_lora_bwd_workspace_bytes(const tk_lora_desc* d) {
-  if (!d || d->rows < 0 || d->num_groups <= 0 || d->max_rank < 0 || d->max_rank > TK_MAX_RANK) return TK_ERR_INVALID;
+  if (!desc_shape_ok(d)) return TK_ERR_INVALID;
   return BwdLayout(*d).total;
 }
 
