@@ -23,7 +23,7 @@ def _check(keys_cpu, groups, dev, dtype=torch.int32, num_tokens=None):
 @pytest.mark.parametrize('rows,groups,seed', [(1, 1, 0), (5, 2, 1), (63, 3, 2), (64, 64, 3), (65, 7, 4), (511, 16, 5),
                                               (512, 16, 6), (513, 5, 7), (4097, 33, 8), (16384, 16, 9),
                                               (20000, 1000, 10), (70001, 4096, 11), (32768, 64, 12), (32769, 64, 13),
-                                              (32768, 65, 14), (40000, 16, 15)])
+                                              (32768, 65, 14), (40000, 16, 15), (50000, 16384, 16)])
 @pytest.mark.parametrize('dtype', [torch.int32, torch.int64])
 def test_random_keys(dev, rows, groups, seed, dtype):
     keys = torch.randint(0, groups, (rows,), generator=torch.Generator().manual_seed(seed))
