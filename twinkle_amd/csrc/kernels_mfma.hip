@@ -9,7 +9,7 @@
 //   k_shrink_pair / k_shrink_finish      h = scale * x A^T (split over column slices when x is wide)
 //   k_expand_mfma / k_expand_multi       y += h B^T in place (rank <= 16 / above)
 //   k_dy_fused                           backward, rank <= 16: dB and the slices of dh from one pass over dy
-//   k_wgrad_pipe / k_wgrad_coop64        dA, dB: contraction over the rows of a chunk (rank <= 32 / 33..64)
+//   k_wgrad_pipe / k_wgrad_coop          dA, dB: contraction over the rows of a chunk (rank <= 16 / above)
 //   k_transpose_job                      B^T, A^T copies for the backward shrink / expand
 //   *_multi                              the same bodies for several projections in one launch
 //
@@ -24,7 +24,7 @@
 
 #include "tk_mfma.h"
 
-// depths of the software pipelines of k_dy_fused, k_wgrad_pipe<1, S> and k_wgrad_coop64<S> (tiles in registers per wave)
+// depths of the software pipelines of k_dy_fused, k_wgrad_pipe<1, S> and k_wgrad_coop<NB, S> (tiles in registers per wave)
 #ifndef TK_DY_STAGES
 #define TK_DY_STAGES 2
 #endif
@@ -554,8 +554,7 @@ __global__ __launch_bounds__(256) void k_transpose_job(TransposeJob t, const int
 // partial buffer (groups that span several chunks; k_wgrad_reduce adds the chunks in order) or straight
 // into the gradient (single-chunk groups).  No atomics: the result is bitwise repeatable.
 //
-// Padded rank 64 (128 columns x 64 rank indices of accumulators would leave one wave per SIMD) has its own
-// kernel below.
+// This one-wave form serves padded rank 16; above it two waves share the tiles (k_wgrad_coop below).
 // ---------------------------------------------------------------------------
 template <int NB, int S>
 __global__ __launch_bounds__(64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo* __restrict__ chunks,
@@ -650,24 +649,26 @@ __global__ __launch_bounds__(64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo*
 }
 
 // ---------------------------------------------------------------------------
-// Weight gradient at padded rank 64: (chunk, 128 columns), two waves, each owning 32 rank indices and both
-// needing every tile of the source.  Two independent readers of a tile drift apart and the later one misses
-// the CU's cache (measured: 1.66 x the source bytes fetched from memory), so here the tile crosses the
+// Weight gradient at padded rank 32 and 64: (chunk, 128 columns), two waves, each owning half of the rank
+// indices and both needing every tile of the source (one wave with all of them would hold 64 or 128
+// accumulator registers next to its tiles in flight: measured 49 against 41 us at rank 32, one wave per SIMD
+// at rank 64).  Two independent readers of a tile drift apart and the later one misses the CU's cache
+// (measured at rank 64: 1.66 x the source bytes fetched from memory), so here the tile crosses the
 // memory system once: each wave requests half of it (4 of the 8 rows of every lane's 8 x 8 block), S - 1
 // tiles ahead, the halves meet in a double-buffered LDS tile behind an LDS-only barrier (global loads stay
 // in flight), and every wave reads the whole tile back in the operand layout.  Padding rows are zeroed when
 // they are written to LDS.  One barrier per tile: a wave overwrites a buffer two tiles later, after the
 // barrier that every reader of it has passed.
 // ---------------------------------------------------------------------------
-template <int S>
-__global__ __launch_bounds__(128) void k_wgrad_coop64(WgradArgs a, const ChunkInfo* __restrict__ chunks,
+template <int NB, int S>
+__global__ __launch_bounds__(128) void k_wgrad_coop(WgradArgs a, const ChunkInfo* __restrict__ chunks,
                                                       const int32_t* __restrict__ slot_rows) {
-  constexpr int NB = 4, RS = 2, NBW = 2;
+  constexpr int RS = 2, NBW = NB / 2;
   constexpr int OS = kWgradStageStride;
   constexpr int XS = 136;  // row stride of a staged tile in bf16 (272 B)
   // the tile buffers are dead when the result is staged: one array serves both
-  __shared__ __attribute__((aligned(16))) float lds[16 * NB * OS];
-  static_assert(sizeof(float) * 16 * NB * OS >= sizeof(bf16_t) * 2 * kTileRows * XS, "two staged tiles fit");
+  constexpr int kLdsFloats = 16 * NB * OS > kTileRows * XS ? 16 * NB * OS : kTileRows * XS;  // >= two staged bf16 tiles
+  __shared__ __attribute__((aligned(16))) float lds[kLdsFloats];
   extern __shared__ __attribute__((aligned(16))) int32_t rows_s[];  // the chunk's row indices
   const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kb = lane >> 4, rs = tid >> 6;
   if ((int)blockIdx.y < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
@@ -976,7 +977,8 @@ void launch_wgrad_pipe(const WgradArgs& a0, const SegView& seg, const SegLayout&
                      seg.slot_table(a.map_rows));
 }
 
-void launch_wgrad_coop64(const WgradArgs& a0, const SegView& seg, const SegLayout& L, hipStream_t s) {
+template <int NB>
+void launch_wgrad_coop(const WgradArgs& a0, const SegView& seg, const SegLayout& L, hipStream_t s) {
   constexpr int S = TK_COOP_STAGES;
   WgradArgs a = a0;
   a.tr.y_blocks = 0;
@@ -986,7 +988,7 @@ void launch_wgrad_coop64(const WgradArgs& a0, const SegView& seg, const SegLayou
   }
   const dim3 grid((unsigned)(a.width / 128), (unsigned)(L.max_chunks + a.tr.y_blocks));
   const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);
-  hipLaunchKernelGGL((k_wgrad_coop64<S>), grid, dim3(128), dyn, s, a, seg.chunks, seg.slot_table(a.map_rows));
+  hipLaunchKernelGGL((k_wgrad_coop<NB, S>), grid, dim3(128), dyn, s, a, seg.chunks, seg.slot_table(a.map_rows));
 }
 
 }  // namespace
@@ -1091,8 +1093,8 @@ bool wgrad_mfma_supported(const WgradArgs& a) {
 int launch_wgrad_mfma(const WgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
   if (L.rows == 0) return TK_OK;
   if (a.rpad <= 16) launch_wgrad_pipe<1, TK_WGRAD_STAGES>(a, seg, L, s);
-  else if (a.rpad <= 32) launch_wgrad_pipe<2, 3>(a, seg, L, s);
-  else launch_wgrad_coop64(a, seg, L, s);
+  else if (a.rpad <= 32) launch_wgrad_coop<2>(a, seg, L, s);
+  else launch_wgrad_coop<4>(a, seg, L, s);
   return check_launch();
 }
 
