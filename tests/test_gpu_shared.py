@@ -262,3 +262,44 @@ def test_shared_random_projection_sets(dev, seed):
     print(f'case {seed}: t={t} k={k} outs={outs} n={n} ranks={ranks}', flush=True)
     # forward through the shared kernels always; backward too when every width is a multiple of 512
     _compare(dev, torch.bfloat16, t, k, outs, n, 16, ranks, seed=seed)
+
+
+def test_shared_custom_ops_match_direct_calls(dev):
+    """torch.ops.twinkle_amd.lora_fwd_shared / lora_bwd_shared give what the ctypes wrappers give, bit for bit."""
+    from twinkle_amd import lora_bwd_shared_, lora_bwd_workspace_bytes, lora_fwd_shared_, lora_h_bytes
+    t, k, outs, n = 900, 1024, (1024, 512), 3
+    dt = torch.bfloat16
+    g = torch.Generator().manual_seed(41)
+    x = torch.randn(t, k, generator=g).to(dt).to(dev)
+    bases = [torch.randn(t, m, generator=g).to(dt).to(dev) for m in outs]
+    dys = [torch.randn(t, m, generator=g).to(dt).to(dev) for m in outs]
+    keys = torch.randint(0, n, (t,), generator=g).to(torch.int32).to(dev)
+    groups = [grp for grp, _, _ in _groups(_projections(k, outs, n, 16, [(16, 5, 9), (8, 16, 0)], 9, dt, dev), dev)]
+    seg = build_segments(keys, n, want_perm=False, want_offsets=False)
+
+    def buffers():
+        return ([b.clone() for b in bases], torch.zeros_like(x),
+                [torch.empty(lora_h_bytes(seg, grp), dtype=torch.uint8, device=dev) for grp in groups],
+                [torch.empty(lora_bwd_workspace_bytes(seg, grp), dtype=torch.uint8, device=dev) for grp in groups],
+                [torch.zeros(grp.a_arena_elems, dtype=dt, device=dev) for grp in groups],
+                [torch.zeros(grp.b_arena_elems, dtype=dt, device=dev) for grp in groups])
+
+    ys, dx, hs, wss, gas, gbs = buffers()
+    pas = [grp._grad_a_rel + ga.data_ptr() for grp, ga in zip(groups, gas)]
+    pbs = [grp._grad_b_rel + gb.data_ptr() for grp, gb in zip(groups, gbs)]
+    lora_fwd_shared_(x, ys, seg, groups, hs=hs)
+    lora_bwd_shared_(dys, x, hs, dx, pas, pbs, seg, groups, workspaces=wss)
+
+    ys2, dx2, hs2, wss2, gas2, gbs2 = buffers()
+    pas2 = [grp._grad_a_rel + ga.data_ptr() for grp, ga in zip(groups, gas2)]
+    pbs2 = [grp._grad_b_rel + gb.data_ptr() for grp, gb in zip(groups, gbs2)]
+    for grp in groups:
+        grp.refresh()
+    meta = [v for grp in groups for v in (grp.max_rank, grp.lda, grp.ldb)]
+    common = (seg.workspace, [grp.a_ptrs for grp in groups], [grp.b_ptrs for grp in groups],
+              [grp.rank_dev for grp in groups], [grp.scale_dev for grp in groups], meta, True)
+    torch.ops.twinkle_amd.lora_fwd_shared(x, ys2, hs2, *common)
+    torch.ops.twinkle_amd.lora_bwd_shared(dys, x, hs2, dx2, gas2, gbs2, pas2, pbs2, wss2, *common, False)
+    for a, b in zip((*ys, dx, *gas, *gbs), (*ys2, dx2, *gas2, *gbs2)):
+        assert torch.equal(a, b)
+    assert dx.abs().max() > 0 and gas[0].abs().max() > 0

@@ -181,8 +181,12 @@ def test_custom_ops_are_registered_and_traceable():
     import twinkle_amd  # noqa: F401
     from torch._subclasses.fake_tensor import FakeTensorMode
     from twinkle_amd import _lib
-    for name in ('segment_build', 'lora_fwd', 'lora_bwd'):
+    for name in ('segment_build', 'lora_fwd', 'lora_bwd', 'lora_fwd_shared', 'lora_bwd_shared'):
         assert hasattr(torch.ops.twinkle_amd, name)
+    schema = str(torch.ops.twinkle_amd.lora_fwd_shared.default._schema)
+    assert '!)[] ys' in schema and '!)[] hs' in schema
+    schema = str(torch.ops.twinkle_amd.lora_bwd_shared.default._schema)
+    assert '!) dx' in schema and '!)[] grad_a' in schema and '!)[] grad_b' in schema and '!)[] workspaces' in schema
     schema = str(torch.ops.twinkle_amd.lora_fwd.default._schema)
     assert 'Tensor(a1!) y' in schema and 'Tensor(a2!) h' in schema
     schema = str(torch.ops.twinkle_amd.lora_bwd.default._schema)

@@ -13,10 +13,13 @@ passed as the int64 / int32 / float32 device tensors it already holds.
     lora_fwd(x, y, h, seg_ws, a_ptrs, b_ptrs, rank, scale, ...)         y, h written
     lora_bwd(dy, x, h, dx, grad_a, grad_b, grad_a_ptrs, grad_b_ptrs, ws, seg_ws, ...)
                                                      dx, grad_a, grad_b, ws written
+    lora_fwd_shared(x, ys, hs, seg_ws, ...) / lora_bwd_shared(dys, x, hs, dx, ...)
+                                                     the same for projections that share x (tensor lists)
 """
 from __future__ import annotations
 
 import ctypes
+from typing import List
 
 import torch
 
@@ -118,4 +121,67 @@ def lora_bwd(dy: torch.Tensor, x: torch.Tensor, h: torch.Tensor, dx: torch.Tenso
 @lora_bwd.register_fake
 def _(dy, x, h, dx, grad_a, grad_b, grad_a_ptrs, grad_b_ptrs, workspace, seg_ws, a_ptrs, b_ptrs, rank, scale, max_rank,
       lda, ldb, map_rows, accumulate):
+    return None
+
+
+# ---- projections that share their input: one op for all of them -------------------------------------------------
+# Per-projection tensors arrive as lists; `meta` holds (max_rank, lda, ldb) of every projection.
+
+def _shared_descs(x, outs_like, seg_ws, a_ptrs, b_ptrs, rank, scale, meta, map_rows):
+    descs = [_desc(x.shape[0], x.shape[1], o.shape[1], meta[3 * p], x.dtype, map_rows, seg_ws, a_ptrs[p], b_ptrs[p],
+                   meta[3 * p + 1], meta[3 * p + 2], rank[p], scale[p]) for p, o in enumerate(outs_like)]
+    table = (ctypes.c_void_p * len(descs))(*[ctypes.addressof(d) for d in descs])
+    return descs, table
+
+
+def _host(ctype, values):
+    return (ctype * len(values))(*values)
+
+
+@torch.library.custom_op('twinkle_amd::lora_fwd_shared', mutates_args=('ys', 'hs'))
+def lora_fwd_shared(x: torch.Tensor, ys: List[torch.Tensor], hs: List[torch.Tensor], seg_ws: torch.Tensor,
+                    a_ptrs: List[torch.Tensor], b_ptrs: List[torch.Tensor], rank: List[torch.Tensor],
+                    scale: List[torch.Tensor], meta: List[int], map_rows: bool) -> None:
+    """``ys[p][row] += scale (x[row] A_p^T) B_p^T`` for 1..4 projections that read the same ``x``; ``hs[p]``
+    receives projection p's saved shrink output (``tk_lora_fwd_shared``)."""
+    for t, n in ((x, 'x'), (seg_ws, 'seg_ws'), *((y, 'y') for y in ys), *((h, 'h') for h in hs)):
+        _need_gpu(t, n)
+    descs, table = _shared_descs(x, ys, seg_ws, a_ptrs, b_ptrs, rank, scale, meta, map_rows)
+    code = _lib.load().tk_lora_fwd_shared(table, len(descs), x.data_ptr(), x.stride(0),
+                                          _host(ctypes.c_void_p, [y.data_ptr() for y in ys]),
+                                          _host(ctypes.c_int64, [y.stride(0) for y in ys]),
+                                          _host(ctypes.c_void_p, [h.data_ptr() for h in hs]), _lib.stream_ptr())
+    _lib.check(code, 'tk_lora_fwd_shared')
+
+
+@lora_fwd_shared.register_fake
+def _(x, ys, hs, seg_ws, a_ptrs, b_ptrs, rank, scale, meta, map_rows):
+    return None
+
+
+@torch.library.custom_op('twinkle_amd::lora_bwd_shared', mutates_args=('dx', 'grad_a', 'grad_b', 'workspaces'))
+def lora_bwd_shared(dys: List[torch.Tensor], x: torch.Tensor, hs: List[torch.Tensor], dx: torch.Tensor,
+                    grad_a: List[torch.Tensor], grad_b: List[torch.Tensor], grad_a_ptrs: List[torch.Tensor],
+                    grad_b_ptrs: List[torch.Tensor], workspaces: List[torch.Tensor], seg_ws: torch.Tensor,
+                    a_ptrs: List[torch.Tensor], b_ptrs: List[torch.Tensor], rank: List[torch.Tensor],
+                    scale: List[torch.Tensor], meta: List[int], map_rows: bool, accumulate: bool) -> None:
+    """``dx += sum_p dx_p`` in place and every projection's dA / dB through its pointer arrays, which point into
+    ``grad_a[p]`` / ``grad_b[p]`` (``tk_lora_bwd_shared``)."""
+    for t, n in ((x, 'x'), (dx, 'dx'), (seg_ws, 'seg_ws'), *((d, 'dy') for d in dys)):
+        _need_gpu(t, n)
+    descs, table = _shared_descs(x, dys, seg_ws, a_ptrs, b_ptrs, rank, scale, meta, map_rows)
+    code = _lib.load().tk_lora_bwd_shared(
+        table, len(descs), _host(ctypes.c_void_p, [d.data_ptr() for d in dys]),
+        _host(ctypes.c_int64, [d.stride(0) for d in dys]), x.data_ptr(), x.stride(0),
+        _host(ctypes.c_void_p, [h.data_ptr() for h in hs]), dx.data_ptr(), dx.stride(0),
+        _host(ctypes.c_void_p, [t.data_ptr() for t in grad_a_ptrs]),
+        _host(ctypes.c_void_p, [t.data_ptr() for t in grad_b_ptrs]), 1 if accumulate else 0,
+        _host(ctypes.c_void_p, [w.data_ptr() for w in workspaces]),
+        _host(ctypes.c_int64, [w.numel() * w.element_size() for w in workspaces]), _lib.stream_ptr())
+    _lib.check(code, 'tk_lora_bwd_shared')
+
+
+@lora_bwd_shared.register_fake
+def _(dys, x, hs, dx, grad_a, grad_b, grad_a_ptrs, grad_b_ptrs, workspaces, seg_ws, a_ptrs, b_ptrs, rank, scale, meta,
+      map_rows, accumulate):
     return None
