@@ -290,6 +290,114 @@ def cfg5_layer_bench(dev, steps=5):
     return res
 
 
+def cfg5_stack_bench(dev, layers=32, steps=2):
+    """BASELINE config 5: a Llama-3-8B-shaped stack (hidden 4096, 32 heads / 8 KV heads, intermediate 14336, random
+    init, bf16) with LoRA rank 64 on q, k, v, o, gate, up, down, 8 tenants, 8 packed sequences of 4096 tokens (tenant
+    j owns sequence j), dY ~ N(0,1) at the final hidden state; activation checkpointing per layer (as the reference
+    enables it).  Forward + backward per step with the adapters off and with all tenants in one mixed batch."""
+    import torch
+    from torch import nn
+    from torch.utils.checkpoint import checkpoint
+    from twinkle_amd import LoraConfig, MultiLora
+
+    class RMSNorm(nn.Module):
+        def __init__(self, d):
+            super().__init__()
+            self.weight = nn.Parameter(torch.ones(d))
+
+        def forward(self, x):
+            v = x.float()
+            return (v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + 1e-5)).to(x.dtype) * self.weight
+
+    class Layer(nn.Module):
+        def __init__(self, d=4096, heads=32, kv_heads=8, inter=14336):
+            super().__init__()
+            self.heads, self.kv_heads, self.hd = heads, kv_heads, d // heads
+            self.input_layernorm, self.post_attention_layernorm = RMSNorm(d), RMSNorm(d)
+            self.q_proj = nn.Linear(d, d, bias=False)
+            self.k_proj = nn.Linear(d, kv_heads * self.hd, bias=False)
+            self.v_proj = nn.Linear(d, kv_heads * self.hd, bias=False)
+            self.o_proj = nn.Linear(d, d, bias=False)
+            self.gate_proj, self.up_proj = nn.Linear(d, inter, bias=False), nn.Linear(d, inter, bias=False)
+            self.down_proj = nn.Linear(inter, d, bias=False)
+
+        def forward(self, x):                                      # [sequences, tokens, d], causal per sequence
+            b, s, _ = x.shape
+            h = self.input_layernorm(x)
+            q = self.q_proj(h).view(b, s, self.heads, self.hd).transpose(1, 2)
+            k = self.k_proj(h).view(b, s, self.kv_heads, self.hd).transpose(1, 2)
+            v = self.v_proj(h).view(b, s, self.kv_heads, self.hd).transpose(1, 2)
+            rep = self.heads // self.kv_heads
+            a = nn.functional.scaled_dot_product_attention(q, k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1),
+                                                           is_causal=True)
+            x = x + self.o_proj(a.transpose(1, 2).reshape(b, s, -1))
+            h = self.post_attention_layernorm(x)
+            return x + self.down_proj(nn.functional.silu(self.gate_proj(h)) * self.up_proj(h))
+
+    class Stack(nn.Module):
+        def __init__(self, n):
+            super().__init__()
+            self.layers = nn.ModuleList(Layer() for _ in range(n))
+            self.norm = RMSNorm(4096)
+
+        def forward(self, x):
+            for layer in self.layers:
+                x = checkpoint(layer, x, use_reentrant=False)
+            return self.norm(x)
+
+    dt, seqs, toks, d = torch.bfloat16, 8, 4096, 4096
+    torch.manual_seed(7)
+    with torch.device(dev):
+        model = Stack(layers).to(dt)
+    with torch.no_grad():
+        for p in model.parameters():
+            if p.dim() == 2:
+                p.normal_(0, 0.02)
+    ml = MultiLora(max_loras=8, max_r=64, max_length=seqs * toks)
+    model = ml.patch(model, target_modules='all-linear')
+    for n, p in model.named_parameters():
+        if 'lora_' not in n:
+            p.requires_grad_(False)
+        elif '.lora_B.' in n:
+            with torch.no_grad():
+                p.normal_(0, 0.02)
+    names = [f'tenant_{i}' for i in range(8)]
+    for n in names:
+        ml.acquire_lora(n, LoraConfig(r=64, lora_alpha=128, target_modules='all-linear'))
+    x = torch.randn(seqs, toks, d, device=dev, dtype=dt).requires_grad_(True)
+    dy = torch.randn(seqs, toks, d, device=dev, dtype=dt)
+    row_tenant = torch.repeat_interleave(torch.arange(8, device=dev), toks)
+
+    def run(mode):
+        if mode == 'base':
+            with ml.adapter(names[0], disable_lora=True):
+                model(x).backward(dy)
+        else:
+            with ml.batch(names, row_tenant):
+                model(x).backward(dy)
+        x.grad = None
+        for p in model.parameters():
+            p.grad = None
+
+    res = {}
+    for mode in ('base', 'lora'):
+        run(mode)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            run(mode)
+        torch.cuda.synchronize()
+        res[mode + '_ms'] = (time.perf_counter() - t0) * 1e3 / steps
+        print(f'{mode}: {res[mode + "_ms"]:.1f} ms per step', file=sys.stderr, flush=True)
+    T = seqs * toks
+    res.update({'layers': layers, 'tokens': T, 'lora_share_of_step': 1 - res['base_ms'] / res['lora_ms'],
+                'tokens_per_s_with_lora': T / (res['lora_ms'] * 1e-3), 'activation_checkpointing': True,
+                'peak_memory_GiB': torch.cuda.max_memory_allocated() / 2**30,
+                'workload': 'Llama-3-8B-shaped stack, LoRA rank 64 on 7 projections, 8 tenants x 4096 packed tokens, '
+                            'fwd + recompute + bwd; base frozen'})
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -314,6 +422,9 @@ def main():
                     help='run only the q / k / v micro-benchmark (one shared call against one call per projection)')
     ap.add_argument('--layer-cfg5', action='store_true',
                     help='run only the one-layer measurement of BASELINE config 5 (seven projections, rank 64)')
+    ap.add_argument('--stack-cfg5', action='store_true',
+                    help='run only the Llama-3-8B-shaped stack of BASELINE config 5 (see --layers)')
+    ap.add_argument('--layers', type=int, default=32)
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run five plain 128 MiB device copies (a known-size kernel to scale rocprofv3 --pmc '
                          'FETCH_SIZE / WRITE_SIZE readings by)')
@@ -333,6 +444,9 @@ def main():
     dev = torch.device('cuda:0')
     if args.optimizer_only:
         print(json.dumps({'optimizer_step': optimizer_step_bench(dev)}))
+        return
+    if args.stack_cfg5:
+        print(json.dumps({'cfg5_stack': cfg5_stack_bench(dev, layers=args.layers)}))
         return
     if args.layer_cfg5:
         print(json.dumps({'cfg5_layer': cfg5_layer_bench(dev)}))
