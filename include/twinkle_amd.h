@@ -7,6 +7,13 @@
  * allocates, frees, synchronises the device or keeps state between calls,
  * except where stated.  Return value: TK_OK or a negative TK_ERR_* code.
  *
+ * Host threads: every entry point may be called from any thread.  The one
+ * per-device resource the library keeps (the side stream of tk_lora_bwd and
+ * its events) is guarded, so concurrent calls on one device are enqueued one
+ * after the other; what they compute may still overlap on the GPU only as
+ * far as their streams allow, and two calls that share a workspace, an h
+ * buffer or gradient tensors must be ordered by the caller.
+ *
  * The reference (modelscope/twinkle) is pure Python and has no FFI for this
  * path; each entry point below names the reference code whose work it takes
  * over (paths relative to the reference checkout).

@@ -426,3 +426,60 @@ def test_environment_switches_in_a_child_process(dev, env):
     out = subprocess.run([sys.executable, '-c', _ENV_CHILD, root], env={**os.environ, **env}, capture_output=True,
                          text=True, timeout=300)
     assert out.returncode == 0, out.stdout[-2000:] + out.stderr[-2000:]
+
+
+def test_two_host_threads_call_the_two_stream_backward(dev):
+    """Rank 32 takes the backward that forks onto the library's per-device side stream; two host threads, each on
+    its own stream with its own buffers, must get what they get alone (the kernels are deterministic: bit-equal)."""
+    import threading
+    dt = torch.bfloat16
+
+    def make(seed):
+        t, k, m, n, max_r = 3000, 512, 384, 3, 32
+        x, base, dy, a, b, ids, ranks, scales = _problem(t, k, m, n, max_r, [32, 20, 32], seed=seed)
+        p = {'x': x.to(dt).to(dev), 'dy': dy.to(dt).to(dev), 'y0': base.to(dt).to(dev)}
+        ad, bd = [v.to(dt).to(dev) for v in a], [v.to(dt).to(dev) for v in b]
+        p['seg'] = build_segments(ids.to(torch.int32).to(dev), n)
+        p['groups'] = AdapterGroups(ad, bd, ranks, scales)
+        p['keep'] = (ad, bd)
+        return p
+
+    def run(p, iters, out, stream=None):
+        try:
+            with torch.cuda.stream(stream if stream is not None else torch.cuda.current_stream()):
+                for _ in range(iters):
+                    ad, bd = p['keep']
+                    y = p['y0'].clone()
+                    h = lora_fwd_(p['x'], y, p['seg'], p['groups'])
+                    ga, gb = [torch.zeros_like(v) for v in ad], [torch.zeros_like(v) for v in bd]
+                    pa = torch.tensor([v.data_ptr() for v in ga], dtype=torch.int64, device=dev)
+                    pb = torch.tensor([v.data_ptr() for v in gb], dtype=torch.int64, device=dev)
+                    dx = torch.zeros_like(p['x'])
+                    lora_bwd_(p['dy'], p['x'], h, dx, pa, pb, p['seg'], p['groups'])
+                    res = [y, dx] + ga + gb
+                (stream or torch.cuda.current_stream()).synchronize()
+                out.append([v.clone() for v in res])
+        except Exception as e:  # surfaced by the assertion on the main thread
+            out.append(e)
+
+    probs = [make(21), make(22)]
+    alone = []
+    for p in probs:
+        o = []
+        run(p, 1, o)
+        alone.append(o[0])
+    torch.cuda.synchronize()
+    outs = [[], []]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for s in streams:
+        s.wait_stream(torch.cuda.current_stream())
+    threads = [threading.Thread(target=run, args=(probs[i], 8, outs[i], streams[i])) for i in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert len(outs[i]) == 1 and not isinstance(outs[i][0], Exception), outs[i]
+        for got, want in zip(outs[i][0], alone[i]):
+            assert torch.equal(got, want)

@@ -39,6 +39,7 @@ struct SideStream {
   hipStream_t stream = nullptr;
   hipEvent_t fork = nullptr, mid = nullptr, join = nullptr;
   int state = 0;  // 0: not created yet, 1: ready, -1: creation failed (single-stream fallback)
+  std::mutex use;  // held while a call enqueues its fork .. join sequence: the events are shared per device
 };
 
 SideStream* side_stream() {
@@ -317,6 +318,9 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
   // Without a side stream everything runs in the same order on the caller's stream.
   SideStream* side = (grad_B && need_wT) ? side_stream() : nullptr;
   hipStream_t s2 = side ? side->stream : s;
+  // two host threads must not interleave their records and waits on the device's one set of events
+  std::unique_lock<std::mutex> side_guard;
+  if (side) side_guard = std::unique_lock<std::mutex>(side->use);
   if (side) {
     if (hipEventRecord(side->fork, s) != hipSuccess || hipStreamWaitEvent(s2, side->fork, 0) != hipSuccess)
       return TK_ERR_LAUNCH;
