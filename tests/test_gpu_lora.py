@@ -346,6 +346,9 @@ def test_hip_graph_replay_matches_eager(dev, max_r, ranks):
     (torch.bfloat16, 20000, 128, 1024, 16, [16, 5, 16]),    # 32-tile chunks, single pass over dy
     (torch.bfloat16, 40000, 128, 256, 64, [64, 17, 40]),    # 64-tile chunks, rank indices split over two waves
     (torch.float32, 17000, 24, 40, 8, [8, 3]),              # generic kernels walk a chunk in passes of 512 slots
+    (torch.bfloat16, 140000, 128, 1024, 16, [16, 5, 16]),   # 128-tile chunks (the largest), single pass over dy
+    (torch.bfloat16, 140000, 256, 128, 64, [64, 30]),       # 128-tile chunks on the two-wave kernels
+    (torch.float32, 140000, 24, 40, 8, [8, 3]),             # and on the generic ones
 ])
 def test_chunks_larger_than_512_rows(dev, dtype, t, k, m, max_r, ranks):
     """Above 16384 rows a chunk of the row contractions holds 32 or more tiles; groups span several such chunks."""
