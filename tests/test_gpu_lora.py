@@ -72,6 +72,8 @@ def test_config1_fp32_plumbing(dev):
     (1500, 384, 640, 6, 64, [64, 8, 16, 32, 64, 4]),
     (900, 256, 1024, 5, 16, [16, 3, 0, 9, 16]),    # rank <= 16, out width a multiple of 512: one pass over dy
     (2100, 128, 1536, 4, 8, [8, 8, 1, 5]),         # ... with groups that span several chunks
+    (1300, 256, 1024, 5, 32, [32, 17, 0, 24, 5]),  # the same at rank 17..32 (two rank blocks per wave)
+    (2600, 128, 2048, 3, 24, [24, 24, 20]),
 ])
 def test_small_shapes(dev, dtype, t, k, m, n, max_r, ranks):
     _run(dev, dtype, *_problem(t, k, m, n, max_r, ranks, seed=t))

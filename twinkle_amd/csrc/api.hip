@@ -299,12 +299,14 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
   void *bT = plan.bT, *aT = plan.aT;
   const bool mfma = d->dtype == TK_DTYPE_BF16 && !force_generic();
 
-  if (grad_B && need_wT && mfma && pass_mfma_supported(a) && dy_fused_supported(gb, a.kslices)) {
+  const int fused_ks = fused_dy_kslices(d->out_features, a.rpad);
+  if (grad_B && need_wT && mfma && pass_mfma_supported(a) && fused_ks && dy_fused_supported(gb, fused_ks)) {
     // One pass over dy yields dB and the slices of dh (and, on the side, the A^T copy for dX).
+    a.kslices = fused_ks;
     gb.tr = tr;
     gb.tr.bT = nullptr;
-    gb.tr.swizzle_a = 1;  // written here, read only by the expand below
-    a.expand_swizzled = 1;
+    // written here, read only by the expand below (the flat kernel of padded rank 16 wants its rows permuted)
+    gb.tr.swizzle_a = a.expand_swizzled = (a.rpad == 16);
     rc = launch_dy_fused(gb, d->lora_B, d->ldb, a.hpart, a.kslices, V, L, s);
     gb.tr = TransposeJob{};
     if (rc != TK_OK) return rc;

@@ -8,7 +8,7 @@
 //
 //   k_shrink_pair / k_shrink_finish      h = scale * x A^T (split over column slices when x is wide)
 //   k_expand_mfma / k_expand_multi       y += h B^T in place (rank <= 16 / above)
-//   k_dy_fused                           backward, rank <= 16: dB and the slices of dh from one pass over dy
+//   k_dy_fused<NB>                       backward, rank <= 32: dB and the slices of dh from one pass over dy
 //   k_wgrad_pipe / k_wgrad_coop          dA, dB: contraction over the rows of a chunk (rank <= 16 / above)
 //   k_transpose_job                      B^T, A^T copies for the backward shrink / expand
 //   *_multi                              the same bodies for several projections in one launch
@@ -24,9 +24,13 @@
 
 #include "tk_mfma.h"
 
-// depths of the software pipelines of k_dy_fused, k_wgrad_pipe<1, S> and k_wgrad_coop<NB, S> (tiles in registers per wave)
+// depths of the software pipelines of k_dy_fused<1>, k_dy_fused<2> (one tile: with two blocks of accumulators a second
+// tile in registers leaves one wave per SIMD), k_wgrad_pipe<1, S> and k_wgrad_coop<NB, S> (tiles in registers per wave)
 #ifndef TK_DY_STAGES
 #define TK_DY_STAGES 2
+#endif
+#ifndef TK_DY_STAGES2
+#define TK_DY_STAGES2 1
 #endif
 #ifndef TK_COOP_STAGES
 #define TK_COOP_STAGES 3
@@ -765,7 +769,7 @@ __global__ __launch_bounds__(128) void k_wgrad_coop(WgradArgs a, const ChunkInfo
 }
 
 // ---------------------------------------------------------------------------
-// Backward, both uses of dy in one pass (rank <= 16, width a multiple of 512): a block of four waves owns
+// Backward, both uses of dy in one pass (rank <= 16 NB, NB = 1 or 2; width a multiple of 512): a block of four waves owns
 // (chunk of one group, 512 columns), wave w the columns [128 w, 128 w + 128) of it.
 // Per tile a wave loads its 32 x 128 piece once, in the weight-gradient layout (a lane holds 8 rows x 8
 // columns), and uses it twice:
@@ -778,16 +782,18 @@ __global__ __launch_bounds__(128) void k_wgrad_coop(WgradArgs a, const ChunkInfo
 //        k_shrink_finish turns into dh like after a separate shrink.
 // dy crosses the memory system once instead of twice.  Sums are formed in a fixed order.
 // ---------------------------------------------------------------------------
+template <int NB>
 __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* const* __restrict__ lora_B, int64_t ldb,
                                               float* __restrict__ hpart, int kslices,
                                               const ChunkInfo* __restrict__ chunks,
                                               const int32_t* __restrict__ slot_rows, int bx, int by, int x_blocks) {
-  constexpr int SS = 136;  // row stride of the staged piece in bf16 (272 B)
-  constexpr int PR = 17;   // row stride of the partial dh in floats
-  __shared__ int32_t rows_s[kChunkTilesMax * kTileRows];
+  constexpr int RP = 16 * NB;
+  constexpr int SS = 136;     // row stride of the staged piece in bf16 (272 B)
+  constexpr int PR = RP + 1;  // row stride of the partial dh in floats
+  extern __shared__ int32_t rows_s[];  // the chunk's row indices (chunk_tiles x 32)
   __shared__ __attribute__((aligned(16))) bf16_t stage[4][kTileRows * SS];
   __shared__ float part[2][4][kTileRows * PR];
-  static_assert(sizeof(bf16_t) * kTileRows * SS >= sizeof(float) * 16 * kWgradStageStride, "stage holds the dB block too");
+  static_assert(sizeof(bf16_t) * kTileRows * SS >= sizeof(float) * 16 * kWgradStageStride, "stage holds a dB block too");
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
   if (by < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
     transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)by * x_blocks + bx) * 256 + tid,
@@ -797,22 +803,24 @@ __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* co
   const ChunkInfo ci = chunks[by - a.tr.y_blocks];
   const int g = ci.group;
   if (g < 0) return;
-  const int r = min(a.rank[g], 16);
+  const int r = min(a.rank[g], RP);
   if (r <= 0) return;
   const int slab = bx;
   const int c0 = slab * 512 + wave * 128;
   const int nt = ci.ntiles;
   for (int i = tid; i < nt * kTileRows; i += 256) rows_s[i] = slot_rows[ci.tile0 * kTileRows + i];
-  // this wave's block of B as MFMA B operand: lane (n = li, kb) holds B[c0 + 32 s + 8 kb + i][n], i = 0..7
-  uint4 wB[4];
-  {
-    const bf16_t* Bg = (const bf16_t*)lora_B[g] + (int64_t)(c0 + 8 * kb) * ldb + li;
+  // this wave's block of B as MFMA B operand: lane (n = 16 nb + li, kb) holds B[c0 + 32 s + 8 kb + i][n], i = 0..7
+  uint4 wB[NB][4];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const int n = 16 * nb + li;
+    const bf16_t* Bg = (const bf16_t*)lora_B[g] + (int64_t)(c0 + 8 * kb) * ldb + (n < r ? n : 0);
 #pragma unroll
     for (int s4 = 0; s4 < 4; ++s4) {
       uint32_t e[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) e[i] = li < r ? Bg[(int64_t)(32 * s4 + i) * ldb] : 0;
-      wB[s4] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
+      for (int i = 0; i < 8; ++i) e[i] = n < r ? Bg[(int64_t)(32 * s4 + i) * ldb] : 0;
+      wB[nb][s4] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
     }
   }
   __syncthreads();
@@ -820,13 +828,15 @@ __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* co
   const bf16_t* src = (const bf16_t*)a.src + c0 + 8 * li;
   const bf16_t* hT = (const bf16_t*)a.hT + (int64_t)li * a.ldh + (int64_t)ci.tile0 * kTileRows + 8 * kb;
   bf16_t* my_stage = stage[wave];
-  f32x4 acc[8][1];
+  f32x4 acc[8][NB];
 #pragma unroll
-  for (int q = 0; q < 8; ++q) acc[q][0] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int q = 0; q < 8; ++q)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[q][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // loads are unconditional (tiles past the end re-read the last one, padding slots read row 0) and what
   // must not count is zeroed when it is consumed: no branch between a load and its use
-  auto issue = [&](int t, uint4 (&x)[8], uint4& h, uint32_t& live) {
+  auto issue = [&](int t, uint4 (&x)[8], uint4 (&h)[NB], uint32_t& live) {
     const int tc = min(t, nt - 1);
     const int4 ra = *reinterpret_cast<const int4*>(rows_s + tc * kTileRows + 8 * kb);
     const int4 rb = *reinterpret_cast<const int4*>(rows_s + tc * kTileRows + 8 * kb + 4);
@@ -837,9 +847,10 @@ __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* co
       x[q] = ld16(src + (int64_t)max(rows[q], 0) * a.ld_src);
       live |= (t < nt && rows[q] >= 0) ? (1u << q) : 0u;
     }
-    h = ld16(hT + tc * kTileRows);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) h[nb] = ld16(hT + (int64_t)(16 * nb) * a.ldh + tc * kTileRows);
   };
-  auto consume = [&](int t, uint4 (&x)[8], const uint4& h, uint32_t live) {
+  auto consume = [&](int t, uint4 (&x)[8], const uint4 (&h)[NB], uint32_t live) {
 #pragma unroll
     for (int q = 0; q < 8; ++q)
       if (!((live >> q) & 1u)) x[q] = zero4();
@@ -862,24 +873,33 @@ __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* co
       tr.y = __builtin_amdgcn_perm(e[3], e[2], sel);
       tr.z = __builtin_amdgcn_perm(e[5], e[4], sel);
       tr.w = __builtin_amdgcn_perm(e[7], e[6], sel);
-      acc[q][0] = mfma16(tr, h, acc[q][0]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) acc[q][nb] = mfma16(tr, h[nb], acc[q][nb]);
     }
     // dh: partial over this wave's 128 columns (LDS operations of one wave complete in order)
     float* mine = part[t & 1][wave];
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
-      f32x4 d = {0.f, 0.f, 0.f, 0.f};
+      f32x4 d[NB];
 #pragma unroll
-      for (int s4 = 0; s4 < 4; ++s4) d = mfma16(ld16(my_stage + (16 * tt + li) * SS + 32 * s4 + 8 * kb), wB[s4], d);
+      for (int nb = 0; nb < NB; ++nb) d[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int v = 0; v < 4; ++v) mine[(16 * tt + 4 * kb + v) * PR + li] = d[v];
+      for (int s4 = 0; s4 < 4; ++s4) {
+        const uint4 piece = ld16(my_stage + (16 * tt + li) * SS + 32 * s4 + 8 * kb);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) d[nb] = mfma16(piece, wB[nb][s4], d[nb]);
+      }
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) mine[(16 * tt + 4 * kb + v) * PR + 16 * nb + li] = d[nb][v];
     }
     lds_barrier();
     if (wave == (t & 3)) {
-      float* o = hpart + ((int64_t)(ci.tile0 + t) * kslices + slab) * (kTileRows * 16);
+      float* o = hpart + ((int64_t)(ci.tile0 + t) * kslices + slab) * (kTileRows * RP);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int idx = lane + 64 * i, row = idx >> 4, n = idx & 15;
+      for (int i = 0; i < 8 * NB; ++i) {
+        const int idx = lane + 64 * i, row = idx / RP, n = idx % RP;
         float sum = part[t & 1][0][row * PR + n];
         sum += part[t & 1][1][row * PR + n];
         sum += part[t & 1][2][row * PR + n];
@@ -889,10 +909,10 @@ __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* co
     }
   };
 
-  constexpr int S = TK_DY_STAGES;  // software pipeline: S - 1 tiles in flight while one is consumed
+  constexpr int S = NB == 1 ? TK_DY_STAGES : TK_DY_STAGES2;  // software pipeline: S - 1 tiles in flight while one is consumed
   struct Tile {
     uint4 x[8];
-    uint4 h;
+    uint4 h[NB];
     uint32_t live;
   };
   Tile T[S];
@@ -911,15 +931,23 @@ __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* co
 #pragma unroll
   for (int i = 0; i < S - 1; ++i)
     if (t + i < nt) consume(t + i, T[i].x, T[i].h, T[i].live);
-  // every wave has its own 128 columns of dB
-  wgrad_store<1>(acc, reinterpret_cast<float*>(my_stage), a, ci, g, r, c0, lane);
+  // every wave has its own 128 columns of dB; they leave 16 rank indices at a time through the wave's stage
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    if (16 * nb >= r) break;
+    f32x4 one[8][1];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) one[q][0] = acc[q][nb];
+    wgrad_store<1>(one, reinterpret_cast<float*>(my_stage), a, ci, g, r, c0, lane, 16 * nb);
+  }
 }
 
+template <int NB>
 __global__ __launch_bounds__(256) void k_dy_fused(WgradArgs a, const void* const* __restrict__ lora_B, int64_t ldb,
                                                   float* __restrict__ hpart, int kslices,
                                                   const ChunkInfo* __restrict__ chunks,
                                                   const int32_t* __restrict__ slot_rows) {
-  dy_fused_body(a, lora_B, ldb, hpart, kslices, chunks, slot_rows, blockIdx.x, blockIdx.y, gridDim.x);
+  dy_fused_body<NB>(a, lora_B, ldb, hpart, kslices, chunks, slot_rows, blockIdx.x, blockIdx.y, gridDim.x);
 }
 
 // Up to kMaxShared projections in one launch: a narrow projection alone has too few (chunk, 512 columns)
@@ -932,8 +960,8 @@ __global__ __launch_bounds__(256) void k_dy_fused_multi(DyFusedJobs jobs, const 
   for (int i = 1; i < kMaxShared; ++i) p += (i < jobs.n && (int)blockIdx.x >= jobs.x_first[i]) ? 1 : 0;
   const DyFusedJob& j = jobs.j[p];
   if ((int)blockIdx.y >= j.a.tr.y_blocks + max_chunks) return;
-  dy_fused_body(j.a, j.lora_B, j.ldb, j.hpart, j.kslices, chunks, slot_rows, blockIdx.x - jobs.x_first[p], blockIdx.y,
-                j.x_blocks);
+  dy_fused_body<1>(j.a, j.lora_B, j.ldb, j.hpart, j.kslices, chunks, slot_rows, blockIdx.x - jobs.x_first[p],
+                   blockIdx.y, j.x_blocks);
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -994,7 +1022,8 @@ void launch_wgrad_coop(const WgradArgs& a0, const SegView& seg, const SegLayout&
 }  // namespace
 
 bool dy_fused_supported(const WgradArgs& a, int kslices) {
-  return a.rpad == 16 && a.width % 512 == 0 && kslices >= 2 && kslices == a.width / 512 && wgrad_mfma_supported(a);
+  return (a.rpad == 16 || a.rpad == 32) && a.width % 512 == 0 && kslices >= 2 && kslices == a.width / 512 &&
+         wgrad_mfma_supported(a);
 }
 
 int launch_dy_fused(const WgradArgs& a0, const void* const* lora_B, int64_t ldb, float* hpart, int kslices,
@@ -1007,8 +1036,13 @@ int launch_dy_fused(const WgradArgs& a0, const void* const* lora_B, int64_t ldb,
     a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 512) * 256)));
   }
   const dim3 grid((unsigned)(a.width / 512), (unsigned)(L.max_chunks + a.tr.y_blocks));
-  hipLaunchKernelGGL(k_dy_fused, grid, dim3(256), 0, s, a, lora_B, ldb, hpart, kslices, seg.chunks,
-                     seg.slot_table(a.map_rows));
+  const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);  // a chunk's row indices
+  if (a.rpad == 16)
+    hipLaunchKernelGGL(k_dy_fused<1>, grid, dim3(256), dyn, s, a, lora_B, ldb, hpart, kslices, seg.chunks,
+                       seg.slot_table(a.map_rows));
+  else
+    hipLaunchKernelGGL(k_dy_fused<2>, grid, dim3(256), dyn, s, a, lora_B, ldb, hpart, kslices, seg.chunks,
+                       seg.slot_table(a.map_rows));
   return check_launch();
 }
 
@@ -1030,7 +1064,8 @@ int launch_dy_fused_multi(const DyFusedJob* jobs, int n, const SegView& seg, con
     J.x_first[p + 1] = J.x_first[p] + j.x_blocks;
     gy = std::max(gy, (int)L.max_chunks + j.a.tr.y_blocks);
   }
-  hipLaunchKernelGGL(k_dy_fused_multi, dim3((unsigned)J.x_first[n], (unsigned)gy), dim3(256), 0, s, J, seg.chunks,
+  const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);
+  hipLaunchKernelGGL(k_dy_fused_multi, dim3((unsigned)J.x_first[n], (unsigned)gy), dim3(256), dyn, s, J, seg.chunks,
                      seg.slot_table(J.j[0].a.map_rows), (int)L.max_chunks);
   return check_launch();
 }

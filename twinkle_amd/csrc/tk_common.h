@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <algorithm>
+
 #include "twinkle_amd.h"
 
 namespace tk {
@@ -151,6 +153,16 @@ static inline int64_t shrink_partial_bytes(int64_t rows, int64_t groups, int wid
   return ks > 1 ? round_up(SegLayout(rows, groups).max_tiles * ks * (int64_t)kTileRows * rpad * 4, 256) : 0;
 }
 
+// The single-pass backward kernel (padded rank 16 or 32, width a multiple of 512) leaves one slice of dh per
+// 512 columns, which at rank 32 is twice the slices of the shrink kernel it replaces.
+static inline int fused_dy_kslices(int width, int rpad) {
+  return ((rpad == 16 || rpad == 32) && width % 512 == 0 && width >= 1024) ? width / 512 : 0;
+}
+static inline int64_t bwd_partial_bytes(int64_t rows, int64_t groups, int width, int rpad) {
+  const int ks = std::max(shrink_kslices(width, rpad), fused_dy_kslices(width, rpad));
+  return ks > 1 ? round_up(SegLayout(rows, groups).max_tiles * ks * (int64_t)kTileRows * rpad * 4, 256) : 0;
+}
+
 // Backward workspace carving.
 struct BwdLayout {
   int64_t off_dh, off_hpart, off_wT_shrink, off_wT_expand, off_part_a, off_part_b, total;
@@ -162,7 +174,7 @@ struct BwdLayout {
     const int64_t e = elt_bytes(d.dtype);
     int64_t o = 0;
     off_dh = o;         o += round_up(2 * rpad * ldh * e, 256);  // rank-major + slot-major copies
-    off_hpart = o;      o += shrink_partial_bytes(d.rows, d.num_groups, d.out_features, (int)rpad);
+    off_hpart = o;      o += bwd_partial_bytes(d.rows, d.num_groups, d.out_features, (int)rpad);
     // B^T per group [rpad][M]  (shrink weight of the backward pass)
     off_wT_shrink = o;  o += round_up((int64_t)d.num_groups * rpad * d.out_features * e, 256);
     // A^T per group [K][rpad]  (expand weight of the backward pass)
