@@ -876,7 +876,10 @@ __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* co
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) acc[q][nb] = mfma16(tr, h[nb], acc[q][nb]);
     }
-    // dh: partial over this wave's 128 columns (LDS operations of one wave complete in order)
+  };
+  // dh of tile t from the staged piece: partial over this wave's 128 columns (LDS operations of one wave complete
+  // in order); needs no register of the tile any more
+  auto consume_dh = [&](int t) {
     float* mine = part[t & 1][wave];
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
@@ -916,21 +919,36 @@ __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* co
     uint32_t live;
   };
   Tile T[S];
-#pragma unroll
-  for (int i = 0; i < S - 1; ++i) issue(i, T[i].x, T[i].h, T[i].live);
-  int t = 0;
-  for (; t + S <= nt; t += S) {  // every tile consumed in here exists (the youngest requests may lie past the end)
-#pragma unroll
-    for (int i = 0; i < S; ++i) {
-      Tile& Y = T[(i + S - 1) % S];
-      issue(t + i + S - 1, Y.x, Y.h, Y.live);
-      consume(t + i, T[i].x, T[i].h, T[i].live);
+  if constexpr (S == 1) {
+    // one tile in registers: its successor is requested as soon as the dB products have used it up, and is in
+    // flight during the dh half of the iteration
+    issue(0, T[0].x, T[0].h, T[0].live);
+    for (int t = 0; t < nt; ++t) {
+      consume(t, T[0].x, T[0].h, T[0].live);
+      issue(t + 1, T[0].x, T[0].h, T[0].live);
+      consume_dh(t);
     }
-  }
-  // fewer than S tiles are left, all of them requested already
+  } else {
 #pragma unroll
-  for (int i = 0; i < S - 1; ++i)
-    if (t + i < nt) consume(t + i, T[i].x, T[i].h, T[i].live);
+    for (int i = 0; i < S - 1; ++i) issue(i, T[i].x, T[i].h, T[i].live);
+    int t = 0;
+    for (; t + S <= nt; t += S) {  // every tile consumed in here exists (the youngest requests may lie past the end)
+#pragma unroll
+      for (int i = 0; i < S; ++i) {
+        Tile& Y = T[(i + S - 1) % S];
+        issue(t + i + S - 1, Y.x, Y.h, Y.live);
+        consume(t + i, T[i].x, T[i].h, T[i].live);
+        consume_dh(t + i);
+      }
+    }
+    // fewer than S tiles are left, all of them requested already
+#pragma unroll
+    for (int i = 0; i < S - 1; ++i)
+      if (t + i < nt) {
+        consume(t + i, T[i].x, T[i].h, T[i].live);
+        consume_dh(t + i);
+      }
+  }
   // every wave has its own 128 columns of dB; they leave 16 rank indices at a time through the wave's stage
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
