@@ -488,3 +488,42 @@ def test_two_host_threads_call_the_two_stream_backward(dev):
         assert len(outs[i]) == 1 and not isinstance(outs[i][0], Exception), outs[i]
         for got, want in zip(outs[i][0], alone[i]):
             assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize('max_r,ranks', [(16, [16, 7, 0]), (32, [32, 20, 9]), (64, [64, 33, 16])])
+def test_backward_with_a_subset_of_the_outputs(dev, max_r, ranks):
+    """A caller may want only dX (frozen adapters), only the weight gradients (input without gradient) or one side
+    of them: every subset goes through a different sequence of kernels and must agree with the full call."""
+    dt = torch.bfloat16
+    t, k, m, n = 1500, 256, 1024, 3
+    x, base, dy, a, b, ids, _, scales = _problem(t, k, m, n, max_r, ranks, seed=77)
+    xd, dyd = x.to(dt).to(dev), dy.to(dt).to(dev)
+    ad, bd = [v.to(dt).to(dev) for v in a], [v.to(dt).to(dev) for v in b]
+    seg = build_segments(ids.to(torch.int32).to(dev), n)
+    groups = AdapterGroups(ad, bd, ranks, scales)
+    h = lora_fwd_(xd, base.to(dt).to(dev), seg, groups)
+
+    def call(want_dx, want_a, want_b):
+        ga, gb = [torch.zeros_like(v) for v in ad], [torch.zeros_like(v) for v in bd]
+        pa = torch.tensor([v.data_ptr() for v in ga], dtype=torch.int64, device=dev) if want_a else None
+        pb = torch.tensor([v.data_ptr() for v in gb], dtype=torch.int64, device=dev) if want_b else None
+        dx = torch.zeros_like(xd) if want_dx else None
+        lora_bwd_(dyd, xd if want_a else None, h if want_b else None, dx, pa, pb, seg, groups)
+        torch.cuda.synchronize()
+        return dx, ga, gb
+
+    full = call(True, True, True)
+    for want in [(True, False, False), (False, True, True), (False, False, True), (False, True, False),
+                 (True, True, False), (True, False, True)]:
+        dx, ga, gb = call(*want)
+        if want[0]:
+            assert max_rel_err(dx, full[0].double().cpu()) < 1e-2, want
+        for g in range(n):
+            if want[1]:
+                assert max_rel_err(ga[g], full[1][g].double().cpu()) < 1e-2, want
+            else:
+                assert torch.count_nonzero(ga[g]) == 0
+            if want[2]:
+                assert max_rel_err(gb[g], full[2][g].double().cpu()) < 1e-2, want
+            else:
+                assert torch.count_nonzero(gb[g]) == 0
