@@ -287,13 +287,13 @@ def test_custom_ops_match_direct_calls(dev):
     assert y1.float().sub(bf(base).float()).abs().max() > 0
 
 
-@pytest.mark.parametrize('max_r,ranks', [(16, [16, 7, 16]), (32, [32, 16, 24])])
+@pytest.mark.parametrize('max_r,ranks', [(16, [16, 7, 16]), (32, [32, 16, 24]), (64, [64, 16, 40])])
 def test_hip_graph_replay_matches_eager(dev, max_r, ranks):
     """Segment build + forward + backward captured in a HIP graph and replayed: every replay equals the eager result.
 
-    Rank 16 takes the single-pass dy kernel; rank 32 takes the separate kernels, whose backward forks onto the
-    library's side stream and joins back (both must be capturable).  Eager work and synchronisations run between
-    the replays.
+    Ranks 16 and 32 take the single-pass dy kernel; rank 64 takes the separate kernels, whose backward forks onto
+    the library's side stream and joins back (both must be capturable).  Eager work and synchronisations run
+    between the replays.
     """
     from twinkle_amd import lora_bwd_, lora_bwd_workspace_bytes, lora_fwd_, lora_h_bytes
     t, k, m, n = 1200, 256, 1024, 3
