@@ -434,8 +434,9 @@ def test_environment_switches_in_a_child_process(dev, env):
 
 
 def test_two_host_threads_call_the_two_stream_backward(dev):
-    """Rank 32 takes the backward that forks onto the library's per-device side stream; two host threads, each on
-    its own stream with its own buffers, must get what they get alone (the kernels are deterministic: bit-equal)."""
+    """Rank 32 at an output width of 384 takes the backward that forks onto the library's per-device side stream;
+    two host threads, each on its own stream with its own buffers, must get what they get alone (the kernels are
+    deterministic: bit-equal)."""
     import threading
     dt = torch.bfloat16
 
