@@ -239,6 +239,41 @@ int tk_lora_bwd_shared(const tk_lora_desc* const* descs, int32_t num_proj, const
                        int32_t accumulate, void* const* workspace_device, const int64_t* workspace_bytes,
                        tk_stream_t stream);
 
+/* ---- packed experts: grouped base GEMM with the LoRA term in its epilogue -------------------------------
+ *
+ * y[row] = x[row] W_e^T (+ h[row] B_g^T) for every row of the segment table, where the table was built from
+ * keys g = e * groups_per_expert + tenant and expert e's weight [out_features][in_features] starts at
+ * weight_device + e * weight_stride elements (row stride ldw).  Replaces the per-expert host loop of
+ * F.linear calls with one synchronisation per expert (reference: moe/expert_parallel.py:347-371, the
+ * gate_up and the down projection each); with `lora` it also takes over the expert LoRA delta that the
+ * reference merges into the weights (multi_lora_target_parameters.py:158-179): call tk_lora_shrink(lora, x, h)
+ * first and pass that h here, y is then written once with both terms.  The backward of the base term is the
+ * same call on the transposed weights (dx = dy W_e: pass a [in_features][out_features] copy); the LoRA
+ * gradients come from tk_lora_bwd with dx accumulated onto this call's result.
+ *
+ * bf16 only; in_features a multiple of 64, out_features of 128, ldx / ldw / weight_stride multiples of 8 and
+ * ldy of 4 elements, 16-byte aligned x and weight, 8-byte aligned y: anything else is TK_ERR_UNSUPPORTED
+ * (run the experts one by one then).  y rows of the table are overwritten; x and y must not overlap.
+ * lora (optional) must describe the same rows, groups, features, seg_ws and map_rows. */
+typedef struct {
+  int64_t rows;
+  int32_t num_groups;        /* experts * groups_per_expert */
+  int32_t groups_per_expert; /* tenants per expert in the key; 1 for the reference's expert-only grouping */
+  int32_t in_features;
+  int32_t out_features;
+  int32_t dtype;             /* TK_DTYPE_BF16 */
+  int32_t map_rows;          /* as in tk_lora_desc */
+  const void* seg_ws;        /* device: segment table of tk_segment_build for (rows, num_groups) */
+  const void* weight_device;
+  int64_t weight_stride;     /* elements between consecutive experts */
+  int64_t ldw;
+} tk_grouped_desc;
+
+int64_t tk_grouped_linear_workspace_bytes(const tk_grouped_desc* desc);
+int tk_grouped_linear(const tk_grouped_desc* desc, const tk_lora_desc* lora, const void* x_device, int64_t ldx,
+                      void* y_device, int64_t ldy, const void* h_device, void* workspace_device,
+                      int64_t workspace_bytes, tk_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

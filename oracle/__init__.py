@@ -23,8 +23,9 @@ unpermute                                                  : pinned
     (index_add_ closed form; permute∘unpermute identity)
 lora_linear_forward / multi_lora_linear / grads            : pinned
     (fp64 closed form, gradcheck, B=0, r<max_r, single segment ≡ F.linear)
-expert_delta_weight / expert_lora_low_rank                 : pinned
-    (merged-weight form ≡ low-rank form; shape KAT of the reference test)
+expert_delta_weight / expert_lora_low_rank / experts_linear : pinned
+    (merged-weight form ≡ low-rank form; shape KAT of the reference test; the chunk loop
+    against a row-by-row product with each row's own expert and against one F.linear for E = 1)
 packed_cu_seqlens                                          : pinned (brute force)
 slice_rank_tensor / copy_rank_tensor / match_target_modules : pinned
     (round-trip + hand-written cases from the reference's comments)
@@ -51,6 +52,7 @@ from .lora import (  # noqa: F401
     copy_rank_tensor,
     expert_delta_weight,
     expert_lora_low_rank,
+    experts_linear,
     lora_linear_forward,
     lora_scaling,
     match_target_modules,

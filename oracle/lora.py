@@ -104,6 +104,20 @@ def expert_delta_weight(lora_A: torch.Tensor, lora_B: torch.Tensor, r: int, scal
     return torch.einsum('eor,eri->eio', wb, wa) * scaling
 
 
+def experts_linear(x_sorted: torch.Tensor, offsets: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``y_e = F.linear(x_e, weight[e])`` over the contiguous per-expert chunks of rows in expert order.
+
+    Follows src/twinkle/model/transformers/moe/expert_parallel.py:347-371 (one ``F.linear`` per projection per
+    expert, empty experts skipped, chunks concatenated); ``offsets`` is the ``cumsum`` of :347-349,
+    ``weight`` the packed ``[E, out, in]`` parameter (``gate_up_proj`` or ``down_proj``).
+    """
+    chunks = []
+    for e in range(weight.shape[0]):
+        s, t = int(offsets[e]), int(offsets[e + 1])
+        chunks.append(F.linear(x_sorted[s:t], weight[e]))
+    return torch.cat(chunks, dim=0) if chunks else x_sorted.new_empty(0, weight.shape[1])
+
+
 def expert_lora_low_rank(x_sorted: torch.Tensor, offsets: torch.Tensor, base_out: torch.Tensor, lora_A: torch.Tensor,
                          lora_B: torch.Tensor, r: int, scaling: float) -> torch.Tensor:
     """``y_e = base_e + s (x_e A_e^T) B_e^T`` over contiguous per-expert chunks.

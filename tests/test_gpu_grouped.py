@@ -1,0 +1,121 @@
+"""Grouped base GEMM of packed experts (tk_grouped_linear), alone and with the LoRA term in its epilogue,
+against the CPU oracle's per-expert loop.  bf16 bar: max |got - ref| / max |ref| < 2e-2 against float64."""
+import pytest
+import torch
+
+import oracle
+from conftest import max_rel_err
+from twinkle_amd import AdapterGroups, build_segments, grouped_linear_, lora_h_bytes, lora_shrink_
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(e, nt, t, k, n, seed, empty=()):
+    g = torch.Generator().manual_seed(seed)
+    probs = torch.rand(e, generator=g) + 0.2
+    for i in empty:
+        probs[i] = 0
+    expert = torch.multinomial(probs, t, replacement=True, generator=g)
+    tenant = torch.randint(0, nt, (t,), generator=g)
+    x = torch.randn(t, k, generator=g).bfloat16()
+    w = (torch.randn(e, n, k, generator=g) / k**0.5).bfloat16()
+    return expert, tenant, x, w
+
+
+def _reference(x, w, expert):
+    """Oracle's chunk loop on rows sorted by expert (stable), scattered back to the original row order."""
+    order = torch.argsort(expert, stable=True)
+    counts = torch.bincount(expert, minlength=w.shape[0])
+    offsets = torch.cat([torch.zeros(1, dtype=torch.long), counts.cumsum(0)])
+    out_sorted = oracle.experts_linear(x.double()[order], offsets, w.double())
+    out = torch.empty_like(out_sorted)
+    out[order] = out_sorted
+    return out
+
+
+@pytest.mark.parametrize('e,nt,t,k,n,empty', [
+    (1, 1, 1, 64, 128, ()),            # one row, one expert, smallest legal widths
+    (6, 1, 1000, 128, 256, (2,)),      # expert-only grouping (the reference's), one expert without rows
+    (5, 3, 1500, 192, 384, (0, 4)),    # three tenants per expert: weights shared by consecutive groups
+    (16, 4, 6000, 256, 128, ()),       # experts with more than one 128-row block
+    (3, 2, 700, 64, 640, ()),
+])
+@pytest.mark.parametrize('map_rows', [True, False])
+def test_base_term_matches_the_per_expert_loop(dev, e, nt, t, k, n, empty, map_rows):
+    expert, tenant, x, w = _case(e, nt, t, k, n, seed=t + n, empty=empty)
+    keys = (expert * nt + tenant).to(torch.int32).to(dev)
+    seg = build_segments(keys, e * nt)
+    want = _reference(x, w, expert)
+    xd, wd = x.to(dev), w.to(dev)
+    if map_rows:
+        y = grouped_linear_(xd, wd, seg, nt, map_rows=True)
+        got = y
+    else:                                # rows already in segment order, as after permute()
+        perm = seg.perm
+        y = grouped_linear_(xd[perm].contiguous(), wd, seg, nt, map_rows=False)
+        got = torch.empty_like(y)
+        got[perm] = y
+    assert max_rel_err(got, want) < 2e-2
+    # bf16 rounding of an fp32 accumulation: far inside the bar
+    assert max_rel_err(got, want) < 6e-3
+
+
+@pytest.mark.parametrize('max_r,ranks', [(8, [8, 4, 8]), (16, [16, 0, 9]), (32, [32, 17, 8]), (64, [64, 40, 16])])
+def test_lora_term_in_the_epilogue(dev, max_r, ranks):
+    """y = x W_e^T + s (x A_{e,t}^T) B_{e,t}^T per (expert, tenant) segment: oracle's low-rank form per tenant."""
+    e, nt, t, k, n = 4, len(ranks), 1800, 256, 384
+    expert, tenant, x, w = _case(e, nt, t, k, n, seed=max_r)
+    keys = (expert * nt + tenant).to(torch.int32).to(dev)
+    seg = build_segments(keys, e * nt)
+    g = torch.Generator().manual_seed(3)
+    a = [(torch.randn(e, max_r, k, generator=g) / k**0.5).bfloat16().to(dev) for _ in range(nt)]
+    b = [(torch.randn(e, n, max_r, generator=g) * 0.05).bfloat16().to(dev) for _ in range(nt)]
+    idx = [i % nt for i in range(e * nt)]
+    # group i = expert i // nt, tenant i % nt: one block of the tenant's packed tensors (a rank-0 tenant is legal at
+    # the kernel boundary: its term is skipped)
+    groups = AdapterGroups(a, b, [ranks[i % nt] for i in range(e * nt)], [2.0] * (e * nt),
+                           a_index=idx, a_offset=[(i // nt) * max_r * k for i in range(e * nt)],
+                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)])
+    xd, wd = x.to(dev), w.to(dev)
+    h = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=dev)
+    lora_shrink_(xd, seg, groups, h, map_rows=True)
+    got = grouped_linear_(xd, wd, seg, nt, groups=groups, h=h, map_rows=True)
+    want = _reference(x, w, expert)
+    xs = x.double()
+    for ei in range(e):
+        for ti in range(nt):
+            rows = ((expert == ei) & (tenant == ti)).nonzero().flatten()
+            r = ranks[ti]
+            if rows.numel() == 0 or r == 0:
+                continue
+            want[rows] += 2.0 * (xs[rows] @ a[ti][ei, :r].double().cpu().t()) @ b[ti][ei, :, :r].double().cpu().t()
+    assert max_rel_err(got, want) < 2e-2
+
+
+def test_backward_of_the_base_term_is_the_same_call_on_transposed_weights(dev):
+    e, nt, t, k, n = 5, 2, 1200, 128, 256
+    expert, tenant, x, w = _case(e, nt, t, k, n, seed=9)
+    dy = torch.randn(t, n, generator=torch.Generator().manual_seed(10)).bfloat16()
+    keys = (expert * nt + tenant).to(torch.int32).to(dev)
+    seg = build_segments(keys, e * nt)
+    wt = w.transpose(1, 2).contiguous()                     # [E, in, out]: dx = dy W_e
+    got = grouped_linear_(dy.to(dev), wt.to(dev), seg, nt, map_rows=True)
+    want = _reference(dy, wt, expert)
+    assert max_rel_err(got, want) < 6e-3
+
+
+def test_unsupported_shapes_are_refused(dev):
+    e, nt, t = 2, 1, 64
+    keys = torch.zeros(t, dtype=torch.int32, device=dev)
+    seg = build_segments(keys, e * nt)
+    for k, n in [(96, 128), (64, 192), (32, 128)]:
+        x = torch.zeros(t, k, dtype=torch.bfloat16, device=dev)
+        w = torch.zeros(e, n, k, dtype=torch.bfloat16, device=dev)
+        with pytest.raises(ValueError):
+            grouped_linear_(x, w, seg, nt)
+    x = torch.zeros(t, 64, dtype=torch.float32, device=dev)
+    w = torch.zeros(e, 128, 64, dtype=torch.float32, device=dev)
+    with pytest.raises(ValueError):
+        grouped_linear_(x, w, seg, nt)                      # fp32: run the experts one by one
+    with pytest.raises(ValueError):
+        grouped_linear_(x.bfloat16(), w.bfloat16(), seg, 3)  # 2 experts x 3 tenants != 2 groups

@@ -124,6 +124,23 @@ def test_expert_merged_weight_equals_low_rank(out_in):
     assert torch.allclose(merged, low, atol=1e-12)
 
 
+def test_experts_linear_is_each_rows_own_expert():
+    """The chunk loop against a row-by-row product with each row's own expert (empty experts included), and
+    against one F.linear when there is a single expert."""
+    g = torch.Generator().manual_seed(5)
+    e, hid, out = 5, 6, 4
+    counts = [3, 0, 4, 1, 0]
+    offsets = torch.tensor([0, 3, 3, 7, 8, 8])
+    x = torch.randn(8, hid, generator=g, dtype=torch.double)
+    w = torch.randn(e, out, hid, generator=g, dtype=torch.double)
+    got = oracle.experts_linear(x, offsets, w)
+    expert_of_row = [i for i, c in enumerate(counts) for _ in range(c)]
+    want = torch.stack([sum(w[expert_of_row[i]][:, k] * x[i, k] for k in range(hid)) for i in range(8)])
+    assert got.shape == (8, out) and torch.allclose(got, want, atol=1e-12)
+    one = oracle.experts_linear(x, torch.tensor([0, 8]), w[:1])
+    assert torch.equal(one, F.linear(x, w[0]))
+
+
 def test_slice_copy_round_trip():
     g = torch.Generator().manual_seed(8)
     for name, shape, r in [('m.lora_A.weight', (8, 5), 3), ('m.lora_B.weight', (5, 8), 3),

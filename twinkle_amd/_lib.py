@@ -49,6 +49,23 @@ class LoraDesc(Structure):
     ]
 
 
+class GroupedDesc(Structure):
+    """Mirror of ``tk_grouped_desc``."""
+    _fields_ = [
+        ('rows', c_int64),
+        ('num_groups', c_int32),
+        ('groups_per_expert', c_int32),
+        ('in_features', c_int32),
+        ('out_features', c_int32),
+        ('dtype', c_int32),
+        ('map_rows', c_int32),
+        ('seg_ws', c_void_p),
+        ('weight', c_void_p),
+        ('weight_stride', c_int64),
+        ('ldw', c_int64),
+    ]
+
+
 EXPORTS = {
     'tk_version': (c_char_p, []),
     'tk_error_string': (c_char_p, [c_int32]),
@@ -73,6 +90,9 @@ EXPORTS = {
     'tk_lora_fwd_shared': (c_int32, [c_void_p, c_int32, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     'tk_lora_bwd_shared': (c_int32, [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
                                      c_int64, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p]),
+    'tk_grouped_linear_workspace_bytes': (c_int64, [POINTER(GroupedDesc)]),
+    'tk_grouped_linear': (c_int32, [POINTER(GroupedDesc), POINTER(LoraDesc), c_void_p, c_int64, c_void_p, c_int64,
+                                    c_void_p, c_void_p, c_int64, c_void_p]),
     'tk_opt_workspace_bytes': (c_int64, [c_int32, c_int64]),
     'tk_opt_grad_norm': (c_int32, [c_void_p, c_int32, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p,
                                    c_int64, c_void_p]),

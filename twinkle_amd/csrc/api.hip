@@ -368,6 +368,64 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
   return rc;
 }
 
+// ---- packed experts: grouped base GEMM (+ LoRA term) ---------------------------------------------------------------
+
+static bool grouped_desc_ok(const tk_grouped_desc* g) {
+  return g && g->rows >= 0 && g->num_groups > 0 && g->groups_per_expert > 0 &&
+         g->num_groups % g->groups_per_expert == 0 && g->in_features > 0 && g->out_features > 0;
+}
+
+struct GroupedLayout {
+  int64_t off_plan, off_count, total;
+  GroupedLayout(const tk_grouped_desc& g) {
+    SegLayout L(g.rows, g.num_groups);
+    int64_t o = 0;
+    off_count = o;  o += 256;
+    off_plan = o;   o += round_up(grouped_plan_entries(L, g.num_groups / g.groups_per_expert) * (int64_t)sizeof(GroupedPlanEntry), 256);
+    total = o;
+  }
+};
+
+int64_t tk_grouped_linear_workspace_bytes(const tk_grouped_desc* g) {
+  if (!grouped_desc_ok(g)) return TK_ERR_INVALID;
+  return GroupedLayout(*g).total;
+}
+
+int tk_grouped_linear(const tk_grouped_desc* g, const tk_lora_desc* lora, const void* x, int64_t ldx, void* y,
+                      int64_t ldy, const void* h, void* ws, int64_t ws_bytes, tk_stream_t stream) {
+  if (!grouped_desc_ok(g) || !g->seg_ws || !g->weight_device) return TK_ERR_INVALID;
+  if (g->rows == 0) return TK_OK;
+  if (!x || !y || !ws || ldx < g->in_features || ldy < g->out_features || g->ldw < g->in_features)
+    return TK_ERR_INVALID;
+  if (g->weight_stride < (int64_t)(g->out_features - 1) * g->ldw + g->in_features) return TK_ERR_INVALID;
+  const GroupedLayout W(*g);
+  if (ws_bytes < W.total) return TK_ERR_WORKSPACE;
+  if (g->dtype != TK_DTYPE_BF16 || force_generic()) return TK_ERR_UNSUPPORTED;
+  GroupedArgs a{};
+  a.x = (const uint16_t*)x;  a.ldx = ldx;
+  a.w = (const uint16_t*)g->weight_device;  a.w_stride = g->weight_stride;  a.ldw = g->ldw;
+  a.y = (uint16_t*)y;  a.ldy = ldy;
+  a.K = g->in_features;  a.N = g->out_features;  a.src_rows = (int32_t)g->rows;  a.map_rows = g->map_rows;
+  if (lora && lora->max_rank > 0) {
+    if (!desc_ok(lora) || !h) return TK_ERR_INVALID;
+    if (lora->rows != g->rows || lora->num_groups != g->num_groups || lora->in_features != g->in_features ||
+        lora->out_features != g->out_features || lora->dtype != g->dtype || lora->seg_ws != g->seg_ws ||
+        lora->map_rows != g->map_rows)
+      return TK_ERR_INVALID;
+    if (lora->max_rank > 64) return TK_ERR_UNSUPPORTED;
+    a.rpad = rank_pad(lora->max_rank);
+    a.lora_B = lora->lora_B;  a.ldb = lora->ldb;  a.rank = lora->rank;
+    a.hrow = (const uint16_t*)h + (int64_t)a.rpad * h_ld(g->rows, g->num_groups);  // slot-major half of h
+  }
+  if (!grouped_gemm_supported(a)) return TK_ERR_UNSUPPORTED;
+  SegLayout L(g->rows, g->num_groups);
+  SegView V(g->seg_ws, L);
+  char* w = (char*)ws;
+  return launch_grouped_gemm(a, g->num_groups / g->groups_per_expert, g->groups_per_expert,
+                             (GroupedPlanEntry*)(w + W.off_plan), (int32_t*)(w + W.off_count), V, L,
+                             (hipStream_t)stream);
+}
+
 // ---- projections that share their input ------------------------------------------------------------------------
 
 static bool shared_descs_ok(const tk_lora_desc* const* descs, int32_t n) {

@@ -288,6 +288,25 @@ int launch_shrink_shared(const SharedShrinkArgs& a, const SegView& seg, const Se
 int launch_expand_shared(const SharedExpandArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
 int launch_wgrad_shared(const SharedWgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
 
+// kernels_grouped.hip
+struct GroupedPlanEntry {  // a row block of the grouped GEMM: up to 4 consecutive tiles of one expert
+  int32_t tile0, ntiles, expert, pad;
+};
+struct GroupedArgs {
+  const uint16_t* x;  int64_t ldx;                     // activations, rows reached through the slot table
+  const uint16_t* w;  int64_t w_stride, ldw;           // packed weights: expert e at w + e * w_stride, [N][K]
+  uint16_t* y;        int64_t ldy;
+  int32_t K, N, src_rows, map_rows;
+  // LoRA term (rpad = 0: none): y += h B_g^T with h[slot][rpad] as the shrink kernels leave it
+  const void* const* lora_B;  int64_t ldb;
+  const int32_t* rank;  int32_t rpad;
+  const uint16_t* hrow;
+};
+bool grouped_gemm_supported(const GroupedArgs& a);
+int64_t grouped_plan_entries(const SegLayout& L, int64_t experts);
+int launch_grouped_gemm(const GroupedArgs& a, int experts, int nt, GroupedPlanEntry* plan, int32_t* nblocks,
+                        const SegView& seg, const SegLayout& L, hipStream_t s);
+
 // kernels_segments.hip
 int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t groups, int64_t* perm_out,
                          int64_t* offsets_out, void* ws, hipStream_t s);

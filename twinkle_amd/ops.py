@@ -249,6 +249,50 @@ def lora_bwd_(dy: torch.Tensor, x: Optional[torch.Tensor], h: Optional[torch.Ten
     _lib.check(code, 'tk_lora_bwd')
 
 
+def grouped_linear_(x: torch.Tensor, weight: torch.Tensor, seg: SegmentTable, groups_per_expert: int = 1,
+                    y: Optional[torch.Tensor] = None, groups: Optional[AdapterGroups] = None,
+                    h: Optional[torch.Tensor] = None, map_rows: bool = False,
+                    workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``y[row] = x[row] @ weight[e].T (+ h[row] @ B_g.T)`` for every row of the table, ``e = g // groups_per_expert``
+    (see ``tk_grouped_linear``).  ``weight`` is packed ``[E, out, in]``; with ``groups`` the LoRA term of the
+    (expert, tenant) groups is added on the accumulators, from ``h`` as :func:`lora_shrink_` left it."""
+    if not (x.is_cuda and weight.is_cuda):
+        raise RuntimeError('x and weight must live on the GPU: this path has no CPU implementation')
+    if weight.dim() != 3 or weight.stride(2) != 1 or weight.dtype != x.dtype:
+        raise ValueError('weight must be [experts, out, in] with unit inner stride and the dtype of x')
+    experts, out_f, in_f = weight.shape
+    if seg.num_groups != experts * groups_per_expert:
+        raise ValueError(f'segment table has {seg.num_groups} groups, weights give {experts} x {groups_per_expert}')
+    _check_rows(x, 'x', seg.rows, in_f, weight.dtype)
+    if y is None:
+        y = torch.empty(seg.rows, out_f, dtype=x.dtype, device=x.device)
+    _check_rows(y, 'y', seg.rows, out_f, weight.dtype)
+    g = _lib.GroupedDesc()
+    g.rows, g.num_groups, g.groups_per_expert = seg.rows, seg.num_groups, groups_per_expert
+    g.in_features, g.out_features = in_f, out_f
+    g.dtype = _lib.dtype_code(weight.dtype)
+    g.map_rows = 1 if map_rows else 0
+    g.seg_ws = seg.workspace.data_ptr()
+    g.weight, g.weight_stride, g.ldw = weight.data_ptr(), weight.stride(0), weight.stride(1)
+    lib = _lib.load()
+    if workspace is None:
+        n = lib.tk_grouped_linear_workspace_bytes(ctypes.byref(g))
+        _lib.check(n, 'tk_grouped_linear_workspace_bytes')
+        workspace = torch.empty(n, dtype=torch.uint8, device=x.device)
+    d = None
+    if groups is not None:
+        if h is None:
+            raise ValueError('the LoRA term needs the h that lora_shrink_ wrote')
+        if groups.num_groups != seg.num_groups or groups.in_features != in_f or groups.out_features != out_f:
+            raise ValueError('adapters and weights describe different layers')
+        d = ctypes.byref(_desc(seg, groups, map_rows))
+    code = lib.tk_grouped_linear(ctypes.byref(g), d, x.data_ptr(), x.stride(0), y.data_ptr(), y.stride(0),
+                                 h.data_ptr() if h is not None else None, workspace.data_ptr(), workspace.numel(),
+                                 _lib.stream_ptr())
+    _lib.check(code, 'tk_grouped_linear')
+    return y
+
+
 def _weight_grads(ctx_groups: AdapterGroups, needs_a: bool, needs_b: bool, device):
     groups = ctx_groups
     arena_a = arena_b = pa = pb = None
