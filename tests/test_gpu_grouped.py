@@ -119,3 +119,57 @@ def test_unsupported_shapes_are_refused(dev):
         grouped_linear_(x, w, seg, nt)                      # fp32: run the experts one by one
     with pytest.raises(ValueError):
         grouped_linear_(x.bfloat16(), w.bfloat16(), seg, 3)  # 2 experts x 3 tenants != 2 groups
+
+
+def test_experts_forward_grouped_equals_the_per_expert_loop(dev):
+    """experts_forward with the grouped GEMMs (the default for frozen bf16 weights of these widths) against its
+    per-expert loop (the reference's form, checked against the float64 restatement elsewhere): outputs, dx and
+    every tenant's adapter gradients."""
+    from twinkle_amd import LoraConfig
+    from twinkle_amd.expert_lora import ExpertLoraSlots, experts_forward
+    torch.manual_seed(0)
+    e, nt, hid, inter, t = 6, 2, 128, 256, 1400
+
+    class Experts(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.gate_up_proj = torch.nn.Parameter((torch.randn(e, 2 * inter, hid) * 0.08).bfloat16(),
+                                                   requires_grad=False)
+            self.down_proj = torch.nn.Parameter((torch.randn(e, hid, inter) * 0.08).bfloat16(), requires_grad=False)
+            self.act_fn = torch.nn.functional.silu
+
+    experts = Experts().to(dev)
+    names = ['lora_0', 'lora_1']
+    gu = ExpertLoraSlots(e, hid, 2 * inter, max_loras=2, max_r=16, dtype=torch.bfloat16, device=dev)
+    dn = ExpertLoraSlots(e, inter, hid, max_loras=2, max_r=16, dtype=torch.bfloat16, device=dev)
+    for slots in (gu, dn):
+        for name, r in zip(names, (16, 6)):
+            slots.configure_slot(name, LoraConfig(r=r, lora_alpha=2 * r))
+            with torch.no_grad():
+                slots.lora_B[name].normal_(0, 0.05)
+    g = torch.Generator().manual_seed(2)
+    expert = torch.multinomial(torch.tensor([1.0, 0.2, 0.0, 2.0, 1.0, 0.5]), t, replacement=True, generator=g)
+    tenant = torch.randint(0, nt, (t,), generator=g)
+    keys = torch.sort(expert * nt + tenant).values.to(torch.int32).to(dev)      # rows already in segment order
+    seg = build_segments(keys, e * nt)
+    x0 = torch.randn(t, hid, generator=g).bfloat16().to(dev)
+    dy = torch.randn(t, hid, generator=g).bfloat16().to(dev)
+
+    def run(grouped):
+        for slots in (gu, dn):
+            for p in slots.parameters():
+                p.grad = None
+        x = x0.clone().requires_grad_(True)
+        y = experts_forward(experts, x, seg, names, gu, dn, grouped=grouped)
+        y.backward(dy)
+        grads = [slots.lora_A[n].grad.clone() for slots in (gu, dn) for n in names] + \
+                [slots.lora_B[n].grad.clone() for slots in (gu, dn) for n in names]
+        return [y.detach(), x.grad] + grads
+
+    loop, fused = run(False), run(True)
+    default = run(None)
+    for a, b in zip(fused, default):
+        assert torch.equal(a, b), 'grouped is the default for these shapes'
+    for i, (a, b) in enumerate(zip(fused, loop)):
+        assert max_rel_err(a, b.double().cpu()) < 2e-2, i
+    assert experts.gate_up_proj.grad is None and experts.down_proj.grad is None

@@ -16,6 +16,7 @@
 // wave owns 64 x 64 as 4 x 4 MFMA 16x16x32 tiles.  The weight fragment is the MFMA A operand and the x fragment
 // the B operand, so a lane ends up with four consecutive output columns of one row.
 #include <algorithm>
+#include <type_traits>
 
 #include "tk_mfma.h"
 
@@ -25,6 +26,10 @@ namespace {
 
 constexpr int kGBM = 128, kGBN = 128, kGBK = 64, kGLS = kGBK + 8;
 constexpr int kPlanTiles = kGBM / kTileRows;  // tiles per row block
+#ifndef TK_GROUPED_ITEMS
+#define TK_GROUPED_ITEMS 6144
+#endif
+constexpr int kGroupedItems = TK_GROUPED_ITEMS;  // work items aimed at per launch
 
 __global__ __launch_bounds__(256) void k_grouped_plan(const int32_t* __restrict__ tile_first, int experts, int nt,
                                                       GroupedPlanEntry* __restrict__ plan,
@@ -55,15 +60,19 @@ __global__ __launch_bounds__(256) void k_grouped_plan(const int32_t* __restrict_
 
 // NKS: MFMA steps of the LoRA term (0: none; 1: padded rank 16 or 32; 2: padded rank 64)
 template <int NKS>
-__global__ __launch_bounds__(256) void k_grouped_gemm(GroupedArgs a, const GroupedPlanEntry* __restrict__ plan,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k_grouped_gemm(GroupedArgs a, const GroupedPlanEntry* __restrict__ plan,
                                                       const int32_t* __restrict__ nblocks,
                                                       const int32_t* __restrict__ tile_group,
-                                                      const int32_t* __restrict__ slot_rows) {
+                                                      const int32_t* __restrict__ slot_rows, int nsplit, int cpi) {
   __shared__ __attribute__((aligned(16))) bf16_t As[2][kGBM * kGLS];  // x rows
   __shared__ __attribute__((aligned(16))) bf16_t Bs[2][kGBN * kGLS];  // weight rows
-  const int blocks = *nblocks;
+  // work item = (row block, run of cpi column blocks); the items of a row block and then of its expert's other row
+  // blocks are neighbours and reach one XCD together
+  const int blocks = *nblocks * nsplit;
   if ((int)blockIdx.x >= blocks) return;
-  const GroupedPlanEntry pe = plan[xcd_contiguous(blockIdx.x, blocks)];
+  const int item = xcd_contiguous(blockIdx.x, blocks);
+  const GroupedPlanEntry pe = plan[item / nsplit];
+  const int nb_first = (item % nsplit) * cpi, nb_last = min(nb_first + cpi, a.N / kGBN);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
   const int wm = wave >> 1, wn = wave & 1;
   const int slot0 = pe.tile0 * kTileRows, live = pe.ntiles * kTileRows;
@@ -89,7 +98,7 @@ __global__ __launch_bounds__(256) void k_grouped_gemm(GroupedArgs a, const Group
   const int nk = a.K / kGBK;
   const int ldsw = lrow * kGLS + lchunk;  // + 32 i rows
 
-  for (int nb = 0; nb < a.N / kGBN; ++nb) {
+  for (int nb = nb_first; nb < nb_last; ++nb) {
     const bf16_t* wp[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) wp[i] = wbase + (int64_t)(nb * kGBN + lrow + 32 * i) * a.ldw + lchunk;
@@ -99,29 +108,27 @@ __global__ __launch_bounds__(256) void k_grouped_gemm(GroupedArgs a, const Group
 #pragma unroll
       for (int cb = 0; cb < 4; ++cb) acc[rb][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    uint4 gx[4], gw[4];
+    // Two register sets: the loads of step ks + 2 are issued before step ks is computed and wait in registers
+    // across one barrier (which orders LDS traffic only), so a load has two steps of MFMA work to arrive.
+    uint4 gx[2][4], gw[2][4];
+    auto fetch = [&](int ks, auto set) {
+      const int k0 = ks * kGBK;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      gx[i] = ld16(xp[i]);
-      gw[i] = ld16(wp[i]);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      st16(&As[0][ldsw + 32 * i * kGLS], gx[i]);
-      st16(&Bs[0][ldsw + 32 * i * kGLS], gw[i]);
-    }
-    __syncthreads();
-    for (int ks = 0; ks < nk; ++ks) {
-      const int cur = ks & 1;
-      const bool more = ks + 1 < nk;
-      if (more) {
-        const int k1 = (ks + 1) * kGBK;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          gx[i] = ld16(xp[i] + k1);
-          gw[i] = ld16(wp[i] + k1);
-        }
+      for (int i = 0; i < 4; ++i) {
+        gx[set][i] = ld16(xp[i] + k0);
+        gw[set][i] = ld16(wp[i] + k0);
       }
+    };
+    auto stash = [&](int buf, auto set) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        st16(&As[buf][ldsw + 32 * i * kGLS], gx[set][i]);
+        st16(&Bs[buf][ldsw + 32 * i * kGLS], gw[set][i]);
+      }
+    };
+    auto step = [&](int ks, auto parity) {  // parity = ks & 1 as a compile-time constant
+      constexpr int cur = decltype(parity)::value;
+      if (ks + 2 < nk) fetch(ks + 2, std::integral_constant<int, cur>{});
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         uint4 fx[4], fw[4];
@@ -134,14 +141,16 @@ __global__ __launch_bounds__(256) void k_grouped_gemm(GroupedArgs a, const Group
 #pragma unroll
           for (int cb = 0; cb < 4; ++cb) acc[rb][cb] = mfma16(fw[cb], fx[rb], acc[rb][cb]);
       }
-      if (more) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          st16(&As[cur ^ 1][ldsw + 32 * i * kGLS], gx[i]);
-          st16(&Bs[cur ^ 1][ldsw + 32 * i * kGLS], gw[i]);
-        }
-      }
-      __syncthreads();
+      if (ks + 1 < nk) stash(cur ^ 1, std::integral_constant<int, cur ^ 1>{});
+      lds_barrier();
+    };
+    fetch(0, std::integral_constant<int, 0>{});
+    if (nk > 1) fetch(1, std::integral_constant<int, 1>{});
+    stash(0, std::integral_constant<int, 0>{});
+    lds_barrier();
+    for (int ks = 0; ks < nk; ks += 2) {
+      step(ks, std::integral_constant<int, 0>{});
+      if (ks + 1 < nk) step(ks + 1, std::integral_constant<int, 1>{});
     }
 
     if constexpr (NKS > 0) {
@@ -210,13 +219,18 @@ int launch_grouped_gemm(const GroupedArgs& a, int experts, int nt, GroupedPlanEn
   const int max_entries = (int)grouped_plan_entries(L, experts);
   hipLaunchKernelGGL(k_grouped_plan, dim3(1), dim3(256), 0, s, seg.tile_first, experts, nt, plan, nblocks, max_entries);
   const int32_t* rows = seg.slot_table(a.map_rows);
-  const dim3 grid((unsigned)max_entries);
+  // several thousand work items, so that the last round of blocks on the 256 CUs is a small part of the run
+  const int ncb = a.N / kGBN;
+  const int64_t row_blocks = ceil_div(L.max_tiles, kPlanTiles);
+  const int cpi = (int)std::min<int64_t>(ncb, std::max<int64_t>(1, ceil_div(ncb * row_blocks, kGroupedItems)));
+  const int nsplit = (int)ceil_div(ncb, cpi);
+  const dim3 grid((unsigned)((int64_t)max_entries * nsplit));
   if (a.rpad == 0)
-    hipLaunchKernelGGL(k_grouped_gemm<0>, grid, dim3(256), 0, s, a, plan, nblocks, seg.tile_group, rows);
+    hipLaunchKernelGGL(k_grouped_gemm<0>, grid, dim3(256), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit, cpi);
   else if (a.rpad <= 32)
-    hipLaunchKernelGGL(k_grouped_gemm<1>, grid, dim3(256), 0, s, a, plan, nblocks, seg.tile_group, rows);
+    hipLaunchKernelGGL(k_grouped_gemm<1>, grid, dim3(256), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit, cpi);
   else
-    hipLaunchKernelGGL(k_grouped_gemm<2>, grid, dim3(256), 0, s, a, plan, nblocks, seg.tile_group, rows);
+    hipLaunchKernelGGL(k_grouped_gemm<2>, grid, dim3(256), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit, cpi);
   return check_launch();
 }
 

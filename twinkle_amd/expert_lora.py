@@ -277,9 +277,29 @@ class ExpertLoraManager:
         return consumed
 
 
+def _transposed_copy(experts_mod: nn.Module, name: str) -> torch.Tensor:
+    """``[E, in, out]`` copy of the frozen packed weight ``name`` (kept on the module, redone if the weight changed):
+    the backward of the grouped GEMM is the same kernel on this copy."""
+    weight = getattr(experts_mod, name)
+    cache = experts_mod.__dict__.setdefault('_tk_transposed', {})
+    hit = cache.get(name)
+    if hit is None or hit[0] != (weight.data_ptr(), weight._version, tuple(weight.shape)):
+        with torch.no_grad():
+            hit = ((weight.data_ptr(), weight._version, tuple(weight.shape)), weight.transpose(1, 2).contiguous())
+        cache[name] = hit
+    return hit[1]
+
+
+def grouped_gemm_applies(weight: torch.Tensor, rows: torch.Tensor) -> bool:
+    """Frozen bf16 packed weights whose two widths are multiples of 128: what ``tk_grouped_linear`` takes in the
+    forward direction (``in`` a multiple of 64, ``out`` of 128) and, on the transposed copy, in the backward one."""
+    return (weight.dtype == torch.bfloat16 and rows.dtype == torch.bfloat16 and weight.is_contiguous() and
+            not weight.requires_grad and weight.shape[1] % 128 == 0 and weight.shape[2] % 128 == 0)
+
+
 def experts_forward(experts_mod: nn.Module, rows: torch.Tensor, seg: SegmentTable, tenant_slots: Sequence[str],
                     gate_up_slots: Optional[ExpertLoraSlots] = None,
-                    down_slots: Optional[ExpertLoraSlots] = None) -> torch.Tensor:
+                    down_slots: Optional[ExpertLoraSlots] = None, grouped: Optional[bool] = None) -> torch.Tensor:
     """Packed experts on rows in (expert, tenant) segment order, every tenant's LoRA terms included.
 
     The per-expert loop of the reference's expert forward (moe/expert_parallel.py:333-378: ``F.linear`` with
@@ -289,17 +309,40 @@ def experts_forward(experts_mod: nn.Module, rows: torch.Tensor, seg: SegmentTabl
     segmented kernels instead of being merged into the weights.  ``seg`` was built from keys
     ``expert * len(tenant_slots) + tenant`` with ``want_offsets=True``; ``experts_mod`` holds
     ``gate_up_proj [E, 2 I, H]`` and ``down_proj [E, H, I]`` and either ``_apply_gate`` or ``act_fn``.
+
+    ``grouped`` (default: whenever the shapes allow, i.e. frozen bf16 weights with widths that are multiples of
+    64 / 128 in both directions) replaces the loop by one grouped GEMM per projection with the LoRA terms in its
+    epilogue: no host copy of the boundaries at all, one launch instead of one per expert, and the expert outputs
+    are written once.  Its backward runs the same kernel on a transposed copy of the frozen weights.
     """
     if rows.shape[0] == 0:
         return rows                                                   # keeps the autograd edge (reference :340-344)
     nt = len(tenant_slots)
     gate_up, down = experts_mod.gate_up_proj, experts_mod.down_proj
     experts = gate_up.shape[0]
-    if seg.num_groups != experts * nt or seg.offsets is None:
-        raise ValueError('the segment table must hold offsets for expert * num_tenants + tenant keys')
-    bounds = seg.offsets[::nt].tolist()                               # first sorted position of every expert
+    if seg.num_groups != experts * nt:
+        raise ValueError('the segment table must be built from expert * num_tenants + tenant keys')
     input_dtype = rows.dtype
     x = rows if rows.dtype == gate_up.dtype else rows.to(gate_up.dtype)
+    can_group = x.is_cuda and grouped_gemm_applies(gate_up, x) and grouped_gemm_applies(down, x)
+    if grouped and not can_group:
+        raise ValueError('grouped=True needs frozen bf16 expert weights with widths that are multiples of 128')
+    if grouped or (grouped is None and can_group):
+        from .ops import grouped_experts_linear
+        x = x.contiguous()
+        gate_up_out = grouped_experts_linear(x, gate_up, _transposed_copy(experts_mod, 'gate_up_proj'), seg, nt,
+                                             gate_up_slots.groups(tenant_slots) if gate_up_slots is not None else None)
+        if hasattr(experts_mod, '_apply_gate'):
+            hidden = experts_mod._apply_gate(gate_up_out)
+        else:
+            gate, up = gate_up_out.chunk(2, dim=-1)
+            hidden = experts_mod.act_fn(gate) * up
+        out = grouped_experts_linear(hidden.contiguous(), down, _transposed_copy(experts_mod, 'down_proj'), seg, nt,
+                                     down_slots.groups(tenant_slots) if down_slots is not None else None)
+        return out if out.dtype == input_dtype else out.to(input_dtype)
+    if seg.offsets is None:
+        raise ValueError('the per-expert loop needs a segment table built with want_offsets=True')
+    bounds = seg.offsets[::nt].tolist()                               # first sorted position of every expert
 
     def per_expert(inp, weight):
         chunks = [torch.nn.functional.linear(inp[bounds[e]:bounds[e + 1]], weight[e]) for e in range(experts)

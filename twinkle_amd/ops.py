@@ -362,6 +362,54 @@ class _LoraLinear(torch.autograd.Function):
         return (dx, dw, db, None, None, None, *ga, *gb)
 
 
+class _GroupedExpertsLinear(torch.autograd.Function):
+    """Frozen packed expert weights and the (expert, tenant) LoRA terms as one node on rows in segment order.
+
+    Forward: shrink, then the grouped GEMM with the LoRA term in its epilogue.  Backward: the same grouped GEMM on
+    the transposed weights gives the base part of ``dx``; the segmented backward adds the LoRA part onto it in place
+    and yields the adapters' gradients.  The weights get no gradient (the reference freezes them)."""
+
+    @staticmethod
+    def forward(ctx, x, weight, weight_t, seg, groups_per_expert, groups, *weights):
+        h = None
+        if groups is not None:
+            h = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=x.device)
+            lora_shrink_(x, seg, groups, h, map_rows=False)
+        y = grouped_linear_(x, weight, seg, groups_per_expert, groups=groups, h=h, map_rows=False)
+        ctx.save_for_backward(x, weight_t, h)
+        ctx.seg, ctx.groups, ctx.groups_per_expert = seg, groups, groups_per_expert
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight_t, h = ctx.saved_tensors
+        seg, groups = ctx.seg, ctx.groups
+        dy = dy.contiguous()
+        needs_dx = ctx.needs_input_grad[0]
+        dx = grouped_linear_(dy, weight_t, seg, ctx.groups_per_expert, map_rows=False) if needs_dx else None
+        if groups is None:
+            return (dx, None, None, None, None, None)
+        na, nb = len(groups.a_tensors), len(groups.b_tensors)
+        needs_a = any(ctx.needs_input_grad[6:6 + na])
+        needs_b = any(ctx.needs_input_grad[6 + na:6 + na + nb])
+        arena_a, arena_b, pa, pb = _weight_grads(groups, needs_a, needs_b, dy.device)
+        if needs_dx or needs_a or needs_b:
+            lora_bwd_(dy, x, h, dx, pa, pb, seg, groups, False, accumulate=False)
+        ga = groups.grad_views(arena_a, 'a') if needs_a else [None] * na
+        gb = groups.grad_views(arena_b, 'b') if needs_b else [None] * nb
+        return (dx, None, None, None, None, None, *ga, *gb)
+
+
+def grouped_experts_linear(x: torch.Tensor, weight: torch.Tensor, weight_t: torch.Tensor, seg: SegmentTable,
+                           groups_per_expert: int, groups: Optional[AdapterGroups] = None) -> torch.Tensor:
+    """``y = x W_e^T`` plus every (expert, tenant) group's LoRA term, for rows in segment order; differentiable in
+    ``x`` and the adapters.  ``weight_t`` is the ``[E, in, out]`` copy of the frozen ``weight [E, out, in]``."""
+    extra = groups.autograd_tensors() if groups is not None else []
+    if groups is not None:
+        groups.sync_masters()
+    return _GroupedExpertsLinear.apply(x, weight, weight_t, seg, groups_per_expert, groups, *extra)
+
+
 def multi_lora_delta(x: torch.Tensor, base_out: torch.Tensor, seg: SegmentTable, groups: AdapterGroups,
                      map_rows: bool = True) -> torch.Tensor:
     """``base_out`` with every adapter's LoRA term added to its own rows (in place, differentiable)."""
