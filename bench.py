@@ -217,6 +217,83 @@ def shared_qkv_bench(dev, steps=20, calibrate_copy=False):
     return res
 
 
+def moe_experts_bench(dev, steps=10):
+    """BASELINE config 4 as a whole expert block: 8192 tokens x top-8 of 128 experts (65536 routed rows in
+    (expert, tenant) order), experts 2048 -> 2 x 768 -> 2048, 4 tenants with rank-8 LoRA on both packed
+    parameters, bf16.  experts_forward with the reference's per-expert loop for the frozen weights (plus the
+    segmented LoRA kernels) against the grouped GEMMs with the LoRA term in their epilogue; forward alone and
+    forward + backward (dx and the adapters' gradients; the frozen weights get none)."""
+    import torch
+    from twinkle_amd import LoraConfig, build_segments, flat_keys_from_topk, grouped_linear_, workloads
+    from twinkle_amd.expert_lora import ExpertLoraSlots, experts_forward
+    sel, _, tenant = workloads.moe_routing()
+    tokens, top_k = sel.shape
+    e, hid, inter, nt = 128, 2048, 768, 4
+    dt = torch.bfloat16
+
+    class Experts(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            g = torch.Generator().manual_seed(3)
+            self.gate_up_proj = torch.nn.Parameter((torch.randn(e, 2 * inter, hid, generator=g) * 0.02).to(dt),
+                                                   requires_grad=False)
+            self.down_proj = torch.nn.Parameter((torch.randn(e, hid, inter, generator=g) * 0.02).to(dt),
+                                                requires_grad=False)
+            self.act_fn = torch.nn.functional.silu
+
+    experts = Experts().to(dev)
+    names = [f'lora_{i}' for i in range(nt)]
+    gu = ExpertLoraSlots(e, hid, 2 * inter, max_loras=nt, max_r=8, dtype=dt, device=dev)
+    dn = ExpertLoraSlots(e, inter, hid, max_loras=nt, max_r=8, dtype=dt, device=dev)
+    for slots in (gu, dn):
+        for name in names:
+            slots.configure_slot(name, LoraConfig(r=8, lora_alpha=16))
+            with torch.no_grad():
+                slots.lora_B[name].normal_(0, 0.02)
+    keys = flat_keys_from_topk(sel.to(dev), tenant.to(dev), nt)
+    seg = build_segments(keys, e * nt, num_tokens=tokens)
+    rows = tokens * top_k
+    gen = torch.Generator().manual_seed(4)
+    x0 = torch.randn(rows, hid, generator=gen).to(dt).to(dev)
+    dy = torch.randn(rows, hid, generator=gen).to(dt).to(dev)
+
+    def fwd(grouped):
+        with torch.no_grad():
+            experts_forward(experts, x0, seg, names, gu, dn, grouped=grouped)
+
+    def fwd_bwd(grouped):
+        x = x0.detach().requires_grad_(True)
+        y = experts_forward(experts, x, seg, names, gu, dn, grouped=grouped)
+        y.backward(dy)
+
+    def base_only():
+        y = grouped_linear_(x0, experts.gate_up_proj, seg, nt)
+        grouped_linear_(y[:, :inter].contiguous(), experts.down_proj, seg, nt)
+
+    res = {}
+    for name, fn in (('loop_fwd_ms', lambda: fwd(False)), ('grouped_fwd_ms', lambda: fwd(True)),
+                     ('loop_fwd_bwd_ms', lambda: fwd_bwd(False)), ('grouped_fwd_bwd_ms', lambda: fwd_bwd(True)),
+                     ('grouped_gemms_alone_ms', base_only)):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        res[name] = (time.perf_counter() - t0) * 1e3 / steps
+    flops_fwd = 2 * rows * hid * (2 * inter) + 2 * rows * inter * hid       # the two base GEMMs
+    res.update({'workload': f'{tokens} tokens x top-{top_k} of {e} experts, {hid} -> 2x{inter} -> {hid}, {nt} tenants '
+                            'rank 8 on gate_up and down, bf16, rows in (expert, tenant) order',
+                'base_gemm_flops_fwd': flops_fwd,
+                'grouped_gemms_alone_tflops': flops_fwd / (res['grouped_gemms_alone_ms'] * 1e-3) / 1e12,
+                'mfma_frac_grouped_gemms': flops_fwd / (res['grouped_gemms_alone_ms'] * 1e-3) / 1e12 / 2500.0,
+                'speedup_fwd': res['loop_fwd_ms'] / res['grouped_fwd_ms'],
+                'speedup_fwd_bwd': res['loop_fwd_bwd_ms'] / res['grouped_fwd_bwd_ms'],
+                'routed_rows_per_s_fwd_bwd': rows / (res['grouped_fwd_bwd_ms'] * 1e-3)})
+    return res
+
+
 def cfg5_layer_bench(dev, steps=5):
     """The seven projections of one Llama-3-8B-shaped layer (4096 hidden, 1024 k/v, 14336 intermediate) with LoRA
     rank 64 on all of them, 8 tenants, one per packed 4096-token sequence (T = 32768), bf16: forward + backward
@@ -425,6 +502,8 @@ def main():
     ap.add_argument('--stack-cfg5', action='store_true',
                     help='run only the Llama-3-8B-shaped stack of BASELINE config 5 (see --layers)')
     ap.add_argument('--layers', type=int, default=32)
+    ap.add_argument('--moe-experts', action='store_true',
+                    help='run only the expert block of BASELINE config 4: per-expert loop against the grouped GEMMs')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run five plain 128 MiB device copies (a known-size kernel to scale rocprofv3 --pmc '
                          'FETCH_SIZE / WRITE_SIZE readings by)')
@@ -450,6 +529,9 @@ def main():
         return
     if args.layer_cfg5:
         print(json.dumps({'cfg5_layer': cfg5_layer_bench(dev)}))
+        return
+    if args.moe_experts:
+        print(json.dumps({'moe_experts': moe_experts_bench(dev)}))
         return
     if args.shared_qkv:
         print(json.dumps({'shared_qkv': shared_qkv_bench(dev, calibrate_copy=args.calibrate_copy)}))

@@ -119,6 +119,16 @@ class ExpertLoraSlots(nn.Module):
     def groups(self, tenant_slots: Sequence[str]) -> AdapterGroups:
         """Group table for keys ``expert * len(tenant_slots) + tenant``: one block of a slot tensor per group."""
         nt = len(tenant_slots)
+        # building the table costs a few host-to-device copies: kept until a slot's rank or scaling changes (moved
+        # parameter storage is picked up by AdapterGroups.refresh at every call)
+        key = (tuple(tenant_slots), tuple(self.r[s] for s in tenant_slots),
+               tuple(self.scaling[s] for s in tenant_slots))
+        cache = self.__dict__.setdefault('_groups_cache', {})
+        hit = cache.get(key)
+        if hit is not None and all(x is y for x, y in zip(hit.a_tensors + hit.b_tensors,
+                                                           [self.lora_A[s] for s in tenant_slots] +
+                                                           [self.lora_B[s] for s in tenant_slots])):
+            return hit
         a = [self.lora_A[s] for s in tenant_slots]
         b = [self.lora_B[s] for s in tenant_slots]
         n = self.num_experts * nt
@@ -127,7 +137,10 @@ class ExpertLoraSlots(nn.Module):
         b_off = [(i // nt) * self.out_features * self.max_r for i in range(n)]
         ranks = [self.r[tenant_slots[i % nt]] for i in range(n)]
         scales = [self.scaling[tenant_slots[i % nt]] for i in range(n)]
-        return AdapterGroups(a, b, ranks, scales, a_index=idx, a_offset=a_off, b_index=idx, b_offset=b_off)
+        if len(cache) > 16:
+            cache.clear()
+        cache[key] = AdapterGroups(a, b, ranks, scales, a_index=idx, a_offset=a_off, b_index=idx, b_offset=b_off)
+        return cache[key]
 
 
 def expert_lora_delta(x_sorted: torch.Tensor, y_sorted: torch.Tensor, seg: SegmentTable, slots: ExpertLoraSlots,
