@@ -531,7 +531,7 @@ def main():
         print(json.dumps({'cfg5_layer': cfg5_layer_bench(dev)}))
         return
     if args.moe_experts:
-        print(json.dumps({'moe_experts': moe_experts_bench(dev)}))
+        print(json.dumps({'moe_experts': moe_experts_bench(dev, steps=max(1, min(args.steps, 10)))}))
         return
     if args.shared_qkv:
         print(json.dumps({'shared_qkv': shared_qkv_bench(dev, calibrate_copy=args.calibrate_copy)}))
