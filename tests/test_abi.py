@@ -133,6 +133,29 @@ def test_entry_points_reject_malformed_arguments_on_the_host():
     assert lib.tk_lora_fwd(ref, P, 256, P, 128, P, None) == bad                              # lda below in_features
     d.lda, d.dtype = 256, 5
     assert lib.tk_lora_h_bytes(ref) == bad                                                   # unknown dtype
+    # grouped expert GEMM
+    g = _lib.GroupedDesc()
+    g.rows, g.num_groups, g.groups_per_expert, g.in_features, g.out_features = 64, 4, 2, 128, 256
+    g.dtype, g.map_rows, g.weight_stride, g.ldw = 1, 0, 256 * 128, 128
+    g.seg_ws = g.weight = P
+    gref = ctypes.byref(g)
+    need = lib.tk_grouped_linear_workspace_bytes(gref)
+    assert need > 0
+    assert lib.tk_grouped_linear(gref, None, P, 128, P, 256, None, P, need - 1, None) == small
+    assert lib.tk_grouped_linear(gref, None, P, 127, P, 256, None, P, need, None) == bad      # ldx below in_features
+    assert lib.tk_grouped_linear(gref, None, None, 128, P, 256, None, P, need, None) == bad   # no x
+    assert lib.tk_grouped_linear(None, None, P, 128, P, 256, None, P, need, None) == bad      # no descriptor
+    assert lib.tk_grouped_linear(gref, ref, P, 128, P, 256, P, P, need, None) == bad          # LoRA of another layer
+    g.groups_per_expert = 3
+    assert lib.tk_grouped_linear_workspace_bytes(gref) == bad                                 # 4 groups, 3 per expert
+    g.groups_per_expert, g.in_features, g.ldw = 2, 96, 96
+    assert lib.tk_grouped_linear(gref, None, P, 96, P, 256, None, P, need, None) == unsupported   # width not a multiple of 64
+    g.in_features, g.ldw, g.dtype = 128, 128, 0
+    assert lib.tk_grouped_linear(gref, None, P, 128, P, 256, None, P, need, None) == unsupported  # fp32
+    g.dtype, g.weight_stride = 1, 100
+    assert lib.tk_grouped_linear(gref, None, P, 128, P, 256, None, P, need, None) == bad      # experts overlap
+    g.rows, g.weight_stride = 0, 256 * 128
+    assert lib.tk_grouped_linear(gref, None, None, 128, None, 256, None, None, 0, None) == _lib.TK_OK  # nothing to do
     # optimizer
     assert lib.tk_opt_workspace_bytes(-1, 10) == bad
     assert lib.tk_opt_grad_norm(P, 4, P, 0, 100, 1, P, P, P, 1 << 20, None) == bad           # no tenants
