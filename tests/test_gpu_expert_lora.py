@@ -106,10 +106,13 @@ def test_config4_shapes_bf16(dev):
     assert max_rel_err(final, want) < 2e-2
 
 
-def test_moe_block_with_expert_lora_equals_merged_weights_per_tenant(dev):
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_moe_block_with_expert_lora_equals_merged_weights_per_tenant(dev, dtype):
     """Router outputs -> permute -> packed experts (gate_up, SiLU gate, down) with per-(expert, tenant) LoRA ->
     weighted unpermute, against the reference's form in float64: merged weights W + B A * scaling of every token's
-    own tenant (multi_lora_target_parameters.py:158-209), the per-expert loop, zero-init + index_add."""
+    own tenant (multi_lora_target_parameters.py:158-209), the per-expert loop, zero-init + index_add.
+    float32 takes the per-expert loop for the frozen weights, bfloat16 the grouped GEMMs (widths are multiples
+    of 128); the float64 restatement starts from the same rounded values."""
     from twinkle_amd import LoraTenant, MultiLora
     from twinkle_amd.expert_lora import moe_experts_block
     torch.manual_seed(0)
@@ -118,8 +121,9 @@ def test_moe_block_with_expert_lora_equals_merged_weights_per_tenant(dev):
     class Experts(torch.nn.Module):
         def __init__(self):
             super().__init__()
-            self.gate_up_proj = torch.nn.Parameter(torch.randn(e, 2 * inter, hid) * 0.05, requires_grad=False)
-            self.down_proj = torch.nn.Parameter(torch.randn(e, hid, inter) * 0.05, requires_grad=False)
+            self.gate_up_proj = torch.nn.Parameter((torch.randn(e, 2 * inter, hid) * 0.05).to(dtype),
+                                                   requires_grad=False)
+            self.down_proj = torch.nn.Parameter((torch.randn(e, hid, inter) * 0.05).to(dtype), requires_grad=False)
             self.act_fn = torch.nn.functional.silu
 
     model = torch.nn.Module()
@@ -142,11 +146,13 @@ def test_moe_block_with_expert_lora_equals_merged_weights_per_tenant(dev):
                 if '.lora_B.' in key:
                     p.normal_(0, 0.05)
     g = torch.Generator().manual_seed(1)
-    x = torch.randn(t, hid, generator=g)
+    x = torch.randn(t, hid, generator=g).to(dtype)
     logits = torch.randn(t, e, generator=g)
     weights, sel = torch.topk(torch.softmax(logits, -1), k)
+    weights = weights.to(dtype)
     tenant = torch.randint(0, 2, (t,), generator=g)
     xd = x.to(dev).requires_grad_(True)
+    assert gu_slots.lora_A['lora_0'].dtype == dtype
     slots = manager.slots_of(tenants)
     y = moe_experts_block(xd, sel.to(dev), weights.to(dev), tenant.to(dev), model.experts, slots, gu_slots, down_slots)
     y.pow(2).sum().backward()
@@ -174,10 +180,11 @@ def test_moe_block_with_expert_lora_equals_merged_weights_per_tenant(dev):
                 o = (torch.nn.functional.silu(gate) * up) @ merged[1].t()
                 out = out.index_add(0, idx, o * weights[idx, kk].double()[:, None])
     out.pow(2).sum().backward()
-    assert max_rel_err(y, out) < 2e-5
-    assert max_rel_err(xd.grad, x64.grad) < 1e-4
+    tight = dtype == torch.float32
+    assert max_rel_err(y, out) < (2e-5 if tight else 2e-2)
+    assert max_rel_err(xd.grad, x64.grad) < (1e-4 if tight else 2e-2)
     for s in slots:
         for w in (gu_slots, down_slots):
-            assert max_rel_err(w.lora_A[s].grad, leaf[(id(w), s, 'a')].grad) < 2e-4
-            assert max_rel_err(w.lora_B[s].grad, leaf[(id(w), s, 'b')].grad) < 2e-4
+            assert max_rel_err(w.lora_A[s].grad, leaf[(id(w), s, 'a')].grad) < (2e-4 if tight else 2e-2)
+            assert max_rel_err(w.lora_B[s].grad, leaf[(id(w), s, 'b')].grad) < (2e-4 if tight else 2e-2)
     assert gu_slots.lora_A['lora_2'].grad is None                      # the free slot
