@@ -52,8 +52,9 @@ __global__ __launch_bounds__(256) void k_grouped_plan(const int32_t* __restrict_
   int at = sums[tid] - cnt;
   for (int e = e0; e < e1; ++e) {
     const int t0 = tile_first[e * nt], t1 = tile_first[(e + 1) * nt];
+    const int first = at, count = (t1 - t0 + kPlanTiles - 1) / kPlanTiles;
     for (int t = t0; t < t1; t += kPlanTiles, ++at)
-      if (at < max_entries) plan[at] = GroupedPlanEntry{t, min(kPlanTiles, t1 - t), e, 0};
+      if (at < max_entries) plan[at] = GroupedPlanEntry{t, min(kPlanTiles, t1 - t), e, first, count, 0};
   }
   if (tid == 255) *nblocks = min(sums[255], max_entries);
 }
@@ -66,13 +67,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void k
                                                       const int32_t* __restrict__ slot_rows, int nsplit, int cpi) {
   __shared__ __attribute__((aligned(16))) bf16_t As[2][kGBM * kGLS];  // x rows
   __shared__ __attribute__((aligned(16))) bf16_t Bs[2][kGBN * kGLS];  // weight rows
-  // work item = (row block, run of cpi column blocks); the items of a row block and then of its expert's other row
-  // blocks are neighbours and reach one XCD together
+  // work item = (row block, run of cpi column blocks); the items of one expert are neighbours and reach one XCD
+  // together
   const int blocks = *nblocks * nsplit;
   if ((int)blockIdx.x >= blocks) return;
   const int item = xcd_contiguous(blockIdx.x, blocks);
-  const GroupedPlanEntry pe = plan[item / nsplit];
-  const int nb_first = (item % nsplit) * cpi, nb_last = min(nb_first + cpi, a.N / kGBN);
+  // within an expert: column run major, row block minor, so that the blocks that read the same weight rows start
+  // side by side (the expert's entries are contiguous: any of them names the range)
+  const GroupedPlanEntry any = plan[item / nsplit];
+  const int local = item - any.first * nsplit;
+  const GroupedPlanEntry pe = plan[any.first + local % any.count];
+  const int nb_first = (local / any.count) * cpi, nb_last = min(nb_first + cpi, a.N / kGBN);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
   const int wm = wave >> 1, wn = wave & 1;
   const int slot0 = pe.tile0 * kTileRows, live = pe.ntiles * kTileRows;

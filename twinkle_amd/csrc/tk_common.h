@@ -290,7 +290,9 @@ int launch_wgrad_shared(const SharedWgradArgs& a, const SegView& seg, const SegL
 
 // kernels_grouped.hip
 struct GroupedPlanEntry {  // a row block of the grouped GEMM: up to 4 consecutive tiles of one expert
-  int32_t tile0, ntiles, expert, pad;
+  int32_t tile0, ntiles, expert;
+  int32_t first, count;  // the expert's row blocks are the entries [first, first + count)
+  int32_t pad;
 };
 struct GroupedArgs {
   const uint16_t* x;  int64_t ldx;                     // activations, rows reached through the slot table
