@@ -173,3 +173,35 @@ def test_experts_forward_grouped_equals_the_per_expert_loop(dev):
     for i, (a, b) in enumerate(zip(fused, loop)):
         assert max_rel_err(a, b.double().cpu()) < 2e-2, i
     assert experts.gate_up_proj.grad is None and experts.down_proj.grad is None
+
+
+def test_custom_op_matches_the_direct_call(dev):
+    """torch.ops.twinkle_amd.grouped_linear gives bit-identical results to the direct binding, with and without
+    the LoRA term."""
+    import twinkle_amd.custom_ops  # noqa: F401  (registers the ops)
+    e, nt, t, k, n, max_r = 4, 2, 900, 128, 256, 16
+    expert, tenant, x, w = _case(e, nt, t, k, n, seed=5)
+    keys = (expert * nt + tenant).to(torch.int32).to(dev)
+    seg = build_segments(keys, e * nt)
+    g = torch.Generator().manual_seed(6)
+    a = [(torch.randn(e, max_r, k, generator=g) / k**0.5).bfloat16().to(dev) for _ in range(nt)]
+    b = [(torch.randn(e, n, max_r, generator=g) * 0.05).bfloat16().to(dev) for _ in range(nt)]
+    idx = [i % nt for i in range(e * nt)]
+    groups = AdapterGroups(a, b, [16, 7] * e, [2.0] * (e * nt),
+                           a_index=idx, a_offset=[(i // nt) * max_r * k for i in range(e * nt)],
+                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)])
+    xd, wd = x.to(dev), w.to(dev)
+    h = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=dev)
+    lora_shrink_(xd, seg, groups, h, map_rows=True)
+    want_base = grouped_linear_(xd, wd, seg, nt, map_rows=True)
+    want_lora = grouped_linear_(xd, wd, seg, nt, groups=groups, h=h, map_rows=True)
+    empty_i64 = torch.empty(0, dtype=torch.int64, device=dev)
+    y = torch.empty_like(want_base)
+    torch.ops.twinkle_amd.grouped_linear(xd, wd, y, seg.workspace, nt, e * nt, True, h[:0], empty_i64, empty_i64,
+                                         groups.rank_dev[:0], groups.scale_dev[:0], 0, 0, 0)
+    assert torch.equal(y, want_base)
+    y2 = torch.empty_like(want_base)
+    torch.ops.twinkle_amd.grouped_linear(xd, wd, y2, seg.workspace, nt, e * nt, True, h, groups.a_ptrs, groups.b_ptrs,
+                                         groups.rank_dev, groups.scale_dev, groups.max_rank, groups.lda, groups.ldb)
+    assert torch.equal(y2, want_lora)
+    assert not torch.equal(want_base, want_lora)

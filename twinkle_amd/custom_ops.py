@@ -15,6 +15,7 @@ passed as the int64 / int32 / float32 device tensors it already holds.
                                                      dx, grad_a, grad_b, ws written
     lora_fwd_shared(x, ys, hs, seg_ws, ...) / lora_bwd_shared(dys, x, hs, dx, ...)
                                                      the same for projections that share x (tensor lists)
+    grouped_linear(x, weight, y, seg_ws, ...)        y written: packed experts' base GEMM (+ LoRA term from h)
 """
 from __future__ import annotations
 
@@ -121,6 +122,43 @@ def lora_bwd(dy: torch.Tensor, x: torch.Tensor, h: torch.Tensor, dx: torch.Tenso
 @lora_bwd.register_fake
 def _(dy, x, h, dx, grad_a, grad_b, grad_a_ptrs, grad_b_ptrs, workspace, seg_ws, a_ptrs, b_ptrs, rank, scale, max_rank,
       lda, ldb, map_rows, accumulate):
+    return None
+
+
+@torch.library.custom_op('twinkle_amd::grouped_linear', mutates_args=('y',))
+def grouped_linear(x: torch.Tensor, weight: torch.Tensor, y: torch.Tensor, seg_ws: torch.Tensor,
+                   groups_per_expert: int, num_groups: int, map_rows: bool, h: torch.Tensor, a_ptrs: torch.Tensor,
+                   b_ptrs: torch.Tensor, rank: torch.Tensor, scale: torch.Tensor, max_rank: int, lda: int,
+                   ldb: int) -> None:
+    """``y[row] = x[row] @ weight[e].T (+ h[row] @ B_g.T)``, ``weight`` packed ``[E, out, in]`` (``tk_grouped_linear``).
+
+    ``max_rank = 0`` leaves the LoRA term out; ``h`` and the adapter tables are then ignored (pass empty tensors).
+    """
+    for t, n in ((x, 'x'), (weight, 'weight'), (y, 'y'), (seg_ws, 'seg_ws')):
+        _need_gpu(t, n)
+    g = _lib.GroupedDesc()
+    g.rows, g.num_groups, g.groups_per_expert = x.shape[0], num_groups, groups_per_expert
+    g.in_features, g.out_features = weight.shape[2], weight.shape[1]
+    g.dtype = _lib.dtype_code(weight.dtype)
+    g.map_rows = 1 if map_rows else 0
+    g.seg_ws = seg_ws.data_ptr()
+    g.weight, g.weight_stride, g.ldw = weight.data_ptr(), weight.stride(0), weight.stride(1)
+    lib = _lib.load()
+    need = lib.tk_grouped_linear_workspace_bytes(ctypes.byref(g))
+    _lib.check(need, 'tk_grouped_linear_workspace_bytes')
+    ws = torch.empty(need, dtype=torch.uint8, device=x.device)
+    d = None
+    if max_rank > 0:
+        d = ctypes.byref(_desc(x.shape[0], weight.shape[2], weight.shape[1], max_rank, x.dtype, map_rows, seg_ws,
+                               a_ptrs, b_ptrs, lda, ldb, rank, scale))
+    code = lib.tk_grouped_linear(ctypes.byref(g), d, x.data_ptr(), x.stride(0), y.data_ptr(), y.stride(0),
+                                 h.data_ptr() if max_rank > 0 else None, ws.data_ptr(), ws.numel(), _lib.stream_ptr())
+    _lib.check(code, 'tk_grouped_linear')
+
+
+@grouped_linear.register_fake
+def _(x, weight, y, seg_ws, groups_per_expert, num_groups, map_rows, h, a_ptrs, b_ptrs, rank, scale, max_rank, lda,
+      ldb):
     return None
 
 
