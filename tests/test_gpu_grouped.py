@@ -39,6 +39,8 @@ def _reference(x, w, expert):
     (5, 3, 1500, 192, 384, (0, 4)),    # three tenants per expert: weights shared by consecutive groups
     (16, 4, 6000, 256, 128, ()),       # experts with more than one 128-row block
     (3, 2, 700, 64, 640, ()),
+    (8, 2, 5000, 128, 512, (3,)),      # out_features a multiple of 256: 256-row blocks on 8 waves, experts of
+    (2, 1, 300, 64, 256, ()),          # more and of less than one block, dead strips of rows
 ])
 @pytest.mark.parametrize('map_rows', [True, False])
 def test_base_term_matches_the_per_expert_loop(dev, e, nt, t, k, n, empty, map_rows):
@@ -61,9 +63,11 @@ def test_base_term_matches_the_per_expert_loop(dev, e, nt, t, k, n, empty, map_r
 
 
 @pytest.mark.parametrize('max_r,ranks', [(8, [8, 4, 8]), (16, [16, 0, 9]), (32, [32, 17, 8]), (64, [64, 40, 16])])
-def test_lora_term_in_the_epilogue(dev, max_r, ranks):
-    """y = x W_e^T + s (x A_{e,t}^T) B_{e,t}^T per (expert, tenant) segment: oracle's low-rank form per tenant."""
-    e, nt, t, k, n = 4, len(ranks), 1800, 256, 384
+@pytest.mark.parametrize('n', [384, 512])
+def test_lora_term_in_the_epilogue(dev, max_r, ranks, n):
+    """y = x W_e^T + s (x A_{e,t}^T) B_{e,t}^T per (expert, tenant) segment: oracle's low-rank form per tenant
+    (out_features 384: 128-row blocks on 4 waves; 512: 256-row blocks on 8 waves)."""
+    e, nt, t, k = 4, len(ranks), 1800, 256
     expert, tenant, x, w = _case(e, nt, t, k, n, seed=max_r)
     keys = (expert * nt + tenant).to(torch.int32).to(dev)
     seg = build_segments(keys, e * nt)
