@@ -63,11 +63,12 @@ def test_base_term_matches_the_per_expert_loop(dev, e, nt, t, k, n, empty, map_r
 
 
 @pytest.mark.parametrize('max_r,ranks', [(8, [8, 4, 8]), (16, [16, 0, 9]), (32, [32, 17, 8]), (64, [64, 40, 16])])
-@pytest.mark.parametrize('n', [384, 512])
-def test_lora_term_in_the_epilogue(dev, max_r, ranks, n):
-    """y = x W_e^T + s (x A_{e,t}^T) B_{e,t}^T per (expert, tenant) segment: oracle's low-rank form per tenant
-    (out_features 384: 128-row blocks on 4 waves; 512: 256-row blocks on 8 waves)."""
-    e, nt, t, k = 4, len(ranks), 1800, 256
+@pytest.mark.parametrize('e,t,n', [(4, 1800, 384), (4, 1800, 512), (2, 2600, 512)])
+def test_lora_term_in_the_epilogue(dev, max_r, ranks, e, t, n):
+    """y = x W_e^T + s (x A_{e,t}^T) B_{e,t}^T per (expert, tenant) segment: oracle's low-rank form per tenant.
+    The last shape (out_features a multiple of 256, more than 1024 rows per expert) takes the 256-row blocks on
+    8 waves, the others the 128-row blocks on 4 waves."""
+    nt, k = len(ranks), 256
     expert, tenant, x, w = _case(e, nt, t, k, n, seed=max_r)
     keys = (expert * nt + tenant).to(torch.int32).to(dev)
     seg = build_segments(keys, e * nt)
