@@ -248,8 +248,8 @@ int tk_lora_bwd_shared(const tk_lora_desc* const* descs, int32_t num_proj, const
  * gate_up and the down projection each); with `lora` it also takes over the expert LoRA delta that the
  * reference merges into the weights (multi_lora_target_parameters.py:158-179): call tk_lora_shrink(lora, x, h)
  * first and pass that h here, y is then written once with both terms.  The backward of the base term is the
- * same call on the transposed weights (dx = dy W_e: pass a [in_features][out_features] copy); the LoRA
- * gradients come from tk_lora_bwd with dx accumulated onto this call's result.
+ * same call with weight_layout = 1 on the same weights (dx = dy W_e, in_features and out_features swapped);
+ * the LoRA gradients come from tk_lora_bwd with dx accumulated onto this call's result.
  *
  * bf16 only; in_features a multiple of 64, out_features of 128, ldx / ldw / weight_stride multiples of 8 and
  * ldy of 4 elements, 16-byte aligned x and weight, 8-byte aligned y: anything else is TK_ERR_UNSUPPORTED
@@ -267,6 +267,10 @@ typedef struct {
   const void* weight_device;
   int64_t weight_stride;     /* elements between consecutive experts */
   int64_t ldw;
+  int32_t weight_layout;     /* 0: [out_features][in_features] per expert (y = x W^T);
+                                1: [in_features][out_features] per expert (y = x W): the backward of a layout-0
+                                   call on the same memory, dx = dy W.  No LoRA term with layout 1. */
+  int32_t reserved;          /* 0 */
 } tk_grouped_desc;
 
 int64_t tk_grouped_linear_workspace_bytes(const tk_grouped_desc* desc);

@@ -154,6 +154,11 @@ def test_entry_points_reject_malformed_arguments_on_the_host():
     assert lib.tk_grouped_linear(gref, None, P, 128, P, 256, None, P, need, None) == unsupported  # fp32
     g.dtype, g.weight_stride = 1, 100
     assert lib.tk_grouped_linear(gref, None, P, 128, P, 256, None, P, need, None) == bad      # experts overlap
+    g.weight_stride, g.weight_layout = 256 * 128, 2
+    assert lib.tk_grouped_linear(gref, None, P, 128, P, 256, None, P, need, None) == bad      # unknown layout
+    g.weight_layout = 1
+    assert lib.tk_grouped_linear(gref, None, P, 128, P, 256, None, P, need, None) == bad      # ldw below out_features
+    g.weight_layout = 0
     g.rows, g.weight_stride = 0, 256 * 128
     assert lib.tk_grouped_linear(gref, None, None, 128, None, 256, None, None, 0, None) == _lib.TK_OK  # nothing to do
     # optimizer

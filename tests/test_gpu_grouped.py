@@ -97,16 +97,25 @@ def test_lora_term_in_the_epilogue(dev, max_r, ranks, e, t, n):
     assert max_rel_err(got, want) < 2e-2
 
 
-def test_backward_of_the_base_term_is_the_same_call_on_transposed_weights(dev):
-    e, nt, t, k, n = 5, 2, 1200, 128, 256
+@pytest.mark.parametrize('k,n', [(128, 256), (512, 192), (384, 64), (256, 1024)])
+def test_backward_of_the_base_term_on_the_same_weights(dev, k, n):
+    """dx = dy W_e is the call with transposed=True on the forward's own weights (the kernel transposes the weight
+    tiles on their way into LDS), and equally the plain call on a transposed copy.  in_features k of the forward is
+    the output width here: 128 and 384 take the 4-wave kernel, 512 and 256 the 8-wave one."""
+    e, nt, t = 5, 2, 1200
     expert, tenant, x, w = _case(e, nt, t, k, n, seed=9)
     dy = torch.randn(t, n, generator=torch.Generator().manual_seed(10)).bfloat16()
     keys = (expert * nt + tenant).to(torch.int32).to(dev)
     seg = build_segments(keys, e * nt)
-    wt = w.transpose(1, 2).contiguous()                     # [E, in, out]: dx = dy W_e
-    got = grouped_linear_(dy.to(dev), wt.to(dev), seg, nt, map_rows=True)
+    wt = w.transpose(1, 2).contiguous()                     # [E, in, out]
     want = _reference(dy, wt, expert)
+    got = grouped_linear_(dy.to(dev), w.to(dev), seg, nt, map_rows=True, transposed=True)
     assert max_rel_err(got, want) < 6e-3
+    if n % 64 == 0 and k % 128 == 0:
+        copy = grouped_linear_(dy.to(dev), wt.to(dev), seg, nt, map_rows=True)
+        assert torch.equal(copy, got), 'same products, same order of the sums'
+    with pytest.raises(ValueError):
+        grouped_linear_(dy.to(dev), w.to(dev), seg, nt, map_rows=True, transposed=True, groups=object(), h=None)
 
 
 def test_unsupported_shapes_are_refused(dev):

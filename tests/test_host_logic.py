@@ -419,10 +419,9 @@ def test_target_parameter_slots_keys_shapes_release_and_round_trip(is_transposed
                                                 target_parameters=['mlp.experts.down_proj']))
 
 
-def test_grouped_gemm_applicability_and_transposed_copy_cache():
-    """experts_forward takes the grouped GEMMs only for frozen bf16 weights whose widths are multiples of 128, and
-    keeps one transposed copy per weight that is redone when the weight changes."""
-    from twinkle_amd.expert_lora import _transposed_copy, grouped_gemm_applies
+def test_grouped_gemm_applicability():
+    """experts_forward takes the grouped GEMMs only for frozen bf16 weights whose widths are multiples of 128."""
+    from twinkle_amd.expert_lora import grouped_gemm_applies
     rows = torch.zeros(4, 256, dtype=torch.bfloat16)
     ok = torch.nn.Parameter(torch.zeros(3, 384, 256, dtype=torch.bfloat16), requires_grad=False)
     assert grouped_gemm_applies(ok, rows)
@@ -431,15 +430,3 @@ def test_grouped_gemm_applicability_and_transposed_copy_cache():
     assert not grouped_gemm_applies(torch.zeros(3, 384, 192, dtype=torch.bfloat16), rows)          # in = 192
     assert not grouped_gemm_applies(torch.zeros(3, 320, 256, dtype=torch.bfloat16), rows)          # out = 320
     assert not grouped_gemm_applies(ok.transpose(1, 2), rows)                                       # not contiguous
-
-    mod = torch.nn.Module()
-    mod.gate_up_proj = torch.nn.Parameter(torch.arange(2 * 3 * 4, dtype=torch.float32).reshape(2, 3, 4),
-                                          requires_grad=False)
-    first = _transposed_copy(mod, 'gate_up_proj')
-    assert first.shape == (2, 4, 3) and first.is_contiguous()
-    assert torch.equal(first, mod.gate_up_proj.transpose(1, 2))
-    assert _transposed_copy(mod, 'gate_up_proj') is first                                           # cached
-    with torch.no_grad():
-        mod.gate_up_proj.mul_(2)
-    second = _transposed_copy(mod, 'gate_up_proj')
-    assert second is not first and torch.equal(second, mod.gate_up_proj.transpose(1, 2))

@@ -63,6 +63,8 @@ class GroupedDesc(Structure):
         ('weight', c_void_p),
         ('weight_stride', c_int64),
         ('ldw', c_int64),
+        ('weight_layout', c_int32),
+        ('reserved', c_int32),
     ]
 
 

@@ -395,9 +395,12 @@ int tk_grouped_linear(const tk_grouped_desc* g, const tk_lora_desc* lora, const 
                       int64_t ldy, const void* h, void* ws, int64_t ws_bytes, tk_stream_t stream) {
   if (!grouped_desc_ok(g) || !g->seg_ws || !g->weight_device) return TK_ERR_INVALID;
   if (g->rows == 0) return TK_OK;
-  if (!x || !y || !ws || ldx < g->in_features || ldy < g->out_features || g->ldw < g->in_features)
-    return TK_ERR_INVALID;
-  if (g->weight_stride < (int64_t)(g->out_features - 1) * g->ldw + g->in_features) return TK_ERR_INVALID;
+  if (g->weight_layout != 0 && g->weight_layout != 1) return TK_ERR_INVALID;
+  const int64_t w_rows = g->weight_layout ? g->in_features : g->out_features;
+  const int64_t w_cols = g->weight_layout ? g->out_features : g->in_features;
+  if (!x || !y || !ws || ldx < g->in_features || ldy < g->out_features || g->ldw < w_cols) return TK_ERR_INVALID;
+  if (g->weight_stride < (w_rows - 1) * g->ldw + w_cols) return TK_ERR_INVALID;
+  if (g->weight_layout && lora && lora->max_rank > 0) return TK_ERR_INVALID;
   const GroupedLayout W(*g);
   if (ws_bytes < W.total) return TK_ERR_WORKSPACE;
   if (g->dtype != TK_DTYPE_BF16 || force_generic()) return TK_ERR_UNSUPPORTED;
@@ -406,6 +409,7 @@ int tk_grouped_linear(const tk_grouped_desc* g, const tk_lora_desc* lora, const 
   a.w = (const uint16_t*)g->weight_device;  a.w_stride = g->weight_stride;  a.ldw = g->ldw;
   a.y = (uint16_t*)y;  a.ldy = ldy;
   a.K = g->in_features;  a.N = g->out_features;  a.src_rows = (int32_t)g->rows;  a.map_rows = g->map_rows;
+  a.w_rows_are_inputs = g->weight_layout;
   if (lora && lora->max_rank > 0) {
     if (!desc_ok(lora) || !h) return TK_ERR_INVALID;
     if (lora->rows != g->rows || lora->num_groups != g->num_groups || lora->in_features != g->in_features ||

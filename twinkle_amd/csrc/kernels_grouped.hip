@@ -65,7 +65,12 @@ __global__ __launch_bounds__(256) void k_grouped_plan(const int32_t* __restrict_
 //      1: 8 waves (2 x 4), wave tile 128 x 64, block tile 256 x 256, one block per CU: half the operand bytes per
 //         FLOP out of L2 and three LDS reads per eight MFMAs instead of four; a wave whose rows are dead (the tail
 //         of an expert) skips its MFMAs, so a half-empty block takes about half the time
-template <int NKS, int BIG>
+// TR:  0: weight rows are output features (y = x W^T, the contraction runs along the weight's rows in memory);
+//      1: weight rows are input features (y = x W: the backward of TR = 0 on the same memory).  The lower half of
+//         the block then loads the weight tile as 8 x 8 blocks, transposes them in registers and writes them to LDS
+//         with the 16-byte chunks of a row XOR-swizzled by the row's block number (conflict-free on both sides);
+//         the upper half loads the x tile.
+template <int NKS, int BIG, int TR>
 __global__ __launch_bounds__(BIG ? 512 : 256) __attribute__((amdgpu_waves_per_eu(2))) void k_grouped_gemm(
     GroupedArgs a, const GroupedPlanEntry* __restrict__ plan, const int32_t* __restrict__ nblocks,
     const int32_t* __restrict__ tile_group, const int32_t* __restrict__ slot_rows, int nsplit, int cpi) {
@@ -73,7 +78,7 @@ __global__ __launch_bounds__(BIG ? 512 : 256) __attribute__((amdgpu_waves_per_eu
   constexpr int BM = 2 * 16 * RB, BN = WN * 16 * CB;  // 128 x 128 or 256 x 256
   constexpr int LROWS = THREADS / 8;                   // rows moved per pass of the block's loads
   constexpr int XP = BM / LROWS, WP = BN / LROWS;      // passes: 4 and 4
-  constexpr int SETS = BIG ? 1 : 2;                    // register sets of loads in flight
+  constexpr int SETS = (BIG || TR) ? 1 : 2;            // register sets of loads in flight
   __shared__ __attribute__((aligned(16))) bf16_t As[2][BM * kGLS];  // x rows
   __shared__ __attribute__((aligned(16))) bf16_t Bs[2][BN * kGLS];  // weight rows
   // work item = (row block, run of cpi column blocks); the items of one expert are neighbours and reach one XCD
@@ -92,16 +97,22 @@ __global__ __launch_bounds__(BIG ? 512 : 256) __attribute__((amdgpu_waves_per_eu
   const int slot0 = pe.tile0 * kTileRows, live = pe.ntiles * kTileRows;
   const int live_w = min(max(live - 16 * RB * wm, 0), 16 * RB);  // live rows of this wave's strip (uniform)
 
-  // global -> LDS: thread t moves 16 bytes of rows (t >> 3) + LROWS i at column chunk t & 7
-  const int lrow = tid >> 3, lchunk = (tid & 7) * 8;
-  const bf16_t* xp[XP];
+  // global -> LDS (TR = 0): thread t moves 16 bytes of rows (t >> 3) + LROWS i at column chunk t & 7, of x and of
+  // the weights alike.  (TR = 1): the upper half of the threads does that for x alone (XR rows per pass, 8 passes),
+  // the lower half owns one 8 x 8 block of the weight tile each.
+  constexpr int XR = TR ? THREADS / 16 : LROWS, XN = TR ? 8 : XP;
+  const bool w_thread = TR && tid < THREADS / 2;           // uniform over a wave
+  const int xt = TR ? (tid & (THREADS / 2 - 1)) : tid;
+  const int lrow = xt >> 3, lchunk = (xt & 7) * 8;
+  const bf16_t* xp[XN];
 #pragma unroll
-  for (int i = 0; i < XP; ++i) {
-    const int r = lrow + LROWS * i;
+  for (int i = 0; i < XN; ++i) {
+    const int r = lrow + XR * i;
     int row = r < live ? slot_rows[slot0 + r] : -1;  // padding and dead rows read row 0 and are never stored
     row = min(max(row, 0), a.src_rows - 1);
     xp[i] = a.x + (int64_t)row * a.ldx + lchunk;
   }
+  const int cblk = tid / (BN / 8), jblk = tid % (BN / 8);  // TR: this thread's block of the weight tile
   // rows this lane stores: slots 16 RB wm + 16 rb + li
   int out_row[RB];
 #pragma unroll
@@ -114,9 +125,13 @@ __global__ __launch_bounds__(BIG ? 512 : 256) __attribute__((amdgpu_waves_per_eu
   const int ldsw = lrow * kGLS + lchunk;  // + LROWS i rows
 
   for (int nb = nb_first; nb < nb_last; ++nb) {
-    const bf16_t* wp[WP];
+    const bf16_t* wp[TR ? 1 : WP];
+    if constexpr (TR) {
+      wp[0] = wbase + (int64_t)(8 * cblk) * a.ldw + nb * BN + 8 * jblk;
+    } else {
 #pragma unroll
-    for (int i = 0; i < WP; ++i) wp[i] = wbase + (int64_t)(nb * BN + lrow + LROWS * i) * a.ldw + lchunk;
+      for (int i = 0; i < WP; ++i) wp[i] = wbase + (int64_t)(nb * BN + lrow + LROWS * i) * a.ldw + lchunk;
+    }
     f32x4 acc[RB][CB];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
@@ -125,19 +140,56 @@ __global__ __launch_bounds__(BIG ? 512 : 256) __attribute__((amdgpu_waves_per_eu
 
     // The loads of step ks + SETS are issued before step ks is computed and wait in registers across the barrier
     // (which orders LDS traffic only).
-    uint4 gx[SETS][XP], gw[SETS][WP];
+    uint4 gx[SETS][TR ? 8 : XP], gw[SETS][TR ? 1 : WP];  // TR: gx holds a thread's eight pieces of either tile
     auto fetch = [&](int ks, auto set) {
       const int k0 = ks * kGBK;
+      if constexpr (TR) {
+        if (w_thread) {
+          const bf16_t* p = wp[0] + (int64_t)k0 * a.ldw;
 #pragma unroll
-      for (int i = 0; i < XP; ++i) gx[set][i] = ld16(xp[i] + k0);
+          for (int i = 0; i < 8; ++i) gx[set][i] = ld16(p + (int64_t)i * a.ldw);
+        } else {
 #pragma unroll
-      for (int i = 0; i < WP; ++i) gw[set][i] = ld16(wp[i] + k0);
+          for (int i = 0; i < 8; ++i) gx[set][i] = ld16(xp[i] + k0);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < XP; ++i) gx[set][i] = ld16(xp[i] + k0);
+#pragma unroll
+        for (int i = 0; i < WP; ++i) gw[set][i] = ld16(wp[i] + k0);
+      }
     };
     auto stash = [&](int buf, auto set) {
+      if constexpr (TR) {
+        if (w_thread) {
+          // 8 x 8 transpose inside the thread: piece q becomes column q of the block, the eight contraction indices
 #pragma unroll
-      for (int i = 0; i < XP; ++i) st16(&As[buf][ldsw + LROWS * i * kGLS], gx[set][i]);
+          for (int q = 0; q < 8; ++q) {
+            const int d = q >> 1;
+            const uint32_t sel = (q & 1) ? 0x07060302u : 0x05040100u;
+            uint32_t e[8];
 #pragma unroll
-      for (int i = 0; i < WP; ++i) st16(&Bs[buf][ldsw + LROWS * i * kGLS], gw[set][i]);
+            for (int i = 0; i < 8; ++i) {
+              const uint32_t wsrc[4] = {gx[set][i].x, gx[set][i].y, gx[set][i].z, gx[set][i].w};
+              e[i] = wsrc[d];
+            }
+            uint4 tr;
+            tr.x = __builtin_amdgcn_perm(e[1], e[0], sel);
+            tr.y = __builtin_amdgcn_perm(e[3], e[2], sel);
+            tr.z = __builtin_amdgcn_perm(e[5], e[4], sel);
+            tr.w = __builtin_amdgcn_perm(e[7], e[6], sel);
+            st16(&Bs[buf][(8 * jblk + q) * kGLS + 8 * (cblk ^ (jblk & 7))], tr);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) st16(&As[buf][ldsw + XR * i * kGLS], gx[set][i]);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < XP; ++i) st16(&As[buf][ldsw + LROWS * i * kGLS], gx[set][i]);
+#pragma unroll
+        for (int i = 0; i < WP; ++i) st16(&Bs[buf][ldsw + LROWS * i * kGLS], gw[set][i]);
+      }
     };
     auto step = [&](int ks, auto parity) {  // parity = ks & 1 as a compile-time constant
       constexpr int cur = decltype(parity)::value;
@@ -146,8 +198,11 @@ __global__ __launch_bounds__(BIG ? 512 : 256) __attribute__((amdgpu_waves_per_eu
       for (int s = 0; s < 2; ++s) {
         uint4 fw[CB];
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb)
-          fw[cb] = ld16(&Bs[cur][(16 * CB * wn + 16 * cb + li) * kGLS + 32 * s + 8 * kb]);
+        for (int cb = 0; cb < CB; ++cb) {
+          const int j = 16 * CB * wn + 16 * cb + li;
+          const int chunk = TR ? ((4 * s + kb) ^ ((j >> 3) & 7)) : 4 * s + kb;
+          fw[cb] = ld16(&Bs[cur][j * kGLS + 8 * chunk]);
+        }
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
           if (16 * rb >= live_w) break;
@@ -248,10 +303,17 @@ int launch_grouped_gemm(const GroupedArgs& a, int experts, int nt, GroupedPlanEn
   const int cpi = (int)std::min<int64_t>(ncb, std::max<int64_t>(1, ceil_div(ncb * row_blocks, kGroupedItems)));
   const int nsplit = (int)ceil_div(ncb, cpi);
   const dim3 grid((unsigned)((int64_t)max_entries * nsplit));
-#define TK_LAUNCH_GROUPED(NKS, BIG)                                                                               \
-  hipLaunchKernelGGL((k_grouped_gemm<NKS, BIG>), grid, dim3(BIG ? 512 : 256), 0, s, a, plan, nblocks, seg.tile_group, \
+#define TK_LAUNCH_GROUPED(NKS, BIG)                                                                                  \
+  hipLaunchKernelGGL((k_grouped_gemm<NKS, BIG, 0>), grid, dim3(BIG ? 512 : 256), 0, s, a, plan, nblocks, seg.tile_group, \
                      rows, nsplit, cpi)
-  if (big) {
+  if (a.w_rows_are_inputs) {  // never with the LoRA term (the caller checks)
+    if (big)
+      hipLaunchKernelGGL((k_grouped_gemm<0, 1, 1>), grid, dim3(512), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit,
+                         cpi);
+    else
+      hipLaunchKernelGGL((k_grouped_gemm<0, 0, 1>), grid, dim3(256), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit,
+                         cpi);
+  } else if (big) {
     if (nks == 0) TK_LAUNCH_GROUPED(0, 1);
     else if (nks == 1) TK_LAUNCH_GROUPED(1, 1);
     else TK_LAUNCH_GROUPED(2, 1);

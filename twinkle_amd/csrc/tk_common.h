@@ -297,6 +297,7 @@ struct GroupedPlanEntry {  // a row block of the grouped GEMM: up to 4 consecuti
 struct GroupedArgs {
   const uint16_t* x;  int64_t ldx;                     // activations, rows reached through the slot table
   const uint16_t* w;  int64_t w_stride, ldw;           // packed weights: expert e at w + e * w_stride, [N][K]
+  int32_t w_rows_are_inputs;                           // ... or [K][N]: y = x W (no LoRA term then)
   uint16_t* y;        int64_t ldy;
   int32_t K, N, src_rows, map_rows;
   // LoRA term (rpad = 0: none): y += h B_g^T with h[slot][rpad] as the shrink kernels leave it

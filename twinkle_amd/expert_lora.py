@@ -290,22 +290,9 @@ class ExpertLoraManager:
         return consumed
 
 
-def _transposed_copy(experts_mod: nn.Module, name: str) -> torch.Tensor:
-    """``[E, in, out]`` copy of the frozen packed weight ``name`` (kept on the module, redone if the weight changed):
-    the backward of the grouped GEMM is the same kernel on this copy."""
-    weight = getattr(experts_mod, name)
-    cache = experts_mod.__dict__.setdefault('_tk_transposed', {})
-    hit = cache.get(name)
-    if hit is None or hit[0] != (weight.data_ptr(), weight._version, tuple(weight.shape)):
-        with torch.no_grad():
-            hit = ((weight.data_ptr(), weight._version, tuple(weight.shape)), weight.transpose(1, 2).contiguous())
-        cache[name] = hit
-    return hit[1]
-
-
 def grouped_gemm_applies(weight: torch.Tensor, rows: torch.Tensor) -> bool:
     """Frozen bf16 packed weights whose two widths are multiples of 128: what ``tk_grouped_linear`` takes in the
-    forward direction (``in`` a multiple of 64, ``out`` of 128) and, on the transposed copy, in the backward one."""
+    forward direction (``in`` a multiple of 64, ``out`` of 128) and, with the roles swapped, in the backward one."""
     return (weight.dtype == torch.bfloat16 and rows.dtype == torch.bfloat16 and weight.is_contiguous() and
             not weight.requires_grad and weight.shape[1] % 128 == 0 and weight.shape[2] % 128 == 0)
 
@@ -326,7 +313,7 @@ def experts_forward(experts_mod: nn.Module, rows: torch.Tensor, seg: SegmentTabl
     ``grouped`` (default: whenever the shapes allow, i.e. frozen bf16 weights with widths that are multiples of
     64 / 128 in both directions) replaces the loop by one grouped GEMM per projection with the LoRA terms in its
     epilogue: no host copy of the boundaries at all, one launch instead of one per expert, and the expert outputs
-    are written once.  Its backward runs the same kernel on a transposed copy of the frozen weights.
+    are written once.  Its backward runs the same kernel in its transposing form on the same weights.
     """
     if rows.shape[0] == 0:
         return rows                                                   # keeps the autograd edge (reference :340-344)
@@ -343,14 +330,14 @@ def experts_forward(experts_mod: nn.Module, rows: torch.Tensor, seg: SegmentTabl
     if grouped or (grouped is None and can_group):
         from .ops import grouped_experts_linear
         x = x.contiguous()
-        gate_up_out = grouped_experts_linear(x, gate_up, _transposed_copy(experts_mod, 'gate_up_proj'), seg, nt,
+        gate_up_out = grouped_experts_linear(x, gate_up, seg, nt,
                                              gate_up_slots.groups(tenant_slots) if gate_up_slots is not None else None)
         if hasattr(experts_mod, '_apply_gate'):
             hidden = experts_mod._apply_gate(gate_up_out)
         else:
             gate, up = gate_up_out.chunk(2, dim=-1)
             hidden = experts_mod.act_fn(gate) * up
-        out = grouped_experts_linear(hidden.contiguous(), down, _transposed_copy(experts_mod, 'down_proj'), seg, nt,
+        out = grouped_experts_linear(hidden.contiguous(), down, seg, nt,
                                      down_slots.groups(tenant_slots) if down_slots is not None else None)
         return out if out.dtype == input_dtype else out.to(input_dtype)
     if seg.offsets is None:

@@ -252,15 +252,21 @@ def lora_bwd_(dy: torch.Tensor, x: Optional[torch.Tensor], h: Optional[torch.Ten
 def grouped_linear_(x: torch.Tensor, weight: torch.Tensor, seg: SegmentTable, groups_per_expert: int = 1,
                     y: Optional[torch.Tensor] = None, groups: Optional[AdapterGroups] = None,
                     h: Optional[torch.Tensor] = None, map_rows: bool = False,
-                    workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    workspace: Optional[torch.Tensor] = None, transposed: bool = False) -> torch.Tensor:
     """``y[row] = x[row] @ weight[e].T (+ h[row] @ B_g.T)`` for every row of the table, ``e = g // groups_per_expert``
     (see ``tk_grouped_linear``).  ``weight`` is packed ``[E, out, in]``; with ``groups`` the LoRA term of the
-    (expert, tenant) groups is added on the accumulators, from ``h`` as :func:`lora_shrink_` left it."""
+    (expert, tenant) groups is added on the accumulators, from ``h`` as :func:`lora_shrink_` left it.
+    ``transposed=True`` computes ``y[row] = x[row] @ weight[e]`` instead (``weight [E, in, out]``): the backward of
+    the plain call on the same weights."""
     if not (x.is_cuda and weight.is_cuda):
         raise RuntimeError('x and weight must live on the GPU: this path has no CPU implementation')
     if weight.dim() != 3 or weight.stride(2) != 1 or weight.dtype != x.dtype:
         raise ValueError('weight must be [experts, out, in] with unit inner stride and the dtype of x')
+    if transposed and groups is not None:
+        raise ValueError('the LoRA term goes with the plain call, not with transposed=True')
     experts, out_f, in_f = weight.shape
+    if transposed:
+        out_f, in_f = in_f, out_f
     if seg.num_groups != experts * groups_per_expert:
         raise ValueError(f'segment table has {seg.num_groups} groups, weights give {experts} x {groups_per_expert}')
     _check_rows(x, 'x', seg.rows, in_f, weight.dtype)
@@ -274,6 +280,7 @@ def grouped_linear_(x: torch.Tensor, weight: torch.Tensor, seg: SegmentTable, gr
     g.map_rows = 1 if map_rows else 0
     g.seg_ws = seg.workspace.data_ptr()
     g.weight, g.weight_stride, g.ldw = weight.data_ptr(), weight.stride(0), weight.stride(1)
+    g.weight_layout = 1 if transposed else 0
     lib = _lib.load()
     if workspace is None:
         n = lib.tk_grouped_linear_workspace_bytes(ctypes.byref(g))
@@ -365,49 +372,50 @@ class _LoraLinear(torch.autograd.Function):
 class _GroupedExpertsLinear(torch.autograd.Function):
     """Frozen packed expert weights and the (expert, tenant) LoRA terms as one node on rows in segment order.
 
-    Forward: shrink, then the grouped GEMM with the LoRA term in its epilogue.  Backward: the same grouped GEMM on
-    the transposed weights gives the base part of ``dx``; the segmented backward adds the LoRA part onto it in place
-    and yields the adapters' gradients.  The weights get no gradient (the reference freezes them)."""
+    Forward: shrink, then the grouped GEMM with the LoRA term in its epilogue.  Backward: the grouped GEMM in its
+    transposing form on the same weights gives the base part of ``dx``; the segmented backward adds the LoRA part
+    onto it in place and yields the adapters' gradients.  The weights get no gradient (the reference freezes them)."""
 
     @staticmethod
-    def forward(ctx, x, weight, weight_t, seg, groups_per_expert, groups, *weights):
+    def forward(ctx, x, weight, seg, groups_per_expert, groups, *weights):
         h = None
         if groups is not None:
             h = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=x.device)
             lora_shrink_(x, seg, groups, h, map_rows=False)
         y = grouped_linear_(x, weight, seg, groups_per_expert, groups=groups, h=h, map_rows=False)
-        ctx.save_for_backward(x, weight_t, h)
+        ctx.save_for_backward(x, weight, h)
         ctx.seg, ctx.groups, ctx.groups_per_expert = seg, groups, groups_per_expert
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        x, weight_t, h = ctx.saved_tensors
+        x, weight, h = ctx.saved_tensors
         seg, groups = ctx.seg, ctx.groups
         dy = dy.contiguous()
         needs_dx = ctx.needs_input_grad[0]
-        dx = grouped_linear_(dy, weight_t, seg, ctx.groups_per_expert, map_rows=False) if needs_dx else None
+        dx = grouped_linear_(dy, weight, seg, ctx.groups_per_expert, map_rows=False, transposed=True) \
+            if needs_dx else None
         if groups is None:
-            return (dx, None, None, None, None, None)
+            return (dx, None, None, None, None)
         na, nb = len(groups.a_tensors), len(groups.b_tensors)
-        needs_a = any(ctx.needs_input_grad[6:6 + na])
-        needs_b = any(ctx.needs_input_grad[6 + na:6 + na + nb])
+        needs_a = any(ctx.needs_input_grad[5:5 + na])
+        needs_b = any(ctx.needs_input_grad[5 + na:5 + na + nb])
         arena_a, arena_b, pa, pb = _weight_grads(groups, needs_a, needs_b, dy.device)
         if needs_dx or needs_a or needs_b:
             lora_bwd_(dy, x, h, dx, pa, pb, seg, groups, False, accumulate=False)
         ga = groups.grad_views(arena_a, 'a') if needs_a else [None] * na
         gb = groups.grad_views(arena_b, 'b') if needs_b else [None] * nb
-        return (dx, None, None, None, None, None, *ga, *gb)
+        return (dx, None, None, None, None, *ga, *gb)
 
 
-def grouped_experts_linear(x: torch.Tensor, weight: torch.Tensor, weight_t: torch.Tensor, seg: SegmentTable,
-                           groups_per_expert: int, groups: Optional[AdapterGroups] = None) -> torch.Tensor:
+def grouped_experts_linear(x: torch.Tensor, weight: torch.Tensor, seg: SegmentTable, groups_per_expert: int,
+                           groups: Optional[AdapterGroups] = None) -> torch.Tensor:
     """``y = x W_e^T`` plus every (expert, tenant) group's LoRA term, for rows in segment order; differentiable in
-    ``x`` and the adapters.  ``weight_t`` is the ``[E, in, out]`` copy of the frozen ``weight [E, out, in]``."""
+    ``x`` and the adapters, not in the frozen ``weight [E, out, in]`` (both widths multiples of 128)."""
     extra = groups.autograd_tensors() if groups is not None else []
     if groups is not None:
         groups.sync_masters()
-    return _GroupedExpertsLinear.apply(x, weight, weight_t, seg, groups_per_expert, groups, *extra)
+    return _GroupedExpertsLinear.apply(x, weight, seg, groups_per_expert, groups, *extra)
 
 
 def multi_lora_delta(x: torch.Tensor, base_out: torch.Tensor, seg: SegmentTable, groups: AdapterGroups,
