@@ -219,3 +219,61 @@ def test_custom_op_matches_the_direct_call(dev):
                                          groups.rank_dev, groups.scale_dev, groups.max_rank, groups.lda, groups.ldb)
     assert torch.equal(y2, want_lora)
     assert not torch.equal(want_base, want_lora)
+
+
+def test_hip_graph_replay_of_the_grouped_calls(dev):
+    """Segment build, shrink, grouped GEMM with the LoRA term and the transposing backward call captured in one HIP
+    graph (no host synchronisation anywhere in them) and replayed with fresh inputs: every replay equals eager."""
+    e, nt, k, n, max_r = 4, 2, 256, 512, 16
+    t = 3000
+    g = torch.Generator().manual_seed(12)
+    a = [(torch.randn(e, max_r, k, generator=g) / k**0.5).bfloat16().to(dev) for _ in range(nt)]
+    b = [(torch.randn(e, n, max_r, generator=g) * 0.05).bfloat16().to(dev) for _ in range(nt)]
+    idx = [i % nt for i in range(e * nt)]
+    groups = AdapterGroups(a, b, [16, 5] * e, [2.0] * (e * nt),
+                           a_index=idx, a_offset=[(i // nt) * max_r * k for i in range(e * nt)],
+                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)])
+    w = (torch.randn(e, n, k, generator=g) / k**0.5).bfloat16().to(dev)
+    keys = torch.empty(t, dtype=torch.int32, device=dev)
+    x = torch.empty(t, k, dtype=torch.bfloat16, device=dev)
+    dy = torch.empty(t, n, dtype=torch.bfloat16, device=dev)
+
+    def fill(seed):
+        gg = torch.Generator().manual_seed(seed)
+        keys.copy_(torch.randint(0, e * nt, (t,), generator=gg).to(torch.int32))
+        x.copy_(torch.randn(t, k, generator=gg).bfloat16())
+        dy.copy_(torch.randn(t, n, generator=gg).bfloat16())
+
+    fill(0)
+    seg0 = build_segments(keys, e * nt, want_perm=False, want_offsets=False)
+    h = torch.empty(lora_h_bytes(seg0, groups), dtype=torch.uint8, device=dev)
+    y = torch.empty(t, n, dtype=torch.bfloat16, device=dev)
+    dx = torch.empty(t, k, dtype=torch.bfloat16, device=dev)
+
+    def step():
+        seg = build_segments(keys, e * nt, want_perm=False, want_offsets=False)
+        lora_shrink_(x, seg, groups, h, map_rows=True)
+        grouped_linear_(x, w, seg, nt, y=y, groups=groups, h=h, map_rows=True)
+        grouped_linear_(dy, w, seg, nt, y=dx, map_rows=True, transposed=True)
+
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                       # warm-up on the capture stream
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    for seed in (1, 2, 3):
+        fill(seed)
+        step()
+        torch.cuda.synchronize()
+        want_y, want_dx = y.clone(), dx.clone()
+        y.zero_()
+        dx.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want_y) and torch.equal(dx, want_dx), seed
