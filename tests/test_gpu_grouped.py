@@ -277,3 +277,60 @@ def test_hip_graph_replay_of_the_grouped_calls(dev):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(y, want_y) and torch.equal(dx, want_dx), seed
+
+
+def _random_grouped_case(seed):
+    g = torch.Generator().manual_seed(5000 + seed)
+    pick = lambda xs: xs[int(torch.randint(0, len(xs), (1,), generator=g))]  # noqa: E731
+    e = pick([1, 2, 3, 7, 16, 40])
+    nt = pick([1, 1, 2, 4])
+    t = pick([1, 31, 200, 1000, 2500, 6000])
+    k = pick([64, 128, 192, 256, 512, 1024])
+    n = pick([128, 256, 384, 512, 768, 1024])
+    max_r = pick([0, 8, 16, 32, 64])
+    return g, e, nt, t, k, n, max_r
+
+
+@pytest.mark.parametrize('seed', range(24))
+def test_random_shapes_of_the_grouped_gemm(dev, seed):
+    """Random expert counts, tenant counts, row counts (experts of no, few and thousands of rows), widths (both
+    block sizes) and ranks; the forward with the LoRA term where there is one, and the transposing backward
+    whenever in_features allows it as an output width."""
+    g, e, nt, t, k, n, max_r = _random_grouped_case(seed)
+    probs = torch.rand(e, generator=g) ** 3 + 1e-3
+    probs[torch.rand(e, generator=g) < 0.2] = 0
+    if probs.sum() == 0:
+        probs[0] = 1
+    expert = torch.multinomial(probs, t, replacement=True, generator=g)
+    tenant = torch.randint(0, nt, (t,), generator=g)
+    x = torch.randn(t, k, generator=g).bfloat16()
+    w = (torch.randn(e, n, k, generator=g) / k**0.5).bfloat16()
+    seg = build_segments((expert * nt + tenant).to(torch.int32).to(dev), e * nt)
+    xd, wd = x.to(dev), w.to(dev)
+    want = _reference(x, w, expert)
+    if max_r == 0:
+        got = grouped_linear_(xd, wd, seg, nt, map_rows=True)
+    else:
+        ranks = [int(torch.randint(0, max_r + 1, (1,), generator=g)) for _ in range(nt)]
+        ranks[0] = max_r
+        a = [(torch.randn(e, max_r, k, generator=g) / k**0.5).bfloat16().to(dev) for _ in range(nt)]
+        b = [(torch.randn(e, n, max_r, generator=g) * 0.05).bfloat16().to(dev) for _ in range(nt)]
+        idx = [i % nt for i in range(e * nt)]
+        groups = AdapterGroups(a, b, [ranks[i % nt] for i in range(e * nt)], [0.5] * (e * nt),
+                               a_index=idx, a_offset=[(i // nt) * max_r * k for i in range(e * nt)],
+                               b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)])
+        h = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=dev)
+        lora_shrink_(xd, seg, groups, h, map_rows=True)
+        got = grouped_linear_(xd, wd, seg, nt, groups=groups, h=h, map_rows=True)
+        for ei in range(e):
+            for ti in range(nt):
+                rows = ((expert == ei) & (tenant == ti)).nonzero().flatten()
+                r = ranks[ti]
+                if rows.numel() and r:
+                    want[rows] += 0.5 * (x.double()[rows] @ a[ti][ei, :r].double().cpu().t()) @ \
+                        b[ti][ei, :, :r].double().cpu().t()
+    assert max_rel_err(got, want) < 2e-2
+    if k % 128 == 0:                     # the backward of the base term: output width k, contraction over n
+        dy = torch.randn(t, n, generator=g).bfloat16()
+        dx = grouped_linear_(dy.to(dev), wd, seg, nt, map_rows=True, transposed=True)
+        assert max_rel_err(dx, _reference(dy, w.transpose(1, 2).contiguous(), expert)) < 6e-3
