@@ -278,6 +278,19 @@ int tk_grouped_linear(const tk_grouped_desc* desc, const tk_lora_desc* lora, con
                       void* y_device, int64_t ldy, const void* h_device, void* workspace_device,
                       int64_t workspace_bytes, tk_stream_t stream);
 
+/* ---- gated activation of the packed experts --------------------------------------------------------------
+ *
+ * hidden[row][c] = silu(gate_up[row][c]) * gate_up[row][inter + c], c < inter: what the reference computes
+ * between the two expert projections as `gate, up = gate_up_out.chunk(2, -1); act_fn(gate) * up` with
+ * act_fn = SiLU (moe/expert_parallel.py:363-366), in one pass, fp32 arithmetic, one rounding.
+ * tk_swiglu_bwd writes d(gate | up) from gate_up and d(hidden).  bf16 or fp32; inter and the row strides
+ * multiples of 8 elements, pointers aligned to 8 elements: TK_ERR_UNSUPPORTED otherwise. */
+int tk_swiglu_fwd(const void* gate_up_device, int64_t ld_gate_up, void* hidden_device, int64_t ld_hidden,
+                  int64_t rows, int32_t inter, int32_t dtype, tk_stream_t stream);
+int tk_swiglu_bwd(const void* gate_up_device, int64_t ld_gate_up, const void* dhidden_device, int64_t ld_dhidden,
+                  void* dgate_up_device, int64_t ld_dgate_up, int64_t rows, int32_t inter, int32_t dtype,
+                  tk_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -23,6 +23,7 @@ unpermute                                                  : pinned
     (index_add_ closed form; permute∘unpermute identity)
 lora_linear_forward / multi_lora_linear / grads            : pinned
     (fp64 closed form, gradcheck, B=0, r<max_r, single segment ≡ F.linear)
+swiglu                                                     : pinned (x sigmoid(x) u in closed form, gradcheck)
 expert_delta_weight / expert_lora_low_rank / experts_linear : pinned
     (merged-weight form ≡ low-rank form; shape KAT of the reference test; the chunk loop
     against a row-by-row product with each row's own expert and against one F.linear for E = 1)
@@ -53,6 +54,7 @@ from .lora import (  # noqa: F401
     expert_delta_weight,
     expert_lora_low_rank,
     experts_linear,
+    swiglu,
     lora_linear_forward,
     lora_scaling,
     match_target_modules,

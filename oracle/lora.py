@@ -118,6 +118,15 @@ def experts_linear(x_sorted: torch.Tensor, offsets: torch.Tensor, weight: torch.
     return torch.cat(chunks, dim=0) if chunks else x_sorted.new_empty(0, weight.shape[1])
 
 
+def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
+    """``act_fn(gate) * up`` with ``gate, up = gate_up.chunk(2, dim=-1)`` and ``act_fn = SiLU``.
+
+    Follows src/twinkle/model/transformers/moe/expert_parallel.py:363-366 (the branch without ``_apply_gate``).
+    """
+    gate, up = gate_up.chunk(2, dim=-1)
+    return F.silu(gate) * up
+
+
 def expert_lora_low_rank(x_sorted: torch.Tensor, offsets: torch.Tensor, base_out: torch.Tensor, lora_A: torch.Tensor,
                          lora_B: torch.Tensor, r: int, scaling: float) -> torch.Tensor:
     """``y_e = base_e + s (x_e A_e^T) B_e^T`` over contiguous per-expert chunks.

@@ -161,6 +161,15 @@ def test_entry_points_reject_malformed_arguments_on_the_host():
     g.weight_layout = 0
     g.rows, g.weight_stride = 0, 256 * 128
     assert lib.tk_grouped_linear(gref, None, None, 128, None, 256, None, None, 0, None) == _lib.TK_OK  # nothing to do
+    # gated activation
+    assert lib.tk_swiglu_fwd(P, 32, P, 16, -1, 16, 1, None) == bad                            # negative rows
+    assert lib.tk_swiglu_fwd(P, 31, P, 16, 4, 16, 1, None) == bad                             # ld below 2 * inter
+    assert lib.tk_swiglu_fwd(P, 32, None, 16, 4, 16, 1, None) == bad                          # no output
+    assert lib.tk_swiglu_fwd(P, 32, P, 16, 4, 16, 7, None) == bad                             # unknown dtype
+    assert lib.tk_swiglu_fwd(P, 24, P, 12, 4, 12, 1, None) == unsupported                     # inter not a multiple of 8
+    assert lib.tk_swiglu_bwd(P, 32, None, 16, P, 32, 4, 16, 1, None) == bad                   # no d(hidden)
+    assert lib.tk_swiglu_bwd(P, 32, P, 16, P, 31, 4, 16, 1, None) == bad                      # ld of d(gate | up)
+    assert lib.tk_swiglu_fwd(None, 32, None, 16, 0, 16, 1, None) == _lib.TK_OK                # nothing to do
     # optimizer
     assert lib.tk_opt_workspace_bytes(-1, 10) == bad
     assert lib.tk_opt_grad_norm(P, 4, P, 0, 100, 1, P, P, P, 1 << 20, None) == bad           # no tenants

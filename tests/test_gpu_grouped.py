@@ -334,3 +334,32 @@ def test_random_shapes_of_the_grouped_gemm(dev, seed):
         dy = torch.randn(t, n, generator=g).bfloat16()
         dx = grouped_linear_(dy.to(dev), wd, seg, nt, map_rows=True, transposed=True)
         assert max_rel_err(dx, _reference(dy, w.transpose(1, 2).contiguous(), expert)) < 6e-3
+
+
+@pytest.mark.parametrize('dtype,tol', [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize('rows,inter', [(1, 8), (37, 24), (1000, 768), (5000, 1408)])
+def test_swiglu_forward_and_backward(dev, dtype, tol, rows, inter):
+    """silu(gate) * up in one pass and its backward against the oracle in float64 on the same rounded inputs."""
+    from twinkle_amd import swiglu
+    g = torch.Generator().manual_seed(rows + inter)
+    gu = (torch.randn(rows, 2 * inter, generator=g) * 2).to(dtype)
+    dout = torch.randn(rows, inter, generator=g).to(dtype)
+    gud = gu.to(dev).requires_grad_(True)
+    out = swiglu(gud)
+    out.backward(dout.to(dev))
+    gu64 = gu.double().requires_grad_(True)
+    want = oracle.swiglu(gu64)
+    want.backward(dout.double())
+    assert out.dtype == dtype and max_rel_err(out, want) < tol
+    assert max_rel_err(gud.grad, gu64.grad) < tol
+
+
+def test_swiglu_refuses_what_it_cannot_vectorise(dev):
+    from twinkle_amd import swiglu
+    from twinkle_amd.ops import swiglu_applies
+    bad = torch.zeros(4, 20, dtype=torch.bfloat16, device=dev)           # inter = 10
+    assert not swiglu_applies(bad)
+    with pytest.raises(ValueError):
+        swiglu(bad)
+    assert swiglu_applies(torch.zeros(4, 32, dtype=torch.bfloat16, device=dev))
+    assert not swiglu_applies(torch.zeros(4, 32, dtype=torch.float16, device=dev))

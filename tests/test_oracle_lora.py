@@ -141,6 +141,15 @@ def test_experts_linear_is_each_rows_own_expert():
     assert torch.equal(one, F.linear(x, w[0]))
 
 
+def test_swiglu_closed_form_and_gradient():
+    g = torch.Generator().manual_seed(6)
+    gu = torch.randn(5, 8, generator=g, dtype=torch.double, requires_grad=True)
+    gate, up = gu[:, :4], gu[:, 4:]
+    want = gate / (1 + torch.exp(-gate)) * up
+    assert torch.allclose(oracle.swiglu(gu), want, atol=1e-14)
+    assert torch.autograd.gradcheck(oracle.swiglu, (gu,))
+
+
 def test_slice_copy_round_trip():
     g = torch.Generator().manual_seed(8)
     for name, shape, r in [('m.lora_A.weight', (8, 5), 3), ('m.lora_B.weight', (5, 8), 3),

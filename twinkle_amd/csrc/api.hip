@@ -430,6 +430,25 @@ int tk_grouped_linear(const tk_grouped_desc* g, const tk_lora_desc* lora, const 
                              (hipStream_t)stream);
 }
 
+// ---- gated activation ---------------------------------------------------------------------------------------------
+
+int tk_swiglu_fwd(const void* gu, int64_t ld_in, void* out, int64_t ld_out, int64_t rows, int32_t inter, int32_t dtype,
+                  tk_stream_t stream) {
+  if (rows < 0 || inter <= 0 || (dtype != TK_DTYPE_F32 && dtype != TK_DTYPE_BF16)) return TK_ERR_INVALID;
+  if (rows == 0) return TK_OK;
+  if (!gu || !out || ld_in < 2 * (int64_t)inter || ld_out < inter) return TK_ERR_INVALID;
+  return launch_swiglu(gu, ld_in, nullptr, 0, out, ld_out, rows, inter, dtype, (hipStream_t)stream);
+}
+
+int tk_swiglu_bwd(const void* gu, int64_t ld_in, const void* dout, int64_t ld_dout, void* dgu, int64_t ld_dgu,
+                  int64_t rows, int32_t inter, int32_t dtype, tk_stream_t stream) {
+  if (rows < 0 || inter <= 0 || (dtype != TK_DTYPE_F32 && dtype != TK_DTYPE_BF16)) return TK_ERR_INVALID;
+  if (rows == 0) return TK_OK;
+  if (!gu || !dout || !dgu || ld_in < 2 * (int64_t)inter || ld_dout < inter || ld_dgu < 2 * (int64_t)inter)
+    return TK_ERR_INVALID;
+  return launch_swiglu(gu, ld_in, dout, ld_dout, dgu, ld_dgu, rows, inter, dtype, (hipStream_t)stream);
+}
+
 // ---- projections that share their input ------------------------------------------------------------------------
 
 static bool shared_descs_ok(const tk_lora_desc* const* descs, int32_t n) {

@@ -310,6 +310,10 @@ int64_t grouped_plan_entries(const SegLayout& L, int64_t experts);
 int launch_grouped_gemm(const GroupedArgs& a, int experts, int nt, GroupedPlanEntry* plan, int32_t* nblocks,
                         const SegView& seg, const SegLayout& L, hipStream_t s);
 
+// kernels_act.hip: out = silu(gate) * up (dout null) or its backward into out = d(gate | up)
+int launch_swiglu(const void* gate_up, int64_t ld_in, const void* dout, int64_t ld_dout, void* out, int64_t ld_out,
+                  int64_t rows, int inter, int dtype, hipStream_t s);
+
 // kernels_segments.hip
 int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t groups, int64_t* perm_out,
                          int64_t* offsets_out, void* ws, hipStream_t s);

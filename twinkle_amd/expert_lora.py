@@ -290,6 +290,22 @@ class ExpertLoraManager:
         return consumed
 
 
+def _is_silu(fn) -> bool:
+    return fn is torch.nn.functional.silu or isinstance(fn, nn.SiLU)
+
+
+def _gated_activation(experts_mod: nn.Module, gate_up_out: torch.Tensor, fused: bool = True) -> torch.Tensor:
+    """``_apply_gate`` if the module has one, else ``act_fn(gate) * up`` (moe/expert_parallel.py:363-366); with
+    SiLU on the GPU the one-pass kernel does the same arithmetic in fp32 with one rounding."""
+    from .ops import swiglu, swiglu_applies
+    if hasattr(experts_mod, '_apply_gate'):
+        return experts_mod._apply_gate(gate_up_out)
+    if fused and _is_silu(experts_mod.act_fn) and swiglu_applies(gate_up_out):
+        return swiglu(gate_up_out)
+    gate, up = gate_up_out.chunk(2, dim=-1)
+    return experts_mod.act_fn(gate) * up
+
+
 def grouped_gemm_applies(weight: torch.Tensor, rows: torch.Tensor) -> bool:
     """Frozen bf16 packed weights whose two widths are multiples of 128: what ``tk_grouped_linear`` takes in the
     forward direction (``in`` a multiple of 64, ``out`` of 128) and, with the roles swapped, in the backward one."""
@@ -299,7 +315,8 @@ def grouped_gemm_applies(weight: torch.Tensor, rows: torch.Tensor) -> bool:
 
 def experts_forward(experts_mod: nn.Module, rows: torch.Tensor, seg: SegmentTable, tenant_slots: Sequence[str],
                     gate_up_slots: Optional[ExpertLoraSlots] = None,
-                    down_slots: Optional[ExpertLoraSlots] = None, grouped: Optional[bool] = None) -> torch.Tensor:
+                    down_slots: Optional[ExpertLoraSlots] = None, grouped: Optional[bool] = None,
+                    fused_activation: bool = True) -> torch.Tensor:
     """Packed experts on rows in (expert, tenant) segment order, every tenant's LoRA terms included.
 
     The per-expert loop of the reference's expert forward (moe/expert_parallel.py:333-378: ``F.linear`` with
@@ -314,6 +331,7 @@ def experts_forward(experts_mod: nn.Module, rows: torch.Tensor, seg: SegmentTabl
     64 / 128 in both directions) replaces the loop by one grouped GEMM per projection with the LoRA terms in its
     epilogue: no host copy of the boundaries at all, one launch instead of one per expert, and the expert outputs
     are written once.  Its backward runs the same kernel in its transposing form on the same weights.
+    ``fused_activation`` lets a SiLU gate run as one kernel forward and one backward instead of torch's five.
     """
     if rows.shape[0] == 0:
         return rows                                                   # keeps the autograd edge (reference :340-344)
@@ -332,11 +350,7 @@ def experts_forward(experts_mod: nn.Module, rows: torch.Tensor, seg: SegmentTabl
         x = x.contiguous()
         gate_up_out = grouped_experts_linear(x, gate_up, seg, nt,
                                              gate_up_slots.groups(tenant_slots) if gate_up_slots is not None else None)
-        if hasattr(experts_mod, '_apply_gate'):
-            hidden = experts_mod._apply_gate(gate_up_out)
-        else:
-            gate, up = gate_up_out.chunk(2, dim=-1)
-            hidden = experts_mod.act_fn(gate) * up
+        hidden = _gated_activation(experts_mod, gate_up_out, fused_activation)
         out = grouped_experts_linear(hidden.contiguous(), down, seg, nt,
                                      down_slots.groups(tenant_slots) if down_slots is not None else None)
         return out if out.dtype == input_dtype else out.to(input_dtype)
@@ -352,12 +366,7 @@ def experts_forward(experts_mod: nn.Module, rows: torch.Tensor, seg: SegmentTabl
     gate_up_out = per_expert(x, gate_up)
     if gate_up_slots is not None:
         gate_up_out = expert_lora_delta(x, gate_up_out, seg, gate_up_slots, tenant_slots)
-    if hasattr(experts_mod, '_apply_gate'):
-        hidden = experts_mod._apply_gate(gate_up_out)
-    else:
-        gate, up = gate_up_out.chunk(2, dim=-1)
-        hidden = experts_mod.act_fn(gate) * up
-    hidden = hidden.contiguous()
+    hidden = _gated_activation(experts_mod, gate_up_out, fused_activation).contiguous()
     out = per_expert(hidden, down)
     if down_slots is not None:
         out = expert_lora_delta(hidden, out, seg, down_slots, tenant_slots)

@@ -369,6 +369,47 @@ class _LoraLinear(torch.autograd.Function):
         return (dx, dw, db, None, None, None, *ga, *gb)
 
 
+class _SwiGLU(torch.autograd.Function):
+    """``silu(gate) * up`` for ``gate | up`` side by side in the rows of one tensor (see ``tk_swiglu_fwd``)."""
+
+    @staticmethod
+    def forward(ctx, gate_up):
+        rows, two_i = gate_up.shape
+        inter = two_i // 2
+        out = torch.empty(rows, inter, dtype=gate_up.dtype, device=gate_up.device)
+        code = _lib.load().tk_swiglu_fwd(gate_up.data_ptr(), gate_up.stride(0), out.data_ptr(), out.stride(0), rows,
+                                         inter, _lib.dtype_code(gate_up.dtype), _lib.stream_ptr())
+        _lib.check(code, 'tk_swiglu_fwd')
+        ctx.save_for_backward(gate_up)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        gate_up, = ctx.saved_tensors
+        dout = dout.contiguous()
+        rows, two_i = gate_up.shape
+        dgu = torch.empty_like(gate_up)
+        code = _lib.load().tk_swiglu_bwd(gate_up.data_ptr(), gate_up.stride(0), dout.data_ptr(), dout.stride(0),
+                                         dgu.data_ptr(), dgu.stride(0), rows, two_i // 2,
+                                         _lib.dtype_code(gate_up.dtype), _lib.stream_ptr())
+        _lib.check(code, 'tk_swiglu_bwd')
+        return dgu
+
+
+def swiglu_applies(gate_up: torch.Tensor) -> bool:
+    """Shapes the fused gated activation takes: 2-D, unit inner stride, ``inter`` and the row stride multiples of 8."""
+    return (gate_up.is_cuda and gate_up.dim() == 2 and gate_up.stride(1) == 1 and gate_up.shape[1] % 16 == 0 and
+            gate_up.stride(0) % 8 == 0 and gate_up.dtype in (torch.float32, torch.bfloat16) and
+            gate_up.data_ptr() % (8 * gate_up.element_size()) == 0)
+
+
+def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
+    """``F.silu(gate) * up`` with ``gate, up = gate_up.chunk(2, -1)`` in one pass (and one in backward)."""
+    if not gate_up.is_cuda:
+        raise RuntimeError('gate_up must live on the GPU: this path has no CPU implementation')
+    return _SwiGLU.apply(gate_up)
+
+
 class _GroupedExpertsLinear(torch.autograd.Function):
     """Frozen packed expert weights and the (expert, tenant) LoRA terms as one node on rows in segment order.
 
