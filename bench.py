@@ -270,10 +270,22 @@ def moe_experts_bench(dev, steps=10):
         y = grouped_linear_(x0, experts.gate_up_proj, seg, nt)
         grouped_linear_(y[:, :inter].contiguous(), experts.down_proj, seg, nt)
 
+    # the whole block from the router's outputs: segment build, permute, experts, weighted unpermute, and back
+    from twinkle_amd.expert_lora import moe_experts_block
+    tok0 = torch.randn(tokens, hid, generator=gen).to(dt).to(dev)
+    dtok = torch.randn(tokens, hid, generator=gen).to(dt).to(dev)
+    sel_d, tenant_d = sel.to(dev), tenant.to(dev)
+    rw = torch.softmax(torch.randn(tokens, top_k, generator=gen), -1).to(dt).to(dev)
+
+    def block():
+        t = tok0.detach().requires_grad_(True)
+        out = moe_experts_block(t, sel_d, rw, tenant_d, experts, names, gu, dn)
+        out.backward(dtok)
+
     res = {}
     for name, fn in (('loop_fwd_ms', lambda: fwd(False)), ('grouped_fwd_ms', lambda: fwd(True)),
                      ('loop_fwd_bwd_ms', lambda: fwd_bwd(False)), ('grouped_fwd_bwd_ms', lambda: fwd_bwd(True)),
-                     ('grouped_gemms_alone_ms', base_only)):
+                     ('grouped_gemms_alone_ms', base_only), ('block_from_router_fwd_bwd_ms', block)):
         for _ in range(3):
             fn()
         torch.cuda.synchronize()
@@ -290,7 +302,8 @@ def moe_experts_bench(dev, steps=10):
                 'mfma_frac_grouped_gemms': flops_fwd / (res['grouped_gemms_alone_ms'] * 1e-3) / 1e12 / 2500.0,
                 'speedup_fwd': res['loop_fwd_ms'] / res['grouped_fwd_ms'],
                 'speedup_fwd_bwd': res['loop_fwd_bwd_ms'] / res['grouped_fwd_bwd_ms'],
-                'routed_rows_per_s_fwd_bwd': rows / (res['grouped_fwd_bwd_ms'] * 1e-3)})
+                'routed_rows_per_s_fwd_bwd': rows / (res['grouped_fwd_bwd_ms'] * 1e-3),
+                'tokens_per_s_block_fwd_bwd': tokens / (res['block_from_router_fwd_bwd_ms'] * 1e-3)})
     return res
 
 
