@@ -13,6 +13,8 @@
 //                 padding of slot_row
 //   k_seg_scatter one wave per 512 rows: stable rank inside the wave by
 //                 bit-sliced ballots, cursor per group in LDS -> inv, slot_row
+#include <initializer_list>
+
 #include "tk_device.h"
 
 namespace tk {
@@ -447,8 +449,16 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
   }
 }
 
+// 16 bytes of a row: the unit the row movers below load and store when width, strides and pointers allow
+// (V = 8 bf16 / 4 fp32 elements), else V = 1.  The arithmetic per element and the order of every sum are the
+// same for both.
+template <typename T, int V>
+struct alignas(V * sizeof(T)) RowVec {
+  T v[V];
+};
+
 // dst[j] = src[perm[j] mod tokens] * w[token, k], one block per padded slot (slot_row is perm in padded order)
-template <typename T>
+template <typename T, int V>
 __global__ __launch_bounds__(256) void k_permute(const T* __restrict__ src, int64_t ld_src, T* __restrict__ dst,
                                                  int64_t ld_dst, const T* __restrict__ w,
                                                  const int32_t* __restrict__ slot_row,
@@ -458,41 +468,56 @@ __global__ __launch_bounds__(256) void k_permute(const T* __restrict__ src, int6
   const int j = slot_pos[blockIdx.x];
   if (f < 0 || j < 0) return;
   const int t = f % tokens, k = f / tokens;
-  const T* s = src + (int64_t)t * ld_src;
-  T* d = dst + (int64_t)j * ld_dst;
+  const RowVec<T, V>* s = reinterpret_cast<const RowVec<T, V>*>(src + (int64_t)t * ld_src);
+  RowVec<T, V>* d = reinterpret_cast<RowVec<T, V>*>(dst + (int64_t)j * ld_dst);
   if (w) {
     const float wt = to_f32(w[(int64_t)t * top_k + k]);
-    for (int c = threadIdx.x; c < width; c += 256) from_f32(to_f32(s[c]) * wt, &d[c]);
+    for (int c = threadIdx.x; c < width / V; c += 256) {
+      RowVec<T, V> x = s[c];
+#pragma unroll
+      for (int i = 0; i < V; ++i) from_f32(to_f32(x.v[i]) * wt, &x.v[i]);
+      d[c] = x;
+    }
   } else {
-    for (int c = threadIdx.x; c < width; c += 256) d[c] = s[c];
+    for (int c = threadIdx.x; c < width / V; c += 256) d[c] = s[c];
   }
 }
 
 // out[t] = sum_k rows[inv[k * tokens + t]] * w[t, k], k ascending, fp32 accumulation
-template <typename T>
+template <typename T, int V>
 __global__ __launch_bounds__(256) void k_unpermute(const T* __restrict__ rows_, int64_t ld_rows, T* __restrict__ out,
                                                    int64_t ld_out, const T* __restrict__ w,
                                                    const int32_t* __restrict__ inv, int tokens, int top_k, int width) {
   const int t = blockIdx.x;
   if (t >= tokens) return;
-  for (int c = threadIdx.x; c < width; c += 256) {
-    float acc = 0.f;
+  for (int c = threadIdx.x; c < width / V; c += 256) {
+    float acc[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[i] = 0.f;
     for (int k = 0; k < top_k; ++k) {
       const int j = inv[(int64_t)k * tokens + t];
-      float v = to_f32(rows_[(int64_t)j * ld_rows + c]);
-      if (w) {
-        // the reference scales the row in the activation dtype before adding (ep_utils.py:142)
-        T r;
-        from_f32(v * to_f32(w[(int64_t)t * top_k + k]), &r);
-        v = to_f32(r);
+      const RowVec<T, V> x = reinterpret_cast<const RowVec<T, V>*>(rows_ + (int64_t)j * ld_rows)[c];
+      const float wt = w ? to_f32(w[(int64_t)t * top_k + k]) : 1.f;
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        float v = to_f32(x.v[i]);
+        if (w) {
+          // the reference scales the row in the activation dtype before adding (ep_utils.py:142)
+          T r;
+          from_f32(v * wt, &r);
+          v = to_f32(r);
+        }
+        acc[i] += v;
       }
-      acc += v;
     }
-    from_f32(acc, &out[(int64_t)t * ld_out + c]);
+    RowVec<T, V> o;
+#pragma unroll
+    for (int i = 0; i < V; ++i) from_f32(acc[i], &o.v[i]);
+    reinterpret_cast<RowVec<T, V>*>(out + (int64_t)t * ld_out)[c] = o;
   }
 }
 
-template <typename T>
+template <typename T, int V>
 __global__ __launch_bounds__(64) void k_unpermute_wgrad(const T* __restrict__ dout, int64_t ld_dout,
                                                         const T* __restrict__ rows_, int64_t ld_rows,
                                                         float* __restrict__ dw, const int32_t* __restrict__ inv,
@@ -500,12 +525,29 @@ __global__ __launch_bounds__(64) void k_unpermute_wgrad(const T* __restrict__ do
   const int f = blockIdx.x;  // flat row k * tokens + t
   const int t = f % tokens, k = f / tokens;
   const int j = inv[f];
+  const RowVec<T, V>* a = reinterpret_cast<const RowVec<T, V>*>(dout + (int64_t)t * ld_dout);
+  const RowVec<T, V>* b = reinterpret_cast<const RowVec<T, V>*>(rows_ + (int64_t)j * ld_rows);
   float acc = 0.f;
-  for (int c = threadIdx.x; c < width; c += 64)
-    acc += to_f32(dout[(int64_t)t * ld_dout + c]) * to_f32(rows_[(int64_t)j * ld_rows + c]);
+  for (int c = threadIdx.x; c < width / V; c += 64) {
+    const RowVec<T, V> x = a[c], y = b[c];
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc += to_f32(x.v[i]) * to_f32(y.v[i]);
+  }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) acc += __shfl_xor(acc, d, 64);
   if (threadIdx.x == 0) dw[(int64_t)t * top_k + k] = acc;
+}
+
+// whether rows of `width` elements at these strides and addresses can move in 16-byte pieces
+template <typename T>
+inline bool rows_vectorise(int width, std::initializer_list<int64_t> lds, std::initializer_list<const void*> ptrs) {
+  constexpr int V = 16 / (int)sizeof(T);
+  if (width % V != 0) return false;
+  for (int64_t ld : lds)
+    if (ld % V != 0) return false;
+  for (const void* p : ptrs)
+    if (reinterpret_cast<uintptr_t>(p) & 15u) return false;
+  return true;
 }
 
 }  // namespace
@@ -546,18 +588,30 @@ int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t 
   return check_launch();
 }
 
+// T = element type; the kernel is instantiated for 16-byte pieces and for single elements
+#define TK_ROW_MOVER(KERNEL, T, VEC_OK, GRID, BLOCK, ...)                                    \
+  do {                                                                                       \
+    if (VEC_OK)                                                                              \
+      hipLaunchKernelGGL((KERNEL<T, 16 / (int)sizeof(T)>), GRID, BLOCK, 0, s, __VA_ARGS__);  \
+    else                                                                                     \
+      hipLaunchKernelGGL((KERNEL<T, 1>), GRID, BLOCK, 0, s, __VA_ARGS__);                    \
+  } while (0)
+
 int launch_permute(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, const void* w, const void* ws,
                    int64_t rows, int64_t tokens, int32_t width, int32_t groups, int dtype, hipStream_t s) {
   if (rows == 0) return TK_OK;
   SegLayout L(rows, groups);
   SegView V(ws, L);
   const int top_k = (int)(rows / tokens);
+  const dim3 grid((unsigned)L.slots), block(256);
   if (dtype == TK_DTYPE_F32)
-    hipLaunchKernelGGL(k_permute<float>, dim3((unsigned)L.slots), dim3(256), 0, s, (const float*)src, ld_src,
-                       (float*)dst, ld_dst, (const float*)w, V.slot_row, V.slot_pos, (int)tokens, top_k, width);
+    TK_ROW_MOVER(k_permute, float, rows_vectorise<float>(width, {ld_src, ld_dst}, {src, dst}), grid, block,
+                 (const float*)src, ld_src, (float*)dst, ld_dst, (const float*)w, V.slot_row, V.slot_pos, (int)tokens,
+                 top_k, width);
   else
-    hipLaunchKernelGGL(k_permute<uint16_t>, dim3((unsigned)L.slots), dim3(256), 0, s, (const uint16_t*)src, ld_src,
-                       (uint16_t*)dst, ld_dst, (const uint16_t*)w, V.slot_row, V.slot_pos, (int)tokens, top_k, width);
+    TK_ROW_MOVER(k_permute, uint16_t, rows_vectorise<uint16_t>(width, {ld_src, ld_dst}, {src, dst}), grid, block,
+                 (const uint16_t*)src, ld_src, (uint16_t*)dst, ld_dst, (const uint16_t*)w, V.slot_row, V.slot_pos,
+                 (int)tokens, top_k, width);
   return check_launch();
 }
 
@@ -567,12 +621,14 @@ int launch_unpermute(const void* rows_, int64_t ld_rows, void* out, int64_t ld_o
   SegLayout L(rows, groups);
   SegView V(ws, L);
   const int top_k = (int)(rows / tokens);
+  const dim3 grid((unsigned)tokens), block(256);
   if (dtype == TK_DTYPE_F32)
-    hipLaunchKernelGGL(k_unpermute<float>, dim3((unsigned)tokens), dim3(256), 0, s, (const float*)rows_, ld_rows,
-                       (float*)out, ld_out, (const float*)w, V.inv, (int)tokens, top_k, width);
+    TK_ROW_MOVER(k_unpermute, float, rows_vectorise<float>(width, {ld_rows, ld_out}, {rows_, out}), grid, block,
+                 (const float*)rows_, ld_rows, (float*)out, ld_out, (const float*)w, V.inv, (int)tokens, top_k, width);
   else
-    hipLaunchKernelGGL(k_unpermute<uint16_t>, dim3((unsigned)tokens), dim3(256), 0, s, (const uint16_t*)rows_,
-                       ld_rows, (uint16_t*)out, ld_out, (const uint16_t*)w, V.inv, (int)tokens, top_k, width);
+    TK_ROW_MOVER(k_unpermute, uint16_t, rows_vectorise<uint16_t>(width, {ld_rows, ld_out}, {rows_, out}), grid, block,
+                 (const uint16_t*)rows_, ld_rows, (uint16_t*)out, ld_out, (const uint16_t*)w, V.inv, (int)tokens, top_k,
+                 width);
   return check_launch();
 }
 
@@ -583,13 +639,17 @@ int launch_unpermute_wgrad(const void* dout, int64_t ld_dout, const void* rows_,
   SegLayout L(rows, groups);
   SegView V(ws, L);
   const int top_k = (int)(rows / tokens);
+  const dim3 grid((unsigned)rows), block(64);
   if (dtype == TK_DTYPE_F32)
-    hipLaunchKernelGGL(k_unpermute_wgrad<float>, dim3((unsigned)rows), dim3(64), 0, s, (const float*)dout, ld_dout,
-                       (const float*)rows_, ld_rows, dw, V.inv, (int)tokens, top_k, width);
+    TK_ROW_MOVER(k_unpermute_wgrad, float, rows_vectorise<float>(width, {ld_dout, ld_rows}, {dout, rows_}), grid, block,
+                 (const float*)dout, ld_dout, (const float*)rows_, ld_rows, dw, V.inv, (int)tokens, top_k, width);
   else
-    hipLaunchKernelGGL(k_unpermute_wgrad<uint16_t>, dim3((unsigned)rows), dim3(64), 0, s, (const uint16_t*)dout,
-                       ld_dout, (const uint16_t*)rows_, ld_rows, dw, V.inv, (int)tokens, top_k, width);
+    TK_ROW_MOVER(k_unpermute_wgrad, uint16_t, rows_vectorise<uint16_t>(width, {ld_dout, ld_rows}, {dout, rows_}), grid,
+                 block, (const uint16_t*)dout, ld_dout, (const uint16_t*)rows_, ld_rows, dw, V.inv, (int)tokens, top_k,
+                 width);
   return check_launch();
 }
+
+#undef TK_ROW_MOVER
 
 }  // namespace tk
