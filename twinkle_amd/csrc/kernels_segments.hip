@@ -457,29 +457,31 @@ struct alignas(V * sizeof(T)) RowVec {
   T v[V];
 };
 
-// dst[j] = src[perm[j] mod tokens] * w[token, k], one block per padded slot (slot_row is perm in padded order)
+// dst[j] = src[perm[j] mod tokens] * w[token, k], one wave per padded slot (slot_row is perm in padded order)
 template <typename T, int V>
 __global__ __launch_bounds__(256) void k_permute(const T* __restrict__ src, int64_t ld_src, T* __restrict__ dst,
                                                  int64_t ld_dst, const T* __restrict__ w,
                                                  const int32_t* __restrict__ slot_row,
                                                  const int32_t* __restrict__ slot_pos, int tokens, int top_k,
-                                                 int width) {
-  const int f = slot_row[blockIdx.x];
-  const int j = slot_pos[blockIdx.x];
+                                                 int width, int slots) {
+  const int slot = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (slot >= slots) return;
+  const int f = slot_row[slot];
+  const int j = slot_pos[slot];
   if (f < 0 || j < 0) return;
   const int t = f % tokens, k = f / tokens;
   const RowVec<T, V>* s = reinterpret_cast<const RowVec<T, V>*>(src + (int64_t)t * ld_src);
   RowVec<T, V>* d = reinterpret_cast<RowVec<T, V>*>(dst + (int64_t)j * ld_dst);
   if (w) {
     const float wt = to_f32(w[(int64_t)t * top_k + k]);
-    for (int c = threadIdx.x; c < width / V; c += 256) {
+    for (int c = lane; c < width / V; c += 64) {
       RowVec<T, V> x = s[c];
 #pragma unroll
       for (int i = 0; i < V; ++i) from_f32(to_f32(x.v[i]) * wt, &x.v[i]);
       d[c] = x;
     }
   } else {
-    for (int c = threadIdx.x; c < width / V; c += 256) d[c] = s[c];
+    for (int c = lane; c < width / V; c += 64) d[c] = s[c];
   }
 }
 
@@ -603,15 +605,15 @@ int launch_permute(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, c
   SegLayout L(rows, groups);
   SegView V(ws, L);
   const int top_k = (int)(rows / tokens);
-  const dim3 grid((unsigned)L.slots), block(256);
+  const dim3 grid((unsigned)ceil_div(L.slots, 4)), block(256);
   if (dtype == TK_DTYPE_F32)
     TK_ROW_MOVER(k_permute, float, rows_vectorise<float>(width, {ld_src, ld_dst}, {src, dst}), grid, block,
                  (const float*)src, ld_src, (float*)dst, ld_dst, (const float*)w, V.slot_row, V.slot_pos, (int)tokens,
-                 top_k, width);
+                 top_k, width, (int)L.slots);
   else
     TK_ROW_MOVER(k_permute, uint16_t, rows_vectorise<uint16_t>(width, {ld_src, ld_dst}, {src, dst}), grid, block,
                  (const uint16_t*)src, ld_src, (uint16_t*)dst, ld_dst, (const uint16_t*)w, V.slot_row, V.slot_pos,
-                 (int)tokens, top_k, width);
+                 (int)tokens, top_k, width, (int)L.slots);
   return check_launch();
 }
 
