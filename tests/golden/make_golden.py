@@ -55,7 +55,37 @@ def segment_cases():
     return cases
 
 
+def experts_inputs():
+    """Inputs of the packed-experts fixture, from integer formulas instead of stored numbers (the weights alone
+    would be 16 k values): coarse-grid values, exactly representable in bf16."""
+    e, nt, t, k, n, inter = 2, 2, 12, 64, 128, 64
+    ar = torch.arange
+    x = ((ar(t)[:, None] * 5 + ar(k)[None, :] * 3) % 17 - 8).double() / 8
+    w = ((ar(e)[:, None, None] * 7 + ar(n)[None, :, None] * 3 + ar(k)[None, None, :] * 5) % 13 - 6).double() / 16
+    expert = torch.tensor([1, 0, 0, 1, 1, 0, 1, 1, 0, 1, 0, 1])
+    tenant = torch.tensor([0, 1, 1, 0, 1, 0, 0, 1, 1, 1, 0, 0])
+    return {'experts': e, 'tenants': nt, 'tokens': t, 'in': k, 'out': n, 'inter': inter,
+            'x': x, 'w': w, 'expert': expert, 'tenant': tenant}
+
+
+def experts_case():
+    c = experts_inputs()
+    order = torch.argsort(c['expert'], stable=True)
+    counts = torch.bincount(c['expert'], minlength=c['experts'])
+    offsets = torch.cat([torch.zeros(1, dtype=torch.long), counts.cumsum(0)])
+    y_sorted = oracle.experts_linear(c['x'][order], offsets, c['w'])
+    y = torch.empty_like(y_sorted)
+    y[order] = y_sorted
+    return {'inputs': 'tests/golden/make_golden.py::experts_inputs (integer formulas)',
+            'shape': {k: c[k] for k in ('experts', 'tenants', 'tokens', 'in', 'out', 'inter')},
+            'expert': c['expert'].tolist(), 'tenant': c['tenant'].tolist(),
+            'Y': y.tolist(),                                  # y[row] = x[row] W_e^T, rows in their original order
+            'swiglu_of_Y': oracle.swiglu(y).tolist()}         # silu(Y[:, :64]) * Y[:, 64:]
+
+
 if __name__ == '__main__':
+    with open(os.path.join(HERE, 'experts_small.json'), 'w') as f:
+        json.dump(experts_case(), f)
     with open(os.path.join(HERE, 'lora_small.json'), 'w') as f:
         json.dump(lora_case(), f)
     with open(os.path.join(HERE, 'segments_small.json'), 'w') as f:

@@ -64,3 +64,34 @@ def test_hip_lora_matches_fixture(dev, dtype, tol):
     assert max_rel_err(y, t64(c['Y'])) < tol and max_rel_err(x.grad, t64(c['dX'])) < tol
     for g in range(len(a)):
         assert max_rel_err(a[g].grad, t64(c['dA'][g])) < tol and max_rel_err(b[g].grad, t64(c['dB'][g])) < tol
+
+
+def _experts_inputs():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location('make_golden', os.path.join(GOLDEN, 'make_golden.py'))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod.experts_inputs()
+
+
+def test_oracle_reproduces_experts_fixture():
+    c, want = _experts_inputs(), _load('experts_small.json')
+    assert want['expert'] == c['expert'].tolist() and want['shape']['out'] == c['out']
+    order = torch.argsort(c['expert'], stable=True)
+    offsets = torch.cat([torch.zeros(1, dtype=torch.long), torch.bincount(c['expert'], minlength=c['experts']).cumsum(0)])
+    y = torch.empty(c['tokens'], c['out'], dtype=torch.double)
+    y[order] = oracle.experts_linear(c['x'][order], offsets, c['w'])
+    assert torch.allclose(y, torch.tensor(want['Y'], dtype=torch.double), atol=1e-12)
+    assert torch.allclose(oracle.swiglu(y), torch.tensor(want['swiglu_of_Y'], dtype=torch.double), atol=1e-12)
+
+
+@pytest.mark.gpu
+def test_hip_grouped_linear_and_swiglu_match_fixture(dev):
+    from twinkle_amd import build_segments, grouped_linear_, swiglu
+    c, want = _experts_inputs(), _load('experts_small.json')
+    keys = (c['expert'] * c['tenants'] + c['tenant']).to(torch.int32).to(dev)
+    seg = build_segments(keys, c['experts'] * c['tenants'])
+    y = grouped_linear_(c['x'].bfloat16().to(dev), c['w'].bfloat16().to(dev), seg, c['tenants'], map_rows=True)
+    y64 = torch.tensor(want['Y'], dtype=torch.double)
+    assert max_rel_err(y, y64) < 2e-2
+    assert max_rel_err(swiglu(y64.float().to(dev)), torch.tensor(want['swiglu_of_Y'], dtype=torch.double)) < 1e-5
