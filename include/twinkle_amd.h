@@ -243,9 +243,9 @@ int tk_lora_bwd_shared(const tk_lora_desc* const* descs, int32_t num_proj, const
  *
  * y[row] = x[row] W_e^T (+ h[row] B_g^T) for every row of the segment table, where the table was built from
  * keys g = e * groups_per_expert + tenant and expert e's weight [out_features][in_features] starts at
- * weight_device + e * weight_stride elements (row stride ldw).  Replaces the per-expert host loop of
- * F.linear calls with one synchronisation per expert (reference: moe/expert_parallel.py:347-371, the
- * gate_up and the down projection each); with `lora` it also takes over the expert LoRA delta that the
+ * weight_device + e * weight_stride elements (row stride ldw).  Replaces the reference's host loop over the
+ * experts (one F.linear per projection and one host synchronisation per expert for the chunk boundaries,
+ * moe/expert_parallel.py:347-371) by one launch; with `lora` it also takes over the expert LoRA delta that the
  * reference merges into the weights (multi_lora_target_parameters.py:158-179): call tk_lora_shrink(lora, x, h)
  * first and pass that h here, y is then written once with both terms.  The backward of the base term is the
  * same call with weight_layout = 1 on the same weights (dx = dy W_e, in_features and out_features swapped);
