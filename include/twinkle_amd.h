@@ -67,12 +67,14 @@ const char* tk_error_string(int code);
  *
  * keys[f] in [0, num_groups) is the group of flat row f (top-k routing: f = k*T + t).
  * perm_out[j]  = flat row placed at sorted position j (stable: ties keep ascending f),
- * offsets_out[g] = first sorted position of group g, offsets_out[num_groups] = rows.
+ * offsets_out[g] = first sorted position of group g, offsets_out[num_groups] = rows that have a group.
  * Both are int64 like the reference's tensors and may be NULL when only the
  * workspace is wanted.  seg_ws receives the device-side segment table the
  * LoRA and permute calls read; it must stay alive and unmodified while they run.
- * Keys outside [0, num_groups) are clamped for memory safety and counted;
- * tk_segment_bad_keys() reports the count.
+ * A key outside [0, num_groups) (say -1 for a padding row) gives its row no group: the row is
+ * placed after the last group in perm_out (stable among such rows) and no LoRA or grouped-GEMM call
+ * reads or writes it; tk_permute_rows / tk_unpermute_rows move it like any other row.
+ * tk_segment_bad_keys() reports how many such keys there were.
  * Limits: num_groups <= TK_MAX_GROUPS, rows < 2^31.
  * ------------------------------------------------------------------------ */
 int64_t tk_segment_workspace_bytes(int64_t rows, int32_t num_groups);

@@ -47,8 +47,11 @@ def segment_build_sort(keys: torch.Tensor, num_groups: int):
     the host at expert_parallel.py:347-349.  All int64, as in the reference.
     """
     keys = keys.reshape(-1).long()
+    # a key outside [0, num_groups) is a row without a group (nothing in the reference, whose mask has no such
+    # row): it sorts after every group and is counted nowhere, so offsets[num_groups] = rows that have a group
+    keys = torch.where((keys < 0) | (keys >= num_groups), torch.full_like(keys, num_groups), keys)
     perm = torch.sort(keys, stable=True).indices
-    counts = torch.bincount(keys, minlength=num_groups)
+    counts = torch.bincount(keys, minlength=num_groups + 1)[:num_groups]
     offsets = torch.zeros(num_groups + 1, dtype=torch.long)
     offsets[1:] = torch.cumsum(counts, 0)
     return perm, counts, offsets
@@ -62,6 +65,7 @@ def segment_build_bruteforce(keys, num_groups: int):
         rows = [f for f, k in enumerate(keys) if k == g]
         counts.append(len(rows))
         perm.extend(rows)
+    perm.extend(f for f, k in enumerate(keys) if k < 0 or k >= num_groups)  # rows without a group come last
     offsets = [0]
     for c in counts:
         offsets.append(offsets[-1] + c)

@@ -42,8 +42,8 @@ def test_size_queries_run_on_the_host():
     d = _lib.LoraDesc()
     d.rows, d.in_features, d.out_features, d.num_groups, d.max_rank, d.dtype = 16384, 4096, 4096, 16, 16, 1
     h = lib.tk_lora_h_bytes(ctypes.byref(d))
-    slots = 16384 + 32 * 16 + 64                      # padded slots
-    split = (16384 // 32 + 16) * 8 * 32 * 16 * 4       # partial sums of the 8 column slices of a 4096-wide shrink
+    slots = 16384 + 32 * 17 + 64                      # padded slots
+    split = (16384 // 32 + 17) * 8 * 32 * 16 * 4       # partial sums of the 8 column slices of a 4096-wide shrink
     assert 2 * 16 * 16384 * 2 <= h <= 2 * 16 * slots * 2 + split + 512
     assert lib.tk_lora_bwd_workspace_bytes(ctypes.byref(d)) > h
     d.max_rank = 1000

@@ -30,6 +30,13 @@ def _problem(t, k, m, n, max_r, ranks, seed, ids=None):
     return x, base, dy, a, b, ids, list(ranks), scales
 
 
+def lora_fwd_zero_base(x, seg, groups, map_rows=True):
+    """The LoRA term of every row on its own: the forward applied to a base output of zeros."""
+    y0 = torch.zeros(x.shape[0], groups.out_features, dtype=x.dtype, device=x.device)
+    lora_fwd_(x, y0, seg, groups, map_rows)
+    return y0
+
+
 def _run(dev, dtype, x, base, dy, a, b, ids, ranks, scales, check_zero_beyond_rank=True):
     """GPU through autograd vs oracle in float64 on the same rounded inputs."""
     cast = lambda t: t.to(dtype)  # noqa: E731
@@ -46,6 +53,10 @@ def _run(dev, dtype, x, base, dy, a, b, ids, ranks, scales, check_zero_beyond_ra
                                                         [f64(t) for t in b], ranks, scales, f64(dy))
     tol = TOL[dtype]
     assert max_rel_err(y, yo) < tol, 'Y'
+    # the LoRA term alone, on a zero base: the bar then scales with the term itself, not with the base output
+    # (which at these shapes is an order of magnitude larger and would hide an error in the term)
+    delta = lora_fwd_zero_base(xd.detach(), seg, groups)
+    assert max_rel_err(delta, yo - f64(base)) < tol, 'LoRA term'
     assert max_rel_err(xd.grad, dxo) < tol, 'dX'
     assert torch.equal(yd.grad.cpu(), cast(dy)), 'dY passes through to the base output unchanged'
     for g in range(len(a)):
@@ -89,6 +100,48 @@ def test_empty_and_huge_segments(dev, dtype):
     _, _, da, db = _run(dev, dtype, x, base, dy, a, b, ids, ranks, scales)
     for g in (1, 2, 4, 5):
         assert torch.count_nonzero(da[g]) == 0 and torch.count_nonzero(db[g]) == 0
+
+
+@pytest.mark.parametrize('dtype,t,k,m,max_r,ranks', [
+    (torch.bfloat16, 3000, 256, 1024, 16, [16, 8, 16]),     # single pass over dy, several chunks per group
+    (torch.bfloat16, 1500, 256, 384, 64, [64, 20, 33]),     # separate kernels, two streams
+    (torch.float32, 700, 40, 24, 8, [8, 3, 5]),             # generic kernels
+])
+def test_rows_without_an_adapter_keep_the_base_output(dev, dtype, t, k, m, max_r, ranks):
+    """Ids outside [0, adapters) (-1 for padding or ignored rows, or too large) belong to no adapter: such rows
+    keep the base output, get no input gradient from the LoRA branch and add to nobody's dA / dB; the
+    permutation places them after the last group.  The oracle skips them the same way."""
+    n = len(ranks)
+    x, base, dy, a, b, ids, _, scales = _problem(t, k, m, n, max_r, ranks, seed=t + 1)
+    g = torch.Generator().manual_seed(t)
+    ids = ids.clone()
+    ids[torch.rand(t, generator=g) < 0.2] = -1
+    ids[torch.rand(t, generator=g) < 0.05] = n + 3
+    ids[:40] = -1                                  # more than a tile of them in a row
+    none = (ids < 0) | (ids >= n)
+    cast = lambda v: v.to(dtype)  # noqa: E731
+    xd = cast(x).to(dev).requires_grad_(True)
+    ad = [cast(v).to(dev).requires_grad_(True) for v in a]
+    bd = [cast(v).to(dev).requires_grad_(True) for v in b]
+    seg = build_segments(ids.to(torch.int32).to(dev), n)
+    assert seg.bad_keys() == int(none.sum())
+    perm, _, offsets = oracle.segment_build_sort(ids, n)
+    assert torch.equal(seg.perm.cpu(), perm) and torch.equal(seg.offsets.cpu(), offsets)
+    assert int(offsets[n]) == t - int(none.sum())
+    groups = AdapterGroups(ad, bd, ranks, scales)
+    based = cast(base).to(dev)
+    y = multi_lora_delta(xd, based * 1.0, seg, groups)
+    y.backward(cast(dy).to(dev))
+    f64 = lambda v: cast(v).double()  # noqa: E731
+    yo, dxo, dao, dbo = oracle.multi_lora_linear_grads(f64(x), f64(base), ids, [f64(v) for v in a],
+                                                        [f64(v) for v in b], ranks, scales, f64(dy))
+    tol = TOL[dtype]
+    assert torch.equal(y[none.to(dev)], based[none.to(dev)]), 'rows without an adapter: base output, bit for bit'
+    assert torch.count_nonzero(xd.grad[none.to(dev)]) == 0
+    assert max_rel_err(y, yo) < tol and max_rel_err(xd.grad, dxo) < tol
+    assert max_rel_err(lora_fwd_zero_base(xd.detach(), seg, groups), yo - f64(base)) < tol
+    for i in range(n):
+        assert max_rel_err(ad[i].grad, dao[i]) < tol and max_rel_err(bd[i].grad, dbo[i]) < tol
 
 
 def test_results_are_bitwise_repeatable(dev):

@@ -34,6 +34,25 @@ def test_sort_equals_bruteforce(n, g, seed):
         assert torch.equal(x, y)
 
 
+@pytest.mark.parametrize('n,g,seed', [(1, 1, 0), (9, 2, 1), (40, 7, 2), (200, 5, 3)])
+def test_keys_outside_the_groups_sort_last_and_are_counted_nowhere(n, g, seed):
+    """Rows whose key is negative or >= groups have no group: they follow every group in ascending row order."""
+    keys = torch.randint(-2, g + 2, (n,), generator=torch.Generator().manual_seed(seed))
+    a = oracle.segment_build_sort(keys, g)
+    b = oracle.segment_build_bruteforce(keys, g)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    perm, counts, offsets = a
+    good = (keys >= 0) & (keys < g)
+    assert sorted(perm.tolist()) == list(range(n))
+    assert int(offsets[g]) == int(good.sum()) == int(counts.sum())
+    tail = perm[int(offsets[g]):]
+    assert torch.equal(tail, torch.nonzero(~good).flatten())
+    # hand-computed: keys [1, -1, 0, 5, 0] over 2 groups -> rows 2, 4 | 0 | 1, 3
+    p2, c2, o2 = oracle.segment_build_sort(torch.tensor([1, -1, 0, 5, 0]), 2)
+    assert p2.tolist() == [2, 4, 0, 1, 3] and c2.tolist() == [2, 1] and o2.tolist() == [0, 2, 3]
+
+
 def test_invariants_with_empty_groups():
     keys = torch.tensor([3, 3, 0, 7, 0, 3, 7, 7, 7])
     perm, counts, offsets = oracle.segment_build_sort(keys, 9)

@@ -23,12 +23,15 @@ namespace {
 
 constexpr int kKeysPerLane = kSortBlockRows / 64;
 
+// The kernels below sort into `buckets` = groups + 1 buckets: a key outside [0, groups) (a padding row, a row
+// the caller marks with -1) goes to the last bucket, whose tiles and chunks carry group -1, so that such rows
+// belong to no adapter: they keep their place in the permutation (after every group) and nothing else.
 template <typename KeyT>
-__device__ inline int load_key(const KeyT* keys, int64_t f, int groups, int* bad) {
+__device__ inline int load_key(const KeyT* keys, int64_t f, int buckets, int* bad) {
   long long k = (long long)keys[f];
-  if (k < 0 || k >= groups) {
+  if (k < 0 || k >= buckets - 1) {
     *bad += 1;
-    k = k < 0 ? 0 : groups - 1;
+    k = buckets - 1;
   }
   return (int)k;
 }
@@ -147,7 +150,7 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
     }
     const int ntile = (count + kTileRows - 1) / kTileRows;
     const int nchunk = (ntile + chunk_tiles - 1) / chunk_tiles;
-    const int npart = nchunk > 1 ? nchunk : 0;
+    const int npart = (nchunk > 1 && g != groups - 1) ? nchunk : 0;  // rows without a group need no partials
     int tot;
     const int e_rows = block_exclusive_scan(count, wave_sums, &tot) + carry_rows;
     carry_rows += tot;
@@ -162,7 +165,7 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
       V.tile_first[g] = e_tiles;
       V.chunk_first[g] = e_chunks;
       V.partial_first[g] = e_part;
-      if (offsets_out) offsets_out[g] = e_rows;
+      if (offsets_out) offsets_out[g] = e_rows;  // [groups - 1] (the caller's last entry): rows that have a group
       if (in_lds) {
         lds_first[0][g] = e_rows;
         lds_first[1][g] = e_tiles;
@@ -176,7 +179,6 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
     V.tile_first[groups] = carry_tiles;
     V.chunk_first[groups] = carry_chunks;
     V.partial_first[groups] = carry_part;
-    if (offsets_out) offsets_out[groups] = carry_rows;
     if (in_lds) {
       lds_first[0][groups] = carry_rows;
       lds_first[1][groups] = carry_tiles;
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
     SegHeader* hdr = V.header;
     hdr->magic = kSegMagic;
     hdr->rows = rows;
-    hdr->groups = groups;
+    hdr->groups = groups - 1;
     hdr->num_tiles = carry_tiles;
     hdr->num_chunks = carry_chunks;
     hdr->num_partials = carry_part;
@@ -207,7 +209,7 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
       pos0 = offs[g] + (i - tfirst[g]) * kTileRows;   // sorted position of the tile's first slot
       valid = min(kTileRows, offs[g + 1] - pos0);       // padding is at the end of a group's last tile
     }
-    V.tile_group[i] = g;
+    V.tile_group[i] = g == groups - 1 ? -1 : g;
     int4* sp = reinterpret_cast<int4*>(V.slot_pos + (int64_t)i * kTileRows);
 #pragma unroll
     for (int j = 0; j < kTileRows; j += 4)
@@ -222,10 +224,10 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
       const int g = group_of(cfirst, groups, i);
       const int j = i - cfirst[g];
       const int ntile = tfirst[g + 1] - tfirst[g];
-      c.group = g;
+      c.group = g == groups - 1 ? -1 : g;
       c.tile0 = tfirst[g] + j * chunk_tiles;
       c.ntiles = min(chunk_tiles, ntile - j * chunk_tiles);
-      c.partial = cfirst[g + 1] - cfirst[g] > 1 ? pfirst[g] + j : -1;
+      c.partial = (cfirst[g + 1] - cfirst[g] > 1 && g != groups - 1) ? pfirst[g] + j : -1;
     }
     V.chunks[i] = c;
   }
@@ -352,7 +354,7 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
     const int count = before + rest;
     const int ntile = (count + kTileRows - 1) / kTileRows;
     const int nchunk = (ntile + chunk_tiles - 1) / chunk_tiles;
-    const int npart = nchunk > 1 ? nchunk : 0;
+    const int npart = (nchunk > 1 && lane != groups - 1) ? nchunk : 0;
     int v[4] = {count, ntile, nchunk, npart}, excl[4], total[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
@@ -387,13 +389,12 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
         V.tile_first[groups] = total[1];
         V.chunk_first[groups] = total[2];
         V.partial_first[groups] = total[3];
-        if (offsets_out) offsets_out[groups] = total[0];
         int bad_total = 0;
         for (int w = 0; w < kOneWaves; ++w) bad_total += bad_s[w];
         SegHeader* hdr = V.header;
         hdr->magic = kSegMagic;
         hdr->rows = rows;
-        hdr->groups = groups;
+        hdr->groups = groups - 1;
         hdr->num_tiles = total[1];
         hdr->num_chunks = total[2];
         hdr->num_partials = total[3];
@@ -426,7 +427,7 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
       pos0 = offs[g] + (i - tfirst[g]) * kTileRows;  // sorted position of the tile's first slot
       valid = min(kTileRows, offs[g + 1] - pos0);      // padding is at the end of a group's last tile
     }
-    V.tile_group[i] = g;
+    V.tile_group[i] = g == groups - 1 ? -1 : g;
     int4* sp = reinterpret_cast<int4*>(V.slot_pos + (int64_t)i * kTileRows);
 #pragma unroll
     for (int j = 0; j < kTileRows; j += 4)
@@ -440,10 +441,10 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
       const int g = group_of(cfirst, groups, i);
       const int j = i - cfirst[g];
       const int ntile = tfirst[g + 1] - tfirst[g];
-      c.group = g;
+      c.group = g == groups - 1 ? -1 : g;
       c.tile0 = tfirst[g] + j * chunk_tiles;
       c.ntiles = min(chunk_tiles, ntile - j * chunk_tiles);
-      c.partial = cfirst[g + 1] - cfirst[g] > 1 ? pfirst[g] + j : -1;
+      c.partial = (cfirst[g + 1] - cfirst[g] > 1 && g != groups - 1) ? pfirst[g] + j : -1;
     }
     V.chunks[i] = c;
   }
@@ -559,6 +560,8 @@ int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t 
   SegLayout L(rows, groups);
   SegView V(ws, L);
   const int nblk = (int)L.sort_blocks;
+  const int user_groups = groups;
+  groups = user_groups + 1;  // the kernels' bucket count: one more for the rows without a group
   const size_t lds = sizeof(int32_t) * (size_t)groups;
   int key_bits = 0;
   while ((1 << key_bits) < groups) ++key_bits;

@@ -35,7 +35,7 @@ struct SegHeader {       // 64 x int32, at the start of the workspace
   int32_t num_tiles;     // filled on the device
   int32_t num_chunks;    // filled on the device
   int32_t num_partials;  // chunks that belong to multi-chunk groups
-  int32_t bad_keys;      // keys outside [0, groups), clamped
+  int32_t bad_keys;      // keys outside [0, groups): rows without a group
   int32_t pad[57];
 };
 
@@ -70,23 +70,26 @@ struct SegLayout {
       off_chunk_first, off_partial_first, off_hist, off_bad, total;
 
   SegLayout(int64_t rows_, int64_t groups_) : rows(rows_), groups(groups_) {
+    // the builder sorts into groups + 1 buckets: the last one takes the rows whose key is outside
+    // [0, groups); its tiles and chunks carry group -1, so no kernel touches those rows
+    const int64_t buckets = groups + 1;
     sort_blocks = ceil_div(rows > 0 ? rows : 1, kSortBlockRows);
-    max_tiles = ceil_div(rows, kTileRows) + groups;
+    max_tiles = ceil_div(rows, kTileRows) + buckets;
     chunk_tiles = chunk_tiles_for(rows);
-    max_chunks = ceil_div(rows, chunk_tiles * kTileRows) + groups;
+    max_chunks = ceil_div(rows, chunk_tiles * kTileRows) + buckets;
     max_partials = 2 * ceil_div(rows, chunk_tiles * kTileRows) + 1;
     slots = max_tiles * kTileRows;
     int64_t o = round_up(sizeof(SegHeader), 256);
     off_inv = o;           o += round_up(4 * (rows + 64), 256);
     off_slot_row = o;      o += round_up(4 * slots, 256);
     off_slot_pos = o;      o += round_up(4 * slots, 256);
-    off_offsets = o;       o += round_up(4 * (groups + 1), 256);
+    off_offsets = o;       o += round_up(4 * (buckets + 1), 256);
     off_tile_group = o;    o += round_up(4 * (max_tiles + 1), 256);
     off_chunks = o;        o += round_up(16 * (max_chunks + 1), 256);
-    off_tile_first = o;    o += round_up(4 * (groups + 1), 256);
-    off_chunk_first = o;   o += round_up(4 * (groups + 1), 256);
-    off_partial_first = o; o += round_up(4 * (groups + 1), 256);
-    off_hist = o;          o += round_up(4 * groups * sort_blocks, 256);
+    off_tile_first = o;    o += round_up(4 * (buckets + 1), 256);
+    off_chunk_first = o;   o += round_up(4 * (buckets + 1), 256);
+    off_partial_first = o; o += round_up(4 * (buckets + 1), 256);
+    off_hist = o;          o += round_up(4 * buckets * sort_blocks, 256);
     off_bad = o;           o += round_up(4 * sort_blocks, 256);
     total = o;
   }
@@ -97,13 +100,13 @@ struct SegView {  // typed device pointers into a segment workspace
   int32_t* inv;            // [rows]    flat row -> sorted position
   int32_t* slot_row;       // [slots]   padded slot -> flat row (perm), -1 in padding
   int32_t* slot_pos;       // [slots]   padded slot -> sorted position, -1 in padding
-  int32_t* offsets;        // [G + 1]
-  int32_t* tile_group;     // [max_tiles]  group of each tile, -1 past the last tile
+  int32_t* offsets;        // [G + 2]  first sorted position of each group; [G] = first row without a group
+  int32_t* tile_group;     // [max_tiles]  group of each tile, -1 for rows without a group and past the last tile
   ChunkInfo* chunks;       // [max_chunks]
-  int32_t* tile_first;     // [G + 1]  first tile of each group
-  int32_t* chunk_first;    // [G + 1]  first chunk of each group
-  int32_t* partial_first;  // [G + 1]  first partial slot of each multi-chunk group
-  int32_t* hist;           // [sort_blocks][G]  per-block histogram, then per-block exclusive bases
+  int32_t* tile_first;     // [G + 2]  first tile of each group
+  int32_t* chunk_first;    // [G + 2]  first chunk of each group
+  int32_t* partial_first;  // [G + 2]  first partial slot of each multi-chunk group
+  int32_t* hist;           // [sort_blocks][G + 1]  per-block histogram, then per-block exclusive bases
   int32_t* bad;            // [sort_blocks]  out-of-range keys seen by each block
   SegView(const void* base, const SegLayout& L) {
     char* b = (char*)base;

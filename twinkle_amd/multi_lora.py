@@ -225,9 +225,10 @@ class MultiLora:
         ``row_tenant`` is an integer GPU tensor with one entry per row of the
         flattened ``[rows, features]`` activations (so ``batch * seq`` entries for
         ``[batch, seq, features]`` inputs).  The segment table is built once here
-        and shared by every patched layer called inside the context.  ``check=True`` verifies that every entry
-        of ``row_tenant`` indexes ``tenant_adapter_names`` (one device synchronisation) and raises ``ValueError``
-        otherwise; unchecked, an entry out of range is an out-of-bounds index on the device.
+        and shared by every patched layer called inside the context.  A row whose entry is negative (padding,
+        ignored rows) or not below ``len(tenant_adapter_names)`` belongs to no tenant: it keeps the base output and
+        adds to nobody's gradients.  ``check=True`` instead verifies that every entry of ``row_tenant`` indexes
+        ``tenant_adapter_names`` (one device synchronisation) and raises ``ValueError`` otherwise.
         """
         slots = [self.find_lora_by_tenant(n).index for n in tenant_adapter_names]
         if check and row_tenant.numel():
@@ -235,8 +236,13 @@ class MultiLora:
             if lo < 0 or hi >= len(slots):
                 raise ValueError(f'row_tenant holds {lo}..{hi} but the batch has {len(slots)} tenants')
         lut = torch.tensor(slots, dtype=torch.int32, device=row_tenant.device)
-        keys = lut[row_tenant.reshape(-1).long()]
+        rt = row_tenant.reshape(-1).long()
+        known = (rt >= 0) & (rt < len(slots))
+        keys = torch.where(known, lut[rt.clamp(0, len(slots) - 1)], torch.full_like(lut[:1], -1))
         table = build_segments(keys, self.max_loras, want_perm=False, want_offsets=False)
+        # only the tenants of this batch are live inside the context: the others get no gradient, like the
+        # adapters the reference leaves inactive
+        table.live_slots = tuple(sorted({self.loras[i].adapter_name for i in slots}))
         previous, self._batch_table = self._batch_table, table
         try:
             yield table
@@ -253,8 +259,9 @@ class MultiLora:
         return table
 
     # ------------------------------------------------------------- patching
-    def _groups_for(self, layer, only_slot: Optional[str]) -> Optional[AdapterGroups]:
-        """Rank/scale table of a layer: slots whose tenant targets this layer are live, the rest rank 0."""
+    def _groups_for(self, layer, only_slot: Union[None, str, Tuple[str, ...]]) -> Optional[AdapterGroups]:
+        """Rank/scale table of a layer: slots whose tenant targets this layer are live, the rest rank 0.
+        ``only_slot`` narrows the live slots to one name or a tuple of names (``None``: every slot with a tenant)."""
         key = (id(layer), only_slot)
         cached = self._layer_groups.get(key)
         if cached is not None and cached[0] == self._version:
@@ -267,8 +274,8 @@ class MultiLora:
             a.append(layer.lora_A[name].weight)
             b.append(layer.lora_B[name].weight)
             cfg = slot.tenant_config
-            live = (cfg is not None and (only_slot is None or only_slot == name)
-                    and self.match_target_modules(layer.layer_name, cfg.target_modules))
+            wanted = only_slot is None or only_slot == name or (isinstance(only_slot, tuple) and name in only_slot)
+            live = cfg is not None and wanted and self.match_target_modules(layer.layer_name, cfg.target_modules)
             if live:
                 ranks.append(cfg.r)
                 scales.append(cfg.lora_alpha / (cfg.r**0.5 if getattr(cfg, 'use_rslora', False) else cfg.r))
@@ -314,7 +321,8 @@ class MultiLora:
                 active = [n for n in self.active_adapters if n in self.lora_A.keys()]
                 only_slot = active[0] if active else None
             skip = self.disable_adapters or (table is None and only_slot is None)
-            groups = None if skip else _self._groups_for(self, only_slot)
+            groups = None if skip else _self._groups_for(
+                self, only_slot if table is None else getattr(table, 'live_slots', None))
             if groups is None:
                 return self.base_layer(x, *args, **kwargs)
             groups.sync_masters()
@@ -403,7 +411,8 @@ class MultiLora:
                     ok = False
                     break
                 only_slot = slot
-            groups = None if layer.disable_adapters else self._groups_for(layer, only_slot)
+            groups = None if layer.disable_adapters else self._groups_for(
+                layer, only_slot if table is None else getattr(table, 'live_slots', None))
             base = layer.base_layer
             slot_for_dropout = only_slot if only_slot is not None else self.loras[0].adapter_name
             if (groups is None or groups.dtype != x.dtype or type(base) is not torch.nn.Linear

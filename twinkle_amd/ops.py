@@ -78,9 +78,17 @@ class AdapterGroups:
         dev = self.device
         self.rank_dev = torch.tensor(self.ranks, dtype=torch.int32, device=dev)
         self.scale_dev = torch.tensor(self.scales, dtype=torch.float32, device=dev)
-        # gradient arena: one flat buffer per side, every tensor at a fixed element offset
-        self._a_arena_off, self.a_arena_elems = self._arena(self.a_tensors)
-        self._b_arena_off, self.b_arena_elems = self._arena(self.b_tensors)
+        # gradient arena: one flat buffer per side, every live tensor at a fixed element offset.  A tensor is live
+        # when a group of positive rank reads it; the others (free slots, tenants that do not target this layer or
+        # are not part of the batch) get no gradient at all, like the adapters the reference leaves inactive.
+        self.a_live = [False] * len(self.a_tensors)
+        self.b_live = [False] * len(self.b_tensors)
+        for i, r in enumerate(self.ranks):
+            if r > 0:
+                self.a_live[self.a_index[i]] = True
+                self.b_live[self.b_index[i]] = True
+        self._a_arena_off, self.a_arena_elems = self._arena(self.a_tensors, self.a_live)
+        self._b_arena_off, self.b_arena_elems = self._arena(self.b_tensors, self.b_live)
         esz = a0.element_size()
         self._grad_a_rel = torch.tensor([(self._a_arena_off[self.a_index[i]] + self.a_offset[i]) * esz
                                          for i in range(g)], dtype=torch.int64, device=dev)
@@ -93,11 +101,12 @@ class AdapterGroups:
         self.refresh()
 
     @staticmethod
-    def _arena(tensors):
+    def _arena(tensors, live):
         offs, total = [], 0
-        for t in tensors:
-            offs.append(total)
-            total += (t.numel() + 127) // 128 * 128
+        for t, keep in zip(tensors, live):
+            offs.append(total if keep else 0)     # groups of rank 0 are never written: any offset will do
+            if keep:
+                total += (t.numel() + 127) // 128 * 128
         return offs, total
 
     def refresh(self) -> None:
@@ -113,12 +122,14 @@ class AdapterGroups:
                                     for i in range(g)], dtype=torch.int64, device=self.device)
         self._ptr_key = key
 
-    def grad_views(self, arena: torch.Tensor, side: str) -> List[torch.Tensor]:
-        tensors, offs = (self.a_tensors, self._a_arena_off) if side == 'a' else (self.b_tensors, self._b_arena_off)
+    def grad_views(self, arena: torch.Tensor, side: str) -> List[Optional[torch.Tensor]]:
+        """Per-tensor views of a gradient arena; ``None`` for tensors no live group reads."""
+        tensors, offs, live = (self.a_tensors, self._a_arena_off, self.a_live) if side == 'a' else \
+            (self.b_tensors, self._b_arena_off, self.b_live)
         masters = self.master_a if side == 'a' else self.master_b
         if masters is not None and masters[0].dtype != arena.dtype:
             arena = arena.to(masters[0].dtype)        # one cast for the whole side; the views below share it
-        return [arena[o:o + t.numel()].view(t.shape) for t, o in zip(tensors, offs)]
+        return [arena[o:o + t.numel()].view(t.shape) if keep else None for t, o, keep in zip(tensors, offs, live)]
 
     def autograd_tensors(self) -> List[torch.Tensor]:
         """The tensors gradients are reported for: the masters where there are any, else the tensors read."""
