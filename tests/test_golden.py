@@ -62,6 +62,12 @@ def test_hip_lora_matches_fixture(dev, dtype, tol):
     y.backward(td(c['dy']))
     t64 = lambda v: torch.tensor(v, dtype=torch.double)  # noqa: E731
     assert max_rel_err(y, t64(c['Y'])) < tol and max_rel_err(x.grad, t64(c['dX'])) < tol
+    # the LoRA term alone (zero base) against fixture Y minus fixture base: the bar scales with the term itself
+    from twinkle_amd import lora_fwd_
+    delta = torch.zeros_like(y)
+    lora_fwd_(x.detach(), delta, seg, AdapterGroups([v.detach() for v in a], [v.detach() for v in b], c['ranks'],
+                                                    c['scales']))
+    assert max_rel_err(delta, t64(c['Y']) - td(c['base']).double().cpu()) < tol
     for g in range(len(a)):
         assert max_rel_err(a[g].grad, t64(c['dA'][g])) < tol and max_rel_err(b[g].grad, t64(c['dB'][g])) < tol
 

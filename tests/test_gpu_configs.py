@@ -27,6 +27,8 @@ def _check_sampled(w, dev, sample_groups, sample_rows=64):
     y = w.base_out.to(dt).to(dev)
     dy = w.dy.to(dt).to(dev)
     h = lora_fwd_(x, y, seg, groups)
+    delta = torch.zeros_like(y)                   # the LoRA term alone, on a zero base
+    lora_fwd_(x, delta, seg, groups)
     ga = [torch.full_like(t, 7.0) for t in a]
     gb = [torch.full_like(t, 7.0) for t in b]
     pa = torch.tensor([t.data_ptr() for t in ga], dtype=torch.int64, device=dev)
@@ -47,6 +49,7 @@ def _check_sampled(w, dev, sample_groups, sample_rows=64):
         dh = s * dyg @ bg
         sub = rows[:sample_rows]
         assert max_rel_err(y[sub.to(dev)], f64(w.base_out[sub]) + (hg[:sample_rows] @ bg.t())) < 2e-2
+        assert max_rel_err(delta[sub.to(dev)], hg[:sample_rows] @ bg.t()) < 2e-2, f'LoRA term of adapter {g}'
         assert max_rel_err(dx[sub.to(dev)], dh[:sample_rows] @ ag) < 2e-2
         assert max_rel_err(ga[g][:r], dh.t() @ xg) < 2e-2, f'dA[{g}] ({int(counts[g])} rows)'
         assert max_rel_err(gb[g][:, :r], dyg.t() @ (hg / 1.0)) < 2e-2, f'dB[{g}]'
@@ -100,3 +103,174 @@ def test_config5_packed_sequences_one_tenant_each(dev):
     b = [torch.randn(m, r, generator=g) * 0.02 for _ in range(n)]
     w = workloads.LoraWorkload('cfg5_k_proj', t, k, m, [r] * n, [2.0] * n, r, ids.cpu(), x, dy, base, a, b)
     _check_sampled(w, dev, sample_groups=[0, 4, 7])
+
+
+def _config4_keys(dev, with_edge_groups):
+    """(expert, tenant) keys of BASELINE config 4 in the reference's row order; optionally one group emptied and
+    one cut down to a single row (their rows go to the neighbouring group)."""
+    from twinkle_amd import flat_keys_from_topk
+    sel, weights, tenant = workloads.moe_routing()
+    keys = flat_keys_from_topk(sel.to(dev), tenant.to(dev), 4)
+    if with_edge_groups:
+        keys = keys.clone()
+        keys[keys == 7] = 8                                   # group 7: empty
+        rows300 = (keys == 300).nonzero().flatten()
+        keys[rows300[1:]] = 301                               # group 300: one row
+    return keys, sel.shape[0]
+
+
+@pytest.mark.parametrize('k_in,m_out', [(2048, 1536), (768, 2048)])
+def test_config4_backward_full_size(dev, k_in, m_out):
+    """BASELINE config 4 at its own size, forward and backward: 65536 routed rows in (expert, tenant) order, 512
+    groups of rank 8 reading blocks of packed [E, max_r, in] / [E, out, max_r] tensors, rows already in segment
+    order (map_rows = 0); gate_up (2048 -> 1536) and down (768 -> 2048).  The LoRA term, dX on all rows of sampled
+    groups, dA / dB of sampled groups (an empty one and a one-row one among them) against the closed forms in
+    float64; gradients of groups that were not sampled are checked for finiteness and for zeros beyond the rank."""
+    e, nt, r, max_r = 128, 4, 8, 8
+    keys, tokens = _config4_keys(dev, with_edge_groups=True)
+    rows = keys.numel()
+    assert rows == 65536
+    seg = build_segments(keys, e * nt, num_tokens=tokens, check=True)
+    offsets = seg.offsets.cpu()
+    assert int(offsets[8] - offsets[7]) == 0 and int(offsets[301] - offsets[300]) == 1
+    g = torch.Generator().manual_seed(44)
+    dt = torch.bfloat16
+    x = torch.randn(rows, k_in, generator=g).to(dt)                      # rows in segment order
+    dy = torch.randn(rows, m_out, generator=g).to(dt)
+    a = [((torch.rand(e, max_r, k_in, generator=g) * 2 - 1) / k_in**0.5).to(dt) for _ in range(nt)]
+    b = [(torch.randn(e, m_out, max_r, generator=g) * 0.02).to(dt) for _ in range(nt)]
+    ad, bd = [v.to(dev) for v in a], [v.to(dev) for v in b]
+    n = e * nt
+    groups = AdapterGroups(ad, bd, [r] * n, [2.0] * n, a_index=[i % nt for i in range(n)],
+                           a_offset=[(i // nt) * max_r * k_in for i in range(n)], b_index=[i % nt for i in range(n)],
+                           b_offset=[(i // nt) * m_out * max_r for i in range(n)])
+    xd, dyd = x.to(dev), dy.to(dev)
+    y = torch.zeros(rows, m_out, dtype=dt, device=dev)                   # zero base: the LoRA term alone
+    h = lora_fwd_(xd, y, seg, groups, map_rows=False)
+    ga = torch.full((groups.a_arena_elems,), 7.0, dtype=dt, device=dev)
+    gb = torch.full((groups.b_arena_elems,), 7.0, dtype=dt, device=dev)
+    dx = torch.zeros_like(xd)
+    lora_bwd_(dyd, xd, h, dx, groups._grad_a_rel + ga.data_ptr(), groups._grad_b_rel + gb.data_ptr(), seg, groups,
+              map_rows=False, accumulate=False)
+    grad_a, grad_b = groups.grad_views(ga, 'a'), groups.grad_views(gb, 'b')
+    for i in (0, 7, 8, 77, 300, 301, 302, 511):
+        s0, s1 = int(offsets[i]), int(offsets[i + 1])
+        ex, tn = i // nt, i % nt
+        got_a, got_b = grad_a[tn][ex].cpu(), grad_b[tn][ex].cpu()
+        if s0 == s1:
+            assert torch.count_nonzero(got_a[:r]) == 0 and torch.count_nonzero(got_b[:, :r]) == 0, i
+            continue
+        ag, bg = a[tn][ex, :r].double(), b[tn][ex, :, :r].double()
+        xg, dyg = x[s0:s1].double(), dy[s0:s1].double()
+        hg = 2.0 * xg @ ag.t()
+        dh = 2.0 * dyg @ bg
+        assert max_rel_err(y[s0:s1], hg @ bg.t()) < 2e-2, f'LoRA term, group {i} ({s1 - s0} rows)'
+        assert max_rel_err(dx[s0:s1], dh @ ag) < 2e-2, f'dX, group {i}'
+        assert max_rel_err(got_a[:r], dh.t() @ xg) < 2e-2, f'dA, group {i}'
+        assert max_rel_err(got_b[:, :r], dyg.t() @ hg) < 2e-2, f'dB, group {i}'
+    for tn in range(nt):
+        assert torch.isfinite(grad_a[tn].float()).all() and torch.isfinite(grad_b[tn].float()).all()
+
+
+def test_config4_grouped_linear_128_experts_both_directions(dev):
+    """tk_grouped_linear at config 4's size (128 experts x 4 tenants, 65536 routed rows): y = x W_e^T for
+    gate_up (2048 -> 1536) and the transposing form dx = dy W_e on the same weights, all rows of sampled experts
+    against float64."""
+    from twinkle_amd import grouped_linear_
+    e, nt, hid, out = 128, 4, 2048, 1536
+    keys, tokens = _config4_keys(dev, with_edge_groups=False)
+    rows = keys.numel()
+    seg = build_segments(keys, e * nt, num_tokens=tokens)
+    offsets = seg.offsets.cpu()
+    g = torch.Generator().manual_seed(45)
+    dt = torch.bfloat16
+    x = torch.randn(rows, hid, generator=g).to(dt)
+    dy = torch.randn(rows, out, generator=g).to(dt)
+    w = (torch.randn(e, out, hid, generator=g) * 0.02).to(dt)
+    wd = w.to(dev)
+    y = grouped_linear_(x.to(dev), wd, seg, nt, map_rows=False)
+    dx = grouped_linear_(dy.to(dev), wd, seg, nt, map_rows=False, transposed=True)
+    for ex in (0, 1, 63, 100, 127):
+        s0, s1 = int(offsets[ex * nt]), int(offsets[(ex + 1) * nt])
+        assert s1 > s0
+        assert max_rel_err(y[s0:s1], x[s0:s1].double() @ w[ex].double().t()) < 2e-2, ex
+        assert max_rel_err(dx[s0:s1], dy[s0:s1].double() @ w[ex].double()) < 2e-2, ex
+
+
+def test_config5_one_full_layer_through_multilora_batch(dev):
+    """BASELINE config 5, one decoder layer at full size: hidden 4096, 32 heads / 8 KV heads, intermediate 14336,
+    rank 64 alpha 128 on all seven projections, 8 tenants, 8 packed sequences x 4096 with tenant j owning
+    sequence j, through MultiLora.batch with q/k/v and gate/up declared as shared inputs.  Every projection's
+    input, output, output gradient and input gradient is captured on the GPU and checked on the CPU in float64:
+    outputs and input gradients on sampled rows of sampled tenants (base GEMM included: the same rows through the
+    frozen weight), dA / dB of sampled tenants over all of their 4096 rows."""
+    from test_gpu_multilora import _LlamaLayer
+    from twinkle_amd import LoraConfig, MultiLora
+    torch.manual_seed(7)
+    d, heads, kv, inter, r, n, seq = 4096, 32, 8, 14336, 64, 8, 4096
+    dt = torch.bfloat16
+    layer = _LlamaLayer(d, heads, kv, inter).to(dt).to(dev)
+    ml = MultiLora(max_loras=n, max_r=r)
+    model = ml.patch(layer, target_modules='all-linear')
+    names = [f'tenant_{j}' for j in range(n)]
+    for name in names:
+        ml.acquire_lora(name, LoraConfig(r=r, lora_alpha=2 * r, target_modules='all-linear'))
+    gen = torch.Generator(device=dev).manual_seed(8)
+    proj = ['q_proj', 'k_proj', 'v_proj', 'o_proj', 'gate_proj', 'up_proj', 'down_proj']
+    mods = {p: getattr(model.model, p) for p in proj}
+    with torch.no_grad():
+        for p in proj:
+            for s in mods[p].lora_B.keys():
+                mods[p].lora_B[s].weight.copy_(torch.randn(mods[p].lora_B[s].weight.shape, generator=gen, device=dev) * 0.02)
+    ml.share_inputs([['model.q_proj', 'model.k_proj', 'model.v_proj'], ['model.gate_proj', 'model.up_proj']])
+    x = torch.randn(n, seq, d, generator=gen, device=dev, dtype=torch.float32).to(dt).requires_grad_(True)
+    w = torch.randn(n, seq, d, generator=gen, device=dev, dtype=torch.float32).to(dt)
+    cu = packed_cu_seqlens(torch.arange(seq, device=dev).repeat(n)[None])
+    row_tenant = token_groups_from_sequences(cu, torch.arange(n, device=dev))
+    seen = {}
+
+    def capture(name):
+        def hook(mod, args, out):
+            inp = args[0]
+            seen[name] = {'x': inp.detach(), 'y': out.detach()}
+            out.register_hook(lambda gr: seen[name].__setitem__('dy', gr.detach()))
+            if inp.requires_grad and name in ('q_proj', 'o_proj', 'gate_proj', 'down_proj'):
+                inp.register_hook(lambda gr: seen[name].__setitem__('dx', gr.detach()))
+        return hook
+
+    handles = [mods[p].register_forward_hook(capture(p)) for p in proj]
+    with ml.batch(names, row_tenant):
+        y = model(x)
+    (y * w).sum().backward()
+    for hnd in handles:
+        hnd.remove()
+    assert torch.isfinite(y.float()).all() and torch.isfinite(x.grad.float()).all()
+
+    f64 = lambda t: t.detach().double().cpu()  # noqa: E731
+    sample = torch.arange(0, seq, 97)[:40]
+    sharing = {'q_proj': ['q_proj', 'k_proj', 'v_proj'], 'o_proj': ['o_proj'], 'gate_proj': ['gate_proj', 'up_proj'],
+               'down_proj': ['down_proj']}
+    for j in (0, 5):                                                   # sampled tenants
+        slot = ml.find_lora_by_tenant(names[j]).adapter_name
+        rows = j * seq + sample
+        allrows = slice(j * seq, (j + 1) * seq)
+        dx_want = {}
+        for p in proj:
+            m = mods[p]
+            wb = f64(m.base_layer.weight)
+            a, b = f64(m.lora_A[slot].weight), f64(m.lora_B[slot].weight)
+            xin = seen[p]['x'].reshape(-1, seen[p]['x'].shape[-1])
+            yout = seen[p]['y'].reshape(-1, seen[p]['y'].shape[-1])
+            dyo = seen[p]['dy'].reshape(-1, yout.shape[-1])
+            xs, dys = f64(xin[rows.to(dev)]), f64(dyo[rows.to(dev)])
+            want = xs @ wb.t() + 2.0 * (xs @ a.t()) @ b.t()
+            assert max_rel_err(yout[rows.to(dev)], want) < 2e-2, (p, j, 'Y')
+            assert max_rel_err(f64(yout[rows.to(dev)]) - xs @ wb.t(), want - xs @ wb.t()) < 5e-2, (p, j, 'LoRA part of Y')
+            dx_want[p] = dys @ wb + 2.0 * (dys @ b) @ a
+            xa, dya = f64(xin[allrows]), f64(dyo[allrows])
+            ha, dha = 2.0 * xa @ a.t(), 2.0 * dya @ b
+            assert max_rel_err(m.lora_A[slot].weight.grad, dha.t() @ xa) < 2e-2, (p, j, 'dA')
+            assert max_rel_err(m.lora_B[slot].weight.grad, dya.t() @ ha) < 2e-2, (p, j, 'dB')
+        for first, group in sharing.items():
+            got = seen[first]['dx'].reshape(-1, seen[first]['dx'].shape[-1])[rows.to(dev)]
+            assert max_rel_err(got, sum(dx_want[p] for p in group)) < 2e-2, (first, j, 'dX')

@@ -171,7 +171,7 @@ def test_expert_slots_follow_the_reference_rules():
         other.set_state_dict('lora_1', {'m.experts.lora_A.weight': sd['m.experts.lora_A.weight']})
     with pytest.raises(ValueError):
         other.set_state_dict('lora_1', {k: v[:1] for k, v in sd.items()})
-    a0 = slots._initial_lora_A['lora_0'].clone()
+    a0 = slots._first_A['lora_0'].clone()
     slots.reset_slot('lora_0')
     assert torch.equal(slots.lora_A['lora_0'].detach(), a0) and torch.count_nonzero(slots.lora_B['lora_0']) == 0
 
@@ -252,7 +252,7 @@ def test_adapter_checkpoint_round_trip_in_peft_format(tmp_path):
         assert torch.equal(v, saved['base_model.' + k])
 
 
-def test_share_inputs_bookkeeping_without_a_gpu():
+def test_share_inputs_bookkeeping_without_a_gpu(monkeypatch):
     """share_inputs: the first sibling that sees a tensor computes the group, the others collect; no stale results."""
     from torch import nn
 
@@ -272,8 +272,9 @@ def test_share_inputs_bookkeeping_without_a_gpu():
     with ml.adapter('alice', disable_lora=True):                    # base path only: runs on the CPU
         want = model(x)
         calls = []
-        original = ml.forward_shared
-        ml.forward_shared = lambda layers, t: calls.append(len(layers)) or original(layers, t)
+        import twinkle_amd.multi_lora as host
+        original = host.forward_shared
+        monkeypatch.setattr(host, 'forward_shared', lambda m, layers, t: calls.append(len(layers)) or original(m, layers, t))
         ml.share_inputs([['model.q_proj', 'model.k_proj', 'model.v_proj']])
         got = model(x)
         assert calls == [3]                                         # one group computation for three layer calls
@@ -392,10 +393,13 @@ def test_target_parameter_slots_keys_shapes_release_and_round_trip(is_transposed
     ml2.set_state_dict('adapter_a', state)
     for w1, w2 in zip(manager.wrappers, ml2.target_parameter_manager.wrappers):
         assert torch.allclose(w1.get_delta_weight('lora_0'), w2.get_delta_weight('lora_0'), atol=1e-6)
-    # adapter() tells every slot storage which slot is the active one, and restores it
+    # adapter() tells the manager which slot the expert modules apply, and restores what was there before
     with ml.adapter('adapter_a'):
-        assert gate_up.active_adapter == 'lora_0' and not gate_up.disable_adapters
-    assert gate_up.active_adapter is None
+        assert manager.active_pass.slots == ['lora_0'] and not manager.active_pass.disabled
+        with ml.adapter('adapter_a', disable_lora=True):
+            assert manager.active_pass.disabled
+        assert not manager.active_pass.disabled
+    assert manager.active_pass is None
     # release: A back to its first initialisation, B to zero (reference test :103-134)
     ml3, _, cfg3 = _expert_model(is_transposed)
     ml3.acquire_lora('adapter_a', cfg3(2))
@@ -430,3 +434,154 @@ def test_grouped_gemm_applicability():
     assert not grouped_gemm_applies(torch.zeros(3, 384, 192, dtype=torch.bfloat16), rows)          # in = 192
     assert not grouped_gemm_applies(torch.zeros(3, 320, 256, dtype=torch.bfloat16), rows)          # out = 320
     assert not grouped_gemm_applies(ok.transpose(1, 2), rows)                                       # not contiguous
+
+
+# ---- the documented way of installing the path into the reference's own MultiLora ------------------------------------
+
+class ReferenceSurfaceMultiLora:
+    """An object with the attributes and methods of the reference's ``MultiLora`` (src/twinkle/model/multi_lora.py:
+    33-40 ``__init__``, :209-254 ``acquire_lora / release_lora / find_lora*``, :256-287 ``match_target_modules``,
+    :126-163 ``activate_adapter / adapter``) and nothing of this package's own class."""
+
+    def __init__(self, module, max_loras, max_r):
+        from twinkle_amd import LoraTenant
+        self.max_loras, self.max_r, self.max_length = max_loras, max_r, 8192
+        self.module = module
+        self.loras = [LoraTenant(index=i, adapter_name=f'lora_{i}', config=None) for i in range(max_loras)]
+
+    def has_lora(self, name):
+        return any(t.tenant_adapter_name == name for t in self.loras)
+
+    def find_lora_by_tenant(self, name):
+        found = [t for t in self.loras if t.tenant_adapter_name == name]
+        if not found:
+            raise ValueError(f'No lora found for tenant {name}')
+        return found[0]
+
+    def find_lora(self, adapter_name):
+        found = [t for t in self.loras if t.adapter_name == adapter_name]
+        if not found:
+            raise ValueError(f'No lora found for real adapter_name {adapter_name}')
+        return found[0]
+
+    def acquire_lora(self, tenant, config):
+        free = [t for t in self.loras if t.tenant_adapter_name is None]
+        if self.has_lora(tenant):
+            raise ValueError(f'Lora {tenant} already exists')
+        if not free or config.r > self.max_r:
+            raise RuntimeError('no slot / rank too big')
+        free[0].tenant_adapter_name, free[0].tenant_config = tenant, config
+        return free[0].adapter_name
+
+    def release_lora(self, tenant):
+        slot = self.find_lora_by_tenant(tenant)
+        slot.tenant_adapter_name = slot.tenant_config = None
+
+    match_target_modules = staticmethod(oracle.match_target_modules)
+
+    def adapter(self, tenant, disable_lora=False):
+        from contextlib import contextmanager
+
+        @contextmanager
+        def ctx():
+            self.module.set_adapter(self.find_lora_by_tenant(tenant).adapter_name)
+            if disable_lora:
+                self.module.disable_adapter_layers()
+            try:
+                yield
+            finally:
+                if disable_lora:
+                    self.module.enable_adapter_layers()
+        return ctx()
+
+
+def reference_surface_setup(device='cpu', dtype=torch.float32):
+    """TinyBlock with three slots of rank 8 injected, held by an object that has only the reference's surface."""
+    from twinkle_amd import inject_adapter
+    torch.manual_seed(0)
+    holder = TinyBlock().to(dtype).to(device)
+    for i in range(3):
+        holder = inject_adapter(holder, LoraConfig(r=8, lora_alpha=32, target_modules='all-linear'), f'lora_{i}')
+    ref = ReferenceSurfaceMultiLora(holder, max_loras=3, max_r=8)
+    with torch.no_grad():
+        for n, p in holder.named_parameters():
+            if '.lora_B.' in n:
+                p.normal_(0, 0.05)
+    return ref, holder
+
+
+def test_use_mi355x_path_on_an_object_with_only_the_reference_surface():
+    """The installer of twinkle_amd.integration needs nothing but the reference's MultiLora surface: after it, a
+    forward under adapter() gets as far as the HIP op (which refuses CPU tensors), disable_lora gives the base
+    model, and acquire / release through the object's own methods are seen without any notification."""
+    import twinkle_amd
+    ref, holder = reference_surface_setup()
+    assert not hasattr(ref, '_groups_for') and not hasattr(ref, 'batch') and not hasattr(ref, '_version')
+    twinkle_amd.use_mi355x_path(ref)
+    x = torch.randn(6, 16)
+    base_only = TinyBlock.forward(holder.model, x)         # no tenant holds the active slot: LoRA is skipped
+    assert torch.isfinite(base_only).all()
+    ref.acquire_lora('alice', LoraConfig(r=4, lora_alpha=8, target_modules='all-linear'))
+    with ref.adapter('alice', disable_lora=True):
+        assert torch.equal(holder(x), base_only)
+    with ref.adapter('alice'):
+        with pytest.raises(RuntimeError, match='GPU'):     # reached the op: the path has no CPU implementation
+            holder(x)
+    with pytest.raises(RuntimeError, match='GPU'):
+        with twinkle_amd.batch(ref, ['alice'], torch.zeros(6, dtype=torch.long)):
+            holder(x)
+    ref.release_lora('alice')                              # the slot is free again: base output, no op call
+    holder.set_adapter('lora_0')
+    assert torch.equal(holder(x), base_only)
+    with pytest.raises(ValueError):
+        twinkle_amd.use_mi355x_path(ReferenceSurfaceMultiLora(TinyBlock(), 1, 8))   # nothing patched yet
+
+
+def test_adapter_checkpoint_keys_with_linear_and_packed_expert_parameters(tmp_path):
+    """One naming root in adapter_model.safetensors: base_model.model.<path inside the wrapped model> for linear
+    layers and packed expert parameters alike (reference: PeftModel parameter names for the former,
+    multi_lora_target_parameters.py:321-330 for the latter), and the file loads back into a fresh model."""
+    from safetensors.torch import load_file
+
+    class Moe(nn.Module):
+
+        def __init__(self):
+            super().__init__()
+            self.q_proj = nn.Linear(4, 4, bias=False)
+            self.mlp = nn.Module()
+            self.mlp.experts = _PackedExperts()
+
+        def forward(self, x):
+            return self.q_proj(x)
+
+    def build():
+        torch.manual_seed(0)
+        ml = MultiLora(max_loras=2, max_r=4)
+        model = ml.patch(Moe(), target_modules=['q_proj'])
+        ml.save_initial_weights()
+        targets = ['mlp.experts.gate_up_proj', 'mlp.experts.down_proj']
+        ml.patch_target_parameters(model, targets)
+        ml.acquire_lora('alice', LoraConfig(r=2, lora_alpha=4, target_modules=['q_proj'], target_parameters=targets))
+        return ml, model
+
+    ml, model = build()
+    with torch.no_grad():
+        for n, p in model.named_parameters():
+            if 'lora_' in n:
+                p.uniform_(-0.1, 0.1)
+    out = ml.save_adapter('alice', str(tmp_path / 'ckpt'))
+    saved = load_file(f'{out}/adapter_model.safetensors')
+    assert {k: tuple(v.shape) for k, v in saved.items()} == {
+        'base_model.model.q_proj.lora_A.weight': (2, 4),
+        'base_model.model.q_proj.lora_B.weight': (4, 2),
+        'base_model.model.mlp.experts.base_layer.lora_A.weight': (2, 2, 4),
+        'base_model.model.mlp.experts.base_layer.lora_B.weight': (2, 12, 2),
+        'base_model.model.mlp.experts.lora_A.weight': (2, 2, 6),
+        'base_model.model.mlp.experts.lora_B.weight': (2, 4, 2),
+    }
+    ml2, model2 = build()
+    ml2.load_adapter('alice', out)
+    want, got = ml.get_state_dict('alice'), ml2.get_state_dict('alice')
+    assert want.keys() == got.keys()
+    for k in want:
+        assert torch.equal(want[k], got[k]), k

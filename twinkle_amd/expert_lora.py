@@ -15,6 +15,7 @@ from __future__ import annotations
 
 import math
 from contextlib import contextmanager
+from types import MethodType
 from typing import Dict, List, Optional, Sequence
 
 import torch
@@ -24,123 +25,134 @@ from .ops import AdapterGroups, multi_lora_delta
 from .segments import SegmentTable
 
 
+# what a tenant's config may not ask of packed-parameter LoRA (the reference refuses the same four,
+# multi_lora_target_parameters.py:143-150)
+_REFUSED_OPTIONS = (('lora_dropout', 'lora_dropout != 0'), ('fan_in_fan_out', 'fan_in_fan_out=True'),
+                    ('use_dora', 'use_dora=True'), ('lora_bias', 'lora_bias=True'))
+
+
 class ExpertLoraSlots(nn.Module):
-    """Slot storage of one packed expert parameter (the reference's ``TargetParameterLoraWrapper`` state)."""
+    """Slot storage of one packed expert parameter: per slot ``lora_A [E, max_r, in]`` and ``lora_B [E, out, max_r]``
+    (the tensors of the reference's ``TargetParameterLoraWrapper``, multi_lora_target_parameters.py:97-114), the
+    rank and scaling of the tenant that holds the slot, and the group table the segmented kernels read them by."""
 
     def __init__(self, num_experts: int, in_features: int, out_features: int, max_loras: int, max_r: int,
                  dtype=torch.float32, device=None, key_prefix: str = ''):
         super().__init__()
-        self.num_experts = num_experts
-        self.in_features = in_features
-        self.out_features = out_features
-        self.max_loras = max_loras
-        self.max_r = max_r
+        self.num_experts, self.in_features, self.out_features = num_experts, in_features, out_features
+        self.max_loras, self.max_r = max_loras, max_r
         self.peft_key_prefix = key_prefix
-        self.lora_A = nn.ParameterDict()
-        self.lora_B = nn.ParameterDict()
-        self.scaling: Dict[str, float] = {}
-        self.r: Dict[str, int] = {}
-        self._initial_lora_A: Dict[str, torch.Tensor] = {}
-        for index in range(max_loras):
-            name = f'lora_{index}'
-            self.lora_A[name] = nn.Parameter(torch.empty(num_experts, max_r, in_features, device=device, dtype=dtype))
-            self.lora_B[name] = nn.Parameter(torch.empty(num_experts, out_features, max_r, device=device, dtype=dtype))
-            self.r[name] = max_r
-            self.scaling[name] = 1.0
-            self.reset_slot(name)
+        self.parameter_key = key_prefix       # name of the packed parameter inside the patched model
+        self.out_in_layout = True             # the parameter is stored [E, out, in]
+        names = [f'lora_{i}' for i in range(max_loras)]
+        self.lora_A = nn.ParameterDict(
+            {n: nn.Parameter(torch.empty(num_experts, max_r, in_features, device=device, dtype=dtype)) for n in names})
+        self.lora_B = nn.ParameterDict(
+            {n: nn.Parameter(torch.zeros(num_experts, out_features, max_r, device=device, dtype=dtype)) for n in names})
+        self.r: Dict[str, int] = dict.fromkeys(names, max_r)
+        self.scaling: Dict[str, float] = dict.fromkeys(names, 1.0)
+        # the first initialisation of every slot's A (kaiming-uniform with a = sqrt(5), reference :119-123), kept on
+        # the CPU: a released slot goes back to exactly these values
+        self._first_A: Dict[str, torch.Tensor] = {}
+        for n in names:
+            nn.init.kaiming_uniform_(self.lora_A[n], a=math.sqrt(5))
+            self._first_A[n] = self.lora_A[n].detach().to('cpu', copy=True)
+        self._groups_cache: Dict[tuple, AdapterGroups] = {}
+
+    def _slot(self, slot_name: str):
+        if slot_name not in self.lora_A:
+            raise ValueError(f'Unknown target-parameter LoRA slot: {slot_name}')
+        return self.lora_A[slot_name], self.lora_B[slot_name]
 
     def reset_slot(self, slot_name: str) -> None:
-        """A back to its first initialisation (kaiming-uniform, a = sqrt(5)), B to zero (reference :119-134)."""
-        if slot_name not in self._initial_lora_A:
-            nn.init.kaiming_uniform_(self.lora_A[slot_name], a=math.sqrt(5))
-            self._initial_lora_A[slot_name] = self.lora_A[slot_name].detach().clone().cpu()
-        else:
-            init = self._initial_lora_A[slot_name]
-            self.lora_A[slot_name].data.copy_(init.to(device=self.lora_A[slot_name].device,
-                                                      dtype=self.lora_A[slot_name].dtype))
-        nn.init.zeros_(self.lora_B[slot_name])
+        """What releasing a tenant does to its slot: A back to its first values, B to zero (reference :119-134)."""
+        a, b = self._slot(slot_name)
+        with torch.no_grad():
+            a.copy_(self._first_A[slot_name])
+            b.zero_()
 
     def configure_slot(self, slot_name: str, config) -> None:
-        """Rank and scaling of the tenant that takes the slot; same checks and messages as reference :136-156."""
-        if slot_name not in self.lora_A:
-            raise ValueError(f'Unknown target-parameter LoRA slot: {slot_name}')
-        if config.r <= 0:
-            raise ValueError(f'`r` should be a positive integer value but the value passed is {config.r}')
-        if config.r > self.max_r:
-            raise ValueError(f'LoRA rank {config.r} exceeds max_r={self.max_r}')
-        if getattr(config, 'lora_dropout', 0):
-            raise ValueError('target_parameters LoRA does not support lora_dropout != 0')
-        if getattr(config, 'fan_in_fan_out', False):
-            raise ValueError('target_parameters LoRA does not support fan_in_fan_out=True')
-        if getattr(config, 'use_dora', False):
-            raise ValueError('target_parameters LoRA does not support use_dora=True')
-        if getattr(config, 'lora_bias', False):
-            raise ValueError('target_parameters LoRA does not support lora_bias=True')
-        self.r[slot_name] = config.r
-        self.scaling[slot_name] = config.lora_alpha / (math.sqrt(config.r) if getattr(config, 'use_rslora', False)
-                                                       else config.r)
+        """Rank and scaling of the tenant that takes the slot.  ``ValueError`` for an unknown slot, a rank outside
+        ``1 .. max_r`` and the options packed-parameter LoRA does not have (reference :136-156)."""
+        self._slot(slot_name)
+        r = config.r
+        if r <= 0:
+            raise ValueError(f'`r` should be a positive integer value but the value passed is {r}')
+        if r > self.max_r:
+            raise ValueError(f'LoRA rank {r} exceeds max_r={self.max_r}')
+        for attr, what in _REFUSED_OPTIONS:
+            if getattr(config, attr, None):
+                raise ValueError(f'target_parameters LoRA does not support {what}')
+        self.r[slot_name] = r
+        self.scaling[slot_name] = config.lora_alpha / (math.sqrt(r) if getattr(config, 'use_rslora', False) else r)
+
+    def live_blocks(self, slot_name: str):
+        """``A[:, :r, :]`` and ``B[:, :, :r]`` of a slot: what its tenant trains and what a checkpoint holds."""
+        a, b = self._slot(slot_name)
+        r = self.r[slot_name]
+        return a[:, :r, :], b[:, :, :r]
 
     def get_delta_weight(self, slot_name: str, out_in_layout: bool = True) -> torch.Tensor:
-        """The merged ``[E, out, in]`` (or ``[E, in, out]``) delta of the reference (:158-179); for export and checks."""
-        if slot_name not in self.lora_A:
-            raise ValueError(f'Unknown target-parameter LoRA slot: {slot_name}')
-        r = self.r[slot_name]
-        a, b = self.lora_A[slot_name][:, :r, :], self.lora_B[slot_name][:, :, :r]
-        pattern = 'eor,eri->eoi' if out_in_layout else 'eor,eri->eio'
-        return torch.einsum(pattern, b, a) * self.scaling[slot_name]
+        """The merged delta ``B A * scaling`` per expert as the reference forms it (:158-179), ``[E, out, in]`` or
+        ``[E, in, out]``.  The kernels never build it; it is there for export and for checks."""
+        a, b = self.live_blocks(slot_name)
+        delta = torch.bmm(b, a) * self.scaling[slot_name]
+        return delta if out_in_layout else delta.transpose(1, 2)
+
+    def _keys(self):
+        return f'{self.peft_key_prefix}.lora_A.weight', f'{self.peft_key_prefix}.lora_B.weight'
 
     def get_state_dict(self, slot_name: str) -> Dict[str, torch.Tensor]:
-        r = self.r[slot_name]
-        return {
-            f'{self.peft_key_prefix}.lora_A.weight': self.lora_A[slot_name][:, :r, :].detach().clone(),
-            f'{self.peft_key_prefix}.lora_B.weight': self.lora_B[slot_name][:, :, :r].detach().clone(),
-        }
+        return {k: v.detach().clone() for k, v in zip(self._keys(), self.live_blocks(slot_name))}
 
     def set_state_dict(self, slot_name: str, state_dict: Dict[str, torch.Tensor]) -> set:
-        key_a, key_b = f'{self.peft_key_prefix}.lora_A.weight', f'{self.peft_key_prefix}.lora_B.weight'
-        if key_a not in state_dict and key_b not in state_dict:
+        """Load a tenant's ``[:r]`` blocks (the rest of the slot becomes zero); returns the keys it used.  Neither
+        key present: nothing to do; one of the two: ``KeyError``; a wrong shape: ``ValueError``."""
+        keys = self._keys()
+        have = [k in state_dict for k in keys]
+        if not any(have):
             return set()
-        if key_a not in state_dict or key_b not in state_dict:
+        if not all(have):
             raise KeyError(f'Missing target-parameter LoRA pair for {self.peft_key_prefix}')
-        r = self.r[slot_name]
-        a, b = state_dict[key_a], state_dict[key_b]
-        if tuple(a.shape) != (self.num_experts, r, self.in_features):
-            raise ValueError(f'Expected lora_A shape {(self.num_experts, r, self.in_features)}, got {tuple(a.shape)}')
-        if tuple(b.shape) != (self.num_experts, self.out_features, r):
-            raise ValueError(f'Expected lora_B shape {(self.num_experts, self.out_features, r)}, got {tuple(b.shape)}')
+        blocks = self.live_blocks(slot_name)
+        for side, key, block in zip(('lora_A', 'lora_B'), keys, blocks):
+            if tuple(state_dict[key].shape) != tuple(block.shape):
+                raise ValueError(f'Expected {side} shape {tuple(block.shape)}, got {tuple(state_dict[key].shape)}')
         with torch.no_grad():
-            pa, pb = self.lora_A[slot_name], self.lora_B[slot_name]
-            pa.zero_()
-            pb.zero_()
-            pa[:, :r, :].copy_(a.to(device=pa.device, dtype=pa.dtype))
-            pb[:, :, :r].copy_(b.to(device=pb.device, dtype=pb.dtype))
-        return {key_a, key_b}
+            for full, key, block in zip(self._slot(slot_name), keys, blocks):
+                full.zero_()
+                block.copy_(state_dict[key].to(device=full.device, dtype=full.dtype))
+        return set(keys)
 
-    def groups(self, tenant_slots: Sequence[str]) -> AdapterGroups:
-        """Group table for keys ``expert * len(tenant_slots) + tenant``: one block of a slot tensor per group."""
+    def groups(self, tenant_slots: Sequence[Optional[str]]) -> AdapterGroups:
+        """Group table for keys ``expert * len(tenant_slots) + tenant``: one block of a slot tensor per group.
+        A ``None`` entry is a tenant without LoRA on this parameter (its groups have rank 0)."""
         nt = len(tenant_slots)
+        live = [s for s in tenant_slots if s is not None]
+        if not live:
+            raise ValueError('at least one tenant of the batch must hold a slot')
         # building the table costs a few host-to-device copies: kept until a slot's rank or scaling changes (moved
         # parameter storage is picked up by AdapterGroups.refresh at every call)
-        key = (tuple(tenant_slots), tuple(self.r[s] for s in tenant_slots),
-               tuple(self.scaling[s] for s in tenant_slots))
-        cache = self.__dict__.setdefault('_groups_cache', {})
-        hit = cache.get(key)
-        if hit is not None and all(x is y for x, y in zip(hit.a_tensors + hit.b_tensors,
-                                                           [self.lora_A[s] for s in tenant_slots] +
-                                                           [self.lora_B[s] for s in tenant_slots])):
+        key = (tuple(tenant_slots), tuple(self.r[s] for s in live), tuple(self.scaling[s] for s in live))
+        hit = self._groups_cache.get(key)
+        tensors = [self.lora_A[s] for s in live] + [self.lora_B[s] for s in live]
+        if hit is not None and all(x is y for x, y in zip(hit.a_tensors + hit.b_tensors, tensors)):
             return hit
-        a = [self.lora_A[s] for s in tenant_slots]
-        b = [self.lora_B[s] for s in tenant_slots]
-        n = self.num_experts * nt
-        idx = [i % nt for i in range(n)]
-        a_off = [(i // nt) * self.max_r * self.in_features for i in range(n)]
-        b_off = [(i // nt) * self.out_features * self.max_r for i in range(n)]
-        ranks = [self.r[tenant_slots[i % nt]] for i in range(n)]
-        scales = [self.scaling[tenant_slots[i % nt]] for i in range(n)]
-        if len(cache) > 16:
-            cache.clear()
-        cache[key] = AdapterGroups(a, b, ranks, scales, a_index=idx, a_offset=a_off, b_index=idx, b_offset=b_off)
-        return cache[key]
+        which = {s: i for i, s in enumerate(live)}
+        idx, a_off, b_off, ranks, scales = [], [], [], [], []
+        for g in range(self.num_experts * nt):
+            e, s = divmod(g, nt)[0], tenant_slots[g % nt]
+            idx.append(which.get(s, 0))
+            a_off.append(e * self.max_r * self.in_features)
+            b_off.append(e * self.out_features * self.max_r)
+            ranks.append(self.r[s] if s is not None else 0)
+            scales.append(self.scaling[s] if s is not None else 0.0)
+        if len(self._groups_cache) > 16:
+            self._groups_cache.clear()
+        table = AdapterGroups(tensors[:len(live)], tensors[len(live):], ranks, scales, a_index=idx, a_offset=a_off,
+                              b_index=idx, b_offset=b_off)
+        self._groups_cache[key] = table
+        return table
 
 
 def expert_lora_delta(x_sorted: torch.Tensor, y_sorted: torch.Tensor, seg: SegmentTable, slots: ExpertLoraSlots,
@@ -156,21 +168,49 @@ def expert_lora_delta(x_sorted: torch.Tensor, y_sorted: torch.Tensor, seg: Segme
     return multi_lora_delta(x_sorted, y_sorted, seg, groups, map_rows=False)
 
 
+class _ExpertPass:
+    """What the patched expert modules apply while a context of the manager is open."""
+
+    def __init__(self, slots: List[Optional[str]], token_tenant: Optional[torch.Tensor], disabled: bool):
+        self.slots = slots                  # slot name per tenant index (None: that tenant has no expert LoRA)
+        self.token_tenant = token_tenant    # [tokens] index into slots, or None: slots[0] for every token
+        self.disabled = disabled
+
+
+def _raw_module_path(root: nn.Module, module_name: str) -> str:
+    """Path of a submodule inside the model PEFT wraps, whatever ``root`` is: the model itself, the holder that
+    :func:`twinkle_amd.lora_layer.inject_adapter` returns (``model.`` in front) or a ``PeftModel``
+    (``base_model.model.`` in front)."""
+    from .lora_layer import LoraModel
+    if isinstance(root, LoraModel):
+        lead = 'model'
+    elif hasattr(root, 'peft_config') and hasattr(root, 'base_model'):
+        lead = 'base_model.model'
+    else:
+        return module_name
+    if module_name == lead:
+        return ''
+    return module_name[len(lead) + 1:] if module_name.startswith(lead + '.') else module_name
+
+
 class ExpertLoraManager:
-    """Finds packed expert parameters in a model, gives each its slot storage and keeps the tenant -> slot map.
+    """Finds packed expert parameters in a model, gives each its slot storage, keeps the tenant -> slot map and
+    makes the owning expert modules apply the active tenants' LoRA.
 
-    Host-side mirror of the reference's ``TargetParameterLoraManager``
-    (src/twinkle/model/multi_lora_target_parameters.py:281-383): same method names, arguments and errors.  What
-    differs is how a slot takes effect: the reference merges ``W + B A * scaling`` into the parameter through a
-    parametrization while a tenant is active (:182-209); here the expert forward adds the low-rank term of every
-    (expert, tenant) segment with :func:`expert_lora_delta`, and :meth:`adapter` only records which tenant is the
-    active one for callers that run one tenant per pass.
+    Host-side counterpart of the reference's ``TargetParameterLoraManager``
+    (src/twinkle/model/multi_lora_target_parameters.py:281-383): same method names, arguments and exception types.
+    How a slot takes effect differs.  The reference registers a parametrization that merges ``W + B A * scaling``
+    into the packed parameter while a tenant is active (:182-209), so the model's own expert forward sees merged
+    weights.  Here :meth:`patch` rebinds the forward of every module that owns a patched ``gate_up_proj`` /
+    ``down_proj`` pair (the packed-experts layout of transformers: ``forward(hidden_states, top_k_index,
+    top_k_weights)``) to :func:`moe_experts_block`, which adds the low-rank term per (expert, tenant) segment:
+    under :meth:`adapter` every token uses the one tenant's slot, under :meth:`batch` every token its own
+    tenant's, with ``disable_lora`` or outside any context the module's original forward runs untouched.
 
-    The slot tensors have the reference's shapes for both storage layouts (``lora_A [E, max_r, in_features]``,
-    ``lora_B [E, out_features, max_r]`` with the reference's naming of the two trailing dimensions).  The segmented
-    kernels apply ``scale * (x A^T) B^T``, which is the reference's merged form when the expert computes
-    ``F.linear(x, W[e])`` on ``[E, out, in]`` storage (its expert forward, moe/expert_parallel.py:360-371);
-    for modules that compute ``x @ W[e]`` the merged delta of :meth:`ExpertLoraSlots.get_delta_weight` applies.
+    The slot tensors have the reference's shapes for both storage layouts.  The segmented kernels apply
+    ``scale * (x A^T) B^T``, the reference's merged form for experts that compute ``F.linear(x, W[e])`` on
+    ``[E, out, in]`` storage (its expert forward, moe/expert_parallel.py:360-371); a module that stores
+    ``[E, in, out]`` keeps its own forward and can merge :meth:`ExpertLoraSlots.get_delta_weight` itself.
     """
 
     def __init__(self, max_loras: int, max_r: int):
@@ -179,115 +219,145 @@ class ExpertLoraManager:
         self.wrappers: List[ExpertLoraSlots] = []
         self.tenant_to_slot: Dict[str, str] = {}
         self.tenant_configs: Dict[str, object] = {}
+        self.active_pass: Optional[_ExpertPass] = None
         self._target_parameters: Optional[tuple] = None
 
+    # ---- installing -----------------------------------------------------------------------------------------------
     def patch(self, model: nn.Module, target_parameters) -> None:
-        """Attach slot storage to every parameter named (or suffixed ``.name``) in ``target_parameters``
-        (reference :291-319).  3-D parameters are ``[E, out, in]`` unless the owning module says
-        ``is_transposed`` (then ``[E, in, out]``), 2-D ones ``[out, in]`` with one expert (:47-52)."""
-        target_parameters = tuple(target_parameters)
-        if not target_parameters:
+        """Attach slot storage to every parameter whose dotted name equals an entry of ``target_parameters`` or ends
+        in ``.entry`` (reference :291-319).  A 3-D parameter is ``[E, out, in]``, or ``[E, in, out]`` when its module
+        says ``is_transposed``; a 2-D one is ``[out, in]`` with one expert (:47-52).  Patching again with the same
+        list is a no-op, with another list a ``ValueError``; so is a list that matches nothing."""
+        wanted = tuple(target_parameters)
+        if not wanted:
             return
         if self._target_parameters is not None:
-            if self._target_parameters != target_parameters:
-                raise ValueError(
-                    f'target_parameters already patched as {self._target_parameters}, got {target_parameters}')
+            if self._target_parameters != wanted:
+                raise ValueError(f'target_parameters already patched as {self._target_parameters}, got {wanted}')
             return
-        found = []
+        owners: Dict[str, list] = {}       # module name -> [(module, parameter name, slots)], in discovery order
         for module_name, module in model.named_modules():
             for param_name, parameter in module.named_parameters(recurse=False):
-                key = f'{module_name}.{param_name}' if module_name else param_name
-                if key in target_parameters or any(key.endswith(f'.{t}') for t in target_parameters):
-                    if parameter.ndim not in (2, 3):
-                        raise ValueError(
-                            f'target parameter {key} has {parameter.ndim} dimensions; only 2D and 3D are supported')
-                    found.append((module_name, module, param_name, parameter))
-        if not found:
-            raise ValueError(f'target_parameters={target_parameters} were set but no parameter was matched')
-        per_module: Dict[str, List[ExpertLoraSlots]] = {}
-        for module_name, module, param_name, parameter in found:
-            if parameter.ndim == 3:
-                out_in = not getattr(module, 'is_transposed', False)
-                experts = parameter.shape[0]
-                fin, fout = (parameter.shape[-1], parameter.shape[-2]) if out_in else (parameter.shape[-2],
-                                                                                      parameter.shape[-1])
-            else:
-                out_in, experts = True, 1
-                fout, fin = parameter.shape
-            device = 'cpu' if parameter.device.type == 'meta' else parameter.device
-            slots = ExpertLoraSlots(experts, fin, fout, self.max_loras, self.max_r, dtype=parameter.dtype, device=device)
-            slots.parameter_key = f'{module_name}.{param_name}' if module_name else param_name
-            slots.out_in_layout = out_in
-            slots.active_adapter, slots.disable_adapters = None, False
-            module.add_module(f'_twinkle_lora_{param_name}', slots)
-            self.wrappers.append(slots)
-            per_module.setdefault(module_name, []).append(slots)
-        # PEFT nests one wrapper per target parameter of a module: the first one found is the innermost (:321-330)
-        for module_name, group in per_module.items():
-            prefix = f'base_model.model.{module_name}' if module_name else 'base_model.model'
-            for index, slots in enumerate(group):
-                nested = '.'.join(['base_layer'] * (len(group) - index - 1))
-                slots.peft_key_prefix = f'{prefix}.{nested}' if nested else prefix
-        self._target_parameters = target_parameters
+                dotted = f'{module_name}.{param_name}' if module_name else param_name
+                if not any(dotted == t or dotted.endswith('.' + t) for t in wanted):
+                    continue
+                if parameter.ndim == 3:
+                    experts, d1, d2 = parameter.shape
+                    out_in = not getattr(module, 'is_transposed', False)
+                    fout, fin = (d1, d2) if out_in else (d2, d1)
+                elif parameter.ndim == 2:
+                    experts, out_in = 1, True
+                    fout, fin = parameter.shape
+                else:
+                    raise ValueError(f'target parameter {dotted} has {parameter.ndim} dimensions; only 2D and 3D '
+                                     'are supported')
+                device = 'cpu' if parameter.device.type == 'meta' else parameter.device
+                slots = ExpertLoraSlots(experts, fin, fout, self.max_loras, self.max_r, dtype=parameter.dtype,
+                                        device=device)
+                slots.parameter_key, slots.out_in_layout = dotted, out_in
+                owners.setdefault(module_name, []).append((module, param_name, slots))
+        if not owners:
+            raise ValueError(f'target_parameters={wanted} were set but no parameter was matched')
+        for module_name, found in owners.items():
+            # PEFT wraps a module once per target parameter, the first one found innermost: its keys carry one
+            # `base_layer` per wrapper outside it (reference :321-330)
+            raw = _raw_module_path(model, module_name)
+            root = 'base_model.model' + ('.' + raw if raw else '')
+            for depth, (module, param_name, slots) in enumerate(found):
+                slots.peft_key_prefix = '.'.join([root] + ['base_layer'] * (len(found) - 1 - depth))
+                module.add_module(f'_twinkle_lora_{param_name}', slots)
+                self.wrappers.append(slots)
+            self._bind_forward(found[0][0], {name: slots for _, name, slots in found})
+        self._target_parameters = wanted
 
+    def _bind_forward(self, module: nn.Module, by_param: Dict[str, ExpertLoraSlots]) -> None:
+        """Route a packed-experts module through :func:`moe_experts_block` while a tenant is active."""
+        gate_up, down = by_param.get('gate_up_proj'), by_param.get('down_proj')
+        packed = (all(isinstance(getattr(module, n, None), torch.Tensor) and getattr(module, n).ndim == 3
+                      for n in ('gate_up_proj', 'down_proj')) and not getattr(module, 'is_transposed', False)
+                  and (hasattr(module, 'act_fn') or hasattr(module, '_apply_gate')))
+        if not packed or (gate_up is None and down is None):
+            return
+        manager, original = self, module.forward
+
+        def forward(mod, hidden_states, top_k_index, top_k_weights):
+            now = manager.active_pass
+            if now is None or now.disabled or all(s is None for s in now.slots):
+                return original(hidden_states, top_k_index, top_k_weights)
+            if not hidden_states.is_cuda:
+                raise RuntimeError('expert LoRA needs the activations on the GPU: this path has no CPU implementation')
+            tokens = hidden_states.reshape(-1, hidden_states.shape[-1])
+            tenant = now.token_tenant
+            if tenant is not None and tenant.numel() != tokens.shape[0]:
+                raise ValueError(f'the batch has {tenant.numel()} rows but the experts see {tokens.shape[0]} tokens')
+            out = moe_experts_block(tokens, top_k_index.reshape(tokens.shape[0], -1),
+                                    top_k_weights.reshape(tokens.shape[0], -1), tenant, mod, now.slots, gate_up, down)
+            return out.view(hidden_states.shape)
+
+        module.forward = MethodType(forward, module)
+        module._tk_original_forward = original
+
+    # ---- tenants --------------------------------------------------------------------------------------------------
     def acquire(self, tenant_adapter_name: str, slot_name: str, config) -> None:
         if tenant_adapter_name in self.tenant_to_slot:
             raise ValueError(f'Lora {tenant_adapter_name} already exists')
         if getattr(config, 'target_parameters', None) and not self.wrappers:
             raise ValueError('target_parameters LoRA slots must be patched before acquire')
+        for slots in self.wrappers:           # all checks pass before anything is recorded
+            slots.configure_slot(slot_name, config)
         self.tenant_to_slot[tenant_adapter_name] = slot_name
         self.tenant_configs[tenant_adapter_name] = config
-        for slots in self.wrappers:
-            slots.configure_slot(slot_name, config)
 
     def release(self, tenant_adapter_name: str) -> None:
-        slot_name = self.tenant_to_slot.pop(tenant_adapter_name, None)
         self.tenant_configs.pop(tenant_adapter_name, None)
-        if slot_name is None:
-            return
-        for slots in self.wrappers:
-            slots.reset_slot(slot_name)
+        slot_name = self.tenant_to_slot.pop(tenant_adapter_name, None)
+        if slot_name is not None:
+            for slots in self.wrappers:
+                slots.reset_slot(slot_name)
 
     @contextmanager
-    def adapter(self, tenant_adapter_name: str, disable_lora: bool = False):
-        """One tenant per pass: every slot storage learns which slot is active (``None`` for unknown tenants)."""
-        slot_name = self.tenant_to_slot.get(tenant_adapter_name)
-        previous = [(s.active_adapter, s.disable_adapters) for s in self.wrappers]
-        for s in self.wrappers:
-            s.active_adapter, s.disable_adapters = slot_name, disable_lora
+    def _during(self, expert_pass: _ExpertPass):
+        previous, self.active_pass = self.active_pass, expert_pass
         try:
-            yield
+            yield expert_pass
         finally:
-            for s, (a, d) in zip(self.wrappers, previous):
-                s.active_adapter, s.disable_adapters = a, d
+            self.active_pass = previous
+
+    def adapter(self, tenant_adapter_name: str, disable_lora: bool = False):
+        """One tenant for every token of the calls inside; a tenant without expert LoRA leaves the experts as they
+        are, and so does ``disable_lora`` (reference :352-358)."""
+        return self._during(_ExpertPass([self.tenant_to_slot.get(tenant_adapter_name)], None, disable_lora))
+
+    def batch(self, tenant_adapter_names: Sequence[str], token_tenant: torch.Tensor):
+        """Many tenants in one pass: token ``i`` uses ``tenant_adapter_names[token_tenant[i]]``; an index outside
+        the list (``-1`` for padding) gives the token the frozen experts alone.  No counterpart in the reference,
+        which activates one tenant per call."""
+        slots = [self.tenant_to_slot.get(t) for t in tenant_adapter_names] + [None]
+        index = token_tenant.reshape(-1).to(torch.int32)
+        index = torch.where((index >= 0) & (index < len(slots) - 1), index, torch.full_like(index, len(slots) - 1))
+        return self._during(_ExpertPass(slots, index, False))
 
     def slots_of(self, tenant_adapter_names: Sequence[str]) -> List[str]:
         """Slot names of the tenants of a mixed batch, in the order their ids appear in the group keys."""
         return [self.tenant_to_slot[t] for t in tenant_adapter_names]
 
-    def parameters_for_tenant(self, tenant_adapter_name: str) -> List[nn.Parameter]:
-        return [p for _, p in self.named_slot_parameters(tenant_adapter_name)]
-
+    # ---- parameters and state ---------------------------------------------------------------------------------------
     def named_slot_parameters(self, tenant_adapter_name: str):
         slot_name = self.tenant_to_slot[tenant_adapter_name]
         for slots in self.wrappers:
-            if slot_name in slots.lora_A:
-                yield f'{slots.parameter_key}.lora_A.{slot_name}.weight', slots.lora_A[slot_name]
-                yield f'{slots.parameter_key}.lora_B.{slot_name}.weight', slots.lora_B[slot_name]
+            for side in ('lora_A', 'lora_B'):
+                yield f'{slots.parameter_key}.{side}.{slot_name}.weight', getattr(slots, side)[slot_name]
+
+    def parameters_for_tenant(self, tenant_adapter_name: str) -> List[nn.Parameter]:
+        return [p for _, p in self.named_slot_parameters(tenant_adapter_name)]
 
     def get_state_dict(self, tenant_adapter_name: str) -> Dict[str, torch.Tensor]:
         slot_name = self.tenant_to_slot[tenant_adapter_name]
-        state = {}
-        for slots in self.wrappers:
-            state.update(slots.get_state_dict(slot_name))
-        return state
+        return {k: v for slots in self.wrappers for k, v in slots.get_state_dict(slot_name).items()}
 
     def set_state_dict(self, tenant_adapter_name: str, state_dict: Dict[str, torch.Tensor]) -> set:
         slot_name = self.tenant_to_slot[tenant_adapter_name]
-        consumed = set()
-        for slots in self.wrappers:
-            consumed.update(slots.set_state_dict(slot_name, state_dict))
-        return consumed
+        return set().union(*[slots.set_state_dict(slot_name, state_dict) for slots in self.wrappers])
 
 
 def _is_silu(fn) -> bool:

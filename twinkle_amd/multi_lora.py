@@ -64,6 +64,233 @@ def _is_lora_layer(module) -> bool:
     return all(hasattr(module, a) for a in ('base_layer', 'lora_A', 'lora_B', 'lora_dropout'))
 
 
+# ---------------------------------------------------------------------------------------------------------------
+# What the patched forward needs beyond the reference's ``MultiLora`` surface (``loras``, ``find_lora``,
+# ``find_lora_by_tenant``, ``match_target_modules``, ``max_loras``): the per-layer group tables, the segment table of
+# the open batch and the one-segment tables of ``adapter()``.  It lives in one object that is attached to the
+# ``MultiLora`` instance the first time it is needed, and every helper below takes that instance as an argument,
+# so the functions work on the reference's own class as well as on the one in this file.
+# ---------------------------------------------------------------------------------------------------------------
+class _PathState:
+
+    def __init__(self):
+        self.layer_groups: Dict[tuple, tuple] = {}
+        self.batch_table: Optional[SegmentTable] = None
+        self.uniform_tables: Dict[tuple, SegmentTable] = {}
+
+
+def _path_state(ml) -> _PathState:
+    state = ml.__dict__.get('_tk_path_state')
+    if state is None:
+        state = ml.__dict__['_tk_path_state'] = _PathState()
+    return state
+
+
+def _hashable(v):
+    return tuple(sorted(v)) if isinstance(v, (list, set, tuple)) else v
+
+
+def _ownership(ml):
+    """Changes whenever a slot changes hands or its tenant's settings do: the key the group tables are cached by.
+    The class in this file counts its acquire / release calls; for any other object the tenants' settings are read."""
+    version = ml.__dict__.get('_version')
+    if version is not None:
+        return version
+    return tuple((t.tenant_adapter_name, getattr(t.tenant_config, 'r', None), getattr(t.tenant_config, 'lora_alpha', None),
+                  bool(getattr(t.tenant_config, 'use_rslora', False)),
+                  _hashable(getattr(t.tenant_config, 'target_modules', None))) for t in ml.loras)
+
+
+def _table_for(ml, rows: int, slot_index: int, device) -> SegmentTable:
+    """The one-segment table of ``adapter()``: every row belongs to slot ``slot_index``."""
+    tables = _path_state(ml).uniform_tables
+    key = (rows, slot_index, str(device))
+    table = tables.get(key)
+    if table is None:
+        if len(tables) >= 64:
+            tables.clear()
+        keys = torch.full((rows,), slot_index, dtype=torch.int32, device=device)
+        table = tables[key] = build_segments(keys, len(ml.loras), want_perm=False, want_offsets=False)
+    return table
+
+
+def _groups_for(ml, layer, only_slot: Union[None, str, Tuple[str, ...]]) -> Optional[AdapterGroups]:
+    """Rank/scale table of a layer: slots whose tenant targets this layer are live, the rest rank 0.
+    ``only_slot`` narrows the live slots to one name or a tuple of names (``None``: every slot with a tenant)."""
+    cache = _path_state(ml).layer_groups
+    key = (id(layer), only_slot)
+    owners = _ownership(ml)
+    cached = cache.get(key)
+    if cached is not None and cached[0] == owners:
+        return cached[1]
+    a, b, ranks, scales = [], [], [], []
+    for slot in ml.loras:
+        name = slot.adapter_name
+        if name not in layer.lora_A.keys():
+            raise ValueError(f'layer {layer.layer_name} has no slot {name}')
+        a.append(layer.lora_A[name].weight)
+        b.append(layer.lora_B[name].weight)
+        cfg = slot.tenant_config
+        wanted = only_slot is None or only_slot == name or (isinstance(only_slot, tuple) and name in only_slot)
+        live = cfg is not None and wanted and ml.match_target_modules(layer.layer_name, cfg.target_modules)
+        if live:
+            ranks.append(cfg.r)
+            scales.append(cfg.lora_alpha / (cfg.r**0.5 if getattr(cfg, 'use_rslora', False) else cfg.r))
+        else:
+            ranks.append(0)
+            scales.append(0.0)
+    compute_dtype = getattr(ml, 'lora_compute_dtype', None)
+    if max(ranks) == 0:
+        groups = None
+    elif compute_dtype is not None and a[0].dtype != compute_dtype:
+        groups = AdapterGroups([torch.empty_like(t, dtype=compute_dtype) for t in a],
+                               [torch.empty_like(t, dtype=compute_dtype) for t in b], ranks, scales, master_a=a,
+                               master_b=b)
+    else:
+        groups = AdapterGroups(a, b, ranks, scales)
+    if len(cache) > 8192:   # batches over ever-changing tenant sets: start over
+        cache.clear()
+    cache[key] = (owners, groups)
+    return groups
+
+
+def _slot_dropout(ml, layer, only_slot: Optional[str], table):
+    """The dropout module the LoRA branch applies: the slot's own (reference :317).  In a mixed batch one module
+    serves every row, which is what the reference computes only if the live slots' modules agree (identity, or
+    one probability): anything else is refused rather than applied to the wrong rows."""
+    if only_slot is not None:
+        return layer.lora_dropout[only_slot]
+    names = getattr(table, 'live_slots', None) or [t.adapter_name for t in ml.loras]
+    mods = [layer.lora_dropout[n] for n in names if n in layer.lora_dropout.keys()]
+    first = mods[0] if mods else torch.nn.Identity()
+    for m in mods[1:]:
+        if type(m) is not type(first) or getattr(m, 'p', 0.0) != getattr(first, 'p', 0.0):
+            raise NotImplementedError(
+                f'layer {layer.layer_name}: the slots of a mixed batch have different lora_dropout modules')
+    return first
+
+
+@contextmanager
+def batch(ml, tenant_adapter_names: Sequence[str], row_tenant: torch.Tensor, check: bool = False):
+    """Many tenants in one forward/backward: row ``i`` uses ``tenant_adapter_names[row_tenant[i]]``.
+
+    ``ml`` is a ``MultiLora`` whose layers carry the forward of :meth:`MultiLora._patch_lora_forward` (the class in
+    this file, or the reference's ``twinkle.model.multi_lora.MultiLora``).
+    ``row_tenant`` is an integer GPU tensor with one entry per row of the
+    flattened ``[rows, features]`` activations (so ``batch * seq`` entries for
+    ``[batch, seq, features]`` inputs).  The segment table is built once here
+    and shared by every patched layer called inside the context.  A row whose entry is negative (padding,
+    ignored rows) or not below ``len(tenant_adapter_names)`` belongs to no tenant: it keeps the base output and
+    adds to nobody's gradients.  ``check=True`` instead verifies that every entry of ``row_tenant`` indexes
+    ``tenant_adapter_names`` (one device synchronisation) and raises ``ValueError`` otherwise.
+    """
+    slots = [ml.find_lora_by_tenant(n).index for n in tenant_adapter_names]
+    if check and row_tenant.numel():
+        lo, hi = int(row_tenant.min()), int(row_tenant.max())
+        if lo < 0 or hi >= len(slots):
+            raise ValueError(f'row_tenant holds {lo}..{hi} but the batch has {len(slots)} tenants')
+    lut = torch.tensor(slots, dtype=torch.int32, device=row_tenant.device)
+    rt = row_tenant.reshape(-1).long()
+    known = (rt >= 0) & (rt < len(slots))
+    keys = torch.where(known, lut[rt.clamp(0, len(slots) - 1)], torch.full_like(lut[:1], -1))
+    table = build_segments(keys, len(ml.loras), want_perm=False, want_offsets=False)
+    # only the tenants of this batch are live inside the context: the others get no gradient, like the
+    # adapters the reference leaves inactive
+    table.live_slots = tuple(sorted({ml.loras[i].adapter_name for i in slots}))
+    state = _path_state(ml)
+    previous, state.batch_table = state.batch_table, table
+    experts = getattr(getattr(ml, 'target_parameter_manager', None), 'batch', None)   # this file's manager only
+    try:
+        if experts is not None:
+            with experts(tenant_adapter_names, rt):
+                yield table
+        else:
+            yield table
+    finally:
+        state.batch_table = previous
+
+
+def _modules_of(ml):
+    return ml.module if isinstance(ml.module, list) else [ml.module]
+
+
+def share_inputs(ml, layer_groups: Sequence[Sequence]) -> None:
+    """Declare groups of patched layers that the model calls one after the other on the same tensor
+    (``[[q_proj, k_proj, v_proj], [gate_proj, up_proj]]`` per block; modules or their names inside the
+    patched module).  Model code stays as it is: the first layer of a group that sees a new input computes
+    the outputs of the whole group through :func:`forward_shared` and the siblings, called with the same
+    tensor, pick theirs up.  A sibling called with another tensor (or twice) simply starts a new group
+    computation, so results never depend on the call pattern; outputs nobody collects are dropped at the next
+    call.  ``share_inputs([])`` clears nothing: call :func:`unshare_inputs` for that.
+    """
+    named = {n: sub for m in _modules_of(ml) for n, sub in m.named_modules()}
+    for group in layer_groups:
+        layers = [named[m] if isinstance(m, str) else m for m in group]
+        if not 2 <= len(layers) <= 4:
+            raise ValueError(f'a group of shared inputs has 2 to 4 layers, got {len(layers)}')
+        for layer in layers:
+            if not _is_lora_layer(layer) or not hasattr(layer, 'layer_name'):
+                raise ValueError('share_inputs takes layers that patch() has patched')
+        if len({layer.in_features for layer in layers}) != 1:
+            raise ValueError('layers that share an input must agree in in_features')
+        state = _SharedInputGroup(layers)
+        for layer in layers:
+            layer._tk_shared_inputs = state
+
+def unshare_inputs(ml) -> None:
+    for m in _modules_of(ml):
+        for sub in m.modules():
+            if hasattr(sub, '_tk_shared_inputs'):
+                del sub._tk_shared_inputs
+
+def forward_shared(ml, layers: Sequence, x: torch.Tensor) -> Tuple[torch.Tensor, ...]:
+    """``tuple(layer(x) for layer in layers)`` for patched layers that read the same ``x`` (q / k / v,
+    gate / up), with the LoRA terms of all of them computed by one shared call: ``x`` is read once in
+    forward, and once in backward for every layer's dA, and the gradient of ``x`` is updated once.
+
+    The reference has no per-input entry (every projection runs its own two ``F.linear`` calls, :322-326);
+    a caller opts in by routing such a group of projections through this function.  Falls back to calling
+    the layers one by one whenever one of them would not take the plain in-place path (adapters disabled,
+    a layer without a live adapter, dtype casts, non-``nn.Linear`` base layers).
+    """
+    layers = list(layers)
+    table = _path_state(ml).batch_table
+    only_slot = None
+    ok = 2 <= len(layers) <= 4 and x.is_cuda
+    groups_list = []
+    for layer in layers if ok else ():
+        if table is None:
+            active = [n for n in layer.active_adapters if n in layer.lora_A.keys()]
+            slot = active[0] if active else None
+            if slot is None or (only_slot is not None and slot != only_slot):
+                ok = False
+                break
+            only_slot = slot
+        groups = None if layer.disable_adapters else _groups_for(
+            ml, layer, only_slot if table is None else getattr(table, 'live_slots', None))
+        base = layer.base_layer
+        if (groups is None or groups.dtype != x.dtype or type(base) is not torch.nn.Linear
+                or base.weight.dtype != x.dtype or base._forward_hooks or base._forward_pre_hooks
+                or not isinstance(_slot_dropout(ml, layer, only_slot, table), torch.nn.Identity)):
+            ok = False
+            break
+        groups_list.append(groups)
+    if not ok:
+        return tuple(getattr(layer, '_tk_forward_one', layer)(x) for layer in layers)
+    for groups in groups_list:
+        groups.sync_masters()
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
+        x2 = x2.contiguous()
+    if table is None:
+        table = _table_for(ml, x2.shape[0], ml.find_lora(only_slot).index, x2.device)
+    elif table.rows != x2.shape[0]:
+        raise ValueError(f'batch() was given {table.rows} rows but the shared input has {x2.shape[0]}')
+    outs = multi_lora_linear_shared(x2, [layer.base_layer.weight for layer in layers],
+                                    [layer.base_layer.bias for layer in layers], table, groups_list)
+    return tuple(y.view(*x.shape[:-1], y.shape[-1]) for y in outs)
+
+
 class MultiLora:
 
     def __init__(self, max_loras=5, max_r=32, max_length: int = 8192, lora_compute_dtype: Optional[torch.dtype] = None):
@@ -78,10 +305,7 @@ class MultiLora:
         self.lora_compute_dtype = lora_compute_dtype
         self.loras: List[LoraTenant] = []
         self.module = None
-        self._version = 0                 # bumped whenever slot ownership changes
-        self._layer_groups: Dict[int, tuple] = {}
-        self._batch_table: Optional[SegmentTable] = None
-        self._uniform_tables: Dict[tuple, SegmentTable] = {}
+        self._version = 0                 # bumped whenever slot ownership changes (see _ownership)
         # packed expert parameters (reference :40): slot storage per target parameter, same tenant -> slot map
         self.target_parameter_manager = ExpertLoraManager(max_loras=max_loras, max_r=max_r)
 
@@ -208,7 +432,7 @@ class MultiLora:
                 else:
                     yield self.find_lora_by_tenant(tenant_adapter_name).adapter_name
         finally:
-            self._uniform_tables.clear()
+            _path_state(self).uniform_tables.clear()
 
     @contextmanager
     def _disable_lora_context(self, tenant_adapter_name):
@@ -218,80 +442,19 @@ class MultiLora:
         finally:
             self.activate_adapter(tenant_adapter_name, call_enable=True)
 
-    @contextmanager
     def batch(self, tenant_adapter_names: Sequence[str], row_tenant: torch.Tensor, check: bool = False):
-        """Many tenants in one forward/backward: row ``i`` uses ``tenant_adapter_names[row_tenant[i]]``.
+        """Many tenants in one forward/backward: row ``i`` uses ``tenant_adapter_names[row_tenant[i]]`` (see the
+        module-level :func:`batch`, which this calls).  No counterpart in the reference, whose ``adapter()``
+        activates one tenant per call."""
+        return batch(self, tenant_adapter_names, row_tenant, check)
 
-        ``row_tenant`` is an integer GPU tensor with one entry per row of the
-        flattened ``[rows, features]`` activations (so ``batch * seq`` entries for
-        ``[batch, seq, features]`` inputs).  The segment table is built once here
-        and shared by every patched layer called inside the context.  A row whose entry is negative (padding,
-        ignored rows) or not below ``len(tenant_adapter_names)`` belongs to no tenant: it keeps the base output and
-        adds to nobody's gradients.  ``check=True`` instead verifies that every entry of ``row_tenant`` indexes
-        ``tenant_adapter_names`` (one device synchronisation) and raises ``ValueError`` otherwise.
-        """
-        slots = [self.find_lora_by_tenant(n).index for n in tenant_adapter_names]
-        if check and row_tenant.numel():
-            lo, hi = int(row_tenant.min()), int(row_tenant.max())
-            if lo < 0 or hi >= len(slots):
-                raise ValueError(f'row_tenant holds {lo}..{hi} but the batch has {len(slots)} tenants')
-        lut = torch.tensor(slots, dtype=torch.int32, device=row_tenant.device)
-        rt = row_tenant.reshape(-1).long()
-        known = (rt >= 0) & (rt < len(slots))
-        keys = torch.where(known, lut[rt.clamp(0, len(slots) - 1)], torch.full_like(lut[:1], -1))
-        table = build_segments(keys, self.max_loras, want_perm=False, want_offsets=False)
-        # only the tenants of this batch are live inside the context: the others get no gradient, like the
-        # adapters the reference leaves inactive
-        table.live_slots = tuple(sorted({self.loras[i].adapter_name for i in slots}))
-        previous, self._batch_table = self._batch_table, table
-        try:
-            yield table
-        finally:
-            self._batch_table = previous
-
-    def _table_for(self, rows: int, slot_index: int, device) -> SegmentTable:
-        key = (rows, slot_index, str(device))
-        table = self._uniform_tables.get(key)
-        if table is None:
-            keys = torch.full((rows,), slot_index, dtype=torch.int32, device=device)
-            table = build_segments(keys, self.max_loras, want_perm=False, want_offsets=False)
-            self._uniform_tables[key] = table
-        return table
+    @property
+    def _batch_table(self) -> Optional[SegmentTable]:
+        return _path_state(self).batch_table
 
     # ------------------------------------------------------------- patching
-    def _groups_for(self, layer, only_slot: Union[None, str, Tuple[str, ...]]) -> Optional[AdapterGroups]:
-        """Rank/scale table of a layer: slots whose tenant targets this layer are live, the rest rank 0.
-        ``only_slot`` narrows the live slots to one name or a tuple of names (``None``: every slot with a tenant)."""
-        key = (id(layer), only_slot)
-        cached = self._layer_groups.get(key)
-        if cached is not None and cached[0] == self._version:
-            return cached[1]
-        a, b, ranks, scales = [], [], [], []
-        for slot in self.loras:
-            name = slot.adapter_name
-            if name not in layer.lora_A.keys():
-                raise ValueError(f'layer {layer.layer_name} has no slot {name}')
-            a.append(layer.lora_A[name].weight)
-            b.append(layer.lora_B[name].weight)
-            cfg = slot.tenant_config
-            wanted = only_slot is None or only_slot == name or (isinstance(only_slot, tuple) and name in only_slot)
-            live = cfg is not None and wanted and self.match_target_modules(layer.layer_name, cfg.target_modules)
-            if live:
-                ranks.append(cfg.r)
-                scales.append(cfg.lora_alpha / (cfg.r**0.5 if getattr(cfg, 'use_rslora', False) else cfg.r))
-            else:
-                ranks.append(0)
-                scales.append(0.0)
-        if max(ranks) == 0:
-            groups = None
-        elif self.lora_compute_dtype is not None and a[0].dtype != self.lora_compute_dtype:
-            cd = self.lora_compute_dtype
-            groups = AdapterGroups([torch.empty_like(t, dtype=cd) for t in a], [torch.empty_like(t, dtype=cd) for t in b],
-                                   ranks, scales, master_a=a, master_b=b)
-        else:
-            groups = AdapterGroups(a, b, ranks, scales)
-        self._layer_groups[key] = (self._version, groups)
-        return groups
+    def _groups_for(self, layer, only_slot=None) -> Optional[AdapterGroups]:
+        return _groups_for(self, layer, only_slot)
 
     def _patch_lora_forward(_self, name, base_layer):
         """Rebind ``forward`` on one LoRA layer (reference :289-331, Linear branch)."""
@@ -307,35 +470,34 @@ class MultiLora:
             self._check_forward_args(x)
             out = shared.take(self, x)
             if out is None:
-                outs = _self.forward_shared(shared.layers, x)
+                outs = forward_shared(_self, shared.layers, x)
                 shared.fill(x, outs, self)
                 out = outs[shared.layers.index(self)]
             return out
 
         def _forward_one(self, x: torch.Tensor, *args, **kwargs) -> torch.Tensor:
             self._check_forward_args(x, *args, **kwargs)
-            table = _self._batch_table
+            table = _path_state(_self).batch_table
             only_slot = None
             if table is None:
                 # one adapter per call: the active slot, if this layer has it (reference :306-309)
                 active = [n for n in self.active_adapters if n in self.lora_A.keys()]
                 only_slot = active[0] if active else None
             skip = self.disable_adapters or (table is None and only_slot is None)
-            groups = None if skip else _self._groups_for(
-                self, only_slot if table is None else getattr(table, 'live_slots', None))
+            groups = None if skip else _groups_for(
+                _self, self, only_slot if table is None else getattr(table, 'live_slots', None))
             if groups is None:
                 return self.base_layer(x, *args, **kwargs)
             groups.sync_masters()
 
             wdtype = groups.dtype
             xw = self._cast_input_dtype(x, wdtype)
-            slot_for_dropout = only_slot if only_slot is not None else _self.loras[0].adapter_name
-            xw = self.lora_dropout[slot_for_dropout](xw)
+            xw = _slot_dropout(_self, self, only_slot, table)(xw)
             x2 = xw.reshape(-1, xw.shape[-1])
             if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
                 x2 = x2.contiguous()
             if table is None:
-                table = _self._table_for(x2.shape[0], _self.find_lora(only_slot).index, x2.device)
+                table = _table_for(_self, x2.shape[0], _self.find_lora(only_slot).index, x2.device)
             elif table.rows != x2.shape[0]:
                 raise ValueError(f'batch() was given {table.rows} rows but layer {self.layer_name} sees {x2.shape[0]}')
 
@@ -360,81 +522,16 @@ class MultiLora:
         base_layer.layer_name = name
 
     def share_inputs(self, layer_groups: Sequence[Sequence]) -> None:
-        """Declare groups of patched layers that the model calls one after the other on the same tensor
-        (``[[q_proj, k_proj, v_proj], [gate_proj, up_proj]]`` per block; modules or their names inside the
-        patched module).  Model code stays as it is: the first layer of a group that sees a new input computes
-        the outputs of the whole group through :meth:`forward_shared` and the siblings, called with the same
-        tensor, pick theirs up.  A sibling called with another tensor (or twice) simply starts a new group
-        computation, so results never depend on the call pattern; outputs nobody collects are dropped at the next
-        call.  ``share_inputs([])`` clears nothing: call :meth:`unshare_inputs` for that.
-        """
-        named = {n: sub for m in self._modules() for n, sub in m.named_modules()}
-        for group in layer_groups:
-            layers = [named[m] if isinstance(m, str) else m for m in group]
-            if not 2 <= len(layers) <= 4:
-                raise ValueError(f'a group of shared inputs has 2 to 4 layers, got {len(layers)}')
-            for layer in layers:
-                if not _is_lora_layer(layer) or not hasattr(layer, 'layer_name'):
-                    raise ValueError('share_inputs takes layers that patch() has patched')
-            if len({layer.in_features for layer in layers}) != 1:
-                raise ValueError('layers that share an input must agree in in_features')
-            state = _SharedInputGroup(layers)
-            for layer in layers:
-                layer._tk_shared_inputs = state
+        """Declare groups of patched layers that read the same tensor (see the module-level :func:`share_inputs`)."""
+        share_inputs(self, layer_groups)
 
     def unshare_inputs(self) -> None:
-        for m in self._modules():
-            for sub in m.modules():
-                if hasattr(sub, '_tk_shared_inputs'):
-                    del sub._tk_shared_inputs
+        unshare_inputs(self)
 
     def forward_shared(self, layers: Sequence, x: torch.Tensor) -> Tuple[torch.Tensor, ...]:
-        """``tuple(layer(x) for layer in layers)`` for patched layers that read the same ``x`` (q / k / v,
-        gate / up), with the LoRA terms of all of them computed by one shared call: ``x`` is read once in
-        forward, and once in backward for every layer's dA, and the gradient of ``x`` is updated once.
-
-        The reference has no per-input entry (every projection runs its own two ``F.linear`` calls, :322-326);
-        a caller opts in by routing such a group of projections through this method.  Falls back to calling
-        the layers one by one whenever one of them would not take the plain in-place path (adapters disabled,
-        a layer without a live adapter, dtype casts, non-``nn.Linear`` base layers).
-        """
-        layers = list(layers)
-        table = self._batch_table
-        only_slot = None
-        ok = 2 <= len(layers) <= 4 and x.is_cuda
-        groups_list = []
-        for layer in layers if ok else ():
-            if table is None:
-                active = [n for n in layer.active_adapters if n in layer.lora_A.keys()]
-                slot = active[0] if active else None
-                if slot is None or (only_slot is not None and slot != only_slot):
-                    ok = False
-                    break
-                only_slot = slot
-            groups = None if layer.disable_adapters else self._groups_for(
-                layer, only_slot if table is None else getattr(table, 'live_slots', None))
-            base = layer.base_layer
-            slot_for_dropout = only_slot if only_slot is not None else self.loras[0].adapter_name
-            if (groups is None or groups.dtype != x.dtype or type(base) is not torch.nn.Linear
-                    or base.weight.dtype != x.dtype or base._forward_hooks or base._forward_pre_hooks
-                    or not isinstance(layer.lora_dropout[slot_for_dropout], torch.nn.Identity)):
-                ok = False
-                break
-            groups_list.append(groups)
-        if not ok:
-            return tuple(getattr(layer, '_tk_forward_one', layer)(x) for layer in layers)
-        for groups in groups_list:
-            groups.sync_masters()
-        x2 = x.reshape(-1, x.shape[-1])
-        if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
-            x2 = x2.contiguous()
-        if table is None:
-            table = self._table_for(x2.shape[0], self.find_lora(only_slot).index, x2.device)
-        elif table.rows != x2.shape[0]:
-            raise ValueError(f'batch() was given {table.rows} rows but the shared input has {x2.shape[0]}')
-        outs = multi_lora_linear_shared(x2, [layer.base_layer.weight for layer in layers],
-                                        [layer.base_layer.bias for layer in layers], table, groups_list)
-        return tuple(y.view(*x.shape[:-1], y.shape[-1]) for y in outs)
+        """``tuple(layer(x) for layer in layers)`` with one shared LoRA call (see the module-level
+        :func:`forward_shared`)."""
+        return forward_shared(self, layers, x)
 
     def patch(self, module, target_modules='all-linear', *args, **kwargs):
         """Pre-allocate ``max_loras`` slots of rank ``max_r`` on ``module`` and patch every LoRA layer.
@@ -557,19 +654,26 @@ class MultiLora:
     # ---- adapter checkpoints in PEFT's on-disk format -----------------------------------------------------------
     _PEFT_PREFIX = 'base_model.'
 
+    @classmethod
+    def _peft_key(cls, key: str) -> str:
+        """A state-dict key under PEFT's root: ``base_model.model.<path inside the wrapped model>...``.  The in-tree
+        holder stands where ``PeftModel.base_model`` stands, so its parameter names lack only ``base_model.``; a real
+        ``PeftModel``'s names and the keys of the packed expert parameters carry the root already."""
+        return key if key.startswith(cls._PEFT_PREFIX) else cls._PEFT_PREFIX + key
+
     def save_adapter(self, tenant_adapter_name: str, checkpoint_dir: str) -> str:
         """Write the tenant's adapter as ``adapter_model.safetensors`` + ``adapter_config.json``.
 
         Same content as the reference's save for a tenant (transformers.py:1001-1033 with the state dict of
         multi_lora_transformers.py:265-267): the live ``[:r]`` blocks, slot name removed from the keys, on the
-        CPU, contiguous.  The holder returned by ``patch`` takes the place of ``PeftModel.base_model``, so keys
-        get the ``base_model.`` prefix PEFT's files carry and load with ``peft.utils.load_peft_weights``."""
+        CPU, contiguous.  Every key starts with ``base_model.model.`` like in PEFT's files (see :meth:`_peft_key`),
+        linear layers and packed expert parameters alike, and loads with ``peft.utils.load_peft_weights``."""
         import json
         import os
 
         from safetensors.torch import save_file
         slot = self.find_lora_by_tenant(tenant_adapter_name)
-        state = {self._PEFT_PREFIX + k: v.detach().to('cpu').contiguous()
+        state = {self._peft_key(k): v.detach().to('cpu').contiguous()
                  for k, v in self.get_state_dict(tenant_adapter_name).items()}
         os.makedirs(checkpoint_dir, exist_ok=True)
         save_file(state, os.path.join(checkpoint_dir, 'adapter_model.safetensors'))
@@ -595,9 +699,11 @@ class MultiLora:
 
         from safetensors.torch import load_file
         state = load_file(os.path.join(checkpoint_dir, 'adapter_model.safetensors'), device='cpu')
+        # the linear layers are looked up under the names this model's parameters have (holder-relative when the
+        # holder is the in-tree one), the packed expert parameters under PEFT's absolute names: offer both
         n = len(self._PEFT_PREFIX)
-        state = {(k[n:] if k.startswith(self._PEFT_PREFIX) else k): v for k, v in state.items()}
-        self.set_state_dict(tenant_adapter_name, state)
+        relative = {k[n:]: v for k, v in state.items() if k.startswith(self._PEFT_PREFIX)}
+        self.set_state_dict(tenant_adapter_name, {**relative, **state})
 
     def get_nb_trainable_parameters(self, tenant_adapter_name):
         """(trainable, all) parameter counts as the tenant sees them (reference :756-813)."""

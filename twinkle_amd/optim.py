@@ -13,6 +13,7 @@ Moments are fp32 whatever the parameter dtype; arithmetic is fp32.
 from __future__ import annotations
 
 import math
+import operator
 import re
 from typing import Dict, Iterable, List, Optional, Sequence
 
@@ -47,6 +48,35 @@ class _Tenant:
         self.step = 0
         self.exp_avg: List[Optional[torch.Tensor]] = [None] * len(self.params)
         self.exp_avg_sq: List[Optional[torch.Tensor]] = [None] * len(self.params)
+        # rows of the device tensor table, kept while the gradient tensors stay the same objects
+        self.grads_seen: Optional[list] = None
+        self.rows: Dict[torch.dtype, list] = {}
+        self.rows_version = 0
+
+    def table_rows(self) -> Dict[torch.dtype, list]:
+        """This tenant's rows of the tensor table per parameter dtype.  Autograd accumulates into an existing
+        ``.grad`` in place and the update kernel clears gradients without replacing them, so from the second step
+        on the same tensor objects come back and the rows (six pointers and sizes per tensor) are reused; the
+        check is one identity comparison per parameter."""
+        grads = [p.grad for p in self.params]
+        seen = self.grads_seen
+        if seen is not None and len(seen) == len(grads) and all(map(operator.is_, grads, seen)):
+            return self.rows
+        rows: Dict[torch.dtype, list] = {}
+        for i, p in enumerate(self.params):
+            g = grads[i]
+            if g is None:
+                continue  # torch optimizers skip parameters without a gradient
+            if g.dtype != p.dtype or not g.is_contiguous() or g.shape != p.shape:
+                g = grads[i] = p.grad = g.to(p.dtype).contiguous()
+            if self.exp_avg[i] is None:
+                self.exp_avg[i] = torch.zeros(p.shape, dtype=torch.float32, device=p.device)
+                self.exp_avg_sq[i] = torch.zeros(p.shape, dtype=torch.float32, device=p.device)
+            rows.setdefault(p.dtype, []).append((p.data_ptr(), g.data_ptr(), self.exp_avg[i].data_ptr(),
+                                                 self.exp_avg_sq[i].data_ptr(), p.numel(), self.index, 0))
+        self.grads_seen, self.rows = grads, rows
+        self.rows_version += 1
+        return rows
 
 
 class MultiTenantAdamW:
@@ -57,6 +87,7 @@ class MultiTenantAdamW:
         self._last_clip: Dict[torch.dtype, torch.Tensor] = {}
         self._last_tables = None
         self._table_cache: Dict[torch.dtype, tuple] = {}
+        self._with_grads: List[str] = []
 
     # ---- tenant management -------------------------------------------------------------------------------
     def add_tenant(self, name: str, params: Iterable[torch.nn.Parameter], lr: float = 1e-3, betas=(0.9, 0.999),
@@ -78,7 +109,8 @@ class MultiTenantAdamW:
         """Drop a tenant and its state (slot released); the remaining tenants keep their rows."""
         self._tenants.pop(name)
         for i, t in enumerate(self._tenants.values()):
-            t.index = i
+            if t.index != i:
+                t.index, t.grads_seen = i, None      # its rows carry the index: rebuild them
 
     def tenants(self) -> List[str]:
         return list(self._tenants)
@@ -97,7 +129,8 @@ class MultiTenantAdamW:
         names = list(names)
         tenant_rows = np.zeros(len(self._tenants), dtype=_TENANT_DTYPE)
         rows: Dict[torch.dtype, list] = {}
-        keep = []
+        versions = []
+        self._with_grads = []
         device = None
         for name in names:
             t = self._tenants[name]
@@ -109,7 +142,8 @@ class MultiTenantAdamW:
             eps = float(over['eps']) if over.get('eps') is not None else t.eps
             b1, b2 = over['betas'] if over.get('betas') is not None else t.betas
             step = t.step + 1 if advance else max(t.step, 1)
-            tokens = int(num_tokens.get(name, 1)) if isinstance(num_tokens, dict) else int(num_tokens)
+            tokens = num_tokens.get(name, 1) if isinstance(num_tokens, dict) else num_tokens
+            tokens = float(tokens)
             row = tenant_rows[t.index]
             row['lr'], row['beta1'], row['beta2'], row['eps'], row['weight_decay'] = lr, b1, b2, eps, wd
             row['one_minus_beta1'], row['one_minus_beta2'] = 1.0 - float(b1), 1.0 - float(b2)
@@ -119,31 +153,26 @@ class MultiTenantAdamW:
             row['max_grad_norm'] = max_grad_norm if max_grad_norm is not None else 0.0
             row['norm_type'] = norm_type
             row['active'] = 1
-            for i, p in enumerate(t.params):
-                g = p.grad
-                if g is None:
-                    continue  # torch optimizers skip parameters without a gradient
-                if g.dtype != p.dtype or not g.is_contiguous() or g.shape != p.shape:
-                    g = g.to(p.dtype).contiguous()
-                    p.grad = g
-                if t.exp_avg[i] is None:
-                    t.exp_avg[i] = torch.zeros(p.shape, dtype=torch.float32, device=p.device)
-                    t.exp_avg_sq[i] = torch.zeros(p.shape, dtype=torch.float32, device=p.device)
-                device = p.device
-                rows.setdefault(p.dtype, []).append((p.data_ptr(), g.data_ptr(), t.exp_avg[i].data_ptr(),
-                                                     t.exp_avg_sq[i].data_ptr(), p.numel(), t.index, 0))
-                keep.append(g)
+            mine = t.table_rows()
+            versions.append((name, t.rows_version))
+            if mine:
+                self._with_grads.append(name)
+                device = t.params[0].device
+            for dtype, lst in mine.items():
+                rows.setdefault(dtype, []).append(lst)
         out = {}
         if device is None:
             return out, tenant_rows
         tenants_dev = torch.from_numpy(tenant_rows.view(np.uint8).copy()).to(device)
-        for dtype, lst in rows.items():
+        key = tuple(versions)
+        for dtype, lists in rows.items():
             cached = self._table_cache.get(dtype)
-            if cached is None or cached[0] != lst:
-                arr = np.array(lst, dtype=_TENSOR_DTYPE)
-                cached = (lst, torch.from_numpy(arr.view(np.uint8).copy()).to(device), int(arr['numel'].max()))
+            if cached is None or cached[0] != key:
+                arr = np.array([r for lst in lists for r in lst], dtype=_TENSOR_DTYPE)
+                cached = (key, torch.from_numpy(arr.view(np.uint8).copy()).to(device), int(arr['numel'].max()),
+                          len(arr))
                 self._table_cache[dtype] = cached
-            out[dtype] = (cached[1], len(lst), cached[2], tenants_dev, keep)
+            out[dtype] = (cached[1], cached[3], cached[2], tenants_dev, None)
         return out, tenant_rows
 
     def _run_norm(self, tables, names, max_grad_norm, norm_type) -> Dict[str, torch.Tensor]:
@@ -187,8 +216,8 @@ class MultiTenantAdamW:
             _lib.check(code, 'tk_opt_adamw_step')
         self._last_tables = tables  # keeps the device tables alive until the next call (stream-ordered use)
         self._last_clip = {}
-        for name in names:
-            self._tenants[name].step += 1
+        for name in self._with_grads:      # a tenant without any gradient takes no step (torch optimizers skip
+            self._tenants[name].step += 1  # parameters whose grad is None, state and step count included)
 
     def clip_grad_norm(self, num_tokens, max_grad_norm: float = 1.0, norm_type: float = 2.0,
                        names: Optional[Sequence[str]] = None) -> Dict[str, torch.Tensor]:
@@ -230,3 +259,112 @@ class MultiTenantAdamW:
                         p.grad = None
                     else:
                         p.grad.zero_()
+
+
+def do_grad_sync(cur_step: int, gradient_accumulation_steps: int) -> bool:
+    """Whether a tenant's optimizer acts after its ``cur_step``-th backward: always without accumulation, else when
+    ``(cur_step - 1) % gradient_accumulation_steps == 0 and cur_step > 1`` (model/optimizer_group.py:56-62)."""
+    return gradient_accumulation_steps == 1 or ((cur_step - 1) % gradient_accumulation_steps == 0 and cur_step > 1)
+
+
+class BatchedStep:
+    """Loss reduction and accumulation schedule of training steps that serve many tenants per batch.
+
+    The reference runs, per tenant and one tenant at a time, ``forward`` → ``calculate_loss`` (its loss object
+    returns the loss and a token count; both are added to the tenant's running ``loss_value`` / ``num_tokens``,
+    transformers.py:617-665) → ``backward`` (``cur_step += 1``, :667-709) → ``clip_grad_and_step``, whose four parts
+    each do nothing unless the tenant's ``do_grad_sync`` holds (:732-785, :835-894).  Here one forward / backward
+    carries rows of many tenants, so this class keeps the same three per-tenant quantities (``cur_step``,
+    accumulated ``num_tokens``, gradient-accumulation setting), reduces the per-token losses of a mixed batch to one
+    loss per tenant, and hands the tenants that are due to :class:`MultiTenantAdamW` in one call.
+
+    ``reduction`` follows the reference's ``CrossEntropyLoss`` (loss/cross_entropy.py:16-33): ``'sum'`` gives each
+    tenant the sum over its unmasked tokens and counts those tokens (the gradients are divided by the count at the
+    step); anything else gives the mean over its unmasked tokens and counts 0, which the reference turns into 1 per
+    backward (:646-648).  The batch loss that is back-propagated is the sum of the tenants' losses: a tenant's
+    adapters only see its own rows, so each tenant gets exactly the gradient of its own loss.
+    """
+
+    def __init__(self, optimizer: MultiTenantAdamW, gradient_accumulation_steps=1, reduction: str = 'sum',
+                 ignore_index: int = -100):
+        self.optimizer = optimizer
+        self.gradient_accumulation_steps = gradient_accumulation_steps   # an int, or a dict per tenant
+        self.reduction = reduction
+        self.ignore_index = ignore_index
+        self.cur_step: Dict[str, int] = {}
+        self.num_tokens: Dict[str, float] = {}
+        self.last_loss: Dict[str, torch.Tensor] = {}
+        self._pending = None       # (tenant names, device token counts) of the loss not yet back-propagated
+        self._last_batch: List[str] = []
+
+    def _accumulation(self, name: str) -> int:
+        g = self.gradient_accumulation_steps
+        return int(g.get(name, 1)) if isinstance(g, dict) else int(g)
+
+    def tenant_losses(self, tenant_adapter_names: Sequence[str], row_tenant: torch.Tensor, per_token: torch.Tensor,
+                      mask: torch.Tensor):
+        """``(loss [n], counts [n])``: every tenant's reduction of ``per_token * mask`` over its own rows and the
+        number of its unmasked rows.  The sums are one small matrix product with the tenants' indicator rows, so
+        they do not depend on the order in which atomics would land."""
+        n = len(tenant_adapter_names)
+        rt = row_tenant.reshape(-1)
+        onehot = (rt[None, :] == torch.arange(n, device=rt.device)[:, None]).to(torch.float32)
+        m = mask.reshape(-1).to(torch.float32)
+        sums = onehot @ (per_token.reshape(-1).to(torch.float32) * m)
+        counts = onehot @ m
+        if self.reduction == 'sum':
+            return sums, counts.clamp(min=1)
+        return sums / counts.clamp(min=1), torch.zeros_like(counts)
+
+    def loss(self, tenant_adapter_names: Sequence[str], row_tenant: torch.Tensor, labels: torch.Tensor,
+             logps: Optional[torch.Tensor] = None, logits: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Cross entropy of a mixed batch, reduced per tenant as the reference's ``CrossEntropyLoss`` reduces one
+        tenant's batch; returns the scalar to back-propagate (the sum of the tenants' losses)."""
+        labels = labels.reshape(-1)
+        if logps is None:
+            flat = logits.reshape(-1, logits.shape[-1])
+            logps = torch.log_softmax(flat, dim=-1).gather(-1, labels.clamp(min=0).unsqueeze(-1)).squeeze(-1)
+        mask = labels != self.ignore_index
+        return self.custom_loss(tenant_adapter_names, row_tenant, -logps.reshape(-1), mask)
+
+    def custom_loss(self, tenant_adapter_names: Sequence[str], row_tenant: torch.Tensor, per_token: torch.Tensor,
+                    mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The same reduction for any per-row loss (``mask``: rows that count, default all)."""
+        if mask is None:
+            mask = torch.ones_like(per_token, dtype=torch.bool)
+        losses, counts = self.tenant_losses(tenant_adapter_names, row_tenant, per_token, mask)
+        names = list(tenant_adapter_names)
+        self.last_loss = {name: losses[i].detach() for i, name in enumerate(names)}
+        self._pending = (names, counts.detach())
+        return losses.sum()
+
+    def backward(self, loss: torch.Tensor) -> None:
+        """``loss.backward()`` and the reference's bookkeeping for every tenant of the batch: one more ``cur_step``,
+        its token count added to the running ``num_tokens`` (one copy of the counts to the host, where the
+        reference reads one ``.item()`` per tenant)."""
+        if self._pending is None:
+            raise RuntimeError('call loss() / custom_loss() before backward()')
+        names, counts = self._pending
+        loss.backward()
+        for name, c in zip(names, counts.tolist()):
+            self.cur_step[name] = self.cur_step.get(name, 0) + 1
+            self.num_tokens[name] = self.num_tokens.get(name, 0.0) + (c if c else 1.0)    # "if not counts: 1"
+        self._last_batch, self._pending = names, None
+
+    def due(self) -> List[str]:
+        """Tenants of the last batch whose optimizer acts now."""
+        return [n for n in self._last_batch if do_grad_sync(self.cur_step.get(n, 0), self._accumulation(n))]
+
+    def clip_grad_and_step(self, max_grad_norm: float = 1.0, norm_type: float = 2.0,
+                           optim_params: Optional[Dict[str, dict]] = None) -> Dict[str, torch.Tensor]:
+        """``clip_grad_norm`` → ``step`` → ``zero_grad`` for the tenants that are due, all in one launch set, each
+        with the tokens it accumulated since its last step; the others keep accumulating.  Returns the due tenants'
+        gradient norms (device scalars)."""
+        names = self.due()
+        if not names:
+            return {}
+        norms = self.optimizer.clip_grad_and_step({n: self.num_tokens[n] for n in names}, max_grad_norm, norm_type,
+                                                  optim_params, names=names)
+        for n in names:
+            self.num_tokens[n] = 0.0
+        return norms
