@@ -5,7 +5,7 @@
  * memory owned by the caller.  All work is ordered on the stream that is
  * passed in (a hipStream_t cast to void*; NULL = the null stream).  No call
  * allocates, frees, synchronises the device or keeps state between calls,
- * except where stated.  Return value: TK_OK or a negative TK_ERR_* code.
+ * except where stated (tk_lora_fwd_noalloc keeps a scratch buffer per GPU).  Return value: TK_OK or a negative TK_ERR_* code.
  *
  * Host threads: every entry point may be called from any thread.  The one
  * per-device resource the library keeps (the side stream of tk_lora_bwd and
@@ -35,7 +35,8 @@ enum {
   TK_ERR_INVALID = -1,     /* bad argument (null pointer, negative size, misaligned stride) */
   TK_ERR_WORKSPACE = -2,   /* workspace smaller than the matching *_bytes() query */
   TK_ERR_UNSUPPORTED = -3, /* shape outside what the kernels handle (see each call) */
-  TK_ERR_LAUNCH = -4       /* HIP reported an error at launch */
+  TK_ERR_LAUNCH = -4,      /* HIP reported an error at launch */
+  TK_ERR_SCRATCH = -5      /* tk_lora_fwd_noalloc: the problem needs more than TK_NOALLOC_SCRATCH_BYTES */
 };
 
 enum { TK_DTYPE_F32 = 0, TK_DTYPE_BF16 = 1 };
@@ -151,6 +152,19 @@ int64_t tk_lora_bwd_workspace_bytes(const tk_lora_desc* desc);
 /* y[row] += scale_g * (x[row] A_g^T) B_g^T in place on the base output; h_device is written. */
 int tk_lora_fwd(const tk_lora_desc* desc, const void* x_device, int64_t ldx, void* y_device, int64_t ldy,
                 void* h_device, tk_stream_t stream);
+
+/* tk_lora_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same result as tk_lora_fwd, bit for bit: y is
+ * updated in place; the shrink output, which tk_lora_fwd leaves in the caller's h buffer for the backward pass, goes
+ * to a buffer of TK_NOALLOC_SCRATCH_BYTES that the library holds in every GPU's memory from the first call on that
+ * GPU until the process ends, so there is no backward after this call (inference and evaluation passes).  The call
+ * allocates and frees nothing and does not synchronise.  TK_ERR_SCRATCH when tk_lora_h_bytes(desc) exceeds
+ * TK_NOALLOC_SCRATCH_BYTES (16 MiB: up to 16384 rows at in_features 4096 for any rank up to 64).  All calls on one
+ * GPU share that GPU's buffer and it keeps the last call's contents: two calls whose execution may overlap on one
+ * GPU (different streams, or different host threads without ordering) race; order them on one stream. */
+#define TK_NOALLOC_SCRATCH_BYTES (16 << 20)
+int tk_lora_fwd_noalloc(const tk_lora_desc* desc, const void* x_device, int64_t ldx, void* y_device, int64_t ldy,
+                        tk_stream_t stream);
 
 /* The two halves of tk_lora_fwd, for callers that time or schedule them separately:
  * tk_lora_shrink writes h = scale_g * x A_g^T (reference: multi_lora.py:322-323, the first F.linear),

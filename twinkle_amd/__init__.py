@@ -11,7 +11,7 @@ from .lora_layer import LoraConfig, LoraLinear, LoraModel, inject_adapter  # noq
 from .multi_lora import LoraTenant, MultiLora, batch, forward_shared, share_inputs, unshare_inputs  # noqa: F401
 from .integration import use_mi355x_path  # noqa: F401
 from .ops import (AdapterGroups, grouped_linear_, swiglu, lora_bwd_, lora_bwd_shared_, lora_bwd_workspace_bytes, lora_expand_,  # noqa: F401
-                  lora_fwd_, lora_fwd_shared_, lora_h_bytes, lora_shrink_, multi_lora_delta, multi_lora_delta_shared,
+                  lora_fwd_, lora_fwd_noalloc_, lora_fwd_shared_, lora_h_bytes, lora_shrink_, multi_lora_delta, multi_lora_delta_shared,
                   multi_lora_linear, multi_lora_linear_shared)
 from .optim import BatchedStep, MultiTenantAdamW, do_grad_sync, trainable_parameters  # noqa: F401
 from .segments import (SegmentTable, build_segments, flat_keys_from_topk, packed_cu_seqlens, permute,  # noqa: F401

@@ -19,6 +19,8 @@ TK_ERR_INVALID = -1
 TK_ERR_WORKSPACE = -2
 TK_ERR_UNSUPPORTED = -3
 TK_ERR_LAUNCH = -4
+TK_ERR_SCRATCH = -5
+TK_NOALLOC_SCRATCH_BYTES = 16 << 20
 TK_DTYPE_F32 = 0
 TK_DTYPE_BF16 = 1
 TK_KEY_I32 = 0
@@ -84,6 +86,7 @@ EXPORTS = {
     'tk_lora_h_bytes': (c_int64, [POINTER(LoraDesc)]),
     'tk_lora_bwd_workspace_bytes': (c_int64, [POINTER(LoraDesc)]),
     'tk_lora_fwd': (c_int32, [POINTER(LoraDesc), c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p]),
+    'tk_lora_fwd_noalloc': (c_int32, [POINTER(LoraDesc), c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     'tk_lora_shrink': (c_int32, [POINTER(LoraDesc), c_void_p, c_int64, c_void_p, c_void_p]),
     'tk_lora_expand': (c_int32, [POINTER(LoraDesc), c_void_p, c_void_p, c_int64, c_void_p]),
     'tk_lora_bwd': (c_int32, [POINTER(LoraDesc), c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64,

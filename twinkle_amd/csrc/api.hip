@@ -66,6 +66,33 @@ SideStream* side_stream() {
   return x.state == 1 ? &x : nullptr;
 }
 
+// Scratch of tk_lora_fwd_noalloc: the shrink output h and the partial sums of a split shrink, which tk_lora_fwd takes
+// from the caller.  One copy per GPU, held until the process ends.  The name below is a host-side stand-in, not a
+// device address: host code only ever uses the address that hipGetSymbolAddress returns for the current device.
+static __device__ __align__(256) unsigned char scratch[TK_NOALLOC_SCRATCH_BYTES];
+
+// Device address of `scratch` on the current device, looked up once per device.
+int scratch_address(void** out) {
+  constexpr int kMaxDevices = 64;
+  static void* ptr[kMaxDevices];
+  static bool known[kMaxDevices];
+  static std::mutex mu;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return TK_ERR_LAUNCH;
+  std::lock_guard<std::mutex> lock(mu);
+  if (!known[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return TK_ERR_LAUNCH;
+    }
+    ptr[dev] = p;
+    known[dev] = true;
+  }
+  *out = ptr[dev];
+  return TK_OK;
+}
+
 int run_pass(const PassArgs& a, const SegView& V, const SegLayout& L, int dtype, int phases, hipStream_t s) {
   if (dtype == TK_DTYPE_BF16 && !force_generic() && pass_mfma_supported(a))
     return launch_pass_mfma(a, V, L, phases, s);
@@ -94,6 +121,7 @@ const char* tk_error_string(int code) {
     case TK_ERR_WORKSPACE: return "workspace too small";
     case TK_ERR_UNSUPPORTED: return "unsupported shape";
     case TK_ERR_LAUNCH: return "HIP launch error";
+    case TK_ERR_SCRATCH: return "problem too large for the library's built-in scratch buffer";
     default: return "unknown error";
   }
 }
@@ -265,6 +293,19 @@ static int lora_pass_fwd(const tk_lora_desc* d, const void* x, int64_t ldx, void
 
 int tk_lora_fwd(const tk_lora_desc* d, const void* x, int64_t ldx, void* y, int64_t ldy, void* h,
                 tk_stream_t stream) {
+  return lora_pass_fwd(d, x, ldx, y, ldy, h, 3, stream);
+}
+
+int tk_lora_fwd_noalloc(const tk_lora_desc* d, const void* x, int64_t ldx, void* y, int64_t ldy, tk_stream_t stream) {
+  if (!desc_ok(d)) return TK_ERR_INVALID;
+  const int64_t need = tk_lora_h_bytes(d);
+  if (need < 0) return (int)need;
+  if (need > (int64_t)TK_NOALLOC_SCRATCH_BYTES) return TK_ERR_SCRATCH;
+  if (d->rows == 0 || d->max_rank == 0) return TK_OK;
+  void* h = nullptr;
+  const int rc = scratch_address(&h);
+  if (rc != TK_OK) return rc;
+  // nothing in h has to start at zero: every entry a live tile reads is written by this call first
   return lora_pass_fwd(d, x, ldx, y, ldy, h, 3, stream);
 }
 

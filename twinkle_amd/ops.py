@@ -219,6 +219,22 @@ def lora_fwd_(x: torch.Tensor, y: torch.Tensor, seg: SegmentTable, groups: Adapt
     return h
 
 
+def lora_fwd_noalloc_(x: torch.Tensor, y: torch.Tensor, seg: SegmentTable, groups: AdapterGroups,
+                      map_rows: bool = True) -> None:
+    """In place ``y += lora(x)`` like :func:`lora_fwd_`, without any device allocation (``tk_lora_fwd_noalloc``):
+    the shrink output goes to a buffer the library holds per GPU, so there is no backward after this call.
+    ``RuntimeError`` when the problem needs more than ``_lib.TK_NOALLOC_SCRATCH_BYTES``; calls that may overlap on
+    one GPU race on that buffer and must be ordered on one stream."""
+    if groups.num_groups != seg.num_groups:
+        raise ValueError(f'segment table has {seg.num_groups} groups, adapters have {groups.num_groups}')
+    _check_rows(x, 'x', seg.rows, groups.in_features, groups.dtype)
+    _check_rows(y, 'y', seg.rows, groups.out_features, groups.dtype)
+    d = _desc(seg, groups, map_rows)
+    code = _lib.load().tk_lora_fwd_noalloc(ctypes.byref(d), x.data_ptr(), x.stride(0), y.data_ptr(), y.stride(0),
+                                           _lib.stream_ptr())
+    _lib.check(code, 'tk_lora_fwd_noalloc')
+
+
 def lora_shrink_(x: torch.Tensor, seg: SegmentTable, groups: AdapterGroups, h: torch.Tensor,
                  map_rows: bool = True) -> None:
     """First half of :func:`lora_fwd_`: ``h = scale * x A^T`` (see ``tk_lora_shrink``)."""
