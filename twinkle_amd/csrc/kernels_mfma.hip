@@ -290,15 +290,22 @@ __global__ __launch_bounds__(256) void k_shrink_finish_multi(PassJobs jobs, cons
 template <int NB>
 __device__ __forceinline__ void expand_flat_body(const PassArgs& a, const bf16_t* __restrict__ hrow,
                                                  const int32_t* __restrict__ tile_group,
-                                                 const int32_t* __restrict__ slot_rows, int num_items, int block) {
+                                                 const int32_t* __restrict__ slot_rows,
+                                                 const int32_t* __restrict__ tile_walk, int num_items, int block) {
   constexpr int RP = 16 * NB;
   constexpr int NKS = (RP + 31) / 32;  // contraction steps of the MFMAs
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
   const int ngroups = a.width_dst >> 7;
   const int item = block * 4 + wave;
   if (item >= num_items) return;
-  const int tile_id = item / ngroups;
-  const int c0 = (item - tile_id * ngroups) << 7;
+  // Items are numbered tile by tile; with a walk order the n-th tile taken is tile_walk[n], the tiles sorted by their
+  // first row.  The table itself is group-major and a group's tiles are spread over all rows, so in table order the
+  // waves in flight at any moment touch rows all over the destination; in walk order they touch neighbouring rows,
+  // and the in-place update runs faster (probe: 43 us against 54 us for 256 MB touched in tiles of 32 random rows
+  // taken from windows of 512 rows instead of from all 16384).
+  const int nth = item / ngroups;
+  const int tile_id = tile_walk ? tile_walk[nth] : nth;
+  const int c0 = (item - nth * ngroups) << 7;
   const int slot0 = tile_id * kTileRows;
   // independent first loads: group id, row indices, h operand (nothing branches before the
   // destination loads are in flight)
@@ -368,16 +375,18 @@ __device__ __forceinline__ void expand_flat_body(const PassArgs& a, const bf16_t
 template <int NB>
 __global__ __launch_bounds__(256) void k_expand_mfma(PassArgs a, const bf16_t* __restrict__ hrow,
                                                      const int32_t* __restrict__ tile_group,
-                                                     const int32_t* __restrict__ slot_rows, int num_items) {
-  expand_flat_body<NB>(a, hrow, tile_group, slot_rows, num_items, blockIdx.x);
+                                                     const int32_t* __restrict__ slot_rows,
+                                                     const int32_t* __restrict__ tile_walk, int num_items) {
+  expand_flat_body<NB>(a, hrow, tile_group, slot_rows, tile_walk, num_items, blockIdx.x);
 }
 
 // Up to kMaxShared projections of padded rank 16 in one launch: blockIdx.y selects the projection; the grid
 // is as wide as the widest projection needs.
 __global__ __launch_bounds__(256) void k_expand_mfma_multi(PassJobs jobs, const int32_t* __restrict__ tile_group,
-                                                           const int32_t* __restrict__ slot_rows, int max_tiles) {
+                                                           const int32_t* __restrict__ slot_rows,
+                                                           const int32_t* __restrict__ tile_walk, int max_tiles) {
   const PassArgs& a = jobs.p[blockIdx.y];
-  expand_flat_body<1>(a, (const bf16_t*)a.hT + (int64_t)a.rpad * a.ldh, tile_group, slot_rows,
+  expand_flat_body<1>(a, (const bf16_t*)a.hT + (int64_t)a.rpad * a.ldh, tile_group, slot_rows, tile_walk,
                       max_tiles * (a.width_dst >> 7), blockIdx.x);
 }
 
@@ -1005,7 +1014,7 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
   } else {
     const int64_t items = L.max_tiles * ngroups;
     hipLaunchKernelGGL((k_expand_mfma<NB>), dim3((unsigned)ceil_div(items, 4)), dim3(256), 0, s, a, hrow,
-                       seg.tile_group, rows, (int)items);
+                       seg.tile_group, rows, seg.tile_walk(a.map_rows), (int)items);
   }
 }
 
@@ -1103,7 +1112,7 @@ int launch_pass_multi(const PassArgs* a, int n, const SegView& seg, const SegLay
                        seg.tile_group, rows);
   if (phases & 2)
     hipLaunchKernelGGL(k_expand_mfma_multi, dim3((unsigned)ceil_div(L.max_tiles * widest, 4), (unsigned)n), dim3(256), 0,
-                       s, J, seg.tile_group, rows, (int)L.max_tiles);
+                       s, J, seg.tile_group, rows, seg.tile_walk(a[0].map_rows), (int)L.max_tiles);
   return check_launch();
 }
 

@@ -210,6 +210,7 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
       valid = min(kTileRows, offs[g + 1] - pos0);       // padding is at the end of a group's last tile
     }
     V.tile_group[i] = g == groups - 1 ? -1 : g;
+    V.tile_order[i] = i;  // this path leaves the tiles in table order
     int4* sp = reinterpret_cast<int4*>(V.slot_pos + (int64_t)i * kTileRows);
 #pragma unroll
     for (int j = 0; j < kTileRows; j += 4)
@@ -299,6 +300,7 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
   __shared__ int32_t round_cnt[kKeysPerLane][kOneGroups];  // this block's keys per 64-row round
   __shared__ int32_t first[4][kOneGroups + 1];          // offsets, tile_first, chunk_first, partial_first
   __shared__ int32_t cursor[kOneGroups];                // sorted position of the block's first row of each group
+  __shared__ int32_t ahead[kKeysPerLane][kOneGroups];   // rows of each group ahead of each 64-row round of the block
   __shared__ int32_t bad_s[kOneWaves];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, blk = blockIdx.x;
   const int64_t base = (int64_t)blk * kSortBlockRows;
@@ -408,17 +410,44 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
   const int32_t* tfirst = first[1];
   const int32_t* cfirst = first[2];
   const int32_t* pfirst = first[3];
-  if (wave < kKeysPerLane && mine >= 0) {
+  // rows of every group ahead of every round: blocks before this one, then the rounds before it
+  for (int i = tid; i < kKeysPerLane * groups; i += kOneWaves * 64) {
+    const int w = i / groups, g2 = i - w * groups;
+    int n = cursor[g2] - offs[g2];
+    for (int w2 = 0; w2 < w; ++w2) n += round_cnt[w2][g2];
+    ahead[w][g2] = n;
+  }
+  __syncthreads();
+  if (wave < kKeysPerLane) {
     const int64_t f = base + wave * 64 + lane;
-    int pos = cursor[mine] + rank_in_round;
-    for (int w = 0; w < wave; ++w) pos += round_cnt[w][mine];
-    V.inv[f] = pos;
-    if (perm_out) perm_out[pos] = f;
-    // padded slot = 32 * first tile of the group + position inside the group
-    V.slot_row[tfirst[mine] * kTileRows + (pos - offs[mine])] = (int32_t)f;
+    const bool valid = mine >= 0;
+    int in_group = 0;  // position of this row inside its group
+    if (valid) {
+      in_group = ahead[wave][mine] + rank_in_round;
+      const int pos = offs[mine] + in_group;
+      V.inv[f] = pos;
+      if (perm_out) perm_out[pos] = f;
+      // padded slot = 32 * first tile of the group + position inside the group
+      V.slot_row[tfirst[mine] * kTileRows + in_group] = (int32_t)f;
+    }
+    // Sweep order of the tiles.  The row that opens a tile (position inside its group a multiple of 32) knows how
+    // many tiles open before it: for every group, the rows of that group ahead of this row, in units of 32, rounded
+    // up.  Those counts are all here (blocks and rounds before this one from the table above, lanes before this
+    // one from a ballot per group), so the tile's place in the order needs no sort and no second launch.
+    const bool opens = valid && mine != groups - 1 && (in_group & (kTileRows - 1)) == 0;
+    if (__ballot(opens)) {  // wave-uniform
+      const unsigned long long below = (1ull << lane) - 1ull;
+      int place = 0;
+      for (int g2 = 0; g2 < groups - 1; ++g2) {
+        const int n = ahead[wave][g2] + __popcll(__ballot(valid && mine == g2) & below);
+        place += (n + kTileRows - 1) / kTileRows;
+      }
+      if (opens) V.tile_order[place] = tfirst[mine] + in_group / kTileRows;
+    }
   }
 
   const int num_tiles = tfirst[groups], num_chunks = cfirst[groups];
+  const int real_tiles = tfirst[groups - 1];  // the tiles of the rows without a group come after them
   const int stride = sort_blocks * kOneWaves * 64;
   for (int i = blk * kOneWaves * 64 + tid; i < max_tiles; i += stride) {
     int g = -1, pos0 = 0, valid = 0;
@@ -428,6 +457,7 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
       valid = min(kTileRows, offs[g + 1] - pos0);      // padding is at the end of a group's last tile
     }
     V.tile_group[i] = g == groups - 1 ? -1 : g;
+    if (i >= real_tiles) V.tile_order[i] = i;  // nothing to do in these: they stay where they are, after the others
     int4* sp = reinterpret_cast<int4*>(V.slot_pos + (int64_t)i * kTileRows);
 #pragma unroll
     for (int j = 0; j < kTileRows; j += 4)

@@ -66,7 +66,7 @@ struct SegLayout {
   int64_t max_tiles, max_chunks, max_partials;
   int64_t slots;         // padded sorted length: 32 * max_tiles
   // byte offsets from the workspace base
-  int64_t off_inv, off_slot_row, off_slot_pos, off_offsets, off_tile_group, off_chunks, off_tile_first,
+  int64_t off_inv, off_slot_row, off_slot_pos, off_offsets, off_tile_group, off_tile_order, off_chunks, off_tile_first,
       off_chunk_first, off_partial_first, off_hist, off_bad, total;
 
   SegLayout(int64_t rows_, int64_t groups_) : rows(rows_), groups(groups_) {
@@ -85,6 +85,7 @@ struct SegLayout {
     off_slot_pos = o;      o += round_up(4 * slots, 256);
     off_offsets = o;       o += round_up(4 * (buckets + 1), 256);
     off_tile_group = o;    o += round_up(4 * (max_tiles + 1), 256);
+    off_tile_order = o;    o += round_up(4 * (max_tiles + 1), 256);
     off_chunks = o;        o += round_up(16 * (max_chunks + 1), 256);
     off_tile_first = o;    o += round_up(4 * (buckets + 1), 256);
     off_chunk_first = o;   o += round_up(4 * (buckets + 1), 256);
@@ -102,6 +103,11 @@ struct SegView {  // typed device pointers into a segment workspace
   int32_t* slot_pos;       // [slots]   padded slot -> sorted position, -1 in padding
   int32_t* offsets;        // [G + 2]  first sorted position of each group; [G] = first row without a group
   int32_t* tile_group;     // [max_tiles]  group of each tile, -1 for rows without a group and past the last tile
+  // [max_tiles]  the tiles in the order of their first row ("sweep order"): kernels whose work items are single tiles
+  // walk the tiles in this order when rows are reached through slot_row, so that the tiles in flight at any time
+  // cover neighbouring rows of the activation tensors whatever their groups (the table is group-major: a group's
+  // tiles are spread over all rows).  Identity where the builder does not compute it.
+  int32_t* tile_order;
   ChunkInfo* chunks;       // [max_chunks]
   int32_t* tile_first;     // [G + 2]  first tile of each group
   int32_t* chunk_first;    // [G + 2]  first chunk of each group
@@ -116,6 +122,7 @@ struct SegView {  // typed device pointers into a segment workspace
     slot_pos = (int32_t*)(b + L.off_slot_pos);
     offsets = (int32_t*)(b + L.off_offsets);
     tile_group = (int32_t*)(b + L.off_tile_group);
+    tile_order = (int32_t*)(b + L.off_tile_order);
     chunks = (ChunkInfo*)(b + L.off_chunks);
     tile_first = (int32_t*)(b + L.off_tile_first);
     chunk_first = (int32_t*)(b + L.off_chunk_first);
@@ -125,6 +132,8 @@ struct SegView {  // typed device pointers into a segment workspace
   }
   // rows of the activation tensors, by padded slot
   const int32_t* slot_table(int map_rows) const { return map_rows ? slot_row : slot_pos; }
+  // order in which single-tile work items take the tiles (null: as numbered; rows in segment order are contiguous)
+  const int32_t* tile_walk(int map_rows) const { return map_rows ? tile_order : nullptr; }
 };
 
 constexpr int32_t kSegMagic = 0x544b5347;  // "TKSG"
