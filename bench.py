@@ -156,6 +156,71 @@ def optimizer_step_bench(dev, steps=10):
                     'per tenant grad.div_, clip_grad_norm_, fused AdamW (bf16 moments), zero_grad'}
 
 
+def yardstick_bench(dev, reps=12):
+    """What this GPU sustains for the memory access patterns of the LoRA kernels, with no arithmetic
+    (`tk_yardstick`): contiguous read / copy / in-place update, and the per-tile patterns of the expand, shrink and
+    row-contraction kernels over a [16384, 4096] bf16 buffer (config 2's activations, 128 MiB), with the rows taken
+    in order, in the sweep order of config 2's segment table (tiles sorted by first row), in the table's own
+    group-major order, and fully shuffled.  Three buffers are rotated so that nothing is served from the last-level
+    cache; every pattern is launched `reps` times between two HIP events, best of four rounds."""
+    import torch
+    from twinkle_amd import _lib, build_segments, workloads
+    lib = _lib.load()
+    T, K = 16384, 4096
+    bufs = [torch.full((T, K), 1.0, dtype=torch.bfloat16, device=dev) for _ in range(3)]
+    sink = torch.zeros(1 << 16, dtype=torch.uint8, device=dev)
+    ids = workloads.zipf_ids(T, 16)
+    order = torch.sort(ids.long(), stable=True).indices                      # the table's group-major order
+    # sweep order: the same tiles of 32 rows, taken in the order of their first row
+    tiles, first = [], []
+    for g in range(16):
+        rows = order[ids[order] == g]
+        for j in range(0, rows.numel(), 32):
+            t = rows[j:j + 32]
+            if t.numel() == 32:
+                tiles.append(t)
+                first.append(int(t[0]))
+    full = torch.stack(tiles)
+    left = torch.tensor(sorted(set(range(T)) - set(full.flatten().tolist())), dtype=torch.long)
+    def pad(rows_2d):
+        flat = torch.cat([rows_2d.flatten(), left])
+        return flat[:T].to(torch.int32).to(dev)
+    perms = {
+        'rows in order': None,
+        'sweep order (tiles by first row)': pad(full[torch.tensor(first).argsort()]),
+        'group-major order (segment table)': pad(full),
+        'shuffled rows': torch.randperm(T, generator=torch.Generator().manual_seed(1)).to(torch.int32).to(dev),
+    }
+    stream = _lib.stream_ptr()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def run(kind, perm, factor):
+        best = 1e9
+        for _ in range(4):
+            e0.record()
+            for i in range(reps):
+                a = bufs[i % 3]
+                b = bufs[(i + 1) % 3] if kind == 1 else sink
+                code = lib.tk_yardstick(kind, a.data_ptr(), b.data_ptr(), perm.data_ptr() if perm is not None else None,
+                                        T, K, stream)
+                _lib.check(code, 'tk_yardstick')
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) / reps)
+        return {'us': best * 1e3, 'GBps': factor * T * K * 2 / (best * 1e-3) / 1e9}
+
+    out = {'buffer': f'[{T}, {K}] bf16 = {T * K * 2 >> 20} MiB, three rotated', 'reps': reps}
+    out['contiguous read'] = run(0, None, 1)
+    out['contiguous copy (read + write)'] = run(1, None, 2)
+    out['contiguous in-place update'] = run(2, None, 2)
+    out['contiguous in-place update, non-temporal'] = run(3, None, 2)
+    for kind, name, factor in ((4, 'expand pattern, read', 1), (5, 'expand pattern, in-place non-temporal', 2),
+                               (6, 'shrink pattern, read', 1), (7, 'row-contraction pattern, read', 1)):
+        for pname, perm in perms.items():
+            out[f'{name}: {pname}'] = run(kind, perm, factor)
+    return out
+
+
 def shared_qkv_bench(dev, steps=20, calibrate_copy=False):
     """q / k / v of one attention block (4096 -> 4096, 1024, 1024; config 2's tokens, adapters and ids):
     one shared call against one call per projection, forward + backward, segment table built once."""
@@ -517,6 +582,8 @@ def main():
     ap.add_argument('--layers', type=int, default=32)
     ap.add_argument('--moe-experts', action='store_true',
                     help='run only the expert block of BASELINE config 4: per-expert loop against the grouped GEMMs')
+    ap.add_argument('--yardstick', action='store_true',
+                    help='run only the memory yardsticks: what the GPU sustains for the kernels\' access patterns')
     ap.add_argument('--calibrate-copy', action='store_true',
                     help='also run five plain 128 MiB device copies (a known-size kernel to scale rocprofv3 --pmc '
                          'FETCH_SIZE / WRITE_SIZE readings by)')
@@ -536,6 +603,9 @@ def main():
     dev = torch.device('cuda:0')
     if args.optimizer_only:
         print(json.dumps({'optimizer_step': optimizer_step_bench(dev)}))
+        return
+    if args.yardstick:
+        print(json.dumps({'yardstick': yardstick_bench(dev)}, indent=1))
         return
     if args.stack_cfg5:
         print(json.dumps({'cfg5_stack': cfg5_stack_bench(dev, layers=args.layers)}))

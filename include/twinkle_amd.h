@@ -307,6 +307,27 @@ int tk_swiglu_bwd(const void* gate_up_device, int64_t ld_gate_up, const void* dh
                   void* dgate_up_device, int64_t ld_dgate_up, int64_t rows, int32_t inter, int32_t dtype,
                   tk_stream_t stream);
 
+/* ---- memory yardsticks ---------------------------------------------------------------------------------------
+ *
+ * One launch of a kernel that only moves memory in the access pattern of one of the kernels above, over a
+ * [rows][width] bf16 buffer `a` (`b`: the destination of TK_YS_COPY, a sink of at least 4 KB otherwise):
+ * what bench.py --yardstick times to say how fast this GPU runs each pattern with no arithmetic at all.
+ * `row_of` (device, [rows] int32, optional) is a permutation of the rows, taken 32 entries per tile like the
+ * segment table's slots; NULL takes the rows in order.  rows and width multiples of 512.  A measurement aid:
+ * no counterpart in the reference. */
+enum {
+  TK_YS_READ = 0,        /* contiguous read */
+  TK_YS_COPY = 1,        /* contiguous a -> b */
+  TK_YS_RMW = 2,         /* contiguous in-place update */
+  TK_YS_RMW_NT = 3,      /* ... with non-temporal accesses */
+  TK_YS_TILE_READ = 4,   /* (tile, 128 columns) per wave, read: the expand kernel's loads */
+  TK_YS_TILE_RMW_NT = 5, /* (tile, 128 columns) per wave, in-place update, non-temporal: the expand kernel */
+  TK_YS_SHRINK_READ = 6, /* (two tiles, 512 columns) per wave in MFMA operand order: the shrink kernel's loads */
+  TK_YS_WALK_READ = 7    /* one wave walks 16 tiles for 128 columns: the row-contraction kernels' loads */
+};
+int tk_yardstick(int32_t kind, void* a_device, void* b_device, const int32_t* row_of_device, int64_t rows,
+                 int32_t width, tk_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

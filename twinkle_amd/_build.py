@@ -7,7 +7,7 @@ import subprocess
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'csrc')
 INCLUDE = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), 'include')
 LIB_PATH = os.path.join(CSRC, 'libtwinkle_amd.so')
-SOURCES = ['api.hip', 'kernels_segments.hip', 'kernels_generic.hip', 'kernels_mfma.hip', 'kernels_shared.hip', 'kernels_optim.hip', 'kernels_grouped.hip', 'kernels_act.hip']
+SOURCES = ['api.hip', 'kernels_segments.hip', 'kernels_generic.hip', 'kernels_mfma.hip', 'kernels_shared.hip', 'kernels_optim.hip', 'kernels_grouped.hip', 'kernels_act.hip', 'kernels_yardstick.hip']
 
 # -packed-fp32-ops is switched off on purpose: the compiler must not form packed fp32 VALU ops.
 HIPCC_FLAGS = [

@@ -101,6 +101,7 @@ EXPORTS = {
     'tk_swiglu_fwd': (c_int32, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p]),
     'tk_swiglu_bwd': (c_int32, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int32, c_int32,
                                 c_void_p]),
+    'tk_yardstick': (c_int32, [c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_void_p]),
     'tk_opt_workspace_bytes': (c_int64, [c_int32, c_int64]),
     'tk_opt_grad_norm': (c_int32, [c_void_p, c_int32, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p,
                                    c_int64, c_void_p]),
