@@ -293,3 +293,26 @@ def test_batched_steps_with_gradient_accumulation_equal_each_tenant_alone(dev):
         assert did == [i for i in range(steps) if n in stepped[i]], (n, did, stepped)
         for k, p in params.items():
             assert max_rel_err(got[n][k], p.detach()) < 5e-5, (n, k)
+
+
+@pytest.mark.parametrize('dtype,tol', [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+def test_several_active_adapters_on_one_layer_add_up(dev, dtype, tol):
+    """The reference's patched forward loops over ``active_adapters`` and adds every adapter's term
+    (multi_lora.py:306-326); with two active slots the layer gives base + term(alice) + term(bob)."""
+    ml, model, cfgs = _setup(dev, dtype)
+    slot = {n: ml.find_lora_by_tenant(n).adapter_name for n in cfgs}
+    layer = model.model.q_proj
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(70, 128, generator=g).to(dtype)
+    layer.set_adapter([slot['alice'], slot['bob']])
+    y = layer(x.to(dev))
+    want = layer.base_layer(x.to(dev)).double().cpu()
+    for n in ('alice', 'bob'):
+        cfg = cfgs[n]
+        want = oracle.lora_linear_forward(x.double(), want, layer.lora_A[slot[n]].weight.detach().double().cpu(),
+                                          layer.lora_B[slot[n]].weight.detach().double().cpu(), cfg.r,
+                                          oracle.lora_scaling(cfg.lora_alpha, cfg.r, cfg.use_rslora))
+    assert max_rel_err(y, want) < tol
+    layer.set_adapter([slot['alice']])
+    one = layer(x.to(dev))
+    assert (y.float() - one.float()).abs().max() > 0

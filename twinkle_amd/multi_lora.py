@@ -477,17 +477,31 @@ class MultiLora:
 
         def _forward_one(self, x: torch.Tensor, *args, **kwargs) -> torch.Tensor:
             self._check_forward_args(x, *args, **kwargs)
+            if _path_state(_self).batch_table is None and not self.disable_adapters:
+                # the reference adds the term of every active adapter the layer has, one after the other
+                # (:306-326); one is the usual case, the others are added onto its result the same way
+                active = [n for n in self.active_adapters if n in self.lora_A.keys()]
+                if len(active) > 1:
+                    out = _with_slot(self, x, active[0], None, args, kwargs)
+                    for slot in active[1:]:
+                        out = _with_slot(self, x, slot, out, (), {})
+                    return out
+            return _with_slot(self, x, None, None, args, kwargs)
+
+        def _with_slot(self, x, forced_slot, onto, args, kwargs):
+            """The layer's output with one adapter's term (``forced_slot``; ``None``: the open batch, or the first
+            active adapter) added onto ``onto`` (``None``: onto the base layer's output)."""
             table = _path_state(_self).batch_table
             only_slot = None
             if table is None:
                 # one adapter per call: the active slot, if this layer has it (reference :306-309)
                 active = [n for n in self.active_adapters if n in self.lora_A.keys()]
-                only_slot = active[0] if active else None
+                only_slot = forced_slot if forced_slot is not None else (active[0] if active else None)
             skip = self.disable_adapters or (table is None and only_slot is None)
             groups = None if skip else _groups_for(
                 _self, self, only_slot if table is None else getattr(table, 'live_slots', None))
             if groups is None:
-                return self.base_layer(x, *args, **kwargs)
+                return self.base_layer(x, *args, **kwargs) if onto is None else onto
             groups.sync_masters()
 
             wdtype = groups.dtype
@@ -502,13 +516,14 @@ class MultiLora:
                 raise ValueError(f'batch() was given {table.rows} rows but layer {self.layer_name} sees {x2.shape[0]}')
 
             base = self.base_layer
-            plain = (type(base) is torch.nn.Linear and not args and not kwargs and xw is x and x.dtype == wdtype
-                     and base.weight.dtype == wdtype and not base._forward_hooks and not base._forward_pre_hooks)
+            plain = (onto is None and type(base) is torch.nn.Linear and not args and not kwargs and xw is x
+                     and x.dtype == wdtype and base.weight.dtype == wdtype and not base._forward_hooks
+                     and not base._forward_pre_hooks)
             if plain:
                 y2 = multi_lora_linear(x2, base.weight, base.bias, table, groups)
                 return y2.reshape(*x.shape[:-1], y2.shape[-1])
 
-            result = base(x, *args, **kwargs)
+            result = base(x, *args, **kwargs) if onto is None else onto
             result_dtype = result.dtype
             if result_dtype == wdtype and result.is_contiguous():
                 y2 = multi_lora_delta(x2, result.view(-1, result.shape[-1]), table, groups)
