@@ -238,10 +238,13 @@ int tk_opt_adamw_step(const tk_opt_tensor* tensors_device, int32_t num_tensors, 
 /* ---------------------------------------------------------------------------
  * Projections that share their input (q / k / v, gate / up): one call for all of them, with the shared
  * tensors crossing memory once.  Same results contract as one tk_lora_fwd / tk_lora_bwd per projection, which
- * is also what runs when the shapes are outside the shared kernels (bf16, every max_rank <= 16, 2..4
- * projections, in_features a multiple of 1024 .. see the single-projection fast-path limits): forward reads
- * x once instead of once per projection; backward reads x once for all dA and updates dx once with the sum
- * over the projections (one rounding instead of one per projection).  The descriptors must agree in rows,
+ * is also what runs when the shapes are outside the shared kernels (bf16, 2..4 projections whose max_rank
+ * round up to the same padded rank 16, 32 or 64, in_features a multiple of 1024 .. see the single-projection
+ * fast-path limits): forward reads x once instead of once per projection; backward reads x once for all dA
+ * and updates dx once with the sum over the projections (one rounding instead of one per projection).  At
+ * padded rank 16 the reads of x are shared inside one kernel; at 32 and 64 the projections' blocks that need
+ * the same piece of x are launched side by side on one XCD, so the piece comes from memory once and from that
+ * L2 afterwards.  The descriptors must agree in rows,
  * in_features, num_groups, dtype, map_rows and seg_ws.  Arrays indexed by projection are host arrays.
  * No counterpart in the reference, which runs every projection's two F.linear calls on its own
  * (multi_lora.py:322-326).

@@ -17,9 +17,10 @@ pytestmark = pytest.mark.gpu
 def _projections(k, outs, n, max_r, ranks_per_proj, seed, dtype, dev):
     g = torch.Generator().manual_seed(seed)
     projs = []
-    for m, ranks in zip(outs, ranks_per_proj):
-        a = [((torch.rand(max_r, k, generator=g) * 2 - 1) / k**0.5).to(dtype) for _ in range(n)]
-        b = [(torch.randn(m, max_r, generator=g) * 0.05).to(dtype) for _ in range(n)]
+    max_rs = max_r if isinstance(max_r, tuple) else (max_r,) * len(outs)
+    for m, ranks, mr in zip(outs, ranks_per_proj, max_rs):
+        a = [((torch.rand(mr, k, generator=g) * 2 - 1) / k**0.5).to(dtype) for _ in range(n)]
+        b = [(torch.randn(m, mr, generator=g) * 0.05).to(dtype) for _ in range(n)]
         scales = [2.0 if i % 2 == 0 else 0.5 for i in range(n)]
         projs.append((a, b, list(ranks), scales))
     return projs
@@ -89,6 +90,24 @@ def test_shared_matches_separate_calls_bf16(dev, outs, ranks_per_proj):
     _compare(dev, torch.bfloat16, 777, 2048, outs, 5, 16, ranks_per_proj)
 
 
+@pytest.mark.parametrize('max_r,outs,ranks_per_proj', [
+    (32, (1024, 512), ((32, 17, 4, 32, 1), (32, 32, 2, 24, 16))),                              # gate / up
+    (32, (1024, 512, 512), ((32, 8, 4, 16, 1), (24, 24, 24, 24, 24), (32, 0, 3, 16, 5))),       # q / k / v, a dead adapter
+    (32, (384, 640), ((32, 8, 4, 16, 1), (17, 32, 3, 16, 5))),                                  # widths off the fused dy pass
+    (64, (1024, 512), ((64, 33, 4, 16, 1), (64, 64, 2, 48, 16))),
+    (64, (512, 512, 1024, 512), ((64,) * 5, (33,) * 5, (1, 20, 33, 48, 64), (0, 0, 64, 40, 0))),
+])
+def test_shared_matches_separate_calls_above_rank_16(dev, max_r, outs, ranks_per_proj):
+    """Padded rank 32 and 64: one shrink launch for all projections, one dX read-modify-write, one dA launch."""
+    _compare(dev, torch.bfloat16, 777, 2048, outs, 5, max_r, ranks_per_proj)
+
+
+def test_shared_rank_64_attention_shape(dev):
+    """q / k / v at rank 64: 4096 -> 4096, 1024, 1024 on 2048 tokens of 8 adapters, one of them without rows."""
+    ranks = [(64, 64, 48, 64, 33, 64, 64, 64)] * 3
+    _compare(dev, torch.bfloat16, 2048, 4096, (4096, 1024, 1024), 8, 64, ranks, seed=11)
+
+
 def test_shared_llama_qkv_shape(dev):
     """q / k / v of a grouped-query attention block: 4096 -> 4096, 1024, 1024 on 4096 tokens of 16 adapters."""
     _compare(dev, torch.bfloat16, 4096, 4096, (4096, 1024, 1024), 16, 16, [(16,) * 16, (8,) * 16, (16,) * 16], seed=3)
@@ -96,13 +115,17 @@ def test_shared_llama_qkv_shape(dev):
 
 @pytest.mark.parametrize('dtype,k,outs,max_r', [
     (torch.float32, 256, (128, 64), 8),         # fp32: one call per projection inside the library
-    (torch.bfloat16, 2048, (1024, 512), 32),    # rank above 16
     (torch.bfloat16, 200, (96, 40), 8),         # shapes outside the MFMA kernels
     (torch.bfloat16, 2048, (1024,), 16),        # a single projection
 ])
 def test_shared_falls_back_to_one_call_per_projection(dev, dtype, k, outs, max_r):
     ranks = [(max_r, max_r // 2, 1)] * len(outs)
     _compare(dev, dtype, 300, k, outs, 3, max_r, ranks, seed=5, exact=False)
+
+
+def test_shared_projections_of_different_padded_rank(dev):
+    """One projection of rank 16, one of rank 64: no common kernel family, so one call per projection."""
+    _compare(dev, torch.bfloat16, 300, 2048, (1024, 512), 3, (16, 64), [(16, 8, 1), (64, 32, 1)], seed=6, exact=True)
 
 
 def test_shared_argument_errors(dev):

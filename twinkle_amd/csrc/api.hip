@@ -512,6 +512,17 @@ static bool shared_fast_path(const tk_lora_desc* const* descs, int32_t n) {
   return shrink_kslices(descs[0]->in_features, 16) > 1;
 }
 
+// ... or the multi-projection launches of the kernels of padded rank 32 / 64: bf16, 2..4 projections whose padded
+// ranks agree (and exceed 16)
+static bool shared_wide_path(const tk_lora_desc* const* descs, int32_t n) {
+  if (n < 2 || descs[0]->dtype != TK_DTYPE_BF16 || force_generic()) return false;
+  const int rpad = rank_pad(descs[0]->max_rank);
+  if (rpad != 32 && rpad != 64) return false;
+  for (int p = 0; p < n; ++p)
+    if (descs[p]->max_rank < 1 || rank_pad(descs[p]->max_rank) != rpad) return false;
+  return true;
+}
+
 int tk_lora_fwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* x, int64_t ldx, void* const* y,
                        const int64_t* ldy, void* const* h, tk_stream_t stream) {
   if (!shared_descs_ok(descs, n) || !y || !ldy || !h) return TK_ERR_INVALID;
@@ -531,6 +542,15 @@ int tk_lora_fwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* 
   }
   int rc;
   if (!fast) {
+    bool wide = shared_wide_path(descs, n);
+    for (int p = 0; p < n && wide; ++p) wide = pass_mfma_supported(a[p]) && a[p].kslices == a[0].kslices;
+    if (wide) {
+      // every projection's shrink in one launch, the pieces of x crossing memory once; then y_p += h_p B_p^T
+      if ((rc = launch_shrink_multi(a, n, V, L, s)) != TK_OK) return rc;
+      for (int p = 0; p < n; ++p)
+        if ((rc = launch_pass_mfma(a[p], V, L, 2, s)) != TK_OK) return rc;
+      return TK_OK;
+    }
     for (int p = 0; p < n; ++p)
       if ((rc = tk_lora_fwd(descs[p], x, ldx, y[p], ldy[p], h[p], stream)) != TK_OK) return rc;
     return TK_OK;
@@ -576,6 +596,47 @@ int tk_lora_bwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* 
   }
   int rc;
   if (!fast) {
+    bool wide = shared_wide_path(descs, n);
+    for (int p = 0; p < n && wide; ++p)
+      wide = pass_mfma_supported(plan[p].a) && wgrad_mfma_supported(plan[p].ga) && wgrad_mfma_supported(plan[p].gb) &&
+             descs[p]->out_features % 8 == 0;
+    if (wide) {
+      // Per projection what only it touches (its dy: the transposed weight copies, dh_p = s dy_p B_p and dB_p), then
+      // once for all of them what touches the shared tensors: dx += sum_p dh_p A_p in one read-modify-write, and
+      // every dA_p = dh_p^T x from launches that fetch each tile of x once.
+      const int rpad = plan[0].a.rpad;
+      SharedExpandArgs ea{};
+      ea.dst = dx;  ea.ld_dst = lddx;  ea.width_dst = d0->in_features;  ea.map_rows = d0->map_rows;  ea.nproj = n;
+      SharedWgradArgs wa{};
+      wa.nproj = n;
+      WgradArgs red[2 * TK_MAX_SHARED] = {};
+      for (int p = 0; p < n; ++p) {
+        BwdPlan& P = plan[p];
+        const int fused_ks = fused_dy_kslices(descs[p]->out_features, rpad);
+        if (fused_ks && dy_fused_supported(P.gb, fused_ks)) {  // one pass over dy_p: dB_p, the slices of dh_p, A_p^T
+          P.a.kslices = fused_ks;
+          WgradArgs gb = P.gb;
+          gb.tr = P.tr;
+          gb.tr.bT = nullptr;
+          if ((rc = launch_dy_fused(gb, descs[p]->lora_B, descs[p]->ldb, P.a.hpart, fused_ks, V, L, s)) != TK_OK)
+            return rc;
+          if ((rc = launch_pass_mfma(P.a, V, L, 4, s)) != TK_OK) return rc;
+        } else {
+          if ((rc = launch_transpose_job(P.tr, descs[p]->rank, rpad, s)) != TK_OK) return rc;
+          if ((rc = launch_pass_mfma(P.a, V, L, 1, s)) != TK_OK) return rc;
+          if ((rc = launch_wgrad_mfma(P.gb, V, L, s)) != TK_OK) return rc;
+        }
+        ea.hrow[p] = (const char*)P.dh + (int64_t)rpad * P.a.ldh * 2;  // slot-major half of the dh buffer (bf16)
+        ea.aT[p] = P.aT;
+        ea.rank[p] = descs[p]->rank;
+        wa.w[p] = P.ga;
+        red[2 * p] = P.ga;
+        red[2 * p + 1] = P.gb;
+      }
+      if ((rc = launch_expand_shared_wide(ea, rpad, V, L, s)) != TK_OK) return rc;
+      if ((rc = launch_wgrad_coop_multi(wa, V, L, s)) != TK_OK) return rc;
+      return launch_wgrad_reduce_multi(red, 2 * n, V, L, s);
+    }
     for (int p = 0; p < n; ++p)
       if ((rc = tk_lora_bwd(descs[p], dy[p], lddy[p], x, ldx, h[p], dx, lddx, grad_A[p], grad_B[p], accumulate, ws[p],
                             ws_bytes[p], stream)) != TK_OK)

@@ -253,11 +253,13 @@ __global__ __launch_bounds__(256) void k_wgrad_reduce(WgradArgs a0, WgradArgs a1
   wgrad_reduce_body<T>(second ? a1 : a0, 8 * (second ? blockIdx.z - zsets : blockIdx.z), chunk_first, partial_first);
 }
 
-// Any number of argument sets of padded rank 16 (dA and dB of several projections) in one launch:
-// blockIdx.z = 2 * set + octet of rank indices.
-__global__ __launch_bounds__(256) void k_wgrad_reduce_multi(WgradReduceJobs jobs, const int32_t* __restrict__ chunk_first,
+// Any number of argument sets of one padded rank (dA and dB of several projections) in one launch:
+// blockIdx.z = octets * set + octet of rank indices, octets = rpad / 8.
+__global__ __launch_bounds__(256) void k_wgrad_reduce_multi(WgradReduceJobs jobs, int octets,
+                                                            const int32_t* __restrict__ chunk_first,
                                                             const int32_t* __restrict__ partial_first) {
-  wgrad_reduce_body<bf16_t>(jobs.a[blockIdx.z >> 1], 8 * (blockIdx.z & 1), chunk_first, partial_first);
+  const int set = blockIdx.z / octets;
+  wgrad_reduce_body<bf16_t>(jobs.a[set], 8 * (blockIdx.z - set * octets), chunk_first, partial_first);
 }
 
 // bT_g[n][m] = B_g[m][n], aT_g[k][n] = A_g[n][k]; zero for n >= rank[g].
@@ -340,8 +342,9 @@ int launch_wgrad_reduce_multi(const WgradArgs* sets, int n, const SegView& seg, 
     J.a[i] = sets[i];
     width = std::max(width, sets[i].width);
   }
-  const dim3 grid((unsigned)L.groups, (unsigned)ceil_div(width, 256), (unsigned)(2 * n));
-  hipLaunchKernelGGL(k_wgrad_reduce_multi, grid, dim3(256), 0, s, J, seg.chunk_first, seg.partial_first);
+  const int octets = sets[0].rpad / 8;  // the sets share their padded rank
+  const dim3 grid((unsigned)L.groups, (unsigned)ceil_div(width, 256), (unsigned)(octets * n));
+  hipLaunchKernelGGL(k_wgrad_reduce_multi, grid, dim3(256), 0, s, J, octets, seg.chunk_first, seg.partial_first);
   return check_launch();
 }
 

@@ -193,11 +193,11 @@ __device__ inline void shrink_tiles(const PassArgs& a, bf16_t* __restrict__ hrow
 }
 
 template <int NB, int NW>
-__global__ __launch_bounds__(NW * 64) void k_shrink_pair(PassArgs a, bf16_t* __restrict__ hrow,
-                                                         const int32_t* __restrict__ tile_group,
-                                                         const int32_t* __restrict__ slot_rows, int max_tiles) {
+__device__ __forceinline__ void shrink_pair_body(const PassArgs& a, bf16_t* __restrict__ hrow,
+                                                 const int32_t* __restrict__ tile_group,
+                                                 const int32_t* __restrict__ slot_rows, int max_tiles, int item) {
   __shared__ float part[NW][kTileRows][16 * NB + 1];
-  const int pair = blockIdx.x / a.kslices, ks = blockIdx.x - pair * a.kslices;
+  const int pair = item / a.kslices, ks = item - pair * a.kslices;
   const int t0 = 2 * pair, t1 = t0 + 1;
   const int g0 = tile_group[t0];
   const int g1 = t1 < max_tiles ? tile_group[t1] : -1;
@@ -214,6 +214,37 @@ __global__ __launch_bounds__(NW * 64) void k_shrink_pair(PassArgs a, bf16_t* __r
     const int tiles[1] = {t1};
     shrink_tiles<NB, NW, 1>(a, hrow, slot_rows, tiles, g1, ks, part);
   }
+}
+
+template <int NB, int NW>
+__global__ __launch_bounds__(NW * 64) void k_shrink_pair(PassArgs a, bf16_t* __restrict__ hrow,
+                                                         const int32_t* __restrict__ tile_group,
+                                                         const int32_t* __restrict__ slot_rows, int max_tiles) {
+  shrink_pair_body<NB, NW>(a, hrow, tile_group, slot_rows, max_tiles, blockIdx.x);
+}
+
+// Work item `item` of projection p out of nproj that read the same rows: blocks go to the eight XCDs (each with an
+// L2 of its own) round-robin by block number, so the items are numbered in runs of eight per projection: blocks
+// 8 (g nproj + p) + j, j < 8, are items 8 g + j of projection p.  The nproj blocks that read the same piece of the
+// source then lie eight apart, run on the same XCD at about the same time, and the piece comes from memory once and
+// from that L2 afterwards.
+__device__ inline void shared_source_item(int block, int nproj, int& p, int& item) {
+  const int run = block >> 3;
+  p = run % nproj;
+  item = ((run / nproj) << 3) + (block & 7);
+}
+
+// The shrink of up to kMaxShared projections of one padded rank that read the same source, in one launch: the
+// bodies of k_shrink_pair, every piece of the source crossing memory once (see shared_source_item).
+template <int NB, int NW>
+__global__ __launch_bounds__(NW * 64) void k_shrink_pair_multi(PassJobs jobs, int nproj, int items,
+                                                               const int32_t* __restrict__ tile_group,
+                                                               const int32_t* __restrict__ slot_rows, int max_tiles) {
+  int p, item;
+  shared_source_item(blockIdx.x, nproj, p, item);
+  if (item >= items) return;
+  const PassArgs& a = jobs.p[p];
+  shrink_pair_body<NB, NW>(a, (bf16_t*)a.hT + (int64_t)a.rpad * a.ldh, tile_group, slot_rows, max_tiles, item);
 }
 
 // Adds the slices of a split shrink in slice order and writes h (one block per tile).
@@ -511,40 +542,95 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
   }
 }
 
-// Transposed weight copies (see TransposeJob): a thread writes 8 consecutive outputs with one 16-byte
-// store and gathers them with 8 element loads (the weights are L2 resident and small).
+// 8 x 8 block of bf16 transposed inside a lane: in[i] holds 8 consecutive elements of row i, out[q] the 8 rows'
+// q-th elements (v_perm_b32 picks the low or the high halves of a register pair).
+__device__ inline void transpose8x8(const uint4 (&in)[8], uint4 (&out)[8]) {
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const int d = q >> 1;
+    const uint32_t sel = (q & 1) ? 0x07060302u : 0x05040100u;
+    uint32_t e[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t w[4] = {in[i].x, in[i].y, in[i].z, in[i].w};
+      e[i] = w[d];
+    }
+    out[q].x = __builtin_amdgcn_perm(e[1], e[0], sel);
+    out[q].y = __builtin_amdgcn_perm(e[3], e[2], sel);
+    out[q].z = __builtin_amdgcn_perm(e[5], e[4], sel);
+    out[q].w = __builtin_amdgcn_perm(e[7], e[6], sel);
+  }
+}
+
+// Transposed weight copies (see TransposeJob).  A work unit is an 8 x 8 block: eight 16-byte loads along the
+// source's contiguous dimension, a transpose inside the lane, eight 16-byte stores along the copy's contiguous
+// dimension; consecutive threads take neighbouring blocks so that a wave's accesses cover whole rows (128 bytes and
+// more).  A source whose row stride or address rules out 16-byte loads is gathered element by element.
 __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_t* __restrict__ rank, int rpad,
                                              int64_t thread, int64_t threads) {
-  const int m8 = t.out_features >> 3, n8 = rpad >> 3;
-  const int64_t units_b = t.bT ? (int64_t)t.groups * m8 * rpad : 0;  // (g, m-octet, n), n fastest
-  const int64_t units_a = (int64_t)t.groups * n8 * t.in_features;  // (g, n-octet, k), k fastest
+  const int m8 = t.out_features >> 3, n8 = rpad >> 3, k8 = t.in_features >> 3;
+  const int64_t units_b = t.bT ? (int64_t)t.groups * m8 * n8 : 0;  // (g, m-octet, n-octet), n-octet fastest
+  const int64_t units_a = (int64_t)t.groups * n8 * k8;              // (g, n-octet, k-octet), k-octet fastest
   for (int64_t u = thread; u < units_b + units_a; u += threads) {
-    uint32_t e[8];
-    bf16_t* out;
+    uint4 in[8], out[8];
     if (u < units_b) {
-      const int n = (int)(u % rpad);
-      const int64_t q = u / rpad;
+      // bT[g][n][m] = B_g[m][n]: rows m of B hold the rank index contiguously
+      const int no = (int)(u % n8);
+      const int64_t q = u / n8;
       const int mo = (int)(q % m8), g = (int)(q / m8);
-      const bf16_t* B = (const bf16_t*)t.lora_B[g] + (int64_t)(8 * mo) * t.ldb + n;
-      const bool live = n < rank[g];
-      if (!live && t.skip_dead) continue;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) e[i] = live ? B[(int64_t)i * t.ldb] : 0;
-      out = (bf16_t*)t.bT + ((int64_t)g * rpad + n) * t.out_features + 8 * mo;
-    } else {
-      const int64_t v = u - units_b;
-      const int kd = (int)(v % t.in_features);  // row of aT; which column of A lies there:
-      const int k = t.swizzle_a ? ((kd & ~127) | ((kd & 15) << 3) | ((kd >> 4) & 7)) : kd;
-      const int64_t q = v / t.in_features;
-      const int no = (int)(q % n8), g = (int)(q / n8);
-      const bf16_t* A = (const bf16_t*)t.lora_A[g] + (int64_t)(8 * no) * t.lda + k;
-      const int r = rank[g];
+      const int r = min(rank[g], rpad);
       if (8 * no >= r && t.skip_dead) continue;
+      const bf16_t* B = (const bf16_t*)t.lora_B[g] + (int64_t)(8 * mo) * t.ldb + 8 * no;
+      const bool vec = (t.ldb & 7) == 0 && 8 * no + 8 <= t.ldb && (reinterpret_cast<uintptr_t>(t.lora_B[g]) & 15u) == 0;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) e[i] = 8 * no + i < r ? A[(int64_t)i * t.lda] : 0;
-      out = (bf16_t*)t.aT + ((int64_t)g * t.in_features + kd) * rpad + 8 * no;
+      for (int i = 0; i < 8; ++i) {
+        if (8 * no >= r) {
+          in[i] = zero4();
+        } else if (vec) {
+          in[i] = keep_first(ld16(B + (int64_t)i * t.ldb), r - 8 * no);
+        } else {
+          uint32_t e[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) e[j] = 8 * no + j < r ? B[(int64_t)i * t.ldb + j] : 0;
+          in[i] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
+        }
+      }
+      transpose8x8(in, out);
+      bf16_t* o = (bf16_t*)t.bT + ((int64_t)g * rpad + 8 * no) * t.out_features + 8 * mo;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (8 * no + j < r || !t.skip_dead) st16(o + (int64_t)j * t.out_features, out[j]);
+    } else {
+      // aT[g][k][n] = A_g[n][k]: rows n of A hold the input features contiguously
+      const int64_t v = u - units_b;
+      const int ko = (int)(v % k8);
+      const int64_t q = v / k8;
+      const int no = (int)(q % n8), g = (int)(q / n8);
+      const int r = min(rank[g], rpad);
+      if (8 * no >= r && t.skip_dead) continue;
+      const bf16_t* A = (const bf16_t*)t.lora_A[g] + (int64_t)(8 * no) * t.lda + 8 * ko;
+      const bool vec = (t.lda & 7) == 0 && (reinterpret_cast<uintptr_t>(t.lora_A[g]) & 15u) == 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (8 * no + i >= r) {
+          in[i] = zero4();
+        } else if (vec) {
+          in[i] = ld16(A + (int64_t)i * t.lda);
+        } else {
+          uint32_t e[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) e[j] = A[(int64_t)i * t.lda + j];
+          in[i] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
+        }
+      }
+      transpose8x8(in, out);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int k = 8 * ko + j;  // column of A; which row of aT holds it:
+        const int kd = t.swizzle_a ? ((k & ~127) | ((k & 7) << 4) | ((k >> 3) & 15)) : k;
+        st16((bf16_t*)t.aT + ((int64_t)g * t.in_features + kd) * rpad + 8 * no, out[j]);
+      }
     }
-    st16(out, make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)));
   }
 }
 
@@ -674,8 +760,8 @@ __global__ __launch_bounds__(64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo*
 // barrier that every reader of it has passed.
 // ---------------------------------------------------------------------------
 template <int NB, int S>
-__global__ __launch_bounds__(128) void k_wgrad_coop(WgradArgs a, const ChunkInfo* __restrict__ chunks,
-                                                      const int32_t* __restrict__ slot_rows) {
+__device__ __forceinline__ void wgrad_coop_body(const WgradArgs& a, const ChunkInfo* __restrict__ chunks,
+                                                const int32_t* __restrict__ slot_rows, int bx, int by, int nx) {
   constexpr int RS = 2, NBW = NB / 2;
   constexpr int OS = kWgradStageStride;
   constexpr int XS = 136;  // row stride of a staged tile in bf16 (272 B)
@@ -684,13 +770,13 @@ __global__ __launch_bounds__(128) void k_wgrad_coop(WgradArgs a, const ChunkInfo
   __shared__ __attribute__((aligned(16))) float lds[kLdsFloats];
   extern __shared__ __attribute__((aligned(16))) int32_t rows_s[];  // the chunk's row indices
   const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kb = lane >> 4, rs = tid >> 6;
-  if ((int)blockIdx.y < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
-    transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)blockIdx.y * gridDim.x + blockIdx.x) * (RS * 64) + tid,
-                          (int64_t)a.tr.y_blocks * gridDim.x * (RS * 64));
+  if (by < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
+    transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)by * nx + bx) * (RS * 64) + tid,
+                          (int64_t)a.tr.y_blocks * nx * (RS * 64));
     return;
   }
-  const int c0 = blockIdx.x * 128;
-  const ChunkInfo ci = chunks[blockIdx.y - a.tr.y_blocks];
+  const int c0 = bx * 128;
+  const ChunkInfo ci = chunks[by - a.tr.y_blocks];
   const int g = ci.group;
   if (g < 0) return;
   const int r = min(a.rank[g], 16 * NB);
@@ -775,6 +861,25 @@ __global__ __launch_bounds__(128) void k_wgrad_coop(WgradArgs a, const ChunkInfo
     if (t + i < nt) consume(t + i, T[i]);
   __syncthreads();  // the last tile has been read everywhere: its buffer becomes the staging area
   if (mine) wgrad_store<NBW>(acc, lds + n_base * OS, a, ci, g, r, c0, lane, n_base);
+}
+
+template <int NB, int S>
+__global__ __launch_bounds__(128) void k_wgrad_coop(WgradArgs a, const ChunkInfo* __restrict__ chunks,
+                                                      const int32_t* __restrict__ slot_rows) {
+  wgrad_coop_body<NB, S>(a, chunks, slot_rows, blockIdx.x, blockIdx.y, gridDim.x);
+}
+
+// The same contraction for up to kMaxShared projections that read the same source (dA_p = dh_p^T x for the
+// projections of one input): one launch, the bodies of k_wgrad_coop, every tile of the source crossing memory
+// once (see shared_source_item).  Work item = (chunk, 128 columns), column block fastest.
+template <int NB, int S>
+__global__ __launch_bounds__(128) void k_wgrad_coop_multi(SharedWgradArgs jobs, int items, int nx,
+                                                            const ChunkInfo* __restrict__ chunks,
+                                                            const int32_t* __restrict__ slot_rows) {
+  int p, item;
+  shared_source_item(blockIdx.x, jobs.nproj, p, item);
+  if (item >= items) return;
+  wgrad_coop_body<NB, S>(jobs.w[p], chunks, slot_rows, item % nx, item / nx, nx);
 }
 
 // ---------------------------------------------------------------------------
@@ -1023,8 +1128,8 @@ void launch_wgrad_pipe(const WgradArgs& a0, const SegView& seg, const SegLayout&
   WgradArgs a = a0;
   a.tr.y_blocks = 0;
   if (a.tr.aT) {  // about four 16-byte outputs per thread of the side job
-    const int64_t units = (int64_t)a.tr.groups * a.rpad * ((a.tr.out_features + a.tr.in_features) / 8);
-    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 128) * 64)));
+    const int64_t units = (int64_t)a.tr.groups * a.rpad * ((a.tr.out_features + a.tr.in_features) / 64);
+    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (2 * (a.width / 128) * 64)));
   }
   const dim3 grid((unsigned)(a.width / 128), (unsigned)(L.max_chunks + a.tr.y_blocks));
   const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);  // a chunk's row indices
@@ -1038,8 +1143,8 @@ void launch_wgrad_coop(const WgradArgs& a0, const SegView& seg, const SegLayout&
   WgradArgs a = a0;
   a.tr.y_blocks = 0;
   if (a.tr.aT) {
-    const int64_t units = (int64_t)a.tr.groups * a.rpad * ((a.tr.out_features + a.tr.in_features) / 8);
-    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 128) * 128)));
+    const int64_t units = (int64_t)a.tr.groups * a.rpad * ((a.tr.out_features + a.tr.in_features) / 64);
+    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (2 * (a.width / 128) * 128)));
   }
   const dim3 grid((unsigned)(a.width / 128), (unsigned)(L.max_chunks + a.tr.y_blocks));
   const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);
@@ -1059,8 +1164,8 @@ int launch_dy_fused(const WgradArgs& a0, const void* const* lora_B, int64_t ldb,
   WgradArgs a = a0;
   a.tr.y_blocks = 0;
   if (a.tr.aT) {
-    const int64_t units = (int64_t)a.tr.groups * a.rpad * ((a.tr.bT ? a.tr.out_features : 0) + a.tr.in_features) / 8;
-    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * (a.width / 512) * 256)));
+    const int64_t units = (int64_t)a.tr.groups * a.rpad * ((a.tr.bT ? a.tr.out_features : 0) + a.tr.in_features) / 64;
+    a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (2 * (a.width / 512) * 256)));
   }
   const dim3 grid((unsigned)(a.width / 512), (unsigned)(L.max_chunks + a.tr.y_blocks));
   const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);  // a chunk's row indices
@@ -1085,8 +1190,8 @@ int launch_dy_fused_multi(const DyFusedJob* jobs, int n, const SegView& seg, con
     j.a.tr.y_blocks = 0;
     if (j.a.tr.aT) {
       const int64_t units =
-          (int64_t)j.a.tr.groups * j.a.rpad * ((j.a.tr.bT ? j.a.tr.out_features : 0) + j.a.tr.in_features) / 8;
-      j.a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (4 * j.x_blocks * 256)));
+          (int64_t)j.a.tr.groups * j.a.rpad * ((j.a.tr.bT ? j.a.tr.out_features : 0) + j.a.tr.in_features) / 64;
+      j.a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (2 * j.x_blocks * 256)));
     }
     J.x_first[p + 1] = J.x_first[p] + j.x_blocks;
     gy = std::max(gy, (int)L.max_chunks + j.a.tr.y_blocks);
@@ -1122,9 +1227,54 @@ int launch_transpose_job(const TransposeJob& t0, const int32_t* rank, int rpad, 
   if (t0.groups == 0) return TK_OK;
   TransposeJob t = t0;
   t.skip_dead = 1;
-  const int64_t units = (int64_t)t.groups * rpad * ((t.bT ? t.out_features : 0) + t.in_features) / 8;
-  const int64_t blocks = std::min<int64_t>(4096, std::max<int64_t>(1, units / (2 * 256)));
+  const int64_t units = (int64_t)t.groups * rpad * ((t.bT ? t.out_features : 0) + t.in_features) / 64;  // 8 x 8 blocks
+  const int64_t blocks = std::min<int64_t>(8192, std::max<int64_t>(1, units / 256));
   hipLaunchKernelGGL(k_transpose_job, dim3((unsigned)blocks), dim3(256), 0, s, t, rank, rpad);
+  return check_launch();
+}
+
+// Shrink (with the slice sums) of n projections of one padded rank above 16 that read the same source.
+int launch_shrink_multi(const PassArgs* a, int n, const SegView& seg, const SegLayout& L, hipStream_t s) {
+  if (L.rows == 0 || n == 0) return TK_OK;
+  PassJobs J{};
+  for (int p = 0; p < n; ++p) J.p[p] = a[p];
+  const int32_t* rows = seg.slot_table(a[0].map_rows);
+  const int items = (int)(ceil_div(L.max_tiles, 2) * a[0].kslices);
+  const dim3 grid((unsigned)(ceil_div(items, 8) * 8 * n));
+  if (a[0].rpad <= 32)
+    hipLaunchKernelGGL((k_shrink_pair_multi<2, 2>), grid, dim3(128), 0, s, J, n, items, seg.tile_group, rows,
+                       (int)L.max_tiles);
+  else
+    hipLaunchKernelGGL((k_shrink_pair_multi<4, 4>), grid, dim3(256), 0, s, J, n, items, seg.tile_group, rows,
+                       (int)L.max_tiles);
+  if (a[0].kslices > 1) {
+    for (int p = 0; p < n; ++p) {
+      bf16_t* hrow = (bf16_t*)a[p].hT + (int64_t)a[p].rpad * a[p].ldh;
+      if (a[0].rpad <= 32)
+        hipLaunchKernelGGL(k_shrink_finish<2>, dim3((unsigned)L.max_tiles), dim3(256), 0, s, a[p], hrow,
+                           seg.tile_group, rows);
+      else
+        hipLaunchKernelGGL(k_shrink_finish<4>, dim3((unsigned)L.max_tiles), dim3(256), 0, s, a[p], hrow,
+                           seg.tile_group, rows);
+    }
+  }
+  return check_launch();
+}
+
+// Row contractions of n projections of one padded rank above 16 over the same source (see k_wgrad_coop_multi).
+int launch_wgrad_coop_multi(const SharedWgradArgs& a0, const SegView& seg, const SegLayout& L, hipStream_t s) {
+  if (L.rows == 0 || a0.nproj == 0) return TK_OK;
+  SharedWgradArgs a = a0;
+  for (int p = 0; p < a.nproj; ++p) a.w[p].tr = TransposeJob{};
+  const int nx = a.w[0].width / 128;
+  const int items = nx * (int)L.max_chunks;
+  const dim3 grid((unsigned)(ceil_div(items, 8) * 8 * a.nproj));
+  const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);
+  const int32_t* rows = seg.slot_table(a.w[0].map_rows);
+  if (a.w[0].rpad <= 32)
+    hipLaunchKernelGGL((k_wgrad_coop_multi<2, TK_COOP_STAGES>), grid, dim3(128), dyn, s, a, items, nx, seg.chunks, rows);
+  else
+    hipLaunchKernelGGL((k_wgrad_coop_multi<4, TK_COOP_STAGES>), grid, dim3(128), dyn, s, a, items, nx, seg.chunks, rows);
   return check_launch();
 }
 

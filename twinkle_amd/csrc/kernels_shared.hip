@@ -6,9 +6,15 @@
 //   backward  k_expand_shared   dx += sum_p dh_p A_p in one read-modify-write of dx instead of one per projection
 //             k_wgrad_shared    dA_p = dh_p^T x for every projection from one pass over x
 //
-// Each projection has padded rank 16 here, so projection p is simply block p of 16 rank indices of the
+// Each projection has padded rank 16 in these three, so projection p is simply block p of 16 rank indices of the
 // single-projection kernels: same operand layouts, same order of every sum, hence the same h, dA and dB bit
 // for bit; only dx differs (one rounding to bf16 instead of one per projection).
+//
+// At padded rank 32 and 64 a wave cannot hold several projections' operands at once.  There the single-projection
+// shrink and row-contraction bodies are launched for all projections together, blocks that read the same piece of
+// x next to each other on one XCD (k_shrink_pair_multi, k_wgrad_coop_multi in kernels_mfma.hip), and
+//             k_expand_shared_wide   takes the projections one after the other into the same accumulators:
+//                                    again one read-modify-write of dx.
 #include "tk_mfma.h"
 
 namespace tk {
@@ -363,7 +369,102 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(P <= 3 ? 2 :
   }
 }
 
+// ---------------------------------------------------------------------------
+// dx[row] += sum_p dh_p[row] A_p for projections of padded rank 32 or 64: one wave = one tile x 128 columns as in
+// k_expand_shared, but the projections are taken one after the other (a projection's block of A^T, 128 columns x
+// rank, is as large as the wave's piece of the tile, so only one of them is held at a time) while the products of all
+// of them add up in the same accumulators: dx is read and written once.  Weights come from the transposed copies
+// [G][K][rpad] of every projection (not permuted).  Tiles are taken in sweep order when rows are gathered.
+// ---------------------------------------------------------------------------
+template <int NB>
+__global__ __launch_bounds__(256) void k_expand_shared_wide(SharedExpandArgs a, const int32_t* __restrict__ tile_group,
+                                                            const int32_t* __restrict__ slot_rows,
+                                                            const int32_t* __restrict__ tile_walk, int num_items) {
+  constexpr int RP = 16 * NB, NKS = RP / 32;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  const int ngroups = a.width_dst >> 7;
+  const int item = blockIdx.x * 4 + wave;
+  if (item >= num_items) return;
+  const int nth = item / ngroups;
+  const int tile_id = tile_walk ? tile_walk[nth] : nth;
+  const int c0 = (item - nth * ngroups) << 7;
+  const int slot0 = tile_id * kTileRows;
+  const int g_raw = tile_group[tile_id];
+  const int4 r0 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 4 * kb);
+  const int4 r1 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 16 + 4 * kb);
+  const int g = max(g_raw, 0);
+  const int rows[2][4] = {{r0.x, r0.y, r0.z, r0.w}, {r1.x, r1.y, r1.z, r1.w}};
+  bool rok[2][4];
+  bf16_t* yp[2][4];
+  uint4 y[2][4];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      rok[tt][v] = g_raw >= 0 && rows[tt][v] >= 0;
+      yp[tt][v] = (bf16_t*)a.dst + (int64_t)(rok[tt][v] ? rows[tt][v] : 0) * a.ld_dst + 8 * li + c0;
+      y[tt][v] = rok[tt][v] ? ld16_nt(yp[tt][v]) : zero4();
+    }
+  f32x4 d[2][8];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int q = 0; q < 8; ++q) d[tt][q] = f32x4{0.f, 0.f, 0.f, 0.f};
+  bool any = false;
+  for (int p = 0; p < a.nproj; ++p) {
+    const int r = g_raw < 0 ? 0 : min(pick(a.rank, p)[g], RP);  // uniform over the wave
+    if (r <= 0) continue;
+    any = true;
+    const bf16_t* hp = (const bf16_t*)pick(a.hrow, p);
+    const bf16_t* wt = (const bf16_t*)pick(a.aT, p) + ((int64_t)g * a.width_dst + c0 + 8 * li) * RP;
+    uint4 hop[2][NKS], bq[8][NKS];
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      const int n0 = 32 * ks + 8 * kb;
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) hop[tt][ks] = ld16(hp + (int64_t)(slot0 + 16 * tt + li) * RP + n0);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) bq[q][ks] = n0 < r ? keep_first(ld16(wt + (int64_t)q * RP + n0), r - n0) : zero4();
+    }
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) d[tt][q] = mfma16(hop[tt][ks], bq[q][ks], d[tt][q]);
+  }
+  if (!any) return;  // unused tile, or no projection live on this layer (uniform over the wave)
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      if (!rok[tt][v]) continue;
+      const uint4 yy = y[tt][v];
+      uint4 o;
+      o.x = pack_bf16(bf16_lo(yy.x) + d[tt][0][v], bf16_hi(yy.x) + d[tt][1][v]);
+      o.y = pack_bf16(bf16_lo(yy.y) + d[tt][2][v], bf16_hi(yy.y) + d[tt][3][v]);
+      o.z = pack_bf16(bf16_lo(yy.z) + d[tt][4][v], bf16_hi(yy.z) + d[tt][5][v]);
+      o.w = pack_bf16(bf16_lo(yy.w) + d[tt][6][v], bf16_hi(yy.w) + d[tt][7][v]);
+      st16_nt(yp[tt][v], o);
+    }
+}
+
 }  // namespace
+
+int launch_expand_shared_wide(const SharedExpandArgs& a, int rpad, const SegView& seg, const SegLayout& L,
+                              hipStream_t s) {
+  if (L.rows == 0) return TK_OK;
+  const int64_t items = L.max_tiles * (a.width_dst >> 7);
+  const dim3 grid((unsigned)ceil_div(items, 4));
+  const int32_t* rows = seg.slot_table(a.map_rows);
+  if (rpad <= 32)
+    hipLaunchKernelGGL(k_expand_shared_wide<2>, grid, dim3(256), 0, s, a, seg.tile_group, rows,
+                       seg.tile_walk(a.map_rows), (int)items);
+  else
+    hipLaunchKernelGGL(k_expand_shared_wide<4>, grid, dim3(256), 0, s, a, seg.tile_group, rows,
+                       seg.tile_walk(a.map_rows), (int)items);
+  return check_launch();
+}
 
 int launch_shrink_shared(const SharedShrinkArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s) {
   if (L.rows == 0) return TK_OK;

@@ -252,7 +252,7 @@ struct WgradArgs {
   TransposeJob tr;
 };
 
-// Projections that share their input (kernels_shared.hip); every projection has padded rank 16 there.
+// Projections that share their input (kernels_shared.hip).
 constexpr int kMaxShared = 4;
 struct SharedShrinkArgs {
   const void* src;  int64_t ld_src;      // x
@@ -265,8 +265,8 @@ struct SharedShrinkArgs {
 struct SharedExpandArgs {
   void* dst;  int64_t ld_dst;            // dx
   int32_t width_dst, map_rows, nproj;
-  const void* hrow[kMaxShared];          // slot-major dh of projection p, [slots][16]
-  const void* aT[kMaxShared];            // A_p^T copies, [G][K][16]
+  const void* hrow[kMaxShared];          // slot-major dh of projection p, [slots][rpad]
+  const void* aT[kMaxShared];            // A_p^T copies, [G][K][rpad]
   const int32_t* rank[kMaxShared];
 };
 struct SharedWgradArgs {                 // dA_p for all p from one pass over x (w[p].src / ld_src / width agree)
@@ -299,6 +299,10 @@ int launch_wgrad_reduce_multi(const WgradArgs* sets, int n, const SegView& seg, 
 int launch_shrink_shared(const SharedShrinkArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
 int launch_expand_shared(const SharedExpandArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
 int launch_wgrad_shared(const SharedWgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
+// projections of one padded rank 32 or 64 that share their input
+int launch_shrink_multi(const PassArgs* a, int n, const SegView& seg, const SegLayout& L, hipStream_t s);
+int launch_expand_shared_wide(const SharedExpandArgs& a, int rpad, const SegView& seg, const SegLayout& L, hipStream_t s);
+int launch_wgrad_coop_multi(const SharedWgradArgs& a, const SegView& seg, const SegLayout& L, hipStream_t s);
 
 // kernels_grouped.hip
 struct GroupedPlanEntry {  // a row block of the grouped GEMM: up to 4 consecutive tiles of one expert
