@@ -36,6 +36,38 @@ __device__ inline int load_key(const KeyT* keys, int64_t f, int buckets, int* ba
   return (int)k;
 }
 
+// Eight consecutive keys starting at row f0 (a multiple of 8), as 16-byte loads where the array allows;
+// rows past the end give -1.
+template <typename KeyT>
+__device__ inline void load_keys8(const KeyT* keys, int64_t f0, int64_t rows, bool aligned16, int buckets, int* bad,
+                                  int (&out)[8]) {
+  if (aligned16 && f0 + 8 <= rows) {
+    long long raw[8];
+    if constexpr (sizeof(KeyT) == 4) {
+      const int4 a = *reinterpret_cast<const int4*>(keys + f0), b = *reinterpret_cast<const int4*>(keys + f0 + 4);
+      const int v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) raw[j] = v[j];
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; j += 2) {
+        const longlong2 a = *reinterpret_cast<const longlong2*>(keys + f0 + j);
+        raw[j] = a.x;
+        raw[j + 1] = a.y;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const bool off = raw[j] < 0 || raw[j] >= buckets - 1;
+      *bad += off;
+      out[j] = off ? buckets - 1 : (int)raw[j];
+    }
+    return;
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) out[j] = f0 + j < rows ? load_key(keys, f0 + j, buckets, bad) : -1;
+}
+
 // lanes of this wave that are valid and hold the same key as the calling lane
 __device__ inline unsigned long long same_key_lanes(bool valid, int key, int key_bits) {
   unsigned long long same = __ballot(valid);
@@ -312,14 +344,13 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
     const int64_t f = base + wave * 64 + lane;
     mine = f < rows ? load_key(keys, f, groups, &unused) : -1;
   }
+  // (which lane counts which key of a sort block is free: a lane takes eight neighbours)
+  static_assert(kKeysPerLane == 8, "a lane loads eight consecutive keys of a sort block");
+  const bool aligned16 = (reinterpret_cast<uintptr_t>(keys) & 15u) == 0;
   int k[kOneBatch][kKeysPerLane];
 #pragma unroll
   for (int u = 0; u < kOneBatch; ++u)
-#pragma unroll
-    for (int j = 0; j < kKeysPerLane; ++j) {
-      const int64_t f = (int64_t)(wave + u * kOneWaves) * kSortBlockRows + j * 64 + lane;
-      k[u][j] = f < rows ? load_key(keys, f, groups, &bad) : -1;
-    }
+    load_keys8(keys, (int64_t)(wave + u * kOneWaves) * kSortBlockRows + 8 * lane, rows, aligned16, groups, &bad, k[u]);
   for (int i = tid; i < 2 * kOneSubs * (kOneGroups + 1); i += kOneWaves * 64) (&cnt[0][0][0])[i] = 0;
   for (int i = tid; i < kKeysPerLane * kOneGroups; i += kOneWaves * 64) (&round_cnt[0][0])[i] = 0;
   __syncthreads();
@@ -448,8 +479,9 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
 
   const int num_tiles = tfirst[groups], num_chunks = cfirst[groups];
   const int real_tiles = tfirst[groups - 1];  // the tiles of the rows without a group come after them
+  // spread over the blocks: entry i belongs to thread i / sort_blocks of block i % sort_blocks
   const int stride = sort_blocks * kOneWaves * 64;
-  for (int i = blk * kOneWaves * 64 + tid; i < max_tiles; i += stride) {
+  for (int i = tid * sort_blocks + blk; i < max_tiles; i += stride) {
     int g = -1, pos0 = 0, valid = 0;
     if (i < num_tiles) {
       g = group_of(tfirst, groups, i);
@@ -465,7 +497,7 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
                             j + 2 < valid ? pos0 + j + 2 : -1, j + 3 < valid ? pos0 + j + 3 : -1);
     for (int j = valid; j < kTileRows; ++j) V.slot_row[(int64_t)i * kTileRows + j] = -1;
   }
-  for (int i = blk * kOneWaves * 64 + tid; i < max_chunks; i += stride) {
+  for (int i = tid * sort_blocks + blk; i < max_chunks; i += stride) {
     ChunkInfo c{-1, 0, 0, -1};
     if (i < num_chunks) {
       const int g = group_of(cfirst, groups, i);
