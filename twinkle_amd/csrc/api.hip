@@ -220,7 +220,8 @@ static PassArgs fwd_pass_args(const tk_lora_desc* d, const void* x, int64_t ldx,
   a.width_src = d->in_features;  a.width_dst = d->out_features;
   a.map_rows = d->map_rows;  a.rpad = rank_pad(d->max_rank);  a.src_rows = (int32_t)d->rows;
   a.hpart = (float*)((char*)h + round_up(2 * (int64_t)a.rpad * a.ldh * elt_bytes(d->dtype), 256));
-  a.kslices = shrink_kslices(d->in_features, a.rpad);
+  const ShrinkPlan plan = shrink_plan(d->rows, d->num_groups, d->in_features, a.rpad);
+  a.kslices = plan.kslices;  a.quad_steps = plan.quad_steps;
   return a;
 }
 
@@ -270,7 +271,8 @@ static BwdPlan bwd_plan(const tk_lora_desc* d, const BwdLayout& B, const void* d
   a.width_src = d->out_features;  a.width_dst = d->in_features;
   a.map_rows = d->map_rows;  a.rpad = (int32_t)B.rpad;  a.src_rows = (int32_t)d->rows;
   a.hpart = (float*)(w + B.off_hpart);
-  a.kslices = shrink_kslices(d->out_features, a.rpad);
+  const ShrinkPlan plan = shrink_plan(d->rows, d->num_groups, d->out_features, a.rpad);
+  a.kslices = plan.kslices;  a.quad_steps = plan.quad_steps;
   TransposeJob& tr = p.tr;
   tr.lora_A = d->lora_A;  tr.lda = d->lda;
   tr.lora_B = d->lora_B;  tr.ldb = d->ldb;

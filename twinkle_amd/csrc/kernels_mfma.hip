@@ -247,6 +247,167 @@ __global__ __launch_bounds__(NW * 64) void k_shrink_pair_multi(PassJobs jobs, in
   shrink_pair_body<NB, NW>(a, (bf16_t*)a.hT + (int64_t)a.rpad * a.ldh, tile_group, slot_rows, max_tiles, item);
 }
 
+// ---------------------------------------------------------------------------
+// Shrink with the weights shared through LDS, for groups of many tiles.  In k_shrink_pair every wave fetches the
+// weight columns of its own steps, 16 * NB rank indices for 64 rows: at rank 64 as many bytes of weights (from L2)
+// as of activations (from memory), and the two share the path between L2 and the CUs, which is what sets the pace
+// (measured at rank 64: 536 MB of L2 reads for 268 MB of activations, 7.6 TB/s together).  Here a block of four
+// waves owns (eight consecutive tiles, slice of 64 * STEPS columns): wave w takes tiles 2 w and 2 w + 1 of the
+// eight through all steps, and the weight block of a step (16 * NB x 64) is fetched once per block, 16 B per
+// thread, into a double-buffered LDS tile from which every wave reads its MFMA operands: a quarter of the weight
+// traffic.  One LDS-only barrier per step: a buffer is overwritten one step after the barrier behind its last
+// reader.  The eight tiles are taken in runs of equal group (almost always one run); waves whose tiles lie
+// outside the run still help to stage the weights.  The slice length (a.quad_steps) is chosen per launch.  Activations: three steps in registers per wave, loads two
+// steps ahead.  Every block leaves its sums as one slice of the split-shrink buffer (k_shrink_finish follows);
+// each entry is the sum of one wave's MFMA chain, so results do not depend on timing.
+// ---------------------------------------------------------------------------
+template <int NB>
+__device__ __forceinline__ void shrink_quad_body(const PassArgs& a, const int32_t* __restrict__ tile_group,
+                                                 const int32_t* __restrict__ slot_rows, int max_tiles, int item) {
+  constexpr int RP = 16 * NB;
+  constexpr int WS = 72;                    // row stride of a staged weight block in bf16 (144 B: conflict-free)
+  constexpr int NLD = (RP * 8 + 255) / 256;  // 16-byte pieces of a weight block per thread
+  constexpr int S = NB == 4 ? 2 : 3;  // steps of activations in registers (rank 64: the accumulators take the room)
+  __shared__ __attribute__((aligned(16))) bf16_t wbuf[2][RP * WS];
+  __shared__ int32_t gts[8];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  const int set = item / a.kslices, ks = item - set * a.kslices;
+  const int t_first = set * 8;
+  if (tid < 8) gts[tid] = t_first + tid < max_tiles ? tile_group[t_first + tid] : -1;
+  const int nsteps = a.width_src >> 6;
+  const int s0 = ks * a.quad_steps;
+  const int ns = min(a.quad_steps, nsteps - s0);  // >= 1 for every slice
+  // this wave's two tiles
+  const bf16_t* src = (const bf16_t*)a.src;
+  const bf16_t *xa[2], *xb[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int t = min(t_first + 2 * wave + u, max_tiles - 1);
+    int ra = slot_rows[t * kTileRows + li], rb = slot_rows[t * kTileRows + 16 + li];
+    ra = min(max(ra, 0), a.src_rows - 1);
+    rb = min(max(rb, 0), a.src_rows - 1);
+    xa[u] = src + (int64_t)ra * a.ld_src + 16 * kb + (int64_t)s0 * 64;
+    xb[u] = src + (int64_t)rb * a.ld_src + 16 * kb + (int64_t)s0 * 64;
+  }
+  __syncthreads();
+  for (int j = 0; j < 8;) {
+    const int g = gts[j];
+    int e = j + 1;
+    while (e < 8 && gts[e] == g) ++e;
+    const int lo = j, hi = e;  // the run: tiles t_first + lo .. t_first + hi - 1, all of group g
+    j = e;
+    if (g < 0) continue;
+    const int r = min(a.rank[g], RP);
+    if (r <= 0) continue;  // adapter not live on this layer
+    bool mine[2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) mine[u] = 2 * wave + u >= lo && 2 * wave + u < hi;
+    const bool active = mine[0] || mine[1];  // wave-uniform
+    const bf16_t* W1 = group_weight<bf16_t>(a.w_shrink, a.w_shrink_base, a.shrink_group_stride, g) + (int64_t)s0 * 64;
+    // staging: piece p = tid + 256 i is columns 8 (p % 8) .. + 8 of rank index p / 8
+    auto stage_load = [&](int s, uint4 (&wr)[NLD]) {
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const int p = tid + 256 * i, n = p >> 3;
+        wr[i] = (n < r && s < ns) ? ld16(W1 + (int64_t)n * a.ld_shrink + (s << 6) + 8 * (p & 7)) : zero4();
+      }
+    };
+    auto stage_store = [&](int buf, const uint4 (&wr)[NLD]) {
+#pragma unroll
+      for (int i = 0; i < NLD; ++i) {
+        const int p = tid + 256 * i, n = p >> 3;
+        if (n < RP) st16(&wbuf[buf][n * WS + 8 * (p & 7)], wr[i]);
+      }
+    };
+    struct Step {
+      uint4 x0[2][2], x1[2][2];
+    };
+    auto issue = [&](int s, Step& X) {
+      const int c = min(s, ns - 1) << 6;  // requests past the slice repeat its last step and are not used
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        X.x0[u][0] = ld16(xa[u] + c);
+        X.x1[u][0] = ld16(xa[u] + c + 8);
+        X.x0[u][1] = ld16(xb[u] + c);
+        X.x1[u][1] = ld16(xb[u] + c + 8);
+      }
+    };
+    f32x4 acc[2][2][NB];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[u][tt][nb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    uint4 wr[NLD];
+    auto step = [&](int s, const Step& X, Step& Xnext) {
+      lds_barrier();  // block s is complete; the other buffer has been read by everyone
+      stage_load(s + 1, wr);
+      if (active) issue(s + S - 1, Xnext);
+      if (active) {
+        const bf16_t* wb = wbuf[s & 1] + li * WS + 16 * kb;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const uint4 w0 = ld16(wb + 16 * nb * WS), w1 = ld16(wb + 16 * nb * WS + 8);
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int tt = 0; tt < 2; ++tt) {
+              acc[u][tt][nb] = mfma16(X.x0[u][tt], w0, acc[u][tt][nb]);
+              acc[u][tt][nb] = mfma16(X.x1[u][tt], w1, acc[u][tt][nb]);
+            }
+        }
+      }
+      stage_store((s + 1) & 1, wr);  // block s + 1 (zeros past the slice), visible behind the next barrier
+    };
+    Step T[S];
+    stage_load(0, wr);
+    if (active) {
+#pragma unroll
+      for (int i = 0; i < S - 1; ++i) issue(i, T[i]);
+    }
+    stage_store(0, wr);
+    int s = 0;
+    for (; s + S <= ns; s += S) {
+#pragma unroll
+      for (int i = 0; i < S; ++i) step(s + i, T[i], T[(i + S - 1) % S]);
+    }
+#pragma unroll
+    for (int i = 0; i < S - 1; ++i)
+      if (s + i < ns) step(s + i, T[i], T[(i + S - 1) % S]);  // block-uniform
+    lds_barrier();  // the next run's first block goes into buffer 0
+    if (!active) continue;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      if (!mine[u]) continue;
+      float* out = a.hpart + ((int64_t)(t_first + 2 * wave + u) * a.kslices + ks) * (kTileRows * RP) + 4 * kb * RP + li;
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) out[(16 * tt + v) * RP + 16 * nb] = acc[u][tt][nb][v];
+    }
+  }
+}
+
+template <int NB>
+__global__ __launch_bounds__(256, 2) void k_shrink_quad(PassArgs a, const int32_t* __restrict__ tile_group,
+                                                     const int32_t* __restrict__ slot_rows, int max_tiles) {
+  shrink_quad_body<NB>(a, tile_group, slot_rows, max_tiles, blockIdx.x);
+}
+
+// The same for up to kMaxShared projections that read the same source (see shared_source_item).
+template <int NB>
+__global__ __launch_bounds__(256, 2) void k_shrink_quad_multi(PassJobs jobs, int nproj, int items,
+                                                           const int32_t* __restrict__ tile_group,
+                                                           const int32_t* __restrict__ slot_rows, int max_tiles) {
+  int p, item;
+  shared_source_item(blockIdx.x, nproj, p, item);
+  if (item >= items) return;
+  shrink_quad_body<NB>(jobs.p[p], tile_group, slot_rows, max_tiles, item);
+}
+
 // Adds the slices of a split shrink in slice order and writes h (one block per tile).
 template <int NB>
 __device__ __forceinline__ void shrink_finish_body(const PassArgs& a, bf16_t* __restrict__ hrow,
@@ -1103,9 +1264,14 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
   bf16_t* hrow = (bf16_t*)a.hT + (int64_t)a.rpad * a.ldh;  // second half of the h buffer
   const int32_t* rows = seg.slot_table(a.map_rows);
   constexpr int NW = NB == 1 ? 1 : (NB == 2 ? 2 : 4);  // shrink_waves(16 * NB)
-  if (phases & 1)
-    hipLaunchKernelGGL((k_shrink_pair<NB, NW>), dim3((unsigned)(ceil_div(L.max_tiles, 2) * a.kslices)), dim3(NW * 64), 0,
-                       s, a, hrow, seg.tile_group, rows, (int)L.max_tiles);
+  if (phases & 1) {
+    if (NB > 1 && a.quad_steps > 0)  // see shrink_plan
+      hipLaunchKernelGGL((k_shrink_quad<NB>), dim3((unsigned)(ceil_div(L.max_tiles, 8) * a.kslices)), dim3(256), 0, s,
+                         a, seg.tile_group, rows, (int)L.max_tiles);
+    else
+      hipLaunchKernelGGL((k_shrink_pair<NB, NW>), dim3((unsigned)(ceil_div(L.max_tiles, 2) * a.kslices)),
+                         dim3(NW * 64), 0, s, a, hrow, seg.tile_group, rows, (int)L.max_tiles);
+  }
   if ((phases & 5) && a.kslices > 1)
     hipLaunchKernelGGL((k_shrink_finish<NB>), dim3((unsigned)L.max_tiles), dim3(256), 0, s, a, hrow, seg.tile_group,
                        rows);
@@ -1239,14 +1405,23 @@ int launch_shrink_multi(const PassArgs* a, int n, const SegView& seg, const SegL
   PassJobs J{};
   for (int p = 0; p < n; ++p) J.p[p] = a[p];
   const int32_t* rows = seg.slot_table(a[0].map_rows);
-  const int items = (int)(ceil_div(L.max_tiles, 2) * a[0].kslices);
+  const bool quad = a[0].quad_steps > 0;
+  const int items = (int)(ceil_div(L.max_tiles, quad ? 8 : 2) * a[0].kslices);
   const dim3 grid((unsigned)(ceil_div(items, 8) * 8 * n));
-  if (a[0].rpad <= 32)
+  if (quad) {  // the single-projection launch makes the same choice: same sums, same bits
+    if (a[0].rpad <= 32)
+      hipLaunchKernelGGL((k_shrink_quad_multi<2>), grid, dim3(256), 0, s, J, n, items, seg.tile_group, rows,
+                         (int)L.max_tiles);
+    else
+      hipLaunchKernelGGL((k_shrink_quad_multi<4>), grid, dim3(256), 0, s, J, n, items, seg.tile_group, rows,
+                         (int)L.max_tiles);
+  } else if (a[0].rpad <= 32) {
     hipLaunchKernelGGL((k_shrink_pair_multi<2, 2>), grid, dim3(128), 0, s, J, n, items, seg.tile_group, rows,
                        (int)L.max_tiles);
-  else
+  } else {
     hipLaunchKernelGGL((k_shrink_pair_multi<4, 4>), grid, dim3(256), 0, s, J, n, items, seg.tile_group, rows,
                        (int)L.max_tiles);
+  }
   if (a[0].kslices > 1) {
     for (int p = 0; p < n; ++p) {
       bf16_t* hrow = (bf16_t*)a[p].hT + (int64_t)a[p].rpad * a[p].ldh;

@@ -160,8 +160,28 @@ static inline int shrink_waves(int rpad) { return rpad <= 16 ? 1 : (rpad <= 32 ?
 static inline int shrink_kslices(int width, int rpad) {
   return (int)ceil_div(ceil_div(width, 64), (int64_t)kShrinkSteps * shrink_waves(rpad));
 }
+// Above rank 16, with long groups and a source of 1024 to 4096 columns, the shrink runs as k_shrink_quad: blocks of
+// (eight tiles, `steps` steps of 64 columns).  The slices are cut so that all blocks are resident at once where
+// the row count allows (two blocks of four waves per CU, 256 CUs): a launch of 1.02 rounds costs two.  Wider
+// sources stay with k_shrink_pair (measured at 14336 columns, rank 64: 304 us against 236; there a block's short
+// look-ahead along each of its 256 rows costs more than the shared weights save).
+constexpr int kQuadResident = 512;
+struct ShrinkPlan {
+  int kslices;     // slices per tile
+  int quad_steps;  // 0: k_shrink_pair; else steps per slice of k_shrink_quad
+};
+static inline ShrinkPlan shrink_plan(int64_t rows, int64_t groups, int width, int rpad) {
+  const int nsteps = (int)ceil_div(width, 64);
+  if (rpad <= 16 || nsteps < 16 || nsteps > 64 || rows < 8 * kTileRows * groups)
+    return ShrinkPlan{shrink_kslices(width, rpad), 0};
+  const int64_t sets = ceil_div(rows, 8 * kTileRows);
+  int ks = (int)std::min<int64_t>(kQuadResident / sets, nsteps / 8);
+  ks = std::max(ks, 2);
+  const int steps = (int)ceil_div(nsteps, ks);
+  return ShrinkPlan{(int)ceil_div(nsteps, steps), steps};  // no empty slice at the end
+}
 static inline int64_t shrink_partial_bytes(int64_t rows, int64_t groups, int width, int rpad) {
-  const int ks = shrink_kslices(width, rpad);
+  const int ks = std::max(shrink_kslices(width, rpad), shrink_plan(rows, groups, width, rpad).kslices);
   return ks > 1 ? round_up(SegLayout(rows, groups).max_tiles * ks * (int64_t)kTileRows * rpad * 4, 256) : 0;
 }
 
@@ -171,7 +191,8 @@ static inline int fused_dy_kslices(int width, int rpad) {
   return ((rpad == 16 || rpad == 32) && width % 512 == 0 && width >= 1024) ? width / 512 : 0;
 }
 static inline int64_t bwd_partial_bytes(int64_t rows, int64_t groups, int width, int rpad) {
-  const int ks = std::max(shrink_kslices(width, rpad), fused_dy_kslices(width, rpad));
+  const int ks = std::max(std::max(shrink_kslices(width, rpad), shrink_plan(rows, groups, width, rpad).kslices),
+                          fused_dy_kslices(width, rpad));
   return ks > 1 ? round_up(SegLayout(rows, groups).max_tiles * ks * (int64_t)kTileRows * rpad * 4, 256) : 0;
 }
 
@@ -217,6 +238,7 @@ struct PassArgs {
   int32_t src_rows;  // rows of src / dst (bound for speculative row addresses)
   float* hpart;          // partial sums of the split shrink, [tile][slice][32][rpad]
   int32_t kslices;       // blocks per tile of the MFMA shrink
+  int32_t quad_steps;    // 0: k_shrink_pair; else k_shrink_quad with this many 64-column steps per slice
   // the expand weight's rows are permuted inside every group of 128 (TransposeJob::swizzle_a): the row of
   // column c0 + 8 i + q lies at c0 + 16 q + i, so that the 16 rows one MFMA operand load touches are adjacent
   int32_t expand_swizzled;
