@@ -571,6 +571,8 @@ def main():
                     help='cfg2 with another number of tokens (a scaling measurement, not the headline configuration)')
     ap.add_argument('--rank', type=int, default=0,
                     help='cfg2 with another adapter rank (alpha = 2 x rank; a scaling measurement like --tokens)')
+    ap.add_argument('--weights-f32', action='store_true',
+                    help='keep the adapters and their gradients in fp32 under the bf16 activations')
     ap.add_argument('--optimizer-only', action='store_true',
                     help='run only the multi-tenant optimizer micro-benchmark and print its JSON (for profiling)')
     ap.add_argument('--shared-qkv', action='store_true',
@@ -646,9 +648,12 @@ def main():
     T, K, M, G = w.tokens, w.in_features, w.out_features, w.num_adapters
 
     ids = w.ids.to(dev)
-    A = [t.to(dt).to(dev) for t in w.lora_A]
-    B = [t.to(dt).to(dev) for t in w.lora_B]
-    groups = AdapterGroups(A, B, w.ranks, w.scales)
+    wdt = torch.float32 if args.weights_f32 else dt     # fp32 adapters under the bf16 activations (PEFT's default)
+    A = [t.to(wdt).to(dev) for t in w.lora_A]
+    B = [t.to(wdt).to(dev) for t in w.lora_B]
+    groups = AdapterGroups(A, B, w.ranks, w.scales, act_dtype=dt)
+    if args.weights_f32:
+        w.name += ', fp32 adapter weights and gradients'
     grad_a = [torch.zeros_like(t) for t in A]
     grad_b = [torch.zeros_like(t) for t in B]
     pa = torch.tensor([t.data_ptr() for t in grad_a], dtype=torch.int64, device=dev)

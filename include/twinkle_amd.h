@@ -143,6 +143,15 @@ typedef struct tk_lora_desc {
   int64_t ldb;                 /* elements */
   const int32_t* rank;         /* device [G] */
   const float* scale;          /* device [G]: alpha/r or alpha/sqrt(r) */
+  int32_t weights_f32;         /* 1 with dtype TK_DTYPE_BF16: A, B and their gradients are fp32 (lda, ldb in fp32
+                                  elements) while x, y and h are bf16, the usual state of a PEFT model whose base is
+                                  bf16 (adapters are kept in fp32; src/twinkle/model/multi_lora.py:320 casts x to
+                                  their dtype).  The kernels read bf16 copies of A and B that every call makes on
+                                  the fly inside h / the backward workspace (round to nearest even), multiply on
+                                  the matrix cores with fp32 accumulation and write fp32 gradients.  0: A, B and
+                                  the gradients have `dtype`.  The shared-input entry points then run one call per
+                                  projection; tk_grouped_linear does not take it (TK_ERR_UNSUPPORTED). */
+  int32_t reserved;            /* 0 */
 } tk_lora_desc;
 
 /* Bytes of the saved shrink output h (scale * x A^T per row, kept for backward). */

@@ -37,21 +37,27 @@ def lora_fwd_zero_base(x, seg, groups, map_rows=True):
     return y0
 
 
-def _run(dev, dtype, x, base, dy, a, b, ids, ranks, scales, check_zero_beyond_rank=True):
-    """GPU through autograd vs oracle in float64 on the same rounded inputs."""
+def _run(dev, dtype, x, base, dy, a, b, ids, ranks, scales, check_zero_beyond_rank=True, weights_f32=False):
+    """GPU through autograd vs oracle in float64 on the same rounded inputs.  ``weights_f32``: the adapters stay
+    fp32 tensors under activations of ``dtype`` (bf16); the oracle then works from the fp32 values, so the bar also
+    covers the rounding of the weights inside the library."""
     cast = lambda t: t.to(dtype)  # noqa: E731
+    wcast = (lambda t: t.float()) if weights_f32 else cast  # noqa: E731
     xd = cast(x).to(dev).requires_grad_(True)
     yd = cast(base).to(dev).requires_grad_(True)
-    ad = [cast(t).to(dev).requires_grad_(True) for t in a]
-    bd = [cast(t).to(dev).requires_grad_(True) for t in b]
+    ad = [wcast(t).to(dev).requires_grad_(True) for t in a]
+    bd = [wcast(t).to(dev).requires_grad_(True) for t in b]
     seg = build_segments(ids.to(torch.int32).to(dev), len(a), check=True)
-    groups = AdapterGroups(ad, bd, ranks, scales)
+    groups = AdapterGroups(ad, bd, ranks, scales, act_dtype=dtype if weights_f32 else None)
     y = multi_lora_delta(xd, yd * 1.0, seg, groups)
     y.backward(cast(dy).to(dev))
     f64 = lambda t: cast(t).double()  # noqa: E731
-    yo, dxo, dao, dbo = oracle.multi_lora_linear_grads(f64(x), f64(base), ids, [f64(t) for t in a],
-                                                        [f64(t) for t in b], ranks, scales, f64(dy))
+    w64 = lambda t: wcast(t).double()  # noqa: E731
+    yo, dxo, dao, dbo = oracle.multi_lora_linear_grads(f64(x), f64(base), ids, [w64(t) for t in a],
+                                                        [w64(t) for t in b], ranks, scales, f64(dy))
     tol = TOL[dtype]
+    if weights_f32:
+        assert all(t.grad is None or t.grad.dtype == torch.float32 for t in ad + bd), 'fp32 gradients'
     assert max_rel_err(y, yo) < tol, 'Y'
     # the LoRA term alone, on a zero base: the bar then scales with the term itself, not with the base output
     # (which at these shapes is an order of magnitude larger and would hide an error in the term)
@@ -93,6 +99,41 @@ def test_config1_fp32_plumbing(dev):
 ])
 def test_small_shapes(dev, dtype, t, k, m, n, max_r, ranks):
     _run(dev, dtype, *_problem(t, k, m, n, max_r, ranks, seed=t))
+
+
+@pytest.mark.parametrize('t,k,m,n,max_r,ranks', [
+    (33, 40, 24, 3, 8, [2, 8, 5]),                 # odd widths: generic kernels
+    (257, 128, 256, 4, 16, [16, 8, 16, 1]),
+    (900, 256, 1024, 5, 16, [16, 3, 0, 9, 16]),    # one pass over dy, a dead adapter
+    (2100, 128, 1536, 4, 8, [8, 8, 1, 5]),         # groups that span several chunks: partial sums, fp32 reduction
+    (1300, 256, 1024, 5, 32, [32, 17, 0, 24, 5]),
+    (1500, 384, 640, 6, 64, [64, 8, 16, 32, 64, 4]),
+    (2304, 2048, 512, 2, 64, [64, 48]),            # rank 64, long groups: the shrink with weights shared in LDS
+])
+def test_fp32_adapters_under_bf16_activations(dev, t, k, m, n, max_r, ranks):
+    """tk_lora_desc::weights_f32: A and B are read as fp32 (converted to bf16 on the fly inside the library), the
+    products run on the bf16 kernels, dA and dB come back as fp32 (PEFT's adapters under a bf16 base,
+    multi_lora.py:320).  Bar: the bf16 bar against the fp64 oracle on the unrounded weights."""
+    _run(dev, torch.bfloat16, *_problem(t, k, m, n, max_r, ranks, seed=t + 1), weights_f32=True)
+
+
+def test_fp32_adapters_gradient_accumulation(dev):
+    """accumulate=1 with fp32 gradients: a second backward adds onto the first in fp32."""
+    from twinkle_amd import lora_bwd_, lora_fwd_
+    x, base, dy, a, b, ids, ranks, scales = _problem(1100, 256, 1024, 3, 16, [16, 8, 16], seed=9)
+    xd, yd, dyd = (t.bfloat16().to(dev) for t in (x, base, dy))
+    ad, bd = [t.float().to(dev) for t in a], [t.float().to(dev) for t in b]
+    seg = build_segments(ids.to(torch.int32).to(dev), 3)
+    groups = AdapterGroups(ad, bd, ranks, scales, act_dtype=torch.bfloat16)
+    h = lora_fwd_(xd, yd.clone(), seg, groups)
+    ga, gb = [torch.zeros_like(t) for t in ad], [torch.zeros_like(t) for t in bd]
+    pa = torch.tensor([t.data_ptr() for t in ga], dtype=torch.int64, device=dev)
+    pb = torch.tensor([t.data_ptr() for t in gb], dtype=torch.int64, device=dev)
+    lora_bwd_(dyd, xd, h, None, pa, pb, seg, groups, accumulate=False)
+    once_a, once_b = [t.clone() for t in ga], [t.clone() for t in gb]
+    lora_bwd_(dyd, xd, h, None, pa, pb, seg, groups, accumulate=True)
+    for one, two in zip(once_a + once_b, ga + gb):
+        assert torch.equal(two, one + one)     # fp32 adds of equal numbers are exact
 
 
 @pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])

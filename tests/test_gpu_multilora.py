@@ -225,6 +225,19 @@ def test_mixed_dtype_base_bf16_adapters_fp32(dev):
                                       layer.lora_B['lora_0'].weight.detach().cpu(), 8, 2.0)
     assert want.dtype == torch.bfloat16
     assert max_rel_err(y, want) < 1e-2
+    # the adapters were read where they are (fp32) by the bf16 kernels, and their gradients arrive in fp32
+    groups = ml._groups_for(layer, 'lora_0', torch.bfloat16)
+    assert groups.dtype == torch.bfloat16 and groups.weights_f32
+    y.float().pow(2).sum().backward()
+    ga, gb = layer.lora_A['lora_0'].weight.grad, layer.lora_B['lora_0'].weight.grad
+    assert ga.dtype == torch.float32 and gb.dtype == torch.float32 and ga.abs().max() > 0 and gb.abs().max() > 0
+    # lora_compute_dtype=float32 asks for the reference's arithmetic instead: activations cast to fp32
+    ml.lora_compute_dtype = torch.float32
+    groups32 = ml._groups_for(layer, 'lora_0', torch.bfloat16)
+    assert groups32.dtype == torch.float32 and not groups32.weights_f32
+    with ml.adapter('alice'):
+        y32 = model(x)
+    assert y32.dtype == torch.bfloat16 and max_rel_err(y32, want) < 1e-2
 
 
 def test_batched_training_step_equals_tenants_one_after_the_other(dev):

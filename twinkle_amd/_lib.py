@@ -48,6 +48,8 @@ class LoraDesc(Structure):
         ('ldb', c_int64),
         ('rank', c_void_p),
         ('scale', c_void_p),
+        ('weights_f32', c_int32),
+        ('reserved', c_int32),
     ]
 
 

@@ -18,7 +18,24 @@ bool desc_ok(const tk_lora_desc* d) {
   if (d->dtype != TK_DTYPE_F32 && d->dtype != TK_DTYPE_BF16) return false;
   if (!d->seg_ws || !d->lora_A || !d->lora_B || !d->rank || !d->scale) return false;
   if (d->lda < d->in_features || d->ldb < d->max_rank) return false;
+  if (d->weights_f32 != 0 && (d->weights_f32 != 1 || d->dtype != TK_DTYPE_BF16)) return false;
   return true;
+}
+
+// fp32 adapter weights next to bf16 activations: make the bf16 copies at `stage` and return the descriptor the
+// kernels work from (the copies' pointer tables and strides; gradients keep the caller's strides, see bwd)
+int stage_weights(const tk_lora_desc* d, void* stage, bool want_a, bool want_b, hipStream_t s, tk_lora_desc* out) {
+  const int rpad = rank_pad(d->max_rank);
+  const WeightStage W(d->num_groups, rpad, d->in_features, d->out_features);
+  const int rc = launch_convert_weights(*d, stage, want_a, want_b, s);
+  if (rc != TK_OK) return rc;
+  *out = *d;
+  out->weights_f32 = 0;
+  out->lora_A = (const void* const*)((char*)stage + W.off_ptr_a);
+  out->lora_B = (const void* const*)((char*)stage + W.off_ptr_b);
+  out->lda = d->in_features;
+  out->ldb = rpad;
+  return TK_OK;
 }
 
 // TK_FORCE_GENERIC=1 in the environment routes every launch to the shape-agnostic kernels
@@ -191,15 +208,22 @@ int tk_unpermute_weight_grad(const void* dout, int64_t ld_dout, const void* rows
 static bool desc_shape_ok(const tk_lora_desc* d) {
   return d && d->rows >= 0 && d->num_groups > 0 && d->num_groups <= TK_MAX_GROUPS && d->max_rank >= 0 &&
          d->max_rank <= TK_MAX_RANK && d->in_features > 0 && d->out_features > 0 &&
-         (d->dtype == TK_DTYPE_F32 || d->dtype == TK_DTYPE_BF16);
+         (d->dtype == TK_DTYPE_F32 || d->dtype == TK_DTYPE_BF16) &&
+         (d->weights_f32 == 0 || (d->weights_f32 == 1 && d->dtype == TK_DTYPE_BF16));
+}
+
+// h without the staged weight copies that follow it when the adapters are fp32
+static int64_t h_core_bytes(const tk_lora_desc* d) {
+  const int rpad = rank_pad(d->max_rank);
+  return round_up(2 * (int64_t)rpad * h_ld(d->rows, d->num_groups) * elt_bytes(d->dtype), 256) +
+         shrink_partial_bytes(d->rows, d->num_groups, d->in_features, rpad);
 }
 
 int64_t tk_lora_h_bytes(const tk_lora_desc* d) {
   if (!desc_shape_ok(d)) return TK_ERR_INVALID;
-  // rank-major copy hT[rpad][ld], slot-major copy hrow[ld][rpad], then the partial sums of a split shrink
-  const int rpad = rank_pad(d->max_rank);
-  return round_up(2 * (int64_t)rpad * h_ld(d->rows, d->num_groups) * elt_bytes(d->dtype), 256) +
-         shrink_partial_bytes(d->rows, d->num_groups, d->in_features, rpad);
+  // rank-major copy hT[rpad][ld], slot-major copy hrow[ld][rpad], then the partial sums of a split shrink, then
+  // the bf16 copies of fp32 adapter weights
+  return h_core_bytes(d) + weight_stage_bytes(*d);
 }
 
 int64_t tk_lora_bwd_workspace_bytes(const tk_lora_desc* d) {
@@ -278,6 +302,9 @@ static BwdPlan bwd_plan(const tk_lora_desc* d, const BwdLayout& B, const void* d
   tr.lora_B = d->lora_B;  tr.ldb = d->ldb;
   tr.aT = p.aT;  tr.bT = p.bT;
   tr.in_features = d->in_features;  tr.out_features = d->out_features;  tr.groups = d->num_groups;
+  // fp32 adapters under bf16 activations: the backward kernels read the weights only through the transposed
+  // copies (made from the fp32 matrices directly) and, in the fused pass over dy, B itself; the gradients are fp32
+  tr.src_f32 = p.ga.grad_f32 = p.gb.grad_f32 = mixed_weights(*d) ? 1 : 0;
   return p;
 }
 
@@ -289,6 +316,13 @@ static int lora_pass_fwd(const tk_lora_desc* d, const void* x, int64_t ldx, void
   if ((phases & 2) && (!y || ldy < d->out_features)) return TK_ERR_INVALID;
   SegLayout L(d->rows, d->num_groups);
   SegView V(d->seg_ws, L);
+  tk_lora_desc staged;
+  if (mixed_weights(*d)) {  // each half of the forward converts the matrix it reads
+    const int rc = stage_weights(d, (char*)h + h_core_bytes(d), (phases & 1) != 0, (phases & 2) != 0,
+                                 (hipStream_t)stream, &staged);
+    if (rc != TK_OK) return rc;
+    d = &staged;
+  }
   const PassArgs a = fwd_pass_args(d, x, ldx, y, ldy, h);
   return run_pass(a, V, L, d->dtype, phases, (hipStream_t)stream);
 }
@@ -459,7 +493,7 @@ int tk_grouped_linear(const tk_grouped_desc* g, const tk_lora_desc* lora, const 
         lora->out_features != g->out_features || lora->dtype != g->dtype || lora->seg_ws != g->seg_ws ||
         lora->map_rows != g->map_rows)
       return TK_ERR_INVALID;
-    if (lora->max_rank > 64) return TK_ERR_UNSUPPORTED;
+    if (lora->max_rank > 64 || lora->weights_f32) return TK_ERR_UNSUPPORTED;
     a.rpad = rank_pad(lora->max_rank);
     a.lora_B = lora->lora_B;  a.ldb = lora->ldb;  a.rank = lora->rank;
     a.hrow = (const uint16_t*)h + (int64_t)a.rpad * h_ld(g->rows, g->num_groups);  // slot-major half of h
@@ -494,6 +528,12 @@ int tk_swiglu_bwd(const void* gu, int64_t ld_in, const void* dout, int64_t ld_do
 
 // ---- projections that share their input ------------------------------------------------------------------------
 
+static bool any_weights_f32(const tk_lora_desc* const* descs, int32_t n) {
+  for (int p = 0; descs && p < n && p < TK_MAX_SHARED; ++p)
+    if (descs[p] && descs[p]->weights_f32) return true;
+  return false;
+}
+
 static bool shared_descs_ok(const tk_lora_desc* const* descs, int32_t n) {
   if (!descs || n < 1 || n > TK_MAX_SHARED) return false;
   for (int p = 0; p < n; ++p) {
@@ -508,7 +548,7 @@ static bool shared_descs_ok(const tk_lora_desc* const* descs, int32_t n) {
 
 // the kernels of kernels_shared.hip apply: bf16, 2..4 projections of padded rank 16, a split shrink
 static bool shared_fast_path(const tk_lora_desc* const* descs, int32_t n) {
-  if (n < 2 || descs[0]->dtype != TK_DTYPE_BF16 || force_generic()) return false;
+  if (n < 2 || descs[0]->dtype != TK_DTYPE_BF16 || force_generic() || any_weights_f32(descs, n)) return false;
   for (int p = 0; p < n; ++p)
     if (descs[p]->max_rank < 1 || descs[p]->max_rank > 16) return false;
   return shrink_kslices(descs[0]->in_features, 16) > 1;
@@ -517,7 +557,7 @@ static bool shared_fast_path(const tk_lora_desc* const* descs, int32_t n) {
 // ... or the multi-projection launches of the kernels of padded rank 32 / 64: bf16, 2..4 projections whose padded
 // ranks agree (and exceed 16)
 static bool shared_wide_path(const tk_lora_desc* const* descs, int32_t n) {
-  if (n < 2 || descs[0]->dtype != TK_DTYPE_BF16 || force_generic()) return false;
+  if (n < 2 || descs[0]->dtype != TK_DTYPE_BF16 || force_generic() || any_weights_f32(descs, n)) return false;
   const int rpad = rank_pad(descs[0]->max_rank);
   if (rpad != 32 && rpad != 64) return false;
   for (int p = 0; p < n; ++p)

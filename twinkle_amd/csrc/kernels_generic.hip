@@ -119,6 +119,10 @@ __global__ __launch_bounds__(256) void k_expand_generic(PassArgs a, const int32_
 
 template <typename T>
 __device__ inline void store_grad(const WgradArgs& a, int g, int n, int c, float v) {
+  if (sizeof(T) != 4 && a.grad_f32) {  // fp32 gradient next to bf16 activations
+    store_grad<float>(a, g, n, c, v);
+    return;
+  }
   T* gp = (T*)a.grad[g];
   T* o = a.transposed ? gp + (int64_t)c * a.ld_grad + n : gp + (int64_t)n * a.ld_grad + c;
   if (a.accumulate) v += to_f32(*o);
@@ -263,27 +267,106 @@ __global__ __launch_bounds__(256) void k_wgrad_reduce_multi(WgradReduceJobs jobs
 }
 
 // bT_g[n][m] = B_g[m][n], aT_g[k][n] = A_g[n][k]; zero for n >= rank[g].
-template <typename T>
+// (TS: the adapters' element type, T: that of the copies; they differ for fp32 adapters under bf16 activations)
+template <typename TS, typename T>
 __global__ __launch_bounds__(256) void k_transpose_weights(tk_lora_desc d, int rpad, T* __restrict__ bT,
                                                            T* __restrict__ aT) {
   const int g = blockIdx.y;
   const int r = min(d.rank[g], rpad);
-  const T* A = (const T*)d.lora_A[g];
-  const T* B = (const T*)d.lora_B[g];
+  const TS* A = (const TS*)d.lora_A[g];
+  const TS* B = (const TS*)d.lora_B[g];
   const int64_t nb = (int64_t)rpad * d.out_features, na = (int64_t)rpad * d.in_features;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nb + na; i += (int64_t)gridDim.x * 256) {
     if (i < nb) {
       const int n = (int)(i / d.out_features), m = (int)(i % d.out_features);
-      bT[(int64_t)g * nb + i] = n < r ? B[(int64_t)m * d.ldb + n] : (T)0;
+      T v = (T)0;
+      if (n < r) from_f32(to_f32(B[(int64_t)m * d.ldb + n]), &v);
+      bT[(int64_t)g * nb + i] = v;
     } else {
       const int64_t q = i - nb;
       const int k = (int)(q / rpad), n = (int)(q % rpad);
-      aT[(int64_t)g * na + q] = n < r ? A[(int64_t)n * d.lda + k] : (T)0;
+      T v = (T)0;
+      if (n < r) from_f32(to_f32(A[(int64_t)n * d.lda + k]), &v);
+      aT[(int64_t)g * na + q] = v;
     }
   }
 }
 
+// bf16 copies of fp32 adapter weights (see WeightStage): the live rows of A_g as [rpad][in_features], the live
+// columns of B_g as [out_features][rpad], eight elements per thread, and the two pointer tables.  Round to
+// nearest even, as a cast of the tensors would.
+__global__ __launch_bounds__(256) void k_convert_weights(tk_lora_desc d, int rpad, char* stage, WeightStage W,
+                                                         int want_a, int want_b) {
+  const int g = blockIdx.y;
+  bf16_t* ac = (bf16_t*)(stage + W.off_a) + (int64_t)g * W.stride_a;
+  bf16_t* bc = (bf16_t*)(stage + W.off_b) + (int64_t)g * W.stride_b;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (want_a) ((const void**)(stage + W.off_ptr_a))[g] = ac;
+    if (want_b) ((const void**)(stage + W.off_ptr_b))[g] = bc;
+  }
+  const int r = min(d.rank[g], rpad);
+  const float* A = (const float*)d.lora_A[g];
+  const float* B = (const float*)d.lora_B[g];
+  const int k8 = (d.in_features + 7) >> 3, n8 = rpad >> 3;
+  const bool vec_a = (d.lda & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15u) == 0;
+  const bool vec_b = (d.ldb & 3) == 0 && (reinterpret_cast<uintptr_t>(B) & 15u) == 0;
+  const int64_t units_a = want_a ? (int64_t)r * k8 : 0;                 // (n, k-octet)
+  const int64_t units_b = want_b ? (int64_t)d.out_features * n8 : 0;    // (m, n-octet)
+  for (int64_t u = (int64_t)blockIdx.x * 256 + threadIdx.x; u < units_a + units_b; u += (int64_t)gridDim.x * 256) {
+    float v[8];
+    bf16_t* o;
+    int keep;
+    if (u < units_a) {
+      const int n = (int)(u / k8), k0 = (int)(u % k8) * 8;
+      keep = min(8, d.in_features - k0);
+      const float* src = A + (int64_t)n * d.lda + k0;
+      if (vec_a && keep == 8) {
+        const float4 lo = *reinterpret_cast<const float4*>(src), hi = *reinterpret_cast<const float4*>(src + 4);
+        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = j < keep ? src[j] : 0.f;
+      }
+      o = ac + (int64_t)n * d.in_features + k0;
+    } else {
+      const int64_t q = u - units_a;
+      const int m = (int)(q / n8), n0 = (int)(q % n8) * 8;
+      keep = 8;  // the copy's rows are rpad long: columns past the rank are written as zeros
+      const float* src = B + (int64_t)m * d.ldb + n0;
+      if (vec_b && n0 + 8 <= r) {
+        const float4 lo = *reinterpret_cast<const float4*>(src), hi = *reinterpret_cast<const float4*>(src + 4);
+        v[0] = lo.x; v[1] = lo.y; v[2] = lo.z; v[3] = lo.w; v[4] = hi.x; v[5] = hi.y; v[6] = hi.z; v[7] = hi.w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = n0 + j < r ? src[j] : 0.f;
+      }
+      o = bc + (int64_t)m * rpad + n0;
+    }
+    if (keep == 8 && (reinterpret_cast<uintptr_t>(o) & 15u) == 0) {  // one 16-byte store
+      uint16_t h[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) from_f32(v[j], &h[j]);
+      *reinterpret_cast<uint4*>(o) = make_uint4(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16),
+                                                h[4] | ((uint32_t)h[5] << 16), h[6] | ((uint32_t)h[7] << 16));
+      continue;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (j < keep) from_f32(v[j], &o[j]);
+  }
+}
+
 }  // namespace
+
+int launch_convert_weights(const tk_lora_desc& d, void* stage, bool want_a, bool want_b, hipStream_t s) {
+  const int rpad = rank_pad(d.max_rank);
+  const WeightStage W(d.num_groups, rpad, d.in_features, d.out_features);
+  const int64_t per_group = (int64_t)rpad * (d.in_features / 8 + 1) + (int64_t)d.out_features * (rpad / 8);
+  const dim3 grid((unsigned)std::min<int64_t>(ceil_div(per_group, 512), 64), (unsigned)d.num_groups);
+  hipLaunchKernelGGL(k_convert_weights, grid, dim3(256), 0, s, d, rpad, (char*)stage, W, want_a ? 1 : 0,
+                     want_b ? 1 : 0);
+  return check_launch();
+}
 
 int launch_pass_generic(const PassArgs& a, const SegView& seg, const SegLayout& L, int dtype, int phases,
                         hipStream_t s) {
@@ -325,7 +408,7 @@ int launch_wgrad_reduce(const WgradArgs* a0, const WgradArgs* a1, const SegView&
   const int rpad = a0 ? a0->rpad : a1->rpad;
   const int width = std::max(a0 ? a0->width : 0, a1 ? a1->width : 0);
   const dim3 grid((unsigned)L.groups, (unsigned)ceil_div(width, 256), (unsigned)(a1 ? 2 * (rpad / 8) : rpad / 8));
-  if (dtype == TK_DTYPE_F32)
+  if (dtype == TK_DTYPE_F32 || x0.grad_f32 || x1.grad_f32)  // (both sets have the gradient type of their descriptor)
     hipLaunchKernelGGL(k_wgrad_reduce<float>, grid, dim3(256), 0, s, x0, x1, rpad, seg.chunk_first, seg.partial_first);
   else
     hipLaunchKernelGGL(k_wgrad_reduce<bf16_t>, grid, dim3(256), 0, s, x0, x1, rpad, seg.chunk_first,
@@ -354,9 +437,12 @@ int launch_transpose_weights(const tk_lora_desc& d, void* bT, void* aT, hipStrea
   const int64_t per_group = (int64_t)rpad * (d.out_features + d.in_features);
   const dim3 grid((unsigned)std::min<int64_t>(ceil_div(per_group, 256), 64), (unsigned)d.num_groups);
   if (d.dtype == TK_DTYPE_F32)
-    hipLaunchKernelGGL(k_transpose_weights<float>, grid, dim3(256), 0, s, d, rpad, (float*)bT, (float*)aT);
+    hipLaunchKernelGGL((k_transpose_weights<float, float>), grid, dim3(256), 0, s, d, rpad, (float*)bT, (float*)aT);
+  else if (mixed_weights(d))
+    hipLaunchKernelGGL((k_transpose_weights<float, bf16_t>), grid, dim3(256), 0, s, d, rpad, (bf16_t*)bT, (bf16_t*)aT);
   else
-    hipLaunchKernelGGL(k_transpose_weights<bf16_t>, grid, dim3(256), 0, s, d, rpad, (bf16_t*)bT, (bf16_t*)aT);
+    hipLaunchKernelGGL((k_transpose_weights<bf16_t, bf16_t>), grid, dim3(256), 0, s, d, rpad, (bf16_t*)bT,
+                       (bf16_t*)aT);
   return check_launch();
 }
 

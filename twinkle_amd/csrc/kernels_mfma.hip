@@ -723,6 +723,18 @@ __device__ inline void transpose8x8(const uint4 (&in)[8], uint4 (&out)[8]) {
   }
 }
 
+// Eight consecutive weights as bf16, from a bf16 or an fp32 matrix (element index e, a multiple of 8 for the
+// vector form; fp32 is rounded to nearest even).
+__device__ inline uint4 load8_weights(const void* base, int64_t e, bool f32) {
+  if (!f32) return ld16((const bf16_t*)base + e);
+  const float4 lo = *reinterpret_cast<const float4*>((const float*)base + e);
+  const float4 hi = *reinterpret_cast<const float4*>((const float*)base + e + 4);
+  return make_uint4(pack_bf16(lo.x, lo.y), pack_bf16(lo.z, lo.w), pack_bf16(hi.x, hi.y), pack_bf16(hi.z, hi.w));
+}
+__device__ inline uint32_t load_weight(const void* base, int64_t e, bool f32) {
+  return f32 ? (pack_bf16(((const float*)base)[e], 0.f) & 0xffffu) : (uint32_t)((const bf16_t*)base)[e];
+}
+
 // Transposed weight copies (see TransposeJob).  A work unit is an 8 x 8 block: eight 16-byte loads along the
 // source's contiguous dimension, a transpose inside the lane, eight 16-byte stores along the copy's contiguous
 // dimension; consecutive threads take neighbouring blocks so that a wave's accesses cover whole rows (128 bytes and
@@ -732,6 +744,8 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
   const int m8 = t.out_features >> 3, n8 = rpad >> 3, k8 = t.in_features >> 3;
   const int64_t units_b = t.bT ? (int64_t)t.groups * m8 * n8 : 0;  // (g, m-octet, n-octet), n-octet fastest
   const int64_t units_a = (int64_t)t.groups * n8 * k8;              // (g, n-octet, k-octet), k-octet fastest
+  const bool f32 = t.src_f32 != 0;
+  const int ld_mask = f32 ? 3 : 7;  // row strides that keep every row 16-byte aligned
   for (int64_t u = thread; u < units_b + units_a; u += threads) {
     uint4 in[8], out[8];
     if (u < units_b) {
@@ -741,18 +755,19 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
       const int mo = (int)(q % m8), g = (int)(q / m8);
       const int r = min(rank[g], rpad);
       if (8 * no >= r && t.skip_dead) continue;
-      const bf16_t* B = (const bf16_t*)t.lora_B[g] + (int64_t)(8 * mo) * t.ldb + 8 * no;
-      const bool vec = (t.ldb & 7) == 0 && 8 * no + 8 <= t.ldb && (reinterpret_cast<uintptr_t>(t.lora_B[g]) & 15u) == 0;
+      const void* B = t.lora_B[g];
+      const int64_t b0 = (int64_t)(8 * mo) * t.ldb + 8 * no;
+      const bool vec = (t.ldb & ld_mask) == 0 && 8 * no + 8 <= t.ldb && (reinterpret_cast<uintptr_t>(B) & 15u) == 0;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         if (8 * no >= r) {
           in[i] = zero4();
         } else if (vec) {
-          in[i] = keep_first(ld16(B + (int64_t)i * t.ldb), r - 8 * no);
+          in[i] = keep_first(load8_weights(B, b0 + (int64_t)i * t.ldb, f32), r - 8 * no);
         } else {
           uint32_t e[8];
 #pragma unroll
-          for (int j = 0; j < 8; ++j) e[j] = 8 * no + j < r ? B[(int64_t)i * t.ldb + j] : 0;
+          for (int j = 0; j < 8; ++j) e[j] = 8 * no + j < r ? load_weight(B, b0 + (int64_t)i * t.ldb + j, f32) : 0;
           in[i] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
         }
       }
@@ -769,18 +784,19 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
       const int no = (int)(q % n8), g = (int)(q / n8);
       const int r = min(rank[g], rpad);
       if (8 * no >= r && t.skip_dead) continue;
-      const bf16_t* A = (const bf16_t*)t.lora_A[g] + (int64_t)(8 * no) * t.lda + 8 * ko;
-      const bool vec = (t.lda & 7) == 0 && (reinterpret_cast<uintptr_t>(t.lora_A[g]) & 15u) == 0;
+      const void* A = t.lora_A[g];
+      const int64_t a0 = (int64_t)(8 * no) * t.lda + 8 * ko;
+      const bool vec = (t.lda & ld_mask) == 0 && (reinterpret_cast<uintptr_t>(A) & 15u) == 0;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         if (8 * no + i >= r) {
           in[i] = zero4();
         } else if (vec) {
-          in[i] = ld16(A + (int64_t)i * t.lda);
+          in[i] = load8_weights(A, a0 + (int64_t)i * t.lda, f32);
         } else {
           uint32_t e[8];
 #pragma unroll
-          for (int j = 0; j < 8; ++j) e[j] = A[(int64_t)i * t.lda + j];
+          for (int j = 0; j < 8; ++j) e[j] = load_weight(A, a0 + (int64_t)i * t.lda + j, f32);
           in[i] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
         }
       }
@@ -1086,15 +1102,20 @@ __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* co
   for (int i = tid; i < nt * kTileRows; i += 256) rows_s[i] = slot_rows[ci.tile0 * kTileRows + i];
   // this wave's block of B as MFMA B operand: lane (n = 16 nb + li, kb) holds B[c0 + 32 s + 8 kb + i][n], i = 0..7
   uint4 wB[NB][4];
+  const void* Bsrc = lora_B[g];
+  const bool b_f32 = a.grad_f32 != 0;  // fp32 adapters: converted as they are loaded
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
     const int n = 16 * nb + li;
-    const bf16_t* Bg = (const bf16_t*)lora_B[g] + (int64_t)(c0 + 8 * kb) * ldb + (n < r ? n : 0);
+    const int64_t b0 = (int64_t)(c0 + 8 * kb) * ldb + (n < r ? n : 0);
 #pragma unroll
     for (int s4 = 0; s4 < 4; ++s4) {
       uint32_t e[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) e[i] = n < r ? Bg[(int64_t)(32 * s4 + i) * ldb] : 0;
+      for (int i = 0; i < 8; ++i)  // (the address is valid for every lane: loads first, masks after)
+        e[i] = load_weight(Bsrc, b0 + (int64_t)(32 * s4 + i) * ldb, b_f32);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) e[i] = n < r ? e[i] : 0;
       wB[nb][s4] = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
     }
   }

@@ -196,6 +196,27 @@ static inline int64_t bwd_partial_bytes(int64_t rows, int64_t groups, int width,
   return ks > 1 ? round_up(SegLayout(rows, groups).max_tiles * ks * (int64_t)kTileRows * rpad * 4, 256) : 0;
 }
 
+// bf16 copies of fp32 adapter weights (tk_lora_desc::weights_f32): pointer tables [G] for A and B, then
+// A_g as [rpad][in_features] and B_g as [out_features][rpad] for every group.
+struct WeightStage {
+  int64_t off_ptr_a, off_ptr_b, off_a, off_b, total;
+  int64_t stride_a, stride_b;  // elements per group
+  WeightStage(int64_t groups, int64_t rpad, int64_t in_features, int64_t out_features) {
+    stride_a = rpad * in_features;
+    stride_b = out_features * rpad;
+    int64_t o = 0;
+    off_ptr_a = o;  o += round_up(8 * groups, 256);
+    off_ptr_b = o;  o += round_up(8 * groups, 256);
+    off_a = o;      o += round_up(2 * groups * stride_a, 256);
+    off_b = o;      o += round_up(2 * groups * stride_b, 256);
+    total = o;
+  }
+};
+static inline bool mixed_weights(const tk_lora_desc& d) { return d.weights_f32 != 0 && d.dtype == TK_DTYPE_BF16; }
+static inline int64_t weight_stage_bytes(const tk_lora_desc& d) {
+  return mixed_weights(d) ? WeightStage(d.num_groups, rank_pad(d.max_rank), d.in_features, d.out_features).total : 0;
+}
+
 // Backward workspace carving.
 struct BwdLayout {
   int64_t off_dh, off_hpart, off_wT_shrink, off_wT_expand, off_part_a, off_part_b, total;
@@ -256,6 +277,7 @@ struct TransposeJob {
   int32_t y_blocks;  // 0: no job
   int32_t swizzle_a; // aT rows permuted inside every 128 (see PassArgs::expand_swizzled); in_features % 128 == 0
   int32_t skip_dead; // leave entries at and beyond a group's rank unwritten (the MFMA kernels never read them)
+  int32_t src_f32;   // lora_A / lora_B hold fp32 (lda, ldb in fp32 elements); the copies are bf16 all the same
 };
 
 // Row-contraction (weight gradient) pass: out_g[n][c] = sum_p hT[n][p] * src[row(p)][c].
@@ -271,6 +293,8 @@ struct WgradArgs {
   int32_t accumulate;
   int32_t map_rows;
   int32_t rpad;
+  int32_t grad_f32;    // the gradients (and the adapter weights a kernel reads next to them) are fp32 whatever the
+                       // element type of src (tk_lora_desc::weights_f32)
   TransposeJob tr;
 };
 
@@ -314,6 +338,8 @@ struct WgradReduceJobs {
   int32_t n;
   WgradArgs a[2 * kMaxShared];
 };
+// bf16 copies of the fp32 weights of `d` (layout: WeightStage at `stage`), with their pointer tables
+int launch_convert_weights(const tk_lora_desc& d, void* stage, bool want_a, bool want_b, hipStream_t s);
 int launch_transpose_job(const TransposeJob& t, const int32_t* rank, int rpad, hipStream_t s);
 int launch_dy_fused_multi(const DyFusedJob* jobs, int n, const SegView& seg, const SegLayout& L, hipStream_t s);
 int launch_pass_multi(const PassArgs* a, int n, const SegView& seg, const SegLayout& L, int phases, hipStream_t s);

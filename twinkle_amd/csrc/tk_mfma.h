@@ -91,6 +91,26 @@ __device__ inline void store_bf16x8(bf16_t* o, const float (&v)[8], int keep, bo
   }
 }
 
+// The same into an fp32 gradient: two 16-byte stores when `vec` (destination 16-byte aligned).
+__device__ inline void store_f32x8(float* o, const float (&v)[8], int keep, bool accumulate, bool vec) {
+  if (vec && keep >= 8) {
+    float4 lo = make_float4(v[0], v[1], v[2], v[3]), hi = make_float4(v[4], v[5], v[6], v[7]);
+    if (accumulate) {
+      const float4 a = *reinterpret_cast<const float4*>(o), b = *reinterpret_cast<const float4*>(o + 4);
+      lo.x += a.x; lo.y += a.y; lo.z += a.z; lo.w += a.w;
+      hi.x += b.x; hi.y += b.y; hi.z += b.z; hi.w += b.w;
+    }
+    *reinterpret_cast<float4*>(o) = lo;
+    *reinterpret_cast<float4*>(o + 4) = hi;
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    if (i >= keep) break;
+    o[i] = accumulate ? o[i] + v[i] : v[i];
+  }
+}
+
 // Blocks go to the XCDs (each with an L2 of its own) round-robin.  This renumbering gives every XCD one
 // contiguous eighth of the work items, so that an XCD's L2 fetches the weights of few groups instead of all.
 __device__ inline int xcd_contiguous(int block, int blocks) {
@@ -125,6 +145,35 @@ __device__ inline void wgrad_store(const f32x4 (&acc)[8][NB], float* lds, const 
     for (int i = 0; i < RP / 2; ++i) {
       const int n = 2 * i + (lane >> 5), c = 4 * (lane & 31);
       if (n < r) *reinterpret_cast<float4*>(part + (int64_t)n * a.width + c) = *reinterpret_cast<const float4*>(lds + n * OS + c);
+    }
+    return;
+  }
+  if (a.grad_f32) {  // fp32 gradients next to bf16 activations: the same two walks with fp32 stores
+    float* gf = (float*)a.grad[g];
+    const bool vecf = (reinterpret_cast<uintptr_t>(gf) & 15u) == 0 && (a.ld_grad & 3) == 0;
+    if (!a.transposed) {
+#pragma unroll
+      for (int i = 0; i < RP / 4; ++i) {
+        const int n = 4 * i + kb, c = 8 * li;
+        if (n >= r) continue;
+        const float4 lo = *reinterpret_cast<const float4*>(lds + n * OS + c);
+        const float4 hi = *reinterpret_cast<const float4*>(lds + n * OS + c + 4);
+        const float v8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        store_f32x8(gf + (int64_t)(n_base + n) * a.ld_grad + c0 + c, v8, 8, a.accumulate != 0, vecf);
+      }
+    } else {
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int c = lane + 64 * half;
+#pragma unroll
+        for (int n8 = 0; n8 < RP; n8 += 8) {
+          if (n8 >= r) break;
+          float v8[8];
+#pragma unroll
+          for (int i = 0; i < 8; ++i) v8[i] = lds[(n8 + i) * OS + c];
+          store_f32x8(gf + (int64_t)(c0 + c) * a.ld_grad + n_base + n8, v8, min(8, r - n8), a.accumulate != 0, vecf);
+        }
+      }
     }
     return;
   }

@@ -114,11 +114,17 @@ def _table_for(ml, rows: int, slot_index: int, device) -> SegmentTable:
     return table
 
 
-def _groups_for(ml, layer, only_slot: Union[None, str, Tuple[str, ...]]) -> Optional[AdapterGroups]:
+def _groups_for(ml, layer, only_slot: Union[None, str, Tuple[str, ...]],
+                x_dtype: Optional[torch.dtype] = None) -> Optional[AdapterGroups]:
     """Rank/scale table of a layer: slots whose tenant targets this layer are live, the rest rank 0.
-    ``only_slot`` narrows the live slots to one name or a tuple of names (``None``: every slot with a tenant)."""
+    ``only_slot`` narrows the live slots to one name or a tuple of names (``None``: every slot with a tenant).
+    ``x_dtype`` is the dtype of the activations the layer is called with: fp32 adapters under bf16 activations
+    (PEFT keeps adapters in fp32 under a bf16 base) run on the bf16 matrix-core kernels, which read the fp32
+    parameters where they are and write fp32 gradients, unless ``lora_compute_dtype=torch.float32`` asks for the
+    reference's arithmetic (activations cast to fp32, :320)."""
     cache = _path_state(ml).layer_groups
-    key = (id(layer), only_slot)
+    mixed = (x_dtype == torch.bfloat16 and getattr(ml, 'lora_compute_dtype', None) != torch.float32)
+    key = (id(layer), only_slot, mixed)
     owners = _ownership(ml)
     cached = cache.get(key)
     if cached is not None and cached[0] == owners:
@@ -139,13 +145,10 @@ def _groups_for(ml, layer, only_slot: Union[None, str, Tuple[str, ...]]) -> Opti
         else:
             ranks.append(0)
             scales.append(0.0)
-    compute_dtype = getattr(ml, 'lora_compute_dtype', None)
     if max(ranks) == 0:
         groups = None
-    elif compute_dtype is not None and a[0].dtype != compute_dtype:
-        groups = AdapterGroups([torch.empty_like(t, dtype=compute_dtype) for t in a],
-                               [torch.empty_like(t, dtype=compute_dtype) for t in b], ranks, scales, master_a=a,
-                               master_b=b)
+    elif mixed and a[0].dtype == torch.float32:
+        groups = AdapterGroups(a, b, ranks, scales, act_dtype=torch.bfloat16)
     else:
         groups = AdapterGroups(a, b, ranks, scales)
     if len(cache) > 8192:   # batches over ever-changing tenant sets: start over
@@ -267,7 +270,7 @@ def forward_shared(ml, layers: Sequence, x: torch.Tensor) -> Tuple[torch.Tensor,
                 break
             only_slot = slot
         groups = None if layer.disable_adapters else _groups_for(
-            ml, layer, only_slot if table is None else getattr(table, 'live_slots', None))
+            ml, layer, only_slot if table is None else getattr(table, 'live_slots', None), x.dtype)
         base = layer.base_layer
         if (groups is None or groups.dtype != x.dtype or type(base) is not torch.nn.Linear
                 or base.weight.dtype != x.dtype or base._forward_hooks or base._forward_pre_hooks
@@ -277,8 +280,6 @@ def forward_shared(ml, layers: Sequence, x: torch.Tensor) -> Tuple[torch.Tensor,
         groups_list.append(groups)
     if not ok:
         return tuple(getattr(layer, '_tk_forward_one', layer)(x) for layer in layers)
-    for groups in groups_list:
-        groups.sync_masters()
     x2 = x.reshape(-1, x.shape[-1])
     if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
         x2 = x2.contiguous()
@@ -297,11 +298,11 @@ class MultiLora:
         self.max_loras = max_loras
         self.max_r = max_r
         self.max_length = max_length
-        # Adapter weights kept in fp32 under a bf16 base model (what PEFT's adapter autocast produces): by default
-        # the activations are cast to the adapters' dtype like in the reference (:320) and the fp32 kernels run.
-        # With lora_compute_dtype=torch.bfloat16 the kernels instead read bf16 copies of the adapter weights,
-        # refreshed from the fp32 masters at every forward, and the gradients come back in fp32: the bf16 kernels'
-        # speed (13x at the Llama-3-8B projection shape) at bf16 accuracy.
+        # Adapter weights kept in fp32 under a bf16 base model (what PEFT's adapter autocast produces): the bf16
+        # matrix-core kernels run, reading the fp32 parameters where they are (converted on the fly inside the
+        # library, no copies kept on this side) and writing fp32 gradients: the bf16 kernels' speed at bf16
+        # accuracy of the LoRA term.  lora_compute_dtype=torch.float32 instead casts the activations to fp32 like
+        # the reference (:320) and runs the fp32 kernels.
         self.lora_compute_dtype = lora_compute_dtype
         self.loras: List[LoraTenant] = []
         self.module = None
@@ -453,8 +454,8 @@ class MultiLora:
         return _path_state(self).batch_table
 
     # ------------------------------------------------------------- patching
-    def _groups_for(self, layer, only_slot=None) -> Optional[AdapterGroups]:
-        return _groups_for(self, layer, only_slot)
+    def _groups_for(self, layer, only_slot=None, x_dtype=None) -> Optional[AdapterGroups]:
+        return _groups_for(self, layer, only_slot, x_dtype)
 
     def _patch_lora_forward(_self, name, base_layer):
         """Rebind ``forward`` on one LoRA layer (reference :289-331, Linear branch)."""
@@ -499,12 +500,11 @@ class MultiLora:
                 only_slot = forced_slot if forced_slot is not None else (active[0] if active else None)
             skip = self.disable_adapters or (table is None and only_slot is None)
             groups = None if skip else _groups_for(
-                _self, self, only_slot if table is None else getattr(table, 'live_slots', None))
+                _self, self, only_slot if table is None else getattr(table, 'live_slots', None), x.dtype)
             if groups is None:
                 return self.base_layer(x, *args, **kwargs) if onto is None else onto
-            groups.sync_masters()
 
-            wdtype = groups.dtype
+            wdtype = groups.dtype    # what the kernels take as activations: the adapters' dtype, or bf16 (see _groups_for)
             xw = self._cast_input_dtype(x, wdtype)
             xw = _slot_dropout(_self, self, only_slot, table)(xw)
             x2 = xw.reshape(-1, xw.shape[-1])

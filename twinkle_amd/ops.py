@@ -30,7 +30,7 @@ class AdapterGroups:
                  scales: Sequence[float], a_index: Optional[Sequence[int]] = None,
                  a_offset: Optional[Sequence[int]] = None, b_index: Optional[Sequence[int]] = None,
                  b_offset: Optional[Sequence[int]] = None, master_a: Optional[Sequence[torch.Tensor]] = None,
-                 master_b: Optional[Sequence[torch.Tensor]] = None):
+                 master_b: Optional[Sequence[torch.Tensor]] = None, act_dtype: Optional[torch.dtype] = None):
         self.a_tensors = list(a_tensors)
         self.b_tensors = list(b_tensors)
         # mixed precision: the kernels read `a_tensors` / `b_tensors` (compute copies, e.g. bf16) while the
@@ -56,17 +56,25 @@ class AdapterGroups:
                 == g):
             raise ValueError('per-group lists must have one entry per group')
         a0, b0 = self.a_tensors[0], self.b_tensors[0]
-        self.dtype = a0.dtype
+        # `dtype` is the element type of x, y and h; the adapters' own type differs from it in one supported case:
+        # fp32 adapters under bf16 activations (tk_lora_desc::weights_f32: the library converts the weights on the
+        # fly and writes fp32 gradients)
+        self.weight_dtype = a0.dtype
+        self.dtype = act_dtype if act_dtype is not None else a0.dtype
+        if self.dtype != self.weight_dtype and (self.dtype, self.weight_dtype) != (torch.bfloat16, torch.float32):
+            raise ValueError(f'adapters of {self.weight_dtype} under activations of {self.dtype} are not supported')
+        self.weights_f32 = self.dtype != self.weight_dtype
         self.device = a0.device
         self.in_features = a0.shape[-1]
         self.out_features = b0.shape[-2]
         self.lda = a0.stride(-2)
         self.ldb = b0.stride(-2)
         for t in self.a_tensors:
-            if t.dtype != self.dtype or t.shape[-1] != self.in_features or t.stride(-1) != 1 or t.stride(-2) != self.lda:
+            if t.dtype != self.weight_dtype or t.shape[-1] != self.in_features or t.stride(-1) != 1 or \
+                    t.stride(-2) != self.lda:
                 raise ValueError('all lora_A tensors of a layer must share dtype, width and row stride')
         for t in self.b_tensors:
-            if t.dtype != self.dtype or t.shape[-2] != self.out_features or t.stride(-1) != 1 or \
+            if t.dtype != self.weight_dtype or t.shape[-2] != self.out_features or t.stride(-1) != 1 or \
                     t.stride(-2) != self.ldb:
                 raise ValueError('all lora_B tensors of a layer must share dtype, height and row stride')
         self.max_rank = max(self.ranks)
@@ -162,6 +170,7 @@ def _desc(seg: SegmentTable, groups: AdapterGroups, map_rows: bool) -> _lib.Lora
         template.ldb = groups.ldb
         template.rank = groups.rank_dev.data_ptr()
         template.scale = groups.scale_dev.data_ptr()
+        template.weights_f32 = 1 if groups.weights_f32 else 0
         groups._desc_template, groups._desc_key = template, groups._ptr_key
     d = _lib.LoraDesc.from_buffer_copy(template)
     d.rows = seg.rows
@@ -331,10 +340,10 @@ def _weight_grads(ctx_groups: AdapterGroups, needs_a: bool, needs_b: bool, devic
     groups = ctx_groups
     arena_a = arena_b = pa = pb = None
     if needs_a:
-        arena_a = torch.zeros(groups.a_arena_elems, dtype=groups.dtype, device=device)
+        arena_a = torch.zeros(groups.a_arena_elems, dtype=groups.weight_dtype, device=device)
         pa = groups._grad_a_rel + arena_a.data_ptr()
     if needs_b:
-        arena_b = torch.zeros(groups.b_arena_elems, dtype=groups.dtype, device=device)
+        arena_b = torch.zeros(groups.b_arena_elems, dtype=groups.weight_dtype, device=device)
         pb = groups._grad_b_rel + arena_b.data_ptr()
     return arena_a, arena_b, pa, pb
 
