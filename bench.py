@@ -27,17 +27,47 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
+TRAFFIC_PROFILE = os.path.join('profiles', 'bench_cfg2_hbm_traffic_pmc.txt')
+KERNEL_SOURCES = ('kernels_mfma.hip', 'tk_mfma.h', 'tk_common.h')     # what the expand kernel is compiled from
+
+
+def kernel_source_digest():
+    """sha256 over the sources of the dominant kernel, as the traffic profile records it when it is taken."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, 'twinkle_amd', 'csrc', name), 'rb') as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
 def measured_traffic(kernel):
-    """HBM bytes per launch of `kernel` from the committed rocprofv3 --pmc summary (None if it is not there)."""
-    path = os.path.join(ROOT, 'profiles', 'bench_cfg2_hbm_traffic_pmc.txt')
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 --pmc summary, with where it comes from.
+
+    The counters need a profiler pass of their own, so a plain run cannot measure them; the committed summary
+    records the digest of the kernel's sources it was taken with, and the number is only reported while those
+    sources are unchanged (otherwise ``traffic`` is null and the note says why)."""
+    value = digest = commit = None
     try:
-        with open(path) as f:
+        with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as f:
             for line in f:
                 if line.startswith(f'traffic_bytes_per_launch[{kernel}]:'):
-                    return float(line.split(':')[1])
+                    value = float(line.split(':')[1])
+                elif line.startswith('kernel_source_sha256:'):
+                    digest = line.split(':')[1].strip()
+                elif line.startswith('source_commit:'):
+                    commit = line.split(':')[1].strip()
     except OSError:
-        pass
-    return None
+        return None, {'profile': TRAFFIC_PROFILE, 'note': 'profile not found'}
+    source = {'profile': TRAFFIC_PROFILE, 'source_commit': commit, 'kernel_source_sha256': digest}
+    try:
+        current = kernel_source_digest()
+    except OSError:
+        current = None
+    if value is None or digest is None or digest != current:
+        source['note'] = 'kernel sources changed since the profile was taken: traffic not reported'
+        return None, source
+    return value, source
 
 
 def cpu_baseline(w, budget_s=15.0):
@@ -696,7 +726,7 @@ def main():
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
-    every = max(1, args.event_every)
+    every = 1 if args.steps <= 20 else max(1, args.event_every)     # short runs: events around every step
     events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] if i % every == 0 else None
               for i in range(args.steps)]
     torch.cuda.synchronize()
@@ -735,6 +765,9 @@ def main():
     expand_bytes = elt * T * 2 * M + elt * sum(r * M for r in w.ranks)
     flops = w.flops()
     achieved = expand_bytes / (expand_ms * 1e-3) / 1e9
+    traffic, traffic_source = (None, None)
+    if args.workload == 'cfg2' and not args.tokens and not args.weights_f32:
+        traffic, traffic_source = measured_traffic('k_expand_mfma<1>')
     out = {
         'metric': 'multi-LoRA fwd+bwd tokens/s + % roofline (HBM/MFMA), 8B proj, 16 adapters',
         'value': T / (ms_per_step * 1e-3),
@@ -753,7 +786,7 @@ def main():
                                '; step = segment build + LoRA fwd + LoRA bwd (dX, dA, dB); base GEMM excluded',
                    'tokens': T, 'in': K, 'out': M, 'adapters': G, 'rank': max(w.ranks)},
         'roofline': {'bound': 'hbm', 'achieved': achieved, 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                     'frac': achieved / HBM_PEAK_GBS, 'traffic': measured_traffic('k_expand_mfma<1>') if args.workload == 'cfg2' and not args.tokens else None,
+                     'frac': achieved / HBM_PEAK_GBS, 'traffic': traffic, 'traffic_source': traffic_source,
                      'kernel': ('k_expand_mfma<1>' if max(w.ranks) <= 16 else
                                 f'k_expand_multi<{2 if max(w.ranks) <= 32 else 4},4>') + ' (y += h B^T in place), forward launch',
                      'algorithmic_bytes_per_launch': expand_bytes, 'avg_launch_ms': expand_ms,
