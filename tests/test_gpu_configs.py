@@ -11,18 +11,20 @@ from twinkle_amd import packed_cu_seqlens, token_groups_from_sequences, workload
 pytestmark = pytest.mark.gpu
 
 
-def _device_problem(w, dev):
+def _device_problem(w, dev, weights_f32=False):
     dt = torch.bfloat16
-    a = [t.to(dt).to(dev) for t in w.lora_A]
-    b = [t.to(dt).to(dev) for t in w.lora_B]
+    wdt = torch.float32 if weights_f32 else dt     # fp32 adapters under bf16 activations: tk_lora_desc::weights_f32
+    a = [t.to(wdt).to(dev) for t in w.lora_A]
+    b = [t.to(wdt).to(dev) for t in w.lora_B]
     seg = build_segments(w.ids.to(dev), w.num_adapters, check=True)
-    return a, b, seg, AdapterGroups(a, b, w.ranks, w.scales)
+    return a, b, seg, AdapterGroups(a, b, w.ranks, w.scales, act_dtype=dt)
 
 
-def _check_sampled(w, dev, sample_groups, sample_rows=64):
-    """Forward/backward at full size; Y and dX on sampled rows, dA/dB of sampled adapters, against float64."""
+def _check_sampled(w, dev, sample_groups, sample_rows=64, weights_f32=False):
+    """Forward/backward at full size; Y and dX on sampled rows, dA/dB of sampled adapters, against float64
+    (with ``weights_f32`` on the unrounded fp32 weights, and the gradients must come back as fp32)."""
     dt = torch.bfloat16
-    a, b, seg, groups = _device_problem(w, dev)
+    a, b, seg, groups = _device_problem(w, dev, weights_f32)
     x = w.x.to(dt).to(dev)
     y = w.base_out.to(dt).to(dev)
     dy = w.dy.to(dt).to(dev)
@@ -36,11 +38,13 @@ def _check_sampled(w, dev, sample_groups, sample_rows=64):
     dx = torch.zeros_like(x)
     lora_bwd_(dy, x, h, dx, pa, pb, seg, groups, accumulate=False)
     f64 = lambda t: t.to(dt).double()  # noqa: E731
+    w64 = (lambda t: t.float().double()) if weights_f32 else f64  # noqa: E731
+    assert all(t.dtype == (torch.float32 if weights_f32 else dt) for t in ga + gb)
     counts = torch.bincount(w.ids.long(), minlength=w.num_adapters)
     for g in sample_groups:
         r, s = w.ranks[g], w.scales[g]
         rows = (w.ids == g).nonzero().flatten()
-        ag, bg = f64(w.lora_A[g])[:r], f64(w.lora_B[g])[:, :r]
+        ag, bg = w64(w.lora_A[g])[:r], w64(w.lora_B[g])[:, :r]
         if rows.numel() == 0:
             assert torch.count_nonzero(ga[g][:r]) == 0 and torch.count_nonzero(gb[g][:, :r]) == 0
             continue
@@ -63,6 +67,69 @@ def test_config3_mixed_ranks_full_size(dev, direction):
     w = workloads.config3_mlp(direction)
     assert int((w.ids == 5).sum()) == 0 and int((w.ids == 17).sum()) == 0
     _check_sampled(w, dev, sample_groups=[0, 3, 5, 9, 17, 22, 31])
+
+
+def test_config2_fp32_adapters_full_size(dev):
+    """BASELINE config 2 with PEFT-style fp32 adapters under the bf16 activations: every adapter, at full size."""
+    w = workloads.config2_qproj()
+    _check_sampled(w, dev, sample_groups=list(range(w.num_adapters)), weights_f32=True)
+
+
+def test_config5_qkv_shared_inputs_rank64_full_size(dev):
+    """q / k / v of one config-5 layer (4096 -> 4096, 1024, 1024; T = 32768, 8 tenants of rank 64, one per packed
+    sequence) through the shared-input entry points: y, dA, dB equal to one call per projection bit for bit, dX
+    (one rounding of the sum over the projections) against float64 on sampled rows."""
+    from twinkle_amd import lora_bwd_shared_, lora_fwd_shared_
+    dt, t, k, n, r = torch.bfloat16, 32768, 4096, 8, 64
+    outs = (4096, 1024, 1024)
+    g = torch.Generator().manual_seed(21)
+    ids = torch.repeat_interleave(torch.arange(n, dtype=torch.int32), t // n)
+    x = torch.randn(t, k, generator=g).to(dt)
+    seg = build_segments(ids.to(dev), n, check=True)
+    xd = x.to(dev)
+    a_all, b_all, dys, groups = [], [], [], []
+    for m in outs:
+        a = [((torch.rand(r, k, generator=g) * 2 - 1) / 64).to(dt) for _ in range(n)]
+        b = [(torch.randn(m, r, generator=g) * 0.02).to(dt) for _ in range(n)]
+        a_all.append(a)
+        b_all.append(b)
+        dys.append(torch.randn(t, m, generator=g).to(dt))
+        groups.append(AdapterGroups([w.to(dev) for w in a], [w.to(dev) for w in b], [r] * n, [2.0] * n))
+
+    def grads():
+        ga = [[torch.zeros(r, k, dtype=dt, device=dev) for _ in range(n)] for _ in outs]
+        gb = [[torch.zeros(m, r, dtype=dt, device=dev) for _ in range(n)] for m in outs]
+        pa = [torch.tensor([w.data_ptr() for w in ws], dtype=torch.int64, device=dev) for ws in ga]
+        pb = [torch.tensor([w.data_ptr() for w in ws], dtype=torch.int64, device=dev) for ws in gb]
+        return ga, gb, pa, pb
+
+    # one call per projection
+    ys = [torch.zeros(t, m, dtype=dt, device=dev) for m in outs]
+    ga1, gb1, pa1, pb1 = grads()
+    dx1 = torch.zeros(t, k, dtype=dt, device=dev)
+    for p in range(3):
+        h = lora_fwd_(xd, ys[p], seg, groups[p])
+        lora_bwd_(dys[p].to(dev), xd, h, dx1, pa1[p], pb1[p], seg, groups[p])
+    # all three at once
+    yj = [torch.zeros(t, m, dtype=dt, device=dev) for m in outs]
+    ga2, gb2, pa2, pb2 = grads()
+    dx2 = torch.zeros(t, k, dtype=dt, device=dev)
+    hs = lora_fwd_shared_(xd, yj, seg, groups)
+    lora_bwd_shared_([d.to(dev) for d in dys], xd, hs, dx2, pa2, pb2, seg, groups)
+    for p in range(3):
+        assert torch.equal(yj[p], ys[p]), f'y[{p}]'
+        for i in range(n):
+            assert torch.equal(ga2[p][i], ga1[p][i]) and torch.equal(gb2[p][i], gb1[p][i]), f'gradients of {p}, {i}'
+    for tenant in (0, 5):
+        rows = (ids == tenant).nonzero().flatten()[:48]
+        want = torch.zeros(rows.numel(), k, dtype=torch.float64)
+        for p in range(3):
+            dh = 2.0 * dys[p][rows].double() @ b_all[p][tenant].double()
+            want += dh @ a_all[p][tenant].double()
+            yo = (2.0 * x[rows].double() @ a_all[p][tenant].double().t()) @ b_all[p][tenant].double().t()
+            assert max_rel_err(yj[p][rows.to(dev)], yo) < 2e-2
+        assert max_rel_err(dx2[rows.to(dev)], want) < 2e-2, 'dX of the shared call'
+        assert max_rel_err(dx1[rows.to(dev)], want) < 2e-2, 'dX of the separate calls'
 
 
 def test_config3_linearity_and_repeatability(dev):
