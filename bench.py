@@ -11,7 +11,9 @@ one full step earlier).
 
 Prints one JSON line (see the keys below).  `roofline` describes the dominant kernel, the expand
 kernel (y += h B^T, a read-modify-write of the whole output), on its forward launches: algorithmic
-bytes of one launch over its mean duration between HIP events on the launch stream.
+bytes of one launch over its mean duration between HIP events on the launch stream.  The `steps` timed steps
+behind `value` carry no events (an event record idles the queue for a few microseconds); the same steps are then run
+once more with events around the kernels of every step, and those launches are the ones `roofline` averages.
 """
 import argparse
 import json
@@ -590,9 +592,6 @@ def main():
     ap.add_argument('--warmup', type=int, default=10)
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--sets', type=int, default=3, help='rotated buffer sets')
-    ap.add_argument('--event-every', type=int, default=4,
-                    help='bracket the kernels with HIP events on every n-th timed step (an event record costs a few '
-                         'microseconds of idle queue, so not every step carries them)')
     ap.add_argument('--workload', default='cfg2', choices=['cfg2', 'cfg3_up', 'cfg3_down', 'cfg5_q', 'cfg4_gate_up'],
                     help='cfg2 is the headline configuration; the others are the wider BASELINE shapes '
                          '(cfg3: 4096<->14336, T=32768, 32 adapters of rank 8..64; cfg5_q: 4096->4096, T=32768, 8 tenants '
@@ -726,17 +725,24 @@ def main():
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
-    every = 1 if args.steps <= 20 else max(1, args.event_every)     # short runs: events around every step
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] if i % every == 0 else None
-              for i in range(args.steps)]
+    # First timed region: exactly `steps` steps with nothing but the step's own launches on the stream -> ms_per_step.
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(i, events[i])
+        step(i)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
-    events = [e for e in events if e is not None]
+    # Second timed region: the same `steps` steps again with HIP events around the kernels of every step (on the
+    # launch stream).  An event record costs a few microseconds of idle queue, which is why these steps are not the
+    # ones behind `value`; their own rate is reported as ms_per_step_with_events.
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for i in range(args.steps):
+        step(args.steps + i, events[i])
+    torch.cuda.synchronize()
+    ms_per_step_with_events = (time.perf_counter() - t1) * 1e3 / args.steps
     shrink_ms = sum(e[0].elapsed_time(e[1]) for e in events) / len(events)
     expand_ms = sum(e[1].elapsed_time(e[2]) for e in events) / len(events)
     fwd_ms = shrink_ms + expand_ms
@@ -791,7 +797,7 @@ def main():
                                 f'k_expand_multi<{2 if max(w.ranks) <= 32 else 4},4>') + ' (y += h B^T in place), forward launch',
                      'algorithmic_bytes_per_launch': expand_bytes, 'avg_launch_ms': expand_ms,
                      'launches_timed': len(events)},
-        'step_detail': {'shrink_ms': shrink_ms, 'expand_ms': expand_ms, 'fwd_ms': fwd_ms, 'bwd_ms': bwd_ms, 'segment_build_and_gaps_ms': ms_per_step - fwd_ms - bwd_ms,
+        'step_detail': {'ms_per_step_with_events': ms_per_step_with_events, 'shrink_ms': shrink_ms, 'expand_ms': expand_ms, 'fwd_ms': fwd_ms, 'bwd_ms': bwd_ms, 'segment_build_and_gaps_ms': ms_per_step_with_events - fwd_ms - bwd_ms,
                         'algorithmic_bytes_per_step': step_bytes, 'flops_per_step': flops,
                         'tflops': flops / (ms_per_step * 1e-3) / 1e12,
                         'hbm_frac_step': step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
