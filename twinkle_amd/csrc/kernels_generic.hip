@@ -176,7 +176,7 @@ __global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkI
         const int n = n0 + j;
         if (n < r) {
           if (ci.partial >= 0)
-            a.partial[((int64_t)ci.partial * a.rpad + n) * a.width + c] = acc[j];
+            a.partial[partial_index(ci.partial, n, c, a.rpad, a.width)] = acc[j];
           else
             store_grad<T>(a, g, n, c, acc[j]);
         }
@@ -205,8 +205,8 @@ __device__ __forceinline__ void wgrad_reduce_body(const WgradArgs& a, int n0, co
   if (nchunk == 0 && a.accumulate) return;
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= a.width) return;
-  const float* p = a.partial + ((int64_t)pf * a.rpad + n0) * a.width + c;
-  const int64_t stride = (int64_t)a.rpad * a.width;
+  const float* p = a.partial + partial_index(pf, n0, c, a.rpad, a.width);
+  const int64_t stride = partial_slot_floats(a.rpad, a.width);
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
@@ -217,7 +217,7 @@ __device__ __forceinline__ void wgrad_reduce_body(const WgradArgs& a, int n0, co
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-        v[j][i] = (j0 + j < nchunk && n0 + i < r) ? p[(j0 + j) * stride + (int64_t)i * a.width] : 0.f;
+        v[j][i] = (j0 + j < nchunk && n0 + i < r) ? p[(j0 + j) * stride + i * 128] : 0.f;
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll

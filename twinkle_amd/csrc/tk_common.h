@@ -59,6 +59,19 @@ static inline int chunk_tiles_for(int64_t rows) {
   return t;
 }
 
+// Element (partial slot p, rank index n, column c) of a weight-gradient partial buffer.  Blocks of 128 columns are
+// contiguous, [slot][column block][rpad][128]: a launch block leaves its rpad x 128 sums as one run of memory and
+// the reduction reads runs of KBs, instead of 512-byte pieces a whole row of the gradient apart.
+#ifdef __HIPCC__
+#define TK_HD __host__ __device__
+#else
+#define TK_HD
+#endif
+TK_HD static inline int64_t partial_slot_floats(int rpad, int width) { return (int64_t)((width + 127) >> 7) * rpad * 128; }
+TK_HD static inline int64_t partial_index(int64_t p, int n, int c, int rpad, int width) {
+  return (((p * ((width + 127) >> 7) + (c >> 7)) * rpad + n) << 7) + (c & 127);
+}
+
 struct SegLayout {
   int64_t rows, groups;
   int64_t sort_blocks;   // ceil(rows / kSortBlockRows)
@@ -233,8 +246,8 @@ struct BwdLayout {
     off_wT_shrink = o;  o += round_up((int64_t)d.num_groups * rpad * d.out_features * e, 256);
     // A^T per group [K][rpad]  (expand weight of the backward pass)
     off_wT_expand = o;  o += round_up((int64_t)d.num_groups * rpad * d.in_features * e, 256);
-    off_part_a = o;     o += round_up(S.max_partials * rpad * (int64_t)d.in_features * 4, 256);
-    off_part_b = o;     o += round_up(S.max_partials * rpad * (int64_t)d.out_features * 4, 256);
+    off_part_a = o;     o += round_up(S.max_partials * rpad * round_up(d.in_features, 128) * 4, 256);
+    off_part_b = o;     o += round_up(S.max_partials * rpad * round_up(d.out_features, 128) * 4, 256);
     total = o;
   }
 };
@@ -284,7 +297,7 @@ struct TransposeJob {
 struct WgradArgs {
   const void* src;  int64_t ld_src;   // x | dy
   const void* hT;   int64_t ldh;      // dh | h
-  float* partial;                     // [max_partials][rpad][width]
+  float* partial;                     // [max_partials][width / 128][rpad][128], see partial_index
   void* const* grad;                  // device array [G]
   int64_t ld_grad;
   const int32_t* rank;

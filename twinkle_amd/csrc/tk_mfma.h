@@ -140,11 +140,11 @@ __device__ inline void wgrad_store(const f32x4 (&acc)[8][NB], float* lds, const 
   __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
 
   if (ci.partial >= 0) {
-    float* part = a.partial + ((int64_t)ci.partial * a.rpad + n_base) * a.width + c0;
+    float* part = a.partial + partial_index(ci.partial, n_base, c0, a.rpad, a.width);  // c0 is a multiple of 128
 #pragma unroll
     for (int i = 0; i < RP / 2; ++i) {
       const int n = 2 * i + (lane >> 5), c = 4 * (lane & 31);
-      if (n < r) *reinterpret_cast<float4*>(part + (int64_t)n * a.width + c) = *reinterpret_cast<const float4*>(lds + n * OS + c);
+      if (n < r) *reinterpret_cast<float4*>(part + n * 128 + c) = *reinterpret_cast<const float4*>(lds + n * OS + c);
     }
     return;
   }
