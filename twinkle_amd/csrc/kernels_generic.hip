@@ -199,14 +199,76 @@ __device__ __forceinline__ void wgrad_reduce_body(const WgradArgs& a, int n0, co
   // independent loads first
   const int rk = a.rank[g], cf0 = chunk_first[g], cf1 = chunk_first[g + 1], pf = partial_first[g];
   const int r = min(rk, a.rpad);
-  if (n0 >= r) return;
   const int nchunk = cf1 - cf0;
   if (nchunk == 1) return;
   if (nchunk == 0 && a.accumulate) return;
+  const int64_t stride = partial_slot_floats(a.rpad, a.width);
+  T* const gt = (T*)a.grad[g];
+  if (sizeof(T) == 2 && a.transposed && (a.ld_grad & 7) == 0 && (reinterpret_cast<uintptr_t>(gt) & 15u) == 0 &&
+      (r & 7) == 0) {
+    // A transposed gradient ([width][r], dB) whose rows are whole 16-byte pieces.  With a thread per column and an
+    // octet of rank indices per block every 128-byte line of it was written in up to eight partial stores from eight
+    // blocks (measured at 14336 columns, rank 64: 40 of the kernel's 79 us).  Here a block owns all octets of its
+    // columns: it reads the partial sums with neighbouring threads on neighbouring columns (whole lines of the
+    // partial buffer), turns the sums over in LDS and writes with neighbouring threads on neighbouring octets,
+    // i.e. whole rows of the gradient.  The blocks of a group are renumbered: block (y, octet z) takes the columns
+    // [b cpb, b cpb + cpb), b = y * (rpad / 8) + z, cpb = 256 / octets per column.
+    __shared__ __attribute__((aligned(16))) float turn[256 * 8];
+    if (r == 0) return;
+    int noct = 1;
+    while (8 * noct < r) noct <<= 1;  // octets per column, padded to a power of two
+    const int cpb = 256 / noct, tid = threadIdx.x;
+    const int col0 = (blockIdx.y * (a.rpad >> 3) + (n0 >> 3)) * cpb;
+    if (col0 >= a.width) return;  // (block-uniform, like every return above)
+    {
+      const int oct = tid / cpb, cl = tid % cpb, c = col0 + cl;
+      float acc[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+      if (c < a.width && 8 * oct < r) {
+        const float* p = a.partial + partial_index(pf, 8 * oct, c, a.rpad, a.width);
+        for (int j0 = 0; j0 < nchunk; j0 += 2) {
+          float v[2][8];
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[j][i] = j0 + j < nchunk ? p[(j0 + j) * stride + i * 128] : 0.f;
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] += v[j][i];
+        }
+      }
+      float4* o = reinterpret_cast<float4*>(turn + (cl * noct + oct) * 8);
+      o[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+      o[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+    }
+    __syncthreads();
+    const int oct = tid & (noct - 1), c = col0 + tid / noct;
+    if (c >= a.width || 8 * oct >= r) return;
+    const float4 lo = *reinterpret_cast<const float4*>(turn + tid * 8), hi = *reinterpret_cast<const float4*>(turn + tid * 8 + 4);
+    float acc[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    uint4* o = reinterpret_cast<uint4*>(gt + (int64_t)c * a.ld_grad + 8 * oct);
+    if (a.accumulate) {
+      const uint4 old = *o;
+      const uint32_t w[4] = {old.x, old.y, old.z, old.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[2 * i] += __uint_as_float(w[i] << 16);
+        acc[2 * i + 1] += __uint_as_float(w[i] & 0xffff0000u);
+      }
+    }
+    uint16_t h[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) from_f32(acc[i], &h[i]);
+    *o = make_uint4(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16), h[4] | ((uint32_t)h[5] << 16),
+                    h[6] | ((uint32_t)h[7] << 16));
+    return;
+  }
+  if (n0 >= r) return;
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= a.width) return;
   const float* p = a.partial + partial_index(pf, n0, c, a.rpad, a.width);
-  const int64_t stride = partial_slot_floats(a.rpad, a.width);
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
