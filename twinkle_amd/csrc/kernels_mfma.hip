@@ -743,7 +743,7 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
                                              int64_t thread, int64_t threads) {
   const int m8 = t.out_features >> 3, n8 = rpad >> 3, k8 = t.in_features >> 3;
   const int64_t units_b = t.bT ? (int64_t)t.groups * m8 * n8 : 0;  // (g, m-octet, n-octet), n-octet fastest
-  const int64_t units_a = (int64_t)t.groups * n8 * k8;              // (g, n-octet, k-octet), k-octet fastest
+  const int64_t units_a = (int64_t)t.groups * n8 * k8;              // (g, k-octet, n-octet), n-octet fastest
   const bool f32 = t.src_f32 != 0;
   const int ld_mask = f32 ? 3 : 7;  // row strides that keep every row 16-byte aligned
   for (int64_t u = thread; u < units_b + units_a; u += threads) {
@@ -778,10 +778,13 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
         if (8 * no + j < r || !t.skip_dead) st16(o + (int64_t)j * t.out_features, out[j]);
     } else {
       // aT[g][k][n] = A_g[n][k]: rows n of A hold the input features contiguously
+      // rank octet fastest: the threads that hold the octets of one column of A are neighbours, so a wave-wide
+      // store covers whole rows of the copy (a row is rpad elements), and a wave-wide load still covers 128-byte
+      // runs of A's rows (eight neighbouring column octets per rank octet)
       const int64_t v = u - units_b;
-      const int ko = (int)(v % k8);
-      const int64_t q = v / k8;
-      const int no = (int)(q % n8), g = (int)(q / n8);
+      const int no = (int)(v % n8);
+      const int64_t q = v / n8;
+      const int ko = (int)(q % k8), g = (int)(q / k8);
       const int r = min(rank[g], rpad);
       if (8 * no >= r && t.skip_dead) continue;
       const void* A = t.lora_A[g];
