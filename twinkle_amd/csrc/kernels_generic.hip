@@ -204,7 +204,7 @@ __device__ __forceinline__ void wgrad_reduce_body(const WgradArgs& a, int n0, co
   if (nchunk == 0 && a.accumulate) return;
   const int64_t stride = partial_slot_floats(a.rpad, a.width);
   T* const gt = (T*)a.grad[g];
-  if (sizeof(T) == 2 && a.transposed && (a.ld_grad & 7) == 0 && (reinterpret_cast<uintptr_t>(gt) & 15u) == 0 &&
+  if (a.transposed && (a.ld_grad & (sizeof(T) == 2 ? 7 : 3)) == 0 && (reinterpret_cast<uintptr_t>(gt) & 15u) == 0 &&
       (r & 7) == 0) {
     // A transposed gradient ([width][r], dB) whose rows are whole 16-byte pieces.  With a thread per column and an
     // octet of rank indices per block every 128-byte line of it was written in up to eight partial stores from eight
@@ -248,6 +248,17 @@ __device__ __forceinline__ void wgrad_reduce_body(const WgradArgs& a, int n0, co
     if (c >= a.width || 8 * oct >= r) return;
     const float4 lo = *reinterpret_cast<const float4*>(turn + tid * 8), hi = *reinterpret_cast<const float4*>(turn + tid * 8 + 4);
     float acc[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    if constexpr (sizeof(T) == 4) {  // fp32 gradient: the octet is two 16-byte pieces
+      float4* of = reinterpret_cast<float4*>(gt + (int64_t)c * a.ld_grad + 8 * oct);
+      if (a.accumulate) {
+        const float4 o0 = of[0], o1 = of[1];
+        acc[0] += o0.x; acc[1] += o0.y; acc[2] += o0.z; acc[3] += o0.w;
+        acc[4] += o1.x; acc[5] += o1.y; acc[6] += o1.z; acc[7] += o1.w;
+      }
+      of[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+      of[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+      return;
+    }
     uint4* o = reinterpret_cast<uint4*>(gt + (int64_t)c * a.ld_grad + 8 * oct);
     if (a.accumulate) {
       const uint4 old = *o;
