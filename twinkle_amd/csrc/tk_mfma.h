@@ -162,17 +162,16 @@ __device__ inline void wgrad_store(const f32x4 (&acc)[8][NB], float* lds, const 
         store_f32x8(gf + (int64_t)(n_base + n) * a.ld_grad + c0 + c, v8, 8, a.accumulate != 0, vecf);
       }
     } else {
+      // grad[c0 + c][n]: neighbouring lanes take neighbouring rank octets of one column, so that a wave-wide store
+      // covers runs of whole rows of the gradient instead of one 16-byte (32-byte) piece of each of 64 rows
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        const int c = lane + 64 * half;
+      for (int k = 0; k < RP / 4; ++k) {
+        const int piece = lane + 64 * k, c = piece / (RP / 8), n8 = 8 * (piece % (RP / 8));
+        if (n8 >= r) continue;
+        float v8[8];
 #pragma unroll
-        for (int n8 = 0; n8 < RP; n8 += 8) {
-          if (n8 >= r) break;
-          float v8[8];
-#pragma unroll
-          for (int i = 0; i < 8; ++i) v8[i] = lds[(n8 + i) * OS + c];
-          store_f32x8(gf + (int64_t)(c0 + c) * a.ld_grad + n_base + n8, v8, min(8, r - n8), a.accumulate != 0, vecf);
-        }
+        for (int i = 0; i < 8; ++i) v8[i] = lds[(n8 + i) * OS + c];
+        store_f32x8(gf + (int64_t)(c0 + c) * a.ld_grad + n_base + n8, v8, min(8, r - n8), a.accumulate != 0, vecf);
       }
     }
     return;
@@ -191,18 +190,15 @@ __device__ inline void wgrad_store(const f32x4 (&acc)[8][NB], float* lds, const 
       store_bf16x8(gp + (int64_t)(n_base + n) * a.ld_grad + c0 + c, v8, 8, a.accumulate != 0, vec);
     }
   } else {
-    // grad[c0 + c][n]: a lane owns columns c = lane and lane + 64
+    // grad[c0 + c][n]: neighbouring lanes take neighbouring rank octets of one column (see above)
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      const int c = lane + 64 * half;
+    for (int k = 0; k < RP / 4; ++k) {
+      const int piece = lane + 64 * k, c = piece / (RP / 8), n8 = 8 * (piece % (RP / 8));
+      if (n8 >= r) continue;
+      float v8[8];
 #pragma unroll
-      for (int n8 = 0; n8 < RP; n8 += 8) {
-        if (n8 >= r) break;
-        float v8[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v8[i] = lds[(n8 + i) * OS + c];
-        store_bf16x8(gp + (int64_t)(c0 + c) * a.ld_grad + n_base + n8, v8, min(8, r - n8), a.accumulate != 0, vec);
-      }
+      for (int i = 0; i < 8; ++i) v8[i] = lds[(n8 + i) * OS + c];
+      store_bf16x8(gp + (int64_t)(c0 + c) * a.ld_grad + n_base + n8, v8, min(8, r - n8), a.accumulate != 0, vec);
     }
   }
 }
