@@ -593,14 +593,25 @@ __global__ __launch_bounds__(256) void k_expand_mfma_multi(PassJobs jobs, const 
 template <int NB, int TPI>
 __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* __restrict__ hrow,
                                                       const int32_t* __restrict__ tile_group,
-                                                      const int32_t* __restrict__ slot_rows, int max_tiles) {
+                                                      const int32_t* __restrict__ slot_rows,
+                                                      const int32_t* __restrict__ set_walk,
+                                                      const SegHeader* __restrict__ header, int max_tiles) {
+  static_assert(TPI == kSetTiles, "the segment table's set order is built for sets of kSetTiles tiles");
   constexpr int RP = 16 * NB;
   constexpr int NKS = (RP + 31) / 32;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
   const int ngroups = a.width_dst >> 7;
   const int nbt = (ngroups + 3) >> 2;  // blocks per tile set: column block fastest
-  const int block = TK_XCD_MAP(blockIdx.x, gridDim.x);
-  const int cb = block % nbt, tile0 = (block / nbt) * TPI;
+  // Gathered rows whose groups interleave: the sets of tiles in the order of their first row, so that neighbouring
+  // rows are in flight together (measured at config 3: 2.5 % of the step).  Rows in segment order, or a table built
+  // from sorted keys (then that order is the identity): contiguous runs of sets per XCD, whose L2 then fetches the
+  // weights of few groups (1.2 % at config 5's q projection; combining the two loses the first gain).
+  // (the flag and the order entry are requested together: one round trip in front of the tile's first loads)
+  const int swept_set = set_walk ? set_walk[blockIdx.x / nbt] : 0;
+  const bool sweep = set_walk != nullptr && header->sorted_input == 0;
+  const int block = sweep ? (int)blockIdx.x : TK_XCD_MAP(blockIdx.x, gridDim.x);
+  const int cb = block % nbt, set = block / nbt;
+  const int tile0 = (sweep ? swept_set : set) * TPI;
   const int cg = cb * 4 + wave;
   if (cg >= ngroups) return;
   const int nt = min(TPI, max_tiles - tile0);
@@ -1305,7 +1316,7 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
     constexpr int TPI = 4;
     const int64_t blocks = ceil_div(L.max_tiles, TPI) * ceil_div(ngroups, 4);
     hipLaunchKernelGGL((k_expand_multi<NB, TPI>), dim3((unsigned)blocks), dim3(256), 0, s, a, hrow, seg.tile_group,
-                       rows, (int)L.max_tiles);
+                       rows, seg.set_walk(a.map_rows), seg.header, (int)L.max_tiles);
   } else {
     const int64_t items = L.max_tiles * ngroups;
     hipLaunchKernelGGL((k_expand_mfma<NB>), dim3((unsigned)ceil_div(items, 4)), dim3(256), 0, s, a, hrow,

@@ -225,6 +225,7 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
     hdr->num_chunks = carry_chunks;
     hdr->num_partials = carry_part;
     hdr->bad_keys = bad_total;
+    hdr->sorted_input = 1;  // this path leaves tile_order and set_order as the identity
   }
   // the firsts were written by this block: make them visible to all of its threads, then fill the
   // per-tile (with its 32 slots) and per-chunk tables in parallel
@@ -243,6 +244,7 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
     }
     V.tile_group[i] = g == groups - 1 ? -1 : g;
     V.tile_order[i] = i;  // this path leaves the tiles in table order
+    if (i % kSetTiles == 0) V.set_order[i / kSetTiles] = i / kSetTiles;
     int4* sp = reinterpret_cast<int4*>(V.slot_pos + (int64_t)i * kTileRows);
 #pragma unroll
     for (int j = 0; j < kTileRows; j += 4)
@@ -334,6 +336,8 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
   __shared__ int32_t cursor[kOneGroups];                // sorted position of the block's first row of each group
   __shared__ int32_t ahead[kKeysPerLane][kOneGroups];   // rows of each group ahead of each 64-row round of the block
   __shared__ int32_t bad_s[kOneWaves];
+  __shared__ int32_t sorted_s[kOneWaves];
+  __shared__ int32_t first_key[kOneBlocks + 1];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, blk = blockIdx.x;
   const int64_t base = (int64_t)blk * kSortBlockRows;
 
@@ -351,6 +355,12 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
 #pragma unroll
   for (int u = 0; u < kOneBatch; ++u)
     load_keys8(keys, (int64_t)(wave + u * kOneWaves) * kSortBlockRows + 8 * lane, rows, aligned16, groups, &bad, k[u]);
+  // the first key of every sort block, for the order check below
+  if (lane == 0) {
+#pragma unroll
+    for (int u = 0; u < kOneBatch; ++u) first_key[wave + u * kOneWaves] = k[u][0];
+  }
+  if (tid == 0) first_key[kOneBlocks] = -1;
   for (int i = tid; i < 2 * kOneSubs * (kOneGroups + 1); i += kOneWaves * 64) (&cnt[0][0][0])[i] = 0;
   for (int i = tid; i < kKeysPerLane * kOneGroups; i += kOneWaves * 64) (&round_cnt[0][0])[i] = 0;
   __syncthreads();
@@ -373,6 +383,22 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) bad += __shfl_xor(bad, d, 64);
   if (lane == 0) bad_s[wave] = bad;
+  // Are the keys non-decreasing?  Every block holds all keys anyway: a lane compares its eight keys with each other,
+  // with the first key of the next lane and, as the last lane of a sort block, with the first key of the next
+  // sort block (-1: past the last row).
+  bool sorted = true;
+#pragma unroll
+  for (int u = 0; u < kOneBatch; ++u) {
+    const int from_next_lane = __shfl_down(k[u][0], 1, 64);
+    const int after = lane == 63 ? first_key[wave + u * kOneWaves + 1] : from_next_lane;
+#pragma unroll
+    for (int j = 0; j < kKeysPerLane; ++j) {
+      const int nxt = j + 1 < kKeysPerLane ? k[u][j + 1] : after;
+      sorted = sorted && (nxt < 0 || k[u][j] <= nxt);
+    }
+  }
+  if (lane == 0) sorted_s[wave] = 0;
+  if (__ballot(!sorted) == 0ull && lane == 0) sorted_s[wave] = 1;
   __syncthreads();
 
   if (wave == 0) {
@@ -422,8 +448,11 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
         V.tile_first[groups] = total[1];
         V.chunk_first[groups] = total[2];
         V.partial_first[groups] = total[3];
-        int bad_total = 0;
-        for (int w = 0; w < kOneWaves; ++w) bad_total += bad_s[w];
+        int bad_total = 0, all_sorted = 1;
+        for (int w = 0; w < kOneWaves; ++w) {
+          bad_total += bad_s[w];
+          all_sorted &= sorted_s[w];
+        }
         SegHeader* hdr = V.header;
         hdr->magic = kSegMagic;
         hdr->rows = rows;
@@ -432,6 +461,7 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
         hdr->num_chunks = total[2];
         hdr->num_partials = total[3];
         hdr->bad_keys = bad_total;
+        hdr->sorted_input = all_sorted;
       }
     }
   }
@@ -468,12 +498,21 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
     const bool opens = valid && mine != groups - 1 && (in_group & (kTileRows - 1)) == 0;
     if (__ballot(opens)) {  // wave-uniform
       const unsigned long long below = (1ull << lane) - 1ull;
-      int place = 0;
+      // the same count over sets of kSetTiles tiles (those of a group's tiles ahead whose number is a multiple of
+      // kSetTiles), for the tiles that open a set
+      int place = 0, set_place = 0;
       for (int g2 = 0; g2 < groups - 1; ++g2) {
         const int n = ahead[wave][g2] + __popcll(__ballot(valid && mine == g2) & below);
-        place += (n + kTileRows - 1) / kTileRows;
+        const int tiles_ahead = (n + kTileRows - 1) / kTileRows;
+        place += tiles_ahead;
+        const int t0 = tfirst[g2];  // sets opened by the tiles t0 .. t0 + tiles_ahead - 1
+        set_place += (t0 + tiles_ahead + kSetTiles - 1) / kSetTiles - (t0 + kSetTiles - 1) / kSetTiles;
       }
-      if (opens) V.tile_order[place] = tfirst[mine] + in_group / kTileRows;
+      if (opens) {
+        const int tile = tfirst[mine] + in_group / kTileRows;
+        V.tile_order[place] = tile;
+        if (tile % kSetTiles == 0) V.set_order[set_place] = tile / kSetTiles;
+      }
     }
   }
 
@@ -490,6 +529,7 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
     }
     V.tile_group[i] = g == groups - 1 ? -1 : g;
     if (i >= real_tiles) V.tile_order[i] = i;  // nothing to do in these: they stay where they are, after the others
+    if (i >= real_tiles && i % kSetTiles == 0) V.set_order[i / kSetTiles] = i / kSetTiles;
     int4* sp = reinterpret_cast<int4*>(V.slot_pos + (int64_t)i * kTileRows);
 #pragma unroll
     for (int j = 0; j < kTileRows; j += 4)

@@ -12,6 +12,7 @@ namespace tk {
 
 constexpr int kWave = 64;
 constexpr int kTileRows = TK_TILE_ROWS;    // rows per forward tile (two 16-row MFMA tiles)
+constexpr int kSetTiles = 4;                                    // tiles per work item of the expand above rank 16
 constexpr int kChunkTilesMin = TK_CHUNK_ROWS / TK_TILE_ROWS;  // smallest weight-gradient chunk: 4 tiles (128 rows)
 constexpr int kChunkTilesMax = 128;                             // largest: 4096 rows
 constexpr int kSortBlockRows = 512;        // rows one single-wave block orders in the scatter pass
@@ -36,7 +37,9 @@ struct SegHeader {       // 64 x int32, at the start of the workspace
   int32_t num_chunks;    // filled on the device
   int32_t num_partials;  // chunks that belong to multi-chunk groups
   int32_t bad_keys;      // keys outside [0, groups): rows without a group
-  int32_t pad[57];
+  int32_t sorted_input;  // 1: the keys came in non-decreasing order (the table's order is the row order: tile_order and
+                         // set_order are the identity), or the builder did not compute those orders
+  int32_t pad[56];
 };
 
 struct ChunkInfo {  // one weight-gradient chunk: tiles [tile0, tile0 + ntiles) of group `group`, ntiles <= chunk_tiles
@@ -79,7 +82,7 @@ struct SegLayout {
   int64_t max_tiles, max_chunks, max_partials;
   int64_t slots;         // padded sorted length: 32 * max_tiles
   // byte offsets from the workspace base
-  int64_t off_inv, off_slot_row, off_slot_pos, off_offsets, off_tile_group, off_tile_order, off_chunks, off_tile_first,
+  int64_t off_inv, off_slot_row, off_slot_pos, off_offsets, off_tile_group, off_tile_order, off_set_order, off_chunks, off_tile_first,
       off_chunk_first, off_partial_first, off_hist, off_bad, total;
 
   SegLayout(int64_t rows_, int64_t groups_) : rows(rows_), groups(groups_) {
@@ -99,6 +102,7 @@ struct SegLayout {
     off_offsets = o;       o += round_up(4 * (buckets + 1), 256);
     off_tile_group = o;    o += round_up(4 * (max_tiles + 1), 256);
     off_tile_order = o;    o += round_up(4 * (max_tiles + 1), 256);
+    off_set_order = o;     o += round_up(4 * (max_tiles / kSetTiles + 2), 256);
     off_chunks = o;        o += round_up(16 * (max_chunks + 1), 256);
     off_tile_first = o;    o += round_up(4 * (buckets + 1), 256);
     off_chunk_first = o;   o += round_up(4 * (buckets + 1), 256);
@@ -121,6 +125,9 @@ struct SegView {  // typed device pointers into a segment workspace
   // cover neighbouring rows of the activation tensors whatever their groups (the table is group-major: a group's
   // tiles are spread over all rows).  Identity where the builder does not compute it.
   int32_t* tile_order;
+  // [ceil(max_tiles / kSetTiles)]  the same for kernels whose work items are sets of kSetTiles consecutive tiles
+  // (tiles kSetTiles s .. kSetTiles s + kSetTiles - 1): the sets in the order of the first row of their first tile
+  int32_t* set_order;
   ChunkInfo* chunks;       // [max_chunks]
   int32_t* tile_first;     // [G + 2]  first tile of each group
   int32_t* chunk_first;    // [G + 2]  first chunk of each group
@@ -136,6 +143,7 @@ struct SegView {  // typed device pointers into a segment workspace
     offsets = (int32_t*)(b + L.off_offsets);
     tile_group = (int32_t*)(b + L.off_tile_group);
     tile_order = (int32_t*)(b + L.off_tile_order);
+    set_order = (int32_t*)(b + L.off_set_order);
     chunks = (ChunkInfo*)(b + L.off_chunks);
     tile_first = (int32_t*)(b + L.off_tile_first);
     chunk_first = (int32_t*)(b + L.off_chunk_first);
@@ -147,6 +155,7 @@ struct SegView {  // typed device pointers into a segment workspace
   const int32_t* slot_table(int map_rows) const { return map_rows ? slot_row : slot_pos; }
   // order in which single-tile work items take the tiles (null: as numbered; rows in segment order are contiguous)
   const int32_t* tile_walk(int map_rows) const { return map_rows ? tile_order : nullptr; }
+  const int32_t* set_walk(int map_rows) const { return map_rows ? set_order : nullptr; }
 };
 
 constexpr int32_t kSegMagic = 0x544b5347;  // "TKSG"
