@@ -595,7 +595,9 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
                                                       const int32_t* __restrict__ tile_group,
                                                       const int32_t* __restrict__ slot_rows,
                                                       const int32_t* __restrict__ set_walk,
-                                                      const SegHeader* __restrict__ header, int max_tiles) {
+                                                      const SegHeader* __restrict__ header,
+                                                      const uint8_t* __restrict__ round_moved, int sort_blocks,
+                                                      int max_tiles) {
   static_assert(TPI == kSetTiles, "the segment table's set order is built for sets of kSetTiles tiles");
   constexpr int RP = 16 * NB;
   constexpr int NKS = (RP + 31) / 32;
@@ -604,11 +606,18 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
   const int nbt = (ngroups + 3) >> 2;  // blocks per tile set: column block fastest
   // Gathered rows whose groups interleave: the sets of tiles in the order of their first row, so that neighbouring
   // rows are in flight together (measured at config 3: 2.5 % of the step).  Rows in segment order, or a table built
-  // from sorted keys (then that order is the identity): contiguous runs of sets per XCD, whose L2 then fetches the
-  // weights of few groups (1.2 % at config 5's q projection; combining the two loses the first gain).
-  // (the flag and the order entry are requested together: one round trip in front of the tile's first loads)
-  const int swept_set = set_walk ? set_walk[blockIdx.x / nbt] : 0;
-  const bool sweep = set_walk != nullptr && header->sorted_input == 0;
+  // from keys that came in order (then that order is the identity): contiguous runs of sets per XCD, whose L2 then
+  // fetches the weights of few groups (1.2 % at config 5's q projection; combining the two loses the first gain).
+  // Whether the keys came in order is in the builder's flags, one byte per 64 rows, eight per lane here.
+  // (the flags and the order entry are requested together: one round trip in front of the tile's first loads)
+  int swept_set = 0;
+  bool sweep = false;
+  if (set_walk != nullptr) {
+    swept_set = set_walk[blockIdx.x / nbt];
+    uint2 moved = make_uint2(0u, 0u);
+    if (lane < sort_blocks) moved = reinterpret_cast<const uint2*>(round_moved)[lane];
+    sweep = header->identity_order == 0 && __ballot((moved.x | moved.y) != 0u) != 0ull;
+  }
   const int block = sweep ? (int)blockIdx.x : TK_XCD_MAP(blockIdx.x, gridDim.x);
   const int cb = block % nbt, set = block / nbt;
   const int tile0 = (sweep ? swept_set : set) * TPI;
@@ -1316,7 +1325,8 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
     constexpr int TPI = 4;
     const int64_t blocks = ceil_div(L.max_tiles, TPI) * ceil_div(ngroups, 4);
     hipLaunchKernelGGL((k_expand_multi<NB, TPI>), dim3((unsigned)blocks), dim3(256), 0, s, a, hrow, seg.tile_group,
-                       rows, seg.set_walk(a.map_rows), seg.header, (int)L.max_tiles);
+                       rows, seg.set_walk(a.map_rows), seg.header, seg.round_moved,
+                       (int)std::min<int64_t>(L.sort_blocks, 64), (int)L.max_tiles);
   } else {
     const int64_t items = L.max_tiles * ngroups;
     hipLaunchKernelGGL((k_expand_mfma<NB>), dim3((unsigned)ceil_div(items, 4)), dim3(256), 0, s, a, hrow,

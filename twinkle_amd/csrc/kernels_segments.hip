@@ -225,7 +225,7 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
     hdr->num_chunks = carry_chunks;
     hdr->num_partials = carry_part;
     hdr->bad_keys = bad_total;
-    hdr->sorted_input = 1;  // this path leaves tile_order and set_order as the identity
+    hdr->identity_order = 1;
   }
   // the firsts were written by this block: make them visible to all of its threads, then fill the
   // per-tile (with its 32 slots) and per-chunk tables in parallel
@@ -336,8 +336,6 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
   __shared__ int32_t cursor[kOneGroups];                // sorted position of the block's first row of each group
   __shared__ int32_t ahead[kKeysPerLane][kOneGroups];   // rows of each group ahead of each 64-row round of the block
   __shared__ int32_t bad_s[kOneWaves];
-  __shared__ int32_t sorted_s[kOneWaves];
-  __shared__ int32_t first_key[kOneBlocks + 1];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, blk = blockIdx.x;
   const int64_t base = (int64_t)blk * kSortBlockRows;
 
@@ -355,12 +353,6 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
 #pragma unroll
   for (int u = 0; u < kOneBatch; ++u)
     load_keys8(keys, (int64_t)(wave + u * kOneWaves) * kSortBlockRows + 8 * lane, rows, aligned16, groups, &bad, k[u]);
-  // the first key of every sort block, for the order check below
-  if (lane == 0) {
-#pragma unroll
-    for (int u = 0; u < kOneBatch; ++u) first_key[wave + u * kOneWaves] = k[u][0];
-  }
-  if (tid == 0) first_key[kOneBlocks] = -1;
   for (int i = tid; i < 2 * kOneSubs * (kOneGroups + 1); i += kOneWaves * 64) (&cnt[0][0][0])[i] = 0;
   for (int i = tid; i < kKeysPerLane * kOneGroups; i += kOneWaves * 64) (&round_cnt[0][0])[i] = 0;
   __syncthreads();
@@ -383,22 +375,6 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) bad += __shfl_xor(bad, d, 64);
   if (lane == 0) bad_s[wave] = bad;
-  // Are the keys non-decreasing?  Every block holds all keys anyway: a lane compares its eight keys with each other,
-  // with the first key of the next lane and, as the last lane of a sort block, with the first key of the next
-  // sort block (-1: past the last row).
-  bool sorted = true;
-#pragma unroll
-  for (int u = 0; u < kOneBatch; ++u) {
-    const int from_next_lane = __shfl_down(k[u][0], 1, 64);
-    const int after = lane == 63 ? first_key[wave + u * kOneWaves + 1] : from_next_lane;
-#pragma unroll
-    for (int j = 0; j < kKeysPerLane; ++j) {
-      const int nxt = j + 1 < kKeysPerLane ? k[u][j + 1] : after;
-      sorted = sorted && (nxt < 0 || k[u][j] <= nxt);
-    }
-  }
-  if (lane == 0) sorted_s[wave] = 0;
-  if (__ballot(!sorted) == 0ull && lane == 0) sorted_s[wave] = 1;
   __syncthreads();
 
   if (wave == 0) {
@@ -448,11 +424,8 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
         V.tile_first[groups] = total[1];
         V.chunk_first[groups] = total[2];
         V.partial_first[groups] = total[3];
-        int bad_total = 0, all_sorted = 1;
-        for (int w = 0; w < kOneWaves; ++w) {
-          bad_total += bad_s[w];
-          all_sorted &= sorted_s[w];
-        }
+        int bad_total = 0;
+        for (int w = 0; w < kOneWaves; ++w) bad_total += bad_s[w];
         SegHeader* hdr = V.header;
         hdr->magic = kSegMagic;
         hdr->rows = rows;
@@ -461,7 +434,7 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
         hdr->num_chunks = total[2];
         hdr->num_partials = total[3];
         hdr->bad_keys = bad_total;
-        hdr->sorted_input = all_sorted;
+        hdr->identity_order = 0;
       }
     }
   }
@@ -483,9 +456,11 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
     const int64_t f = base + wave * 64 + lane;
     const bool valid = mine >= 0;
     int in_group = 0;  // position of this row inside its group
+    bool moved = false;
     if (valid) {
       in_group = ahead[wave][mine] + rank_in_round;
       const int pos = offs[mine] + in_group;
+      moved = pos != f;
       V.inv[f] = pos;
       if (perm_out) perm_out[pos] = f;
       // padded slot = 32 * first tile of the group + position inside the group
@@ -495,18 +470,29 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
     // many tiles open before it: for every group, the rows of that group ahead of this row, in units of 32, rounded
     // up.  Those counts are all here (blocks and rounds before this one from the table above, lanes before this
     // one from a ballot per group), so the tile's place in the order needs no sort and no second launch.
+    // No row of the round moved in any round <=> the keys came in order <=> that order is the identity.
+    const unsigned long long any_moved = __ballot(moved);
+    if (lane == 0) V.round_moved[blk * kKeysPerLane + wave] = any_moved != 0ull;
     const bool opens = valid && mine != groups - 1 && (in_group & (kTileRows - 1)) == 0;
     if (__ballot(opens)) {  // wave-uniform
-      const unsigned long long below = (1ull << lane) - 1ull;
-      // the same count over sets of kSetTiles tiles (those of a group's tiles ahead whose number is a multiple of
-      // kSetTiles), for the tiles that open a set
+      // The same count over sets of kSetTiles tiles, for the tiles that open a set: of the tiles t0 .. t0 + n - 1 of a
+      // group ahead, ceil((t0 + n) / kSetTiles) - ceil(t0 / kSetTiles) open one.
+      // Lane g2 holds the figures of group g2 (at most 64 groups here); the loop reads them lane by lane.
+      static_assert(kOneGroups <= 64, "one lane per group");
+      const int gl = min(lane, groups - 1);
+      const int ahead_up = ahead[wave][gl] + kTileRows - 1;  // rounds the tile count up
+      const int first_up = tfirst[gl] + kSetTiles - 1;
       int place = 0, set_place = 0;
       for (int g2 = 0; g2 < groups - 1; ++g2) {
-        const int n = ahead[wave][g2] + __popcll(__ballot(valid && mine == g2) & below);
-        const int tiles_ahead = (n + kTileRows - 1) / kTileRows;
+        const unsigned long long in_g2 = __ballot(mine == g2);
+        // rows of the group ahead of this row: earlier rounds and blocks, and the lanes below this one
+        const unsigned n_up = __builtin_amdgcn_mbcnt_hi(
+            (unsigned)(in_g2 >> 32),
+            __builtin_amdgcn_mbcnt_lo((unsigned)in_g2, (unsigned)__builtin_amdgcn_readlane(ahead_up, g2)));
+        const unsigned tiles_ahead = n_up / kTileRows;
+        const unsigned t0_up = (unsigned)__builtin_amdgcn_readlane(first_up, g2);
         place += tiles_ahead;
-        const int t0 = tfirst[g2];  // sets opened by the tiles t0 .. t0 + tiles_ahead - 1
-        set_place += (t0 + tiles_ahead + kSetTiles - 1) / kSetTiles - (t0 + kSetTiles - 1) / kSetTiles;
+        set_place += (t0_up + tiles_ahead) / kSetTiles - t0_up / kSetTiles;
       }
       if (opens) {
         const int tile = tfirst[mine] + in_group / kTileRows;

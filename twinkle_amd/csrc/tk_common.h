@@ -13,6 +13,7 @@ namespace tk {
 constexpr int kWave = 64;
 constexpr int kTileRows = TK_TILE_ROWS;    // rows per forward tile (two 16-row MFMA tiles)
 constexpr int kSetTiles = 4;                                    // tiles per work item of the expand above rank 16
+constexpr int kRoundFlagBytes = 512;                            // SegView::round_moved: 64 sort blocks x 8 rounds
 constexpr int kChunkTilesMin = TK_CHUNK_ROWS / TK_TILE_ROWS;  // smallest weight-gradient chunk: 4 tiles (128 rows)
 constexpr int kChunkTilesMax = 128;                             // largest: 4096 rows
 constexpr int kSortBlockRows = 512;        // rows one single-wave block orders in the scatter pass
@@ -37,8 +38,8 @@ struct SegHeader {       // 64 x int32, at the start of the workspace
   int32_t num_chunks;    // filled on the device
   int32_t num_partials;  // chunks that belong to multi-chunk groups
   int32_t bad_keys;      // keys outside [0, groups): rows without a group
-  int32_t sorted_input;  // 1: the keys came in non-decreasing order (the table's order is the row order: tile_order and
-                         // set_order are the identity), or the builder did not compute those orders
+  int32_t identity_order;  // 1: the builder left tile_order and set_order as the identity; 0: it computed them, and
+                           // SegView::round_moved says whether they differ from the identity
   int32_t pad[56];
 };
 
@@ -82,7 +83,8 @@ struct SegLayout {
   int64_t max_tiles, max_chunks, max_partials;
   int64_t slots;         // padded sorted length: 32 * max_tiles
   // byte offsets from the workspace base
-  int64_t off_inv, off_slot_row, off_slot_pos, off_offsets, off_tile_group, off_tile_order, off_set_order, off_chunks, off_tile_first,
+  int64_t off_inv, off_slot_row, off_slot_pos, off_offsets, off_tile_group, off_tile_order, off_set_order, off_round_moved, off_chunks,
+      off_tile_first,
       off_chunk_first, off_partial_first, off_hist, off_bad, total;
 
   SegLayout(int64_t rows_, int64_t groups_) : rows(rows_), groups(groups_) {
@@ -103,6 +105,7 @@ struct SegLayout {
     off_tile_group = o;    o += round_up(4 * (max_tiles + 1), 256);
     off_tile_order = o;    o += round_up(4 * (max_tiles + 1), 256);
     off_set_order = o;     o += round_up(4 * (max_tiles / kSetTiles + 2), 256);
+    off_round_moved = o;   o += kRoundFlagBytes;
     off_chunks = o;        o += round_up(16 * (max_chunks + 1), 256);
     off_tile_first = o;    o += round_up(4 * (buckets + 1), 256);
     off_chunk_first = o;   o += round_up(4 * (buckets + 1), 256);
@@ -128,6 +131,11 @@ struct SegView {  // typed device pointers into a segment workspace
   // [ceil(max_tiles / kSetTiles)]  the same for kernels whose work items are sets of kSetTiles consecutive tiles
   // (tiles kSetTiles s .. kSetTiles s + kSetTiles - 1): the sets in the order of the first row of their first tile
   int32_t* set_order;
+  // [64 sort blocks][8 rounds of 64 rows]  one byte per round of the single-launch builder: non-zero when the sort
+  // moved a row of the round (its sorted position differs from its row number).  All zero for the rounds of a build
+  // <=> the keys came in order <=> tile_order and set_order are the identity.  Bytes of rounds past the last row of
+  // the current build are stale.
+  uint8_t* round_moved;
   ChunkInfo* chunks;       // [max_chunks]
   int32_t* tile_first;     // [G + 2]  first tile of each group
   int32_t* chunk_first;    // [G + 2]  first chunk of each group
@@ -144,6 +152,7 @@ struct SegView {  // typed device pointers into a segment workspace
     tile_group = (int32_t*)(b + L.off_tile_group);
     tile_order = (int32_t*)(b + L.off_tile_order);
     set_order = (int32_t*)(b + L.off_set_order);
+    round_moved = (uint8_t*)(b + L.off_round_moved);
     chunks = (ChunkInfo*)(b + L.off_chunks);
     tile_first = (int32_t*)(b + L.off_tile_first);
     chunk_first = (int32_t*)(b + L.off_chunk_first);
