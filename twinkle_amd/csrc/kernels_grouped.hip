@@ -31,6 +31,9 @@ constexpr int kGBK = 64, kGLS = kGBK + 8;
 #ifndef TK_GROUPED_BIG
 #define TK_GROUPED_BIG 1
 #endif
+#ifndef TK_GROUPED_DL
+#define TK_GROUPED_DL 1  // forward form, 8 waves: tiles go from global memory straight into LDS
+#endif
 constexpr int kGroupedItems = TK_GROUPED_ITEMS;  // work items aimed at per launch
 
 __global__ __launch_bounds__(256) void k_grouped_plan(const int32_t* __restrict__ tile_first, int experts, int nt,
@@ -270,6 +273,216 @@ __global__ __launch_bounds__(BIG ? 512 : 256) __attribute__((amdgpu_waves_per_eu
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same product with the operand tiles going from global memory straight into LDS (global_load_lds, 16 bytes per
+// lane): no staging registers and no LDS stores, so the wave has room for all operand fragments of a 32-deep half
+// step (12 x 16 bytes per lane) and reads them ahead of the MFMAs that use them.  Block tile 256 x 256 x 64, eight
+// waves (2 x 4), wave tile 128 x 64, two stages of 64 KB.
+//
+// Stage layout: x rows and weight rows alike, row r of the tile at byte 128 r, its 16-byte chunk c at position
+// c ^ (r & 7).  A wave-wide load brings eight rows: lane L lands at byte 16 L of the wave's 1 KB window (the
+// hardware's rule), i.e. row L >> 3, position L & 7, so it fetches chunk (L & 7) ^ (L >> 3) of that row: eight
+// neighbouring lanes cover one whole 128-byte line of global memory.  An operand read (lane = row li, chunk
+// 4 s + kb) goes to position (4 s + kb) ^ (li & 7): the eight lanes of one pass hit eight different 16-byte bank
+// groups.  Row offsets are 32-bit (the launcher checks that x and one expert's weights span less than 4 GB).
+//
+// Per 64-deep step: one block barrier (behind a wait for the wave's own loads of this stage: the stage is complete
+// when every wave has passed), then the loads of the next step into the other stage, then 24 operand reads and 64
+// MFMAs per wave.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void load16_to_lds(const bf16_t* base, uint32_t byte_offset, bf16_t* window) {
+  __builtin_amdgcn_global_load_lds(
+      (const __attribute__((address_space(1))) void*)(reinterpret_cast<const char*>(base) + byte_offset),
+      (__attribute__((address_space(3))) void*)window, 16, 0, 0);
+}
+
+template <int NKS>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k_grouped_gemm_dl(
+    GroupedArgs a, const GroupedPlanEntry* __restrict__ plan, const int32_t* __restrict__ nblocks,
+    const int32_t* __restrict__ tile_group, const int32_t* __restrict__ slot_rows, int nsplit, int cpi) {
+  constexpr int WN = 4, RB = 8, CB = 4, BM = 256, BN = 256;
+  __shared__ __attribute__((aligned(1024))) bf16_t As0[BM * kGBK];
+  __shared__ __attribute__((aligned(1024))) bf16_t As1[BM * kGBK];
+  __shared__ __attribute__((aligned(1024))) bf16_t Bs0[BN * kGBK];
+  __shared__ __attribute__((aligned(1024))) bf16_t Bs1[BN * kGBK];
+  const int blocks = *nblocks * nsplit;
+  if ((int)blockIdx.x >= blocks) return;
+  const int item = xcd_contiguous(blockIdx.x, blocks);
+  const GroupedPlanEntry any = plan[item / nsplit];
+  const int local = item - any.first * nsplit;
+  const GroupedPlanEntry pe = plan[any.first + local % any.count];
+  const int nb_first = (local / any.count) * cpi, nb_last = min(nb_first + cpi, a.N / BN);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  const int wm = wave / WN, wn = wave % WN;
+  const int slot0 = pe.tile0 * kTileRows, live = pe.ntiles * kTileRows;
+  const int live_w = min(max(live - 16 * RB * wm, 0), 16 * RB);  // live rows of this wave's strip (uniform)
+
+  // this wave's share of a stage: rows 32 wave + 8 i + (lane >> 3), i = 0..3, of the x tile and of the weight tile
+  const int lrow = lane >> 3;
+  const uint32_t lchunk = (uint32_t)(((lane & 7) ^ lrow) * 16);
+  uint32_t xoff[4], woff[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 32 * wave + 8 * i + lrow;
+    int row = r < live ? slot_rows[slot0 + r] : -1;  // padding and dead rows read row 0 and are never stored
+    row = min(max(row, 0), a.src_rows - 1);
+    xoff[i] = (uint32_t)row * (uint32_t)(a.ldx * 2) + lchunk;
+    woff[i] = (uint32_t)r * (uint32_t)(a.ldw * 2) + lchunk;
+  }
+  // operand reads: byte offsets inside a stage for s = 0, 1 (the row blocks are immediate offsets of 2 KB)
+  uint32_t a_rd[2], b_rd[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    const uint32_t pos = (uint32_t)(((4 * s + kb) ^ (li & 7)) * 16);
+    a_rd[s] = (uint32_t)(16 * RB * wm + li) * 128u + pos;
+    b_rd[s] = (uint32_t)(16 * CB * wn + li) * 128u + pos;
+  }
+  int out_row[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const int r = 16 * RB * wm + 16 * rb + li;
+    out_row[rb] = r < live ? slot_rows[slot0 + r] : -1;
+  }
+  const bf16_t* wbase = a.w + (int64_t)pe.expert * a.w_stride;
+  const int nk = a.K / kGBK;
+  const int window = (32 * wave) * kGBK;  // first element of this wave's rows in a stage
+
+  for (int nb = nb_first; nb < nb_last; ++nb) {
+    const bf16_t* wnb = wbase + (int64_t)nb * BN * a.ldw;
+    f32x4 acc[RB][CB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) acc[rb][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    auto fetch = [&](int ks, bf16_t* As, bf16_t* Bs) {
+      const bf16_t* xk = a.x + ks * kGBK;
+      const bf16_t* wk = wnb + ks * kGBK;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) load16_to_lds(xk, xoff[i], As + window + 8 * i * kGBK);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) load16_to_lds(wk, woff[i], Bs + window + 8 * i * kGBK);
+    };
+    auto compute = [&](const bf16_t* As, const bf16_t* Bs, auto full_strip) {
+      const char* Ab = reinterpret_cast<const char*>(As);
+      const char* Bb = reinterpret_cast<const char*>(Bs);
+      if constexpr (decltype(full_strip)::value) {
+        // The step in four quarters of 16 MFMAs (half of the row blocks of one 32-deep half step); the operand reads
+        // of a quarter are requested one quarter ahead, so they land while the matrix cores work (the fences keep
+        // the compiler from moving them back next to their use).
+        uint4 fw[2][CB], fx[2][RB / 2];
+        auto read_w = [&](int s) {
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb) fw[s][cb] = *reinterpret_cast<const uint4*>(Bb + b_rd[s] + 2048 * cb);
+        };
+        auto read_x = [&](int s, int half) {
+#pragma unroll
+          for (int i = 0; i < RB / 2; ++i)
+            fx[half][i] = *reinterpret_cast<const uint4*>(Ab + a_rd[s] + 2048 * (RB / 2 * half + i));
+        };
+        auto quarter = [&](int s, int half) {
+#pragma unroll
+          for (int i = 0; i < RB / 2; ++i)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb)
+              acc[RB / 2 * half + i][cb] = mfma16(fw[s][cb], fx[half][i], acc[RB / 2 * half + i][cb]);
+        };
+        read_w(0);
+        read_x(0, 0);
+        read_x(0, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        quarter(0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        read_w(1);
+        read_x(1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        quarter(0, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        read_x(1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+        quarter(1, 0);
+        quarter(1, 1);
+        __builtin_amdgcn_sched_barrier(0);
+      } else {
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+          uint4 fw[CB];
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb) fw[cb] = *reinterpret_cast<const uint4*>(Bb + b_rd[s] + 2048 * cb);
+#pragma unroll
+          for (int rb = 0; rb < RB; ++rb) {
+            if (16 * rb >= live_w) break;
+            const uint4 fx = *reinterpret_cast<const uint4*>(Ab + a_rd[s] + 2048 * rb);
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) acc[rb][cb] = mfma16(fw[cb], fx, acc[rb][cb]);
+          }
+        }
+      }
+    };
+    auto k_loop = [&](auto full_strip) {
+      fetch(0, As0, Bs0);
+      for (int ks = 0; ks < nk; ks += 2) {
+        __syncthreads();  // stage 0 has landed (every wave waited for its own loads), stage 1 has been read
+        if (ks + 1 < nk) fetch(ks + 1, As1, Bs1);
+        compute(As0, Bs0, full_strip);
+        if (ks + 1 < nk) {
+          __syncthreads();
+          if (ks + 2 < nk) fetch(ks + 2, As0, Bs0);
+          compute(As1, Bs1, full_strip);
+        }
+      }
+      __syncthreads();  // both stages have been read: the next column block may load
+    };
+    if (live_w == 16 * RB) k_loop(std::true_type{});
+    else k_loop(std::false_type{});
+
+    if constexpr (NKS > 0) {
+      // LoRA term: h[slot][0 .. rpad) against B_g[n][0 .. rank), per 32-row tile (a tile has one group)
+#pragma unroll
+      for (int tl = 0; tl < RB / 2; ++tl) {
+        const int tile_in_block = (RB / 2) * wm + tl;
+        if (tile_in_block >= pe.ntiles) break;
+        const int g = tile_group[pe.tile0 + tile_in_block];
+        const int r = g >= 0 ? min(a.rank[g], a.rpad) : 0;
+        if (r <= 0) continue;
+        const bf16_t* Bg = (const bf16_t*)a.lora_B[g];
+#pragma unroll
+        for (int s = 0; s < NKS; ++s) {
+          const int n0 = 32 * s + 8 * kb;  // first rank index of this lane's operand piece
+          if (32 * s >= r) break;          // uniform over the wave
+          uint4 fh[2], fb[CB];
+#pragma unroll
+          for (int q = 0; q < 2; ++q) {
+            const int slot = slot0 + 32 * tile_in_block + 16 * q + li;
+            fh[q] = n0 < a.rpad ? ld16(a.hrow + (int64_t)slot * a.rpad + n0) : zero4();
+          }
+#pragma unroll
+          for (int cb = 0; cb < CB; ++cb) {
+            const int n = nb * BN + 16 * CB * wn + 16 * cb + li;
+            fb[cb] = n0 < r ? keep_first(ld16(Bg + (int64_t)n * a.ldb + n0), r - n0) : zero4();
+          }
+#pragma unroll
+          for (int q = 0; q < 2; ++q)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) acc[2 * tl + q][cb] = mfma16(fb[cb], fh[q], acc[2 * tl + q][cb]);
+        }
+      }
+    }
+
+    // lane holds y[slot 16 RB wm + 16 rb + li][nb BN + 16 CB wn + 16 cb + 4 kb + v], v = 0..3: 8-byte stores
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      if (out_row[rb] < 0) continue;
+      bf16_t* yp = a.y + (int64_t)out_row[rb] * a.ldy + nb * BN + 16 * CB * wn + 4 * kb;
+#pragma unroll
+      for (int cb = 0; cb < CB; ++cb) {
+        const f32x4 v = acc[rb][cb];
+        *reinterpret_cast<uint2*>(yp + 16 * cb) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+      }
+    }
+  }
+}
+
 }  // namespace
 
 bool grouped_gemm_supported(const GroupedArgs& a) {
@@ -313,6 +526,14 @@ int launch_grouped_gemm(const GroupedArgs& a, int experts, int nt, GroupedPlanEn
     else
       hipLaunchKernelGGL((k_grouped_gemm<0, 0, 1>), grid, dim3(256), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit,
                          cpi);
+  } else if (big && TK_GROUPED_DL && (int64_t)a.src_rows * a.ldx * 2 < (1ll << 32) &&
+             (int64_t)a.N * a.ldw * 2 < (1ll << 32)) {
+    if (nks == 0)
+      hipLaunchKernelGGL((k_grouped_gemm_dl<0>), grid, dim3(512), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit, cpi);
+    else if (nks == 1)
+      hipLaunchKernelGGL((k_grouped_gemm_dl<1>), grid, dim3(512), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit, cpi);
+    else
+      hipLaunchKernelGGL((k_grouped_gemm_dl<2>), grid, dim3(512), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit, cpi);
   } else if (big) {
     if (nks == 0) TK_LAUNCH_GROUPED(0, 1);
     else if (nks == 1) TK_LAUNCH_GROUPED(1, 1);
