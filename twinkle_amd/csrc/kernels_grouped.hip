@@ -313,9 +313,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
   const GroupedPlanEntry pe = plan[any.first + local % any.count];
   const int nb_first = (local / any.count) * cpi, nb_last = min(nb_first + cpi, a.N / BN);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  // The two strips of waves take the 16-row blocks of the tile alternately: strip wm owns rows 16 (2 rb + wm) + li,
+  // rb = 0..7, i.e. half of every 32-row tile.  A block with fewer than eight tiles (the last of an expert) then
+  // leaves both strips the same, smaller number of live row blocks, and its time shrinks with its rows.
   const int wm = wave / WN, wn = wave % WN;
   const int slot0 = pe.tile0 * kTileRows, live = pe.ntiles * kTileRows;
-  const int live_w = min(max(live - 16 * RB * wm, 0), 16 * RB);  // live rows of this wave's strip (uniform)
 
   // this wave's share of a stage: rows 32 wave + 8 i + (lane >> 3), i = 0..3, of the x tile and of the weight tile
   const int lrow = lane >> 3;
@@ -329,19 +331,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
     xoff[i] = (uint32_t)row * (uint32_t)(a.ldx * 2) + lchunk;
     woff[i] = (uint32_t)r * (uint32_t)(a.ldw * 2) + lchunk;
   }
-  // operand reads: byte offsets inside a stage for s = 0, 1 (the row blocks are immediate offsets of 2 KB)
+  // operand reads: byte offsets inside a stage for s = 0, 1 (row block rb of the strip: + 4 KB rb, column block cb of
+  // the wave: + 2 KB cb, as immediate offsets)
   uint32_t a_rd[2], b_rd[2];
 #pragma unroll
   for (int s = 0; s < 2; ++s) {
     const uint32_t pos = (uint32_t)(((4 * s + kb) ^ (li & 7)) * 16);
-    a_rd[s] = (uint32_t)(16 * RB * wm + li) * 128u + pos;
+    a_rd[s] = (uint32_t)(16 * wm + li) * 128u + pos;
     b_rd[s] = (uint32_t)(16 * CB * wn + li) * 128u + pos;
-  }
-  int out_row[RB];
-#pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
-    const int r = 16 * RB * wm + 16 * rb + li;
-    out_row[rb] = r < live ? slot_rows[slot0 + r] : -1;
   }
   const bf16_t* wbase = a.w + (int64_t)pe.expert * a.w_stride;
   const int nk = a.K / kGBK;
@@ -363,86 +360,75 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
 #pragma unroll
       for (int i = 0; i < 4; ++i) load16_to_lds(wk, woff[i], Bs + window + 8 * i * kGBK);
     };
-    auto compute = [&](const bf16_t* As, const bf16_t* Bs, auto full_strip) {
+    // One 64-deep step on NRB live row blocks per strip (NRB even).  In four quarters of 2 NRB MFMAs (half of the
+    // row blocks of one 32-deep half step); the operand reads of a quarter are requested one quarter ahead, so
+    // they land while the matrix cores work (the fences keep the compiler from moving them back next to their use).
+    auto compute = [&](const bf16_t* As, const bf16_t* Bs, auto nrb_c) {
+      constexpr int NRB = decltype(nrb_c)::value, H = NRB / 2;
       const char* Ab = reinterpret_cast<const char*>(As);
       const char* Bb = reinterpret_cast<const char*>(Bs);
-      if constexpr (decltype(full_strip)::value) {
-        // The step in four quarters of 16 MFMAs (half of the row blocks of one 32-deep half step); the operand reads
-        // of a quarter are requested one quarter ahead, so they land while the matrix cores work (the fences keep
-        // the compiler from moving them back next to their use).
-        uint4 fw[2][CB], fx[2][RB / 2];
-        auto read_w = [&](int s) {
+      uint4 fw[2][CB], fx[2][H];
+      auto read_w = [&](int s) {
 #pragma unroll
-          for (int cb = 0; cb < CB; ++cb) fw[s][cb] = *reinterpret_cast<const uint4*>(Bb + b_rd[s] + 2048 * cb);
-        };
-        auto read_x = [&](int s, int half) {
+        for (int cb = 0; cb < CB; ++cb) fw[s][cb] = *reinterpret_cast<const uint4*>(Bb + b_rd[s] + 2048 * cb);
+      };
+      auto read_x = [&](int s, int half) {
 #pragma unroll
-          for (int i = 0; i < RB / 2; ++i)
-            fx[half][i] = *reinterpret_cast<const uint4*>(Ab + a_rd[s] + 2048 * (RB / 2 * half + i));
-        };
-        auto quarter = [&](int s, int half) {
+        for (int i = 0; i < H; ++i)
+          fx[half][i] = *reinterpret_cast<const uint4*>(Ab + a_rd[s] + 4096 * (H * half + i));
+      };
+      auto quarter = [&](int s, int half) {
 #pragma unroll
-          for (int i = 0; i < RB / 2; ++i)
+        for (int i = 0; i < H; ++i)
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb)
-              acc[RB / 2 * half + i][cb] = mfma16(fw[s][cb], fx[half][i], acc[RB / 2 * half + i][cb]);
-        };
-        read_w(0);
-        read_x(0, 0);
-        read_x(0, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        quarter(0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        read_w(1);
-        read_x(1, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        quarter(0, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        read_x(1, 1);
-        __builtin_amdgcn_sched_barrier(0);
-        quarter(1, 0);
-        quarter(1, 1);
-        __builtin_amdgcn_sched_barrier(0);
-      } else {
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-          uint4 fw[CB];
-#pragma unroll
-          for (int cb = 0; cb < CB; ++cb) fw[cb] = *reinterpret_cast<const uint4*>(Bb + b_rd[s] + 2048 * cb);
-#pragma unroll
-          for (int rb = 0; rb < RB; ++rb) {
-            if (16 * rb >= live_w) break;
-            const uint4 fx = *reinterpret_cast<const uint4*>(Ab + a_rd[s] + 2048 * rb);
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb) acc[rb][cb] = mfma16(fw[cb], fx, acc[rb][cb]);
-          }
-        }
-      }
+          for (int cb = 0; cb < CB; ++cb)
+            acc[H * half + i][cb] = mfma16(fw[s][cb], fx[half][i], acc[H * half + i][cb]);
+      };
+      read_w(0);
+      read_x(0, 0);
+      read_x(0, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      quarter(0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      read_w(1);
+      read_x(1, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      quarter(0, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      read_x(1, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      quarter(1, 0);
+      quarter(1, 1);
+      __builtin_amdgcn_sched_barrier(0);
     };
-    auto k_loop = [&](auto full_strip) {
+    auto k_loop = [&](auto nrb_c) {
       fetch(0, As0, Bs0);
       for (int ks = 0; ks < nk; ks += 2) {
         __syncthreads();  // stage 0 has landed (every wave waited for its own loads), stage 1 has been read
         if (ks + 1 < nk) fetch(ks + 1, As1, Bs1);
-        compute(As0, Bs0, full_strip);
+        compute(As0, Bs0, nrb_c);
         if (ks + 1 < nk) {
           __syncthreads();
           if (ks + 2 < nk) fetch(ks + 2, As0, Bs0);
-          compute(As1, Bs1, full_strip);
+          compute(As1, Bs1, nrb_c);
         }
       }
       __syncthreads();  // both stages have been read: the next column block may load
     };
-    if (live_w == 16 * RB) k_loop(std::true_type{});
-    else k_loop(std::false_type{});
+    // live row blocks per strip = tiles of the block, rounded up to even (dead rows hold row 0 of x: their sums are
+    // never stored)
+    if (pe.ntiles > 6) k_loop(std::integral_constant<int, 8>{});
+    else if (pe.ntiles > 4) k_loop(std::integral_constant<int, 6>{});
+    else if (pe.ntiles > 2) k_loop(std::integral_constant<int, 4>{});
+    else k_loop(std::integral_constant<int, 2>{});
 
     if constexpr (NKS > 0) {
-      // LoRA term: h[slot][0 .. rpad) against B_g[n][0 .. rank), per 32-row tile (a tile has one group)
+      // LoRA term: h[slot][0 .. rpad) against B_g[n][0 .. rank); row block rb of a strip lies in tile rb of the
+      // block (a tile has one group)
 #pragma unroll
-      for (int tl = 0; tl < RB / 2; ++tl) {
-        const int tile_in_block = (RB / 2) * wm + tl;
-        if (tile_in_block >= pe.ntiles) break;
-        const int g = tile_group[pe.tile0 + tile_in_block];
+      for (int rb = 0; rb < RB; ++rb) {
+        if (rb >= pe.ntiles) break;
+        const int g = tile_group[pe.tile0 + rb];
         const int r = g >= 0 ? min(a.rank[g], a.rpad) : 0;
         if (r <= 0) continue;
         const bf16_t* Bg = (const bf16_t*)a.lora_B[g];
@@ -450,30 +436,27 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
         for (int s = 0; s < NKS; ++s) {
           const int n0 = 32 * s + 8 * kb;  // first rank index of this lane's operand piece
           if (32 * s >= r) break;          // uniform over the wave
-          uint4 fh[2], fb[CB];
-#pragma unroll
-          for (int q = 0; q < 2; ++q) {
-            const int slot = slot0 + 32 * tile_in_block + 16 * q + li;
-            fh[q] = n0 < a.rpad ? ld16(a.hrow + (int64_t)slot * a.rpad + n0) : zero4();
-          }
+          const int slot = slot0 + 32 * rb + 16 * wm + li;
+          const uint4 fh = n0 < a.rpad ? ld16(a.hrow + (int64_t)slot * a.rpad + n0) : zero4();
+          uint4 fb[CB];
 #pragma unroll
           for (int cb = 0; cb < CB; ++cb) {
             const int n = nb * BN + 16 * CB * wn + 16 * cb + li;
             fb[cb] = n0 < r ? keep_first(ld16(Bg + (int64_t)n * a.ldb + n0), r - n0) : zero4();
           }
 #pragma unroll
-          for (int q = 0; q < 2; ++q)
-#pragma unroll
-            for (int cb = 0; cb < CB; ++cb) acc[2 * tl + q][cb] = mfma16(fb[cb], fh[q], acc[2 * tl + q][cb]);
+          for (int cb = 0; cb < CB; ++cb) acc[rb][cb] = mfma16(fb[cb], fh, acc[rb][cb]);
         }
       }
     }
 
-    // lane holds y[slot 16 RB wm + 16 rb + li][nb BN + 16 CB wn + 16 cb + 4 kb + v], v = 0..3: 8-byte stores
+    // lane holds y[slot 16 (2 rb + wm) + li][nb BN + 16 CB wn + 16 cb + 4 kb + v], v = 0..3: 8-byte stores
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-      if (out_row[rb] < 0) continue;
-      bf16_t* yp = a.y + (int64_t)out_row[rb] * a.ldy + nb * BN + 16 * CB * wn + 4 * kb;
+      const int r = 16 * (2 * rb + wm) + li;
+      const int out_row = r < live ? slot_rows[slot0 + r] : -1;  // (looked up again: no registers across the loop)
+      if (out_row < 0) continue;
+      bf16_t* yp = a.y + (int64_t)out_row * a.ldy + nb * BN + 16 * CB * wn + 4 * kb;
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb) {
         const f32x4 v = acc[rb][cb];
