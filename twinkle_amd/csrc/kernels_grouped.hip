@@ -290,6 +290,18 @@ __global__ __launch_bounds__(BIG ? 512 : 256) __attribute__((amdgpu_waves_per_eu
 // when every wave has passed), then the loads of the next step into the other stage, then 24 operand reads and 64
 // MFMAs per wave.
 // ---------------------------------------------------------------------------
+// Wait until at most YOUNGER of the wave's loads are in flight (they complete in order) and its LDS reads are done,
+// then the block barrier.  Written out: the fences of __syncthreads() make the compiler wait for every load in
+// flight, the look-ahead ones included.
+template <int YOUNGER>
+__device__ __forceinline__ void loads_landed_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+  __builtin_amdgcn_s_waitcnt(0x0070 | YOUNGER);  // vmcnt(YOUNGER) lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  asm volatile("" ::: "memory");
+}
 __device__ __forceinline__ void load16_to_lds(const bf16_t* base, uint32_t byte_offset, bf16_t* window) {
   __builtin_amdgcn_global_load_lds(
       (const __attribute__((address_space(1))) void*)(reinterpret_cast<const char*>(base) + byte_offset),
@@ -305,6 +317,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
   __shared__ __attribute__((aligned(1024))) bf16_t As1[BM * kGBK];
   __shared__ __attribute__((aligned(1024))) bf16_t Bs0[BN * kGBK];
   __shared__ __attribute__((aligned(1024))) bf16_t Bs1[BN * kGBK];
+  __shared__ __attribute__((aligned(1024))) bf16_t Bs2[BN * kGBK];
   const int blocks = *nblocks * nsplit;
   if ((int)blockIdx.x >= blocks) return;
   const int item = xcd_contiguous(blockIdx.x, blocks);
@@ -352,11 +365,13 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb) acc[rb][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    auto fetch = [&](int ks, bf16_t* As, bf16_t* Bs) {
+    auto fetch_x = [&](int ks, bf16_t* As) {
       const bf16_t* xk = a.x + ks * kGBK;
-      const bf16_t* wk = wnb + ks * kGBK;
 #pragma unroll
       for (int i = 0; i < 4; ++i) load16_to_lds(xk, xoff[i], As + window + 8 * i * kGBK);
+    };
+    auto fetch_w = [&](int ks, bf16_t* Bs) {
+      const bf16_t* wk = wnb + ks * kGBK;
 #pragma unroll
       for (int i = 0; i < 4; ++i) load16_to_lds(wk, woff[i], Bs + window + 8 * i * kGBK);
     };
@@ -401,19 +416,49 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
       quarter(1, 1);
       __builtin_amdgcn_sched_barrier(0);
     };
+    // The weight tiles, most of which come from memory, are requested two steps ahead (three stages), the x tiles,
+    // most of which another column block of the same rows has just brought into this XCD's L2, one step ahead (two
+    // stages).  Step ks: wait until of the wave's loads only the youngest four (the weight tile of step ks + 1) may
+    // still be in flight, block barrier (x and weight tile of step ks are complete, the stages of step ks - 1 have
+    // been read by everybody), request x of step ks + 1 and the weights of step ks + 2, compute.
+    // (Every step requests both tiles, past the last step the last ones again, into stages that are not read any
+    // more: the same count of loads in flight at every barrier, and no branch in the steady state.)
+    auto stage_a = [&](auto i) -> bf16_t* {
+      if constexpr (decltype(i)::value == 0) return As0;
+      else return As1;
+    };
+    auto stage_b = [&](auto i) -> bf16_t* {
+      if constexpr (decltype(i)::value == 0) return Bs0;
+      else if constexpr (decltype(i)::value == 1) return Bs1;
+      else return Bs2;
+    };
+    auto step = [&](int ks, auto phase, auto nrb_c) {  // phase = ks mod 6
+      constexpr int P = decltype(phase)::value;
+      loads_landed_barrier<4>();
+      fetch_x(min(ks + 1, nk - 1), stage_a(std::integral_constant<int, (P + 1) % 2>{}));
+      fetch_w(min(ks + 2, nk - 1), stage_b(std::integral_constant<int, (P + 2) % 3>{}));
+      compute(stage_a(std::integral_constant<int, P % 2>{}), stage_b(std::integral_constant<int, P % 3>{}), nrb_c);
+    };
     auto k_loop = [&](auto nrb_c) {
-      fetch(0, As0, Bs0);
-      for (int ks = 0; ks < nk; ks += 2) {
-        __syncthreads();  // stage 0 has landed (every wave waited for its own loads), stage 1 has been read
-        if (ks + 1 < nk) fetch(ks + 1, As1, Bs1);
-        compute(As0, Bs0, nrb_c);
-        if (ks + 1 < nk) {
-          __syncthreads();
-          if (ks + 2 < nk) fetch(ks + 2, As0, Bs0);
-          compute(As1, Bs1, nrb_c);
-        }
+      fetch_x(0, As0);
+      fetch_w(0, Bs0);
+      fetch_w(min(1, nk - 1), Bs1);
+      int ks = 0;
+      using std::integral_constant;
+      for (; ks + 6 <= nk; ks += 6) {
+        step(ks, integral_constant<int, 0>{}, nrb_c);
+        step(ks + 1, integral_constant<int, 1>{}, nrb_c);
+        step(ks + 2, integral_constant<int, 2>{}, nrb_c);
+        step(ks + 3, integral_constant<int, 3>{}, nrb_c);
+        step(ks + 4, integral_constant<int, 4>{}, nrb_c);
+        step(ks + 5, integral_constant<int, 5>{}, nrb_c);
       }
-      __syncthreads();  // both stages have been read: the next column block may load
+      if (ks < nk) step(ks, integral_constant<int, 0>{}, nrb_c);
+      if (ks + 1 < nk) step(ks + 1, integral_constant<int, 1>{}, nrb_c);
+      if (ks + 2 < nk) step(ks + 2, integral_constant<int, 2>{}, nrb_c);
+      if (ks + 3 < nk) step(ks + 3, integral_constant<int, 3>{}, nrb_c);
+      if (ks + 4 < nk) step(ks + 4, integral_constant<int, 4>{}, nrb_c);
+      loads_landed_barrier<0>();  // every stage has been read, no load is in flight: the next column block may load
     };
     // live row blocks per strip = tiles of the block, rounded up to even (dead rows hold row 0 of x: their sums are
     // never stored)
