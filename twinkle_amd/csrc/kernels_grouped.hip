@@ -496,12 +496,17 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
     }
 
     // lane holds y[slot 16 (2 rb + wm) + li][nb BN + 16 CB wn + 16 cb + 4 kb + v], v = 0..3: 8-byte stores
+    // (the rows are looked up here, all eight together, rather than kept in registers across the loop)
+    int out_row[RB];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
       const int r = 16 * (2 * rb + wm) + li;
-      const int out_row = r < live ? slot_rows[slot0 + r] : -1;  // (looked up again: no registers across the loop)
-      if (out_row < 0) continue;
-      bf16_t* yp = a.y + (int64_t)out_row * a.ldy + nb * BN + 16 * CB * wn + 4 * kb;
+      out_row[rb] = r < live ? slot_rows[slot0 + r] : -1;
+    }
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      if (out_row[rb] < 0) continue;
+      bf16_t* yp = a.y + (int64_t)out_row[rb] * a.ldy + nb * BN + 16 * CB * wn + 4 * kb;
 #pragma unroll
       for (int cb = 0; cb < CB; ++cb) {
         const f32x4 v = acc[rb][cb];
