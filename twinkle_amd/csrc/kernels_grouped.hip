@@ -325,7 +325,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
   const int local = item - any.first * nsplit;
   const GroupedPlanEntry pe = plan[any.first + local % any.count];
   const int nb_first = (local / any.count) * cpi, nb_last = min(nb_first + cpi, a.N / BN);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
+  const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kb = lane >> 4;
+  // (told to be uniform: the LDS windows of the wave's loads then live in scalar registers)
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // The two strips of waves take the 16-row blocks of the tile alternately: strip wm owns rows 16 (2 rb + wm) + li,
   // rb = 0..7, i.e. half of every 32-row tile.  A block with fewer than eight tiles (the last of an expert) then
   // leaves both strips the same, smaller number of live row blocks, and its time shrinks with its rows.
