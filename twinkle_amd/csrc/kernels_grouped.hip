@@ -535,11 +535,15 @@ int64_t grouped_plan_entries(const SegLayout& L, int64_t experts) { return ceil_
 int launch_grouped_gemm(const GroupedArgs& a, int experts, int nt, GroupedPlanEntry* plan, int32_t* nblocks,
                         const SegView& seg, const SegLayout& L, hipStream_t s) {
   if (L.rows == 0) return TK_OK;
-  // The 8-wave variant wins wherever it applies, by a third on experts of thousands of rows, except with the LoRA
-  // term on small experts (its epilogue works on four tiles per wave with no registers to spare): measured at
-  // 512 rows per expert, 4 waves are then 5 % faster.
+  // The 8-wave variants win wherever they apply.  The forward form loads its tiles straight into LDS
+  // (k_grouped_gemm_dl: 32-bit row offsets, so x and one expert's weights must span less than 4 GB); the older
+  // 8-wave kernel serves the transposing form and the rest, except with the LoRA term on small experts (its epilogue
+  // has no registers to spare: measured at 512 rows per expert, 4 waves are then 5 % faster).
   const int nks = a.rpad == 0 ? 0 : (a.rpad <= 32 ? 1 : 2);
-  const bool big = TK_GROUPED_BIG && a.N % 256 == 0 && (nks == 0 || L.rows >= (int64_t)1024 * experts);
+  const bool direct = TK_GROUPED_DL && !a.w_rows_are_inputs && (int64_t)a.src_rows * a.ldx * 2 < (1ll << 32) &&
+                      (int64_t)a.N * a.ldw * 2 < (1ll << 32);
+  const bool big =
+      TK_GROUPED_BIG && a.N % 256 == 0 && (nks == 0 || direct || L.rows >= (int64_t)1024 * experts);
   const int ptiles = big ? 8 : 4, bn = big ? 256 : 128;
   const int max_entries = (int)(ceil_div(L.max_tiles, ptiles) + experts);
   hipLaunchKernelGGL(k_grouped_plan, dim3(1), dim3(256), 0, s, seg.tile_first, experts, nt, plan, nblocks, max_entries,
@@ -561,8 +565,7 @@ int launch_grouped_gemm(const GroupedArgs& a, int experts, int nt, GroupedPlanEn
     else
       hipLaunchKernelGGL((k_grouped_gemm<0, 0, 1>), grid, dim3(256), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit,
                          cpi);
-  } else if (big && TK_GROUPED_DL && (int64_t)a.src_rows * a.ldx * 2 < (1ll << 32) &&
-             (int64_t)a.N * a.ldw * 2 < (1ll << 32)) {
+  } else if (big && direct) {
     if (nks == 0)
       hipLaunchKernelGGL((k_grouped_gemm_dl<0>), grid, dim3(512), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit, cpi);
     else if (nks == 1)
