@@ -308,7 +308,20 @@ __device__ __forceinline__ void load16_to_lds(const bf16_t* base, uint32_t byte_
       (__attribute__((address_space(3))) void*)window, 16, 0, 0);
 }
 
-template <int NKS>
+// 64 bits per lane from LDS, transposed among 16 lanes (ds_read_b64_tr_b16): with M[p][e] the four 16-bit elements
+// e that lane p of a group of 16 points at, lane l receives M[4 e + (l >> 2)][l & 3], e = 0..3.
+__device__ __forceinline__ uint2 lds_read_transposed(const char* p) {
+  typedef short v4s __attribute__((ext_vector_type(4)));
+  const v4s v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s*)p);
+  return __builtin_bit_cast(uint2, v);
+}
+
+// TR = 1: the weight rows are input features (y = x W, the backward of TR = 0 on the same memory).  The weight
+// tile of a step is then 64 rows of 256 outputs, 512 bytes a row, and lies in LDS as it lies in memory (a wave-wide
+// load brings two rows; the 16-byte chunk c of row r at position c ^ ((r & 3) << 1)).  The MFMA operand, eight
+// consecutive contraction indices of one output, is a column of that tile: two transposing LDS reads fetch it, each
+// from four rows (which the swizzle puts on different banks) of 16 outputs.
+template <int NKS, int TR>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k_grouped_gemm_dl(
     GroupedArgs a, const GroupedPlanEntry* __restrict__ plan, const int32_t* __restrict__ nblocks,
     const int32_t* __restrict__ tile_group, const int32_t* __restrict__ slot_rows, int nsplit, int cpi) {
@@ -344,7 +357,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
     int row = r < live ? slot_rows[slot0 + r] : -1;  // padding and dead rows read row 0 and are never stored
     row = min(max(row, 0), a.src_rows - 1);
     xoff[i] = (uint32_t)row * (uint32_t)(a.ldx * 2) + lchunk;
-    woff[i] = (uint32_t)r * (uint32_t)(a.ldw * 2) + lchunk;
+    if constexpr (TR) {
+      const int kr = 8 * wave + 2 * i + (lane >> 5);  // row of the weight tile: two per load, 32 lanes each
+      woff[i] = (uint32_t)kr * (uint32_t)(a.ldw * 2) + (uint32_t)(((lane & 31) ^ ((kr & 3) << 1)) * 16);
+    } else {
+      woff[i] = (uint32_t)r * (uint32_t)(a.ldw * 2) + lchunk;
+    }
   }
   // operand reads: byte offsets inside a stage for s = 0, 1 (row block rb of the strip: + 4 KB rb, column block cb of
   // the wave: + 2 KB cb, as immediate offsets)
@@ -355,12 +373,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
     a_rd[s] = (uint32_t)(16 * wm + li) * 128u + pos;
     b_rd[s] = (uint32_t)(16 * CB * wn + li) * 128u + pos;
   }
+  // TR: this lane's address in the weight tile for column block cb: row 8 kb + (li >> 2) (+ 32 s + 4 h as immediate
+  // offsets), outputs 64 wn + 16 cb + 4 (li & 3) .. + 3
+  uint32_t b_tr[CB];
+#pragma unroll
+  for (int cb = 0; cb < CB; ++cb)
+    b_tr[cb] = (uint32_t)(8 * kb + (li >> 2)) * 512u +
+               (uint32_t)((8 * wn + 2 * (cb ^ (li >> 2)) + ((li & 3) >> 1)) * 16 + (li & 1) * 8);
   const bf16_t* wbase = a.w + (int64_t)pe.expert * a.w_stride;
   const int nk = a.K / kGBK;
   const int window = (32 * wave) * kGBK;  // first element of this wave's rows in a stage
 
   for (int nb = nb_first; nb < nb_last; ++nb) {
-    const bf16_t* wnb = wbase + (int64_t)nb * BN * a.ldw;
+    const bf16_t* wnb = TR ? wbase + nb * BN : wbase + (int64_t)nb * BN * a.ldw;
     f32x4 acc[RB][CB];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb)
@@ -373,9 +398,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
       for (int i = 0; i < 4; ++i) load16_to_lds(xk, xoff[i], As + window + 8 * i * kGBK);
     };
     auto fetch_w = [&](int ks, bf16_t* Bs) {
-      const bf16_t* wk = wnb + ks * kGBK;
+      if constexpr (TR) {
+        const bf16_t* wk = wnb + (int64_t)ks * kGBK * a.ldw;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) load16_to_lds(wk, woff[i], Bs + window + 8 * i * kGBK);
+        for (int i = 0; i < 4; ++i) load16_to_lds(wk, woff[i], Bs + (8 * wave + 2 * i) * BN);
+      } else {
+        const bf16_t* wk = wnb + ks * kGBK;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) load16_to_lds(wk, woff[i], Bs + window + 8 * i * kGBK);
+      }
     };
     // One 64-deep step on NRB live row blocks per strip (NRB even).  In four quarters of 2 NRB MFMAs (half of the
     // row blocks of one 32-deep half step); the operand reads of a quarter are requested one quarter ahead, so
@@ -387,7 +418,15 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
       uint4 fw[2][CB], fx[2][H];
       auto read_w = [&](int s) {
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb) fw[s][cb] = *reinterpret_cast<const uint4*>(Bb + b_rd[s] + 2048 * cb);
+        for (int cb = 0; cb < CB; ++cb) {
+          if constexpr (TR) {
+            const uint2 lo = lds_read_transposed(Bb + b_tr[cb] + 16384 * s);
+            const uint2 hi = lds_read_transposed(Bb + b_tr[cb] + 16384 * s + 2048);
+            fw[s][cb] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+          } else {
+            fw[s][cb] = *reinterpret_cast<const uint4*>(Bb + b_rd[s] + 2048 * cb);
+          }
+        }
       };
       auto read_x = [&](int s, int half) {
 #pragma unroll
@@ -540,8 +579,8 @@ int launch_grouped_gemm(const GroupedArgs& a, int experts, int nt, GroupedPlanEn
   // 8-wave kernel serves the transposing form and the rest, except with the LoRA term on small experts (its epilogue
   // has no registers to spare: measured at 512 rows per expert, 4 waves are then 5 % faster).
   const int nks = a.rpad == 0 ? 0 : (a.rpad <= 32 ? 1 : 2);
-  const bool direct = TK_GROUPED_DL && !a.w_rows_are_inputs && (int64_t)a.src_rows * a.ldx * 2 < (1ll << 32) &&
-                      (int64_t)a.N * a.ldw * 2 < (1ll << 32);
+  const bool direct = TK_GROUPED_DL && (int64_t)a.src_rows * a.ldx * 2 < (1ll << 32) &&
+                      (int64_t)(a.w_rows_are_inputs ? a.K : a.N) * a.ldw * 2 < (1ll << 32);
   const bool big =
       TK_GROUPED_BIG && a.N % 256 == 0 && (nks == 0 || direct || L.rows >= (int64_t)1024 * experts);
   const int ptiles = big ? 8 : 4, bn = big ? 256 : 128;
@@ -558,7 +597,10 @@ int launch_grouped_gemm(const GroupedArgs& a, int experts, int nt, GroupedPlanEn
 #define TK_LAUNCH_GROUPED(NKS, BIG)                                                                                  \
   hipLaunchKernelGGL((k_grouped_gemm<NKS, BIG, 0>), grid, dim3(BIG ? 512 : 256), 0, s, a, plan, nblocks, seg.tile_group, \
                      rows, nsplit, cpi)
-  if (a.w_rows_are_inputs) {  // never with the LoRA term (the caller checks)
+  if (a.w_rows_are_inputs && big && direct) {  // never with the LoRA term (the caller checks)
+    hipLaunchKernelGGL((k_grouped_gemm_dl<0, 1>), grid, dim3(512), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit,
+                       cpi);
+  } else if (a.w_rows_are_inputs) {
     if (big)
       hipLaunchKernelGGL((k_grouped_gemm<0, 1, 1>), grid, dim3(512), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit,
                          cpi);
@@ -567,11 +609,11 @@ int launch_grouped_gemm(const GroupedArgs& a, int experts, int nt, GroupedPlanEn
                          cpi);
   } else if (big && direct) {
     if (nks == 0)
-      hipLaunchKernelGGL((k_grouped_gemm_dl<0>), grid, dim3(512), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit, cpi);
+      hipLaunchKernelGGL((k_grouped_gemm_dl<0, 0>), grid, dim3(512), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit, cpi);
     else if (nks == 1)
-      hipLaunchKernelGGL((k_grouped_gemm_dl<1>), grid, dim3(512), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit, cpi);
+      hipLaunchKernelGGL((k_grouped_gemm_dl<1, 0>), grid, dim3(512), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit, cpi);
     else
-      hipLaunchKernelGGL((k_grouped_gemm_dl<2>), grid, dim3(512), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit, cpi);
+      hipLaunchKernelGGL((k_grouped_gemm_dl<2, 0>), grid, dim3(512), 0, s, a, plan, nblocks, seg.tile_group, rows, nsplit, cpi);
   } else if (big) {
     if (nks == 0) TK_LAUNCH_GROUPED(0, 1);
     else if (nks == 1) TK_LAUNCH_GROUPED(1, 1);
