@@ -250,6 +250,13 @@ def yardstick_bench(dev, reps=12):
                                (6, 'shrink pattern, read', 1), (7, 'row-contraction pattern, read', 1)):
         for pname, perm in perms.items():
             out[f'{name}: {pname}'] = run(kind, perm, factor)
+    # the grouped GEMM's operand path, global memory -> LDS in steps of 64 KB per block with a barrier per step
+    out['global -> LDS, 64 KB steps per block: every line from memory'] = run(8, None, 1)
+    out['global -> LDS, 64 KB steps per block: every line an L2 hit'] = run(9, None, 16)
+    for k in ('global -> LDS, 64 KB steps per block: every line from memory',
+              'global -> LDS, 64 KB steps per block: every line an L2 hit'):
+        steps = T * K * 2 // 256 // 65536 * (16 if 'L2 hit' in k else 1)
+        out[k]['us_per_step'] = out[k]['us'] / steps
     return out
 
 

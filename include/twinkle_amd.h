@@ -335,7 +335,10 @@ enum {
   TK_YS_TILE_READ = 4,   /* (tile, 128 columns) per wave, read: the expand kernel's loads */
   TK_YS_TILE_RMW_NT = 5, /* (tile, 128 columns) per wave, in-place update, non-temporal: the expand kernel */
   TK_YS_SHRINK_READ = 6, /* (two tiles, 512 columns) per wave in MFMA operand order: the shrink kernel's loads */
-  TK_YS_WALK_READ = 7    /* one wave walks 16 tiles for 128 columns: the row-contraction kernels' loads */
+  TK_YS_WALK_READ = 7,   /* one wave walks 16 tiles for 128 columns: the row-contraction kernels' loads */
+  TK_YS_LDS_STREAM = 8,  /* 256 blocks of 8 waves load their share of `a` into LDS, 64 KB per step and barrier: the grouped
+                            GEMM's operand path with every line from memory (rows * width * 2 a multiple of 16 MiB) */
+  TK_YS_LDS_SHARED = 9   /* the same with all blocks walking the first 2 MB, 16 times the steps: every line an L2 hit */
 };
 int tk_yardstick(int32_t kind, void* a_device, void* b_device, const int32_t* row_of_device, int64_t rows,
                  int32_t width, tk_stream_t stream);

@@ -152,6 +152,37 @@ __global__ __launch_bounds__(64) void k_ys_walk(const bf16_t* __restrict__ x, co
   if (s.x == 0x12345678u && s.y == 0x9abcdefu) sink[lane] = s;
 }
 
+// the grouped GEMM's operand path: a block of eight waves brings 64 KB per step from global memory straight into
+// LDS (eight 16-byte global_load_lds per wave), one step ahead, one barrier per step, and never looks at the data.
+// SHARED: every block walks the same 2 MB again and again (every line an L2 hit); else every block walks its own
+// contiguous share of the buffer once (every line from memory).
+template <bool SHARED>
+__global__ __launch_bounds__(512) void k_ys_lds(const char* __restrict__ src, size_t share, int steps,
+                                                uint4* __restrict__ sink) {
+  __shared__ __attribute__((aligned(1024))) char lds[131072];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const size_t span = SHARED ? ((size_t)2 << 20) : share;  // a multiple of 64 KB (the launcher checks)
+  const char* base = SHARED ? src : src + (size_t)blockIdx.x * share;
+  for (int s = 0; s < steps; ++s) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const size_t o = ((size_t)s * 65536 + (size_t)(wave * 8 + i) * 1024) % span + lane * 16;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + o),
+                                       (__attribute__((address_space(3))) void*)(lds + (s & 1) * 65536 + (wave * 8 + i) * 1024),
+                                       16, 0, 0);
+    }
+    if (s >= 1) {  // the previous step has landed everywhere before its stage is loaded again
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_waitcnt(0x0070 | 8);  // vmcnt(8) lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+    }
+  }
+  __syncthreads();
+  if (lds[threadIdx.x * 16] == 0x7f && steps < 0) sink[threadIdx.x] = zero4();
+}
+
 }  // namespace
 
 }  // namespace tk
@@ -184,6 +215,19 @@ extern "C" int tk_yardstick(int32_t kind, void* a, void* b, const int32_t* row_o
     case TK_YS_WALK_READ:
       hipLaunchKernelGGL(k_ys_walk, dim3(width >> 7, tiles / 16), dim3(64), 0, s, x, row_of, width, 16, sink);
       break;
+    case TK_YS_LDS_STREAM:
+    case TK_YS_LDS_SHARED: {
+      // 256 blocks; a block's share of the buffer in 64 KB steps (TK_YS_LDS_SHARED: sixteen times as many steps)
+      const size_t bytes = (size_t)rows * width * 2;
+      if (bytes % ((size_t)256 * 65536) != 0 || bytes < ((size_t)2 << 20)) return TK_ERR_INVALID;
+      const size_t share = bytes / 256;
+      const int steps = (int)(share / 65536);
+      if (kind == TK_YS_LDS_STREAM)
+        hipLaunchKernelGGL(k_ys_lds<false>, dim3(256), dim3(512), 0, s, (const char*)a, share, steps, sink);
+      else
+        hipLaunchKernelGGL(k_ys_lds<true>, dim3(256), dim3(512), 0, s, (const char*)a, share, 16 * steps, sink);
+      break;
+    }
     default: return TK_ERR_INVALID;
   }
   return check_launch();
