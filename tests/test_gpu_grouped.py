@@ -118,6 +118,31 @@ def test_backward_of_the_base_term_on_the_same_weights(dev, k, n):
         grouped_linear_(dy.to(dev), w.to(dev), seg, nt, map_rows=True, transposed=True, groups=object(), h=None)
 
 
+@pytest.mark.parametrize('depth', [64, 128, 192, 320, 384, 448, 832])
+@pytest.mark.parametrize('transposed', [False, True])
+def test_direct_kernel_depths_block_lengths_and_strides(dev, depth, transposed):
+    """The 256-wide kernel that loads its tiles straight into LDS: contractions of 1, 2, 3, 5, 6, 7 and 13 steps of 64
+    (its loop is unrolled six times, with a tail), experts of 1 to 8 tiles and of several row blocks (the step is
+    compiled per number of live row blocks), x and the weights as views of wider buffers (row strides above the
+    widths), in both weight layouts."""
+    out_f, nt = 256, 1
+    sizes = [20, 40, 70, 100, 130, 170, 200, 230, 600, 0, 257]
+    expert = torch.cat([torch.full((c,), i) for i, c in enumerate(sizes)])
+    expert = expert[torch.randperm(expert.numel(), generator=torch.Generator().manual_seed(depth))]
+    e, t = len(sizes), expert.numel()
+    g = torch.Generator().manual_seed(depth + 1)
+    xbig = torch.randn(t, depth + 64, generator=g).bfloat16()
+    rows, cols = (depth, out_f) if transposed else (out_f, depth)   # [E, in, out] when transposed, else [E, out, in]
+    wbig = (torch.randn(e, rows, cols + 64, generator=g) / depth**0.5).bfloat16()
+    x, w = xbig[:, :depth], wbig[:, :, :cols]
+    seg = build_segments(expert.to(torch.int32).to(dev), e)
+    want = _reference(x, w.transpose(1, 2) if transposed else w, expert)
+    got = grouped_linear_(xbig.to(dev)[:, :depth], wbig.to(dev)[:, :, :cols], seg, nt, map_rows=True,
+                          transposed=transposed)
+    assert got.shape == (t, out_f)
+    assert max_rel_err(got, want) < 6e-3
+
+
 def test_unsupported_shapes_are_refused(dev):
     e, nt, t = 2, 1, 64
     keys = torch.zeros(t, dtype=torch.int32, device=dev)
