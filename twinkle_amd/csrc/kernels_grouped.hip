@@ -7,14 +7,19 @@
 // chunk boundary.  The LoRA term enters as extra contraction steps on the accumulators, so y is written once
 // instead of written by the GEMM and then read, updated and written again by the expand kernel.
 //
-//   k_grouped_plan   one small block: the list of row blocks (up to 4 consecutive tiles of one expert)
-//   k_grouped_gemm   one block of 4 waves per row block, looping over the 128-column blocks of the output: the
-//                    row block's x stays in L2 across the column blocks and the row blocks of one expert, which
-//                    reach an XCD together, stream that expert's weights through the XCD's L2 side by side
+//   k_grouped_plan      one small block: the list of row blocks (up to 4 or 8 consecutive tiles of one expert, an
+//                       expert's tiles cut into blocks of equal length)
+//   k_grouped_gemm_dl   out_features a multiple of 256 and operands under 4 GB: block tile 256 x 256 x 64, eight
+//                       waves, the operand tiles loaded from global memory straight into LDS (both weight layouts,
+//                       with and without the LoRA term); described where it is defined
+//   k_grouped_gemm      the rest: operands through registers into LDS; 8 waves on 256 x 256 tiles or 4 waves on
+//                       128 x 128 (row stride 144 B in LDS: conflict-free 16-byte operand reads, a wave owns
+//                       64 x 64 as 4 x 4 MFMA 16x16x32 tiles)
 //
-// Block tile 128 x 128 x 64, double-buffered in LDS (row stride 144 B: conflict-free 16-byte operand reads), a
-// wave owns 64 x 64 as 4 x 4 MFMA 16x16x32 tiles.  The weight fragment is the MFMA A operand and the x fragment
-// the B operand, so a lane ends up with four consecutive output columns of one row.
+// A block takes one row block and a run of column blocks of the output: the row block's x stays in L2 across the
+// column blocks, and the row blocks of one expert, which reach an XCD together, stream that expert's weights through
+// the XCD's L2 side by side.  The weight fragment is the MFMA A operand and the x fragment the B operand, so a lane
+// ends up with four consecutive output columns of one row.
 #include <algorithm>
 #include <type_traits>
 
@@ -32,7 +37,7 @@ constexpr int kGBK = 64, kGLS = kGBK + 8;
 #define TK_GROUPED_BIG 1
 #endif
 #ifndef TK_GROUPED_DL
-#define TK_GROUPED_DL 1  // forward form, 8 waves: tiles go from global memory straight into LDS
+#define TK_GROUPED_DL 1  // 8 waves, 256 x 256 tiles: operand tiles go from global memory straight into LDS
 #endif
 constexpr int kGroupedItems = TK_GROUPED_ITEMS;  // work items aimed at per launch
 
