@@ -143,6 +143,48 @@ def test_direct_kernel_depths_block_lengths_and_strides(dev, depth, transposed):
     assert max_rel_err(got, want) < 6e-3
 
 
+@pytest.mark.parametrize('transposed', [False, True])
+def test_register_staged_kernels_behind_the_switch(dev, monkeypatch, transposed):
+    """TK_GROUPED_DIRECT=0 keeps the 256-wide launches on the kernels that stage their operands through registers
+    (what operands of 4 GB and more take): same bar against the oracle, with and without the LoRA term."""
+    e, nt, t, k, n = 3, 2, 3400, 256, 512
+    expert, tenant, x, w = _case(e, nt, t, k, n, seed=21)
+    keys = (expert * nt + tenant).to(torch.int32).to(dev)
+    seg = build_segments(keys, e * nt)
+    monkeypatch.setenv('TK_GROUPED_DIRECT', '0')
+    if transposed:
+        dy = torch.randn(t, n, generator=torch.Generator().manual_seed(22)).bfloat16()
+        want = _reference(dy, w.transpose(1, 2).contiguous(), expert)
+        got = grouped_linear_(dy.to(dev), w.to(dev), seg, nt, map_rows=True, transposed=True)
+        assert max_rel_err(got, want) < 6e-3
+        monkeypatch.setenv('TK_GROUPED_DIRECT', '1')
+        direct = grouped_linear_(dy.to(dev), w.to(dev), seg, nt, map_rows=True, transposed=True)
+        assert max_rel_err(direct, want) < 6e-3
+        return
+    max_r = 16
+    g = torch.Generator().manual_seed(23)
+    a = [(torch.randn(e, max_r, k, generator=g) / k**0.5).bfloat16().to(dev) for _ in range(nt)]
+    b = [(torch.randn(e, n, max_r, generator=g) * 0.05).bfloat16().to(dev) for _ in range(nt)]
+    idx = [i % nt for i in range(e * nt)]
+    ranks = [16, 9]
+    groups = AdapterGroups(a, b, [ranks[i % nt] for i in range(e * nt)], [2.0] * (e * nt),
+                           a_index=idx, a_offset=[(i // nt) * max_r * k for i in range(e * nt)],
+                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)])
+    xd, wd = x.to(dev), w.to(dev)
+    h = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=dev)
+    lora_shrink_(xd, seg, groups, h, map_rows=True)
+    want = _reference(x, w, expert)
+    assert max_rel_err(grouped_linear_(xd, wd, seg, nt, map_rows=True), want) < 6e-3
+    xs = x.double()
+    for ei in range(e):
+        for ti in range(nt):
+            rows = ((expert == ei) & (tenant == ti)).nonzero().flatten()
+            if rows.numel():
+                r = ranks[ti]
+                want[rows] += 2.0 * (xs[rows] @ a[ti][ei, :r].double().cpu().t()) @ b[ti][ei, :, :r].double().cpu().t()
+    assert max_rel_err(grouped_linear_(xd, wd, seg, nt, groups=groups, h=h, map_rows=True), want) < 2e-2
+
+
 def test_unsupported_shapes_are_refused(dev):
     e, nt, t = 2, 1, 64
     keys = torch.zeros(t, dtype=torch.int32, device=dev)

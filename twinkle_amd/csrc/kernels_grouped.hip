@@ -21,6 +21,7 @@
 // the XCD's L2 side by side.  The weight fragment is the MFMA A operand and the x fragment the B operand, so a lane
 // ends up with four consecutive output columns of one row.
 #include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 
 #include "tk_mfma.h"
@@ -589,7 +590,10 @@ int launch_grouped_gemm(const GroupedArgs& a, int experts, int nt, GroupedPlanEn
   // 8-wave kernel serves the transposing form and the rest, except with the LoRA term on small experts (its epilogue
   // has no registers to spare: measured at 512 rows per expert, 4 waves are then 5 % faster).
   const int nks = a.rpad == 0 ? 0 : (a.rpad <= 32 ? 1 : 2);
-  const bool direct = TK_GROUPED_DL && (int64_t)a.src_rows * a.ldx * 2 < (1ll << 32) &&
+  // (TK_GROUPED_DIRECT=0 in the environment keeps the register-staged kernels in use: an A/B switch, read per call)
+  const char* env_direct = getenv("TK_GROUPED_DIRECT");
+  const bool direct = TK_GROUPED_DL && !(env_direct && env_direct[0] == '0') &&
+                      (int64_t)a.src_rows * a.ldx * 2 < (1ll << 32) &&
                       (int64_t)(a.w_rows_are_inputs ? a.K : a.N) * a.ldw * 2 < (1ll << 32);
   const bool big =
       TK_GROUPED_BIG && a.N % 256 == 0 && (nks == 0 || direct || L.rows >= (int64_t)1024 * experts);
