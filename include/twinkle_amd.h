@@ -151,7 +151,18 @@ typedef struct tk_lora_desc {
                                   the matrix cores with fp32 accumulation and write fp32 gradients.  0: A, B and
                                   the gradients have `dtype`.  The shared-input entry points then run one call per
                                   projection; tk_grouped_linear does not take it (TK_ERR_UNSUPPORTED). */
-  int32_t reserved;            /* 0 */
+  int32_t rank_classes;        /* Which padded ranks occur among rank[] (which lives on the device, so the host
+                                  says it here): bit 0 = some group has rank 1..16, bit 1 = 17..32, bit 2 = 33..64,
+                                  bit 3 = 65..128; the bit of max_rank's class must be among them.  With more than
+                                  one bit set, tk_lora_bwd runs each class of groups on the kernels of its own
+                                  padded rank (a tenant of rank 8 next to one of rank 64 is not padded to 64: every
+                                  tenant carries its own r, src/twinkle/model/multi_lora.py:318-325), the classes
+                                  side by side on streams of the library, and the backward workspace holds one
+                                  region per class (tk_lora_bwd_workspace_bytes accounts for it).  A group whose
+                                  rank lies in no listed class gets no gradients and adds nothing to dx.  The
+                                  forward and the layout of h do not depend on the field.  0 (or one bit): one
+                                  class for all groups, padded to max_rank.  The shared-input entry points ignore
+                                  the field. */
 } tk_lora_desc;
 
 /* Bytes of the saved shrink output h (scale * x A^T per row, kept for backward). */

@@ -80,7 +80,7 @@ def test_lora_term_in_the_epilogue(dev, max_r, ranks, e, t, n):
     # the kernel boundary: its term is skipped)
     groups = AdapterGroups(a, b, [ranks[i % nt] for i in range(e * nt)], [2.0] * (e * nt),
                            a_index=idx, a_offset=[(i // nt) * max_r * k for i in range(e * nt)],
-                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)])
+                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)], rank_classes=False)
     xd, wd = x.to(dev), w.to(dev)
     h = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=dev)
     lora_shrink_(xd, seg, groups, h, map_rows=True)
@@ -169,7 +169,7 @@ def test_register_staged_kernels_behind_the_switch(dev, monkeypatch, transposed)
     ranks = [16, 9]
     groups = AdapterGroups(a, b, [ranks[i % nt] for i in range(e * nt)], [2.0] * (e * nt),
                            a_index=idx, a_offset=[(i // nt) * max_r * k for i in range(e * nt)],
-                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)])
+                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)], rank_classes=False)
     xd, wd = x.to(dev), w.to(dev)
     h = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=dev)
     lora_shrink_(xd, seg, groups, h, map_rows=True)
@@ -270,7 +270,7 @@ def test_custom_op_matches_the_direct_call(dev):
     idx = [i % nt for i in range(e * nt)]
     groups = AdapterGroups(a, b, [16, 7] * e, [2.0] * (e * nt),
                            a_index=idx, a_offset=[(i // nt) * max_r * k for i in range(e * nt)],
-                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)])
+                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)], rank_classes=False)
     xd, wd = x.to(dev), w.to(dev)
     h = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=dev)
     lora_shrink_(xd, seg, groups, h, map_rows=True)
@@ -299,7 +299,7 @@ def test_hip_graph_replay_of_the_grouped_calls(dev):
     idx = [i % nt for i in range(e * nt)]
     groups = AdapterGroups(a, b, [16, 5] * e, [2.0] * (e * nt),
                            a_index=idx, a_offset=[(i // nt) * max_r * k for i in range(e * nt)],
-                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)])
+                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)], rank_classes=False)
     w = (torch.randn(e, n, k, generator=g) / k**0.5).bfloat16().to(dev)
     keys = torch.empty(t, dtype=torch.int32, device=dev)
     x = torch.empty(t, k, dtype=torch.bfloat16, device=dev)
@@ -385,7 +385,7 @@ def test_random_shapes_of_the_grouped_gemm(dev, seed):
         idx = [i % nt for i in range(e * nt)]
         groups = AdapterGroups(a, b, [ranks[i % nt] for i in range(e * nt)], [0.5] * (e * nt),
                                a_index=idx, a_offset=[(i // nt) * max_r * k for i in range(e * nt)],
-                               b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)])
+                               b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)], rank_classes=False)
         h = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=dev)
         lora_shrink_(xd, seg, groups, h, map_rows=True)
         got = grouped_linear_(xd, wd, seg, nt, groups=groups, h=h, map_rows=True)

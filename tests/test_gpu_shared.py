@@ -26,12 +26,12 @@ def _projections(k, outs, n, max_r, ranks_per_proj, seed, dtype, dev):
     return projs
 
 
-def _groups(projs, dev):
+def _groups(projs, dev, rank_classes=True):
     out = []
     for a, b, ranks, scales in projs:
         ad = [t.to(dev).requires_grad_(True) for t in a]
         bd = [t.to(dev).requires_grad_(True) for t in b]
-        out.append((AdapterGroups(ad, bd, ranks, scales), ad, bd))
+        out.append((AdapterGroups(ad, bd, ranks, scales, rank_classes=rank_classes), ad, bd))
     return out
 
 
@@ -44,9 +44,10 @@ def _compare(dev, dtype, t, k, outs, n, max_r, ranks_per_proj, seed=0, exact=Tru
     projs = _projections(k, outs, n, max_r, ranks_per_proj, seed, dtype, dev)
     seg = build_segments(ids.to(torch.int32).to(dev), n, check=True)
 
-    # one call per projection
+    # one call per projection (every group on the kernels of the projection's largest padded rank, like the shared
+    # entry points: the bit-for-bit comparison below is between the same kernels)
     xs = x.to(dev).requires_grad_(True)
-    sep = _groups(projs, dev)
+    sep = _groups(projs, dev, rank_classes=False)
     ys = [multi_lora_delta(xs, b.to(dev) * 1.0, seg, grp) for b, (grp, _, _) in zip(bases, sep)]
     torch.autograd.backward(ys, [d.to(dev) for d in dys])
 

@@ -49,7 +49,7 @@ class LoraDesc(Structure):
         ('rank', c_void_p),
         ('scale', c_void_p),
         ('weights_f32', c_int32),
-        ('reserved', c_int32),
+        ('rank_classes', c_int32),
     ]
 
 

@@ -9,6 +9,16 @@ using namespace tk;
 
 namespace {
 
+// a list of several rank classes must be a list of classes and contain the class of max_rank (every layout is sized
+// from the listed classes)
+bool classes_ok(const tk_lora_desc* d) {
+  const int m = d->rank_classes;
+  if (m < 0 || m >= (1 << kMaxClasses)) return false;
+  if ((m & (m - 1)) == 0) return true;  // none or one: one class, padded to max_rank
+  const int top = d->max_rank <= 16 ? 0 : d->max_rank <= 32 ? 1 : d->max_rank <= 64 ? 2 : 3;
+  return ((m >> top) & 1) != 0 && (m >> (top + 1)) == 0;
+}
+
 bool desc_ok(const tk_lora_desc* d) {
   if (!d) return false;
   if (d->rows < 0 || d->rows >= (1ll << 31)) return false;
@@ -19,6 +29,7 @@ bool desc_ok(const tk_lora_desc* d) {
   if (!d->seg_ws || !d->lora_A || !d->lora_B || !d->rank || !d->scale) return false;
   if (d->lda < d->in_features || d->ldb < d->max_rank) return false;
   if (d->weights_f32 != 0 && (d->weights_f32 != 1 || d->dtype != TK_DTYPE_BF16)) return false;
+  if (!classes_ok(d)) return false;
   return true;
 }
 
@@ -81,6 +92,75 @@ SideStream* side_stream() {
     if (!ok) (void)hipGetLastError();
   }
   return x.state == 1 ? &x : nullptr;
+}
+
+// Several rank classes in one call (tk_lora_desc::rank_classes) are independent chains of launches over disjoint
+// rows and groups, and no single kernel reaches the memory system's peak, so the classes above the first run on
+// streams of the library's own (per device, default priority, non-blocking), forked from and joined to the caller's
+// stream with events: the start-up and the tail of one class's launches are covered by the others' work.
+// TK_CLASS_STREAMS=0 keeps every class on the caller's stream.
+struct ClassStreams {
+  hipStream_t stream[kMaxClasses - 1] = {};
+  hipEvent_t fork = nullptr, join[kMaxClasses - 1] = {};
+  int state = 0;   // 0: not created yet, 1: ready, -1: creation failed (single-stream fallback)
+  std::mutex use;  // held while a call enqueues its fork .. join sequence: the events are shared per device
+};
+
+ClassStreams* class_streams() {
+  static const bool enabled = [] {
+    const char* e = getenv("TK_CLASS_STREAMS");
+    return !(e && e[0] == '0');
+  }();
+  if (!enabled) return nullptr;
+  constexpr int kMaxDevices = 64;
+  static ClassStreams cs[kMaxDevices];
+  static std::mutex mu;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(mu);
+  ClassStreams& x = cs[dev];
+  if (x.state == 0) {
+    bool ok = hipEventCreateWithFlags(&x.fork, hipEventDisableTiming) == hipSuccess;
+    for (int i = 0; ok && i < kMaxClasses - 1; ++i)
+      ok = hipStreamCreateWithFlags(&x.stream[i], hipStreamNonBlocking) == hipSuccess &&
+           hipEventCreateWithFlags(&x.join[i], hipEventDisableTiming) == hipSuccess;
+    x.state = ok ? 1 : -1;
+    if (!ok) (void)hipGetLastError();
+  }
+  return x.state == 1 ? &x : nullptr;
+}
+
+// Runs body(c, stream, forked) for every class: class 0 on the caller's stream, the others on the library's class
+// streams between a fork and a join (forked = true), or all on the caller's stream where there are none.  Everything
+// enqueued on `s` before the call is visible to every class; everything every class enqueued is complete for what
+// follows on `s`.  A body that is told `forked` must not fork again: a fork inside a forked stream is more than the
+// runtime's stream capture takes (it crashed when such a capture was ended), and the classes already overlap.
+template <typename Body>
+int for_each_class(int n, hipStream_t s, Body body) {
+  ClassStreams* cs = n > 1 ? class_streams() : nullptr;
+  if (!cs) {
+    for (int c = 0; c < n; ++c) {
+      const int rc = body(c, s, false);
+      if (rc != TK_OK) return rc;
+    }
+    return TK_OK;
+  }
+  std::lock_guard<std::mutex> guard(cs->use);
+  if (hipEventRecord(cs->fork, s) != hipSuccess) return TK_ERR_LAUNCH;
+  for (int c = 1; c < n; ++c)
+    if (hipStreamWaitEvent(cs->stream[c - 1], cs->fork, 0) != hipSuccess) return TK_ERR_LAUNCH;
+  // once forked, every stream joins again, also after an error: none may be left attached to the caller's stream
+  // (or to a graph capture of it)
+  int rc = TK_OK;
+  for (int c = n - 1; c >= 0; --c) {  // the caller's stream last: the side streams start while it is being filled
+    const int r = body(c, c == 0 ? s : cs->stream[c - 1], true);
+    if (r != TK_OK && rc == TK_OK) rc = r;
+  }
+  for (int c = 1; c < n; ++c)
+    if (hipEventRecord(cs->join[c - 1], cs->stream[c - 1]) != hipSuccess ||
+        hipStreamWaitEvent(s, cs->join[c - 1], 0) != hipSuccess)
+      return TK_ERR_LAUNCH;
+  return rc;
 }
 
 // Scratch of tk_lora_fwd_noalloc: the shrink output h and the partial sums of a split shrink, which tk_lora_fwd takes
@@ -209,7 +289,7 @@ static bool desc_shape_ok(const tk_lora_desc* d) {
   return d && d->rows >= 0 && d->num_groups > 0 && d->num_groups <= TK_MAX_GROUPS && d->max_rank >= 0 &&
          d->max_rank <= TK_MAX_RANK && d->in_features > 0 && d->out_features > 0 &&
          (d->dtype == TK_DTYPE_F32 || d->dtype == TK_DTYPE_BF16) &&
-         (d->weights_f32 == 0 || (d->weights_f32 == 1 && d->dtype == TK_DTYPE_BF16));
+         (d->weights_f32 == 0 || (d->weights_f32 == 1 && d->dtype == TK_DTYPE_BF16)) && classes_ok(d);
 }
 
 // h without the staged weight copies that follow it when the adapters are fp32
@@ -217,6 +297,58 @@ static int64_t h_core_bytes(const tk_lora_desc* d) {
   const int rpad = rank_pad(d->max_rank);
   return round_up(2 * (int64_t)rpad * h_ld(d->rows, d->num_groups) * elt_bytes(d->dtype), 256) +
          shrink_partial_bytes(d->rows, d->num_groups, d->in_features, rpad);
+}
+
+// The rank classes of a backward call (tk_lora_desc::rank_classes): for each class the descriptor its launches work
+// from (max_rank = the top of the class, so every workspace layout takes the class's padded rank) and where its region
+// of the workspace starts.  One class, equal to the caller's descriptor, unless several were listed.  The forward
+// pass is not split: all groups run on the kernels of the largest padded rank there (a launch per class costs the
+// in-place update of y more than the narrower kernels save; measured on 32 adapters of ranks 8 .. 64, 4096 -> 14336:
+// 539 against 472 us), so h has one layout, and every class of the backward reads its groups' rows of it.
+struct ClassPlan {
+  int n;
+  RankClass rc[kMaxClasses];
+  tk_lora_desc d[kMaxClasses];
+  int64_t ws_off[kMaxClasses], ws_bytes[kMaxClasses];
+  int64_t ws_core_total;
+  // several classes: their work lists (ClassListLayout each) follow the classes' regions; every call rebuilds them
+  int64_t list_bytes, ws_total;
+  void* lists[kMaxClasses];  // filled in by build_lists
+};
+
+static ClassPlan class_plan(const tk_lora_desc* d) {
+  ClassPlan P{};
+  P.n = rank_classes_of(*d, P.rc);
+  for (int c = 0; c < P.n; ++c) {
+    P.d[c] = *d;
+    P.d[c].max_rank = P.rc[c].hi;
+    P.ws_off[c] = P.ws_core_total;
+    P.ws_bytes[c] = BwdLayout(P.d[c]).total;
+    P.ws_core_total += P.ws_bytes[c];
+  }
+  P.list_bytes = P.n > 1 ? class_list_bytes(d->rows, d->num_groups) : 0;
+  P.ws_total = P.ws_core_total + P.n * P.list_bytes;
+  return P;
+}
+
+// Several classes: builds their work lists at `base` (see ClassPlan) and hands them to a pass / a contraction.
+static int build_lists(ClassPlan& P, const tk_lora_desc* d, void* base, const SegView& V, const SegLayout& L,
+                       hipStream_t s) {
+  if (P.n <= 1) return TK_OK;
+  for (int c = 0; c < P.n; ++c) P.lists[c] = (char*)base + c * P.list_bytes;
+  return launch_class_lists(d->rank, P.n, P.rc, P.lists, d->map_rows, V, L, s);
+}
+static void use_lists(const ClassPlan& P, int c, const SegLayout& L, PassArgs* a, WgradArgs* ga, WgradArgs* gb) {
+  if (P.n <= 1) return;
+  const ClassListLayout CL(L);
+  if (a) {
+    a->wl_tiles = CL.list(P.lists[c], kListTiles);
+    a->wl_pairs = CL.list(P.lists[c], kListPairs);
+    a->wl_octs = CL.list(P.lists[c], kListOcts);
+    a->wl_sets = CL.list(P.lists[c], kListSets);
+  }
+  if (ga) ga->wl_chunks = CL.list(P.lists[c], kListChunks);
+  if (gb) gb->wl_chunks = CL.list(P.lists[c], kListChunks);
 }
 
 int64_t tk_lora_h_bytes(const tk_lora_desc* d) {
@@ -228,13 +360,15 @@ int64_t tk_lora_h_bytes(const tk_lora_desc* d) {
 
 int64_t tk_lora_bwd_workspace_bytes(const tk_lora_desc* d) {
   if (!desc_shape_ok(d)) return TK_ERR_INVALID;
-  return BwdLayout(*d).total;
+  return class_plan(d).ws_total;
 }
 
 // Arguments of the forward pass h = scale x A^T, y += h B^T.  Null x / y are replaced by placeholders: shapes are
 // checked against what both phases need, so that the two halves of one forward pick the same kernels.
-static PassArgs fwd_pass_args(const tk_lora_desc* d, const void* x, int64_t ldx, void* y, int64_t ldy, void* h) {
+static PassArgs fwd_pass_args(const tk_lora_desc* d, const void* x, int64_t ldx, void* y, int64_t ldy, void* h,
+                              int rank_lo = 0, int class_mode = 0) {
   PassArgs a{};
+  a.rank_lo = rank_lo;  a.class_mode = class_mode;
   a.src = x ? x : h;  a.ld_src = x ? ldx : d->in_features;
   a.dst = y ? y : h;  a.ld_dst = y ? ldy : d->out_features;
   a.hT = h;   a.ldh = h_ld(d->rows, d->num_groups);
@@ -261,8 +395,10 @@ struct BwdPlan {
 
 static BwdPlan bwd_plan(const tk_lora_desc* d, const BwdLayout& B, const void* dy, int64_t lddy, const void* x,
                         int64_t ldx, const void* h, void* dx, int64_t lddx, void* const* grad_A, void* const* grad_B,
-                        int32_t accumulate, void* ws) {
+                        int32_t accumulate, void* ws, int rank_lo = 0, int class_mode = 0) {
   BwdPlan p;
+  p.ga.rank_lo = p.gb.rank_lo = p.a.rank_lo = p.tr.rank_lo = rank_lo;
+  p.a.class_mode = class_mode;
   char* w = (char*)ws;
   p.dh = w + B.off_dh;
   p.bT = w + B.off_wT_shrink;
@@ -353,23 +489,18 @@ int tk_lora_expand(const tk_lora_desc* d, const void* h, void* y, int64_t ldy, t
   return lora_pass_fwd(d, nullptr, 0, y, ldy, const_cast<void*>(h), 2, stream);
 }
 
-int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void* x, int64_t ldx, const void* h,
-                void* dx, int64_t lddx, void* const* grad_A, void* const* grad_B, int32_t accumulate, void* ws,
-                int64_t ws_bytes, tk_stream_t stream) {
-  if (!desc_ok(d)) return TK_ERR_INVALID;
-  if (d->rows == 0 || d->max_rank == 0) return TK_OK;
-  if (!dy || lddy < d->out_features || !ws) return TK_ERR_INVALID;
-  if (dx && lddx < d->in_features) return TK_ERR_INVALID;
-  if (grad_A && (!x || ldx < d->in_features)) return TK_ERR_INVALID;
-  if (grad_B && !h) return TK_ERR_INVALID;
+// The backward of the groups of one rank class (d: the class's descriptor; every group when there is one class).
+static int lora_bwd_class(const tk_lora_desc* d, const ClassPlan& P, int c, const void* dy, int64_t lddy,
+                          const void* x, int64_t ldx, const void* h, void* dx, int64_t lddx, void* const* grad_A,
+                          void* const* grad_B, int32_t accumulate, void* ws, hipStream_t s, bool may_fork) {
+  const int rank_lo = P.rc[c].lo, class_mode = P.n > 1;
   BwdLayout B(*d);
-  if (ws_bytes < B.total) return TK_ERR_WORKSPACE;
-  hipStream_t s = (hipStream_t)stream;
   SegLayout L(d->rows, d->num_groups);
   SegView V(d->seg_ws, L);
   int rc;
   const bool need_wT = dx || grad_A;
-  BwdPlan plan = bwd_plan(d, B, dy, lddy, x, ldx, h, dx, lddx, grad_A, grad_B, accumulate, ws);
+  BwdPlan plan = bwd_plan(d, B, dy, lddy, x, ldx, h, dx, lddx, grad_A, grad_B, accumulate, ws, rank_lo, class_mode);
+  use_lists(P, c, L, &plan.a, &plan.ga, &plan.gb);
   WgradArgs &ga = plan.ga, &gb = plan.gb;
   PassArgs& a = plan.a;
   const TransposeJob& tr = plan.tr;
@@ -395,7 +526,7 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
   // Separate kernels.  Two chains that meet only at the end: dB (reads dy and h) runs on a side stream,
   // the dy shrink -> dX on the caller's; dA follows the shrink on the side stream, next to the expand.
   // Without a side stream everything runs in the same order on the caller's stream.
-  SideStream* side = (grad_B && need_wT) ? side_stream() : nullptr;
+  SideStream* side = (grad_B && need_wT && may_fork) ? side_stream() : nullptr;
   hipStream_t s2 = side ? side->stream : s;
   // two host threads must not interleave their records and waits on the device's one set of events
   std::unique_lock<std::mutex> side_guard;
@@ -422,7 +553,7 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
       if (!wT_done) {
         // both consumers on the MFMA kernels: 16-byte stores, dead rank indices skipped; else the generic copy
         const bool fast = mfma && pass_mfma_supported(a) && d->out_features % 8 == 0;
-        rc = fast ? launch_transpose_job(tr, d->rank, a.rpad, s) : launch_transpose_weights(*d, bT, aT, s);
+        rc = fast ? launch_transpose_job(tr, d->rank, a.rpad, s) : launch_transpose_weights(*d, rank_lo, bT, aT, s);
         if (rc != TK_OK) break;
       }
       if ((rc = run_pass(a, V, L, d->dtype, 1, s)) != TK_OK) break;
@@ -443,6 +574,32 @@ int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void*
       return TK_ERR_LAUNCH;
   }
   return rc;
+}
+
+int tk_lora_bwd(const tk_lora_desc* d, const void* dy, int64_t lddy, const void* x, int64_t ldx, const void* h,
+                void* dx, int64_t lddx, void* const* grad_A, void* const* grad_B, int32_t accumulate, void* ws,
+                int64_t ws_bytes, tk_stream_t stream) {
+  if (!desc_ok(d)) return TK_ERR_INVALID;
+  if (d->rows == 0 || d->max_rank == 0) return TK_OK;
+  if (!dy || lddy < d->out_features || !ws) return TK_ERR_INVALID;
+  if (dx && lddx < d->in_features) return TK_ERR_INVALID;
+  if (grad_A && (!x || ldx < d->in_features)) return TK_ERR_INVALID;
+  if (grad_B && !h) return TK_ERR_INVALID;
+  ClassPlan P = class_plan(d);
+  if (ws_bytes < P.ws_total) return TK_ERR_WORKSPACE;
+  {
+    SegLayout L(d->rows, d->num_groups);
+    SegView V(d->seg_ws, L);
+    const int rc = build_lists(P, d, (char*)ws + P.ws_core_total, V, L, (hipStream_t)stream);
+    if (rc != TK_OK) return rc;
+  }
+  // Every rank class reads and writes the rows and the gradients of its own groups only, in its own region of the
+  // workspace; of h (one layout, written by the forward at the largest padded rank) it reads the rank-major copy,
+  // whose row stride does not depend on the padded rank, up to its own padded rank.
+  return for_each_class(P.n, (hipStream_t)stream, [&](int c, hipStream_t cs, bool forked) {
+    return lora_bwd_class(&P.d[c], P, c, dy, lddy, x, ldx, h, dx, lddx, grad_A, grad_B, accumulate,
+                          (char*)ws + P.ws_off[c], cs, !forked);
+  });
 }
 
 // ---- packed experts: grouped base GEMM (+ LoRA term) ---------------------------------------------------------------
@@ -565,8 +722,26 @@ static bool shared_wide_path(const tk_lora_desc* const* descs, int32_t n) {
   return true;
 }
 
-int tk_lora_fwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* x, int64_t ldx, void* const* y,
+// The shared-input entry points work with one rank class per projection (one layout of h, whatever runs below).
+struct SingleClassDescs {
+  tk_lora_desc d[TK_MAX_SHARED];
+  const tk_lora_desc* p[TK_MAX_SHARED];
+  SingleClassDescs(const tk_lora_desc* const* descs, int32_t n) {
+    for (int i = 0; i < TK_MAX_SHARED; ++i) {
+      p[i] = nullptr;
+      if (descs && i < n && descs[i]) {
+        d[i] = *descs[i];
+        d[i].rank_classes = 0;
+        p[i] = &d[i];
+      }
+    }
+  }
+};
+
+int tk_lora_fwd_shared(const tk_lora_desc* const* descs_in, int32_t n, const void* x, int64_t ldx, void* const* y,
                        const int64_t* ldy, void* const* h, tk_stream_t stream) {
+  const SingleClassDescs local(descs_in, n);
+  const tk_lora_desc* const* descs = descs_in ? local.p : nullptr;
   if (!shared_descs_ok(descs, n) || !y || !ldy || !h) return TK_ERR_INVALID;
   const tk_lora_desc* d0 = descs[0];
   if (d0->rows == 0) return TK_OK;
@@ -610,10 +785,12 @@ int tk_lora_fwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* 
   return launch_pass_multi(a, n, V, L, 4 | 2, s);
 }
 
-int tk_lora_bwd_shared(const tk_lora_desc* const* descs, int32_t n, const void* const* dy, const int64_t* lddy,
+int tk_lora_bwd_shared(const tk_lora_desc* const* descs_in, int32_t n, const void* const* dy, const int64_t* lddy,
                        const void* x, int64_t ldx, const void* const* h, void* dx, int64_t lddx,
                        void* const* const* grad_A, void* const* const* grad_B, int32_t accumulate, void* const* ws,
                        const int64_t* ws_bytes, tk_stream_t stream) {
+  const SingleClassDescs local(descs_in, n);
+  const tk_lora_desc* const* descs = descs_in ? local.p : nullptr;
   if (!shared_descs_ok(descs, n) || !dy || !lddy || !h || !grad_A || !grad_B || !ws || !ws_bytes) return TK_ERR_INVALID;
   const tk_lora_desc* d0 = descs[0];
   if (d0->rows == 0) return TK_OK;

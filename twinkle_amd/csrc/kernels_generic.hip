@@ -21,7 +21,8 @@ __global__ __launch_bounds__(256) void k_shrink_generic(PassArgs a, const int32_
   const int tile_id = blockIdx.x;
   const int g = tile_group[tile_id];
   if (g < 0) return;
-  const int r = min(a.rank[g], a.rpad);
+  const int r = class_rank(a.rank[g], a.rank_lo, a.rpad);
+  if (a.class_mode && r <= 0) return;  // a group of another rank class: its tiles belong to another launch
   const int rpad = a.rpad;
   float* xs = lds_f;                          // [32][kKC + 1]
   float* ws = lds_f + kTileRows * (kKC + 1);  // [rpad][kKC + 1]
@@ -83,7 +84,7 @@ __global__ __launch_bounds__(256) void k_expand_generic(PassArgs a, const int32_
   const int tile_id = blockIdx.x;
   const int g = tile_group[tile_id];
   if (g < 0) return;
-  const int r = min(a.rank[g], a.rpad);
+  const int r = class_rank(a.rank[g], a.rank_lo, a.rpad);
   if (r <= 0) return;
   __shared__ int rows_s[kTileRows];
   const int tid = threadIdx.x;
@@ -140,7 +141,7 @@ __global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkI
   const ChunkInfo ci = chunks[blockIdx.x];
   const int g = ci.group;
   if (g < 0) return;
-  const int r = min(a.rank[g], a.rpad);
+  const int r = class_rank(a.rank[g], a.rank_lo, a.rpad);
   if (r <= 0) return;
   const int tid = threadIdx.x;
   const int c = blockIdx.y * 256 + tid;
@@ -198,7 +199,7 @@ __device__ __forceinline__ void wgrad_reduce_body(const WgradArgs& a, int n0, co
   const int g = blockIdx.x;
   // independent loads first
   const int rk = a.rank[g], cf0 = chunk_first[g], cf1 = chunk_first[g + 1], pf = partial_first[g];
-  const int r = min(rk, a.rpad);
+  const int r = class_rank(rk, a.rank_lo, a.rpad);
   const int nchunk = cf1 - cf0;
   if (nchunk == 1) return;
   if (nchunk == 0 && a.accumulate) return;
@@ -342,10 +343,11 @@ __global__ __launch_bounds__(256) void k_wgrad_reduce_multi(WgradReduceJobs jobs
 // bT_g[n][m] = B_g[m][n], aT_g[k][n] = A_g[n][k]; zero for n >= rank[g].
 // (TS: the adapters' element type, T: that of the copies; they differ for fp32 adapters under bf16 activations)
 template <typename TS, typename T>
-__global__ __launch_bounds__(256) void k_transpose_weights(tk_lora_desc d, int rpad, T* __restrict__ bT,
+__global__ __launch_bounds__(256) void k_transpose_weights(tk_lora_desc d, int rpad, int rank_lo, T* __restrict__ bT,
                                                            T* __restrict__ aT) {
   const int g = blockIdx.y;
-  const int r = min(d.rank[g], rpad);
+  const int r = class_rank(d.rank[g], rank_lo, rpad);
+  if (rank_lo > 0 && r <= 0) return;  // a group of a lower rank class: no launch of this class reads its copies
   const TS* A = (const TS*)d.lora_A[g];
   const TS* B = (const TS*)d.lora_B[g];
   const int64_t nb = (int64_t)rpad * d.out_features, na = (int64_t)rpad * d.in_features;
@@ -504,17 +506,19 @@ int launch_wgrad_reduce_multi(const WgradArgs* sets, int n, const SegView& seg, 
   return check_launch();
 }
 
-int launch_transpose_weights(const tk_lora_desc& d, void* bT, void* aT, hipStream_t s) {
+int launch_transpose_weights(const tk_lora_desc& d, int rank_lo, void* bT, void* aT, hipStream_t s) {
   if (d.num_groups == 0) return TK_OK;
   const int rpad = rank_pad(d.max_rank);
   const int64_t per_group = (int64_t)rpad * (d.out_features + d.in_features);
   const dim3 grid((unsigned)std::min<int64_t>(ceil_div(per_group, 256), 64), (unsigned)d.num_groups);
   if (d.dtype == TK_DTYPE_F32)
-    hipLaunchKernelGGL((k_transpose_weights<float, float>), grid, dim3(256), 0, s, d, rpad, (float*)bT, (float*)aT);
+    hipLaunchKernelGGL((k_transpose_weights<float, float>), grid, dim3(256), 0, s, d, rpad, rank_lo, (float*)bT,
+                       (float*)aT);
   else if (mixed_weights(d))
-    hipLaunchKernelGGL((k_transpose_weights<float, bf16_t>), grid, dim3(256), 0, s, d, rpad, (bf16_t*)bT, (bf16_t*)aT);
+    hipLaunchKernelGGL((k_transpose_weights<float, bf16_t>), grid, dim3(256), 0, s, d, rpad, rank_lo,
+                       (bf16_t*)bT, (bf16_t*)aT);
   else
-    hipLaunchKernelGGL((k_transpose_weights<bf16_t, bf16_t>), grid, dim3(256), 0, s, d, rpad, (bf16_t*)bT,
+    hipLaunchKernelGGL((k_transpose_weights<bf16_t, bf16_t>), grid, dim3(256), 0, s, d, rpad, rank_lo, (bf16_t*)bT,
                        (bf16_t*)aT);
   return check_launch();
 }

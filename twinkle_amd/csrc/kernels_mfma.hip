@@ -112,7 +112,8 @@ __device__ inline void shrink_tiles(const PassArgs& a, bf16_t* __restrict__ hrow
     xa[u] = src + (int64_t)ra * a.ld_src + 16 * kb;
     xb[u] = src + (int64_t)rb * a.ld_src + 16 * kb;
   }
-  const int r = min(a.rank[g], RP);
+  const int r = class_rank(a.rank[g], a.rank_lo, RP);
+  if (a.class_mode && r <= 0) return;  // a group of another rank class (uniform over the block): nothing is requested
   const bf16_t* W1 = group_weight<bf16_t>(a.w_shrink, a.w_shrink_base, a.shrink_group_stride, g);
   const bf16_t* wp[NB];
   bool wv[NB];
@@ -197,7 +198,9 @@ __device__ __forceinline__ void shrink_pair_body(const PassArgs& a, bf16_t* __re
                                                  const int32_t* __restrict__ tile_group,
                                                  const int32_t* __restrict__ slot_rows, int max_tiles, int item) {
   __shared__ float part[NW][kTileRows][16 * NB + 1];
-  const int pair = item / a.kslices, ks = item - pair * a.kslices;
+  const int nth = item / a.kslices, ks = item - nth * a.kslices;
+  const int pair = work_item(a.wl_pairs, nth);
+  if (pair < 0) return;  // past the end of this rank class's list (uniform over the block)
   const int t0 = 2 * pair, t1 = t0 + 1;
   const int g0 = tile_group[t0];
   const int g1 = t1 < max_tiles ? tile_group[t1] : -1;
@@ -271,7 +274,9 @@ __device__ __forceinline__ void shrink_quad_body(const PassArgs& a, const int32_
   __shared__ __attribute__((aligned(16))) bf16_t wbuf[2][RP * WS];
   __shared__ int32_t gts[8];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
-  const int set = item / a.kslices, ks = item - set * a.kslices;
+  const int nth = item / a.kslices, ks = item - nth * a.kslices;
+  const int set = work_item(a.wl_octs, nth);
+  if (set < 0) return;  // past the end of this rank class's list (uniform over the block)
   const int t_first = set * 8;
   if (tid < 8) gts[tid] = t_first + tid < max_tiles ? tile_group[t_first + tid] : -1;
   const int nsteps = a.width_src >> 6;
@@ -297,8 +302,8 @@ __device__ __forceinline__ void shrink_quad_body(const PassArgs& a, const int32_
     const int lo = j, hi = e;  // the run: tiles t_first + lo .. t_first + hi - 1, all of group g
     j = e;
     if (g < 0) continue;
-    const int r = min(a.rank[g], RP);
-    if (r <= 0) continue;  // adapter not live on this layer
+    const int r = class_rank(a.rank[g], a.rank_lo, RP);
+    if (r <= 0) continue;  // adapter not live on this layer, or a group of another rank class
     bool mine[2];
 #pragma unroll
     for (int u = 0; u < 2; ++u) mine[u] = 2 * wave + u >= lo && 2 * wave + u < hi;
@@ -412,13 +417,17 @@ __global__ __launch_bounds__(256, 2) void k_shrink_quad_multi(PassJobs jobs, int
 template <int NB>
 __device__ __forceinline__ void shrink_finish_body(const PassArgs& a, bf16_t* __restrict__ hrow,
                                                    const int32_t* __restrict__ tile_group,
-                                                   const int32_t* __restrict__ slot_rows, int tile_id) {
+                                                   const int32_t* __restrict__ slot_rows, int nth) {
   constexpr int RP = 16 * NB, PR = RP + 1;
   __shared__ float part[kTileRows][PR];
   const int tid = threadIdx.x;
+  const int tile_id = work_item(a.wl_tiles, nth);
+  if (tile_id < 0) return;  // past the end of this rank class's list
   const int slot0 = tile_id * kTileRows;
   // independent loads first: group id, this tile's row indices, the slices themselves
   const int g = tile_group[tile_id];
+  // (with several rank classes most tiles belong to another launch: look before reading their slices)
+  if (a.class_mode && (g < 0 || class_rank(a.rank[g], a.rank_lo, RP) <= 0)) return;
   const int my_row = slot_rows[slot0 + (tid & 31)];
   const float* tile_part = a.hpart + (int64_t)tile_id * a.kslices * (kTileRows * RP);
   constexpr int NI = (kTileRows * RP + 255) / 256;
@@ -441,7 +450,7 @@ __device__ __forceinline__ void shrink_finish_body(const PassArgs& a, bf16_t* __
       for (int k = 0; k < 8; ++k) sums[i] += v[i][k];
   }
   const int gg = max(g, 0);
-  const int rk = a.rank[gg];
+  const int rk = class_rank(a.rank[gg], a.rank_lo, RP);
   const float sc = a.scale[gg];
   if (g < 0 || rk <= 0) return;
   const int cnt = __popcll(__ballot(my_row >= 0) & 0xffffffffull);  // padding is at the end of a tile
@@ -496,7 +505,9 @@ __device__ __forceinline__ void expand_flat_body(const PassArgs& a, const bf16_t
   // and the in-place update runs faster (probe: 43 us against 54 us for 256 MB touched in tiles of 32 random rows
   // taken from windows of 512 rows instead of from all 16384).
   const int nth = item / ngroups;
-  const int tile_id = tile_walk ? tile_walk[nth] : nth;
+  // (one of several rank classes: the class's own list of tiles, which is in the same walk order)
+  const int tile_id = a.wl_tiles.ids ? work_item(a.wl_tiles, nth) : (tile_walk ? tile_walk[nth] : nth);
+  if (tile_id < 0) return;
   const int c0 = (item - nth * ngroups) << 7;
   const int slot0 = tile_id * kTileRows;
   // independent first loads: group id, row indices, h operand (nothing branches before the
@@ -524,7 +535,8 @@ __device__ __forceinline__ void expand_flat_body(const PassArgs& a, const bf16_t
       rok[tt][v] = g_raw >= 0 && rows[tt][v] >= 0;
       yp[tt][v] = (bf16_t*)a.dst + (int64_t)(rok[tt][v] ? rows[tt][v] : 0) * a.ld_dst + 8 * li + c0;
     }
-  const int r = g_raw < 0 ? 0 : min(a.rank[g], RP);
+  const int r = g_raw < 0 ? 0 : class_rank(a.rank[g], a.rank_lo, RP);
+  if (a.class_mode && r <= 0) return;  // a tile of another rank class: its rows are not even requested
   const bf16_t* W2 = group_weight<bf16_t>(a.w_expand, a.w_expand_base, a.expand_group_stride, g);
   uint4 y[2][4];
   uint4 bq[8][NKS];
@@ -612,7 +624,12 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
   // (the flags and the order entry are requested together: one round trip in front of the tile's first loads)
   int swept_set = 0;
   bool sweep = false;
-  if (set_walk != nullptr) {
+  if (a.wl_sets.ids != nullptr) {
+    // one of several rank classes: the class's list of sets, already in the order to take them in
+    swept_set = work_item(a.wl_sets, blockIdx.x / nbt);
+    if (swept_set < 0) return;
+    sweep = true;
+  } else if (set_walk != nullptr) {
     swept_set = set_walk[blockIdx.x / nbt];
     uint2 moved = make_uint2(0u, 0u);
     if (lane < sort_blocks) moved = reinterpret_cast<const uint2*>(round_moved)[lane];
@@ -658,7 +675,7 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
   uint4 bq[8][NKS];
   int r = 0;
   auto load_weights = [&](int g) {  // this wave's block of W2 for group g
-    r = min(a.rank[g], RP);
+    r = class_rank(a.rank[g], a.rank_lo, RP);
     const bf16_t* W2 = group_weight<bf16_t>(a.w_expand, a.w_expand_base, a.expand_group_stride, g);
 #pragma unroll
     for (int q = 0; q < 8; ++q)
@@ -773,7 +790,7 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
       const int no = (int)(u % n8);
       const int64_t q = u / n8;
       const int mo = (int)(q % m8), g = (int)(q / m8);
-      const int r = min(rank[g], rpad);
+      const int r = class_rank(rank[g], t.rank_lo, rpad);
       if (8 * no >= r && t.skip_dead) continue;
       const void* B = t.lora_B[g];
       const int64_t b0 = (int64_t)(8 * mo) * t.ldb + 8 * no;
@@ -805,7 +822,7 @@ __device__ inline void transpose_weights_job(const TransposeJob& t, const int32_
       const int no = (int)(v % n8);
       const int64_t q = v / n8;
       const int ko = (int)(q % k8), g = (int)(q / k8);
-      const int r = min(rank[g], rpad);
+      const int r = class_rank(rank[g], t.rank_lo, rpad);
       if (8 * no >= r && t.skip_dead) continue;
       const void* A = t.lora_A[g];
       const int64_t a0 = (int64_t)(8 * no) * t.lda + 8 * ko;
@@ -869,10 +886,12 @@ __global__ __launch_bounds__(64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo*
   }
   // column block fastest: blocks that run together read neighbouring pieces of the same rows
   const int c0 = blockIdx.x * 128;
-  const ChunkInfo ci = chunks[blockIdx.y - a.tr.y_blocks];
+  const int cidx = work_item(a.wl_chunks, blockIdx.y - a.tr.y_blocks);
+  if (cidx < 0) return;  // past the end of this rank class's list
+  const ChunkInfo ci = chunks[cidx];
   const int g = ci.group;
   if (g < 0) return;
-  const int r = min(a.rank[g], 16 * NB);
+  const int r = class_rank(a.rank[g], a.rank_lo, 16 * NB);
   if (r <= 0) return;
   const int nt = ci.ntiles;
   for (int i = tid; i < nt * kTileRows; i += 64) rows_s[i] = slot_rows[ci.tile0 * kTileRows + i];
@@ -976,10 +995,12 @@ __device__ __forceinline__ void wgrad_coop_body(const WgradArgs& a, const ChunkI
     return;
   }
   const int c0 = bx * 128;
-  const ChunkInfo ci = chunks[by - a.tr.y_blocks];
+  const int cidx = work_item(a.wl_chunks, by - a.tr.y_blocks);
+  if (cidx < 0) return;  // past the end of this rank class's list
+  const ChunkInfo ci = chunks[cidx];
   const int g = ci.group;
   if (g < 0) return;
-  const int r = min(a.rank[g], 16 * NB);
+  const int r = class_rank(a.rank[g], a.rank_lo, 16 * NB);
   if (r <= 0) return;
   const int nt = ci.ntiles;
   for (int i = tid; i < nt * kTileRows; i += RS * 64) rows_s[i] = slot_rows[ci.tile0 * kTileRows + i];
@@ -1114,10 +1135,12 @@ __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* co
                           (int64_t)a.tr.y_blocks * x_blocks * 256);
     return;
   }
-  const ChunkInfo ci = chunks[by - a.tr.y_blocks];
+  const int cidx = work_item(a.wl_chunks, by - a.tr.y_blocks);
+  if (cidx < 0) return;  // past the end of this rank class's list
+  const ChunkInfo ci = chunks[cidx];
   const int g = ci.group;
   if (g < 0) return;
-  const int r = min(a.rank[g], RP);
+  const int r = class_rank(a.rank[g], a.rank_lo, RP);
   if (r <= 0) return;
   const int slab = bx;
   const int c0 = slab * 512 + wave * 128;

@@ -538,6 +538,55 @@ __global__ __launch_bounds__(kOneWaves * 64) void k_seg_one(const KeyT* __restri
   }
 }
 
+// ---------------------------------------------------------------------------
+// Work lists of the rank classes of one call (see WorkList): block (list, class) walks the items of its kind in the
+// order the consumer wants them (tiles and sets of four tiles in sweep order when rows are gathered, everything else
+// as numbered) and keeps those that hold a tile (a chunk) of a group whose rank lies in the class.  A stream
+// compaction with a block-wide scan per 1024 items: the lists are dense, ordered, and the same on every run.
+// ---------------------------------------------------------------------------
+struct ClassListArgs {
+  const int32_t* rank;
+  int32_t n, map_rows;
+  int32_t lo[kMaxClasses], hi[kMaxClasses];
+  char* base[kMaxClasses];
+};
+
+__global__ __launch_bounds__(1024) void k_class_lists(ClassListArgs p, ClassListLayout CL, SegView V, int max_tiles,
+                                                      int max_chunks) {
+  __shared__ int wave_sums[17];
+  const int which = blockIdx.x, c = blockIdx.y, tid = threadIdx.x;
+  const int lo = p.lo[c], hi = p.hi[c];
+  int32_t* out = (int32_t*)(p.base[c] + CL.off[which]);
+  const int n_items = (int)CL.items[which];
+  const int unit = which == kListTiles ? 1 : which == kListPairs ? 2 : which == kListOcts ? 8 : kSetTiles;
+  const int32_t* order = nullptr;
+  if (p.map_rows && which == kListTiles) order = V.tile_order;
+  if (p.map_rows && which == kListSets) order = V.set_order;
+  int running = 0;
+  for (int base = 0; base < n_items; base += 1024) {
+    const int i = base + tid;
+    int id = 0, keep = 0;
+    if (i < n_items) {
+      id = order ? order[i] : i;
+      if (which == kListChunks) {
+        const int g = id < max_chunks ? V.chunks[id].group : -1;
+        keep = g >= 0 && class_rank(p.rank[g], lo, hi) > 0;
+      } else if (id >= 0 && id < n_items) {  // (an order entry is an item number; checked all the same)
+        for (int u = 0; u < unit; ++u) {
+          const int t = id * unit + u;
+          const int g = t < max_tiles ? V.tile_group[t] : -1;
+          keep |= g >= 0 && class_rank(p.rank[g], lo, hi) > 0;
+        }
+      }
+    }
+    int total;
+    const int at = block_exclusive_scan(keep, wave_sums, &total);
+    if (keep) out[running + at] = id;
+    running += total;
+  }
+  if (tid == 0) ((int32_t*)p.base[c])[which] = running;
+}
+
 // 16 bytes of a row: the unit the row movers below load and store when width, strides and pointers allow
 // (V = 8 bf16 / 4 fp32 elements), else V = 1.  The arithmetic per element and the order of every sum are the
 // same for both.
@@ -678,6 +727,23 @@ int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t 
   else
     hipLaunchKernelGGL(k_seg_scatter<int64_t>, dim3(nblk), dim3(64), lds, s, (const int64_t*)keys, (int)rows, groups,
                        key_bits, V, perm_out);
+  return check_launch();
+}
+
+int launch_class_lists(const int32_t* rank, int n, const RankClass* rc, void* const* lists, int map_rows,
+                       const SegView& seg, const SegLayout& L, hipStream_t s) {
+  if (n <= 0 || n > kMaxClasses) return TK_ERR_INVALID;
+  ClassListArgs p{};
+  p.rank = rank;
+  p.n = n;
+  p.map_rows = map_rows;
+  for (int c = 0; c < n; ++c) {
+    p.lo[c] = rc[c].lo;
+    p.hi[c] = rc[c].hi;
+    p.base[c] = (char*)lists[c];
+  }
+  hipLaunchKernelGGL(k_class_lists, dim3(kNumLists, (unsigned)n), dim3(1024), 0, s, p, ClassListLayout(L), seg,
+                     (int)L.max_tiles, (int)L.max_chunks);
   return check_launch();
 }
 

@@ -183,6 +183,30 @@ static inline int32_t rank_pad(int32_t max_rank) {
 }
 static inline int elt_bytes(int dtype) { return dtype == TK_DTYPE_BF16 ? 2 : 4; }
 
+// Rank classes (tk_lora_desc::rank_classes).  A launch serves the groups whose rank lies in (lo, hi]: hi is the
+// launch's padded rank, lo the padded rank of the class below (0 for the lowest class or when there is one class
+// only).  Every kernel turns a group's rank into its live rank with this: 0 (skip) outside the window.
+TK_HD static inline int class_rank(int r, int lo, int hi) { return (r > lo && r <= hi) ? r : 0; }
+constexpr int kMaxClasses = 4;
+struct RankClass {
+  int32_t lo, hi;  // ranks lo < r <= hi; hi is the max_rank of the class's descriptor
+};
+// The classes of a descriptor, lowest first; one class (0, max_rank] unless the caller listed several.
+static inline int rank_classes_of(const tk_lora_desc& d, RankClass (&out)[kMaxClasses]) {
+  static const int32_t bound[kMaxClasses + 1] = {0, 16, 32, 64, 128};
+  int n = 0;
+  const int m = d.rank_classes & ((1 << kMaxClasses) - 1);
+  if ((m & (m - 1)) != 0) {  // more than one bit
+    for (int c = 0; c < kMaxClasses; ++c)
+      if (((m >> c) & 1) && bound[c] < d.max_rank) out[n++] = RankClass{bound[c], std::min(bound[c + 1], d.max_rank)};
+  }
+  if (n <= 1) {
+    out[0] = RankClass{0, d.max_rank};
+    n = 1;
+  }
+  return n;
+}
+
 // The MFMA shrink kernel covers the source width with blocks of shrink_waves() waves, each wave
 // taking kShrinkSteps steps of 64 columns; wider sources are split over several blocks whose
 // partial sums meet in a global buffer.
@@ -270,6 +294,37 @@ struct BwdLayout {
   }
 };
 
+// Work list of a launch that serves one rank class out of several: the ids of the work items (tiles, pairs of tiles,
+// chunks ..) that hold a group of the class, and their number, both on the device (built per call by
+// launch_class_lists from the segment table and the ranks).  The grid still covers every item of the table; blocks
+// past *count leave at once, and the live ones are dense at the front.  ids == nullptr: items are taken as numbered.
+struct WorkList {
+  const int32_t* ids;
+  const int32_t* count;
+};
+enum { kListTiles = 0, kListPairs = 1, kListOcts = 2, kListSets = 3, kListChunks = 4, kNumLists = 5 };
+// One class's lists inside a caller-provided buffer: counts[8], then the five id arrays.
+struct ClassListLayout {
+  int64_t off[kNumLists], items[kNumLists], total;
+  explicit ClassListLayout(const SegLayout& L) {
+    items[kListTiles] = L.max_tiles;                          // tiles, in sweep order when rows are gathered
+    items[kListPairs] = ceil_div(L.max_tiles, 2);             // tiles 2 p, 2 p + 1
+    items[kListOcts] = ceil_div(L.max_tiles, 8);              // tiles 8 o .. 8 o + 7
+    items[kListSets] = ceil_div(L.max_tiles, kSetTiles);      // tiles 4 s .. 4 s + 3, in set order when rows are gathered
+    items[kListChunks] = L.max_chunks;
+    int64_t o = 256;                                          // counts
+    for (int i = 0; i < kNumLists; ++i) {
+      off[i] = o;
+      o += round_up(4 * (items[i] + 1), 256);
+    }
+    total = o;
+  }
+  WorkList list(const void* base, int which) const {
+    return WorkList{(const int32_t*)((const char*)base + off[which]), (const int32_t*)base + which};
+  }
+};
+static inline int64_t class_list_bytes(int64_t rows, int64_t groups) { return ClassListLayout(SegLayout(rows, groups)).total; }
+
 // Everything one pass of the (shrink, expand) pair needs.  The forward pass
 // and the input-gradient pass are the same computation with the roles of the
 // weights swapped, so both are described by this one struct.
@@ -294,6 +349,10 @@ struct PassArgs {
   // the expand weight's rows are permuted inside every group of 128 (TransposeJob::swizzle_a): the row of
   // column c0 + 8 i + q lies at c0 + 16 q + i, so that the 16 rows one MFMA operand load touches are adjacent
   int32_t expand_swizzled;
+  // groups whose rank is not in (rank_lo, rpad] are skipped (see class_rank); class_mode != 0 says that such groups
+  // may exist, and kernels then look at the rank before they request a tile's rows
+  int32_t rank_lo, class_mode;
+  WorkList wl_tiles, wl_pairs, wl_octs, wl_sets;  // class_mode: the items of this class (see WorkList)
 };
 
 // Optional side job of a weight-gradient launch (bf16 MFMA path): the first `y_blocks` rows of the
@@ -309,6 +368,7 @@ struct TransposeJob {
   int32_t swizzle_a; // aT rows permuted inside every 128 (see PassArgs::expand_swizzled); in_features % 128 == 0
   int32_t skip_dead; // leave entries at and beyond a group's rank unwritten (the MFMA kernels never read them)
   int32_t src_f32;   // lora_A / lora_B hold fp32 (lda, ldb in fp32 elements); the copies are bf16 all the same
+  int32_t rank_lo;   // groups of rank <= rank_lo (or above the padded rank) are skipped
 };
 
 // Row-contraction (weight gradient) pass: out_g[n][c] = sum_p hT[n][p] * src[row(p)][c].
@@ -326,6 +386,8 @@ struct WgradArgs {
   int32_t rpad;
   int32_t grad_f32;    // the gradients (and the adapter weights a kernel reads next to them) are fp32 whatever the
                        // element type of src (tk_lora_desc::weights_f32)
+  int32_t rank_lo;     // groups whose rank is not in (rank_lo, rpad] are skipped (see class_rank)
+  WorkList wl_chunks;  // several rank classes: the chunks of this class
   TransposeJob tr;
 };
 
@@ -410,6 +472,9 @@ int launch_swiglu(const void* gate_up, int64_t ld_in, const void* dout, int64_t 
                   int64_t rows, int inter, int dtype, hipStream_t s);
 
 // kernels_segments.hip
+// work lists of `n` rank classes (ranks in (lo[c], hi[c]]) into lists[c] (ClassListLayout each)
+int launch_class_lists(const int32_t* rank, int n, const RankClass* rc, void* const* lists, int map_rows,
+                       const SegView& seg, const SegLayout& L, hipStream_t s);
 int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t groups, int64_t* perm_out,
                          int64_t* offsets_out, void* ws, hipStream_t s);
 int launch_permute(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, const void* w, const void* ws,
@@ -427,7 +492,7 @@ int launch_wgrad_generic(const WgradArgs& a, const SegView& seg, const SegLayout
 // sums the chunk partials of up to two contractions (dA, dB; either may be null) in one launch
 int launch_wgrad_reduce(const WgradArgs* a0, const WgradArgs* a1, const SegView& seg, const SegLayout& L, int dtype,
                         hipStream_t s);
-int launch_transpose_weights(const tk_lora_desc& d, void* bT, void* aT, hipStream_t s);
+int launch_transpose_weights(const tk_lora_desc& d, int rank_lo, void* bT, void* aT, hipStream_t s);
 
 // kernels_optim.hip : multi-tenant gradient norm and AdamW
 int launch_opt_grad_norm(const tk_opt_tensor* tensors, int n_tensors, const tk_opt_tenant* tenants, int n_tenants,

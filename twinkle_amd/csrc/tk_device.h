@@ -26,6 +26,12 @@ __device__ inline const T* group_weight(const void* const* ptrs, const void* bas
   return ptrs ? (const T*)ptrs[g] : (const T*)base + (int64_t)g * stride;
 }
 
+// Work item i of a launch: the i-th id of the launch's work list, -1 past its end (see WorkList); i itself without one.
+__device__ inline int work_item(const WorkList& wl, int i) {
+  if (!wl.ids) return i;
+  return i < *wl.count ? wl.ids[i] : -1;
+}
+
 inline int check_launch() { return hipGetLastError() == hipSuccess ? TK_OK : TK_ERR_LAUNCH; }
 
 }  // namespace tk
