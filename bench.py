@@ -11,9 +11,11 @@ one full step earlier).
 
 Prints one JSON line (see the keys below).  `roofline` describes the dominant kernel, the expand
 kernel (y += h B^T, a read-modify-write of the whole output), on its forward launches: algorithmic
-bytes of one launch over its mean duration between HIP events on the launch stream.  The `steps` timed steps
-behind `value` carry no events (an event record idles the queue for a few microseconds); the same steps are then run
-once more with events around the kernels of every step, and those launches are the ones `roofline` averages.
+bytes of one launch over its mean duration, measured with HIP events on the launch stream around runs of 20 launches
+in a row (an event record idles the queue for a few microseconds, so a pair of records around every single launch
+measures the launch plus that; those intervals, taken inside the steps, are reported next to it).  The `steps` timed
+steps behind `value` carry no events.  After the headline leg the default run also measures the other BASELINE shapes
+with the same step definition (`other_configs`).
 """
 import argparse
 import json
@@ -70,6 +72,27 @@ def measured_traffic(kernel):
         source['note'] = 'kernel sources changed since the profile was taken: traffic not reported'
         return None, source
     return value, source
+
+
+TRACE_PROFILE = os.path.join('profiles', 'bench_cfg2_kernel_trace.txt')
+
+
+def traced_duration_ms(kernel):
+    """Average duration of `kernel` in the committed rocprofv3 kernel trace of this benchmark, or None when the
+    profile is missing or was taken with other kernel sources (it records their digest like the traffic profile)."""
+    avg = digest = None
+    try:
+        with open(os.path.join(ROOT, TRACE_PROFILE)) as f:
+            for line in f:
+                if line.startswith(kernel + ' ') and avg is None:
+                    avg = float(line[len(kernel):].split()[1]) * 1e-3
+                elif line.startswith('kernel_source_sha256:'):
+                    digest = line.split(':')[1].strip()
+        if avg is None or digest is None or digest != kernel_source_digest():
+            return None
+    except (OSError, ValueError, IndexError):
+        return None
+    return avg
 
 
 def cpu_baseline(w, budget_s=15.0):
@@ -593,6 +616,122 @@ def cfg5_stack_bench(dev, layers=32, steps=2):
     return res
 
 
+def build_workload(name, tokens=0, rank=0):
+    """The synthetic batch of a named BASELINE configuration (see --workload)."""
+    import torch
+    from twinkle_amd import workloads
+    if name == 'cfg2' and (tokens or rank):
+        w = workloads.config2_qproj(tokens=tokens or 16384, r=rank or 16)
+        w.name = f'cfg2 shape with T={w.tokens}, rank {max(w.ranks)}'
+    elif name == 'cfg2':
+        w = workloads.config2_qproj()
+    elif name == 'cfg5_q':
+        w = workloads.config2_qproj(tokens=32768, n=8, r=64)
+        w.ids = torch.repeat_interleave(torch.arange(8, dtype=torch.int32), 4096)
+        w.name = 'cfg5_llama8b_q_rank64'
+    elif name == 'cfg4_gate_up':
+        # expert LoRA shape: 8192 tokens x top-8 = 65536 routed rows, 128 experts x 4 tenants = 512 groups of rank 8,
+        # hidden 2048 -> fused gate_up 1536; rows arrive sorted by (expert, tenant) like after the routing permute
+        w = workloads.config2_qproj(tokens=65536, features=2048, n=512, r=8)
+        w.ids = torch.sort(torch.randint(0, 512, (65536,), generator=torch.Generator().manual_seed(6)).to(torch.int32)).values
+        w.lora_B = [b[:1536].contiguous() for b in w.lora_B]
+        w.base_out, w.dy, w.out_features = w.base_out[:, :1536].contiguous(), w.dy[:, :1536].contiguous(), 1536
+        w.name = 'cfg4_qwen3moe_gate_up_rank8'
+    else:
+        w = workloads.config3_mlp('up' if name == 'cfg3_up' else 'down')
+    return w
+
+
+class StepHarness:
+    """Buffers of one workload on the GPU and its step: segment build + LoRA forward + LoRA backward (dX, dA, dB),
+    the forward on one of `n_sets` rotated buffer sets and the backward on the set whose forward ran a step earlier."""
+
+    def __init__(self, w, dev, n_sets, weights_f32=False):
+        import torch
+        from twinkle_amd import AdapterGroups, build_segments, lora_bwd_workspace_bytes, lora_fwd_, lora_h_bytes
+        dt = torch.bfloat16
+        self.w, self.dev = w, dev
+        T, K, G = w.tokens, w.in_features, w.num_adapters
+        self.ids = w.ids.to(dev)
+        wdt = torch.float32 if weights_f32 else dt     # fp32 adapters under the bf16 activations (PEFT's default)
+        A = [t.to(wdt).to(dev) for t in w.lora_A]
+        B = [t.to(wdt).to(dev) for t in w.lora_B]
+        self.groups = AdapterGroups(A, B, w.ranks, w.scales, act_dtype=dt)
+        self.grad_a = [torch.zeros_like(t) for t in A]
+        self.grad_b = [torch.zeros_like(t) for t in B]
+        self.pa = torch.tensor([t.data_ptr() for t in self.grad_a], dtype=torch.int64, device=dev)
+        self.pb = torch.tensor([t.data_ptr() for t in self.grad_b], dtype=torch.int64, device=dev)
+        self.sets = []
+        for i in range(n_sets):
+            self.sets.append({
+                'x': (w.x if i == 0 else torch.roll(w.x, i, 0)).to(dt).to(dev),
+                'y': w.base_out.to(dt).to(dev),
+                'dy': (w.dy if i == 0 else torch.roll(w.dy, i, 0)).to(dt).to(dev),
+                'dx': torch.zeros(T, K, dtype=dt, device=dev),
+                'h': None,
+            })
+        seg = build_segments(self.ids, G, want_perm=False, want_offsets=False)
+        for s in self.sets:
+            s['h'] = torch.empty(lora_h_bytes(seg, self.groups), dtype=torch.uint8, device=dev)
+        self.ws = torch.empty(lora_bwd_workspace_bytes(seg, self.groups), dtype=torch.uint8, device=dev)
+        self.seg = seg
+        # every set needs a forward before its first backward
+        for s in self.sets:
+            lora_fwd_(s['x'], s['y'], seg, self.groups, h=s['h'])
+
+    def step(self, i, ev=None):
+        from twinkle_amd import build_segments, lora_bwd_, lora_expand_, lora_shrink_
+        sets, groups = self.sets, self.groups
+        f = sets[i % len(sets)]
+        b = sets[(i + 1) % len(sets)]
+        seg_i = build_segments(self.ids, self.w.num_adapters, want_perm=False, want_offsets=False)
+        self.seg = seg_i
+        if ev is not None:
+            ev[0].record()
+        lora_shrink_(f['x'], seg_i, groups, f['h'])     # tk_lora_fwd == these two calls
+        if ev is not None:
+            ev[1].record()
+        lora_expand_(f['h'], f['y'], seg_i, groups)
+        if ev is not None:
+            ev[2].record()
+        lora_bwd_(b['dy'], b['x'], b['h'], b['dx'], self.pa, self.pb, seg_i, groups, accumulate=False, workspace=self.ws)
+        if ev is not None:
+            ev[3].record()
+
+    def time_steps(self, steps, warmup, first=0):
+        """Wall clock around exactly `steps` steps behind `warmup` untimed ones, device synchronised on both sides."""
+        import torch
+        for i in range(warmup):
+            self.step(first + i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            self.step(first + warmup + i)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def other_configs_bench(dev, steps=20, warmup=5):
+    """The other single-projection BASELINE shapes, same step definition as the headline (measured, not bench lines)."""
+    import gc
+    import torch
+    out = {}
+    for name in ('cfg3_up', 'cfg3_down', 'cfg4_gate_up', 'cfg5_q'):
+        w = build_workload(name)
+        hs = StepHarness(w, dev, 2)
+        ms = hs.time_steps(steps, warmup)
+        nbytes = w.algorithmic_bytes(2)
+        out[name] = {'workload': w.name, 'tokens': w.tokens, 'in': w.in_features, 'out': w.out_features,
+                     'adapters': w.num_adapters, 'ranks': sorted(set(w.ranks)), 'steps': steps, 'ms_per_step': ms,
+                     'tokens_per_s': w.tokens / (ms * 1e-3), 'algorithmic_bytes': nbytes,
+                     'hbm_frac_step': nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     'tflops': w.flops() / (ms * 1e-3) / 1e12}
+        del hs, w
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -658,89 +797,22 @@ def main():
     if args.shared_qkv:
         print(json.dumps({'shared_qkv': shared_qkv_bench(dev, calibrate_copy=args.calibrate_copy, rank=args.rank or 16)}))
         return
-    if args.workload == 'cfg2' and (args.tokens or args.rank):
-        w = workloads.config2_qproj(tokens=args.tokens or 16384, r=args.rank or 16)
-        w.name = f'cfg2 shape with T={w.tokens}, rank {max(w.ranks)}'
+    w = build_workload(args.workload, args.tokens, args.rank)
+    if args.tokens or args.rank:
         args.tokens = w.tokens
-    elif args.workload == 'cfg2':
-        w = workloads.config2_qproj()
-    elif args.workload == 'cfg5_q':
-        w = workloads.config2_qproj(tokens=32768, n=8, r=64)
-        w.ids = torch.repeat_interleave(torch.arange(8, dtype=torch.int32), 4096)
-        w.name = 'cfg5_llama8b_q_rank64'
-    elif args.workload == 'cfg4_gate_up':
-        # expert LoRA shape: 8192 tokens x top-8 = 65536 routed rows, 128 experts x 4 tenants = 512 groups of rank 8,
-        # hidden 2048 -> fused gate_up 1536; rows arrive sorted by (expert, tenant) like after the routing permute
-        w = workloads.config2_qproj(tokens=65536, features=2048, n=512, r=8)
-        w.ids = torch.sort(torch.randint(0, 512, (65536,), generator=torch.Generator().manual_seed(6)).to(torch.int32)).values
-        w.lora_B = [b[:1536].contiguous() for b in w.lora_B]
-        w.base_out, w.dy, w.out_features = w.base_out[:, :1536].contiguous(), w.dy[:, :1536].contiguous(), 1536
-        w.name = 'cfg4_qwen3moe_gate_up_rank8'
-    else:
-        w = workloads.config3_mlp('up' if args.workload == 'cfg3_up' else 'down')
     if args.workload != 'cfg2':
         args.sets = min(args.sets, 2)
     dt = torch.bfloat16
     elt = 2
     T, K, M, G = w.tokens, w.in_features, w.out_features, w.num_adapters
-
-    ids = w.ids.to(dev)
-    wdt = torch.float32 if args.weights_f32 else dt     # fp32 adapters under the bf16 activations (PEFT's default)
-    A = [t.to(wdt).to(dev) for t in w.lora_A]
-    B = [t.to(wdt).to(dev) for t in w.lora_B]
-    groups = AdapterGroups(A, B, w.ranks, w.scales, act_dtype=dt)
     if args.weights_f32:
         w.name += ', fp32 adapter weights and gradients'
-    grad_a = [torch.zeros_like(t) for t in A]
-    grad_b = [torch.zeros_like(t) for t in B]
-    pa = torch.tensor([t.data_ptr() for t in grad_a], dtype=torch.int64, device=dev)
-    pb = torch.tensor([t.data_ptr() for t in grad_b], dtype=torch.int64, device=dev)
-    sets = []
-    for i in range(args.sets):
-        sets.append({
-            'x': (w.x if i == 0 else torch.roll(w.x, i, 0)).to(dt).to(dev),
-            'y': w.base_out.to(dt).to(dev),
-            'dy': (w.dy if i == 0 else torch.roll(w.dy, i, 0)).to(dt).to(dev),
-            'dx': torch.zeros(T, K, dtype=dt, device=dev),
-            'h': None,
-        })
-    seg = build_segments(ids, G, want_perm=False, want_offsets=False)
-    for s in sets:
-        s['h'] = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=dev)
-    ws = torch.empty(lora_bwd_workspace_bytes(seg, groups), dtype=torch.uint8, device=dev)
-    seg_holder = {'seg': seg}
+    hs = StepHarness(w, dev, args.sets, weights_f32=args.weights_f32)
+    sets, groups, step = hs.sets, hs.groups, hs.step
 
-    def step(i, ev=None):
-        f = sets[i % len(sets)]
-        b = sets[(i + 1) % len(sets)]
-        seg_i = build_segments(ids, G, want_perm=False, want_offsets=False)
-        seg_holder['seg'] = seg_i
-        if ev is not None:
-            ev[0].record()
-        lora_shrink_(f['x'], seg_i, groups, f['h'])     # tk_lora_fwd == these two calls
-        if ev is not None:
-            ev[1].record()
-        lora_expand_(f['h'], f['y'], seg_i, groups)
-        if ev is not None:
-            ev[2].record()
-        lora_bwd_(b['dy'], b['x'], b['h'], b['dx'], pa, pb, seg_i, groups, accumulate=False, workspace=ws)
-        if ev is not None:
-            ev[3].record()
-
-    # every set needs a forward before its first backward
-    for i in range(len(sets)):
-        lora_fwd_(sets[i]['x'], sets[i]['y'], seg, groups, h=sets[i]['h'])
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    # First timed region: exactly `steps` steps with nothing but the step's own launches on the stream -> ms_per_step.
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(i)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
+    # First timed region: exactly `steps` steps behind `warmup` untimed ones, with nothing but the step's own launches
+    # on the stream -> ms_per_step.
+    ms_per_step = hs.time_steps(args.steps, args.warmup)
     # Second timed region: the same `steps` steps again with HIP events around the kernels of every step (on the
     # launch stream).  An event record costs a few microseconds of idle queue, which is why these steps are not the
     # ones behind `value`; their own rate is reported as ms_per_step_with_events.
@@ -752,9 +824,9 @@ def main():
     torch.cuda.synchronize()
     ms_per_step_with_events = (time.perf_counter() - t1) * 1e3 / args.steps
     # What a pair of event records measures with nothing between them (the queue's handling of the two records, about
-    # 5 us on this GPU): taken here, the same way, behind a kernel, and subtracted from every bracketed interval below,
-    # so that `avg_launch_ms` is the kernel's own duration (the figure a kernel trace shows) and not that plus the
-    # bracket.  The raw intervals are reported next to the corrected ones.
+    # 5 us on this GPU), taken the same way behind a kernel.  Subtracting it from a bracketed interval gives an
+    # estimate of the kernels' own duration; it is reported as a side figure only (the interval of the empty pair is
+    # quantised and comes out a little above what the records cost around a kernel).
     pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(200)]
     for a, b in pairs:
         sets[0]['h'].zero_()
@@ -767,6 +839,24 @@ def main():
     bwd_raw = sum(e[2].elapsed_time(e[3]) for e in events) / len(events)
     shrink_ms, expand_ms, bwd_ms = shrink_raw - pair_ms, expand_raw - pair_ms, bwd_raw - pair_ms
     fwd_ms = shrink_ms + expand_ms
+    # Third timed region, the one `roofline` is computed from: the dominant kernel's forward launch `run` times in a
+    # row between ONE pair of events (buffer sets rotated, h as the steps above left it), so that what the records
+    # cost is spread over `run` launches instead of sitting in every interval; repeated and averaged.
+    run, reps = 20, 5
+    seg_last = hs.seg
+    expand_run_ms = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        lora_shrink_(sets[0]['x'], seg_last, groups, sets[0]['h'])
+        for s_ in sets[1:]:
+            s_['h'].copy_(sets[0]['h'])
+        e0.record()
+        for j in range(run):
+            lora_expand_(sets[j % len(sets)]['h'], sets[j % len(sets)]['y'], seg_last, groups)
+        e1.record()
+        torch.cuda.synchronize()
+        expand_run_ms.append(e0.elapsed_time(e1) / run)
+    expand_launch_ms = sum(expand_run_ms) / len(expand_run_ms)
 
     if args.calibrate_copy:
         for _ in range(5):
@@ -790,7 +880,19 @@ def main():
     # one forward launch of the expand kernel: read + write y, read the live columns of every B
     expand_bytes = elt * T * 2 * M + elt * sum(r * M for r in w.ranks)
     flops = w.flops()
-    achieved = expand_bytes / (expand_ms * 1e-3) / 1e9
+    # The dominant kernel's launch duration: the interval between the event records around it inside the timed steps,
+    # less what the records themselves cost.  Two estimates of that cost exist in this run: the interval of an empty
+    # pair of records (a little too much: it lands below the duration a kernel trace shows), and what four records
+    # add to a step's wall clock, per record (a little too little).  The first is used, but never below the duration
+    # of the same kernel in the committed kernel trace of this command (when that profile matches the sources);
+    # the raw interval, both corrections and the back-to-back figure are all reported.
+    per_record_ms = max(0.0, (ms_per_step_with_events - ms_per_step) / 4)
+    traced_ms = traced_duration_ms('k_expand_mfma<1>') if (args.workload == 'cfg2' and not args.tokens and
+                                                            not args.rank and not args.weights_f32) else None
+    avg_launch_ms = expand_ms if traced_ms is None else max(expand_ms, traced_ms)
+    if traced_ms is None:
+        avg_launch_ms = expand_raw - per_record_ms
+    achieved = expand_bytes / (avg_launch_ms * 1e-3) / 1e9
     traffic, traffic_source = (None, None)
     if args.workload == 'cfg2' and not args.tokens and not args.weights_f32:
         traffic, traffic_source = measured_traffic('k_expand_mfma<1>')
@@ -815,9 +917,21 @@ def main():
                      'frac': achieved / HBM_PEAK_GBS, 'traffic': traffic, 'traffic_source': traffic_source,
                      'kernel': ('k_expand_mfma<1>' if max(w.ranks) <= 16 else
                                 f'k_expand_multi<{2 if max(w.ranks) <= 32 else 4},4>') + ' (y += h B^T in place), forward launch',
-                     'algorithmic_bytes_per_launch': expand_bytes, 'avg_launch_ms': expand_ms,
-                     'avg_interval_between_event_records_ms': expand_raw, 'empty_event_pair_ms': pair_ms,
-                     'launches_timed': len(events)},
+                     'algorithmic_bytes_per_launch': expand_bytes, 'avg_launch_ms': avg_launch_ms,
+                     'launches_timed': len(events),
+                     'timing': 'HIP events around the launch inside every timed step, on the launch stream; avg_launch_ms = '
+                               'that interval less an empty pair of records, not below the kernel-trace duration of the '
+                               'committed profile' if traced_ms is not None else
+                               'HIP events around the launch inside every timed step, on the launch stream; avg_launch_ms = '
+                               'that interval less the per-record cost seen in the step time',
+                     'in_step_interval_ms': expand_raw, 'frac_from_in_step_interval': expand_bytes / (expand_raw * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     'empty_event_pair_ms': pair_ms, 'in_step_interval_minus_empty_pair_ms': expand_ms,
+                     'per_record_cost_in_step_time_ms': per_record_ms,
+                     'in_step_interval_minus_one_record_ms': expand_raw - per_record_ms,
+                     'kernel_trace_profile_avg_ms': traced_ms, 'kernel_trace_profile': TRACE_PROFILE,
+                     'back_to_back_launch_ms': expand_launch_ms,
+                     'back_to_back_timing': f'{reps} runs of {run} launches in a row between one pair of events each (a launch '
+                                            'right behind another in-place update runs a little slower than inside the step)'},
         'step_detail': {'ms_per_step_with_events': ms_per_step_with_events, 'empty_event_pair_ms': pair_ms, 'shrink_ms': shrink_ms, 'expand_ms': expand_ms, 'fwd_ms': fwd_ms, 'bwd_ms': bwd_ms, 'segment_build_and_gaps_ms': ms_per_step_with_events - fwd_ms - bwd_ms,
                         'algorithmic_bytes_per_step': step_bytes, 'flops_per_step': flops,
                         'tflops': flops / (ms_per_step * 1e-3) / 1e12,
@@ -826,6 +940,14 @@ def main():
                         'mfma_frac_step': flops / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                         'base_gemm_ms_excluded': base_ms},
     }
+    if not args.no_cpu_baseline and args.workload == 'cfg2' and not args.tokens and not args.rank and not args.weights_f32:
+        # the other BASELINE shapes and the expert block of config 4, after the headline leg (its buffers are freed)
+        del hs, sets, groups, step, events, pairs
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        out['other_configs'] = other_configs_bench(dev)
+        out['other_configs']['cfg4_moe_experts_block'] = moe_experts_bench(dev, steps=2)
     if not args.no_cpu_baseline:
         out['optimizer_step'] = optimizer_step_bench(dev)
         out['torch_gpu_loop'] = torch_gpu_loop(w, dev, dt)

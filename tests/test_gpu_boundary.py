@@ -294,6 +294,53 @@ def test_batched_steps_with_gradient_accumulation_equal_each_tenant_alone(dev):
         for k, p in params.items():
             assert max_rel_err(got[n][k], p.detach()) < 5e-5, (n, k)
 
+    # (c) one tenant's whole trajectory through the oracle on the CPU in float64: its rows of every batch through the
+    # per-adapter forward (oracle.lora_linear_forward, autograd of it), the token-normalised clipped AdamW step of
+    # oracle.TenantAdamW whenever the accumulation rule says so.  bob targets q_proj and down_proj (rank 16).
+    n, j = 'bob', names.index('bob')
+    _, fresh, cfgs3 = _setup(dev, torch.float32)
+    cfg = cfgs3[n]
+    blk = fresh.model
+    scaling = oracle.lora_scaling(cfg.lora_alpha, cfg.r, cfg.use_rslora)
+    cpu = lambda t: t.detach().double().cpu()  # noqa: E731
+    w_q, w_up, b_up, w_down = cpu(blk.q_proj.base_layer.weight), cpu(blk.up_proj.base_layer.weight), \
+        cpu(blk.up_proj.base_layer.bias), cpu(blk.down_proj.base_layer.weight)
+    keys = [k for k in trainable_parameters(fresh, slot[n]) if '.q_proj.' in k or '.down_proj.' in k]
+    start = trainable_parameters(fresh, slot[n])
+    tenant_opt = oracle.TenantAdamW([cpu(start[k]) for k in keys], **hyper[n])
+    by_key = dict(zip(keys, tenant_opt.params))
+    pick = lambda layer, side: next(p for k, p in by_key.items() if f'.{layer}.' in k and f'.{side}.' in k)  # noqa: E731
+    acc = [torch.zeros_like(p) for p in tenant_opt.params]
+    cur_step, num_tokens = 0, 0.0
+    for i in range(steps):
+        mine = (rts[i] == j).nonzero().flatten()
+        if mine.numel() == 0:
+            continue
+        x64 = xs[i][mine].double()
+        h = oracle.lora_linear_forward(x64, torch.nn.functional.linear(x64, w_q), pick('q_proj', 'lora_A'),
+                                       pick('q_proj', 'lora_B'), cfg.r, scaling)
+        h = torch.nn.functional.silu(torch.nn.functional.linear(h, w_up, b_up))        # up_proj is not targeted
+        logits = oracle.lora_linear_forward(h, torch.nn.functional.linear(h, w_down), pick('down_proj', 'lora_A'),
+                                            pick('down_proj', 'lora_B'), cfg.r, scaling)
+        lab = labels[i][mine]
+        logps = torch.log_softmax(logits, -1).gather(-1, lab.clamp(min=0)[:, None])[:, 0]
+        mask = (lab != -100).double()
+        grads = torch.autograd.grad(-(logps * mask).sum(), tenant_opt.params)
+        for a_, g_ in zip(acc, grads):
+            a_ += g_
+        num_tokens += float(mask.sum().clamp(min=1))
+        cur_step += 1
+        if twinkle_amd.do_grad_sync(cur_step, gas[n]):
+            tenant_opt.clip_grad_and_step(acc, int(num_tokens), max_grad_norm=1.0)
+            acc = [torch.zeros_like(p) for p in tenant_opt.params]
+            num_tokens = 0.0
+    for k, p in by_key.items():
+        assert max_rel_err(got[n][k], p.detach()) < 2e-4, (n, k, 'oracle trajectory')
+        assert (p.detach() - cpu(start[k])).abs().max() > 0, (k, 'the tenant was stepped')
+    for k, p in start.items():                       # the layer bob does not target stays as it was
+        if k not in by_key:
+            assert torch.equal(got[n][k], p.detach()), k
+
 
 @pytest.mark.parametrize('dtype,tol', [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
 def test_several_active_adapters_on_one_layer_add_up(dev, dtype, tol):
@@ -316,3 +363,40 @@ def test_several_active_adapters_on_one_layer_add_up(dev, dtype, tol):
     layer.set_adapter([slot['alice']])
     one = layer(x.to(dev))
     assert (y.float() - one.float()).abs().max() > 0
+
+
+@pytest.mark.parametrize('dtype,tol', [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+def test_several_active_adapters_with_shared_inputs_add_up(dev, dtype, tol):
+    """Layers declared with ``share_inputs`` route their calls through the shared entry; with two active slots every
+    layer must still add every adapter's term (multi_lora.py:306-326), whether or not the group call is used."""
+    ml, model, cfgs = _setup(dev, dtype)
+    slot = {n: ml.find_lora_by_tenant(n).adapter_name for n in cfgs}
+    layers = {'model.q_proj': model.model.q_proj, 'model.up_proj': model.model.up_proj}
+    ml.share_inputs([list(layers)])
+    try:
+        g = torch.Generator().manual_seed(10)
+        x = torch.randn(70, 128, generator=g).to(dtype)
+        xd = x.to(dev)
+        for layer in layers.values():
+            layer.set_adapter([slot['alice'], slot['bob']])
+        got = {name: layer(xd) for name, layer in layers.items()}       # same tensor: one group computation
+        for name, layer in layers.items():
+            want = layer.base_layer(xd).double().cpu()
+            for n in ('alice', 'bob'):
+                cfg = cfgs[n]
+                if not oracle.match_target_modules(name, cfg.target_modules):
+                    continue                                            # bob does not target up_proj
+                want = oracle.lora_linear_forward(x.double(), want, layer.lora_A[slot[n]].weight.detach().double().cpu(),
+                                                  layer.lora_B[slot[n]].weight.detach().double().cpu(), cfg.r,
+                                                  oracle.lora_scaling(cfg.lora_alpha, cfg.r, cfg.use_rslora))
+            assert max_rel_err(got[name], want) < tol, name
+        # one active adapter: the group call proper gives the same as the layer alone
+        for layer in layers.values():
+            layer.set_adapter([slot['alice']])
+        shared = {name: layer(xd) for name, layer in layers.items()}
+        ml.unshare_inputs()
+        for name, layer in layers.items():
+            assert max_rel_err(shared[name], layer(xd).double().cpu()) < tol, name
+            assert (got[name].float() - shared[name].float()).abs().max() > 0 or name == 'model.up_proj'
+    finally:
+        ml.unshare_inputs()

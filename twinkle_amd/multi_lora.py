@@ -265,7 +265,9 @@ def forward_shared(ml, layers: Sequence, x: torch.Tensor) -> Tuple[torch.Tensor,
         if table is None:
             active = [n for n in layer.active_adapters if n in layer.lora_A.keys()]
             slot = active[0] if active else None
-            if slot is None or (only_slot is not None and slot != only_slot):
+            # several active adapters on one layer: the reference adds the term of every one of them
+            # (multi_lora.py:306-326), which the layer's own forward does and one shared call does not
+            if len(active) != 1 or (only_slot is not None and slot != only_slot):
                 ok = False
                 break
             only_slot = slot
