@@ -85,6 +85,19 @@ int tk_segment_build(const void* keys_device, int32_t key_dtype, int64_t rows, i
 /* Synchronises the stream and copies one counter back: number of out-of-range keys. */
 int tk_segment_bad_keys(const void* seg_ws_device, tk_stream_t stream, int64_t* count_out_host);
 
+/* Checks a segment table on the host (a debugging and test aid; no counterpart in the reference): copies the whole
+ * workspace back (synchronises the stream) and rebuilds every array from the group sizes and the row order it holds.
+ * TK_OK when every entry is what tk_segment_build writes for some keys of (rows, num_groups): every row in exactly one
+ * slot, rows ascending inside a group, group / tile / chunk / partial numbers inside the table's bounds and consistent
+ * with each other.  Otherwise TK_ERR_INVALID, with the number of the first failing check (1 header, 2 offsets, 3 first
+ * tiles, 4 group of a tile, 5 slot rows / positions, 6 permutation and its inverse, 7 stable order, 8 walk orders,
+ * 9 chunks, 10 first chunks / partial slots) and the index it failed at in the two outputs (either may be NULL).
+ * The kernels themselves compare every table entry they index with against the table's bounds and skip what lies
+ * outside, so a table that was overwritten gives wrong results, not accesses outside the caller's tensors; this
+ * call is how to find out that it was. */
+int tk_segment_validate(const void* seg_ws_device, int64_t rows, int32_t num_groups, tk_stream_t stream,
+                        int32_t* failed_check_out_host, int64_t* index_out_host);
+
 /* ---------------------------------------------------------------------------
  * Row gather / weighted scatter-back in segment order.
  *

@@ -17,6 +17,7 @@ def _check(keys_cpu, groups, dev, dtype=torch.int32, num_tokens=None):
     assert torch.equal(seg.perm.cpu(), perm)
     assert torch.equal(seg.offsets.cpu(), offsets)
     assert torch.equal(seg.counts.cpu(), counts)
+    seg.validate()      # every array of the device-side table, rebuilt on the host from the sizes and the order
     return seg
 
 
@@ -139,3 +140,43 @@ def test_packed_sequences(dev):
     seg = build_segments(ids, 8)
     assert seg.offsets.tolist() == [4096 * i for i in range(9)]
     assert torch.equal(seg.perm.cpu(), torch.arange(32768))
+
+
+def test_tables_of_the_baseline_configs_validate(dev):
+    """The device-side table of every BASELINE configuration's keys passes the host-side check entry by entry
+    (config 1: contiguous segments; 2: Zipf ids shuffled; 3: uneven sizes with two empty adapters; 4: (expert, tenant)
+    keys of top-8 routing; 5: one tenant per packed sequence), and so do keys with rows that have no group."""
+    from twinkle_amd import validate_segment_table
+    cases = [(workloads.config1_plumbing().ids, 4), (workloads.zipf_ids(16384, 16), 16), (workloads.uneven_ids(32768, 32), 32),
+             (torch.repeat_interleave(torch.arange(8), 4096), 8)]
+    selected, _, tenant = workloads.moe_routing()
+    cases.append((flat_keys_from_topk(selected, tenant, 4), 512))
+    keys = workloads.zipf_ids(5000, 16).clone()
+    keys[::7] = -1
+    keys[3::11] = 16
+    cases.append((keys, 16))
+    for keys, groups in cases:
+        seg = build_segments(keys.to(torch.int32).to(dev), groups)
+        validate_segment_table(seg)
+
+
+def test_the_host_side_check_sees_a_changed_entry(dev):
+    """The check itself: a copy of a good table with one entry changed (on the copy only: no kernel ever reads it) is
+    reported, with the check that failed."""
+    import ctypes
+    from twinkle_amd import _lib
+    keys = workloads.zipf_ids(3000, 8).to(dev)
+    seg = build_segments(keys, 8)
+    seg.validate()
+    lib = _lib.load()
+    words = seg.workspace.view(torch.int32)
+    failed = set()
+    for at in (2, 64 + 5):                    # header.groups; inv[5] (the header takes 64 words)
+        copy = words.clone()
+        copy[at] += 1
+        check, index = ctypes.c_int32(0), ctypes.c_int64(-1)
+        code = lib.tk_segment_validate(copy.data_ptr(), seg.rows, seg.num_groups, _lib.stream_ptr(), ctypes.byref(check),
+                                       ctypes.byref(index))
+        assert code == _lib.TK_ERR_INVALID and check.value > 0
+        failed.add(check.value)
+    assert failed == {1, 6}

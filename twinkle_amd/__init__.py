@@ -15,6 +15,6 @@ from .ops import (AdapterGroups, grouped_linear_, swiglu, lora_bwd_, lora_bwd_sh
                   multi_lora_linear, multi_lora_linear_shared)
 from .optim import BatchedStep, MultiTenantAdamW, do_grad_sync, trainable_parameters  # noqa: F401
 from .segments import (SegmentTable, build_segments, flat_keys_from_topk, packed_cu_seqlens, permute,  # noqa: F401
-                       token_groups_from_sequences, unpermute)
+                       token_groups_from_sequences, unpermute, validate_segment_table)
 
 __version__ = '0.1.0'

@@ -79,6 +79,7 @@ EXPORTS = {
     'tk_segment_build': (c_int32, [c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_int64,
                                    c_void_p]),
     'tk_segment_bad_keys': (c_int32, [c_void_p, c_void_p, POINTER(c_int64)]),
+    'tk_segment_validate': (c_int32, [c_void_p, c_int64, c_int32, c_void_p, POINTER(c_int32), POINTER(c_int64)]),
     'tk_permute_rows': (c_int32, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_int32,
                                   c_int32, c_int32, c_void_p]),
     'tk_unpermute_rows': (c_int32, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64,

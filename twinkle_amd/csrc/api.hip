@@ -2,6 +2,7 @@
 #include <stdlib.h>
 
 #include <mutex>
+#include <vector>
 
 #include "tk_common.h"
 
@@ -249,6 +250,108 @@ int tk_segment_bad_keys(const void* seg_ws, tk_stream_t stream, int64_t* count_o
   return TK_OK;
 }
 
+// Host-side check of a segment table: the whole workspace is copied back and every array is rebuilt from the
+// group sizes and the row order it holds, entry by entry.
+int tk_segment_validate(const void* seg_ws, int64_t rows, int32_t num_groups, tk_stream_t stream,
+                        int32_t* failed_check_out, int64_t* index_out) {
+  if (!seg_ws || rows < 0 || rows >= (1ll << 31) || num_groups <= 0 || num_groups > TK_MAX_GROUPS) return TK_ERR_INVALID;
+  const SegLayout L(rows, num_groups);
+  std::vector<char> host((size_t)L.total);
+  if (hipMemcpyAsync(host.data(), seg_ws, (size_t)L.total, hipMemcpyDeviceToHost, (hipStream_t)stream) != hipSuccess)
+    return TK_ERR_LAUNCH;
+  if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return TK_ERR_LAUNCH;
+  const SegView V(host.data(), L);
+  const int G = num_groups, B = G + 1;  // buckets: the groups, then the rows without a group
+  auto fail = [&](int check, int64_t index) {
+    if (failed_check_out) *failed_check_out = check;
+    if (index_out) *index_out = index;
+    return TK_ERR_INVALID;
+  };
+  if (failed_check_out) *failed_check_out = 0;
+  if (index_out) *index_out = -1;
+  const SegHeader& h = *V.header;
+  // 1: header
+  if (h.magic != kSegMagic || h.rows != rows || h.groups != G || h.num_tiles < 0 || h.num_tiles > L.max_tiles ||
+      h.num_chunks < 0 || h.num_chunks > L.max_chunks || h.num_partials < 0 || h.num_partials > L.max_partials ||
+      h.bad_keys < 0 || h.bad_keys > rows)
+    return fail(1, 0);
+  // 2: offsets
+  if (V.offsets[0] != 0 || V.offsets[B] != rows || V.offsets[G] != rows - h.bad_keys) return fail(2, 0);
+  for (int g = 0; g < B; ++g)
+    if (V.offsets[g + 1] < V.offsets[g]) return fail(2, g);
+  // 3: first tile of every bucket
+  if (V.tile_first[0] != 0 || V.tile_first[B] != h.num_tiles) return fail(3, 0);
+  for (int g = 0; g < B; ++g)
+    if (V.tile_first[g + 1] - V.tile_first[g] != ceil_div(V.offsets[g + 1] - V.offsets[g], kTileRows)) return fail(3, g);
+  // 4: group of every tile; 5: rows and positions of every slot; 7: rows ascending inside a group
+  std::vector<int32_t> seen((size_t)rows, 0);
+  for (int g = 0; g < B; ++g) {
+    int32_t prev = -1;
+    for (int t = V.tile_first[g]; t < V.tile_first[g + 1]; ++t) {
+      if (V.tile_group[t] != (g < G ? g : -1)) return fail(4, t);
+      for (int i = 0; i < kTileRows; ++i) {
+        const int64_t s_ = (int64_t)t * kTileRows + i;
+        const int64_t pos = V.offsets[g] + (int64_t)(t - V.tile_first[g]) * kTileRows + i;
+        const int32_t row = V.slot_row[s_];
+        if (pos >= V.offsets[g + 1]) {
+          if (row != -1 || V.slot_pos[s_] != -1) return fail(5, s_);
+          continue;
+        }
+        if (V.slot_pos[s_] != pos || row < 0 || row >= rows) return fail(5, s_);
+        if (seen[row]++) return fail(6, s_);          // 6: every row exactly once
+        if (V.inv[row] != pos) return fail(6, row);   //    and inv is the inverse
+        if (row <= prev) return fail(7, s_);          // 7: stable order
+        prev = row;
+      }
+    }
+  }
+  for (int64_t t = h.num_tiles; t < L.max_tiles; ++t) {
+    if (V.tile_group[t] != -1) return fail(4, t);
+    for (int i = 0; i < kTileRows; ++i)
+      if (V.slot_row[t * kTileRows + i] != -1 || V.slot_pos[t * kTileRows + i] != -1) return fail(5, t * kTileRows + i);
+  }
+  for (int64_t r = 0; r < rows; ++r)
+    if (!seen[r]) return fail(6, r);
+  // 8: the walk orders are permutations of the tiles / of the sets of four tiles
+  {
+    std::vector<char> hit((size_t)L.max_tiles, 0);
+    for (int64_t i = 0; i < L.max_tiles; ++i) {
+      const int32_t t = V.tile_order[i];
+      if (t < 0 || t >= L.max_tiles || hit[t]++) return fail(8, i);
+    }
+    const int64_t sets = ceil_div(L.max_tiles, kSetTiles);
+    std::vector<char> hit_s((size_t)sets, 0);
+    for (int64_t i = 0; i < sets; ++i) {
+      const int32_t t = V.set_order[i];
+      if (t < 0 || t >= sets || hit_s[t]++) return fail(8, L.max_tiles + i);
+    }
+  }
+  // 9: chunks; 10: first chunk and first partial slot of every bucket
+  int32_t chunk = 0, partial = 0;
+  for (int g = 0; g < B; ++g) {
+    if (V.chunk_first[g] != chunk) return fail(10, g);
+    const int ntile = V.tile_first[g + 1] - V.tile_first[g];
+    const int nchunk = (int)ceil_div(ntile, L.chunk_tiles);
+    const bool multi = nchunk > 1 && g < G;
+    if (V.partial_first[g] != partial) return fail(10, g);
+    for (int j = 0; j < nchunk; ++j, ++chunk) {
+      if (chunk >= L.max_chunks) return fail(9, chunk);
+      const ChunkInfo& c = V.chunks[chunk];
+      if (c.group != (g < G ? g : -1) || c.tile0 != V.tile_first[g] + j * (int)L.chunk_tiles ||
+          c.ntiles != std::min<int>((int)L.chunk_tiles, ntile - j * (int)L.chunk_tiles) ||
+          c.partial != (multi ? partial + j : -1))
+        return fail(9, chunk);
+    }
+    if (multi) partial += nchunk;
+  }
+  if (V.chunk_first[B] != chunk || chunk != h.num_chunks || V.partial_first[B] != partial || partial != h.num_partials ||
+      partial > L.max_partials)
+    return fail(10, B);
+  for (int64_t c = chunk; c < L.max_chunks; ++c)
+    if (V.chunks[c].group != -1) return fail(9, c);
+  return TK_OK;
+}
+
 static bool rows_args_ok(const void* a, const void* b, const void* ws, int64_t rows, int64_t tokens, int32_t width,
                          int32_t groups, int32_t dtype) {
   if (!ws || rows < 0 || tokens < 0 || width <= 0 || groups <= 0) return false;
@@ -369,6 +472,7 @@ static PassArgs fwd_pass_args(const tk_lora_desc* d, const void* x, int64_t ldx,
                               int rank_lo = 0, int class_mode = 0) {
   PassArgs a{};
   a.rank_lo = rank_lo;  a.class_mode = class_mode;
+  a.tb = table_bounds(SegLayout(d->rows, d->num_groups));
   a.src = x ? x : h;  a.ld_src = x ? ldx : d->in_features;
   a.dst = y ? y : h;  a.ld_dst = y ? ldy : d->out_features;
   a.hT = h;   a.ldh = h_ld(d->rows, d->num_groups);
@@ -399,6 +503,7 @@ static BwdPlan bwd_plan(const tk_lora_desc* d, const BwdLayout& B, const void* d
   BwdPlan p;
   p.ga.rank_lo = p.gb.rank_lo = p.a.rank_lo = p.tr.rank_lo = rank_lo;
   p.a.class_mode = class_mode;
+  p.ga.tb = p.gb.tb = p.a.tb = table_bounds(SegLayout(d->rows, d->num_groups));
   char* w = (char*)ws;
   p.dh = w + B.off_dh;
   p.bT = w + B.off_wT_shrink;
@@ -644,6 +749,7 @@ int tk_grouped_linear(const tk_grouped_desc* g, const tk_lora_desc* lora, const 
   a.y = (uint16_t*)y;  a.ldy = ldy;
   a.K = g->in_features;  a.N = g->out_features;  a.src_rows = (int32_t)g->rows;  a.map_rows = g->map_rows;
   a.w_rows_are_inputs = g->weight_layout;
+  a.tb = table_bounds(SegLayout(g->rows, g->num_groups));
   if (lora && lora->max_rank > 0) {
     if (!desc_ok(lora) || !h) return TK_ERR_INVALID;
     if (lora->rows != g->rows || lora->num_groups != g->num_groups || lora->in_features != g->in_features ||
@@ -776,6 +882,7 @@ int tk_lora_fwd_shared(const tk_lora_desc* const* descs_in, int32_t n, const voi
   sa.src = x;  sa.ld_src = ldx;
   sa.width_src = d0->in_features;  sa.src_rows = (int32_t)d0->rows;  sa.map_rows = d0->map_rows;
   sa.kslices = a[0].kslices;  sa.nproj = n;
+  sa.tb = a[0].tb;
   for (int p = 0; p < n; ++p) {
     sa.w[p] = descs[p]->lora_A;  sa.ld_w[p] = descs[p]->lda;
     sa.rank[p] = descs[p]->rank;  sa.hpart[p] = a[p].hpart;
@@ -826,6 +933,7 @@ int tk_lora_bwd_shared(const tk_lora_desc* const* descs_in, int32_t n, const voi
       const int rpad = plan[0].a.rpad;
       SharedExpandArgs ea{};
       ea.dst = dx;  ea.ld_dst = lddx;  ea.width_dst = d0->in_features;  ea.map_rows = d0->map_rows;  ea.nproj = n;
+      ea.tb = table_bounds(L);
       SharedWgradArgs wa{};
       wa.nproj = n;
       WgradArgs red[2 * TK_MAX_SHARED] = {};
@@ -864,6 +972,7 @@ int tk_lora_bwd_shared(const tk_lora_desc* const* descs_in, int32_t n, const voi
   }
   SharedExpandArgs ea{};
   ea.dst = dx;  ea.ld_dst = lddx;  ea.width_dst = d0->in_features;  ea.map_rows = d0->map_rows;  ea.nproj = n;
+  ea.tb = table_bounds(L);
   SharedWgradArgs wa{};
   wa.nproj = n;
   DyFusedJob dj[TK_MAX_SHARED] = {};

@@ -19,7 +19,7 @@ __global__ __launch_bounds__(256) void k_shrink_generic(PassArgs a, const int32_
                                                         const int32_t* __restrict__ slot_rows) {
   extern __shared__ float lds_f[];
   const int tile_id = blockIdx.x;
-  const int g = tile_group[tile_id];
+  const int g = checked_group(tile_group[tile_id], a.tb);
   if (g < 0) return;
   const int r = class_rank(a.rank[g], a.rank_lo, a.rpad);
   if (a.class_mode && r <= 0) return;  // a group of another rank class: its tiles belong to another launch
@@ -29,7 +29,7 @@ __global__ __launch_bounds__(256) void k_shrink_generic(PassArgs a, const int32_
   __shared__ int rows_s[kTileRows];
   const int tid = threadIdx.x;
   const int slot0 = tile_id * kTileRows;
-  if (tid < kTileRows) rows_s[tid] = slot_rows[slot0 + tid];
+  if (tid < kTileRows) rows_s[tid] = checked_row(slot_rows[slot0 + tid], a.tb);
   __syncthreads();
   const T* src = (const T*)a.src;
   const T* W = group_weight<T>(a.w_shrink, a.w_shrink_base, a.shrink_group_stride, g);
@@ -82,14 +82,14 @@ __global__ __launch_bounds__(256) void k_expand_generic(PassArgs a, const int32_
                                                         const int32_t* __restrict__ slot_rows) {
   extern __shared__ float lds_f[];  // hs[rpad][32]
   const int tile_id = blockIdx.x;
-  const int g = tile_group[tile_id];
+  const int g = checked_group(tile_group[tile_id], a.tb);
   if (g < 0) return;
   const int r = class_rank(a.rank[g], a.rank_lo, a.rpad);
   if (r <= 0) return;
   __shared__ int rows_s[kTileRows];
   const int tid = threadIdx.x;
   const int slot0 = tile_id * kTileRows;
-  if (tid < kTileRows) rows_s[tid] = slot_rows[slot0 + tid];
+  if (tid < kTileRows) rows_s[tid] = checked_row(slot_rows[slot0 + tid], a.tb);
   const T* hT = (const T*)a.hT;
   for (int i = tid; i < r * kTileRows; i += 256) {
     const int n = i / kTileRows, rr = i % kTileRows;
@@ -138,7 +138,7 @@ __global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkI
   constexpr int kPass = kChunkTilesMin * kTileRows;
   __shared__ float hs[16][kPass];
   __shared__ int rows_s[kPass];
-  const ChunkInfo ci = chunks[blockIdx.x];
+  const ChunkInfo ci = checked_chunk(chunks[blockIdx.x], a.tb);
   const int g = ci.group;
   if (g < 0) return;
   const int r = class_rank(a.rank[g], a.rank_lo, a.rpad);
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkI
       const int slot0 = ci.tile0 * kTileRows + p0;
       const int len = min(kPass, total - p0);
       __syncthreads();
-      for (int i = tid; i < len; i += 256) rows_s[i] = slot_rows[slot0 + i];
+      for (int i = tid; i < len; i += 256) rows_s[i] = checked_row(slot_rows[slot0 + i], a.tb);
       for (int i = tid; i < 16 * len; i += 256) {
         const int j = i / len, pp = i % len;
         hs[j][pp] = (n0 + j) < r ? to_f32(hT[(int64_t)(n0 + j) * a.ldh + slot0 + pp]) : 0.f;
@@ -201,6 +201,8 @@ __device__ __forceinline__ void wgrad_reduce_body(const WgradArgs& a, int n0, co
   const int rk = a.rank[g], cf0 = chunk_first[g], cf1 = chunk_first[g + 1], pf = partial_first[g];
   const int r = class_rank(rk, a.rank_lo, a.rpad);
   const int nchunk = cf1 - cf0;
+  // (table entries are compared with the table's bounds before they index: see TableBounds)
+  if (nchunk < 0 || (nchunk > 1 && (pf < 0 || pf > a.tb.max_partials - nchunk))) return;
   if (nchunk == 1) return;
   if (nchunk == 0 && a.accumulate) return;
   const int64_t stride = partial_slot_floats(a.rpad, a.width);

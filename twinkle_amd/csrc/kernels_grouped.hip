@@ -44,13 +44,16 @@ constexpr int kGroupedItems = TK_GROUPED_ITEMS;  // work items aimed at per laun
 
 __global__ __launch_bounds__(256) void k_grouped_plan(const int32_t* __restrict__ tile_first, int experts, int nt,
                                                       GroupedPlanEntry* __restrict__ plan,
-                                                      int32_t* __restrict__ nblocks, int max_entries, int ptiles) {
+                                                      int32_t* __restrict__ nblocks, int max_entries, int ptiles,
+                                                      int max_tiles) {
   __shared__ int32_t sums[256];
   const int tid = threadIdx.x;
   const int per = (experts + 255) / 256;
   const int e0 = min(experts, tid * per), e1 = min(experts, e0 + per);
   int cnt = 0;
-  for (int e = e0; e < e1; ++e) cnt += (tile_first[(e + 1) * nt] - tile_first[e * nt] + ptiles - 1) / ptiles;
+  // (tile numbers come from the caller's segment table: kept inside [0, max_tiles] and ascending before they index)
+  auto first_tile = [&](int g) { return min(max(tile_first[g], 0), max_tiles); };
+  for (int e = e0; e < e1; ++e) cnt += (max(first_tile((e + 1) * nt) - first_tile(e * nt), 0) + ptiles - 1) / ptiles;
   sums[tid] = cnt;
   __syncthreads();
   for (int off = 1; off < 256; off <<= 1) {
@@ -61,7 +64,7 @@ __global__ __launch_bounds__(256) void k_grouped_plan(const int32_t* __restrict_
   }
   int at = sums[tid] - cnt;
   for (int e = e0; e < e1; ++e) {
-    const int t0 = tile_first[e * nt], t1 = tile_first[(e + 1) * nt];
+    const int t0 = first_tile(e * nt), t1 = max(first_tile((e + 1) * nt), t0);
     // the expert's tiles in `count` row blocks of (almost) equal length: blocks of equal work stay in step, and
     // blocks in step find each other's weight and x tiles in the XCD's L2 (measured at config 4, 18 tiles per expert:
     // as 8 + 8 + 2 the short block runs ahead and L2 fetches 1.6 x the compulsory bytes, as 6 + 6 + 6 it fetches
@@ -132,7 +135,7 @@ __global__ __launch_bounds__(BIG ? 512 : 256) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int r = 16 * RB * wm + 16 * rb + li;
-    out_row[rb] = r < live ? slot_rows[slot0 + r] : -1;
+    out_row[rb] = r < live ? checked_row(slot_rows[slot0 + r], a.tb) : -1;
   }
   const bf16_t* wbase = a.w + (int64_t)pe.expert * a.w_stride;
   const int nk = a.K / kGBK;
@@ -243,7 +246,7 @@ __global__ __launch_bounds__(BIG ? 512 : 256) __attribute__((amdgpu_waves_per_eu
       for (int tl = 0; tl < RB / 2; ++tl) {
         const int tile_in_block = (RB / 2) * wm + tl;
         if (tile_in_block >= pe.ntiles) break;
-        const int g = tile_group[pe.tile0 + tile_in_block];
+        const int g = checked_group(tile_group[pe.tile0 + tile_in_block], a.tb);
         const int r = g >= 0 ? min(a.rank[g], a.rpad) : 0;
         if (r <= 0) continue;
         const bf16_t* Bg = (const bf16_t*)a.lora_B[g];
@@ -525,7 +528,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
         if (rb >= pe.ntiles) break;
-        const int g = tile_group[pe.tile0 + rb];
+        const int g = checked_group(tile_group[pe.tile0 + rb], a.tb);
         const int r = g >= 0 ? min(a.rank[g], a.rpad) : 0;
         if (r <= 0) continue;
         const bf16_t* Bg = (const bf16_t*)a.lora_B[g];
@@ -553,7 +556,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2))) void k
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
       const int r = 16 * (2 * rb + wm) + li;
-      out_row[rb] = r < live ? slot_rows[slot0 + r] : -1;
+      out_row[rb] = r < live ? checked_row(slot_rows[slot0 + r], a.tb) : -1;
     }
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
@@ -600,7 +603,7 @@ int launch_grouped_gemm(const GroupedArgs& a, int experts, int nt, GroupedPlanEn
   const int ptiles = big ? 8 : 4, bn = big ? 256 : 128;
   const int max_entries = (int)(ceil_div(L.max_tiles, ptiles) + experts);
   hipLaunchKernelGGL(k_grouped_plan, dim3(1), dim3(256), 0, s, seg.tile_first, experts, nt, plan, nblocks, max_entries,
-                     ptiles);
+                     ptiles, (int)L.max_tiles);
   const int32_t* rows = seg.slot_table(a.map_rows);
   // several thousand work items, so that the last round of blocks on the 256 CUs is a small part of the run
   const int ncb = a.N / bn;

@@ -202,8 +202,9 @@ __device__ __forceinline__ void shrink_pair_body(const PassArgs& a, bf16_t* __re
   const int pair = work_item(a.wl_pairs, nth);
   if (pair < 0) return;  // past the end of this rank class's list (uniform over the block)
   const int t0 = 2 * pair, t1 = t0 + 1;
-  const int g0 = tile_group[t0];
-  const int g1 = t1 < max_tiles ? tile_group[t1] : -1;
+  if (t0 >= max_tiles) return;
+  const int g0 = checked_group(tile_group[t0], a.tb);
+  const int g1 = t1 < max_tiles ? checked_group(tile_group[t1], a.tb) : -1;
   if (g0 >= 0 && g1 == g0) {
     const int tiles[2] = {t0, t1};
     shrink_tiles<NB, NW, 2>(a, hrow, slot_rows, tiles, g0, ks, part);
@@ -278,7 +279,7 @@ __device__ __forceinline__ void shrink_quad_body(const PassArgs& a, const int32_
   const int set = work_item(a.wl_octs, nth);
   if (set < 0) return;  // past the end of this rank class's list (uniform over the block)
   const int t_first = set * 8;
-  if (tid < 8) gts[tid] = t_first + tid < max_tiles ? tile_group[t_first + tid] : -1;
+  if (tid < 8) gts[tid] = t_first + tid < max_tiles ? checked_group(tile_group[t_first + tid], a.tb) : -1;
   const int nsteps = a.width_src >> 6;
   const int s0 = ks * a.quad_steps;
   const int ns = min(a.quad_steps, nsteps - s0);  // >= 1 for every slice
@@ -421,11 +422,11 @@ __device__ __forceinline__ void shrink_finish_body(const PassArgs& a, bf16_t* __
   constexpr int RP = 16 * NB, PR = RP + 1;
   __shared__ float part[kTileRows][PR];
   const int tid = threadIdx.x;
-  const int tile_id = work_item(a.wl_tiles, nth);
+  const int tile_id = checked_tile(work_item(a.wl_tiles, nth), a.tb);
   if (tile_id < 0) return;  // past the end of this rank class's list
   const int slot0 = tile_id * kTileRows;
   // independent loads first: group id, this tile's row indices, the slices themselves
-  const int g = tile_group[tile_id];
+  const int g = checked_group(tile_group[tile_id], a.tb);
   // (with several rank classes most tiles belong to another launch: look before reading their slices)
   if (a.class_mode && (g < 0 || class_rank(a.rank[g], a.rank_lo, RP) <= 0)) return;
   const int my_row = slot_rows[slot0 + (tid & 31)];
@@ -506,13 +507,13 @@ __device__ __forceinline__ void expand_flat_body(const PassArgs& a, const bf16_t
   // taken from windows of 512 rows instead of from all 16384).
   const int nth = item / ngroups;
   // (one of several rank classes: the class's own list of tiles, which is in the same walk order)
-  const int tile_id = a.wl_tiles.ids ? work_item(a.wl_tiles, nth) : (tile_walk ? tile_walk[nth] : nth);
+  const int tile_id = checked_tile(a.wl_tiles.ids ? work_item(a.wl_tiles, nth) : (tile_walk ? tile_walk[nth] : nth), a.tb);
   if (tile_id < 0) return;
   const int c0 = (item - nth * ngroups) << 7;
   const int slot0 = tile_id * kTileRows;
   // independent first loads: group id, row indices, h operand (nothing branches before the
   // destination loads are in flight)
-  const int g_raw = tile_group[tile_id];
+  const int g_raw = checked_group(tile_group[tile_id], a.tb);
   // rows this lane updates: slots 16 tt + 4 kb + v
   const int4 r0 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 4 * kb);
   const int4 r1 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 16 + 4 * kb);
@@ -532,7 +533,7 @@ __device__ __forceinline__ void expand_flat_body(const PassArgs& a, const bf16_t
   for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      rok[tt][v] = g_raw >= 0 && rows[tt][v] >= 0;
+      rok[tt][v] = g_raw >= 0 && checked_row(rows[tt][v], a.tb) >= 0;
       yp[tt][v] = (bf16_t*)a.dst + (int64_t)(rok[tt][v] ? rows[tt][v] : 0) * a.ld_dst + 8 * li + c0;
     }
   const int r = g_raw < 0 ? 0 : class_rank(a.rank[g], a.rank_lo, RP);
@@ -639,11 +640,11 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
   const int cb = block % nbt, set = block / nbt;
   const int tile0 = (sweep ? swept_set : set) * TPI;
   const int cg = cb * 4 + wave;
-  if (cg >= ngroups) return;
+  if (cg >= ngroups || tile0 < 0 || tile0 >= max_tiles) return;
   const int nt = min(TPI, max_tiles - tile0);
   int gt[TPI];
 #pragma unroll
-  for (int t = 0; t < TPI; ++t) gt[t] = t < nt ? tile_group[tile0 + t] : -1;
+  for (int t = 0; t < TPI; ++t) gt[t] = t < nt ? checked_group(tile_group[tile0 + t], a.tb) : -1;
   const int c0 = cg << 7;
   bf16_t* dst = (bf16_t*)a.dst + c0 + 8 * li;
 
@@ -667,7 +668,7 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
       }
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        T.rows[tt][v] = tok ? rr[tt][v] : -1;
+        T.rows[tt][v] = tok ? checked_row(rr[tt][v], a.tb) : -1;
         T.y[tt][v] = T.rows[tt][v] >= 0 ? ld16_nt(dst + (int64_t)T.rows[tt][v] * a.ld_dst) : zero4();
       }
     }
@@ -888,7 +889,7 @@ __global__ __launch_bounds__(64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo*
   const int c0 = blockIdx.x * 128;
   const int cidx = work_item(a.wl_chunks, blockIdx.y - a.tr.y_blocks);
   if (cidx < 0) return;  // past the end of this rank class's list
-  const ChunkInfo ci = chunks[cidx];
+  const ChunkInfo ci = checked_chunk(chunks[cidx], a.tb);
   const int g = ci.group;
   if (g < 0) return;
   const int r = class_rank(a.rank[g], a.rank_lo, 16 * NB);
@@ -922,8 +923,9 @@ __global__ __launch_bounds__(64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo*
     T.live = 0;
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
-      T.x[q] = ld16(src + (int64_t)max(rows[q], 0) * a.ld_src);
-      T.live |= (t < nt && rows[q] >= 0) ? (1u << q) : 0u;
+      const int row = checked_row(rows[q], a.tb);
+      T.x[q] = ld16(src + (int64_t)max(row, 0) * a.ld_src);
+      T.live |= (t < nt && row >= 0) ? (1u << q) : 0u;
     }
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) T.h[nb] = ld16(hT + (int64_t)(16 * nb) * a.ldh + tc * kTileRows);
@@ -997,7 +999,7 @@ __device__ __forceinline__ void wgrad_coop_body(const WgradArgs& a, const ChunkI
   const int c0 = bx * 128;
   const int cidx = work_item(a.wl_chunks, by - a.tr.y_blocks);
   if (cidx < 0) return;  // past the end of this rank class's list
-  const ChunkInfo ci = chunks[cidx];
+  const ChunkInfo ci = checked_chunk(chunks[cidx], a.tb);
   const int g = ci.group;
   if (g < 0) return;
   const int r = class_rank(a.rank[g], a.rank_lo, 16 * NB);
@@ -1029,8 +1031,9 @@ __device__ __forceinline__ void wgrad_coop_body(const WgradArgs& a, const ChunkI
     P.live = 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      P.x[i] = ld16(src + (int64_t)max(rows[i], 0) * a.ld_src);
-      P.live |= rows[i] >= 0 ? (1u << i) : 0u;
+      const int row = checked_row(rows[i], a.tb);
+      P.x[i] = ld16(src + (int64_t)max(row, 0) * a.ld_src);
+      P.live |= row >= 0 ? (1u << i) : 0u;
     }
 #pragma unroll
     for (int nb = 0; nb < NBW; ++nb) P.h[nb] = ld16(hT + (int64_t)(16 * nb) * a.ldh + tc * kTileRows);
@@ -1137,7 +1140,7 @@ __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* co
   }
   const int cidx = work_item(a.wl_chunks, by - a.tr.y_blocks);
   if (cidx < 0) return;  // past the end of this rank class's list
-  const ChunkInfo ci = chunks[cidx];
+  const ChunkInfo ci = checked_chunk(chunks[cidx], a.tb);
   const int g = ci.group;
   if (g < 0) return;
   const int r = class_rank(a.rank[g], a.rank_lo, RP);
@@ -1186,8 +1189,9 @@ __device__ __forceinline__ void dy_fused_body(const WgradArgs& a, const void* co
     live = 0;
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
-      x[q] = ld16(src + (int64_t)max(rows[q], 0) * a.ld_src);
-      live |= (t < nt && rows[q] >= 0) ? (1u << q) : 0u;
+      const int row = checked_row(rows[q], a.tb);
+      x[q] = ld16(src + (int64_t)max(row, 0) * a.ld_src);
+      live |= (t < nt && row >= 0) ? (1u << q) : 0u;
     }
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) h[nb] = ld16(hT + (int64_t)(16 * nb) * a.ldh + tc * kTileRows);

@@ -606,7 +606,8 @@ __global__ __launch_bounds__(256) void k_permute(const T* __restrict__ src, int6
   if (slot >= slots) return;
   const int f = slot_row[slot];
   const int j = slot_pos[slot];
-  if (f < 0 || j < 0) return;
+  // (table entries are compared with the row count before they index: a row or position outside it is skipped)
+  if (f < 0 || j < 0 || f >= tokens * top_k || j >= tokens * top_k) return;
   const int t = f % tokens, k = f / tokens;
   const RowVec<T, V>* s = reinterpret_cast<const RowVec<T, V>*>(src + (int64_t)t * ld_src);
   RowVec<T, V>* d = reinterpret_cast<RowVec<T, V>*>(dst + (int64_t)j * ld_dst);
@@ -636,6 +637,7 @@ __global__ __launch_bounds__(256) void k_unpermute(const T* __restrict__ rows_, 
     for (int i = 0; i < V; ++i) acc[i] = 0.f;
     for (int k = 0; k < top_k; ++k) {
       const int j = inv[(int64_t)k * tokens + t];
+      if ((unsigned)j >= (unsigned)(tokens * top_k)) continue;  // (a position outside the table's rows adds nothing)
       const RowVec<T, V> x = reinterpret_cast<const RowVec<T, V>*>(rows_ + (int64_t)j * ld_rows)[c];
       const float wt = w ? to_f32(w[(int64_t)t * top_k + k]) : 1.f;
 #pragma unroll
@@ -665,6 +667,10 @@ __global__ __launch_bounds__(64) void k_unpermute_wgrad(const T* __restrict__ do
   const int f = blockIdx.x;  // flat row k * tokens + t
   const int t = f % tokens, k = f / tokens;
   const int j = inv[f];
+  if ((unsigned)j >= (unsigned)(tokens * top_k)) {  // (a position outside the table's rows: no row, no gradient)
+    if (threadIdx.x == 0) dw[(int64_t)t * top_k + k] = 0.f;
+    return;
+  }
   const RowVec<T, V>* a = reinterpret_cast<const RowVec<T, V>*>(dout + (int64_t)t * ld_dout);
   const RowVec<T, V>* b = reinterpret_cast<const RowVec<T, V>*>(rows_ + (int64_t)j * ld_rows);
   float acc = 0.f;

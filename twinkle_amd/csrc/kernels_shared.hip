@@ -131,8 +131,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(P <= 3 ? 3 :
   const int block = xcd_contiguous(blockIdx.x, gridDim.x);
   const int pair = block / a.kslices, ks = block - pair * a.kslices;
   const int t0 = 2 * pair, t1 = t0 + 1;
-  const int g0 = tile_group[t0];
-  const int g1 = t1 < max_tiles ? tile_group[t1] : -1;
+  if (t0 >= max_tiles) return;
+  const int g0 = checked_group(tile_group[t0], a.tb);
+  const int g1 = t1 < max_tiles ? checked_group(tile_group[t1], a.tb) : -1;
   if (g0 >= 0 && g1 == g0) {
     const int tiles[2] = {t0, t1};
     shrink_tiles_shared<P, 2>(a, slot_rows, tiles, g0, ks, part);
@@ -165,7 +166,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void k
   const int tile_id = item / ngroups;
   const int c0 = (item - tile_id * ngroups) << 7;
   const int slot0 = tile_id * kTileRows;
-  const int g_raw = tile_group[tile_id];
+  const int g_raw = checked_group(tile_group[tile_id], a.tb);
   const int4 r0 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 4 * kb);
   const int4 r1 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 16 + 4 * kb);
   const int off = 8 * (kb & 1);  // first rank index of this lane inside its block
@@ -186,7 +187,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void k
   for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      rok[tt][v] = g_raw >= 0 && rows[tt][v] >= 0;
+      rok[tt][v] = g_raw >= 0 && checked_row(rows[tt][v], a.tb) >= 0;
       yp[tt][v] = (bf16_t*)a.dst + (int64_t)(rok[tt][v] ? rows[tt][v] : 0) * a.ld_dst + 8 * li + c0;
     }
   int rblk[NKS];
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(P <= 3 ? 2 :
   extern __shared__ __attribute__((aligned(16))) int32_t rows_s[];  // the chunk's row indices
   const int lane = threadIdx.x & 63, li = lane & 15, kb = lane >> 4;
   const int c0 = blockIdx.x * 128;
-  const ChunkInfo ci = chunks[blockIdx.y];
+  const ChunkInfo ci = checked_chunk(chunks[blockIdx.y], a.w[0].tb);
   const int g = ci.group;
   if (g < 0) return;
   int r[P];
@@ -297,8 +298,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(P <= 3 ? 2 :
     T.live = 0;
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
-      T.x[q] = ld16(src + (int64_t)max(rows[q], 0) * a0.ld_src);
-      T.live |= (t < nt && rows[q] >= 0) ? (1u << q) : 0u;
+      const int row = checked_row(rows[q], a0.tb);
+      T.x[q] = ld16(src + (int64_t)max(row, 0) * a0.ld_src);
+      T.live |= (t < nt && row >= 0) ? (1u << q) : 0u;
     }
 #pragma unroll
     for (int p = 0; p < P; ++p) T.h[p] = ld16(hT[p] + tc * kTileRows);
@@ -386,10 +388,11 @@ __global__ __launch_bounds__(256) void k_expand_shared_wide(SharedExpandArgs a, 
   const int item = blockIdx.x * 4 + wave;
   if (item >= num_items) return;
   const int nth = item / ngroups;
-  const int tile_id = tile_walk ? tile_walk[nth] : nth;
+  const int tile_id = checked_tile(tile_walk ? tile_walk[nth] : nth, a.tb);
+  if (tile_id < 0) return;
   const int c0 = (item - nth * ngroups) << 7;
   const int slot0 = tile_id * kTileRows;
-  const int g_raw = tile_group[tile_id];
+  const int g_raw = checked_group(tile_group[tile_id], a.tb);
   const int4 r0 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 4 * kb);
   const int4 r1 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 16 + 4 * kb);
   const int g = max(g_raw, 0);
@@ -401,7 +404,7 @@ __global__ __launch_bounds__(256) void k_expand_shared_wide(SharedExpandArgs a, 
   for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      rok[tt][v] = g_raw >= 0 && rows[tt][v] >= 0;
+      rok[tt][v] = g_raw >= 0 && checked_row(rows[tt][v], a.tb) >= 0;
       yp[tt][v] = (bf16_t*)a.dst + (int64_t)(rok[tt][v] ? rows[tt][v] : 0) * a.ld_dst + 8 * li + c0;
       y[tt][v] = rok[tt][v] ? ld16_nt(yp[tt][v]) : zero4();
     }

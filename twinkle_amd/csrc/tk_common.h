@@ -294,6 +294,22 @@ struct BwdLayout {
   }
 };
 
+// What a consumer of a segment table may index with: every group number, row number, tile range and partial slot that a
+// kernel reads from the table (caller-held memory) is compared with these before it is used as an index, and an entry
+// outside them is treated as absent (no group, no row, an empty chunk).  A table that was overwritten or belongs to
+// another batch then gives wrong results for the tiles concerned, not accesses outside the caller's tensors.
+struct TableBounds {
+  int32_t groups;        // group numbers are in [0, groups)
+  int32_t rows;          // row numbers (slot_row / slot_pos entries) are in [0, rows)
+  int32_t max_tiles;     // tile numbers are in [0, max_tiles)
+  int32_t chunk_tiles;   // a chunk has at most this many tiles
+  int32_t max_partials;  // partial slots are in [0, max_partials)
+};
+static inline TableBounds table_bounds(const SegLayout& L) {
+  return TableBounds{(int32_t)L.groups, (int32_t)L.rows, (int32_t)L.max_tiles, (int32_t)L.chunk_tiles,
+                     (int32_t)L.max_partials};
+}
+
 // Work list of a launch that serves one rank class out of several: the ids of the work items (tiles, pairs of tiles,
 // chunks ..) that hold a group of the class, and their number, both on the device (built per call by
 // launch_class_lists from the segment table and the ranks).  The grid still covers every item of the table; blocks
@@ -353,6 +369,7 @@ struct PassArgs {
   // may exist, and kernels then look at the rank before they request a tile's rows
   int32_t rank_lo, class_mode;
   WorkList wl_tiles, wl_pairs, wl_octs, wl_sets;  // class_mode: the items of this class (see WorkList)
+  TableBounds tb;
 };
 
 // Optional side job of a weight-gradient launch (bf16 MFMA path): the first `y_blocks` rows of the
@@ -388,6 +405,7 @@ struct WgradArgs {
                        // element type of src (tk_lora_desc::weights_f32)
   int32_t rank_lo;     // groups whose rank is not in (rank_lo, rpad] are skipped (see class_rank)
   WorkList wl_chunks;  // several rank classes: the chunks of this class
+  TableBounds tb;
   TransposeJob tr;
 };
 
@@ -400,6 +418,7 @@ struct SharedShrinkArgs {
   int64_t ld_w[kMaxShared];
   const int32_t* rank[kMaxShared];       // device [G]
   float* hpart[kMaxShared];              // split-shrink buffer of projection p, [tile][slice][32][16]
+  TableBounds tb;
 };
 struct SharedExpandArgs {
   void* dst;  int64_t ld_dst;            // dx
@@ -407,6 +426,7 @@ struct SharedExpandArgs {
   const void* hrow[kMaxShared];          // slot-major dh of projection p, [slots][rpad]
   const void* aT[kMaxShared];            // A_p^T copies, [G][K][rpad]
   const int32_t* rank[kMaxShared];
+  TableBounds tb;
 };
 struct SharedWgradArgs {                 // dA_p for all p from one pass over x (w[p].src / ld_src / width agree)
   int32_t nproj;
@@ -461,6 +481,7 @@ struct GroupedArgs {
   const void* const* lora_B;  int64_t ldb;
   const int32_t* rank;  int32_t rpad;
   const uint16_t* hrow;
+  TableBounds tb;
 };
 bool grouped_gemm_supported(const GroupedArgs& a);
 int64_t grouped_plan_entries(const SegLayout& L, int64_t experts);

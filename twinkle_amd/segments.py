@@ -57,6 +57,24 @@ class SegmentTable:
                    'tk_segment_bad_keys')
         return out.value
 
+    def validate(self) -> None:
+        """Checks every array of the table on the host (``tk_segment_validate``: copies the table back, synchronises).
+        ``ValueError`` naming the first failing check and index if the table is not one ``tk_segment_build`` writes."""
+        check, index = ctypes.c_int32(0), ctypes.c_int64(-1)
+        code = _lib.load().tk_segment_validate(self.workspace.data_ptr(), self.rows, self.num_groups, _lib.stream_ptr(),
+                                               ctypes.byref(check), ctypes.byref(index))
+        if code == _lib.TK_ERR_INVALID and check.value:
+            names = {1: 'header', 2: 'offsets', 3: 'first tiles', 4: 'group of a tile', 5: 'slot rows / positions',
+                     6: 'permutation and its inverse', 7: 'stable order', 8: 'walk orders', 9: 'chunks',
+                     10: 'first chunks / partial slots'}
+            raise ValueError(f'segment table fails check {check.value} ({names.get(check.value)}) at index {index.value}')
+        _lib.check(code, 'tk_segment_validate')
+
+
+def validate_segment_table(seg: SegmentTable) -> None:
+    """See :meth:`SegmentTable.validate`."""
+    seg.validate()
+
 
 def build_segments(keys: torch.Tensor, num_groups: int, num_tokens: Optional[int] = None, want_perm: bool = True,
                    want_offsets: bool = True, check: bool = False) -> SegmentTable:
