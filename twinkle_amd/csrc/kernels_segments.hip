@@ -149,15 +149,19 @@ __device__ inline int group_of(const int32_t* first, int groups, int i) {
   return lo;
 }
 
-constexpr int kScanLdsGroups = 2048;  // up to this many groups the scan keeps its four prefix tables in LDS
+// Per-group prefix over the sort blocks' counts (each block's exclusive base inside its group), then the prefix over
+// the groups: offsets, first tile, first chunk and first partial slot of every group, and the header.  One block; a
+// thread owns a group and requests the counts of 32 sort blocks together: the chain over the sort blocks is what the
+// kernel waits for (eight at a time it took 37 us at 128 sort blocks x 513 groups, 32 at a time 13.6 us; with 64 the
+// registers of a 1024-thread block spill, and a kernel that uses scratch memory slowed every launch behind it on the
+// queue: the whole step 442 -> 597 us).  The per-tile and per-chunk tables are filled by extra blocks of the scatter
+// launch that follows.
+constexpr int kScanBatch = 32;
 
-__global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sort_blocks, int max_tiles,
-                                                   int max_chunks, int chunk_tiles, SegView V,
+__global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sort_blocks, SegView V, int chunk_tiles,
                                                    int64_t* __restrict__ offsets_out) {
   __shared__ int wave_sums[17];
-  __shared__ int32_t lds_first[4][kScanLdsGroups + 1];  // offsets, tile_first, chunk_first, partial_first
   const int tid = threadIdx.x;
-  const bool in_lds = groups <= kScanLdsGroups;
   int bad = 0;
   for (int b = tid; b < sort_blocks; b += 1024) bad += V.bad[b];
   int bad_total;
@@ -167,14 +171,12 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
     const int g = g0 + tid;
     int count = 0;
     if (g < groups) {
-      // per-block counts -> per-block exclusive bases (relative to the group's start); loads are
-      // issued eight at a time so that their latencies overlap
-      for (int b0 = 0; b0 < sort_blocks; b0 += 8) {
-        int c[8];
+      for (int b0 = 0; b0 < sort_blocks; b0 += kScanBatch) {
+        int c[kScanBatch];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) c[j] = b0 + j < sort_blocks ? V.hist[(int64_t)(b0 + j) * groups + g] : 0;
+        for (int j = 0; j < kScanBatch; ++j) c[j] = b0 + j < sort_blocks ? V.hist[(int64_t)(b0 + j) * groups + g] : 0;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < kScanBatch; ++j) {
           if (b0 + j < sort_blocks) V.hist[(int64_t)(b0 + j) * groups + g] = count;
           count += c[j];
         }
@@ -198,12 +200,6 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
       V.chunk_first[g] = e_chunks;
       V.partial_first[g] = e_part;
       if (offsets_out) offsets_out[g] = e_rows;  // [groups - 1] (the caller's last entry): rows that have a group
-      if (in_lds) {
-        lds_first[0][g] = e_rows;
-        lds_first[1][g] = e_tiles;
-        lds_first[2][g] = e_chunks;
-        lds_first[3][g] = e_part;
-      }
     }
   }
   if (tid == 0) {
@@ -211,12 +207,6 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
     V.tile_first[groups] = carry_tiles;
     V.chunk_first[groups] = carry_chunks;
     V.partial_first[groups] = carry_part;
-    if (in_lds) {
-      lds_first[0][groups] = carry_rows;
-      lds_first[1][groups] = carry_tiles;
-      lds_first[2][groups] = carry_chunks;
-      lds_first[3][groups] = carry_part;
-    }
     SegHeader* hdr = V.header;
     hdr->magic = kSegMagic;
     hdr->rows = rows;
@@ -227,17 +217,21 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
     hdr->bad_keys = bad_total;
     hdr->identity_order = 1;
   }
-  // the firsts were written by this block: make them visible to all of its threads, then fill the
-  // per-tile (with its 32 slots) and per-chunk tables in parallel
-  __threadfence_block();
-  __syncthreads();
-  const int32_t* offs = in_lds ? lds_first[0] : V.offsets;
-  const int32_t* tfirst = in_lds ? lds_first[1] : V.tile_first;
-  const int32_t* cfirst = in_lds ? lds_first[2] : V.chunk_first;
-  const int32_t* pfirst = in_lds ? lds_first[3] : V.partial_first;
-  for (int i = tid; i < max_tiles; i += 1024) {
+}
+
+// Per-tile (with its 32 slots) and per-chunk entries of the table from the groups' firsts: entry i by thread i of the
+// fill blocks (the blocks of the scatter launch past its sort blocks).  slot_row: only the padding is written here,
+// the rows come from the scatter blocks.
+__device__ inline void seg_fill_tables(const SegView& V, int groups, int max_tiles, int max_chunks, int chunk_tiles,
+                                       int thread, int threads) {
+  const int32_t* offs = V.offsets;
+  const int32_t* tfirst = V.tile_first;
+  const int32_t* cfirst = V.chunk_first;
+  const int32_t* pfirst = V.partial_first;
+  const int num_tiles = tfirst[groups], num_chunks = cfirst[groups];
+  for (int i = thread; i < max_tiles; i += threads) {
     int g = -1, pos0 = 0, valid = 0;
-    if (i < carry_tiles) {
+    if (i < num_tiles) {
       g = group_of(tfirst, groups, i);
       pos0 = offs[g] + (i - tfirst[g]) * kTileRows;   // sorted position of the tile's first slot
       valid = min(kTileRows, offs[g + 1] - pos0);       // padding is at the end of a group's last tile
@@ -250,12 +244,11 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
     for (int j = 0; j < kTileRows; j += 4)
       sp[j / 4] = make_int4(j < valid ? pos0 + j : -1, j + 1 < valid ? pos0 + j + 1 : -1,
                             j + 2 < valid ? pos0 + j + 2 : -1, j + 3 < valid ? pos0 + j + 3 : -1);
-    // slot_row: only the padding is written here, the rows come from k_seg_scatter
     for (int j = valid; j < kTileRows; ++j) V.slot_row[(int64_t)i * kTileRows + j] = -1;
   }
-  for (int i = tid; i < max_chunks; i += 1024) {
+  for (int i = thread; i < max_chunks; i += threads) {
     ChunkInfo c{-1, 0, 0, -1};
-    if (i < carry_chunks) {
+    if (i < num_chunks) {
       const int g = group_of(cfirst, groups, i);
       const int j = i - cfirst[g];
       const int ntile = tfirst[g + 1] - tfirst[g];
@@ -270,10 +263,16 @@ __global__ __launch_bounds__(1024) void k_seg_scan(int rows, int groups, int sor
 
 template <typename KeyT>
 __global__ __launch_bounds__(64) void k_seg_scatter(const KeyT* __restrict__ keys, int rows, int groups, int key_bits,
-                                                    SegView V, int64_t* __restrict__ perm_out) {
+                                                    SegView V, int64_t* __restrict__ perm_out, int sort_blocks,
+                                                    int max_tiles, int max_chunks, int chunk_tiles) {
   extern __shared__ int32_t cursor[];
   const int lane = threadIdx.x;
   const int blk = blockIdx.x;
+  if (blk >= sort_blocks) {  // the blocks past the sort blocks fill the per-tile and per-chunk tables
+    seg_fill_tables(V, groups, max_tiles, max_chunks, chunk_tiles, (blk - sort_blocks) * 64 + lane,
+                    ((int)gridDim.x - sort_blocks) * 64);
+    return;
+  }
   const int64_t base = (int64_t)blk * kSortBlockRows;
   int unused = 0;
   int k[kKeysPerLane];
@@ -725,14 +724,18 @@ int launch_segment_build(const void* keys, int key_dtype, int64_t rows, int32_t 
   else
     hipLaunchKernelGGL(k_seg_hist<int64_t>, dim3(nblk), dim3(64), lds, s, (const int64_t*)keys, (int)rows, groups,
                        key_bits, V.hist, V.bad);
-  hipLaunchKernelGGL(k_seg_scan, dim3(1), dim3(1024), 0, s, (int)rows, groups, nblk, (int)L.max_tiles,
-                     (int)L.max_chunks, (int)L.chunk_tiles, V, offsets_out);
+  hipLaunchKernelGGL(k_seg_scan, dim3(1), dim3(1024), 0, s, (int)rows, groups, nblk, V, (int)L.chunk_tiles,
+                     offsets_out);
+  // one table entry per thread of the fill blocks (at least one block: an empty input still gets its tables)
+  const int fill_blocks = (int)std::min<int64_t>(1024, std::max<int64_t>(1, ceil_div(L.max_tiles, 64)));
   if (key_dtype == TK_KEY_I32)
-    hipLaunchKernelGGL(k_seg_scatter<int32_t>, dim3(nblk), dim3(64), lds, s, (const int32_t*)keys, (int)rows, groups,
-                       key_bits, V, perm_out);
+    hipLaunchKernelGGL(k_seg_scatter<int32_t>, dim3(nblk + fill_blocks), dim3(64), lds, s, (const int32_t*)keys,
+                       (int)rows, groups, key_bits, V, perm_out, nblk, (int)L.max_tiles, (int)L.max_chunks,
+                       (int)L.chunk_tiles);
   else
-    hipLaunchKernelGGL(k_seg_scatter<int64_t>, dim3(nblk), dim3(64), lds, s, (const int64_t*)keys, (int)rows, groups,
-                       key_bits, V, perm_out);
+    hipLaunchKernelGGL(k_seg_scatter<int64_t>, dim3(nblk + fill_blocks), dim3(64), lds, s, (const int64_t*)keys,
+                       (int)rows, groups, key_bits, V, perm_out, nblk, (int)L.max_tiles, (int)L.max_chunks,
+                       (int)L.chunk_tiles);
   return check_launch();
 }
 

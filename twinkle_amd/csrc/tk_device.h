@@ -26,6 +26,18 @@ __device__ inline const T* group_weight(const void* const* ptrs, const void* bas
   return ptrs ? (const T*)ptrs[g] : (const T*)base + (int64_t)g * stride;
 }
 
+// Entries of the segment table before they are used as indices (see TableBounds).
+__device__ inline int checked_group(int g, const TableBounds& tb) { return (unsigned)g < (unsigned)tb.groups ? g : -1; }
+__device__ inline int checked_row(int r, const TableBounds& tb) { return (unsigned)r < (unsigned)tb.rows ? r : -1; }
+__device__ inline int checked_tile(int t, const TableBounds& tb) { return (unsigned)t < (unsigned)tb.max_tiles ? t : -1; }
+// a chunk whose tile range or partial slot lies outside the table counts as a chunk of no group
+__device__ inline ChunkInfo checked_chunk(ChunkInfo ci, const TableBounds& tb) {
+  const bool ok = ci.tile0 >= 0 && ci.ntiles >= 0 && ci.ntiles <= tb.chunk_tiles && ci.tile0 <= tb.max_tiles - ci.ntiles &&
+                  ci.partial < tb.max_partials;
+  ci.group = ok ? checked_group(ci.group, tb) : -1;
+  return ci;
+}
+
 // Work item i of a launch: the i-th id of the launch's work list, -1 past its end (see WorkList); i itself without one.
 __device__ inline int work_item(const WorkList& wl, int i) {
   if (!wl.ids) return i;
