@@ -153,8 +153,8 @@ __device__ inline int group_of(const int32_t* first, int groups, int i) {
 // the groups: offsets, first tile, first chunk and first partial slot of every group, and the header.  One block; a
 // thread owns a group and requests the counts of 32 sort blocks together: the chain over the sort blocks is what the
 // kernel waits for (eight at a time it took 37 us at 128 sort blocks x 513 groups, 32 at a time 13.6 us; with 64 the
-// registers of a 1024-thread block spill, and a kernel that uses scratch memory slowed every launch behind it on the
-// queue: the whole step 442 -> 597 us).  The per-tile and per-chunk tables are filled by extra blocks of the scatter
+// registers of a 1024-thread block spill to 376 bytes of scratch memory per thread, and with that one kernel in it the
+// whole step went from 442 to 597 us).  The per-tile and per-chunk tables are filled by extra blocks of the scatter
 // launch that follows.
 constexpr int kScanBatch = 32;
 
