@@ -194,7 +194,10 @@ int tk_lora_fwd(const tk_lora_desc* desc, const void* x_device, int64_t ldx, voi
  * allocates and frees nothing and does not synchronise.  TK_ERR_SCRATCH when tk_lora_h_bytes(desc) exceeds
  * TK_NOALLOC_SCRATCH_BYTES (16 MiB: up to 16384 rows at in_features 4096 for any rank up to 64).  All calls on one
  * GPU share that GPU's buffer and it keeps the last call's contents: two calls whose execution may overlap on one
- * GPU (different streams, or different host threads without ordering) race; order them on one stream. */
+ * GPU (different streams, or different host threads without ordering) race; order them on one stream.
+ * The first call on a GPU looks up the buffer's device address (hipGetSymbolAddress, which may load the library's
+ * device code for that GPU): make one call per GPU outside any stream capture before capturing this entry point;
+ * every later call on that GPU only enqueues kernels. */
 #define TK_NOALLOC_SCRATCH_BYTES (16 << 20)
 int tk_lora_fwd_noalloc(const tk_lora_desc* desc, const void* x_device, int64_t ldx, void* y_device, int64_t ldy,
                         tk_stream_t stream);

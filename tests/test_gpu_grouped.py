@@ -62,9 +62,10 @@ def test_base_term_matches_the_per_expert_loop(dev, e, nt, t, k, n, empty, map_r
     assert max_rel_err(got, want) < 6e-3
 
 
+@pytest.mark.parametrize('weights_f32', [False, True])
 @pytest.mark.parametrize('max_r,ranks', [(8, [8, 4, 8]), (16, [16, 0, 9]), (32, [32, 17, 8]), (64, [64, 40, 16])])
 @pytest.mark.parametrize('e,t,n', [(4, 1800, 384), (4, 1800, 512), (2, 2600, 512)])
-def test_lora_term_in_the_epilogue(dev, max_r, ranks, e, t, n):
+def test_lora_term_in_the_epilogue(dev, max_r, ranks, e, t, n, weights_f32):
     """y = x W_e^T + s (x A_{e,t}^T) B_{e,t}^T per (expert, tenant) segment: oracle's low-rank form per tenant.
     The last shape (out_features a multiple of 256, more than 1024 rows per expert) takes the 256-row blocks on
     8 waves, the others the 128-row blocks on 4 waves."""
@@ -75,12 +76,15 @@ def test_lora_term_in_the_epilogue(dev, max_r, ranks, e, t, n):
     g = torch.Generator().manual_seed(3)
     a = [(torch.randn(e, max_r, k, generator=g) / k**0.5).bfloat16().to(dev) for _ in range(nt)]
     b = [(torch.randn(e, n, max_r, generator=g) * 0.05).bfloat16().to(dev) for _ in range(nt)]
+    if weights_f32:      # fp32 adapters under the bf16 activations: the epilogue reads the bf16 copy the call makes
+        a, b = [v.float() for v in a], [v.float() for v in b]
     idx = [i % nt for i in range(e * nt)]
     # group i = expert i // nt, tenant i % nt: one block of the tenant's packed tensors (a rank-0 tenant is legal at
     # the kernel boundary: its term is skipped)
     groups = AdapterGroups(a, b, [ranks[i % nt] for i in range(e * nt)], [2.0] * (e * nt),
                            a_index=idx, a_offset=[(i // nt) * max_r * k for i in range(e * nt)],
-                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)], rank_classes=False)
+                           b_index=idx, b_offset=[(i // nt) * n * max_r for i in range(e * nt)], rank_classes=False,
+                           act_dtype=torch.bfloat16)
     xd, wd = x.to(dev), w.to(dev)
     h = torch.empty(lora_h_bytes(seg, groups), dtype=torch.uint8, device=dev)
     lora_shrink_(xd, seg, groups, h, map_rows=True)
@@ -430,3 +434,33 @@ def test_swiglu_refuses_what_it_cannot_vectorise(dev):
         swiglu(bad)
     assert swiglu_applies(torch.zeros(4, 32, dtype=torch.bfloat16, device=dev))
     assert not swiglu_applies(torch.zeros(4, 32, dtype=torch.float16, device=dev))
+
+
+def test_experts_forward_per_expert_loop_keeps_rows_without_an_expert(dev):
+    """Keys outside [0, groups) sort behind every expert and belong to none: the per-expert loop (the reference's
+    form) returns one row for every input row all the same, zeros for those, and nothing at all still works."""
+    from twinkle_amd.expert_lora import experts_forward
+    e, hid, inter, t = 3, 64, 96, 50
+
+    class Experts(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            g = torch.Generator().manual_seed(1)
+            self.gate_up_proj = torch.nn.Parameter(torch.randn(e, 2 * inter, hid, generator=g) * 0.1, requires_grad=False)
+            self.down_proj = torch.nn.Parameter(torch.randn(e, hid, inter, generator=g) * 0.1, requires_grad=False)
+            self.act_fn = torch.nn.functional.silu
+
+    experts = Experts().to(dev)
+    keys = torch.sort(torch.randint(0, e, (t,), generator=torch.Generator().manual_seed(2))).values.to(torch.int32)
+    keys[-7:] = e + 1                                                     # rows without an expert, last in order
+    seg = build_segments(keys.to(dev), e)
+    x = torch.randn(t, hid, generator=torch.Generator().manual_seed(3)).to(dev)
+    y = experts_forward(experts, x, seg, ['only'], grouped=False)
+    assert y.shape == (t, hid) and torch.count_nonzero(y[-7:]) == 0
+    for ex in range(e):
+        rows = (keys == ex).nonzero().flatten().to(dev)
+        gu = x[rows] @ experts.gate_up_proj[ex].t()
+        want = (torch.nn.functional.silu(gu[:, :inter]) * gu[:, inter:]) @ experts.down_proj[ex].t()
+        assert max_rel_err(y[rows], want.double().cpu()) < 1e-5
+    none = build_segments(torch.full((t,), -1, dtype=torch.int32, device=dev), e)
+    assert torch.count_nonzero(experts_forward(experts, x, none, ['only'], grouped=False)) == 0

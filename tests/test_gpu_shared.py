@@ -14,46 +14,50 @@ from twinkle_amd import AdapterGroups, build_segments, multi_lora_delta, multi_l
 pytestmark = pytest.mark.gpu
 
 
-def _projections(k, outs, n, max_r, ranks_per_proj, seed, dtype, dev):
+def _projections(k, outs, n, max_r, ranks_per_proj, seed, dtype, dev, weights_f32=False):
     g = torch.Generator().manual_seed(seed)
     projs = []
     max_rs = max_r if isinstance(max_r, tuple) else (max_r,) * len(outs)
+    # weights_f32: fp32 adapters under bf16 activations (values that bf16 holds exactly, so the oracle sees what the
+    # kernels' bf16 copies hold)
+    wdt = (lambda v: v.to(dtype).float()) if weights_f32 else (lambda v: v.to(dtype))
     for m, ranks, mr in zip(outs, ranks_per_proj, max_rs):
-        a = [((torch.rand(mr, k, generator=g) * 2 - 1) / k**0.5).to(dtype) for _ in range(n)]
-        b = [(torch.randn(m, mr, generator=g) * 0.05).to(dtype) for _ in range(n)]
+        a = [wdt((torch.rand(mr, k, generator=g) * 2 - 1) / k**0.5) for _ in range(n)]
+        b = [wdt(torch.randn(m, mr, generator=g) * 0.05) for _ in range(n)]
         scales = [2.0 if i % 2 == 0 else 0.5 for i in range(n)]
         projs.append((a, b, list(ranks), scales))
     return projs
 
 
-def _groups(projs, dev, rank_classes=True):
+def _groups(projs, dev, rank_classes=True, act_dtype=None):
     out = []
     for a, b, ranks, scales in projs:
         ad = [t.to(dev).requires_grad_(True) for t in a]
         bd = [t.to(dev).requires_grad_(True) for t in b]
-        out.append((AdapterGroups(ad, bd, ranks, scales, rank_classes=rank_classes), ad, bd))
+        out.append((AdapterGroups(ad, bd, ranks, scales, rank_classes=rank_classes, act_dtype=act_dtype), ad, bd))
     return out
 
 
-def _compare(dev, dtype, t, k, outs, n, max_r, ranks_per_proj, seed=0, exact=True):
+def _compare(dev, dtype, t, k, outs, n, max_r, ranks_per_proj, seed=0, exact=True, weights_f32=False):
     g = torch.Generator().manual_seed(seed + 100)
     x = torch.randn(t, k, generator=g).to(dtype)
     bases = [torch.randn(t, m, generator=g).to(dtype) for m in outs]
     dys = [torch.randn(t, m, generator=g).to(dtype) for m in outs]
     ids = torch.randint(0, n, (t,), generator=g)
-    projs = _projections(k, outs, n, max_r, ranks_per_proj, seed, dtype, dev)
+    projs = _projections(k, outs, n, max_r, ranks_per_proj, seed, dtype, dev, weights_f32)
+    act = dtype if weights_f32 else None
     seg = build_segments(ids.to(torch.int32).to(dev), n, check=True)
 
     # one call per projection (every group on the kernels of the projection's largest padded rank, like the shared
     # entry points: the bit-for-bit comparison below is between the same kernels)
     xs = x.to(dev).requires_grad_(True)
-    sep = _groups(projs, dev, rank_classes=False)
+    sep = _groups(projs, dev, rank_classes=False, act_dtype=act)
     ys = [multi_lora_delta(xs, b.to(dev) * 1.0, seg, grp) for b, (grp, _, _) in zip(bases, sep)]
     torch.autograd.backward(ys, [d.to(dev) for d in dys])
 
     # one call for all
     xj = x.to(dev).requires_grad_(True)
-    joint = _groups(projs, dev)
+    joint = _groups(projs, dev, act_dtype=act)
     yj = multi_lora_delta_shared(xj, [b.to(dev) * 1.0 for b in bases], seg, [grp for grp, _, _ in joint])
     torch.autograd.backward(list(yj), [d.to(dev) for d in dys])
 
@@ -87,8 +91,9 @@ def _compare(dev, dtype, t, k, outs, n, max_r, ranks_per_proj, seed=0, exact=Tru
     ((1024, 512, 512), ((16, 8, 4, 16, 1), (8, 8, 8, 8, 8), (16, 0, 3, 16, 5))),          # q / k / v, a dead adapter
     ((512, 512, 1024, 512), ((4, 4, 4, 4, 4), (16, 16, 16, 16, 16), (1, 2, 3, 4, 5), (0, 0, 16, 16, 0))),
 ])
-def test_shared_matches_separate_calls_bf16(dev, outs, ranks_per_proj):
-    _compare(dev, torch.bfloat16, 777, 2048, outs, 5, 16, ranks_per_proj)
+@pytest.mark.parametrize('weights_f32', [False, True])
+def test_shared_matches_separate_calls_bf16(dev, outs, ranks_per_proj, weights_f32):
+    _compare(dev, torch.bfloat16, 777, 2048, outs, 5, 16, ranks_per_proj, weights_f32=weights_f32)
 
 
 @pytest.mark.parametrize('max_r,outs,ranks_per_proj', [
@@ -98,9 +103,11 @@ def test_shared_matches_separate_calls_bf16(dev, outs, ranks_per_proj):
     (64, (1024, 512), ((64, 33, 4, 16, 1), (64, 64, 2, 48, 16))),
     (64, (512, 512, 1024, 512), ((64,) * 5, (33,) * 5, (1, 20, 33, 48, 64), (0, 0, 64, 40, 0))),
 ])
-def test_shared_matches_separate_calls_above_rank_16(dev, max_r, outs, ranks_per_proj):
-    """Padded rank 32 and 64: one shrink launch for all projections, one dX read-modify-write, one dA launch."""
-    _compare(dev, torch.bfloat16, 777, 2048, outs, 5, max_r, ranks_per_proj)
+@pytest.mark.parametrize('weights_f32', [False, True])
+def test_shared_matches_separate_calls_above_rank_16(dev, max_r, outs, ranks_per_proj, weights_f32):
+    """Padded rank 32 and 64: one shrink launch for all projections, one dX read-modify-write, one dA launch.
+    weights_f32: fp32 adapters and gradients under the bf16 activations (the state of a PEFT model on a bf16 base)."""
+    _compare(dev, torch.bfloat16, 777, 2048, outs, 5, max_r, ranks_per_proj, weights_f32=weights_f32)
 
 
 def test_shared_rank_64_attention_shape(dev):

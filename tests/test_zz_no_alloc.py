@@ -78,3 +78,39 @@ def test_noalloc_forward_rejects_what_does_not_fit(dev):
     from twinkle_amd import lora_fwd_noalloc_
     with pytest.raises(RuntimeError, match='scratch'):
         lora_fwd_noalloc_(x, y, seg, groups)
+
+
+def test_noalloc_forward_in_a_hip_graph(dev):
+    """The caller it is for: a warm-up call outside the capture (the first call on a GPU looks up the address of
+    the library's buffer), then the same call captured in a HIP graph and replayed with eager work and
+    synchronisations between the replays; every replay equals tk_lora_fwd."""
+    lib = _lib.load()
+    x, base, seg, groups = _case(dev, torch.bfloat16, 2500, 1024, 512, 4, 16, [16, 8, 16, 5], seed=300)
+    d = _desc(seg, groups, True)
+    h = torch.empty(lib.tk_lora_h_bytes(ctypes.byref(d)), dtype=torch.uint8, device=dev)
+    want = base.clone()
+    assert lib.tk_lora_fwd(ctypes.byref(d), x.data_ptr(), x.stride(0), want.data_ptr(), want.stride(0), h.data_ptr(),
+                           _lib.stream_ptr()) == _lib.TK_OK
+    y = torch.empty_like(base)
+
+    def step():
+        y.copy_(base)
+        code = lib.tk_lora_fwd_noalloc(ctypes.byref(d), x.data_ptr(), x.stride(0), y.data_ptr(), y.stride(0),
+                                       _lib.stream_ptr())
+        assert code == _lib.TK_OK
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        step()                                   # warm-up on the capture stream, outside the capture
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(3):
+        y.fill_(3)                               # eager work between the replays (a fill kernel)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want)

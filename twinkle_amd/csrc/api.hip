@@ -756,8 +756,17 @@ int tk_grouped_linear(const tk_grouped_desc* g, const tk_lora_desc* lora, const 
         lora->out_features != g->out_features || lora->dtype != g->dtype || lora->seg_ws != g->seg_ws ||
         lora->map_rows != g->map_rows)
       return TK_ERR_INVALID;
-    if (lora->max_rank > 64 || lora->weights_f32) return TK_ERR_UNSUPPORTED;
+    if (lora->max_rank > 64) return TK_ERR_UNSUPPORTED;
     a.rpad = rank_pad(lora->max_rank);
+    tk_lora_desc staged;
+    if (mixed_weights(*lora)) {
+      // fp32 adapters: the epilogue multiplies with the bf16 copy of B, made in the tail of h like tk_lora_expand
+      // makes it (tk_lora_shrink left the copy of A there)
+      const int rc = stage_weights(lora, (char*)const_cast<void*>(h) + h_core_bytes(lora), false, true,
+                                   (hipStream_t)stream, &staged);
+      if (rc != TK_OK) return rc;
+      lora = &staged;
+    }
     a.lora_B = lora->lora_B;  a.ldb = lora->ldb;  a.rank = lora->rank;
     a.hrow = (const uint16_t*)h + (int64_t)a.rpad * h_ld(g->rows, g->num_groups);  // slot-major half of h
   }
@@ -791,10 +800,13 @@ int tk_swiglu_bwd(const void* gu, int64_t ld_in, const void* dout, int64_t ld_do
 
 // ---- projections that share their input ------------------------------------------------------------------------
 
-static bool any_weights_f32(const tk_lora_desc* const* descs, int32_t n) {
-  for (int p = 0; descs && p < n && p < TK_MAX_SHARED; ++p)
-    if (descs[p] && descs[p]->weights_f32) return true;
-  return false;
+// fp32 adapters under bf16 activations are served by the shared kernels when every projection of the call has them
+// (or none has): the forward reads the bf16 copies it makes in the tail of every h, the backward reads the fp32
+// matrices where the single-projection kernels do and writes fp32 gradients
+static bool weights_agree(const tk_lora_desc* const* descs, int32_t n) {
+  for (int p = 1; p < n; ++p)
+    if ((descs[p]->weights_f32 != 0) != (descs[0]->weights_f32 != 0)) return false;
+  return true;
 }
 
 static bool shared_descs_ok(const tk_lora_desc* const* descs, int32_t n) {
@@ -811,7 +823,7 @@ static bool shared_descs_ok(const tk_lora_desc* const* descs, int32_t n) {
 
 // the kernels of kernels_shared.hip apply: bf16, 2..4 projections of padded rank 16, a split shrink
 static bool shared_fast_path(const tk_lora_desc* const* descs, int32_t n) {
-  if (n < 2 || descs[0]->dtype != TK_DTYPE_BF16 || force_generic() || any_weights_f32(descs, n)) return false;
+  if (n < 2 || descs[0]->dtype != TK_DTYPE_BF16 || force_generic() || !weights_agree(descs, n)) return false;
   for (int p = 0; p < n; ++p)
     if (descs[p]->max_rank < 1 || descs[p]->max_rank > 16) return false;
   return shrink_kslices(descs[0]->in_features, 16) > 1;
@@ -820,7 +832,7 @@ static bool shared_fast_path(const tk_lora_desc* const* descs, int32_t n) {
 // ... or the multi-projection launches of the kernels of padded rank 32 / 64: bf16, 2..4 projections whose padded
 // ranks agree (and exceed 16)
 static bool shared_wide_path(const tk_lora_desc* const* descs, int32_t n) {
-  if (n < 2 || descs[0]->dtype != TK_DTYPE_BF16 || force_generic() || any_weights_f32(descs, n)) return false;
+  if (n < 2 || descs[0]->dtype != TK_DTYPE_BF16 || force_generic() || !weights_agree(descs, n)) return false;
   const int rpad = rank_pad(descs[0]->max_rank);
   if (rpad != 32 && rpad != 64) return false;
   for (int p = 0; p < n; ++p)
@@ -859,13 +871,25 @@ int tk_lora_fwd_shared(const tk_lora_desc* const* descs_in, int32_t n, const voi
   SegView V(d0->seg_ws, L);
   PassArgs a[TK_MAX_SHARED] = {};
   bool fast = shared_fast_path(descs, n);
+  bool wide = !fast && shared_wide_path(descs, n);
+  int rc;
+  // fp32 adapters: the shared kernels read bf16 copies, made here in the tail of every projection's h (where
+  // tk_lora_fwd makes them); `kd` are the descriptors the kernels work from
+  tk_lora_desc staged[TK_MAX_SHARED];
+  const tk_lora_desc* kd[TK_MAX_SHARED];
   for (int p = 0; p < n; ++p) {
-    a[p] = fwd_pass_args(descs[p], x, ldx, y[p], ldy[p], h[p]);
+    kd[p] = descs[p];
+    if ((fast || wide) && mixed_weights(*descs[p])) {
+      if ((rc = stage_weights(descs[p], (char*)h[p] + h_core_bytes(descs[p]), true, true, s, &staged[p])) != TK_OK)
+        return rc;
+      kd[p] = &staged[p];
+    }
+  }
+  for (int p = 0; p < n; ++p) {
+    a[p] = fwd_pass_args(kd[p], x, ldx, y[p], ldy[p], h[p]);
     fast = fast && pass_mfma_supported(a[p]);
   }
-  int rc;
   if (!fast) {
-    bool wide = shared_wide_path(descs, n);
     for (int p = 0; p < n && wide; ++p) wide = pass_mfma_supported(a[p]) && a[p].kslices == a[0].kslices;
     if (wide) {
       // every projection's shrink in one launch, the pieces of x crossing memory once; then y_p += h_p B_p^T
@@ -884,8 +908,8 @@ int tk_lora_fwd_shared(const tk_lora_desc* const* descs_in, int32_t n, const voi
   sa.kslices = a[0].kslices;  sa.nproj = n;
   sa.tb = a[0].tb;
   for (int p = 0; p < n; ++p) {
-    sa.w[p] = descs[p]->lora_A;  sa.ld_w[p] = descs[p]->lda;
-    sa.rank[p] = descs[p]->rank;  sa.hpart[p] = a[p].hpart;
+    sa.w[p] = kd[p]->lora_A;  sa.ld_w[p] = kd[p]->lda;
+    sa.rank[p] = kd[p]->rank;  sa.hpart[p] = a[p].hpart;
   }
   if ((rc = launch_shrink_shared(sa, V, L, s)) != TK_OK) return rc;
   // every projection in one launch each: add the slices (h_p), then y_p += h_p B_p^T

@@ -335,11 +335,12 @@ __global__ __launch_bounds__(256) void k_wgrad_reduce(WgradArgs a0, WgradArgs a1
 
 // Any number of argument sets of one padded rank (dA and dB of several projections) in one launch:
 // blockIdx.z = octets * set + octet of rank indices, octets = rpad / 8.
+template <typename T>
 __global__ __launch_bounds__(256) void k_wgrad_reduce_multi(WgradReduceJobs jobs, int octets,
                                                             const int32_t* __restrict__ chunk_first,
                                                             const int32_t* __restrict__ partial_first) {
   const int set = blockIdx.z / octets;
-  wgrad_reduce_body<bf16_t>(jobs.a[set], 8 * (blockIdx.z - set * octets), chunk_first, partial_first);
+  wgrad_reduce_body<T>(jobs.a[set], 8 * (blockIdx.z - set * octets), chunk_first, partial_first);
 }
 
 // bT_g[n][m] = B_g[m][n], aT_g[k][n] = A_g[n][k]; zero for n >= rank[g].
@@ -504,7 +505,12 @@ int launch_wgrad_reduce_multi(const WgradArgs* sets, int n, const SegView& seg, 
   }
   const int octets = sets[0].rpad / 8;  // the sets share their padded rank
   const dim3 grid((unsigned)L.groups, (unsigned)ceil_div(width, 256), (unsigned)(octets * n));
-  hipLaunchKernelGGL(k_wgrad_reduce_multi, grid, dim3(256), 0, s, J, octets, seg.chunk_first, seg.partial_first);
+  if (sets[0].grad_f32)  // fp32 adapters under bf16 activations (all sets of a call alike)
+    hipLaunchKernelGGL(k_wgrad_reduce_multi<float>, grid, dim3(256), 0, s, J, octets, seg.chunk_first,
+                       seg.partial_first);
+  else
+    hipLaunchKernelGGL(k_wgrad_reduce_multi<bf16_t>, grid, dim3(256), 0, s, J, octets, seg.chunk_first,
+                       seg.partial_first);
   return check_launch();
 }
 

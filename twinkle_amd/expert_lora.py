@@ -431,6 +431,11 @@ def experts_forward(experts_mod: nn.Module, rows: torch.Tensor, seg: SegmentTabl
     def per_expert(inp, weight):
         chunks = [torch.nn.functional.linear(inp[bounds[e]:bounds[e + 1]], weight[e]) for e in range(experts)
                   if bounds[e + 1] > bounds[e]]
+        # rows whose key named no expert come after the last expert's rows (offsets[num_groups] counts the rows that
+        # have a group, not all rows): they get zero rows, so that the result has a row for every row of the input
+        tail = inp.shape[0] - bounds[experts]
+        if tail > 0 or not chunks:
+            chunks.append(inp.new_zeros(max(tail, 0), weight.shape[1]))
         return torch.cat(chunks, dim=0)
 
     gate_up_out = per_expert(x, gate_up)

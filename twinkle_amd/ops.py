@@ -226,6 +226,30 @@ def lora_bwd_workspace_bytes(seg: SegmentTable, groups: AdapterGroups) -> int:
     return _cached_size(seg, groups, 'tk_lora_bwd_workspace_bytes')
 
 
+def lora_h_saved_bytes(seg: SegmentTable, groups: AdapterGroups) -> int:
+    """The part of ``h`` the backward reads.  With fp32 adapters under bf16 activations the forward also keeps its
+    bf16 copies of A and B in the tail of ``h`` (``G * rpad * (K + M)`` elements); the backward makes its own copies
+    from the fp32 matrices, so that tail need not stay alive between forward and backward."""
+    if not groups.weights_f32:
+        return lora_h_bytes(seg, groups)
+    key = ('h_saved', seg.rows)
+    n = groups._size_cache.get(key)
+    if n is None:
+        d = _desc(seg, groups, True)
+        d.weights_f32 = 0
+        n = _lib.load().tk_lora_h_bytes(ctypes.byref(d))
+        _lib.check(n, 'tk_lora_h_bytes')
+        groups._size_cache[key] = n
+    return n
+
+
+def _h_for_backward(h: torch.Tensor, seg: SegmentTable, groups: AdapterGroups) -> torch.Tensor:
+    # fp32 adapters: keep a copy of what the backward reads and let the staged weight copies go with the forward's buffer
+    if not groups.weights_f32:
+        return h
+    return h[:lora_h_saved_bytes(seg, groups)].clone()
+
+
 def lora_fwd_(x: torch.Tensor, y: torch.Tensor, seg: SegmentTable, groups: AdapterGroups, map_rows: bool = True,
               h: Optional[torch.Tensor] = None) -> torch.Tensor:
     """In place ``y += lora(x)``; returns the saved shrink output ``h`` (opaque bytes)."""
@@ -368,7 +392,7 @@ class _LoraDelta(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, y, seg, groups, map_rows, *weights):
-        h = lora_fwd_(x, y, seg, groups, map_rows)
+        h = _h_for_backward(lora_fwd_(x, y, seg, groups, map_rows), seg, groups)
         ctx.mark_dirty(y)
         ctx.save_for_backward(x, h)
         ctx.seg, ctx.groups, ctx.map_rows = seg, groups, map_rows
@@ -396,7 +420,7 @@ class _LoraLinear(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, weight, bias, seg, groups, map_rows, *weights):
         y = torch.nn.functional.linear(x, weight, bias)
-        h = lora_fwd_(x, y, seg, groups, map_rows)
+        h = _h_for_backward(lora_fwd_(x, y, seg, groups, map_rows), seg, groups)
         ctx.save_for_backward(x, weight, h)
         ctx.has_bias = bias is not None
         ctx.seg, ctx.groups, ctx.map_rows = seg, groups, map_rows
