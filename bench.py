@@ -283,7 +283,7 @@ def yardstick_bench(dev, reps=12):
     return out
 
 
-def shared_qkv_bench(dev, steps=20, calibrate_copy=False, rank=16):
+def shared_qkv_bench(dev, steps=20, calibrate_copy=False, rank=16, weights_f32=False):
     """q / k / v of one attention block (4096 -> 4096, 1024, 1024; config 2's tokens, adapters and ids):
     one shared call against one call per projection, forward + backward, segment table built once."""
     import torch
@@ -297,9 +297,10 @@ def shared_qkv_bench(dev, steps=20, calibrate_copy=False, rank=16):
     seg = build_segments(w.ids.to(dev), G, want_perm=False, want_offsets=False)
     groups, ys, dys, pas, pbs, keep = [], [], [], [], [], []
     for m in outs:
-        A = [(torch.randn(rank, K, generator=gen) / K**0.5).to(dt).to(dev) for _ in range(G)]
-        B = [(torch.randn(m, rank, generator=gen) * 0.05).to(dt).to(dev) for _ in range(G)]
-        groups.append(AdapterGroups(A, B, w.ranks if rank == 16 else [rank] * G, w.scales))
+        wdt = torch.float32 if weights_f32 else dt      # fp32 adapters and gradients under the bf16 activations
+        A = [(torch.randn(rank, K, generator=gen) / K**0.5).to(wdt).to(dev) for _ in range(G)]
+        B = [(torch.randn(m, rank, generator=gen) * 0.05).to(wdt).to(dev) for _ in range(G)]
+        groups.append(AdapterGroups(A, B, w.ranks if rank == 16 else [rank] * G, w.scales, act_dtype=dt))
         ys.append(torch.randn(T, m, generator=gen).to(dt).to(dev))
         dys.append(torch.randn(T, m, generator=gen).to(dt).to(dev))
         ga, gb = [torch.zeros_like(t) for t in A], [torch.zeros_like(t) for t in B]
@@ -337,7 +338,8 @@ def shared_qkv_bench(dev, steps=20, calibrate_copy=False, rank=16):
     elt = 2
     per_proj = sum(elt * T * (4 * m + 3 * K) for m in outs)            # y rw, dy r | x r (fwd, dA), dx rw
     joint = sum(elt * T * 4 * m for m in outs) + elt * T * 4 * K       # x r twice, dx rw once
-    res.update({'workload': f'T={T}, {K} -> {outs}, {G} adapters rank {rank}, fwd + bwd, segment table prebuilt',
+    res.update({'workload': f'T={T}, {K} -> {outs}, {G} adapters rank {rank}, fwd + bwd, segment table prebuilt' +
+                            (', fp32 adapter weights and gradients' if weights_f32 else ''),
                 'algorithmic_bytes_one_call_per_projection': per_proj, 'algorithmic_bytes_shared': joint,
                 'speedup': res['one_call_per_projection_ms'] / res['shared_ms'],
                 'hbm_frac_shared': joint / (res['shared_ms'] * 1e-3) / 1e9 / HBM_PEAK_GBS})
@@ -795,7 +797,8 @@ def main():
         print(json.dumps({'moe_experts': moe_experts_bench(dev, steps=max(1, min(args.steps, 10)))}))
         return
     if args.shared_qkv:
-        print(json.dumps({'shared_qkv': shared_qkv_bench(dev, calibrate_copy=args.calibrate_copy, rank=args.rank or 16)}))
+        print(json.dumps({'shared_qkv': shared_qkv_bench(dev, calibrate_copy=args.calibrate_copy, rank=args.rank or 16,
+                                                         weights_f32=args.weights_f32)}))
         return
     w = build_workload(args.workload, args.tokens, args.rank)
     if args.tokens or args.rank:

@@ -34,19 +34,25 @@ bool desc_ok(const tk_lora_desc* d) {
   return true;
 }
 
-// fp32 adapter weights next to bf16 activations: make the bf16 copies at `stage` and return the descriptor the
-// kernels work from (the copies' pointer tables and strides; gradients keep the caller's strides, see bwd)
-int stage_weights(const tk_lora_desc* d, void* stage, bool want_a, bool want_b, hipStream_t s, tk_lora_desc* out) {
+// fp32 adapter weights next to bf16 activations: the kernels read bf16 copies made at `stage` (layout: WeightStage).
+// The descriptor the kernels work from once the copies exist: the copies' pointer tables and strides (gradients keep
+// the caller's strides, see bwd).
+void staged_desc(const tk_lora_desc* d, void* stage, tk_lora_desc* out) {
   const int rpad = rank_pad(d->max_rank);
   const WeightStage W(d->num_groups, rpad, d->in_features, d->out_features);
-  const int rc = launch_convert_weights(*d, stage, want_a, want_b, s);
-  if (rc != TK_OK) return rc;
   *out = *d;
   out->weights_f32 = 0;
   out->lora_A = (const void* const*)((char*)stage + W.off_ptr_a);
   out->lora_B = (const void* const*)((char*)stage + W.off_ptr_b);
   out->lda = d->in_features;
   out->ldb = rpad;
+}
+
+// makes the copies and returns that descriptor
+int stage_weights(const tk_lora_desc* d, void* stage, bool want_a, bool want_b, hipStream_t s, tk_lora_desc* out) {
+  const int rc = launch_convert_weights(*d, stage, want_a, want_b, s);
+  if (rc != TK_OK) return rc;
+  staged_desc(d, stage, out);
   return TK_OK;
 }
 
@@ -877,11 +883,13 @@ int tk_lora_fwd_shared(const tk_lora_desc* const* descs_in, int32_t n, const voi
   // tk_lora_fwd makes them); `kd` are the descriptors the kernels work from
   tk_lora_desc staged[TK_MAX_SHARED];
   const tk_lora_desc* kd[TK_MAX_SHARED];
-  for (int p = 0; p < n; ++p) {
-    kd[p] = descs[p];
-    if ((fast || wide) && mixed_weights(*descs[p])) {
-      if ((rc = stage_weights(descs[p], (char*)h[p] + h_core_bytes(descs[p]), true, true, s, &staged[p])) != TK_OK)
-        return rc;
+  for (int p = 0; p < n; ++p) kd[p] = descs[p];
+  if ((fast || wide) && mixed_weights(*d0)) {  // (all projections alike: weights_agree) one launch converts them all
+    void* stage[TK_MAX_SHARED];
+    for (int p = 0; p < n; ++p) stage[p] = (char*)h[p] + h_core_bytes(descs[p]);
+    if ((rc = launch_convert_weights_multi(descs, stage, n, true, true, s)) != TK_OK) return rc;
+    for (int p = 0; p < n; ++p) {
+      staged_desc(descs[p], stage[p], &staged[p]);
       kd[p] = &staged[p];
     }
   }

@@ -373,9 +373,20 @@ __global__ __launch_bounds__(256) void k_transpose_weights(tk_lora_desc d, int r
 // bf16 copies of fp32 adapter weights (see WeightStage): the live rows of A_g as [rpad][in_features], the live
 // columns of B_g as [out_features][rpad], eight elements per thread, and the two pointer tables.  Round to
 // nearest even, as a cast of the tensors would.
-__global__ __launch_bounds__(256) void k_convert_weights(tk_lora_desc d, int rpad, char* stage, WeightStage W,
-                                                         int want_a, int want_b) {
+struct ConvertJobs {  // one job per projection (blockIdx.z); a single call has one
+  tk_lora_desc d[kMaxShared];
+  char* stage[kMaxShared];
+  WeightStage W[kMaxShared];
+  int32_t rpad[kMaxShared];
+};
+
+__global__ __launch_bounds__(256) void k_convert_weights(ConvertJobs jobs, int want_a, int want_b) {
+  const tk_lora_desc& d = jobs.d[blockIdx.z];
+  const WeightStage& W = jobs.W[blockIdx.z];
+  char* stage = jobs.stage[blockIdx.z];
+  const int rpad = jobs.rpad[blockIdx.z];
   const int g = blockIdx.y;
+  if (g >= d.num_groups) return;
   bf16_t* ac = (bf16_t*)(stage + W.off_a) + (int64_t)g * W.stride_a;
   bf16_t* bc = (bf16_t*)(stage + W.off_b) + (int64_t)g * W.stride_b;
   if (blockIdx.x == 0 && threadIdx.x == 0) {
@@ -436,14 +447,29 @@ __global__ __launch_bounds__(256) void k_convert_weights(tk_lora_desc d, int rpa
 
 }  // namespace
 
-int launch_convert_weights(const tk_lora_desc& d, void* stage, bool want_a, bool want_b, hipStream_t s) {
-  const int rpad = rank_pad(d.max_rank);
-  const WeightStage W(d.num_groups, rpad, d.in_features, d.out_features);
-  const int64_t per_group = (int64_t)rpad * (d.in_features / 8 + 1) + (int64_t)d.out_features * (rpad / 8);
-  const dim3 grid((unsigned)std::min<int64_t>(ceil_div(per_group, 512), 64), (unsigned)d.num_groups);
-  hipLaunchKernelGGL(k_convert_weights, grid, dim3(256), 0, s, d, rpad, (char*)stage, W, want_a ? 1 : 0,
-                     want_b ? 1 : 0);
+int launch_convert_weights_multi(const tk_lora_desc* const* d, void* const* stage, int n, bool want_a, bool want_b,
+                                 hipStream_t s) {
+  if (n < 1 || n > kMaxShared) return TK_ERR_INVALID;
+  ConvertJobs J{};
+  int64_t per_group = 0;
+  int groups = 0;
+  for (int p = 0; p < n; ++p) {
+    const int rpad = rank_pad(d[p]->max_rank);
+    J.d[p] = *d[p];
+    J.stage[p] = (char*)stage[p];
+    J.W[p] = WeightStage(d[p]->num_groups, rpad, d[p]->in_features, d[p]->out_features);
+    J.rpad[p] = rpad;
+    per_group = std::max(per_group, (int64_t)rpad * (d[p]->in_features / 8 + 1) + (int64_t)d[p]->out_features * (rpad / 8));
+    groups = std::max(groups, d[p]->num_groups);
+  }
+  const dim3 grid((unsigned)std::min<int64_t>(ceil_div(per_group, 512), 64), (unsigned)groups, (unsigned)n);
+  hipLaunchKernelGGL(k_convert_weights, grid, dim3(256), 0, s, J, want_a ? 1 : 0, want_b ? 1 : 0);
   return check_launch();
+}
+
+int launch_convert_weights(const tk_lora_desc& d, void* stage, bool want_a, bool want_b, hipStream_t s) {
+  const tk_lora_desc* dp = &d;
+  return launch_convert_weights_multi(&dp, &stage, 1, want_a, want_b, s);
 }
 
 int launch_pass_generic(const PassArgs& a, const SegView& seg, const SegLayout& L, int dtype, int phases,

@@ -256,6 +256,7 @@ static inline int64_t bwd_partial_bytes(int64_t rows, int64_t groups, int width,
 struct WeightStage {
   int64_t off_ptr_a, off_ptr_b, off_a, off_b, total;
   int64_t stride_a, stride_b;  // elements per group
+  WeightStage() : off_ptr_a(0), off_ptr_b(0), off_a(0), off_b(0), total(0), stride_a(0), stride_b(0) {}
   WeightStage(int64_t groups, int64_t rpad, int64_t in_features, int64_t out_features) {
     stride_a = rpad * in_features;
     stride_b = out_features * rpad;
@@ -453,6 +454,9 @@ struct WgradReduceJobs {
 };
 // bf16 copies of the fp32 weights of `d` (layout: WeightStage at `stage`), with their pointer tables
 int launch_convert_weights(const tk_lora_desc& d, void* stage, bool want_a, bool want_b, hipStream_t s);
+// the same for up to kMaxShared descriptors (projections that share their input) in one launch
+int launch_convert_weights_multi(const tk_lora_desc* const* d, void* const* stage, int n, bool want_a, bool want_b,
+                                 hipStream_t s);
 int launch_transpose_job(const TransposeJob& t, const int32_t* rank, int rpad, hipStream_t s);
 int launch_dy_fused_multi(const DyFusedJob* jobs, int n, const SegView& seg, const SegLayout& L, hipStream_t s);
 int launch_pass_multi(const PassArgs* a, int n, const SegView& seg, const SegLayout& L, int phases, hipStream_t s);
