@@ -603,7 +603,10 @@ __global__ __launch_bounds__(256) void k_expand_mfma_multi(PassJobs jobs, const 
 // where the group changes inside an item the wave reloads the block.  The next tile's rows, h operand
 // and destination rows are requested before the current tile is consumed.
 // ---------------------------------------------------------------------------
-template <int NB, int TPI>
+// CLS: the launch serves one of several rank classes (work list of sets, ranks outside the class skipped).  A
+// compile-time switch because this kernel's schedule is touchy: with the two forms in one body the single-class
+// launch measured 10 % slower (config 5's q projection: 116 against 106 us).
+template <int NB, int TPI, bool CLS>
 __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* __restrict__ hrow,
                                                       const int32_t* __restrict__ tile_group,
                                                       const int32_t* __restrict__ slot_rows,
@@ -625,8 +628,8 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
   // (the flags and the order entry are requested together: one round trip in front of the tile's first loads)
   int swept_set = 0;
   bool sweep = false;
-  if (a.wl_sets.ids != nullptr) {
-    // one of several rank classes: the class's list of sets, already in the order to take them in
+  if constexpr (CLS) {
+    // the class's list of sets, already in the order to take them in
     swept_set = work_item(a.wl_sets, blockIdx.x / nbt);
     if (swept_set < 0) return;
     sweep = true;
@@ -640,7 +643,7 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
   const int cb = block % nbt, set = block / nbt;
   const int tile0 = (sweep ? swept_set : set) * TPI;
   const int cg = cb * 4 + wave;
-  if (cg >= ngroups || tile0 < 0 || tile0 >= max_tiles) return;
+  if (cg >= ngroups || (unsigned)tile0 >= (unsigned)max_tiles) return;
   const int nt = min(TPI, max_tiles - tile0);
   int gt[TPI];
 #pragma unroll
@@ -655,6 +658,7 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
   };
   auto issue = [&](int t, Tile& T) {
     const bool tok = t < nt;  // wave-uniform
+    const unsigned row_limit = tok ? (unsigned)a.tb.rows : 0u;  // rows of the table are in [0, rows): see TableBounds
     const int slot0 = (tile0 + (tok ? t : 0)) * kTileRows;
     const int4 r0 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 4 * kb);
     const int4 r1 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 16 + 4 * kb);
@@ -668,7 +672,7 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
       }
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        T.rows[tt][v] = tok ? checked_row(rr[tt][v], a.tb) : -1;
+        T.rows[tt][v] = (unsigned)rr[tt][v] < row_limit ? rr[tt][v] : -1;
         T.y[tt][v] = T.rows[tt][v] >= 0 ? ld16_nt(dst + (int64_t)T.rows[tt][v] * a.ld_dst) : zero4();
       }
     }
@@ -676,7 +680,7 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
   uint4 bq[8][NKS];
   int r = 0;
   auto load_weights = [&](int g) {  // this wave's block of W2 for group g
-    r = class_rank(a.rank[g], a.rank_lo, RP);
+    r = CLS ? class_rank(a.rank[g], a.rank_lo, RP) : min(a.rank[g], RP);
     const bf16_t* W2 = group_weight<bf16_t>(a.w_expand, a.w_expand_base, a.expand_group_stride, g);
 #pragma unroll
     for (int q = 0; q < 8; ++q)
@@ -1351,8 +1355,9 @@ void launch_pass(const PassArgs& a, const SegView& seg, const SegLayout& L, int 
   if constexpr (NB > 1) {
     constexpr int TPI = 4;
     const int64_t blocks = ceil_div(L.max_tiles, TPI) * ceil_div(ngroups, 4);
-    hipLaunchKernelGGL((k_expand_multi<NB, TPI>), dim3((unsigned)blocks), dim3(256), 0, s, a, hrow, seg.tile_group,
-                       rows, seg.set_walk(a.map_rows), seg.header, seg.round_moved,
+    const auto kernel = a.wl_sets.ids ? k_expand_multi<NB, TPI, true> : k_expand_multi<NB, TPI, false>;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), 0, s, a, hrow, seg.tile_group, rows,
+                       seg.set_walk(a.map_rows), seg.header, seg.round_moved,
                        (int)std::min<int64_t>(L.sort_blocks, 64), (int)L.max_tiles);
   } else {
     const int64_t items = L.max_tiles * ngroups;
