@@ -162,8 +162,10 @@ typedef struct tk_lora_desc {
                                   their dtype).  The kernels read bf16 copies of A and B that every call makes on
                                   the fly inside h / the backward workspace (round to nearest even), multiply on
                                   the matrix cores with fp32 accumulation and write fp32 gradients.  0: A, B and
-                                  the gradients have `dtype`.  The shared-input entry points then run one call per
-                                  projection; tk_grouped_linear does not take it (TK_ERR_UNSUPPORTED). */
+                                  the gradients have `dtype`.  The shared-input entry points take it when all their
+                                  projections agree (else they run one call per projection), tk_grouped_linear
+                                  converts B into the tail of h like tk_lora_expand.  The backward reads only the
+                                  part of h in front of those copies. */
   int32_t rank_classes;        /* Which padded ranks occur among rank[] (which lives on the device, so the host
                                   says it here): bit 0 = some group has rank 1..16, bit 1 = 17..32, bit 2 = 33..64,
                                   bit 3 = 65..128; the bit of max_rank's class must be among them.  With more than
@@ -172,7 +174,8 @@ typedef struct tk_lora_desc {
                                   tenant carries its own r, src/twinkle/model/multi_lora.py:318-325), the classes
                                   side by side on streams of the library, and the backward workspace holds one
                                   region per class (tk_lora_bwd_workspace_bytes accounts for it).  A group whose
-                                  rank lies in no listed class gets no gradients and adds nothing to dx.  The
+                                  rank lies in a class that is not listed is served by the next listed class above
+                                  it, so a mask may be too coarse but loses no group.  The
                                   forward and the layout of h do not depend on the field.  0 (or one bit): one
                                   class for all groups, padded to max_rank.  The shared-input entry points ignore
                                   the field. */

@@ -136,6 +136,45 @@ def test_fp32_adapters_gradient_accumulation(dev):
         assert torch.equal(two, one + one)     # fp32 adds of equal numbers are exact
 
 
+@pytest.mark.parametrize('mask', [None, 0, 0b101, 0b110, 0b111])
+def test_rank_class_masks_give_the_same_backward(dev, mask):
+    """Per-group ranks (src/twinkle/model/multi_lora.py:318-325) with every way of telling the backward about them:
+    the mask made from the live ranks (None), no mask (one class, everything padded to rank 64), and masks that
+    leave a class out although groups of it exist (0b101: ranks 24 and 32 go to the 33..64 kernels; 0b110: ranks 5
+    to 16 go to the 17..32 kernels).  Every variant against the oracle at the bf16 bar, and dX / dA / dB of every
+    variant close to the single-class result (the classes use kernels with other summation orders, so not bitwise)."""
+    ranks = [8, 16, 24, 32, 48, 64, 0, 5]
+    t, k, m, max_r = 3000, 256, 512, 64
+    x, base, dy, a, b, ids, ranks, scales = _problem(t, k, m, len(ranks), max_r, ranks, seed=77)
+    cast = lambda v: v.bfloat16()  # noqa: E731
+    seg = build_segments(ids.to(torch.int32).to(dev), len(a), check=True)
+    f64 = lambda v: cast(v).double()  # noqa: E731
+    _, dxo, dao, dbo = oracle.multi_lora_linear_grads(f64(x), f64(base), ids, [f64(v) for v in a], [f64(v) for v in b],
+                                                      ranks, scales, f64(dy))
+
+    def backward(rank_classes):
+        xd = cast(x).to(dev).requires_grad_(True)
+        ad = [cast(v).to(dev).requires_grad_(True) for v in a]
+        bd = [cast(v).to(dev).requires_grad_(True) for v in b]
+        groups = AdapterGroups(ad, bd, ranks, scales)
+        assert groups.rank_classes == 0b111, 'ranks 5..64 span three classes'
+        if rank_classes is not None:
+            groups.rank_classes = rank_classes
+        multi_lora_delta(xd, cast(base).to(dev), seg, groups).backward(cast(dy).to(dev))
+        return xd.grad, [v.grad for v in ad], [v.grad for v in bd]
+
+    dx, da, db = backward(mask)
+    dx1, da1, db1 = backward(0)
+    assert max_rel_err(dx, dxo) < 2e-2 and max_rel_err(dx, dx1.double().cpu()) < 1e-2
+    for g, r in enumerate(ranks):
+        if r == 0:
+            assert da[g] is None and db[g] is None
+            continue
+        assert max_rel_err(da[g], dao[g]) < 2e-2 and max_rel_err(db[g], dbo[g]) < 2e-2, f'group {g} (rank {r})'
+        assert max_rel_err(da[g], da1[g].double().cpu()) < 1e-2 and max_rel_err(db[g], db1[g].double().cpu()) < 1e-2
+        assert torch.count_nonzero(da[g][r:]) == 0 and torch.count_nonzero(db[g][:, r:]) == 0
+
+
 @pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
 def test_empty_and_huge_segments(dev, dtype):
     t, n = 2100, 6

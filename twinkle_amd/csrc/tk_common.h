@@ -197,8 +197,13 @@ static inline int rank_classes_of(const tk_lora_desc& d, RankClass (&out)[kMaxCl
   int n = 0;
   const int m = d.rank_classes & ((1 << kMaxClasses) - 1);
   if ((m & (m - 1)) != 0) {  // more than one bit
+    // a class's window starts where the listed class below it ends, so a rank between two listed classes is served
+    // by the upper one (a mask can be too coarse, never lose a group)
     for (int c = 0; c < kMaxClasses; ++c)
-      if (((m >> c) & 1) && bound[c] < d.max_rank) out[n++] = RankClass{bound[c], std::min(bound[c + 1], d.max_rank)};
+      if (((m >> c) & 1) && bound[c] < d.max_rank) {
+        const int32_t lo = n ? out[n - 1].hi : 0;
+        out[n++] = RankClass{lo, std::min(bound[c + 1], d.max_rank)};
+      }
   }
   if (n <= 1) {
     out[0] = RankClass{0, d.max_rank};
