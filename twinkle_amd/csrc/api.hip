@@ -137,8 +137,9 @@ ClassStreams* class_streams() {
   return x.state == 1 ? &x : nullptr;
 }
 
-// Runs body(c, stream, forked) for every class: class 0 on the caller's stream, the others on the library's class
-// streams between a fork and a join (forked = true), or all on the caller's stream where there are none.  Everything
+// Runs body(c, stream, forked) for every class: the highest class on the caller's stream (forked = false), the others
+// on the library's class streams between a fork and a join (forked = true), or all on the caller's stream where
+// there are none.  Everything
 // enqueued on `s` before the call is visible to every class; everything every class enqueued is complete for what
 // follows on `s`.  A body that is told `forked` must not fork again: a fork inside a forked stream is more than the
 // runtime's stream capture takes (it crashed when such a capture was ended), and the classes already overlap.
@@ -154,18 +155,24 @@ int for_each_class(int n, hipStream_t s, Body body) {
   }
   std::lock_guard<std::mutex> guard(cs->use);
   if (hipEventRecord(cs->fork, s) != hipSuccess) return TK_ERR_LAUNCH;
-  for (int c = 1; c < n; ++c)
-    if (hipStreamWaitEvent(cs->stream[c - 1], cs->fork, 0) != hipSuccess) return TK_ERR_LAUNCH;
+  for (int c = 0; c + 1 < n; ++c)
+    if (hipStreamWaitEvent(cs->stream[c], cs->fork, 0) != hipSuccess) return TK_ERR_LAUNCH;
   // once forked, every stream joins again, also after an error: none may be left attached to the caller's stream
   // (or to a graph capture of it)
   int rc = TK_OK;
-  for (int c = n - 1; c >= 0; --c) {  // the caller's stream last: the side streams start while it is being filled
-    const int r = body(c, c == 0 ? s : cs->stream[c - 1], true);
+  for (int c = 0; c + 1 < n; ++c) {  // the library's streams first: they start while the caller's is being filled
+    const int r = body(c, cs->stream[c], true);
     if (r != TK_OK && rc == TK_OK) rc = r;
   }
-  for (int c = 1; c < n; ++c)
-    if (hipEventRecord(cs->join[c - 1], cs->stream[c - 1]) != hipSuccess ||
-        hipStreamWaitEvent(s, cs->join[c - 1], 0) != hipSuccess)
+  {
+    // The highest class stays on the caller's stream, where it may fork once more: it is the one with the longest
+    // chain of kernels (above rank 32 dy is read by two of them, which then run side by side).
+    const int r = body(n - 1, s, false);
+    if (r != TK_OK && rc == TK_OK) rc = r;
+  }
+  for (int c = 0; c + 1 < n; ++c)
+    if (hipEventRecord(cs->join[c], cs->stream[c]) != hipSuccess ||
+        hipStreamWaitEvent(s, cs->join[c], 0) != hipSuccess)
       return TK_ERR_LAUNCH;
   return rc;
 }
