@@ -501,6 +501,20 @@ def test_chunks_larger_than_512_rows(dev, dtype, t, k, m, max_r, ranks):
     _run(dev, dtype, x, base, dy, a, b, ids, ranks, scales)
 
 
+@pytest.mark.parametrize('weights_f32', [False, True])
+def test_rank_64_chunk_pairs_with_odd_and_even_first_slots(dev, weights_f32):
+    """At padded rank 64 a weight-gradient work item is two consecutive chunks of a group and the reduction reads
+    every other partial slot.  Group sizes chosen so that groups start at even and at odd slots and have 1, 2, 3, 4,
+    6 and 8 chunks of 128 rows (3000 rows: four tiles per chunk), one of them ending in a six-row chunk."""
+    sizes = [390, 300, 1000, 130, 128, 700, 352]
+    ranks = [64, 40, 64, 33, 64, 50, 64]
+    t, k, m = sum(sizes), 256, 384
+    ids = torch.cat([torch.full((n,), g) for g, n in enumerate(sizes)])
+    ids = ids[torch.randperm(t, generator=torch.Generator().manual_seed(3))]
+    x, base, dy, a, b, _, _, scales = _problem(t, k, m, len(sizes), 64, ranks, seed=11)
+    _run(dev, torch.bfloat16, x, base, dy, a, b, ids, ranks, scales, weights_f32=weights_f32)
+
+
 def _random_case(seed):
     g = torch.Generator().manual_seed(1000 + seed)
     pick = lambda xs: xs[int(torch.randint(0, len(xs), (1,), generator=g))]  # noqa: E731

@@ -559,6 +559,10 @@ static BwdPlan bwd_plan(const tk_lora_desc* d, const BwdLayout& B, const void* d
   // fp32 adapters under bf16 activations: the backward kernels read the weights only through the transposed
   // copies (made from the fp32 matrices directly) and, in the fused pass over dy, B itself; the gradients are fp32
   tr.src_f32 = p.ga.grad_f32 = p.gb.grad_f32 = mixed_weights(*d) ? 1 : 0;
+  // padded rank 64 on the two-wave MFMA kernel (the test run_wgrad makes): chunks are taken in pairs
+  const bool coop = d->dtype == TK_DTYPE_BF16 && !force_generic() && B.rpad == 64;
+  p.ga.pair_chunks = coop && grad_A && wgrad_mfma_supported(p.ga);
+  p.gb.pair_chunks = coop && grad_B && wgrad_mfma_supported(p.gb);
   return p;
 }
 

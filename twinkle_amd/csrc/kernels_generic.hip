@@ -205,6 +205,10 @@ __device__ __forceinline__ void wgrad_reduce_body(const WgradArgs& a, int n0, co
   if (nchunk < 0 || (nchunk > 1 && (pf < 0 || pf > a.tb.max_partials - nchunk))) return;
   if (nchunk == 1) return;
   if (nchunk == 0 && a.accumulate) return;
+  // paired chunks (WgradArgs::pair_chunks): only every other slot behind the first holds a sum
+  const bool paired = a.pair_chunks != 0;
+  const int nlive = paired && nchunk > 0 ? live_partials(nchunk, pf) : nchunk;  // (no chunks: zeros are written)
+  auto slot = [&](int m) { return paired ? live_partial(m, pf) : m; };
   const int64_t stride = partial_slot_floats(a.rpad, a.width);
   T* const gt = (T*)a.grad[g];
   if (a.transposed && (a.ld_grad & (sizeof(T) == 2 ? 7 : 3)) == 0 && (reinterpret_cast<uintptr_t>(gt) & 15u) == 0 &&
@@ -230,12 +234,12 @@ __device__ __forceinline__ void wgrad_reduce_body(const WgradArgs& a, int n0, co
       for (int i = 0; i < 8; ++i) acc[i] = 0.f;
       if (c < a.width && 8 * oct < r) {
         const float* p = a.partial + partial_index(pf, 8 * oct, c, a.rpad, a.width);
-        for (int j0 = 0; j0 < nchunk; j0 += 2) {
+        for (int j0 = 0; j0 < nlive; j0 += 2) {
           float v[2][8];
 #pragma unroll
           for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[j][i] = j0 + j < nchunk ? p[(j0 + j) * stride + i * 128] : 0.f;
+            for (int i = 0; i < 8; ++i) v[j][i] = j0 + j < nlive ? p[slot(j0 + j) * stride + i * 128] : 0.f;
 #pragma unroll
           for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -287,13 +291,13 @@ __device__ __forceinline__ void wgrad_reduce_body(const WgradArgs& a, int n0, co
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
   // two chunks (16 loads) are requested together; every sum adds its chunks in chunk order
-  for (int j0 = 0; j0 < nchunk; j0 += 2) {
+  for (int j0 = 0; j0 < nlive; j0 += 2) {
     float v[2][8];
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-        v[j][i] = (j0 + j < nchunk && n0 + i < r) ? p[(j0 + j) * stride + i * 128] : 0.f;
+        v[j][i] = (j0 + j < nlive && n0 + i < r) ? p[slot(j0 + j) * stride + i * 128] : 0.f;
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll

@@ -1006,9 +1006,16 @@ __device__ __forceinline__ void wgrad_coop_body(const WgradArgs& a, const ChunkI
   const ChunkInfo ci = checked_chunk(chunks[cidx], a.tb);
   const int g = ci.group;
   if (g < 0) return;
+  int nt = ci.ntiles;
+  if (a.pair_chunks) {  // (the neighbours' entries do not depend on ci: three loads side by side)
+    const ChunkInfo none{-1, 0, 0, -1};
+    const ChunkInfo before = cidx > 0 ? checked_chunk(chunks[cidx - 1], a.tb) : none;
+    const ChunkInfo after = cidx + 1 < a.tb.max_chunks ? checked_chunk(chunks[cidx + 1], a.tb) : none;
+    if (chunk_follows(before, ci)) return;  // the block of the chunk in front takes this one's tiles
+    if (chunk_follows(ci, after)) nt += after.ntiles;
+  }
   const int r = class_rank(a.rank[g], a.rank_lo, 16 * NB);
   if (r <= 0) return;
-  const int nt = ci.ntiles;
   for (int i = tid; i < nt * kTileRows; i += RS * 64) rows_s[i] = slot_rows[ci.tile0 * kTileRows + i];
   __syncthreads();
   const int n_base = rs * NBW * 16;   // first rank index of this wave
@@ -1390,7 +1397,7 @@ void launch_wgrad_coop(const WgradArgs& a0, const SegView& seg, const SegLayout&
     a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (2 * (a.width / 128) * 128)));
   }
   const dim3 grid((unsigned)(a.width / 128), (unsigned)(L.max_chunks + a.tr.y_blocks));
-  const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);
+  const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t) * (a.pair_chunks ? 2 : 1);
   hipLaunchKernelGGL((k_wgrad_coop<NB, S>), grid, dim3(128), dyn, s, a, seg.chunks, seg.slot_table(a.map_rows));
 }
 
@@ -1521,7 +1528,9 @@ int launch_wgrad_coop_multi(const SharedWgradArgs& a0, const SegView& seg, const
   const int nx = a.w[0].width / 128;
   const int items = nx * (int)L.max_chunks;
   const dim3 grid((unsigned)(ceil_div(items, 8) * 8 * a.nproj));
-  const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);
+  size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);
+  for (int p = 0; p < a.nproj; ++p)
+    if (a.w[p].pair_chunks) dyn = 2 * (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t);
   const int32_t* rows = seg.slot_table(a.w[0].map_rows);
   if (a.w[0].rpad <= 32)
     hipLaunchKernelGGL((k_wgrad_coop_multi<2, TK_COOP_STAGES>), grid, dim3(128), dyn, s, a, items, nx, seg.chunks, rows);

@@ -310,10 +310,11 @@ struct TableBounds {
   int32_t max_tiles;     // tile numbers are in [0, max_tiles)
   int32_t chunk_tiles;   // a chunk has at most this many tiles
   int32_t max_partials;  // partial slots are in [0, max_partials)
+  int32_t max_chunks;    // chunk numbers are in [0, max_chunks)
 };
 static inline TableBounds table_bounds(const SegLayout& L) {
   return TableBounds{(int32_t)L.groups, (int32_t)L.rows, (int32_t)L.max_tiles, (int32_t)L.chunk_tiles,
-                     (int32_t)L.max_partials};
+                     (int32_t)L.max_partials, (int32_t)L.max_chunks};
 }
 
 // Work list of a launch that serves one rank class out of several: the ids of the work items (tiles, pairs of tiles,
@@ -410,6 +411,7 @@ struct WgradArgs {
   int32_t grad_f32;    // the gradients (and the adapter weights a kernel reads next to them) are fp32 whatever the
                        // element type of src (tk_lora_desc::weights_f32)
   int32_t rank_lo;     // groups whose rank is not in (rank_lo, rpad] are skipped (see class_rank)
+  int32_t pair_chunks; // the launch takes two consecutive chunks of a group as one work item (see chunk_follows)
   WorkList wl_chunks;  // several rank classes: the chunks of this class
   TableBounds tb;
   TransposeJob tr;

@@ -38,6 +38,22 @@ __device__ inline ChunkInfo checked_chunk(ChunkInfo ci, const TableBounds& tb) {
   return ci;
 }
 
+// Weight-gradient launches at padded rank 64 take two consecutive chunks of a group as one work item
+// (WgradArgs::pair_chunks): their partial sums are 64 x width floats per chunk, written once and read once by the
+// reduction, and half as many of them are worth more there than the parallelism of short chunks (config 5's q
+// projection: 40 partials of 1 MB per gradient).  Chunk `b` is taken by the block of the chunk `a` in front of it
+// when both belong to one group, b's partial slot is odd and the two are neighbours in slots and in tiles; the
+// block of `b` then has nothing to do and the reduction leaves b's slot out (see live_partial).  Both blocks
+// evaluate this on the same two checked entries.
+__device__ inline bool chunk_follows(const ChunkInfo& a, const ChunkInfo& b) {
+  return b.group >= 0 && a.group == b.group && (b.partial & 1) && a.partial == b.partial - 1 &&
+         b.tile0 == a.tile0 + a.ntiles;
+}
+// The m-th partial slot (counted from the group's first, `pf`) that holds a sum when chunks are paired, and how
+// many of a group's `nchunk` slots do: the first always, after it the even slots.
+__device__ inline int live_partial(int m, int pf) { return m == 0 ? 0 : 2 * m - (pf & 1); }
+__device__ inline int live_partials(int nchunk, int pf) { return 1 + ((pf & 1) ? nchunk / 2 : (nchunk - 1) / 2); }
+
 // Work item i of a launch: the i-th id of the launch's work list, -1 past its end (see WorkList); i itself without one.
 __device__ inline int work_item(const WorkList& wl, int i) {
   if (!wl.ids) return i;
