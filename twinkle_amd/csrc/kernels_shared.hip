@@ -13,8 +13,8 @@
 // At padded rank 32 and 64 a wave cannot hold several projections' operands at once.  There the single-projection
 // shrink and row-contraction bodies are launched for all projections together, blocks that read the same piece of
 // x next to each other on one XCD (k_shrink_pair_multi, k_wgrad_coop_multi in kernels_mfma.hip), and
-//             k_expand_shared_wide   takes the projections one after the other into the same accumulators:
-//                                    again one read-modify-write of dx.
+//             k_expand_shared_hold   holds a wave's piece of dx in registers while the projections pass one after
+//                                    the other: again one read-modify-write of dx.
 #include "tk_mfma.h"
 
 namespace tk {
@@ -372,84 +372,135 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(P <= 3 ? 2 :
 }
 
 // ---------------------------------------------------------------------------
-// dx[row] += sum_p dh_p[row] A_p for projections of padded rank 32 or 64: one wave = one tile x 128 columns as in
-// k_expand_shared, but the projections are taken one after the other (a projection's block of A^T, 128 columns x
-// rank, is as large as the wave's piece of the tile, so only one of them is held at a time) while the products of all
-// of them add up in the same accumulators: dx is read and written once.  Weights come from the transposed copies
-// [G][K][rpad] of every projection (not permuted).  Tiles are taken in sweep order when rows are gathered.
+// dx[row] += sum_p dh_p[row] A_p for projections of padded rank 32 or 64, with the weights held across tiles (what
+// k_expand_multi does for one projection): one wave = two consecutive tiles x 128 columns.  Weights come from the
+// transposed copies [G][K][rpad] of every projection (not permuted).  Its piece of dx stays in registers as bf16 (64 registers) while the
+// projections pass one after the other: per projection the wave loads the 128 x rank block of A^T once for both
+// tiles (as long as they belong to one group), multiplies each tile's dh_p with it and adds the product onto the
+// held rows, rounding to bf16 after every projection exactly as one k_expand_multi launch per projection would: dx
+// has the bits of the separate calls, with one read and one write of dx instead of one per projection.  (A form with
+// one tile per wave and fp32 sums over the projections fetched every weight block once per tile; the traffic
+// between L2 and the CUs bounds these kernels above rank 16, and it took 155 us against 123 us for this one at
+// q / k / v of rank 64, 16384 rows; three k_expand_multi launches: 135 us.)
+// Items are numbered by sets of four tiles (the segment table's set order when rows are gathered and the keys were
+// interleaved, contiguous runs per XCD otherwise, as in k_expand_multi), each set as two halves.
 // ---------------------------------------------------------------------------
 template <int NB>
-__global__ __launch_bounds__(256) void k_expand_shared_wide(SharedExpandArgs a, const int32_t* __restrict__ tile_group,
+__global__ __launch_bounds__(256) void k_expand_shared_hold(SharedExpandArgs a, const int32_t* __restrict__ tile_group,
                                                             const int32_t* __restrict__ slot_rows,
-                                                            const int32_t* __restrict__ tile_walk, int num_items) {
-  constexpr int RP = 16 * NB, NKS = RP / 32;
+                                                            const int32_t* __restrict__ set_walk,
+                                                            const SegHeader* __restrict__ header,
+                                                            const uint8_t* __restrict__ round_moved, int sort_blocks,
+                                                            int max_tiles) {
+  constexpr int RP = 16 * NB, NKS = RP / 32, TPI = 2;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
   const int ngroups = a.width_dst >> 7;
-  const int item = blockIdx.x * 4 + wave;
-  if (item >= num_items) return;
-  const int nth = item / ngroups;
-  const int tile_id = checked_tile(tile_walk ? tile_walk[nth] : nth, a.tb);
-  if (tile_id < 0) return;
-  const int c0 = (item - nth * ngroups) << 7;
-  const int slot0 = tile_id * kTileRows;
-  const int g_raw = checked_group(tile_group[tile_id], a.tb);
-  const int4 r0 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 4 * kb);
-  const int4 r1 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 16 + 4 * kb);
-  const int g = max(g_raw, 0);
-  const int rows[2][4] = {{r0.x, r0.y, r0.z, r0.w}, {r1.x, r1.y, r1.z, r1.w}};
-  bool rok[2][4];
-  bf16_t* yp[2][4];
-  uint4 y[2][4];
+  const int nbt = (ngroups + 3) >> 2;  // blocks per pair of tiles: column block fastest
+  const int per_set = nbt * (kSetTiles / TPI);
+  int swept_set = 0;
+  bool sweep = false;
+  if (set_walk != nullptr) {
+    swept_set = set_walk[blockIdx.x / per_set];
+    uint2 moved = make_uint2(0u, 0u);
+    if (lane < sort_blocks) moved = reinterpret_cast<const uint2*>(round_moved)[lane];
+    sweep = header->identity_order == 0 && __ballot((moved.x | moved.y) != 0u) != 0ull;
+  }
+  const int block = sweep ? (int)blockIdx.x : xcd_contiguous(blockIdx.x, gridDim.x);
+  const int in_set = block % per_set, set = block / per_set;
+  const int cb = in_set % nbt, half = in_set / nbt;
+  const int tile0 = (sweep ? swept_set : set) * kSetTiles + half * TPI;
+  const int cg = cb * 4 + wave;
+  if (cg >= ngroups || (unsigned)tile0 >= (unsigned)max_tiles) return;
+  const int nt = min(TPI, max_tiles - tile0);
+  int gt[TPI];
 #pragma unroll
-  for (int tt = 0; tt < 2; ++tt)
+  for (int t = 0; t < TPI; ++t) gt[t] = t < nt ? checked_group(tile_group[tile0 + t], a.tb) : -1;
+  if (gt[0] < 0 && gt[1] < 0) return;
+  const int c0 = cg << 7;
+  bf16_t* dst = (bf16_t*)a.dst + c0 + 8 * li;
+  // the rows this lane updates (slots 16 tt + 4 kb + v of each tile) and their dx
+  int rows[TPI][2][4];
+  uint4 y[TPI][2][4];
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      rok[tt][v] = g_raw >= 0 && checked_row(rows[tt][v], a.tb) >= 0;
-      yp[tt][v] = (bf16_t*)a.dst + (int64_t)(rok[tt][v] ? rows[tt][v] : 0) * a.ld_dst + 8 * li + c0;
-      y[tt][v] = rok[tt][v] ? ld16_nt(yp[tt][v]) : zero4();
-    }
-  f32x4 d[2][8];
-#pragma unroll
-  for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-    for (int q = 0; q < 8; ++q) d[tt][q] = f32x4{0.f, 0.f, 0.f, 0.f};
-  bool any = false;
-  for (int p = 0; p < a.nproj; ++p) {
-    const int r = g_raw < 0 ? 0 : min(pick(a.rank, p)[g], RP);  // uniform over the wave
-    if (r <= 0) continue;
-    any = true;
-    const bf16_t* hp = (const bf16_t*)pick(a.hrow, p);
-    const bf16_t* wt = (const bf16_t*)pick(a.aT, p) + ((int64_t)g * a.width_dst + c0 + 8 * li) * RP;
-    uint4 hop[2][NKS], bq[8][NKS];
-#pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) {
-      const int n0 = 32 * ks + 8 * kb;
-#pragma unroll
-      for (int tt = 0; tt < 2; ++tt) hop[tt][ks] = ld16(hp + (int64_t)(slot0 + 16 * tt + li) * RP + n0);
-#pragma unroll
-      for (int q = 0; q < 8; ++q) bq[q][ks] = n0 < r ? keep_first(ld16(wt + (int64_t)q * RP + n0), r - n0) : zero4();
-    }
+  for (int t = 0; t < TPI; ++t) {
+    const bool tok = gt[t] >= 0;  // wave-uniform
+    const unsigned row_limit = tok ? (unsigned)a.tb.rows : 0u;
+    const int slot0 = (tile0 + (t < nt ? t : 0)) * kTileRows;
+    const int4 r0 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 4 * kb);
+    const int4 r1 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 16 + 4 * kb);
+    const int rr[2][4] = {{r0.x, r0.y, r0.z, r0.w}, {r1.x, r1.y, r1.z, r1.w}};
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-      for (int q = 0; q < 8; ++q)
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) d[tt][q] = mfma16(hop[tt][ks], bq[q][ks], d[tt][q]);
+      for (int v = 0; v < 4; ++v) {
+        rows[t][tt][v] = (unsigned)rr[tt][v] < row_limit ? rr[tt][v] : -1;
+        y[t][tt][v] = rows[t][tt][v] >= 0 ? ld16_nt(dst + (int64_t)rows[t][tt][v] * a.ld_dst) : zero4();
+      }
   }
-  if (!any) return;  // unused tile, or no projection live on this layer (uniform over the wave)
+  bool touched[TPI] = {false, false};
+  for (int p = 0; p < a.nproj; ++p) {
+    const int32_t* rank = pick(a.rank, p);
+    const bf16_t* hp = (const bf16_t*)pick(a.hrow, p);
+    const bf16_t* wT = (const bf16_t*)pick(a.aT, p);
+    int held = -1, r = 0;
+    uint4 bq[8][NKS];
 #pragma unroll
-  for (int tt = 0; tt < 2; ++tt)
+    for (int t = 0; t < TPI; ++t) {
+      const int g = gt[t];
+      if (g < 0) continue;  // (uniform over the wave, like every branch of this loop)
+      // the tile's dh operand is requested in front of the weights it may have to wait for
+      uint4 hop[2][NKS];
+      const int slot0 = (tile0 + t) * kTileRows;
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      if (!rok[tt][v]) continue;
-      const uint4 yy = y[tt][v];
-      uint4 o;
-      o.x = pack_bf16(bf16_lo(yy.x) + d[tt][0][v], bf16_hi(yy.x) + d[tt][1][v]);
-      o.y = pack_bf16(bf16_lo(yy.y) + d[tt][2][v], bf16_hi(yy.y) + d[tt][3][v]);
-      o.z = pack_bf16(bf16_lo(yy.z) + d[tt][4][v], bf16_hi(yy.z) + d[tt][5][v]);
-      o.w = pack_bf16(bf16_lo(yy.w) + d[tt][6][v], bf16_hi(yy.w) + d[tt][7][v]);
-      st16_nt(yp[tt][v], o);
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks)
+          hop[tt][ks] = ld16(hp + (int64_t)(slot0 + 16 * tt + li) * RP + 32 * ks + 8 * kb);
+      if (g != held) {
+        held = g;
+        r = min(rank[g], RP);
+        const bf16_t* wt = wT + ((int64_t)g * a.width_dst + c0 + 8 * li) * RP;
+#pragma unroll
+        for (int q = 0; q < 8; ++q)
+#pragma unroll
+          for (int ks = 0; ks < NKS; ++ks) {
+            const int n0 = 32 * ks + 8 * kb;
+            bq[q][ks] = n0 < r ? keep_first(ld16(wt + (int64_t)q * RP + n0), r - n0) : zero4();
+          }
+      }
+      if (r <= 0) continue;  // the group's adapter is not live in this projection
+      touched[t] = true;
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        f32x4 d[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          d[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < NKS; ++ks) d[q] = mfma16(hop[tt][ks], bq[q][ks], d[q]);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const uint4 yy = y[t][tt][v];
+          uint4 o;
+          o.x = pack_bf16(bf16_lo(yy.x) + d[0][v], bf16_hi(yy.x) + d[1][v]);
+          o.y = pack_bf16(bf16_lo(yy.y) + d[2][v], bf16_hi(yy.y) + d[3][v]);
+          o.z = pack_bf16(bf16_lo(yy.z) + d[4][v], bf16_hi(yy.z) + d[5][v]);
+          o.w = pack_bf16(bf16_lo(yy.w) + d[6][v], bf16_hi(yy.w) + d[7][v]);
+          y[t][tt][v] = o;
+        }
+      }
     }
+  }
+#pragma unroll
+  for (int t = 0; t < TPI; ++t) {
+    if (!touched[t]) continue;
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+        if (rows[t][tt][v] >= 0) st16_nt(dst + (int64_t)rows[t][tt][v] * a.ld_dst, y[t][tt][v]);
+  }
 }
 
 }  // namespace
@@ -457,15 +508,16 @@ __global__ __launch_bounds__(256) void k_expand_shared_wide(SharedExpandArgs a, 
 int launch_expand_shared_wide(const SharedExpandArgs& a, int rpad, const SegView& seg, const SegLayout& L,
                               hipStream_t s) {
   if (L.rows == 0) return TK_OK;
-  const int64_t items = L.max_tiles * (a.width_dst >> 7);
-  const dim3 grid((unsigned)ceil_div(items, 4));
   const int32_t* rows = seg.slot_table(a.map_rows);
+  const int64_t nbt = ceil_div((int64_t)(a.width_dst >> 7), 4);
+  const dim3 grid((unsigned)(ceil_div(L.max_tiles, kSetTiles) * (kSetTiles / 2) * nbt));
+  const int sb = (int)std::min<int64_t>(L.sort_blocks, 64);
   if (rpad <= 32)
-    hipLaunchKernelGGL(k_expand_shared_wide<2>, grid, dim3(256), 0, s, a, seg.tile_group, rows,
-                       seg.tile_walk(a.map_rows), (int)items);
+    hipLaunchKernelGGL(k_expand_shared_hold<2>, grid, dim3(256), 0, s, a, seg.tile_group, rows,
+                       seg.set_walk(a.map_rows), seg.header, seg.round_moved, sb, (int)L.max_tiles);
   else
-    hipLaunchKernelGGL(k_expand_shared_wide<4>, grid, dim3(256), 0, s, a, seg.tile_group, rows,
-                       seg.tile_walk(a.map_rows), (int)items);
+    hipLaunchKernelGGL(k_expand_shared_hold<4>, grid, dim3(256), 0, s, a, seg.tile_group, rows,
+                       seg.set_walk(a.map_rows), seg.header, seg.round_moved, sb, (int)L.max_tiles);
   return check_launch();
 }
 
@@ -509,5 +561,6 @@ int launch_wgrad_shared(const SharedWgradArgs& a, const SegView& seg, const SegL
     hipLaunchKernelGGL(k_wgrad_shared<4>, grid, dim3(64), dyn, s, a, seg.chunks, rows);
   return check_launch();
 }
+
 
 }  // namespace tk
