@@ -192,7 +192,10 @@ __global__ __launch_bounds__(256) void k_wgrad_generic(WgradArgs a, const ChunkI
 // that a transposed gradient ([width][r], dB) leaves as 16-byte pieces instead
 // of single elements; blockIdx.z >= rpad / 8 selects the second argument set,
 // so that the reductions of dA and dB share one launch.
-template <typename T>
+// PAIRED: chunks were taken in pairs (WgradArgs::pair_chunks), so only some slots hold sums.  A compile-time switch:
+// the kernel's time is the chain from its first loads to its stores, and the slot arithmetic in that chain cost the
+// unpaired launch 1 us of its 10.
+template <typename T, bool PAIRED>
 __device__ __forceinline__ void wgrad_reduce_body(const WgradArgs& a, int n0, const int32_t* __restrict__ chunk_first,
                                                   const int32_t* __restrict__ partial_first) {
   if (a.grad == nullptr) return;
@@ -206,9 +209,8 @@ __device__ __forceinline__ void wgrad_reduce_body(const WgradArgs& a, int n0, co
   if (nchunk == 1) return;
   if (nchunk == 0 && a.accumulate) return;
   // paired chunks (WgradArgs::pair_chunks): only every other slot behind the first holds a sum
-  const bool paired = a.pair_chunks != 0;
-  const int nlive = paired && nchunk > 0 ? live_partials(nchunk, pf) : nchunk;  // (no chunks: zeros are written)
-  auto slot = [&](int m) { return paired ? live_partial(m, pf) : m; };
+  const int nlive = PAIRED && nchunk > 0 ? live_partials(nchunk, pf) : nchunk;  // (no chunks: zeros are written)
+  auto slot = [&](int m) { return PAIRED ? live_partial(m, pf) : m; };
   const int64_t stride = partial_slot_floats(a.rpad, a.width);
   T* const gt = (T*)a.grad[g];
   if (a.transposed && (a.ld_grad & (sizeof(T) == 2 ? 7 : 3)) == 0 && (reinterpret_cast<uintptr_t>(gt) & 15u) == 0 &&
@@ -334,7 +336,10 @@ __global__ __launch_bounds__(256) void k_wgrad_reduce(WgradArgs a0, WgradArgs a1
                                                       const int32_t* __restrict__ partial_first) {
   const int zsets = rpad >> 3;
   const bool second = (int)blockIdx.z >= zsets;
-  wgrad_reduce_body<T>(second ? a1 : a0, 8 * (second ? blockIdx.z - zsets : blockIdx.z), chunk_first, partial_first);
+  const WgradArgs& a = second ? a1 : a0;
+  const int n0 = 8 * (second ? blockIdx.z - zsets : blockIdx.z);
+  if (a.pair_chunks) wgrad_reduce_body<T, true>(a, n0, chunk_first, partial_first);
+  else wgrad_reduce_body<T, false>(a, n0, chunk_first, partial_first);
 }
 
 // Any number of argument sets of one padded rank (dA and dB of several projections) in one launch:
@@ -344,7 +349,10 @@ __global__ __launch_bounds__(256) void k_wgrad_reduce_multi(WgradReduceJobs jobs
                                                             const int32_t* __restrict__ chunk_first,
                                                             const int32_t* __restrict__ partial_first) {
   const int set = blockIdx.z / octets;
-  wgrad_reduce_body<T>(jobs.a[set], 8 * (blockIdx.z - set * octets), chunk_first, partial_first);
+  const WgradArgs& a = jobs.a[set];
+  const int n0 = 8 * (blockIdx.z - set * octets);
+  if (a.pair_chunks) wgrad_reduce_body<T, true>(a, n0, chunk_first, partial_first);
+  else wgrad_reduce_body<T, false>(a, n0, chunk_first, partial_first);
 }
 
 // bT_g[n][m] = B_g[m][n], aT_g[k][n] = A_g[n][k]; zero for n >= rank[g].
