@@ -393,6 +393,12 @@ __global__ __launch_bounds__(256) void k_expand_shared_hold(SharedExpandArgs a, 
                                                             const uint8_t* __restrict__ round_moved, int sort_blocks,
                                                             int max_tiles) {
   constexpr int RP = 16 * NB, NKS = RP / 32, TPI = 2;
+  // The four waves of a block update the same two tiles (128 columns each), so they multiply with the same dh
+  // operands: these are fetched once per block into LDS (the two tiles' 64 slots x RP of every projection: one
+  // contiguous run of hrow each) instead of once per wave.  Row stride RP + 8 elements: operand reads without bank
+  // conflicts.
+  constexpr int HS = RP + 8;
+  __shared__ __attribute__((aligned(16))) bf16_t dh_s[kMaxShared][TPI * kTileRows * HS];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, li = lane & 15, kb = lane >> 4;
   const int ngroups = a.width_dst >> 7;
   const int nbt = (ngroups + 3) >> 2;  // blocks per pair of tiles: column block fastest
@@ -410,12 +416,37 @@ __global__ __launch_bounds__(256) void k_expand_shared_hold(SharedExpandArgs a, 
   const int cb = in_set % nbt, half = in_set / nbt;
   const int tile0 = (sweep ? swept_set : set) * kSetTiles + half * TPI;
   const int cg = cb * 4 + wave;
-  if (cg >= ngroups || (unsigned)tile0 >= (unsigned)max_tiles) return;
+  if ((unsigned)tile0 >= (unsigned)max_tiles) return;  // (uniform over the block, like the next return)
   const int nt = min(TPI, max_tiles - tile0);
   int gt[TPI];
 #pragma unroll
   for (int t = 0; t < TPI; ++t) gt[t] = t < nt ? checked_group(tile_group[tile0 + t], a.tb) : -1;
   if (gt[0] < 0 && gt[1] < 0) return;
+  {
+    // 16-byte pieces of the nt tiles' dh rows, all projections' requested together
+    constexpr int PPR = RP / 8;                       // pieces per row
+    constexpr int PIECES = TPI * kTileRows * PPR;     // per projection
+    constexpr int PER = (PIECES + 255) / 256;
+    uint4 v[kMaxShared][PER];
+#pragma unroll
+    for (int p = 0; p < kMaxShared; ++p) {
+      const bf16_t* hp = (const bf16_t*)pick(a.hrow, p) + (int64_t)tile0 * kTileRows * RP;
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int e = tid + 256 * i;
+        v[p][i] = (p < a.nproj && e < nt * kTileRows * PPR) ? ld16(hp + 8 * e) : zero4();
+      }
+    }
+#pragma unroll
+    for (int p = 0; p < kMaxShared; ++p)
+#pragma unroll
+      for (int i = 0; i < PER; ++i) {
+        const int e = tid + 256 * i;
+        if (e < PIECES) st16(&dh_s[p][(e / PPR) * HS + 8 * (e % PPR)], v[p][i]);
+      }
+  }
+  __syncthreads();
+  if (cg >= ngroups) return;  // a column group past the width (after the block's only barrier)
   const int c0 = cg << 7;
   bf16_t* dst = (bf16_t*)a.dst + c0 + 8 * li;
   // the rows this lane updates (slots 16 tt + 4 kb + v of each tile) and their dx
@@ -440,7 +471,7 @@ __global__ __launch_bounds__(256) void k_expand_shared_hold(SharedExpandArgs a, 
   bool touched[TPI] = {false, false};
   for (int p = 0; p < a.nproj; ++p) {
     const int32_t* rank = pick(a.rank, p);
-    const bf16_t* hp = (const bf16_t*)pick(a.hrow, p);
+    const bf16_t* hp = dh_s[p];
     const bf16_t* wT = (const bf16_t*)pick(a.aT, p);
     int held = -1, r = 0;
     uint4 bq[8][NKS];
@@ -448,14 +479,12 @@ __global__ __launch_bounds__(256) void k_expand_shared_hold(SharedExpandArgs a, 
     for (int t = 0; t < TPI; ++t) {
       const int g = gt[t];
       if (g < 0) continue;  // (uniform over the wave, like every branch of this loop)
-      // the tile's dh operand is requested in front of the weights it may have to wait for
       uint4 hop[2][NKS];
-      const int slot0 = (tile0 + t) * kTileRows;
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks)
-          hop[tt][ks] = ld16(hp + (int64_t)(slot0 + 16 * tt + li) * RP + 32 * ks + 8 * kb);
+          hop[tt][ks] = ld16(hp + (t * kTileRows + 16 * tt + li) * HS + 32 * ks + 8 * kb);
       if (g != held) {
         held = g;
         r = min(rank[g], RP);
