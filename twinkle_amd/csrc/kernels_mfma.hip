@@ -39,6 +39,11 @@
 #define TK_WGRAD_STAGES 3
 #endif
 
+// h operands of k_expand_multi through LDS (once per block) or straight from memory (once per wave)
+#ifndef TK_EXPAND_LDS_H
+#define TK_EXPAND_LDS_H 1
+#endif
+
 // block renumbering of the rank > 16 expand (contiguous runs of tiles per XCD)
 #ifndef TK_XCD_MAP
 #define TK_XCD_MAP(b, n) xcd_contiguous(b, n)
@@ -643,18 +648,45 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
   const int cb = block % nbt, set = block / nbt;
   const int tile0 = (sweep ? swept_set : set) * TPI;
   const int cg = cb * 4 + wave;
-  if (cg >= ngroups || (unsigned)tile0 >= (unsigned)max_tiles) return;
+  if ((unsigned)tile0 >= (unsigned)max_tiles) return;  // (uniform over the block)
   const int nt = min(TPI, max_tiles - tile0);
   int gt[TPI];
 #pragma unroll
   for (int t = 0; t < TPI; ++t) gt[t] = t < nt ? checked_group(tile_group[tile0 + t], a.tb) : -1;
+#if TK_EXPAND_LDS_H
+  // The block's four waves multiply the same tiles' h operands with their own columns' weights: the operands (one
+  // contiguous run of hrow, nt x 32 slots x RP) are fetched once per block into LDS instead of once per wave.  Row
+  // stride RP + 8 elements: operand reads without bank conflicts.
+  constexpr int HS = RP + 8;
+  __shared__ __attribute__((aligned(16))) bf16_t h_s[TPI * kTileRows * HS];
+  {
+    constexpr int PPR = RP / 8, PIECES = TPI * kTileRows * PPR, PER = (PIECES + 255) / 256;
+    const bf16_t* hp = hrow + (int64_t)tile0 * kTileRows * RP;
+    uint4 v[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int e = tid + 256 * i;
+      v[i] = e < nt * kTileRows * PPR ? ld16(hp + 8 * e) : zero4();
+    }
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int e = tid + 256 * i;
+      if (e < PIECES) st16(&h_s[(e / PPR) * HS + 8 * (e % PPR)], v[i]);
+    }
+  }
+  __syncthreads();
+#endif
+  if (cg >= ngroups) return;  // a column group past the width
   const int c0 = cg << 7;
   bf16_t* dst = (bf16_t*)a.dst + c0 + 8 * li;
 
   struct Tile {
     int rows[2][4];
+#if !TK_EXPAND_LDS_H
     uint4 hop[2][NKS];
+#endif
     uint4 y[2][4];
+    int t;
   };
   auto issue = [&](int t, Tile& T) {
     const bool tok = t < nt;  // wave-uniform
@@ -663,13 +695,16 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
     const int4 r0 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 4 * kb);
     const int4 r1 = *reinterpret_cast<const int4*>(slot_rows + slot0 + 16 + 4 * kb);
     const int rr[2][4] = {{r0.x, r0.y, r0.z, r0.w}, {r1.x, r1.y, r1.z, r1.w}};
+    T.t = tok ? t : 0;
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
+#if !TK_EXPAND_LDS_H
 #pragma unroll
       for (int ks = 0; ks < NKS; ++ks) {
         const int n0 = 32 * ks + 8 * kb;
         T.hop[tt][ks] = (tok && n0 < RP) ? ld16(hrow + (int64_t)(slot0 + 16 * tt + li) * RP + n0) : zero4();
       }
+#endif
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         T.rows[tt][v] = (unsigned)rr[tt][v] < row_limit ? rr[tt][v] : -1;
@@ -693,12 +728,23 @@ __global__ __launch_bounds__(256) void k_expand_multi(PassArgs a, const bf16_t* 
   auto consume = [&](const Tile& T) {
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
+#if TK_EXPAND_LDS_H
+      uint4 hop[NKS];
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks)
+        hop[ks] = 32 * ks + 8 * kb < RP ? ld16(h_s + (T.t * kTileRows + 16 * tt + li) * HS + 32 * ks + 8 * kb) : zero4();
+#endif
       f32x4 d[8];
 #pragma unroll
       for (int q = 0; q < 8; ++q) {
         d[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+#if TK_EXPAND_LDS_H
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) d[q] = mfma16(hop[ks], bq[q][ks], d[q]);
+#else
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) d[q] = mfma16(T.hop[tt][ks], bq[q][ks], d[q]);
+#endif
       }
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
