@@ -110,6 +110,14 @@ def test_shared_matches_separate_calls_above_rank_16(dev, max_r, outs, ranks_per
     _compare(dev, torch.bfloat16, 777, 2048, outs, 5, max_r, ranks_per_proj, weights_f32=weights_f32)
 
 
+@pytest.mark.parametrize('max_r', [32, 64])
+def test_shared_above_rank_16_input_width_off_four_column_groups(dev, max_r):
+    """An input of 1152 columns is nine groups of 128: the last block of the dX kernel has one live wave out of four,
+    and 131 rows end in a tile pair with one tile."""
+    ranks = ((max_r, max_r // 2 + 1, 3), (max_r, max_r, max_r - 7))
+    _compare(dev, torch.bfloat16, 131, 1152, (512, 256), 3, max_r, ranks, seed=5)
+
+
 def test_shared_rank_64_attention_shape(dev):
     """q / k / v at rank 64: 4096 -> 4096, 1024, 1024 on 2048 tokens of 8 adapters, one of them without rows."""
     ranks = [(64, 64, 48, 64, 33, 64, 64, 64)] * 3
