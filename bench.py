@@ -734,6 +734,13 @@ def other_configs_bench(dev, steps=20, warmup=5):
     return out
 
 
+def _side_figure(fn):
+    try:
+        return fn()
+    except Exception as e:  # noqa: BLE001
+        return {'error': f'{type(e).__name__}: {e}'}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -949,11 +956,13 @@ def main():
         import gc
         gc.collect()
         torch.cuda.empty_cache()
-        out['other_configs'] = other_configs_bench(dev)
-        out['other_configs']['cfg4_moe_experts_block'] = moe_experts_bench(dev, steps=2)
+        # (side figures: a failure in one of them is reported in its place and does not take the headline line down)
+        out['other_configs'] = _side_figure(lambda: other_configs_bench(dev))
+        if 'error' not in out['other_configs']:
+            out['other_configs']['cfg4_moe_experts_block'] = _side_figure(lambda: moe_experts_bench(dev, steps=2))
     if not args.no_cpu_baseline:
-        out['optimizer_step'] = optimizer_step_bench(dev)
-        out['torch_gpu_loop'] = torch_gpu_loop(w, dev, dt)
+        out['optimizer_step'] = _side_figure(lambda: optimizer_step_bench(dev))
+        out['torch_gpu_loop'] = _side_figure(lambda: torch_gpu_loop(w, dev, dt))
         out['cpu_baseline'] = cpu_baseline(w)
     print(json.dumps(out))
 
