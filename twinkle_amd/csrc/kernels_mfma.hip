@@ -39,6 +39,11 @@
 #define TK_WGRAD_STAGES 3
 #endif
 
+// pairs of waves per block of k_wgrad_coop (see wgrad_coop_body)
+#ifndef TK_COOP_PAIRS
+#define TK_COOP_PAIRS 2
+#endif
+
 // h operands of k_expand_multi through LDS (once per block) or straight from memory (once per wave)
 #ifndef TK_EXPAND_LDS_H
 #define TK_EXPAND_LDS_H 1
@@ -1030,7 +1035,10 @@ __global__ __launch_bounds__(64) void k_wgrad_pipe(WgradArgs a, const ChunkInfo*
 // they are written to LDS.  One barrier per tile: a wave overwrites a buffer two tiles later, after the
 // barrier that every reader of it has passed.
 // ---------------------------------------------------------------------------
-template <int NB, int S>
+// PAIRS: pairs of waves per block (1 or 2).  Two pairs take neighbouring column blocks of the same chunk: they load
+// the same h operands at about the same time, so the second pair's come from the CU's cache instead of from L2
+// (every 128-column block of a chunk re-reads the chunk's h: a third of this kernel's L2 reads at rank 64).
+template <int NB, int S, int PAIRS = 1>
 __device__ __forceinline__ void wgrad_coop_body(const WgradArgs& a, const ChunkInfo* __restrict__ chunks,
                                                 const int32_t* __restrict__ slot_rows, int bx, int by, int nx) {
   constexpr int RS = 2, NBW = NB / 2;
@@ -1038,9 +1046,10 @@ __device__ __forceinline__ void wgrad_coop_body(const WgradArgs& a, const ChunkI
   constexpr int XS = 136;  // row stride of a staged tile in bf16 (272 B)
   // the tile buffers are dead when the result is staged: one array serves both
   constexpr int kLdsFloats = 16 * NB * OS > kTileRows * XS ? 16 * NB * OS : kTileRows * XS;  // >= two staged bf16 tiles
-  __shared__ __attribute__((aligned(16))) float lds[kLdsFloats];
-  extern __shared__ __attribute__((aligned(16))) int32_t rows_s[];  // the chunk's row indices
-  const int tid = threadIdx.x, lane = tid & 63, li = lane & 15, kb = lane >> 4, rs = tid >> 6;
+  __shared__ __attribute__((aligned(16))) float lds_all[PAIRS * kLdsFloats];
+  float* const lds = lds_all + (PAIRS > 1 ? (threadIdx.x >> 7) * kLdsFloats : 0);
+  extern __shared__ __attribute__((aligned(16))) int32_t rows_s[];  // the chunk's row indices (same for both pairs)
+  const int tid = threadIdx.x & 127, lane = tid & 63, li = lane & 15, kb = lane >> 4, rs = tid >> 6;
   if (by < a.tr.y_blocks) {  // side job: the first rows of the grid transpose the adapter weights
     transpose_weights_job(a.tr, a.rank, a.rpad, ((int64_t)by * nx + bx) * (RS * 64) + tid,
                           (int64_t)a.tr.y_blocks * nx * (RS * 64));
@@ -1144,10 +1153,11 @@ __device__ __forceinline__ void wgrad_coop_body(const WgradArgs& a, const ChunkI
   if (mine) wgrad_store<NBW>(acc, lds + n_base * OS, a, ci, g, r, c0, lane, n_base);
 }
 
-template <int NB, int S>
-__global__ __launch_bounds__(128) void k_wgrad_coop(WgradArgs a, const ChunkInfo* __restrict__ chunks,
-                                                      const int32_t* __restrict__ slot_rows) {
-  wgrad_coop_body<NB, S>(a, chunks, slot_rows, blockIdx.x, blockIdx.y, gridDim.x);
+template <int NB, int S, int PAIRS>
+__global__ __launch_bounds__(128 * PAIRS) void k_wgrad_coop(WgradArgs a, const ChunkInfo* __restrict__ chunks,
+                                                              const int32_t* __restrict__ slot_rows) {
+  wgrad_coop_body<NB, S, PAIRS>(a, chunks, slot_rows, blockIdx.x * PAIRS + (PAIRS > 1 ? threadIdx.x >> 7 : 0), blockIdx.y,
+                                gridDim.x * PAIRS);
 }
 
 // The same contraction for up to kMaxShared projections that read the same source (dA_p = dh_p^T x for the
@@ -1442,9 +1452,18 @@ void launch_wgrad_coop(const WgradArgs& a0, const SegView& seg, const SegLayout&
     const int64_t units = (int64_t)a.tr.groups * a.rpad * ((a.tr.out_features + a.tr.in_features) / 64);
     a.tr.y_blocks = (int)std::min<int64_t>(64, std::max<int64_t>(1, units / (2 * (a.width / 128) * 128)));
   }
-  const dim3 grid((unsigned)(a.width / 128), (unsigned)(L.max_chunks + a.tr.y_blocks));
+  const int nx = a.width / 128;
   const size_t dyn = (size_t)L.chunk_tiles * kTileRows * sizeof(int32_t) * (a.pair_chunks ? 2 : 1);
-  hipLaunchKernelGGL((k_wgrad_coop<NB, S>), grid, dim3(128), dyn, s, a, seg.chunks, seg.slot_table(a.map_rows));
+  // Two pairs per block only where that still leaves every CU several blocks (the grid counts every chunk slot of
+  // the table): measured at config 3 (65 chunk slots x 112 / 32 column blocks) 2.4 % of the step; at config 5's
+  // q projection (41 x 32) the coarser blocks balance worse over the CUs and cost 13 %.
+  if (TK_COOP_PAIRS == 2 && nx % 2 == 0 && (int64_t)nx * L.max_chunks >= 8 * 256) {
+    const dim3 grid((unsigned)(nx / 2), (unsigned)(L.max_chunks + a.tr.y_blocks));
+    hipLaunchKernelGGL((k_wgrad_coop<NB, S, 2>), grid, dim3(256), dyn, s, a, seg.chunks, seg.slot_table(a.map_rows));
+  } else {
+    const dim3 grid((unsigned)nx, (unsigned)(L.max_chunks + a.tr.y_blocks));
+    hipLaunchKernelGGL((k_wgrad_coop<NB, S, 1>), grid, dim3(128), dyn, s, a, seg.chunks, seg.slot_table(a.map_rows));
+  }
 }
 
 }  // namespace
